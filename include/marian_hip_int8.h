@@ -1,0 +1,132 @@
+/*
+ * marian_hip_int8.h - C ABI of the gfx950 (MI355X) int8 affine/dot backend for Marian.
+ *
+ * The functions below are the device-side replacements for the intgemm static interface
+ * as Marian calls it.  Every pointer is a DEVICE pointer unless stated otherwise, every
+ * buffer is owned by the caller (Marian's Allocator slab), nothing is retained between
+ * calls, and all work is enqueued on `stream` (a hipStream_t passed as void*; NULL = the
+ * default stream).  No function synchronises the stream.
+ *
+ * Quantized tensor layout (Marian Type::intgemm8, reference src/common/types.cpp:32-34 and
+ * src/tensors/cpu/integer_common.h:101-106): `elements` int8 values followed by one fp32
+ * quantMult at byte offset `elements`.
+ *   activations  Aq : int8 row-major [M x K]            + quantMult tail  (M*K + 4 bytes)
+ *   weights      Bq : int8 row-major [N x K] = W^T      + quantMult tail  (K*N + 4 bytes)
+ *                     i.e. logical B[k, n] lives at byte n*K + k, exactly the payload of a
+ *                     Type::intgemm8 item in a Marian .bin model file
+ *                     (src/tensors/cpu/expression_graph_packable.h:160-201,242-250).
+ *
+ * Shape rules (intgemm's own): K % 64 == 0, N % 8 == 0, shortlist length % 8 == 0.
+ * Alignment: A, Aq, Bq, out and acc 16 bytes; bias and idx 4 bytes.
+ * M may be any value >= 0 (M == 0 or N == 0 is a no-op).
+ *
+ * Return value: MARIAN_HIP_OK or an error code; a HIP runtime failure returns
+ * MARIAN_HIP_ERR_HIP and the hipError_t is available from marian_hip_last_hip_error().
+ * Nothing aborts or throws across this boundary; the C++ wrappers turn codes into ABORT.
+ */
+#ifndef MARIAN_HIP_INT8_H
+#define MARIAN_HIP_INT8_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum {
+  MARIAN_HIP_OK = 0,
+  MARIAN_HIP_ERR_NULL = 1,      /* a required pointer is NULL */
+  MARIAN_HIP_ERR_SHAPE = 2,     /* negative size, K % 64, N % 8 or n_idx % 8 violated */
+  MARIAN_HIP_ERR_ALIGN = 3,     /* pointer alignment violated */
+  MARIAN_HIP_ERR_WORKSPACE = 4, /* workspace too small */
+  MARIAN_HIP_ERR_HIP = 5,       /* HIP runtime error, see marian_hip_last_hip_error() */
+  MARIAN_HIP_ERR_RANGE = 6      /* size exceeds what the kernels index (2^31 - 1 elements) */
+};
+
+/* Human-readable text for a status code (host pointer, static storage). */
+const char* marian_hip_status_string(int status);
+
+/* hipError_t of the last MARIAN_HIP_ERR_HIP on the calling thread (0 if none). */
+int marian_hip_last_hip_error(void);
+
+/* ABI version of this header; bumped when a signature changes. */
+int marian_hip_int8_abi_version(void);
+
+/* Bytes of device workspace marian_hip_int8_prepare_a / _prepare_b need (a constant). */
+size_t marian_hip_int8_workspace_bytes(void);
+
+/*
+ * Replaces the prepareA node body, reference src/tensors/cpu/intgemm_interface.h:19-29:
+ *   computeQuantMult (integer_common.h:169-173, intgemm::MaxAbsolute), Kernels8::PrepareA
+ *   (quantize) and the getQuantMult(out) = quantMult store.
+ * A: fp32 [M x K].  Aq: M*K + 4 bytes, receives payload and quantMult tail.
+ * quantMult = 127.0f / max|A|; q = clamp(rne(fl32(a * quantMult)), -127, 127).
+ */
+int marian_hip_int8_prepare_a(const float* A, int8_t* Aq, int64_t M, int64_t K,
+                              void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * Replaces the intgemm8 branch of the offline packer, reference
+ * src/tensors/cpu/expression_graph_packable.h:160-201: quantMult over the untransposed fp32
+ * W [K x N], Transpose10, Int8::PrepareA on the transpose, quantMult stored at byte K*N.
+ * Bq: K*N + 4 bytes, receives the [N x K] payload and the tail.
+ */
+int marian_hip_int8_prepare_b(const float* W, int8_t* Bq, int64_t K, int64_t N,
+                              void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * Replaces prepareAndTransposeB<intgemm8>, reference
+ * src/tensors/cpu/integer_common.h:189-216 (Kernels8::PrepareBQuantizedTransposed + tail
+ * copy), which re-tiles the file payload for a CPU.  The GPU kernels consume the file
+ * payload as it is, so this is a device-to-device copy of K*N + 4 bytes.
+ */
+int marian_hip_int8_prepare_b_quantized_transposed(const int8_t* in, int8_t* out, int64_t K,
+                                                   int64_t N, void* stream);
+
+/*
+ * Replaces the multiply node body, reference src/tensors/cpu/intgemm_interface.h:60-88:
+ *   Kernels8::Multiply with callbacks::UnquantizeAndWrite (bias == NULL, dot) or
+ *   UnquantizeAndAddBiasAndWrite (affine).  Both quantMults are read on the device from the
+ *   operand tails (the reference dereferences them on the host, :66-67).
+ *   unquant = (1.0f / (aqm * bqm)) * scale;  out[m,n] = float(acc[m,n]) * unquant (+ bias[n]).
+ * relu != 0 fuses the ReLU that the reference applies as a separate in-place node
+ * (src/graph/expression_operators.cpp:721-731, src/functional/operators.h:128).
+ * out: fp32 [M x N].
+ */
+int marian_hip_int8_affine(const int8_t* Aq, const int8_t* Bq, const float* bias, float* out,
+                           int64_t M, int64_t K, int64_t N, float scale, int relu,
+                           void* stream);
+
+/*
+ * Shortlisted output layer.  Reference (fp32): index_select(Wt, 0, idx), index_select(b, -1,
+ * idx), then dot/affine with transB (src/data/shortlist.cpp:62-79,
+ * src/layers/output.cpp:335-350).  Here rows idx[j] of the [N x K] payload and bias[idx[j]]
+ * are gathered inside the GEMM; bqm is the quantMult of the full matrix.
+ * idx: n_idx sorted unique uint32 ids < N.  out: fp32 [M x n_idx].
+ */
+int marian_hip_int8_affine_shortlist(const int8_t* Aq, const int8_t* Bq, const float* bias,
+                                     const uint32_t* idx, int64_t n_idx, float* out,
+                                     int64_t M, int64_t K, int64_t N, float scale, int relu,
+                                     void* stream);
+
+/*
+ * Parity hooks: the same kernels with the epilogue replaced by a store of the raw int32
+ * accumulators (what Kernels8::Multiply hands to its callback).  acc: int32 [M x N] or
+ * [M x n_idx].  idx == NULL selects the dense form.
+ */
+int marian_hip_int8_multiply_i32(const int8_t* Aq, const int8_t* Bq, const uint32_t* idx,
+                                 int64_t n_idx, int32_t* acc, int64_t M, int64_t K, int64_t N,
+                                 void* stream);
+
+/*
+ * Kernel selection override for measurements: 0 = automatic (default), other values pin one
+ * kernel family for subsequent affine/multiply calls of the calling process.  Returns the
+ * previous value.  Not needed for normal use.
+ */
+int marian_hip_int8_set_kernel(int which);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MARIAN_HIP_INT8_H */

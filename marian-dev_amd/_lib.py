@@ -1,0 +1,75 @@
+"""ctypes binding of libmarian_hip_int8.so (the C ABI declared in include/marian_hip_int8.h).
+
+There is no fallback: if the library has not been built, loading raises."""
+import ctypes
+import os
+import subprocess
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libmarian_hip_int8.so")
+
+OK, ERR_NULL, ERR_SHAPE, ERR_ALIGN, ERR_WORKSPACE, ERR_HIP, ERR_RANGE = range(7)
+
+# name -> (restype, argtypes); the single place the Python side states the ABI
+_c = ctypes
+_vp, _i64, _f, _i, _sz = _c.c_void_p, _c.c_int64, _c.c_float, _c.c_int, _c.c_size_t
+SIGNATURES = {
+    "marian_hip_status_string": (_c.c_char_p, [_i]),
+    "marian_hip_last_hip_error": (_i, []),
+    "marian_hip_int8_abi_version": (_i, []),
+    "marian_hip_int8_workspace_bytes": (_sz, []),
+    "marian_hip_int8_prepare_a": (_i, [_vp, _vp, _i64, _i64, _vp, _sz, _vp]),
+    "marian_hip_int8_prepare_b": (_i, [_vp, _vp, _i64, _i64, _vp, _sz, _vp]),
+    "marian_hip_int8_prepare_b_quantized_transposed": (_i, [_vp, _vp, _i64, _i64, _vp]),
+    "marian_hip_int8_affine": (_i, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _f, _i, _vp]),
+    "marian_hip_int8_affine_shortlist": (_i, [_vp, _vp, _vp, _vp, _i64, _vp, _i64, _i64, _i64,
+                                              _f, _i, _vp]),
+    "marian_hip_int8_multiply_i32": (_i, [_vp, _vp, _vp, _i64, _vp, _i64, _i64, _i64, _vp]),
+    "marian_hip_int8_set_kernel": (_i, [_i]),
+}
+
+_lib = None
+
+
+class MarianHipError(RuntimeError):
+    """Raised where the C++ wrappers would ABORT (reference src/common/logging.h:100-116)."""
+
+    def __init__(self, status, what):
+        self.status = status
+        super().__init__(what)
+
+
+def build(verbose=False):
+    """Compile the HIP library for gfx950 with hipcc (always recompiles)."""
+    cmd = ["make", "-C", os.path.join(_HERE, "csrc"), "-B"]
+    out = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if verbose or out.returncode != 0:
+        print(out.stdout)
+    if out.returncode != 0:
+        raise RuntimeError("hipcc build of libmarian_hip_int8.so failed")
+    return LIB_PATH
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise MarianHipError(
+                -1, "libmarian_hip_int8.so is not built ({}); run __graft_entry__.build() or "
+                "`make -C marian-dev_amd/csrc`. There is no CPU fallback.".format(LIB_PATH))
+        L = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            f = getattr(L, name)  # AttributeError if a declared symbol is not exported
+            f.restype = res
+            f.argtypes = args
+        _lib = L
+    return _lib
+
+
+def check(status, where):
+    if status != OK:
+        L = lib()
+        msg = L.marian_hip_status_string(status).decode()
+        if status == ERR_HIP:
+            msg += " (hipError_t {})".format(L.marian_hip_last_hip_error())
+        raise MarianHipError(status, "{}: {}".format(where, msg))

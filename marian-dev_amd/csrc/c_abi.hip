@@ -1,0 +1,242 @@
+// C ABI of the gfx950 int8 affine backend: argument checks, kernel selection, launches.
+// Declarations and the reference call sites each entry point replaces: include/marian_hip_int8.h
+#include "../../include/marian_hip_int8.h"
+
+#include <hip/hip_runtime.h>
+
+#include <atomic>
+
+#include "gemm_stream_kernel.h"
+#include "gemm_tile_kernel.h"
+#include "quantize_kernels.h"
+
+using namespace marian_hip;
+
+namespace {
+
+thread_local int g_last_hip_error = 0;
+std::atomic<int> g_kernel_override{0};
+
+int hip_fail(hipError_t e) {
+  g_last_hip_error = (int)e;
+  return MARIAN_HIP_ERR_HIP;
+}
+
+#define MH_HIP(expr)                            \
+  do {                                          \
+    hipError_t e_ = (expr);                     \
+    if(e_ != hipSuccess) return hip_fail(e_);   \
+  } while(0)
+
+inline bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
+
+constexpr int64_t kMaxElems = 2147483647LL;
+
+template <typename KernelT>
+int allow_lds(KernelT kernel, int bytes) {
+  if(bytes > 48 * 1024)
+    MH_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                               hipFuncAttributeMaxDynamicSharedMemorySize, bytes));
+  return MARIAN_HIP_OK;
+}
+
+template <int MT, int NT, int WN, int KW, int PF>
+int launch_stream(const GemmArgs& a, hipStream_t st) {
+  using Cfg = StreamCfg<MT, NT, WN, KW, PF>;
+  auto kernel = gemm_stream_kernel<MT, NT, WN, KW, PF>;
+  static const int lds_status = allow_lds(kernel, Cfg::kLdsBytes);
+  if(lds_status != MARIAN_HIP_OK) return lds_status;
+  int blocks = (a.n_out + Cfg::kColsPerBlock - 1) / Cfg::kColsPerBlock;
+  hipLaunchKernelGGL(kernel, dim3(blocks), dim3(Cfg::kThreads), Cfg::kLdsBytes, st, a);
+  MH_HIP(hipGetLastError());
+  return MARIAN_HIP_OK;
+}
+
+template <int WNT, int WMT>
+int launch_tile(const GemmArgs& a, hipStream_t st) {
+  using Cfg = TileCfg<WNT, WMT>;
+  auto kernel = gemm_tile_kernel<WNT, WMT>;
+  static const int lds_status = allow_lds(kernel, Cfg::kLdsBytes);
+  if(lds_status != MARIAN_HIP_OK) return lds_status;
+  int tiles_n = (a.n_out + Cfg::BN - 1) / Cfg::BN;
+  int tiles_m = (a.M + Cfg::BM - 1) / Cfg::BM;
+  hipLaunchKernelGGL(kernel, dim3(tiles_n * tiles_m), dim3(Cfg::kThreads), Cfg::kLdsBytes, st, a,
+                     tiles_n, tiles_m);
+  MH_HIP(hipGetLastError());
+  return MARIAN_HIP_OK;
+}
+
+// wide: many weight rows, every wave streams its own rows over the whole K
+// narrow: few weight rows, the four waves split K and reduce
+template <int MT>
+int launch_stream_mt(const GemmArgs& a, hipStream_t st, bool wide) {
+  if(wide) return launch_stream<MT, 2, 4, 1, 4>(a, st);
+  return launch_stream<MT, 1, 1, 4, (MT >= 8 ? 1 : 2)>(a, st);
+}
+
+int launch_stream_auto(const GemmArgs& a, hipStream_t st, int force_wide) {
+  const int n_tiles = (a.n_out + 15) / 16;
+  bool wide = n_tiles >= 1024;
+  if(force_wide == 1) wide = true;
+  if(force_wide == 2) wide = false;
+  if(a.M <= 16) return launch_stream_mt<1>(a, st, wide);
+  if(a.M <= 32) return launch_stream_mt<2>(a, st, wide);
+  if(a.M <= 64) return launch_stream_mt<4>(a, st, wide);
+  return launch_stream_mt<8>(a, st, wide);
+}
+
+int launch_gemm(const GemmArgs& a, hipStream_t st) {
+  const int which = g_kernel_override.load(std::memory_order_relaxed);
+  switch(which) {
+    case 101: if(a.M <= 128) return launch_stream_auto(a, st, 1); break;
+    case 102: if(a.M <= 128) return launch_stream_auto(a, st, 2); break;
+    case 201: return launch_tile<4, 4>(a, st);
+    case 202: return launch_tile<8, 4>(a, st);
+    case 203: return launch_tile<4, 8>(a, st);
+    case 204: return launch_tile<2, 2>(a, st);
+    default: break;
+  }
+  if(a.M <= 128) return launch_stream_auto(a, st, 0);
+  return launch_tile<4, 4>(a, st);
+}
+
+int check_gemm(const int8_t* Aq, const int8_t* Bq, const void* out, const float* bias,
+               const uint32_t* idx, int64_t n_idx, int64_t M, int64_t K, int64_t N) {
+  if(!Aq || !Bq || !out) return MARIAN_HIP_ERR_NULL;
+  if(M < 0 || K <= 0 || N < 0 || (K % 64) != 0 || (N % 8) != 0) return MARIAN_HIP_ERR_SHAPE;
+  if(idx && (n_idx < 0 || (n_idx % 8) != 0)) return MARIAN_HIP_ERR_SHAPE;
+  const int64_t n_out = idx ? n_idx : N;
+  if(M * K > kMaxElems || K * N > kMaxElems || M * n_out > kMaxElems) return MARIAN_HIP_ERR_RANGE;
+  if(!aligned(Aq, 16) || !aligned(Bq, 16) || !aligned(out, 16)) return MARIAN_HIP_ERR_ALIGN;
+  if((bias && !aligned(bias, 4)) || (idx && !aligned(idx, 4))) return MARIAN_HIP_ERR_ALIGN;
+  return MARIAN_HIP_OK;
+}
+
+int run_gemm(const int8_t* Aq, const int8_t* Bq, const float* bias, const uint32_t* idx,
+             int64_t n_idx, void* out, int64_t M, int64_t K, int64_t N, float scale, int relu,
+             int dump, void* stream) {
+  int st = check_gemm(Aq, Bq, out, bias, idx, n_idx, M, K, N);
+  if(st != MARIAN_HIP_OK) return st;
+  const int64_t n_out = idx ? n_idx : N;
+  if(M == 0 || n_out == 0) return MARIAN_HIP_OK;
+  GemmArgs a;
+  a.Aq = Aq; a.Bq = Bq; a.bias = bias; a.idx = idx; a.out = out;
+  a.M = (int)M; a.K = (int)K; a.N = (int)N; a.n_out = (int)n_out;
+  a.scale = scale; a.relu = relu ? 1 : 0; a.dump = dump;
+  return launch_gemm(a, reinterpret_cast<hipStream_t>(stream));
+}
+
+int absmax_blocks(size_t n4) {
+  size_t per_block = (size_t)kQuantThreads * 8;  // eight 16-byte loads per thread
+  size_t g = (n4 + per_block - 1) / per_block;
+  if(g < 1) g = 1;
+  if(g > (size_t)kMaxPartials) g = kMaxPartials;
+  return (int)g;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* marian_hip_status_string(int status) {
+  switch(status) {
+    case MARIAN_HIP_OK: return "ok";
+    case MARIAN_HIP_ERR_NULL: return "required pointer is null";
+    case MARIAN_HIP_ERR_SHAPE: return "bad shape (need K % 64 == 0, N % 8 == 0, n_idx % 8 == 0, sizes >= 0)";
+    case MARIAN_HIP_ERR_ALIGN: return "pointer alignment (16 bytes for matrices, 4 for bias/idx)";
+    case MARIAN_HIP_ERR_WORKSPACE: return "workspace too small";
+    case MARIAN_HIP_ERR_HIP: return "HIP runtime error";
+    case MARIAN_HIP_ERR_RANGE: return "tensor too large for 32-bit element indices";
+    default: return "unknown status";
+  }
+}
+
+int marian_hip_last_hip_error(void) { return g_last_hip_error; }
+
+int marian_hip_int8_abi_version(void) { return 1; }
+
+size_t marian_hip_int8_workspace_bytes(void) { return kWorkspaceBytes; }
+
+int marian_hip_int8_set_kernel(int which) { return g_kernel_override.exchange(which); }
+
+int marian_hip_int8_prepare_a(const float* A, int8_t* Aq, int64_t M, int64_t K, void* workspace,
+                              size_t workspace_bytes, void* stream) {
+  if(!A || !Aq) return MARIAN_HIP_ERR_NULL;
+  if(M < 0 || K <= 0 || (K % 64) != 0) return MARIAN_HIP_ERR_SHAPE;
+  if(M * K > kMaxElems) return MARIAN_HIP_ERR_RANGE;
+  if(!aligned(A, 16) || !aligned(Aq, 16)) return MARIAN_HIP_ERR_ALIGN;
+  if(M == 0) return MARIAN_HIP_OK;
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  const size_t n = (size_t)M * (size_t)K;
+  if(n <= (size_t)kSingleBlockMaxElems) {
+    hipLaunchKernelGGL(prepare_a_single_block_kernel, dim3(1), dim3(kSingleBlockThreads), 0, st,
+                       A, (int)(n / 16), Aq);
+    MH_HIP(hipGetLastError());
+    return MARIAN_HIP_OK;
+  }
+  if(!workspace) return MARIAN_HIP_ERR_NULL;
+  if(workspace_bytes < kWorkspaceBytes) return MARIAN_HIP_ERR_WORKSPACE;
+  if(!aligned(workspace, 4)) return MARIAN_HIP_ERR_ALIGN;
+  float* partials = reinterpret_cast<float*>(workspace);
+  const int g = absmax_blocks(n / 4);
+  hipLaunchKernelGGL(absmax_partial_kernel, dim3(g), dim3(kQuantThreads), 0, st, A, n / 4,
+                     partials);
+  MH_HIP(hipGetLastError());
+  size_t qblocks = (n / 16 + kQuantThreads - 1) / kQuantThreads;
+  if(qblocks > 4096) qblocks = 4096;
+  hipLaunchKernelGGL(quantize_a_kernel, dim3((int)qblocks), dim3(kQuantThreads), 0, st, A, n / 16,
+                     (const float*)partials, g, Aq);
+  MH_HIP(hipGetLastError());
+  return MARIAN_HIP_OK;
+}
+
+int marian_hip_int8_prepare_b(const float* W, int8_t* Bq, int64_t K, int64_t N, void* workspace,
+                              size_t workspace_bytes, void* stream) {
+  if(!W || !Bq || !workspace) return MARIAN_HIP_ERR_NULL;
+  if(K <= 0 || N <= 0 || (K % 64) != 0 || (N % 8) != 0) return MARIAN_HIP_ERR_SHAPE;
+  if(K * N > kMaxElems) return MARIAN_HIP_ERR_RANGE;
+  if(!aligned(W, 16) || !aligned(Bq, 16) || !aligned(workspace, 4)) return MARIAN_HIP_ERR_ALIGN;
+  if(workspace_bytes < kWorkspaceBytes) return MARIAN_HIP_ERR_WORKSPACE;
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  const size_t n = (size_t)K * (size_t)N;
+  float* partials = reinterpret_cast<float*>(workspace);
+  const int g = absmax_blocks(n / 4);
+  hipLaunchKernelGGL(absmax_partial_kernel, dim3(g), dim3(kQuantThreads), 0, st, W, n / 4,
+                     partials);
+  MH_HIP(hipGetLastError());
+  dim3 grid((unsigned)((N + 63) / 64), (unsigned)(K / 64));
+  hipLaunchKernelGGL(quantize_b_transpose_kernel, grid, dim3(256), 0, st, W, (int)K, (int)N,
+                     (const float*)partials, g, Bq);
+  MH_HIP(hipGetLastError());
+  return MARIAN_HIP_OK;
+}
+
+int marian_hip_int8_prepare_b_quantized_transposed(const int8_t* in, int8_t* out, int64_t K,
+                                                   int64_t N, void* stream) {
+  if(!in || !out) return MARIAN_HIP_ERR_NULL;
+  if(K <= 0 || N <= 0) return MARIAN_HIP_ERR_SHAPE;
+  if(in == out) return MARIAN_HIP_OK;
+  MH_HIP(hipMemcpyAsync(out, in, (size_t)K * (size_t)N + sizeof(float), hipMemcpyDeviceToDevice,
+                        reinterpret_cast<hipStream_t>(stream)));
+  return MARIAN_HIP_OK;
+}
+
+int marian_hip_int8_affine(const int8_t* Aq, const int8_t* Bq, const float* bias, float* out,
+                           int64_t M, int64_t K, int64_t N, float scale, int relu, void* stream) {
+  return run_gemm(Aq, Bq, bias, nullptr, 0, out, M, K, N, scale, relu, 0, stream);
+}
+
+int marian_hip_int8_affine_shortlist(const int8_t* Aq, const int8_t* Bq, const float* bias,
+                                     const uint32_t* idx, int64_t n_idx, float* out, int64_t M,
+                                     int64_t K, int64_t N, float scale, int relu, void* stream) {
+  if(!idx) return MARIAN_HIP_ERR_NULL;
+  return run_gemm(Aq, Bq, bias, idx, n_idx, out, M, K, N, scale, relu, 0, stream);
+}
+
+int marian_hip_int8_multiply_i32(const int8_t* Aq, const int8_t* Bq, const uint32_t* idx,
+                                 int64_t n_idx, int32_t* acc, int64_t M, int64_t K, int64_t N,
+                                 void* stream) {
+  return run_gemm(Aq, Bq, nullptr, idx, idx ? n_idx : 0, acc, M, K, N, 1.0f, 0, 1, stream);
+}
+
+}  // extern "C"

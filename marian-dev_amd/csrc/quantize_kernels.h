@@ -1,0 +1,161 @@
+// abs-max + int8 quantize kernels (activation prepareA and offline weight prepareB).
+#pragma once
+
+#include "int8_common.h"
+
+namespace marian_hip {
+
+constexpr int kQuantThreads = 256;
+constexpr int kMaxPartials = 1024;                  // floats of workspace used
+constexpr size_t kWorkspaceBytes = kMaxPartials * sizeof(float);
+constexpr int kSingleBlockThreads = 1024;
+constexpr int kSingleBlockMaxElems = 64 * 1024;     // one workgroup does abs-max and quantize
+
+// q = clamp(rne(fl32(x * qm)), -127, 127); products that are NaN or outside int32 give -127
+// (x86 cvtps2dq integer-indefinite followed by saturating packs and max(-127)).
+__device__ __forceinline__ int quantize_one(float x, float qm) {
+  float v = x * qm;
+  float r = __builtin_rintf(v);
+  r = fminf(fmaxf(r, -127.0f), 127.0f);
+  int q = (int)r;
+  return (fabsf(v) < 2147483648.0f) ? q : -127;
+}
+
+__device__ __forceinline__ uint32_t quantize_pack4(v4f x, float qm) {
+  uint32_t b0 = (uint32_t)quantize_one(x.x, qm) & 0xffu;
+  uint32_t b1 = (uint32_t)quantize_one(x.y, qm) & 0xffu;
+  uint32_t b2 = (uint32_t)quantize_one(x.z, qm) & 0xffu;
+  uint32_t b3 = (uint32_t)quantize_one(x.w, qm) & 0xffu;
+  return b0 | (b1 << 8) | (b2 << 16) | (b3 << 24);
+}
+
+__device__ __forceinline__ float abs4max(v4f x, float m) {
+  m = fmaxf(m, fabsf(x.x));
+  m = fmaxf(m, fabsf(x.y));
+  m = fmaxf(m, fabsf(x.z));
+  m = fmaxf(m, fabsf(x.w));
+  return m;
+}
+
+__device__ __forceinline__ float wave_max(float m) {
+#pragma unroll
+  for(int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+  return m;
+}
+
+// Max over the workgroup; every thread returns the result.  red: >= blockDim/64 floats of LDS.
+__device__ __forceinline__ float block_max(float m, float* red) {
+  m = wave_max(m);
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  const int nw = blockDim.x / kWave;
+  __syncthreads();
+  if(lane == 0) red[wave] = m;
+  __syncthreads();
+  float r = (lane < nw) ? red[lane] : 0.0f;
+  return wave_max(r);
+}
+
+// quantMult = 127.0f / maxabs as one correctly rounded fp32 division (via double).
+__device__ __forceinline__ float quant_mult_from_maxabs(float maxabs) {
+  return (float)(127.0 / (double)maxabs);
+}
+
+// Pass 1: per-workgroup abs-max of n floats (n % 4 == 0) -> partials[blockIdx.x].
+__global__ __launch_bounds__(kQuantThreads) void absmax_partial_kernel(
+    const float* __restrict__ x, size_t n4, float* __restrict__ partials) {
+  __shared__ float red[kQuantThreads / kWave];
+  const v4f* x4 = reinterpret_cast<const v4f*>(x);
+  float m = 0.0f;
+  size_t stride = (size_t)gridDim.x * blockDim.x;
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  // four independent loads in flight per thread
+  for(; i + 3 * stride < n4; i += 4 * stride) {
+    v4f a = x4[i], b = x4[i + stride], c = x4[i + 2 * stride], d = x4[i + 3 * stride];
+    m = abs4max(a, m); m = abs4max(b, m); m = abs4max(c, m); m = abs4max(d, m);
+  }
+  for(; i < n4; i += stride) m = abs4max(x4[i], m);
+  m = block_max(m, red);
+  if(threadIdx.x == 0) partials[blockIdx.x] = m;
+}
+
+// Pass 2 of prepareA: reduce the partials, quantize 16 values per thread per step, block 0
+// writes the quantMult tail at byte n.
+__global__ __launch_bounds__(kQuantThreads) void quantize_a_kernel(
+    const float* __restrict__ x, size_t n16, const float* __restrict__ partials, int n_partials,
+    int8_t* __restrict__ out) {
+  __shared__ float red[kQuantThreads / kWave];
+  float m = 0.0f;
+  for(int p = threadIdx.x; p < n_partials; p += blockDim.x) m = fmaxf(m, partials[p]);
+  m = block_max(m, red);
+  const float qm = quant_mult_from_maxabs(m);
+  const v4f* x4 = reinterpret_cast<const v4f*>(x);
+  uint4* o16 = reinterpret_cast<uint4*>(out);
+  size_t stride = (size_t)gridDim.x * blockDim.x;
+  for(size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += stride) {
+    v4f a = x4[4 * i], b = x4[4 * i + 1], c = x4[4 * i + 2], d = x4[4 * i + 3];
+    uint4 q;
+    q.x = quantize_pack4(a, qm);
+    q.y = quantize_pack4(b, qm);
+    q.z = quantize_pack4(c, qm);
+    q.w = quantize_pack4(d, qm);
+    o16[i] = q;
+  }
+  if(blockIdx.x == 0 && threadIdx.x == 0) *reinterpret_cast<float*>(out + n16 * 16) = qm;
+}
+
+// Small activations: one workgroup computes abs-max and quantizes (one launch instead of two).
+__global__ __launch_bounds__(kSingleBlockThreads) void prepare_a_single_block_kernel(
+    const float* __restrict__ x, int n16, int8_t* __restrict__ out) {
+  __shared__ float red[kSingleBlockThreads / kWave];
+  const v4f* x4 = reinterpret_cast<const v4f*>(x);
+  float m = 0.0f;
+  for(int i = threadIdx.x; i < n16 * 4; i += blockDim.x) m = abs4max(x4[i], m);
+  m = block_max(m, red);
+  const float qm = quant_mult_from_maxabs(m);
+  uint4* o16 = reinterpret_cast<uint4*>(out);
+  for(int i = threadIdx.x; i < n16; i += blockDim.x) {
+    v4f a = x4[4 * i], b = x4[4 * i + 1], c = x4[4 * i + 2], d = x4[4 * i + 3];
+    uint4 q;
+    q.x = quantize_pack4(a, qm);
+    q.y = quantize_pack4(b, qm);
+    q.z = quantize_pack4(c, qm);
+    q.w = quantize_pack4(d, qm);
+    o16[i] = q;
+  }
+  if(threadIdx.x == 0) *reinterpret_cast<float*>(out + (size_t)n16 * 16) = qm;
+}
+
+// Pass 2 of prepareB: W fp32 [K x N] -> payload int8 [N x K] (quantized transpose) + tail.
+// A workgroup transposes a 64(k) x 64(n) tile through LDS: reads are coalesced along n,
+// writes are 16-byte runs along k.
+__global__ __launch_bounds__(256) void quantize_b_transpose_kernel(
+    const float* __restrict__ W, int K, int N, const float* __restrict__ partials,
+    int n_partials, int8_t* __restrict__ out) {
+  __shared__ float red[256 / kWave];
+  __shared__ __attribute__((aligned(16))) int8_t tile[64][64 + 16];  // [n][k], padded rows
+  float m = 0.0f;
+  for(int p = threadIdx.x; p < n_partials; p += blockDim.x) m = fmaxf(m, partials[p]);
+  m = block_max(m, red);
+  const float qm = quant_mult_from_maxabs(m);
+
+  const int n0 = blockIdx.x * 64, k0 = blockIdx.y * 64;
+  const int tn = threadIdx.x % 64, tk = threadIdx.x / 64;  // 4 k rows per pass
+#pragma unroll 4
+  for(int kk = tk; kk < 64; kk += 4) {
+    int k = k0 + kk, n = n0 + tn;
+    float v = (k < K && n < N) ? W[(size_t)k * N + n] : 0.0f;
+    tile[tn][kk] = (int8_t)quantize_one(v, qm);
+  }
+  __syncthreads();
+  // 64 rows (n) x 64 bytes (k): 4 threads per row, 16 bytes each
+  const int rn = threadIdx.x / 4, ck = (threadIdx.x % 4) * 16;
+  int n = n0 + rn, k = k0 + ck;
+  if(n < N && k < K) {  // K % 64 == 0, so a 16-byte run is inside or outside as a whole
+    uint4 v = *reinterpret_cast<const uint4*>(&tile[rn][ck]);
+    *reinterpret_cast<uint4*>(out + (size_t)n * K + k) = v;
+  }
+  if(blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0)
+    *reinterpret_cast<float*>(out + (size_t)K * N) = qm;
+}
+
+}  // namespace marian_hip

@@ -1,0 +1,242 @@
+"""Host mirror of Marian's intgemm operator glue, running on the HIP library.
+
+Mirrors, name for name:
+  reference src/tensors/cpu/intgemm_interface.h   prepareA, affineOrDotTyped, affineOrDot
+  reference src/tensors/cpu/integer_common.h      cols, rows, getQuantMult, computeQuantMult
+  reference src/graph/expression_operators.cpp    dot (:554-619), affine (:647-718),
+                                                  affineWithReluDropout (:721-731)
+  reference src/tensors/cpu/expression_graph_packable.h:153-253  (prepareB = offline packer)
+
+Tensors are torch tensors on the GPU (device memory and streams only); every arithmetic step
+is a call into the C ABI.  Quantized tensors are `QTensor`: a flat int8 buffer holding the
+payload plus the fp32 quantMult tail, with Marian's logical shape and element type.
+"""
+import numpy as np
+import torch
+
+from . import _lib
+from .types import Type, elements, isFloat, isHardwareSpecific, isIntgemm, requiredBytes, sizeOf
+
+MarianRuntimeError = _lib.MarianHipError
+
+
+def _abort_if(cond, msg, *args):
+    if cond:
+        raise MarianRuntimeError(-2, msg.format(*args))
+
+
+def _align256(n):
+    return (n + 255) // 256 * 256
+
+
+class QTensor:
+    """An intgemm-typed tensor: Marian allocates requiredBytes(shape, type) rounded up to 256
+    bytes (reference src/tensors/allocator.h:86,178-181); `shape` is the logical shape
+    ([.., K] for activations, [K, N] for weights whose payload is the transposed [N, K])."""
+
+    def __init__(self, data, shape, type_):
+        self.data = data
+        self.shape = tuple(int(d) for d in shape)
+        self.type = type_
+
+    @staticmethod
+    def empty(shape, type_, device):
+        nbytes = _align256(requiredBytes(shape, type_))
+        return QTensor(torch.zeros(nbytes, dtype=torch.int8, device=device), shape, type_)
+
+    @staticmethod
+    def from_numpy(flat_int8, shape, type_, device):
+        """Upload payload+tail bytes (e.g. a Type::intgemm8 item of a .bin file) verbatim."""
+        q = QTensor.empty(shape, type_, device)
+        src = torch.from_numpy(np.ascontiguousarray(flat_int8).view(np.int8))
+        n = min(src.numel(), q.data.numel())
+        q.data[:n].copy_(src[:n])
+        return q
+
+    def value_type(self):
+        return self.type
+
+    def elements(self):
+        return elements(self.shape)
+
+    def payload(self):
+        return self.data[: self.elements()]
+
+    def numpy(self):
+        """payload + tail as host bytes (elements + 4)."""
+        return self.data[: self.elements() + 4].cpu().numpy()
+
+    def data_ptr(self):
+        return self.data.data_ptr()
+
+
+def cols(t):
+    """reference src/tensors/cpu/integer_common.h:48"""
+    return int(t.shape[-1])
+
+
+def rows(t):
+    """reference src/tensors/cpu/integer_common.h:49"""
+    return elements(t.shape) // cols(t)
+
+
+def getQuantMult(q):
+    """reference src/tensors/cpu/integer_common.h:101-111 (device read; for tests and tools)."""
+    _abort_if(not isIntgemm(q.type), "getQuantMult does not work for type {}", q.type)
+    n = q.elements()
+    return float(q.data[n:n + 4].cpu().numpy().view(np.float32)[0])
+
+
+class Backend:
+    """Per-device state the path needs: a stream and the abs-max workspace, the counterpart of
+    gpu::Backend (reference src/tensors/gpu/backend.h:23-110) reduced to this path."""
+
+    _instances = {}
+
+    def __init__(self, device):
+        self.device = torch.device(device)
+        self.lib = _lib.lib()
+        self.workspace_bytes = int(self.lib.marian_hip_int8_workspace_bytes())
+        self.workspace = torch.empty(self.workspace_bytes, dtype=torch.uint8, device=self.device)
+
+    @classmethod
+    def get(cls, device):
+        device = torch.device(device)
+        key = (device.type, device.index if device.index is not None else torch.cuda.current_device())
+        if key not in cls._instances:
+            cls._instances[key] = Backend(device)
+        return cls._instances[key]
+
+    def stream(self):
+        return torch.cuda.current_stream(self.device).cuda_stream
+
+    def synchronize(self):
+        torch.cuda.current_stream(self.device).synchronize()
+
+
+def _backend_of(t):
+    dev = t.device if isinstance(t, torch.Tensor) else t.data.device
+    _abort_if(dev.type != "cuda", "the HIP int8 backend needs device tensors, got {}", dev)
+    return Backend.get(dev)
+
+
+def prepareA(a):
+    """reference src/tensors/cpu/intgemm_interface.h:17-32 for vtype = intgemm8."""
+    _abort_if(a.dtype != torch.float32, "Intgemm expects type of A to be float32 not {}", a.dtype)
+    a = a.contiguous()
+    be = _backend_of(a)
+    out = QTensor.empty(a.shape, Type.intgemm8, a.device)
+    K = cols(a)
+    M = rows(a) if a.numel() else 0
+    st = be.lib.marian_hip_int8_prepare_a(a.data_ptr(), out.data_ptr(), M, K,
+                                          be.workspace.data_ptr(), be.workspace_bytes, be.stream())
+    _lib.check(st, "prepareA")
+    return out
+
+
+def prepareB(w, type_=Type.intgemm8):
+    """Offline weight quantizer, reference src/tensors/cpu/expression_graph_packable.h:153-253
+    (intgemm8 branch): fp32 W [K, N] -> Type::intgemm8 tensor of shape [K, N] whose payload is
+    the quantized transpose."""
+    _abort_if(type_ != Type.intgemm8, "Type {} is not supported", type_)
+    _abort_if(w.dtype != torch.float32 or w.dim() != 2, "prepareB expects a float32 matrix, got {}", w.dtype)
+    w = w.contiguous()
+    be = _backend_of(w)
+    K, N = w.shape
+    out = QTensor.empty((K, N), Type.intgemm8, w.device)
+    st = be.lib.marian_hip_int8_prepare_b(w.data_ptr(), out.data_ptr(), K, N,
+                                          be.workspace.data_ptr(), be.workspace_bytes, be.stream())
+    _lib.check(st, "prepareB")
+    return out
+
+
+def affineOrDot(a, bQuant, bias=None, transA=False, transB=False, scale=1.0, relu=False,
+                shortlist=None):
+    """reference src/tensors/cpu/intgemm_interface.h:46-99,102-128.
+
+    a: float32 activations; bQuant: QTensor of type intgemm8 with logical shape [K, N].
+    transB is ignored like in the reference (:47).  `relu` fuses the in-place ReLU node the
+    reference appends (src/graph/expression_operators.cpp:721-731).  `shortlist`: optional
+    uint32 device tensor of sorted unique output ids (multiple of 8 many)."""
+    _abort_if(not isinstance(a, torch.Tensor) or not a.dtype.is_floating_point or a.dtype != torch.float32,
+              "Intgemm expects type of A to be float32 not {}", getattr(a, "dtype", type(a)))
+    _abort_if(not isinstance(bQuant, QTensor) or not isIntgemm(bQuant.type),
+              "Intgemm expects type of B to be a variant of intgemm not {}",
+              getattr(bQuant, "type", type(bQuant)))
+    _abort_if(isHardwareSpecific(bQuant.type) or sizeOf(bQuant.type) != 1,
+              "Unsupported type {} for Intgemm type??", bQuant.type)
+    if transA:
+        a = a.transpose(-1, -2)
+    aQuant = prepareA(a)
+    return multiply(aQuant, bQuant, bias, scale=scale, relu=relu, shortlist=shortlist)
+
+
+def multiply(aQuant, bQuant, bias=None, scale=1.0, relu=False, shortlist=None):
+    """The multiply node of reference src/tensors/cpu/intgemm_interface.h:60-94."""
+    be = _backend_of(aQuant)
+    K, N = cols(aQuant), cols(bQuant)
+    _abort_if(rows(bQuant) != K, "Matrix product requires inner dimensions to match: {} vs {}", K, rows(bQuant))
+    M = rows(aQuant) if aQuant.elements() else 0
+    n_out = N if shortlist is None else int(shortlist.numel())
+    out = torch.empty(aQuant.shape[:-1] + (n_out,), dtype=torch.float32, device=aQuant.data.device)
+    bias_ptr = None
+    if bias is not None:
+        _abort_if(bias.dtype != torch.float32 or bias.numel() != N, "bias must be float32 [1, {}]", N)
+        bias = bias.contiguous()
+        bias_ptr = bias.data_ptr()
+    if shortlist is None:
+        st = be.lib.marian_hip_int8_affine(aQuant.data_ptr(), bQuant.data_ptr(), bias_ptr,
+                                           out.data_ptr(), M, K, N, scale, int(relu), be.stream())
+    else:
+        _abort_if(shortlist.dtype not in (torch.int32, torch.uint32), "shortlist ids must be uint32, got {}", shortlist.dtype)
+        st = be.lib.marian_hip_int8_affine_shortlist(aQuant.data_ptr(), bQuant.data_ptr(), bias_ptr,
+                                                     shortlist.data_ptr(), n_out, out.data_ptr(),
+                                                     M, K, N, scale, int(relu), be.stream())
+    _lib.check(st, "affineOrDot")
+    return out
+
+
+def multiply_i32(aQuant, bQuant, shortlist=None):
+    """int32 accumulators of the multiply (what Kernels8::Multiply hands to its callback)."""
+    be = _backend_of(aQuant)
+    K, N = cols(aQuant), cols(bQuant)
+    M = rows(aQuant) if aQuant.elements() else 0
+    n_out = N if shortlist is None else int(shortlist.numel())
+    acc = torch.empty(aQuant.shape[:-1] + (n_out,), dtype=torch.int32, device=aQuant.data.device)
+    st = be.lib.marian_hip_int8_multiply_i32(aQuant.data_ptr(), bQuant.data_ptr(),
+                                             None if shortlist is None else shortlist.data_ptr(),
+                                             n_out if shortlist is not None else 0, acc.data_ptr(),
+                                             M, K, N, be.stream())
+    _lib.check(st, "multiply_i32")
+    return acc
+
+
+# ---- graph-operator surface (reference src/graph/expression_operators.cpp) --------------------
+
+def _float_b_unsupported(b):
+    raise MarianRuntimeError(
+        -2, "GPU-based GEMM only supports float types in the reference; this backend implements "
+        "the intgemm8 weight path only, got B of type {}".format(getattr(b, "dtype", type(b))))
+
+
+def dot(a, b, transA=False, transB=False, scale=1.0):
+    """reference src/graph/expression_operators.cpp:554-619: isIntgemm(b) selects the int8 path."""
+    if isinstance(b, QTensor) and isIntgemm(b.type):
+        return affineOrDot(a, b, None, transA, transB, scale)
+    _float_b_unsupported(b)
+
+
+def affine(a, b, bias, transA=False, transB=False, scale=1.0):
+    """reference src/graph/expression_operators.cpp:647-718."""
+    if isinstance(b, QTensor) and isIntgemm(b.type):
+        return affineOrDot(a, b, bias, transA, transB, scale)
+    _float_b_unsupported(b)
+
+
+def affineWithReluDropout(x, W, bias, dropProb=0.0):
+    """reference src/graph/expression_operators.cpp:721-731 at inference (dropProb == 0): the
+    reference runs affine() and then an in-place ReLU node; here the ReLU is the GEMM epilogue."""
+    _abort_if(dropProb != 0.0, "dropout is a training feature; inference path expects dropProb == 0, got {}", dropProb)
+    if isinstance(W, QTensor) and isIntgemm(W.type):
+        return affineOrDot(x, W, bias, False, False, 1.0, relu=True)
+    _float_b_unsupported(W)

@@ -1,0 +1,78 @@
+"""The C-ABI library loads and exports every symbol include/marian_hip_int8.h declares; argument
+validation (which runs before any HIP call) behaves as documented.  No compute without a GPU."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from conftest import ROOT, load
+
+HEADER = os.path.join(ROOT, "include", "marian_hip_int8.h")
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(marian_hip_\w+)\s*\(", text)))
+
+
+def test_header_declares_expected_entry_points():
+    names = declared_functions()
+    for must in ("marian_hip_int8_prepare_a", "marian_hip_int8_prepare_b",
+                 "marian_hip_int8_prepare_b_quantized_transposed", "marian_hip_int8_affine",
+                 "marian_hip_int8_affine_shortlist", "marian_hip_int8_multiply_i32"):
+        assert must in names
+
+
+def test_library_exports_every_declared_symbol():
+    L = load("_lib")
+    assert os.path.exists(L.LIB_PATH), "build the library first (__graft_entry__.build())"
+    lib = ctypes.CDLL(L.LIB_PATH)
+    for name in declared_functions():
+        assert hasattr(lib, name), name
+    # and the Python binding covers the same set
+    assert sorted(L.SIGNATURES) == declared_functions()
+
+
+def test_status_strings_and_version():
+    L = load("_lib")
+    lib = L.lib()
+    assert lib.marian_hip_int8_abi_version() == 1
+    assert lib.marian_hip_int8_workspace_bytes() >= 4096
+    seen = {lib.marian_hip_status_string(i) for i in range(7)}
+    assert len(seen) == 7 and lib.marian_hip_status_string(0) == b"ok"
+
+
+def test_argument_validation_returns_codes_not_aborts():
+    L = load("_lib")
+    lib = L.lib()
+    buf = 0x1000  # never dereferenced: every call below is rejected or a no-op before launch
+    assert lib.marian_hip_int8_affine(None, buf, None, buf, 1, 64, 8, 1.0, 0, None) == L.ERR_NULL
+    assert lib.marian_hip_int8_affine(buf, buf, None, buf, 1, 63, 8, 1.0, 0, None) == L.ERR_SHAPE
+    assert lib.marian_hip_int8_affine(buf, buf, None, buf, 1, 64, 12, 1.0, 0, None) == L.ERR_SHAPE
+    assert lib.marian_hip_int8_affine(buf, buf, None, buf, -1, 64, 8, 1.0, 0, None) == L.ERR_SHAPE
+    assert lib.marian_hip_int8_affine(buf + 4, buf, None, buf, 1, 64, 8, 1.0, 0, None) == L.ERR_ALIGN
+    assert lib.marian_hip_int8_affine(buf, buf, buf + 2, buf, 1, 64, 8, 1.0, 0, None) == L.ERR_ALIGN
+    assert lib.marian_hip_int8_affine(buf, buf, None, buf, 1 << 26, 64, 8, 1.0, 0, None) == L.ERR_RANGE
+    assert lib.marian_hip_int8_affine(buf, buf, None, buf, 0, 64, 8, 1.0, 0, None) == L.OK  # empty batch
+    assert lib.marian_hip_int8_affine_shortlist(buf, buf, None, None, 8, buf, 1, 64, 8, 1.0, 0, None) == L.ERR_NULL
+    assert lib.marian_hip_int8_affine_shortlist(buf, buf, None, buf, 12, buf, 1, 64, 8, 1.0, 0, None) == L.ERR_SHAPE
+    assert lib.marian_hip_int8_prepare_a(buf, buf, 4, 100, buf, 4096, None) == L.ERR_SHAPE
+    assert lib.marian_hip_int8_prepare_a(buf, buf, 4096, 1024, buf, 16, None) == L.ERR_WORKSPACE
+    assert lib.marian_hip_int8_prepare_a(buf, buf, 0, 64, None, 0, None) == L.OK
+    assert lib.marian_hip_int8_prepare_b(buf, buf, 64, 8, None, 4096, None) == L.ERR_NULL
+    with pytest.raises(L.MarianHipError):
+        L.check(L.ERR_SHAPE, "test")
+
+
+def test_types_match_marian_enum():
+    T = load("types")
+    # reference src/common/types.h:282,317-323 and src/common/types.cpp:32-34
+    assert int(T.Type.intgemm8) == 0x10000 + 1
+    assert int(T.Type.intgemm8avx512vnni) == 0x10000 + 1 + 0x2000 + 4096
+    assert int(T.Type.float32) == 0x400 + 4
+    assert T.isIntgemm(T.Type.intgemm8) and not T.isIntgemm(T.Type.float32)
+    assert T.isHardwareSpecific(T.Type.intgemm8avx2) and not T.isHardwareSpecific(T.Type.intgemm8)
+    assert T.requiredBytes((512, 2048), T.Type.intgemm8) == 512 * 2048 + 4
+    assert T.requiredBytes((512, 2048), T.Type.float32) == 512 * 2048 * 4

@@ -1,0 +1,336 @@
+"""GPU parity: the HIP path (through the C ABI) against the CPU checker on the same seeded inputs.
+
+Bars: quantized operands, quantMult tails and int32 accumulators bit-exact; fp32 outputs within
+1e-5 relative (plus an absolute floor of 1e-6 * unquant * K * 127 that absorbs cancellation
+against the bias).  The kernels keep multiply and bias add as separate roundings, so the fp32
+outputs are in fact expected to be bit-identical; that stricter check is asserted too.
+"""
+import os
+import sys
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+f32 = np.float32
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "intgemm8_small.npz")
+REL_TOL = 1e-5
+
+
+def say(*a):
+    print(*a, flush=True)
+    sys.stdout.flush()
+
+
+def dev(x):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(x)).cuda()
+
+
+def upload_q(integer, flat, shape):
+    from conftest import load
+    T = load("types")
+    return integer.QTensor.from_numpy(flat, shape, T.Type.intgemm8, "cuda")
+
+
+def assert_close_fp32(got, want, unquant, K):
+    floor = 1e-6 * abs(float(unquant)) * K * 127
+    err = np.abs(got.astype(np.float64) - want.astype(np.float64))
+    bound = REL_TOL * np.abs(want.astype(np.float64)) + floor
+    bad = err > bound
+    assert not bad.any(), "max rel err %g at %s" % (float((err / (np.abs(want) + floor)).max()),
+                                                     np.argwhere(bad)[:4].tolist())
+
+
+def inputs(synth, seed, M, K, N):
+    A = synth.normal(seed, synth.STREAM_A, (M, K), 1.0)
+    W = synth.normal(seed, synth.STREAM_W, (K, N), 0.02)
+    bias = synth.normal(seed, synth.STREAM_BIAS, (N,), 0.01)
+    return A, W, bias
+
+
+# ---------------------------------------------------------------- prepareA / prepareB
+
+@pytest.mark.parametrize("M,K", [(1, 64), (1, 512), (3, 128), (16, 512), (64, 512), (100, 448),
+                                 (128, 1024), (257, 320), (1000, 1024), (4096, 1024)])
+def test_prepare_a_bit_exact(integer, orc, synth, M, K):
+    say("prepare_a", M, K)
+    A = synth.normal(100 + M, synth.STREAM_A, (M, K), 1.0)
+    want = orc.prepare_a(A)
+    got = integer.prepareA(dev(A)).numpy()
+    assert np.array_equal(got[-4:].view(f32), want[-4:].view(f32)), "quantMult tail"
+    assert np.array_equal(got, want)
+
+
+def test_prepare_a_keeps_leading_dims_and_saturates(integer, orc):
+    say("prepare_a 4-d")
+    rng = np.random.default_rng(5)
+    A = rng.standard_normal((2, 3, 5, 64)).astype(f32)
+    A[1, 2, 4, 63] = -77.25   # arg-max is negative and sits in the last element
+    q = integer.prepareA(dev(A))
+    assert q.shape == (2, 3, 5, 64)
+    got = q.numpy()
+    assert np.array_equal(got, orc.prepare_a(A))
+    assert got[30 * 64 - 1] == -127 and got[:-4].min() == -127
+
+
+@pytest.mark.parametrize("K,N", [(64, 8), (128, 24), (512, 2048), (2048, 512), (1024, 1000)])
+def test_prepare_b_bit_exact(integer, orc, synth, K, N):
+    say("prepare_b", K, N)
+    W = synth.normal(200 + N, synth.STREAM_W, (K, N), 0.02)
+    want = orc.prepare_b(W)
+    q = integer.prepareB(dev(W))
+    assert q.shape == (K, N)
+    assert np.array_equal(q.numpy(), want)
+
+
+# ---------------------------------------------------------------- multiply: int32 and fp32
+
+KERNELS = [0, 101, 102, 201, 202, 203, 204]
+
+
+def run_case(integer, orc, synth, seed, M, K, N, kernel, bias_on=True, relu=False, scale=1.0):
+    from conftest import load
+    lib = load("_lib").lib()
+    A, W, bias = inputs(synth, seed, M, K, N)
+    Aq_h, Bq_h = orc.prepare_a(A), orc.prepare_b(W)
+    want_out, want_acc = orc.affine(Aq_h, Bq_h, bias if bias_on else None, M, K, N, scale, relu)
+    Aq, Bq = upload_q(integer, Aq_h, (M, K)), upload_q(integer, Bq_h, (K, N))
+    prev = lib.marian_hip_int8_set_kernel(kernel)
+    try:
+        acc = integer.multiply_i32(Aq, Bq).cpu().numpy()
+        out = integer.multiply(Aq, Bq, dev(bias) if bias_on else None, scale=scale, relu=relu).cpu().numpy()
+    finally:
+        lib.marian_hip_int8_set_kernel(prev)
+    assert np.array_equal(acc, want_acc), "int32 accumulators differ (kernel %d)" % kernel
+    unquant = orc.unquant_mult(orc.tail(Aq_h, M * K), orc.tail(Bq_h, K * N), scale)
+    assert_close_fp32(out, want_out, unquant, K)
+    assert np.array_equal(out, want_out), "fp32 outputs not bit-identical (kernel %d)" % kernel
+
+
+@pytest.mark.parametrize("kernel", KERNELS)
+@pytest.mark.parametrize("M,K,N", [(1, 64, 8), (5, 128, 24), (16, 512, 512), (33, 192, 136),
+                                   (64, 512, 2048), (128, 1024, 1024), (100, 2048, 512)])
+def test_multiply_all_kernels_small_m(integer, orc, synth, M, K, N, kernel):
+    say("multiply", M, K, N, "kernel", kernel)
+    run_case(integer, orc, synth, 300 + M + N, M, K, N, kernel, bias_on=True, relu=(M % 2 == 0))
+
+
+@pytest.mark.parametrize("kernel", [0, 201, 202, 203, 204])
+@pytest.mark.parametrize("M,K,N", [(129, 64, 8), (256, 1024, 504), (300, 320, 1000), (513, 128, 264)])
+def test_multiply_tile_kernels_ragged(integer, orc, synth, M, K, N, kernel):
+    say("multiply ragged", M, K, N, "kernel", kernel)
+    run_case(integer, orc, synth, 400 + M + N, M, K, N, kernel, bias_on=(N % 16 == 8), relu=True,
+             scale=0.5)
+
+
+def test_config1_single_affine_end_to_end(integer, orc, synth):
+    """BASELINE config 1: A[64x512] ~ N(0,1), W[512x2048] ~ N(0,0.02^2), bias ~ N(0,0.01^2), ReLU."""
+    say("config1")
+    M, K, N = 64, 512, 2048
+    A, W, bias = inputs(synth, 1001, M, K, N)
+    Bq_h = orc.prepare_b(W)
+    Aq_h = orc.prepare_a(A)
+    want, want_acc = orc.affine(Aq_h, Bq_h, bias, M, K, N, 1.0, True)
+    Bq = integer.prepareB(dev(W))                       # offline quantizer on the GPU
+    assert np.array_equal(Bq.numpy(), Bq_h)
+    Aq = integer.prepareA(dev(A))
+    assert np.array_equal(Aq.numpy(), Aq_h)
+    assert np.array_equal(integer.multiply_i32(Aq, Bq).cpu().numpy(), want_acc)
+    got = integer.affineWithReluDropout(dev(A), Bq, dev(bias)).cpu().numpy()
+    unquant = orc.unquant_mult(orc.tail(Aq_h, M * K), orc.tail(Bq_h, K * N), 1.0)
+    assert_close_fp32(got, want, unquant, K)
+    assert np.array_equal(got, want)
+    assert (got == 0).mean() > 0.2 and (got > 0).mean() > 0.2   # ReLU really clipped something
+
+
+@pytest.mark.parametrize("K,N", [(512, 1536), (512, 512), (512, 2048), (2048, 512), (512, 32000)])
+@pytest.mark.parametrize("M", [1, 4, 16, 64])
+def test_config2_decode_sweep(integer, orc, synth, M, K, N):
+    """BASELINE config 2: transformer-base decode shapes."""
+    say("config2", M, K, N)
+    A, W, bias = inputs(synth, 1002, M, K, N)
+    Bq_h, Aq_h = orc.prepare_b(W), orc.prepare_a(A)
+    want, want_acc = orc.affine(Aq_h, Bq_h, bias, M, K, N)
+    Bq = upload_q(integer, Bq_h, (K, N))
+    Aq = integer.prepareA(dev(A))
+    assert np.array_equal(Aq.numpy(), Aq_h)
+    assert np.array_equal(integer.multiply_i32(Aq, Bq).cpu().numpy(), want_acc)
+    got = integer.affine(dev(A), Bq, dev(bias)).cpu().numpy()
+    assert np.array_equal(got, want)
+
+
+def test_config3_transformer_big_step_shapes(integer, orc, synth):
+    """BASELINE config 3 GEMM shapes at M = 128 (beam 4 x batch 32), d = 1024, ffn = 4096."""
+    M = 128
+    for K, N, relu in [(1024, 1024, False), (1024, 4096, True), (4096, 1024, False)]:
+        say("config3", M, K, N)
+        A, W, bias = inputs(synth, 1003, M, K, N)
+        Bq_h, Aq_h = orc.prepare_b(W), orc.prepare_a(A)
+        want, want_acc = orc.affine(Aq_h, Bq_h, bias, M, K, N, 1.0, relu)
+        Bq = upload_q(integer, Bq_h, (K, N))
+        Aq = integer.prepareA(dev(A))
+        assert np.array_equal(Aq.numpy(), Aq_h)
+        assert np.array_equal(integer.multiply_i32(Aq, Bq).cpu().numpy(), want_acc)
+        got = integer.multiply(Aq, Bq, dev(bias), relu=relu).cpu().numpy()
+        assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("K,N", [(1024, 4096), (4096, 1024)])
+def test_config4_large_m_full_size(integer, orc, synth, K, N):
+    """BASELINE config 4 at full size (M = 4096).  The checker runs on 96 sampled rows (rows are
+    independent once A is quantized); the rest is covered by a column-sum identity in int64:
+    sum_m acc[m, n] == (sum_m Aq[m, :]) . Bt[n, :]."""
+    M = 4096
+    say("config4", M, K, N)
+    A, W, bias = inputs(synth, 1004, M, K, N)
+    Bq_h, Aq_h = orc.prepare_b(W), orc.prepare_a(A)
+    Bq = upload_q(integer, Bq_h, (K, N))
+    Aq = integer.prepareA(dev(A))
+    assert np.array_equal(Aq.numpy(), Aq_h)
+    acc = integer.multiply_i32(Aq, Bq).cpu().numpy()
+    got = integer.affineWithReluDropout(dev(A), Bq, dev(bias)).cpu().numpy()
+    rows = np.unique(np.concatenate([[0, 1, 15, 16, 127, 128, 255, 256, M - 1],
+                                     np.random.default_rng(4).integers(0, M, 87)]))
+    sub = np.concatenate([Aq_h[:M * K].reshape(M, K)[rows].ravel(), Aq_h[M * K:]])
+    want, want_acc = orc.affine(sub, Bq_h, bias, len(rows), K, N, 1.0, True)
+    assert np.array_equal(acc[rows], want_acc)
+    assert np.array_equal(got[rows], want)
+    colsum = Aq_h[:M * K].reshape(M, K).astype(np.int64).sum(0)
+    Bt = Bq_h[:K * N].reshape(N, K).astype(np.int64)
+    assert np.array_equal(acc.astype(np.int64).sum(0), Bt @ colsum)
+    # the fp32 output is the deterministic image of acc: recompute it everywhere in numpy
+    u = orc.unquant_mult(orc.tail(Aq_h, M * K), orc.tail(Bq_h, K * N), 1.0)
+    y = ((acc.astype(f32) * u).astype(f32) + bias[None, :]).astype(f32)
+    assert np.array_equal(got, np.where(y > 0, y, f32(0)))
+
+
+# ---------------------------------------------------------------- shortlist
+
+@pytest.mark.parametrize("M", [4, 64, 256])
+def test_config5_shortlist(integer, orc, synth, M):
+    """BASELINE config 5: W int8 [32000 x 1024], shortlist of 500-2000 sorted unique ids.
+    gather-GEMM == column pick of the dense GEMM, bit-exactly, and matches the checker."""
+    import torch
+    K, N = 1024, 32000
+    say("config5", M)
+    A = synth.normal(1005, synth.STREAM_A, (M, K), 1.0)
+    Wt = synth.normal(1005, synth.STREAM_W, (N, K), 0.02)   # tied embedding matrix [V x D]
+    bias = synth.normal(1005, synth.STREAM_BIAS, (N,), 0.01)
+    # its int8 form is the payload of logical B = Wt^T: identical bytes, quantMult over all of it
+    bqm = orc.quant_mult(orc.max_abs(Wt))
+    Bq_h = np.concatenate([orc.quantize(Wt, bqm).ravel(), np.array([bqm], f32).view(np.int8)])
+    Aq_h = orc.prepare_a(A)
+    Bq = upload_q(integer, Bq_h, (K, N))
+    Aq = integer.prepareA(dev(A))
+    dense = integer.multiply(Aq, Bq, dev(bias)).cpu().numpy()
+    dense_acc = integer.multiply_i32(Aq, Bq).cpu().numpy()
+    for j, seed in enumerate([1005, 2005, 3005]):
+        idx = synth.shortlist(seed, N)
+        if j == 2:
+            idx = idx[:8]                                   # smallest legal shortlist
+        say("  n_idx", idx.size)
+        want, want_acc = orc.affine_shortlist(Aq_h, Bq_h, bias, idx, M, K, N)
+        didx = torch.from_numpy(idx.view(np.int32)).cuda()
+        acc = integer.multiply_i32(Aq, Bq, shortlist=didx).cpu().numpy()
+        out = integer.multiply(Aq, Bq, dev(bias), shortlist=didx).cpu().numpy()
+        assert np.array_equal(acc, want_acc) and np.array_equal(acc, dense_acc[:, idx])
+        assert np.array_equal(out, want) and np.array_equal(out, dense[:, idx])
+    # dense full-vocabulary case against the checker on a few rows
+    rows = [0, M // 2, M - 1]
+    sub = np.concatenate([Aq_h[:M * K].reshape(M, K)[rows].ravel(), Aq_h[M * K:]])
+    want, want_acc = orc.affine(sub, Bq_h, bias, len(rows), K, N)
+    assert np.array_equal(dense_acc[rows], want_acc) and np.array_equal(dense[rows], want)
+
+
+# ---------------------------------------------------------------- fixtures, contract, errors
+
+def test_golden_fixtures_on_gpu(integer):
+    g = np.load(GOLDEN)
+    for i in range(int(g["n_cases"])):
+        A, W = g["c%d_A" % i], g["c%d_W" % i]
+        M, K = A.shape
+        N = W.shape[1]
+        say("golden", i, M, K, N)
+        Bq = integer.prepareB(dev(W))
+        Aq = integer.prepareA(dev(A))
+        assert np.array_equal(Aq.numpy()[:M * K].reshape(M, K), g["c%d_Aq" % i])
+        assert np.array_equal(Bq.numpy()[:K * N].reshape(N, K), g["c%d_Bt" % i])
+        assert integer.getQuantMult(Aq) == g["c%d_aqm" % i] and integer.getQuantMult(Bq) == g["c%d_bqm" % i]
+        assert np.array_equal(integer.multiply_i32(Aq, Bq).cpu().numpy(), g["c%d_acc" % i])
+        bias = dev(g["c%d_bias" % i]) if int(g["c%d_with_bias" % i]) else None
+        out = integer.affineOrDot(dev(A), Bq, bias, scale=float(g["c%d_scale" % i]),
+                                  relu=bool(g["c%d_relu" % i])).cpu().numpy()
+        assert np.array_equal(out, g["c%d_out" % i])
+
+
+def test_marian_operator_vectors_on_gpu(integer):
+    """reference src/tests/units/operator_tests.cpp:508-534 (dot) and :618-659 (affine,
+    affineWithReluDropout, affine == dot + bias), embedded so that both quantMults are 1 and K is
+    padded with zeros to 64."""
+    say("marian operator vectors")
+    vA = np.arange(1, 13, dtype=f32).reshape(4, 3)
+
+    def embed(A, B, n_pad=8):
+        A2 = np.zeros((A.shape[0] + 1, 64), f32)
+        A2[:-1, :A.shape[1]] = A
+        A2[-1, 0] = 127
+        B2 = np.zeros((64, n_pad), f32)
+        B2[:B.shape[0], :B.shape[1]] = B
+        B2[0, n_pad - 1] = 127
+        return dev(A2), integer.prepareB(dev(B2))
+
+    a, b = embed(vA, np.array([[1, 2], [3, 4], [5, 6]], f32))
+    C = integer.dot(a.reshape(5, 1, 64), b)
+    assert tuple(C.shape) == (5, 1, 8)                      # shape = A's with last dim <- N
+    assert C.cpu().numpy().reshape(5, 8)[:4, :2].ravel().tolist() == [22, 28, 49, 64, 76, 100, 103, 136]
+
+    a, b = embed(vA, np.array([[1, -2], [3, 4], [-5, 6]], f32))
+    bias = dev(np.full(8, 2.0, f32))
+    aff = integer.affine(a, b, bias).cpu().numpy()
+    assert aff[:4, :2].ravel().tolist() == [-6, 26, -9, 50, -12, 74, -15, 98]
+    assert np.array_equal(aff, integer.dot(a, b).cpu().numpy() + 2.0)
+    rel = integer.affineWithReluDropout(a, b, bias).cpu().numpy()
+    assert rel[:4, :2].ravel().tolist() == [0, 26, 0, 50, 0, 74, 0, 98]
+    assert np.array_equal(rel, np.maximum(aff, 0))
+
+
+def test_scale_and_transA(integer, orc, synth):
+    say("scale/transA")
+    M, K, N = 24, 128, 64
+    A, W, bias = inputs(synth, 77, M, K, N)
+    Bq_h = orc.prepare_b(W)
+    Bq = upload_q(integer, Bq_h, (K, N))
+    At = dev(A.T.copy())                                    # [K, M]; transA gives back A
+    got = integer.affine(At, Bq, dev(bias), transA=True, scale=0.25).cpu().numpy()
+    want, _ = orc.affine(orc.prepare_a(A), Bq_h, bias, M, K, N, 0.25)
+    assert np.array_equal(got, want)
+
+
+def test_repeatable_and_input_untouched(integer, synth):
+    say("repeatable")
+    A, W, bias = inputs(synth, 78, 64, 512, 2048)
+    a, b = dev(A), integer.prepareB(dev(W))
+    r1 = integer.affine(a, b, dev(bias)).cpu().numpy()
+    r2 = integer.affine(a, b, dev(bias)).cpu().numpy()
+    assert np.array_equal(r1, r2) and np.array_equal(a.cpu().numpy(), A)
+
+
+def test_type_errors_like_the_reference(integer):
+    import torch
+    from conftest import load
+    T = load("types")
+    say("type errors")
+    b = integer.prepareB(torch.ones(64, 8, device="cuda"))
+    with pytest.raises(integer.MarianRuntimeError, match="Intgemm expects type of A to be float32"):
+        integer.affineOrDot(torch.ones(2, 64, device="cuda", dtype=torch.float16), b)
+    with pytest.raises(integer.MarianRuntimeError, match="Intgemm expects type of B"):
+        integer.affineOrDot(torch.ones(2, 64, device="cuda"), torch.ones(64, 8, device="cuda"))
+    tiled = integer.QTensor(b.data, b.shape, T.Type.intgemm8avx512)  # CPU-tiled payload
+    with pytest.raises(integer.MarianRuntimeError, match="Unsupported type"):
+        integer.affineOrDot(torch.ones(2, 64, device="cuda"), tiled)
+    with pytest.raises(integer.MarianRuntimeError, match="bad shape"):
+        integer.prepareA(torch.ones(2, 100, device="cuda"))
+    empty = integer.affine(torch.ones(0, 64, device="cuda"), b, None)
+    assert tuple(empty.shape) == (0, 8)
