@@ -1,0 +1,341 @@
+#!/usr/bin/env python3
+"""Benchmark of the int8 affine path (Marian intgemm8 semantics) on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+Prints ONE JSON line.  The headline workload is the transformer-base decode GEMM sweep: one
+"step" is one pass over its 20 affine calls (abs-max quantize of the fp32 activations + int8 GEMM
+with fused dequantize and bias), inputs and int8 weights resident in HBM.  Steps are replayed as
+HIP graphs so that launch overhead of the Python host does not enter the number; every step uses
+a different copy of the weights, rotating over more than 512 MB, so weights come from HBM and
+not from the 256 MB Infinity Cache.
+
+Also in the line: the roofline of the dominant kernel (per-launch duration from HIP events), the
+CPU restatement of the reference path timed on this host, and the other workloads (encoder-size
+GEMMs with their MFMA fraction, the shortlisted output layer, transformer-big decode tokens/s).
+"""
+import argparse
+import importlib
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+PKG = "marian-dev_amd"
+
+HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
+INT8_PEAK_TOPS = 5000.0      # MI355X dense int8 MFMA, published (5.0 POP/s)
+
+DECODE_SHAPES = [(512, 1536), (512, 512), (512, 2048), (2048, 512), (512, 32000)]
+DECODE_M = [1, 4, 16, 64]
+
+
+def algorithmic_bytes(M, K, n_out, with_idx=False):
+    """fp32 A read once + int8 W + fp32 bias + fp32 out (+ shortlist ids)."""
+    return 4 * M * K + K * n_out + 4 * n_out + 4 * M * n_out + (4 * n_out if with_idx else 0)
+
+
+def gemm_kernel_bytes(M, K, n_out, with_idx=False):
+    """What the GEMM kernel itself has to move: int8 A, int8 W, bias, fp32 out."""
+    return M * K + K * n_out + 4 * n_out + 4 * M * n_out + (4 * n_out if with_idx else 0)
+
+
+class Op:
+    """One affine call with all buffers preallocated; `copies` distinct weight copies."""
+
+    def __init__(self, torch, integer, M, K, N, relu=False, copies=1, idx=None, seed=0):
+        g = torch.Generator(device="cuda")
+        g.manual_seed(1000 + seed)
+        self.M, self.K, self.N, self.relu = M, K, N, int(relu)
+        self.A = torch.randn(M, K, device="cuda", generator=g)
+        self.bias = torch.randn(N, device="cuda", generator=g) * 0.01
+        self.Aq = integer.QTensor.empty((M, K), integer.Type.intgemm8, "cuda")
+        W = torch.randn(K, N, device="cuda", generator=g) * 0.02
+        first = integer.prepareB(W)
+        self.Bq = [first] + [integer.QTensor(first.data.clone(), first.shape, first.type)
+                             for _ in range(copies - 1)]
+        self.idx = idx
+        self.n_out = N if idx is None else int(idx.numel())
+        self.out = torch.empty(M, self.n_out, device="cuda")
+        self.ops = 2 * M * K * self.n_out
+
+    def launch(self, lib, be, copy=0, prepare=True, gemm=True):
+        st = be.stream()
+        if prepare:
+            r = lib.marian_hip_int8_prepare_a(self.A.data_ptr(), self.Aq.data_ptr(), self.M, self.K,
+                                              be.workspace.data_ptr(), be.workspace_bytes, st)
+            assert r == 0, r
+        if gemm:
+            b = self.Bq[copy % len(self.Bq)]
+            if self.idx is None:
+                r = lib.marian_hip_int8_affine(self.Aq.data_ptr(), b.data_ptr(), self.bias.data_ptr(),
+                                               self.out.data_ptr(), self.M, self.K, self.N, 1.0,
+                                               self.relu, st)
+            else:
+                r = lib.marian_hip_int8_affine_shortlist(self.Aq.data_ptr(), b.data_ptr(),
+                                                         self.bias.data_ptr(), self.idx.data_ptr(),
+                                                         self.n_out, self.out.data_ptr(), self.M,
+                                                         self.K, self.N, 1.0, self.relu, st)
+            assert r == 0, r
+
+
+def capture(torch, fn):
+    """Record fn's launches into a HIP graph (no memset nodes: the path has none)."""
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        fn()  # warm every kernel (module load, LDS attribute) before capture
+    torch.cuda.current_stream().wait_stream(s)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        fn()
+    return g
+
+
+def time_graphs(torch, graphs, steps, warmup):
+    """Replays graphs round-robin; returns seconds for exactly `steps` replays."""
+    for i in range(warmup):
+        graphs[i % len(graphs)].replay()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        graphs[i % len(graphs)].replay()
+    torch.cuda.synchronize()
+    return time.perf_counter() - t0
+
+
+def per_launch_ms(torch, launches, repeat):
+    """Average duration of single launches from HIP events recorded on the launch stream.  The
+    launches are queued behind a spinning kernel so the host never starves the stream and each
+    event pair brackets exactly one kernel."""
+    stream = torch.cuda.current_stream()
+    n = len(launches) * repeat
+    starts = [torch.cuda.Event(enable_timing=True) for _ in range(n)]
+    ends = [torch.cuda.Event(enable_timing=True) for _ in range(n)]
+    for f in launches:
+        f()
+    torch.cuda.synchronize()
+    torch.cuda._sleep(int(2.0e9 * 0.02 * max(1, n // 100)))  # ~20 ms per 100 launches
+    k = 0
+    for _ in range(repeat):
+        for f in launches:
+            starts[k].record(stream)
+            f()
+            ends[k].record(stream)
+            k += 1
+    torch.cuda.synchronize()
+    d = np.array([starts[i].elapsed_time(ends[i]) for i in range(n)])
+    return float(d.mean()), float(np.median(d))
+
+
+def cpu_baseline(seconds=12.0):
+    """The CPU restatement of the reference path (prepareA + VNNI multiply + unquantize/bias,
+    one thread, like one Marian CPU worker) on the same decode sweep, bounded in time."""
+    from oracle import oracle as orc
+    synth = importlib.import_module(PKG + ".synth")
+    work = []
+    total_ops = 0
+    for (K, N) in DECODE_SHAPES:
+        W = synth.normal(1002, synth.STREAM_W, (K, N), 0.02)
+        Bq = orc.prepare_b(W)
+        bias = synth.normal(1002, synth.STREAM_BIAS, (N,), 0.01)
+        for M in DECODE_M:
+            A = synth.normal(1002, synth.STREAM_A, (M, K), 1.0)
+            work.append((orc.AffineF32(M, K, N), A, Bq, bias))
+            total_ops += 2 * M * K * N
+    for f, A, Bq, bias in work:
+        f(A, Bq, bias)
+    passes = 0
+    t0 = time.perf_counter()
+    while True:
+        for f, A, Bq, bias in work:
+            f(A, Bq, bias)
+        passes += 1
+        dt = time.perf_counter() - t0
+        if dt > seconds:
+            break
+    return {"value": round(total_ops * passes / dt / 1e12, 5), "unit": "TOPS", "cores": 1,
+            "kind": "port",
+            "isa": "avx512-vnni" if orc.has_vnni() else "scalar",
+            "host_cpus": os.cpu_count(),
+            "sample": "%d passes of the same 20-shape decode sweep in %.1f s on one core" % (passes, dt)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--only", default="", help="comma list of extra workloads: encoder,shortlist,big")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this path runs on one GPU (no collectives are part of it); use --gpus 1")
+
+    import torch
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    integer = importlib.import_module(PKG + ".integer")
+    integer.Type = importlib.import_module(PKG + ".types").Type
+    lib = importlib.import_module(PKG + "._lib").lib()
+    torch.cuda.set_device(0)
+    be = integer.Backend.get("cuda:0")
+    extras = set(x for x in args.only.split(",") if x) or {"encoder", "shortlist", "big"}
+
+    # ---------------- headline: transformer-base decode sweep -------------------------------
+    sweep_bytes = sum(K * N for K, N in DECODE_SHAPES) * len(DECODE_M)
+    sets = max(2, int(np.ceil(512e6 / sweep_bytes)) + 1)       # rotate > 512 MB of weights
+    ops_list = [Op(torch, integer, M, K, N, copies=sets, seed=i * 10 + j)
+                for i, (K, N) in enumerate(DECODE_SHAPES) for j, M in enumerate(DECODE_M)]
+    step_ops = sum(o.ops for o in ops_list)
+    step_bytes = sum(algorithmic_bytes(o.M, o.K, o.N) for o in ops_list)
+
+    def step(copy):
+        for o in ops_list:
+            o.launch(lib, be, copy)
+
+    graphs = [capture(torch, (lambda c=c: step(c))) for c in range(sets)]
+    dt = time_graphs(torch, graphs, args.steps, args.warmup)
+    ms_per_step = dt / args.steps * 1e3
+    tops = step_ops / (dt / args.steps) / 1e12
+    # same with one weight set (Infinity-Cache resident), and eager launches from the host
+    dt_res = time_graphs(torch, graphs[:1], args.steps, args.warmup)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(20):
+        step(i)
+    torch.cuda.synchronize()
+    eager_ms = (time.perf_counter() - t0) / 20 * 1e3
+
+    # ---------------- roofline of the dominant kernel ----------------------------------------
+    # vocabulary projection of the sweep at M = 64: 16.4 MB of int8 weights per launch
+    dom = [o for o in ops_list if o.N == 32000 and o.M == 64][0]
+    dom.launch(lib, be, 0, prepare=True, gemm=False)
+    mean_ms, med_ms = per_launch_ms(
+        torch, [(lambda c=c: dom.launch(lib, be, c, prepare=False)) for c in range(sets)], 6)
+    dom_bytes = gemm_kernel_bytes(dom.M, dom.K, dom.N)
+    achieved = dom_bytes / (mean_ms * 1e-3) / 1e9
+    roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
+                "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                "kernel": "gemm_stream_kernel M=64 K=512 N=32000",
+                "bytes_per_launch": dom_bytes, "avg_launch_us": round(mean_ms * 1e3, 3),
+                "median_launch_us": round(med_ms * 1e3, 3)}
+
+    per_shape = {}
+    for (K, N) in DECODE_SHAPES:
+        for M in DECODE_M:
+            o = [x for x in ops_list if (x.M, x.K, x.N) == (M, K, N)][0]
+            o.launch(lib, be, 0, prepare=True, gemm=False)
+            g_ms, _ = per_launch_ms(
+                torch, [(lambda c=c, o=o: o.launch(lib, be, c, prepare=False)) for c in range(sets)], 3)
+            p_ms, _ = per_launch_ms(torch, [(lambda o=o: o.launch(lib, be, 0, gemm=False))], 12)
+            per_shape["M%d_%dx%d" % (M, K, N)] = {
+                "gemm_us": round(g_ms * 1e3, 2), "prepare_a_us": round(p_ms * 1e3, 2),
+                "gemm_hbm_frac": round(gemm_kernel_bytes(M, K, N) / (g_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+
+    out = {
+        "metric": "int8 affine TOPS & % roofline; transformer-big int8 decode tokens/sec",
+        "value": round(tops, 4), "unit": "TOPS", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "int8 x int8 -> int32, fp32 epilogue",
+        "data": "synthetic",
+        "config": {"workload": "transformer-base decode GEMM sweep: M in {1,4,16,64} x "
+                               "{512x1536, 512x512, 512x2048, 2048x512, 512x32000}, "
+                               "prepareA + int8 affine with bias per shape",
+                   "launch": "HIP graph replay, %d rotating weight sets (%.0f MB)" % (sets, sets * sweep_bytes / 1e6),
+                   "step_ops": step_ops, "step_algorithmic_bytes": step_bytes},
+        "step_hbm_frac": round(step_bytes / (dt / args.steps) / 1e9 / HBM_PEAK_GBS, 4),
+        "value_cache_resident_tops": round(step_ops / (dt_res / args.steps) / 1e12, 4),
+        "eager_ms_per_step": round(eager_ms, 4),
+        "roofline": roofline,
+        "per_shape": per_shape,
+    }
+    del graphs
+    del ops_list
+
+    # ---------------- encoder-size GEMMs (MFMA-bound case) ------------------------------------
+    if "encoder" in extras:
+        enc = {}
+        for (M, K, N) in [(4096, 1024, 4096), (4096, 4096, 1024)]:
+            o = Op(torch, integer, M, K, N, relu=True, copies=4, seed=77)
+            o.launch(lib, be, 0, prepare=True, gemm=False)
+            g_ms, g_med = per_launch_ms(
+                torch, [(lambda c=c: o.launch(lib, be, c, prepare=False)) for c in range(4)], 10)
+            p_ms, _ = per_launch_ms(torch, [(lambda: o.launch(lib, be, 0, gemm=False))], 10)
+            t_all = (g_ms + p_ms) * 1e-3
+            enc["M%d_K%d_N%d" % (M, K, N)] = {
+                "gemm_us": round(g_ms * 1e3, 2), "gemm_median_us": round(g_med * 1e3, 2),
+                "prepare_a_us": round(p_ms * 1e3, 2),
+                "gemm_tops": round(o.ops / (g_ms * 1e-3) / 1e12, 1),
+                "gemm_mfma_frac": round(o.ops / (g_ms * 1e-3) / 1e12 / INT8_PEAK_TOPS, 4),
+                "gemm_hbm_frac": round(gemm_kernel_bytes(M, K, N) / (g_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                "affine_tops": round(o.ops / t_all / 1e12, 1),
+                "affine_hbm_frac": round(algorithmic_bytes(M, K, N) / t_all / 1e9 / HBM_PEAK_GBS, 4)}
+            del o
+        out["encoder"] = enc
+        out["int8_peak_tops_used"] = INT8_PEAK_TOPS
+
+    # ---------------- shortlisted output layer -------------------------------------------------
+    if "shortlist" in extras:
+        synth = importlib.import_module(PKG + ".synth")
+        sl = {}
+        M, K, N = 256, 1024, 32000
+        for name, ids in [("full", None), ("n504", synth.shortlist(11, N, 504, 504)),
+                          ("n1000", synth.shortlist(12, N, 1000, 1000)),
+                          ("n2000", synth.shortlist(13, N, 2000, 2000))]:
+            idx = None if ids is None else torch.from_numpy(ids.view(np.int32)).cuda()
+            o = Op(torch, integer, M, K, N, copies=8 if ids is None else 2, idx=idx, seed=5)
+            o.launch(lib, be, 0, prepare=True, gemm=False)
+            g_ms, _ = per_launch_ms(
+                torch, [(lambda c=c: o.launch(lib, be, c, prepare=False)) for c in range(len(o.Bq))], 6)
+            sl[name] = {"n_out": o.n_out, "gemm_us": round(g_ms * 1e3, 2),
+                        "gemm_tops": round(o.ops / (g_ms * 1e-3) / 1e12, 2),
+                        "gemm_hbm_frac": round(gemm_kernel_bytes(M, K, o.n_out, ids is not None)
+                                               / (g_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+            del o
+        out["shortlist"] = sl
+
+    # ---------------- transformer-big decode step (GEMMs only) ----------------------------------
+    if "big" in extras:
+        d, ffn, V, M = 1024, 4096, 32000, 128
+        layer = [(d, d, 0)] * 6 + [(d, ffn, 1), (ffn, d, 0)]     # self q,k,v,o; ctx q,o; ffn1, ffn2
+        shapes = layer * 6 + [(d, V, 0)]
+        wbytes = sum(K * N for K, N, _ in shapes)
+        bsets = max(2, int(np.ceil(512e6 / wbytes)) + 1)
+        ops_big = [Op(torch, integer, M, K, N, relu=r, copies=bsets, seed=200 + i)
+                   for i, (K, N, r) in enumerate(shapes)]
+
+        def big_step(copy):
+            for o in ops_big:
+                o.launch(lib, be, copy)
+
+        bgraphs = [capture(torch, (lambda c=c: big_step(c))) for c in range(bsets)]
+        n = max(20, args.steps // 2)
+        bdt = time_graphs(torch, bgraphs, n, max(4, args.warmup // 2))
+        out["transformer_big_decode"] = {
+            "what": "GEMM-only decode step at beam 4 x batch 32 (M=128): 48 layer GEMMs + "
+                    "32000-vocab output GEMM, each with its prepareA; self-attention K/V "
+                    "projections taken at M=128",
+            "ms_per_step": round(bdt / n * 1e3, 4),
+            "hyp_tokens_per_s": round(M * n / bdt, 1),
+            "output_tokens_per_s": round(32 * n / bdt, 1),
+            "tops": round(sum(o.ops for o in ops_big) * n / bdt / 1e12, 2),
+            "weight_hbm_frac": round(wbytes * n / bdt / 1e9 / HBM_PEAK_GBS, 4),
+            "weight_sets": bsets}
+        del bgraphs
+        del ops_big
+
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline()
+    else:
+        out["cpu_baseline"] = None
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

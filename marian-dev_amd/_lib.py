@@ -57,6 +57,10 @@ def lib():
             raise MarianHipError(
                 -1, "libmarian_hip_int8.so is not built ({}); run __graft_entry__.build() or "
                 "`make -C marian-dev_amd/csrc`. There is no CPU fallback.".format(LIB_PATH))
+        # torch must load first: it ships its own libamdhip64.so.7 / HSA runtime, and a process
+        # can hold only one of them - loading ours first would pull in the system copy and
+        # leave torch's runtime without a device (hipErrorNoDevice on the first launch)
+        import torch  # noqa: F401
         L = ctypes.CDLL(LIB_PATH)
         for name, (res, args) in SIGNATURES.items():
             f = getattr(L, name)  # AttributeError if a declared symbol is not exported

@@ -102,10 +102,11 @@ int launch_gemm(const GemmArgs& a, hipStream_t st) {
 
 int check_gemm(const int8_t* Aq, const int8_t* Bq, const void* out, const float* bias,
                const uint32_t* idx, int64_t n_idx, int64_t M, int64_t K, int64_t N) {
-  if(!Aq || !Bq || !out) return MARIAN_HIP_ERR_NULL;
   if(M < 0 || K <= 0 || N < 0 || (K % 64) != 0 || (N % 8) != 0) return MARIAN_HIP_ERR_SHAPE;
   if(idx && (n_idx < 0 || (n_idx % 8) != 0)) return MARIAN_HIP_ERR_SHAPE;
   const int64_t n_out = idx ? n_idx : N;
+  if(M == 0 || n_out == 0) return MARIAN_HIP_OK;  // empty batch: nothing is dereferenced
+  if(!Aq || !Bq || !out) return MARIAN_HIP_ERR_NULL;
   if(M * K > kMaxElems || K * N > kMaxElems || M * n_out > kMaxElems) return MARIAN_HIP_ERR_RANGE;
   if(!aligned(Aq, 16) || !aligned(Bq, 16) || !aligned(out, 16)) return MARIAN_HIP_ERR_ALIGN;
   if((bias && !aligned(bias, 4)) || (idx && !aligned(idx, 4))) return MARIAN_HIP_ERR_ALIGN;
@@ -161,11 +162,11 @@ int marian_hip_int8_set_kernel(int which) { return g_kernel_override.exchange(wh
 
 int marian_hip_int8_prepare_a(const float* A, int8_t* Aq, int64_t M, int64_t K, void* workspace,
                               size_t workspace_bytes, void* stream) {
-  if(!A || !Aq) return MARIAN_HIP_ERR_NULL;
   if(M < 0 || K <= 0 || (K % 64) != 0) return MARIAN_HIP_ERR_SHAPE;
+  if(M == 0) return MARIAN_HIP_OK;  // empty batch: nothing is dereferenced
+  if(!A || !Aq) return MARIAN_HIP_ERR_NULL;
   if(M * K > kMaxElems) return MARIAN_HIP_ERR_RANGE;
   if(!aligned(A, 16) || !aligned(Aq, 16)) return MARIAN_HIP_ERR_ALIGN;
-  if(M == 0) return MARIAN_HIP_OK;
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   const size_t n = (size_t)M * (size_t)K;
   if(n <= (size_t)kSingleBlockMaxElems) {
@@ -192,8 +193,8 @@ int marian_hip_int8_prepare_a(const float* A, int8_t* Aq, int64_t M, int64_t K, 
 
 int marian_hip_int8_prepare_b(const float* W, int8_t* Bq, int64_t K, int64_t N, void* workspace,
                               size_t workspace_bytes, void* stream) {
-  if(!W || !Bq || !workspace) return MARIAN_HIP_ERR_NULL;
   if(K <= 0 || N <= 0 || (K % 64) != 0 || (N % 8) != 0) return MARIAN_HIP_ERR_SHAPE;
+  if(!W || !Bq || !workspace) return MARIAN_HIP_ERR_NULL;
   if(K * N > kMaxElems) return MARIAN_HIP_ERR_RANGE;
   if(!aligned(W, 16) || !aligned(Bq, 16) || !aligned(workspace, 4)) return MARIAN_HIP_ERR_ALIGN;
   if(workspace_bytes < kWorkspaceBytes) return MARIAN_HIP_ERR_WORKSPACE;

@@ -57,6 +57,7 @@ def test_argument_validation_returns_codes_not_aborts():
     assert lib.marian_hip_int8_affine(buf, buf, None, buf, 1 << 26, 64, 8, 1.0, 0, None) == L.ERR_RANGE
     assert lib.marian_hip_int8_affine(buf, buf, None, buf, 0, 64, 8, 1.0, 0, None) == L.OK  # empty batch
     assert lib.marian_hip_int8_affine_shortlist(buf, buf, None, None, 8, buf, 1, 64, 8, 1.0, 0, None) == L.ERR_NULL
+    assert lib.marian_hip_int8_affine(None, None, None, None, 0, 64, 8, 1.0, 0, None) == L.OK
     assert lib.marian_hip_int8_affine_shortlist(buf, buf, None, buf, 12, buf, 1, 64, 8, 1.0, 0, None) == L.ERR_SHAPE
     assert lib.marian_hip_int8_prepare_a(buf, buf, 4, 100, buf, 4096, None) == L.ERR_SHAPE
     assert lib.marian_hip_int8_prepare_a(buf, buf, 4096, 1024, buf, 16, None) == L.ERR_WORKSPACE
