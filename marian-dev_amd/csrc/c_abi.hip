@@ -6,6 +6,8 @@
 
 #include <atomic>
 
+#include "gemm_mfma32_kernel.h"
+#include "gemm_persistent_kernel.h"
 #include "gemm_stream_kernel.h"
 #include "gemm_tile_kernel.h"
 #include "quantize_kernels.h"
@@ -16,6 +18,7 @@ namespace {
 
 thread_local int g_last_hip_error = 0;
 std::atomic<int> g_kernel_override{0};
+std::atomic<long long*> g_prof{nullptr};
 
 int hip_fail(hipError_t e) {
   g_last_hip_error = (int)e;
@@ -66,6 +69,52 @@ int launch_tile(const GemmArgs& a, hipStream_t st) {
   return MARIAN_HIP_OK;
 }
 
+template <int BM, int BN, int WM, int WN, int NSTAGE>
+int launch_big(const GemmArgs& a, hipStream_t st) {
+  using Cfg = BigCfg<BM, BN, WM, WN, NSTAGE>;
+  if(a.K % Cfg::BK != 0) return launch_tile<4, 4>(a, st);  // this family needs K % 128 == 0
+  auto kernel = gemm_mfma32_kernel<BM, BN, WM, WN, NSTAGE>;
+  static const int lds_status = allow_lds(kernel, Cfg::kLdsBytes);
+  if(lds_status != MARIAN_HIP_OK) return lds_status;
+  int tiles_n = (a.n_out + BN - 1) / BN;
+  int tiles_m = (a.M + BM - 1) / BM;
+  hipLaunchKernelGGL(kernel, dim3(tiles_n * tiles_m), dim3(Cfg::kThreads), Cfg::kLdsBytes, st, a,
+                     tiles_n, tiles_m);
+  MH_HIP(hipGetLastError());
+  return MARIAN_HIP_OK;
+}
+
+int compute_units() {
+  static const int cus = [] {
+    int dev = 0, n = 0;
+    if(hipGetDevice(&dev) != hipSuccess) return 256;
+    if(hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+      return 256;
+    return n;
+  }();
+  return cus;
+}
+
+template <int BM, int BN, int WM, int WN, int NSTAGE>
+int launch_persistent(const GemmArgs& a, hipStream_t st) {
+  using Cfg = PersistCfg<BM, BN, WM, WN, NSTAGE>;
+  // needs K % 128 == 0, at least NSTAGE K blocks per tile and a 16-byte aligned bias
+  if(a.K % Cfg::BK != 0 || a.K / Cfg::BK < NSTAGE || (a.bias && !aligned(a.bias, 16)))
+    return launch_big<BM, BN, WM, WN, 2>(a, st);
+  auto dense = gemm_persistent_kernel<BM, BN, WM, WN, NSTAGE, false>;
+  auto gather = gemm_persistent_kernel<BM, BN, WM, WN, NSTAGE, true>;
+  static const int lds_status = allow_lds(dense, Cfg::kLdsBytes) | allow_lds(gather, Cfg::kLdsBytes);
+  if(lds_status != MARIAN_HIP_OK) return lds_status;
+  int tiles_n = (a.n_out + BN - 1) / BN;
+  int tiles_m = (a.M + BM - 1) / BM;
+  int total = tiles_n * tiles_m;
+  int grid = total < compute_units() ? total : compute_units();
+  hipLaunchKernelGGL(a.idx ? gather : dense, dim3(grid), dim3(Cfg::kThreads), Cfg::kLdsBytes, st, a,
+                     tiles_n, tiles_m);
+  MH_HIP(hipGetLastError());
+  return MARIAN_HIP_OK;
+}
+
 // wide: many weight rows, every wave streams its own rows over the whole K
 // narrow: few weight rows, the four waves split K and reduce
 template <int MT>
@@ -86,7 +135,7 @@ int launch_stream_auto(const GemmArgs& a, hipStream_t st, int force_wide) {
 }
 
 int launch_gemm(const GemmArgs& a, hipStream_t st) {
-  const int which = g_kernel_override.load(std::memory_order_relaxed);
+  const int which = g_kernel_override.load(std::memory_order_relaxed) % 1000;
   switch(which) {
     case 101: if(a.M <= 128) return launch_stream_auto(a, st, 1); break;
     case 102: if(a.M <= 128) return launch_stream_auto(a, st, 2); break;
@@ -94,10 +143,33 @@ int launch_gemm(const GemmArgs& a, hipStream_t st) {
     case 202: return launch_tile<8, 4>(a, st);
     case 203: return launch_tile<4, 8>(a, st);
     case 204: return launch_tile<2, 2>(a, st);
+    case 301: return launch_big<256, 256, 2, 4, 2>(a, st);
+    case 302: return launch_big<128, 128, 2, 2, 2>(a, st);
+    case 303: return launch_big<256, 128, 2, 2, 2>(a, st);
+    case 304: return launch_big<256, 128, 4, 2, 2>(a, st);
+    case 305: return launch_big<128, 256, 2, 2, 2>(a, st);
+    case 306: return launch_big<256, 256, 2, 2, 2>(a, st);
+    case 307: return launch_big<128, 128, 2, 2, 3>(a, st);
+    case 308: return launch_big<256, 128, 2, 2, 3>(a, st);
+    case 309: return launch_big<128, 64, 2, 2, 2>(a, st);
+    case 310: return launch_big<64, 128, 2, 2, 2>(a, st);
+    case 311: return launch_big<128, 128, 4, 2, 2>(a, st);
+    case 312: return launch_big<128, 128, 2, 4, 2>(a, st);
+    case 313: return launch_big<128, 64, 2, 2, 3>(a, st);
+    case 314: return launch_big<128, 64, 4, 2, 2>(a, st);
+    case 401: return launch_persistent<128, 128, 2, 2, 4>(a, st);
+    case 402: return launch_persistent<128, 128, 2, 2, 3>(a, st);
+    case 403: return launch_persistent<128, 128, 2, 2, 2>(a, st);
+    case 404: return launch_persistent<256, 128, 2, 2, 2>(a, st);
     default: break;
   }
   if(a.M <= 128) return launch_stream_auto(a, st, 0);
-  return launch_tile<4, 4>(a, st);
+  if(a.K % 128 != 0) return launch_tile<4, 4>(a, st);
+  // large outputs: 256x256 tiles (one per CU keeps operand traffic lowest); otherwise 128x128
+  // tiles with a three-deep LDS ring so that enough loads are in flight per CU
+  const long long tiles256 = ((a.M + 255) / 256) * (long long)((a.n_out + 255) / 256);
+  if(tiles256 >= 192) return launch_big<256, 256, 2, 4, 2>(a, st);
+  return launch_big<128, 128, 2, 2, 3>(a, st);
 }
 
 int check_gemm(const int8_t* Aq, const int8_t* Bq, const void* out, const float* bias,
@@ -124,6 +196,8 @@ int run_gemm(const int8_t* Aq, const int8_t* Bq, const float* bias, const uint32
   a.Aq = Aq; a.Bq = Bq; a.bias = bias; a.idx = idx; a.out = out;
   a.M = (int)M; a.K = (int)K; a.N = (int)N; a.n_out = (int)n_out;
   a.scale = scale; a.relu = relu ? 1 : 0; a.dump = dump;
+  a.dbg = g_kernel_override.load(std::memory_order_relaxed) / 1000;
+  a.prof = g_prof.load(std::memory_order_relaxed);
   return launch_gemm(a, reinterpret_cast<hipStream_t>(stream));
 }
 
@@ -159,6 +233,8 @@ int marian_hip_int8_abi_version(void) { return 1; }
 size_t marian_hip_int8_workspace_bytes(void) { return kWorkspaceBytes; }
 
 int marian_hip_int8_set_kernel(int which) { return g_kernel_override.exchange(which); }
+
+void marian_hip_int8_debug_profile(long long* p) { g_prof.store(p); }
 
 int marian_hip_int8_prepare_a(const float* A, int8_t* Aq, int64_t M, int64_t K, void* workspace,
                               size_t workspace_bytes, void* stream) {

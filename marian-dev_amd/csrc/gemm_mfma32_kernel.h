@@ -1,0 +1,291 @@
+// Compute-bound int8 GEMM for large M (encoder shapes): 32x32x32 i8 MFMA, operands streamed
+// global -> LDS without passing through registers.
+//
+// v_mfma_i32_32x32x32_i8 is the int8 instruction that runs at the full matrix rate on gfx950
+// (32 cycles for 32x32x32 MACs; the 16x16x64 form issues at roughly half that rate).  Operand
+// traffic into a CU (about 64 bytes per clock through the vector L1) is the limit, so a
+// workgroup owns a large BM x BN output tile and each operand byte enters the CU once per tile:
+//   * K advances in 128-byte blocks.  A row of a block is one full 128-byte line in global
+//     memory (both operands are K-contiguous).  One global_load_lds_dwordx4 per wave moves 8
+//     rows (1 KB) straight into LDS; the lane that fills 16-byte slot p of row r fetches chunk
+//     p ^ ((r >> 1) & 7) of that row, so LDS holds each row with its chunks XOR-swizzled and the
+//     MFMA fragment reads (32 consecutive rows, one chunk each) are bank-conflict free.
+//   * NSTAGE LDS buffers; the loads of block k + NSTAGE are issued as soon as block k has been
+//     read, so they have NSTAGE - 1 blocks of MFMA time to land.
+//   * Fragments are double-buffered in registers: the ds_reads of sub-step s + 1 (also across
+//     the barrier into the next block) are issued before the MFMAs of sub-step s.
+// Activations are the row operand and weights the column operand, so a lane ends up with one
+// output column and the 32 lanes of a half-wave write 128 contiguous bytes of an output row.
+// Requires K % 128 == 0.
+#pragma once
+
+#include "int8_common.h"
+
+namespace marian_hip {
+
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+template <int BM_, int BN_, int WAVES_M, int WAVES_N, int NSTAGE_>
+struct BigCfg {
+  static constexpr int BM = BM_, BN = BN_, BK = 128, NSTAGE = NSTAGE_;
+  static constexpr int kWaves = WAVES_M * WAVES_N;
+  static constexpr int kThreads = kWaves * kWave;
+  static constexpr int WTM = BM / WAVES_M / 32;  // 32x32 MFMA tiles per wave along m
+  static constexpr int WTN = BN / WAVES_N / 32;  // and along n
+  static constexpr int kRows = BM + BN;
+  static constexpr int kStageBytes = kRows * BK;
+  static constexpr int kGroups = kRows / 8;            // 8-row groups, one wave load each
+  static constexpr int kLoads = kGroups / kWaves;      // loads per wave per K block
+  static constexpr int kLoadsA = (BM / 8) / kWaves;    // the first of them are activation rows
+  static constexpr int kLdsBytes = NSTAGE * kStageBytes;
+  static_assert((BM / 8) % kWaves == 0 && (BN / 8) % kWaves == 0, "tile rows vs waves");
+  static_assert(BM % (WAVES_M * 32) == 0 && BN % (WAVES_N * 32) == 0, "tile vs wave grid");
+  static_assert(NSTAGE == 2 || NSTAGE == 3, "two or three LDS stages");
+};
+
+// s_waitcnt with only vmcnt (up to 63) or only lgkmcnt constrained (gfx9 encoding).
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+  __builtin_amdgcn_s_waitcnt((N & 0xF) | ((N >> 4) << 14) | (0x7 << 4) | (0xF << 8));
+}
+__device__ __forceinline__ void wait_lgkmcnt0() { __builtin_amdgcn_s_waitcnt(0xC07F); }
+
+// 16 bytes per lane from global memory straight into LDS: lane l of the wave writes LDS bytes
+// lds_addr + 16*l .. +15 (lds_addr is wave-uniform and travels in M0).  Issued as inline assembly
+// on purpose: for the builtin form the compiler assumes that every later LDS read may alias the
+// incoming data and inserts s_waitcnt vmcnt(0) in front of it, which serialises the K pipeline.
+// Completion is tracked by hand with vmcnt (loads and stores of a wave retire in issue order).
+__device__ __forceinline__ void global_load_lds16(const void* gptr, unsigned lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+               :
+               : "s"(lds_addr), "v"(gptr)
+               : "memory", "m0");
+}
+
+
+// Writes one 32x32 accumulator tile.  Element v of the tile is row 8*(v/4) + 4*(lane/32) + v%4,
+// column lane%32; `out` points at this lane's element of tile row 4*(lane/32).
+//   y = float(acc) * unquant (+ bias) ; relu: y > 0 ? y : 0   (mul and add round separately)
+template <bool DUMP, bool BIAS, bool RELU, bool GUARD>
+__device__ __forceinline__ void store_tile32(const v16i& acc, char* out, size_t row_bytes,
+                                             float unquant, float bias_v, int rows_left,
+                                             bool col_valid) {
+#pragma unroll
+  for(int v = 0; v < 16; ++v) {
+    const int r = 8 * (v / 4) + (v % 4);
+    if(GUARD && (!col_valid || r >= rows_left)) continue;
+    char* p = out + (size_t)r * row_bytes;
+    if(DUMP) {
+      *reinterpret_cast<int32_t*>(p) = acc[v];
+    } else {
+      float y = (float)acc[v] * unquant;
+      if(BIAS) y = y + bias_v;
+      if(RELU) y = y > 0.0f ? y : 0.0f;
+      *reinterpret_cast<float*>(p) = y;
+    }
+  }
+}
+
+template <bool GUARD>
+__device__ __forceinline__ void store_tile32_any(const v16i& acc, char* out, size_t row_bytes,
+                                                 float unquant, float bias_v, int rows_left,
+                                                 bool col_valid, int dump, bool bias, int relu) {
+  if(dump) store_tile32<true, false, false, GUARD>(acc, out, row_bytes, unquant, bias_v, rows_left, col_valid);
+  else if(bias && relu) store_tile32<false, true, true, GUARD>(acc, out, row_bytes, unquant, bias_v, rows_left, col_valid);
+  else if(bias) store_tile32<false, true, false, GUARD>(acc, out, row_bytes, unquant, bias_v, rows_left, col_valid);
+  else if(relu) store_tile32<false, false, true, GUARD>(acc, out, row_bytes, unquant, bias_v, rows_left, col_valid);
+  else store_tile32<false, false, false, GUARD>(acc, out, row_bytes, unquant, bias_v, rows_left, col_valid);
+}
+
+template <int BM, int BN, int WAVES_M, int WAVES_N, int NSTAGE>
+__global__ __launch_bounds__(WAVES_M * WAVES_N * kWave) void gemm_mfma32_kernel(
+    GemmArgs args, int tiles_n, int tiles_m) {
+  using Cfg = BigCfg<BM, BN, WAVES_M, WAVES_N, NSTAGE>;
+  extern __shared__ __attribute__((aligned(16))) int8_t lds[];
+  const unsigned lds_base = (unsigned)(size_t)lds;  // LDS byte address of the ring
+
+  const long long t_start = clock64();
+  const int tid = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+  const int lane = tid % kWave;
+  const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+  const int li = lane % 32, lg = lane / 32;
+  const int K = args.K, M = args.M;
+  const int KB = K / Cfg::BK;
+
+  int tn, tm;
+  {
+    // Workgroups of one XCD (ids congruent mod 8 under round-robin dispatch) take a compact
+    // block of tiles - 4 tiles along n by a run along m - so that the XCD's L2 holds few weight
+    // panels and few activation panels at a time.
+    const int total = tiles_n * tiles_m;
+    int t = blockIdx.x;
+    if(total % 8 == 0) t = (blockIdx.x % 8) * (total / 8) + blockIdx.x / 8;
+    const int band = 4;
+    const int b = t / (band * tiles_m);
+    const int r = t % (band * tiles_m);
+    const int bw = (tiles_n - b * band) < band ? (tiles_n - b * band) : band;
+    tn = b * band + r % bw;
+    tm = r / bw;
+  }
+  const int m0 = tm * BM, n0 = tn * BN;
+
+  // ---- global -> LDS: load j of this wave fills rows (j*kWaves + wave)*8 .. +7 of a stage.
+  // Rows past the matrix edge re-read the last valid row; their products are never stored.
+  int goff[Cfg::kLoads];
+#pragma unroll
+  for(int j = 0; j < Cfg::kLoads; ++j) {
+    const int row = (j * Cfg::kWaves + wave) * 8 + lane / 8;
+    const int chunk = (lane % 8) ^ ((row >> 1) & 7);
+    int src;
+    if(j < Cfg::kLoadsA) {
+      src = min(m0 + row, M - 1);
+    } else {
+      const int n = min(n0 + row - BM, args.n_out - 1);
+      src = args.idx ? (int)args.idx[n] : n;
+    }
+    goff[j] = src * K + chunk * 16;
+  }
+  auto issue = [&](int kb) {
+    const int stage = kb % NSTAGE;
+#pragma unroll
+    for(int j = 0; j < Cfg::kLoads; ++j) {
+      const int8_t* base = (j < Cfg::kLoadsA) ? args.Aq : args.Bq;
+      const int8_t* src = base + (size_t)(unsigned)goff[j] + (size_t)kb * Cfg::BK;
+      global_load_lds16(src, lds_base + stage * Cfg::kStageBytes + (j * Cfg::kWaves + wave) * 1024);
+    }
+  };
+
+  // ---- fragment addressing: lane (li, lg) reads row li of a 32-row tile, chunk kk*2 + lg ----
+  int frag_off[4];
+#pragma unroll
+  for(int kk = 0; kk < 4; ++kk) frag_off[kk] = li * 128 + (((kk * 2 + lg) ^ ((li >> 1) & 7)) * 16);
+  const int a_row0 = wm * Cfg::WTM * 32;          // first activation row of this wave in a stage
+  const int b_row0 = BM + wn * Cfg::WTN * 32;     // first weight row
+
+  v4i af[4][Cfg::WTM], bf[4][Cfg::WTN];
+  auto read_frags = [&](int stage, int kk, int set) {
+    const int8_t* buf = lds + stage * Cfg::kStageBytes + frag_off[kk];
+#pragma unroll
+    for(int a = 0; a < Cfg::WTM; ++a)
+      af[set][a] = *reinterpret_cast<const v4i*>(buf + (a_row0 + a * 32) * 128);
+#pragma unroll
+    for(int b = 0; b < Cfg::WTN; ++b)
+      bf[set][b] = *reinterpret_cast<const v4i*>(buf + (b_row0 + b * 32) * 128);
+  };
+
+  v16i acc[Cfg::WTM][Cfg::WTN];
+#pragma unroll
+  for(int a = 0; a < Cfg::WTM; ++a)
+#pragma unroll
+    for(int b = 0; b < Cfg::WTN; ++b)
+#pragma unroll
+      for(int v = 0; v < 16; ++v) acc[a][b][v] = 0;
+  auto multiply = [&](int set) {
+#pragma unroll
+    for(int a = 0; a < Cfg::WTM; ++a)
+#pragma unroll
+      for(int b = 0; b < Cfg::WTN; ++b)
+        acc[a][b] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[set][a], bf[set][b], acc[a][b], 0, 0, 0);
+  };
+  // Scheduler hints.  The fragments of sub-steps 2,3 (and of sub-steps 0,1 of the next block)
+  // are requested two sub-steps ahead, `reads_per_mfma` LDS reads after each MFMA of an even
+  // sub-step, so that they have a whole odd sub-step of MFMA time to arrive.
+  auto interleave = [&]() {
+    constexpr int kMfma = Cfg::WTM * Cfg::WTN;
+    constexpr int kReads = 2 * (Cfg::WTM + Cfg::WTN);
+    constexpr int kPer = (kReads + kMfma - 1) / kMfma;
+#pragma unroll
+    for(int i = 0; i < kMfma; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);     // one MFMA
+      __builtin_amdgcn_sched_group_barrier(0x100, kPer, 0);  // then a few DS reads
+    }
+  };
+  auto mfma_only = [&]() { __builtin_amdgcn_sched_group_barrier(0x008, Cfg::WTM * Cfg::WTN, 0); };
+
+  // ---- prologue: fill all stages, wait for block 0 only ----
+#pragma unroll
+  for(int s = 0; s < NSTAGE; ++s)
+    if(s < KB) issue(s);
+  if(NSTAGE == 3 && KB >= 3) wait_vmcnt<2 * Cfg::kLoads>();
+  else if(KB >= 2) wait_vmcnt<Cfg::kLoads>();
+  else wait_vmcnt<0>();
+  __builtin_amdgcn_s_barrier();
+  const long long t_prologue = clock64();
+  read_frags(0, 0, 0);
+  read_frags(0, 1, 1);
+
+  for(int kb = 0; kb + 1 < KB; ++kb) {
+    const int stage = kb % NSTAGE;
+    read_frags(stage, 2, 2);
+    read_frags(stage, 3, 3);
+    multiply(0);
+    interleave();
+    multiply(1);
+    mfma_only();
+    // All reads of this block were issued one sub-step ago; once they have returned the stage
+    // is free.  Block kb+1 must have landed (this wave's share); later blocks may be in flight.
+    __builtin_amdgcn_sched_barrier(0);  // keep the MFMAs above on this side of the wait
+    wait_lgkmcnt0();
+    if(NSTAGE == 3 && kb + 2 < KB) wait_vmcnt<Cfg::kLoads>();
+    else wait_vmcnt<0>();
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+    if(kb + NSTAGE < KB && !(args.dbg & 1)) issue(kb + NSTAGE);
+    read_frags((kb + 1) % NSTAGE, 0, 0);
+    read_frags((kb + 1) % NSTAGE, 1, 1);
+    multiply(2);
+    interleave();
+    multiply(3);
+    mfma_only();
+  }
+  {
+    const int stage = (KB - 1) % NSTAGE;
+    read_frags(stage, 2, 2);
+    read_frags(stage, 3, 3);
+    multiply(0);
+    interleave();
+    multiply(1);
+    mfma_only();
+    multiply(2);
+    mfma_only();
+    multiply(3);
+    mfma_only();
+  }
+
+  const long long t_main = clock64();
+  // ---- epilogue: element v of a 32x32 tile is row 8*(v/4) + 4*lg + v%4, column li ----
+  float unquant = 0.0f;
+  if(!args.dump) {
+    float aqm = tail_quant_mult(args.Aq, (size_t)M * (size_t)K);
+    float bqm = tail_quant_mult(args.Bq, (size_t)K * (size_t)args.N);
+    unquant = unquant_mult(aqm, bqm, args.scale);
+  }
+  const bool interior = (m0 + BM <= M) && (n0 + BN <= args.n_out);
+  const size_t row_bytes = (size_t)args.n_out * 4;
+  const bool has_bias = args.bias != nullptr;
+  if(!(args.dbg & 2)) {
+#pragma unroll
+    for(int b = 0; b < Cfg::WTN; ++b) {
+      const int n = n0 + (wn * Cfg::WTN + b) * 32 + li;
+      const bool nvalid = n < args.n_out;
+      float bias_v = 0.0f;
+      if(has_bias && nvalid && !args.dump) bias_v = args.bias[args.idx ? args.idx[n] : (uint32_t)n];
+#pragma unroll
+      for(int a = 0; a < Cfg::WTM; ++a) {
+        const int mbase = m0 + (wm * Cfg::WTM + a) * 32 + 4 * lg;
+        char* outp = reinterpret_cast<char*>(args.out) + ((size_t)mbase * (size_t)args.n_out + (size_t)n) * 4;
+        if(interior)
+          store_tile32_any<false>(acc[a][b], outp, row_bytes, unquant, bias_v, 32, true, args.dump, has_bias, args.relu);
+        else
+          store_tile32_any<true>(acc[a][b], outp, row_bytes, unquant, bias_v, M - mbase, nvalid, args.dump, has_bias, args.relu);
+      }
+    }
+  }
+  if(args.prof && tid == 0) {
+    long long* p = args.prof + (size_t)blockIdx.x * 8;
+    p[0] = t_start; p[1] = t_prologue; p[2] = t_main; p[3] = clock64();
+  }
+}
+
+}  // namespace marian_hip

@@ -98,6 +98,8 @@ struct GemmArgs {
   int M, K, N, n_out;
   float scale;
   int relu, dump;
+  int dbg;  // measurement switches (bit 0: no refetch, bit 1: no stores); 0 in normal use
+  long long* prof;  // per-workgroup phase clocks for tuning runs, null in normal use
 };
 
 __device__ __forceinline__ Epilogue make_epilogue(const GemmArgs& a) {
