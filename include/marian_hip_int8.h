@@ -99,6 +99,19 @@ int marian_hip_int8_affine(const int8_t* Aq, const int8_t* Bq, const float* bias
                            void* stream);
 
 /*
+ * prepareA node + multiply node in one call (reference src/tensors/cpu/intgemm_interface.h:52
+ * builds the first inside affineOrDotTyped and :60-94 the second).  Results are those of
+ * marian_hip_int8_prepare_a followed by marian_hip_int8_affine / _affine_shortlist: Aq (M*K + 4
+ * bytes, required) receives the quantized activations and their quantMult, out the product.
+ * For small activations both steps run in one kernel (every workgroup derives the same abs-max);
+ * otherwise the two kernels are launched back to back.  idx == NULL selects the dense form.
+ */
+int marian_hip_int8_affine_f32(const float* A, int8_t* Aq, const int8_t* Bq, const float* bias,
+                               const uint32_t* idx, int64_t n_idx, float* out, int64_t M,
+                               int64_t K, int64_t N, float scale, int relu, void* workspace,
+                               size_t workspace_bytes, void* stream);
+
+/*
  * Shortlisted output layer.  Reference (fp32): index_select(Wt, 0, idx), index_select(b, -1,
  * idx), then dot/affine with transB (src/data/shortlist.cpp:62-79,
  * src/layers/output.cpp:335-350).  Here rows idx[j] of the [N x K] payload and bias[idx[j]]

@@ -22,6 +22,8 @@ SIGNATURES = {
     "marian_hip_int8_prepare_b": (_i, [_vp, _vp, _i64, _i64, _vp, _sz, _vp]),
     "marian_hip_int8_prepare_b_quantized_transposed": (_i, [_vp, _vp, _i64, _i64, _vp]),
     "marian_hip_int8_affine": (_i, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _f, _i, _vp]),
+    "marian_hip_int8_affine_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _i64, _vp, _i64, _i64, _i64, _f, _i,
+                                        _vp, _sz, _vp]),
     "marian_hip_int8_affine_shortlist": (_i, [_vp, _vp, _vp, _vp, _i64, _vp, _i64, _i64, _i64,
                                               _f, _i, _vp]),
     "marian_hip_int8_multiply_i32": (_i, [_vp, _vp, _vp, _i64, _vp, _i64, _i64, _i64, _vp]),

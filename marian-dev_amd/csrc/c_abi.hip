@@ -8,6 +8,7 @@
 
 #include "gemm_mfma32_kernel.h"
 #include "gemm_persistent_kernel.h"
+#include "gemm_stream32_kernel.h"
 #include "gemm_stream_kernel.h"
 #include "gemm_tile_kernel.h"
 #include "quantize_kernels.h"
@@ -84,6 +85,63 @@ int launch_big(const GemmArgs& a, hipStream_t st) {
   return MARIAN_HIP_OK;
 }
 
+// ---- small-M weight-streaming kernels on the 32x32x32 MFMA ----
+inline int stream32_fused_lds_bytes(int mt32, int K) { return mt32 * 32 * K; }
+
+// The fused form keeps the fp32 activations of the whole call in registers and their int8 form
+// for all of K in LDS.
+inline bool stream32_can_fuse(int64_t M, int64_t K) {
+  const int mt32 = M <= 32 ? 1 : (M <= 64 ? 2 : 4);
+  return M <= 128 && M * K <= kFusedMaxElems && stream32_fused_lds_bytes(mt32, (int)K) <= 64 * 1024;
+}
+
+template <int MT32, int WN, int KW, bool FUSED>
+int launch_stream32(const GemmArgs& a, const float* A, int8_t* aq_out, hipStream_t st) {
+  using Cfg = Stream32Cfg<MT32, WN, KW>;
+  auto kernel = gemm_stream32_kernel<MT32, WN, KW, FUSED>;
+  constexpr int kMaxLds = 64 * 1024 > Cfg::kLdsBytes ? 64 * 1024 : Cfg::kLdsBytes;
+  static const int lds_status = allow_lds(kernel, kMaxLds);
+  if(lds_status != MARIAN_HIP_OK) return lds_status;
+  int lds = FUSED ? stream32_fused_lds_bytes(MT32, a.K) : Cfg::kStageBytes;
+  if(lds < Cfg::kReduceBytes) lds = Cfg::kReduceBytes;
+  int blocks = (a.n_out + Cfg::kColsPerBlock - 1) / Cfg::kColsPerBlock;
+  int m_tiles = FUSED ? 1 : (a.M + MT32 * 32 - 1) / (MT32 * 32);
+  hipLaunchKernelGGL(kernel, dim3(blocks, m_tiles), dim3(kStream32Threads), lds, st, a, A, aq_out);
+  MH_HIP(hipGetLastError());
+  return MARIAN_HIP_OK;
+}
+
+template <int MT32, bool FUSED>
+int launch_stream32_kw(const GemmArgs& a, const float* A, int8_t* aq_out, hipStream_t st, int kw) {
+  switch(kw) {
+    case 1: return launch_stream32<MT32, 8, 1, FUSED>(a, A, aq_out, st);
+    case 2: return launch_stream32<MT32, 4, 2, FUSED>(a, A, aq_out, st);
+    case 4: return launch_stream32<MT32, 2, 4, FUSED>(a, A, aq_out, st);
+    default: return launch_stream32<MT32, 1, 8, FUSED>(a, A, aq_out, st);
+  }
+}
+
+// kw_override: 0 = pick the K split from the number of 32-column weight tiles.
+// mt_override: 0 = activation rows per workgroup chosen here (the fused form takes all of M).
+template <bool FUSED>
+int launch_stream32_auto(const GemmArgs& a, const float* A, int8_t* aq_out, hipStream_t st,
+                         int kw_override, int mt_override = 0) {
+  const int tiles = (a.n_out + 31) / 32;
+  int kw = tiles < 512 ? 8 : (tiles < 1000 ? 4 : (tiles < 4096 ? 2 : 1));
+  if(kw_override) kw = kw_override;
+  while(kw > 1 && a.K / 32 < kw) kw >>= 1;
+  int mt = a.M <= 32 ? 1 : (a.M <= 64 ? 2 : 4);
+  if(!FUSED) {
+    // few weight tiles: split M over workgroups as well, so that more CUs pull on the operands
+    // and each workgroup stages fewer activation rows
+    if(tiles < 256 && mt > 1) mt = 1;
+    if(mt_override) mt = mt_override;
+  }
+  if(mt == 1) return launch_stream32_kw<1, FUSED>(a, A, aq_out, st, kw);
+  if(mt == 2) return launch_stream32_kw<2, FUSED>(a, A, aq_out, st, kw);
+  return launch_stream32_kw<4, FUSED>(a, A, aq_out, st, kw);
+}
+
 int compute_units() {
   static const int cus = [] {
     int dev = 0, n = 0;
@@ -157,13 +215,29 @@ int launch_gemm(const GemmArgs& a, hipStream_t st) {
     case 312: return launch_big<128, 128, 2, 4, 2>(a, st);
     case 313: return launch_big<128, 64, 2, 2, 3>(a, st);
     case 314: return launch_big<128, 64, 4, 2, 2>(a, st);
+    case 501: return launch_stream32_auto<false>(a, nullptr, nullptr, st, 0);
+    case 521: return launch_stream32_auto<false>(a, nullptr, nullptr, st, 0, 1);
+    case 522: return launch_stream32_auto<false>(a, nullptr, nullptr, st, 0, 2);
+    case 524: return launch_stream32_auto<false>(a, nullptr, nullptr, st, 0, 4);
+    case 511: return launch_stream32_auto<false>(a, nullptr, nullptr, st, 1);
+    case 512: return launch_stream32_auto<false>(a, nullptr, nullptr, st, 2);
+    case 514: return launch_stream32_auto<false>(a, nullptr, nullptr, st, 4);
+    case 518: return launch_stream32_auto<false>(a, nullptr, nullptr, st, 8);
     case 401: return launch_persistent<128, 128, 2, 2, 4>(a, st);
     case 402: return launch_persistent<128, 128, 2, 2, 3>(a, st);
     case 403: return launch_persistent<128, 128, 2, 2, 2>(a, st);
     case 404: return launch_persistent<256, 128, 2, 2, 2>(a, st);
     default: break;
   }
-  if(a.M <= 128) return launch_stream_auto(a, st, 0);
+  // Small M (decode): the weights are streamed once, the activations sit in LDS.
+  //  - up to 16 rows, and the 32000-column vocabulary at up to 64 rows: 16x16x64 MFMA kernels
+  //  - otherwise the 32x32x32 MFMA kernel, which also tiles M (shortlisted output layer, M = 256)
+  const int tiles32 = (a.n_out + 31) / 32;
+  if(a.M <= 16) return launch_stream_auto(a, st, 2);
+  if(a.M <= 64 && tiles32 >= 512) return launch_stream_auto(a, st, 1);
+  if(a.M <= 128 && tiles32 >= 512) return launch_stream_auto(a, st, 1);
+  if(a.M <= 128 || (a.M <= 512 && tiles32 < 128))
+    return launch_stream32_auto<false>(a, nullptr, nullptr, st, 0);
   if(a.K % 128 != 0) return launch_tile<4, 4>(a, st);
   // large outputs: 256x256 tiles (one per CU keeps operand traffic lowest); otherwise 128x128
   // tiles with a three-deep LDS ring so that enough loads are in flight per CU
@@ -301,6 +375,34 @@ int marian_hip_int8_prepare_b_quantized_transposed(const int8_t* in, int8_t* out
 int marian_hip_int8_affine(const int8_t* Aq, const int8_t* Bq, const float* bias, float* out,
                            int64_t M, int64_t K, int64_t N, float scale, int relu, void* stream) {
   return run_gemm(Aq, Bq, bias, nullptr, 0, out, M, K, N, scale, relu, 0, stream);
+}
+
+int marian_hip_int8_affine_f32(const float* A, int8_t* Aq, const int8_t* Bq, const float* bias,
+                               const uint32_t* idx, int64_t n_idx, float* out, int64_t M,
+                               int64_t K, int64_t N, float scale, int relu, void* workspace,
+                               size_t workspace_bytes, void* stream) {
+  int st = check_gemm(Aq, Bq, out, bias, idx, n_idx, M, K, N);
+  if(st != MARIAN_HIP_OK) return st;
+  const int64_t n_out = idx ? n_idx : N;
+  if(M == 0) return MARIAN_HIP_OK;
+  if(!A) return MARIAN_HIP_ERR_NULL;
+  if(!aligned(A, 16)) return MARIAN_HIP_ERR_ALIGN;
+  const int which = g_kernel_override.load(std::memory_order_relaxed) % 1000;
+  if(n_out > 0 && stream32_can_fuse(M, K) && which != 600) {
+    GemmArgs a;
+    a.Aq = Aq; a.Bq = Bq; a.bias = bias; a.idx = idx; a.out = out;
+    a.M = (int)M; a.K = (int)K; a.N = (int)N; a.n_out = (int)n_out;
+    a.scale = scale; a.relu = relu ? 1 : 0; a.dump = 0; a.dbg = 0; a.prof = nullptr;
+    int kw = 0;
+    if(which == 611) kw = 1;
+    if(which == 612) kw = 2;
+    if(which == 614) kw = 4;
+    if(which == 618) kw = 8;
+    return launch_stream32_auto<true>(a, A, Aq, reinterpret_cast<hipStream_t>(stream), kw);
+  }
+  st = marian_hip_int8_prepare_a(A, Aq, M, K, workspace, workspace_bytes, stream);
+  if(st != MARIAN_HIP_OK) return st;
+  return run_gemm(Aq, Bq, bias, idx, n_idx, out, M, K, N, scale, relu, 0, stream);
 }
 
 int marian_hip_int8_affine_shortlist(const int8_t* Aq, const int8_t* Bq, const float* bias,

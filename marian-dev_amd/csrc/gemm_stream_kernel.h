@@ -41,6 +41,9 @@ __global__ __launch_bounds__(WN * KW * kWave) void gemm_stream_kernel(GemmArgs a
   const int KS = K / 64;
   const int n_chunks = (KS + Cfg::kChunkSteps - 1) / Cfg::kChunkSteps;
 
+  // quantMult tails are requested first so that their latency overlaps the operand loads
+  const Epilogue ep = make_epilogue(args);
+
   // weight rows of this lane
   const int n_base = (blockIdx.x * WN + wn) * NT * 16;
   const int8_t* wrow[NT];
@@ -154,7 +157,6 @@ __global__ __launch_bounds__(WN * KW * kWave) void gemm_stream_kernel(GemmArgs a
   }
 
   if(kw == 0) {
-    const Epilogue ep = make_epilogue(args);
 #pragma unroll
     for(int nt = 0; nt < NT; ++nt)
 #pragma unroll

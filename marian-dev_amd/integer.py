@@ -167,8 +167,36 @@ def affineOrDot(a, bQuant, bias=None, transA=False, transB=False, scale=1.0, rel
               "Unsupported type {} for Intgemm type??", bQuant.type)
     if transA:
         a = a.transpose(-1, -2)
-    aQuant = prepareA(a)
-    return multiply(aQuant, bQuant, bias, scale=scale, relu=relu, shortlist=shortlist)
+    out, _ = affine_f32(a, bQuant, bias, scale=scale, relu=relu, shortlist=shortlist)
+    return out
+
+
+def affine_f32(a, bQuant, bias=None, scale=1.0, relu=False, shortlist=None):
+    """prepareA node + multiply node through the single C-ABI call marian_hip_int8_affine_f32
+    (one fused kernel for small activations).  Returns (out, aQuant): aQuant is what the
+    prepareA node would have produced."""
+    a = a.contiguous()
+    be = _backend_of(a)
+    aQuant = QTensor.empty(a.shape, Type.intgemm8, a.device)
+    K, N = cols(a), cols(bQuant)
+    _abort_if(rows(bQuant) != K, "Matrix product requires inner dimensions to match: {} vs {}", K, rows(bQuant))
+    M = rows(a) if a.numel() else 0
+    n_out = N if shortlist is None else int(shortlist.numel())
+    out = torch.empty(tuple(a.shape[:-1]) + (n_out,), dtype=torch.float32, device=a.device)
+    bias_ptr = None
+    if bias is not None:
+        _abort_if(bias.dtype != torch.float32 or bias.numel() != N, "bias must be float32 [1, {}]", N)
+        bias = bias.contiguous()
+        bias_ptr = bias.data_ptr()
+    if shortlist is not None:
+        _abort_if(shortlist.dtype not in (torch.int32, torch.uint32), "shortlist ids must be uint32, got {}", shortlist.dtype)
+    st = be.lib.marian_hip_int8_affine_f32(
+        a.data_ptr(), aQuant.data_ptr(), bQuant.data_ptr(), bias_ptr,
+        None if shortlist is None else shortlist.data_ptr(), n_out if shortlist is not None else 0,
+        out.data_ptr(), M, K, N, scale, int(relu), be.workspace.data_ptr(), be.workspace_bytes,
+        be.stream())
+    _lib.check(st, "affineOrDot")
+    return out, aQuant
 
 
 def multiply(aQuant, bQuant, bias=None, scale=1.0, relu=False, shortlist=None):

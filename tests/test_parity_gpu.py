@@ -87,7 +87,7 @@ def test_prepare_b_bit_exact(integer, orc, synth, K, N):
 
 # ---------------------------------------------------------------- multiply: int32 and fp32
 
-KERNELS = [0, 101, 102, 201, 202, 203, 204, 301, 302, 303, 304, 305, 306, 307, 308, 401, 402, 403, 404]
+KERNELS = [0, 101, 102, 501, 511, 512, 514, 518, 521, 522, 524, 201, 202, 203, 204, 301, 302, 303, 304, 305, 306, 307, 308, 401, 402, 403, 404]
 
 
 def run_case(integer, orc, synth, seed, M, K, N, kernel, bias_on=True, relu=False, scale=1.0):
@@ -117,12 +117,52 @@ def test_multiply_all_kernels_small_m(integer, orc, synth, M, K, N, kernel):
     run_case(integer, orc, synth, 300 + M + N, M, K, N, kernel, bias_on=True, relu=(M % 2 == 0))
 
 
-@pytest.mark.parametrize("kernel", [0, 201, 202, 203, 204, 301, 302, 303, 304, 305, 306, 307, 308, 401, 402, 403, 404])
+@pytest.mark.parametrize("kernel", [0, 501, 512, 521, 522, 524, 201, 202, 203, 204, 301, 302, 303, 304, 305, 306, 307, 308, 401, 402, 403, 404])
 @pytest.mark.parametrize("M,K,N", [(129, 64, 8), (256, 1024, 504), (300, 320, 1000), (513, 128, 264)])
 def test_multiply_tile_kernels_ragged(integer, orc, synth, M, K, N, kernel):
     say("multiply ragged", M, K, N, "kernel", kernel)
     run_case(integer, orc, synth, 400 + M + N, M, K, N, kernel, bias_on=(N % 16 == 8), relu=True,
              scale=0.5)
+
+
+@pytest.mark.parametrize("kernel", [0, 600, 611, 612, 614, 618])
+@pytest.mark.parametrize("M,K,N", [(1, 64, 8), (1, 512, 512), (4, 2048, 512), (16, 512, 1536),
+                                   (33, 192, 136), (64, 512, 2048), (100, 256, 1000), (128, 256, 64),
+                                   (16, 1024, 32000), (7, 4096, 64)])
+def test_fused_affine_f32(integer, orc, synth, M, K, N, kernel):
+    """prepareA + multiply in one call (one fused kernel where the activations are small):
+    output, quantized activations and quantMult equal those of the two separate steps."""
+    from conftest import load
+    lib = load("_lib").lib()
+    say("fused", M, K, N, "kernel", kernel)
+    A, W, bias = inputs(synth, 500 + M + N, M, K, N)
+    Aq_h, Bq_h = orc.prepare_a(A), orc.prepare_b(W)
+    relu = (M % 2 == 1)
+    want, _ = orc.affine(Aq_h, Bq_h, bias, M, K, N, 0.5, relu)
+    Bq = upload_q(integer, Bq_h, (K, N))
+    prev = lib.marian_hip_int8_set_kernel(kernel)
+    try:
+        out, Aq = integer.affine_f32(dev(A), Bq, dev(bias), scale=0.5, relu=relu)
+        out = out.cpu().numpy()
+        got_aq = Aq.numpy()
+    finally:
+        lib.marian_hip_int8_set_kernel(prev)
+    assert np.array_equal(got_aq, Aq_h), "quantized activations / quantMult of the fused call"
+    assert np.array_equal(out, want)
+
+
+def test_fused_shortlist(integer, orc, synth):
+    import torch
+    say("fused shortlist")
+    M, K, N = 8, 512, 4096
+    A, W, bias = inputs(synth, 606, M, K, N)
+    Aq_h, Bq_h = orc.prepare_a(A), orc.prepare_b(W)
+    idx = synth.shortlist(606, N, 100, 300)
+    want, _ = orc.affine_shortlist(Aq_h, Bq_h, bias, idx, M, K, N)
+    Bq = upload_q(integer, Bq_h, (K, N))
+    didx = torch.from_numpy(idx.view(np.int32)).cuda()
+    out, Aq = integer.affine_f32(dev(A), Bq, dev(bias), shortlist=didx)
+    assert np.array_equal(Aq.numpy(), Aq_h) and np.array_equal(out.cpu().numpy(), want)
 
 
 def test_config1_single_affine_end_to_end(integer, orc, synth):
