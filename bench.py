@@ -31,6 +31,14 @@ PKG = "marian-dev_amd"
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 INT8_PEAK_TOPS = 5000.0      # MI355X dense int8 MFMA, published (5.0 POP/s)
 
+# HBM bytes per launch of the kernels named here, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# runs of `bench.py --pmc-probe` (KiB per dispatch, scaled by the same counters' reading for a
+# plain copy of known size); the runs are summarised under profiles/.  None = not measured.
+MEASURED_TRAFFIC = {
+    # (8700.2 KiB FETCH_SIZE x 1.9992 + 8032.1 KiB WRITE_SIZE) per dispatch
+    "stream32_fused_M64_K512_N32000": int((8700.2 * 1.9992 + 8032.1) * 1024),
+}
+
 DECODE_SHAPES = [(512, 1536), (512, 512), (512, 2048), (2048, 512), (512, 32000)]
 DECODE_M = [1, 4, 16, 64]
 
@@ -121,26 +129,25 @@ def time_graphs(torch, graphs, steps, warmup):
 
 
 def per_launch_ms(torch, launches, repeat):
-    """Average duration of single launches from HIP events recorded on the launch stream.  The
-    launches are queued behind a spinning kernel so the host never starves the stream and each
-    event pair brackets exactly one kernel."""
+    """Average duration of one launch from HIP events recorded on the launch stream: each event
+    pair brackets one pass over `launches` (distinct weight copies) issued back to back, and the
+    passes are queued behind a spinning kernel so the host never starves the stream.  Returns
+    (mean, median) over the passes, per launch, in ms."""
     stream = torch.cuda.current_stream()
-    n = len(launches) * repeat
-    starts = [torch.cuda.Event(enable_timing=True) for _ in range(n)]
-    ends = [torch.cuda.Event(enable_timing=True) for _ in range(n)]
+    n = len(launches)
+    starts = [torch.cuda.Event(enable_timing=True) for _ in range(repeat)]
+    ends = [torch.cuda.Event(enable_timing=True) for _ in range(repeat)]
     for f in launches:
         f()
     torch.cuda.synchronize()
-    torch.cuda._sleep(int(2.0e9 * 0.02 * max(1, n // 100)))  # ~20 ms per 100 launches
-    k = 0
-    for _ in range(repeat):
+    torch.cuda._sleep(int(2.0e9 * 0.02 * max(1, n * repeat // 100)))  # ~20 ms per 100 launches
+    for r in range(repeat):
+        starts[r].record(stream)
         for f in launches:
-            starts[k].record(stream)
             f()
-            ends[k].record(stream)
-            k += 1
+        ends[r].record(stream)
     torch.cuda.synchronize()
-    d = np.array([starts[i].elapsed_time(ends[i]) for i in range(n)])
+    d = np.array([starts[r].elapsed_time(ends[r]) / n for r in range(repeat)])
     return float(d.mean()), float(np.median(d))
 
 
@@ -177,12 +184,37 @@ def cpu_baseline(seconds=12.0):
             "sample": "%d passes of the same 20-shape decode sweep in %.1f s on one core" % (passes, dt)}
 
 
+def pmc_probe(torch, integer, lib, be):
+    """A few launches each of: a plain elementwise copy of 64 MiB (reads 64 MiB, writes 64 MiB:
+    the yardstick the counters are scaled by), the fused decode kernel on the vocabulary
+    projection at M = 64, and the two encoder-size GEMMs.  Each launch uses a fresh weight copy."""
+    src = torch.randn(16 * 1024 * 1024, device="cuda")
+    dst = torch.empty_like(src)
+    for _ in range(3):
+        torch.add(src, 1.0, out=dst)
+    torch.cuda.synchronize()
+    o = Op(torch, integer, 64, 512, 32000, copies=6, seed=43)
+    for c in range(6):
+        o.launch_fused(lib, be, c)
+    torch.cuda.synchronize()
+    for (M, K, N) in [(4096, 1024, 4096), (4096, 4096, 1024)]:
+        e = Op(torch, integer, M, K, N, relu=True, copies=4, seed=77)
+        e.launch(lib, be, 0, prepare=True, gemm=False)
+        for c in range(4):
+            e.launch(lib, be, c, prepare=False)
+        torch.cuda.synchronize()
+        del e
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--pmc-probe", action="store_true",
+                    help="launch the dominant kernels and a plain copy a few times and exit "
+                         "(for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)")
     ap.add_argument("--only", default="", help="comma list of extra workloads: encoder,shortlist,big")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -196,6 +228,10 @@ def main():
     torch.cuda.set_device(0)
     be = integer.Backend.get("cuda:0")
     extras = set(x for x in args.only.split(",") if x) or {"encoder", "shortlist", "big"}
+
+    if args.pmc_probe:
+        pmc_probe(torch, integer, lib, be)
+        return
 
     # ---------------- headline: transformer-base decode sweep -------------------------------
     sweep_bytes = sum(K * N for K, N in DECODE_SHAPES) * len(DECODE_M)
@@ -223,18 +259,20 @@ def main():
     eager_ms = (time.perf_counter() - t0) / 20 * 1e3
 
     # ---------------- roofline of the dominant kernel ----------------------------------------
-    # vocabulary projection of the sweep at M = 64: 16.4 MB of int8 weights per launch
+    # vocabulary projection of the sweep at M = 64 (16.4 MB of int8 weights, 8.2 MB of output):
+    # the fused quantize + GEMM kernel, which moves exactly the algorithmic bytes of the call
     dom = [o for o in ops_list if o.N == 32000 and o.M == 64][0]
-    dom.launch(lib, be, 0, prepare=True, gemm=False)
     mean_ms, med_ms = per_launch_ms(
-        torch, [(lambda c=c: dom.launch(lib, be, c, prepare=False)) for c in range(sets)], 6)
-    dom_bytes = gemm_kernel_bytes(dom.M, dom.K, dom.N)
+        torch, [(lambda c=c: dom.launch_fused(lib, be, c)) for c in range(sets)], 12)
+    dom_bytes = algorithmic_bytes(dom.M, dom.K, dom.N)
     achieved = dom_bytes / (mean_ms * 1e-3) / 1e9
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
-                "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
-                "kernel": "gemm_stream_kernel M=64 K=512 N=32000",
+                "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+                "traffic": MEASURED_TRAFFIC.get("stream32_fused_M64_K512_N32000"),
+                "kernel": "gemm_stream32_kernel<2,4,2,fused> M=64 K=512 N=32000",
                 "bytes_per_launch": dom_bytes, "avg_launch_us": round(mean_ms * 1e3, 3),
-                "median_launch_us": round(med_ms * 1e3, 3)}
+                "median_launch_us": round(med_ms * 1e3, 3),
+                "launches_timed": 12 * sets}
 
     per_shape = {}
     for (K, N) in DECODE_SHAPES:
@@ -243,10 +281,11 @@ def main():
             o.launch(lib, be, 0, prepare=True, gemm=False)
             g_ms, _ = per_launch_ms(
                 torch, [(lambda c=c, o=o: o.launch(lib, be, c, prepare=False)) for c in range(sets)], 3)
-            p_ms, _ = per_launch_ms(torch, [(lambda o=o: o.launch(lib, be, 0, gemm=False))], 12)
+            f_ms, _ = per_launch_ms(
+                torch, [(lambda c=c, o=o: o.launch_fused(lib, be, c)) for c in range(sets)], 3)
             per_shape["M%d_%dx%d" % (M, K, N)] = {
-                "gemm_us": round(g_ms * 1e3, 2), "prepare_a_us": round(p_ms * 1e3, 2),
-                "gemm_hbm_frac": round(gemm_kernel_bytes(M, K, N) / (g_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+                "affine_f32_us": round(f_ms * 1e3, 2), "gemm_only_us": round(g_ms * 1e3, 2),
+                "affine_hbm_frac": round(algorithmic_bytes(M, K, N) / (f_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
 
     out = {
         "metric": "int8 affine TOPS & % roofline; transformer-big int8 decode tokens/sec",

@@ -235,7 +235,7 @@ __global__ __launch_bounds__(kStream32Threads) void gemm_stream32_kernel(GemmArg
     }
     __syncthreads();
     if(kw == 0) {
-#pragma unroll
+#pragma unroll 1   // one partial sum at a time keeps the register count down
       for(int r = 1; r < KW; ++r)
 #pragma unroll
         for(int mt = 0; mt < MT32; ++mt)

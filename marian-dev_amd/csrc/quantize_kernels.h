@@ -21,12 +21,24 @@ __device__ __forceinline__ int quantize_one(float x, float qm) {
   return (fabsf(v) < 2147483648.0f) ? q : -127;
 }
 
+// Same result as quantize_one in the low byte of the returned word, in five VALU operations:
+// clamping to [-127, 127] first commutes with rounding (the bounds are integers; med3 returns
+// -127 for NaN), and adding 1.5 * 2^23 rounds to nearest-even with the integer landing in the
+// low mantissa bits (two's complement in the low byte).  Products >= 2^31 (only possible for
+// non-finite inputs) follow the x86 conversion and give -127.
+__device__ __forceinline__ uint32_t quantize_low_byte(float x, float qm) {
+  float v = x * qm;
+  float c = __builtin_amdgcn_fmed3f(v, -127.0f, 127.0f);
+  c = (v >= 2147483648.0f) ? -127.0f : c;
+  return __float_as_uint(c + 12582912.0f);
+}
+
 __device__ __forceinline__ uint32_t quantize_pack4(v4f x, float qm) {
-  uint32_t b0 = (uint32_t)quantize_one(x.x, qm) & 0xffu;
-  uint32_t b1 = (uint32_t)quantize_one(x.y, qm) & 0xffu;
-  uint32_t b2 = (uint32_t)quantize_one(x.z, qm) & 0xffu;
-  uint32_t b3 = (uint32_t)quantize_one(x.w, qm) & 0xffu;
-  return b0 | (b1 << 8) | (b2 << 16) | (b3 << 24);
+  const uint32_t b0 = quantize_low_byte(x.x, qm), b1 = quantize_low_byte(x.y, qm);
+  const uint32_t b2 = quantize_low_byte(x.z, qm), b3 = quantize_low_byte(x.w, qm);
+  const uint32_t lo = __builtin_amdgcn_perm(b1, b0, 0x0c0c0400u);  // [b0.0, b1.0, 0, 0]
+  const uint32_t hi = __builtin_amdgcn_perm(b3, b2, 0x0c0c0400u);
+  return __builtin_amdgcn_perm(hi, lo, 0x05040100u);               // [lo.0, lo.1, hi.0, hi.1]
 }
 
 __device__ __forceinline__ float abs4max(v4f x, float m) {
