@@ -374,3 +374,33 @@ def test_type_errors_like_the_reference(integer):
         integer.prepareA(torch.ones(2, 100, device="cuda"))
     empty = integer.affine(torch.ones(0, 64, device="cuda"), b, None)
     assert tuple(empty.shape) == (0, 8)
+
+
+def test_model_file_weights_run_verbatim(integer, orc, synth, tmp_path):
+    """A Type::intgemm8 item read from a .bin file is uploaded byte for byte and multiplied."""
+    from conftest import load
+    B = load("binary")
+    say("bin file -> gpu")
+    M, K, N = 12, 128, 40
+    A, W, bias = inputs(synth, 808, M, K, N)
+    path = os.path.join(tmp_path, "m.bin")
+    B.save_items(path, [B.intgemm8_item("decoder_l1_ffn_W1", orc.prepare_b(W), (K, N)),
+                        B.float_item("decoder_l1_ffn_b1", bias.reshape(1, N))])
+    w, b = B.load_items(path)
+    Bq = integer.QTensor.from_numpy(w.bytes, w.shape, w.type, "cuda")
+    got = integer.affineWithReluDropout(dev(A), Bq, dev(b.bytes.view(f32)[:N].copy())).cpu().numpy()
+    want, _ = orc.affine(orc.prepare_a(A), orc.prepare_b(W), bias, M, K, N, 1.0, True)
+    assert np.array_equal(got, want)
+
+
+def test_cpp_host_wrappers(integer):
+    """The C++ mirror of the intgemm glue (host/hip_int8_interface.h) against its own CPU
+    restatement; built by __graft_entry__.build()."""
+    import subprocess
+    from conftest import ROOT
+    exe = os.path.join(ROOT, "marian-dev_amd", "host", "host_check")
+    assert os.path.exists(exe), "host_check not built"
+    say("host_check")
+    r = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=120)
+    print(r.stdout)
+    assert r.returncode == 0 and "-> OK" in r.stdout, r.stdout
