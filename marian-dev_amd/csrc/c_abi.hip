@@ -70,11 +70,11 @@ int launch_tile(const GemmArgs& a, hipStream_t st) {
   return MARIAN_HIP_OK;
 }
 
-template <int BM, int BN, int WM, int WN, int NSTAGE>
+template <int BM, int BN, int WM, int WN, int NSTAGE, bool PAIRED = true>
 int launch_big(const GemmArgs& a, hipStream_t st) {
   using Cfg = BigCfg<BM, BN, WM, WN, NSTAGE>;
   if(a.K % Cfg::BK != 0) return launch_tile<4, 4>(a, st);  // this family needs K % 128 == 0
-  auto kernel = gemm_mfma32_kernel<BM, BN, WM, WN, NSTAGE>;
+  auto kernel = gemm_mfma32_kernel<BM, BN, WM, WN, NSTAGE, PAIRED>;
   static const int lds_status = allow_lds(kernel, Cfg::kLdsBytes);
   if(lds_status != MARIAN_HIP_OK) return lds_status;
   int tiles_n = (a.n_out + BN - 1) / BN;
@@ -153,22 +153,24 @@ int compute_units() {
   return cus;
 }
 
-template <int BM, int BN, int WM, int WN, int NSTAGE>
-int launch_persistent(const GemmArgs& a, hipStream_t st) {
-  using Cfg = PersistCfg<BM, BN, WM, WN, NSTAGE>;
+template <int BM, int BN, int WM, int WN, int NSTAGE, bool DIRECT = false>
+int launch_persistent(const GemmArgs& a, hipStream_t st, int per_cu = 1, int stagger = 0) {
+  using Cfg = PersistCfg<BM, BN, WM, WN, NSTAGE, DIRECT>;
   // needs K % 128 == 0, at least NSTAGE K blocks per tile and a 16-byte aligned bias
   if(a.K % Cfg::BK != 0 || a.K / Cfg::BK < NSTAGE || (a.bias && !aligned(a.bias, 16)))
     return launch_big<BM, BN, WM, WN, 2>(a, st);
-  auto dense = gemm_persistent_kernel<BM, BN, WM, WN, NSTAGE, false>;
-  auto gather = gemm_persistent_kernel<BM, BN, WM, WN, NSTAGE, true>;
+  auto dense = gemm_persistent_kernel<BM, BN, WM, WN, NSTAGE, false, DIRECT>;
+  auto gather = gemm_persistent_kernel<BM, BN, WM, WN, NSTAGE, true, DIRECT>;
   static const int lds_status = allow_lds(dense, Cfg::kLdsBytes) | allow_lds(gather, Cfg::kLdsBytes);
   if(lds_status != MARIAN_HIP_OK) return lds_status;
   int tiles_n = (a.n_out + BN - 1) / BN;
   int tiles_m = (a.M + BM - 1) / BM;
   int total = tiles_n * tiles_m;
-  int grid = total < compute_units() ? total : compute_units();
+  int slots = compute_units() * per_cu;
+  int grid = total < slots ? total : slots;
+  if(grid < slots) stagger = 0;   // fewer workgroups than slots: no two share a CU by design
   hipLaunchKernelGGL(a.idx ? gather : dense, dim3(grid), dim3(Cfg::kThreads), Cfg::kLdsBytes, st, a,
-                     tiles_n, tiles_m);
+                     tiles_n, tiles_m, stagger);
   MH_HIP(hipGetLastError());
   return MARIAN_HIP_OK;
 }
@@ -206,7 +208,10 @@ int launch_gemm(const GemmArgs& a, hipStream_t st) {
     case 303: return launch_big<256, 128, 2, 2, 2>(a, st);
     case 304: return launch_big<256, 128, 4, 2, 2>(a, st);
     case 305: return launch_big<128, 256, 2, 2, 2>(a, st);
-    case 306: return launch_big<256, 256, 2, 2, 2>(a, st);
+    case 306: return launch_big<256, 256, 2, 2, 2, false>(a, st);
+    case 315: return launch_big<256, 256, 2, 4, 2, false>(a, st);
+    case 316: return launch_big<256, 128, 2, 2, 2, false>(a, st);
+    case 317: return launch_big<128, 256, 2, 2, 2, false>(a, st);
     case 307: return launch_big<128, 128, 2, 2, 3>(a, st);
     case 308: return launch_big<256, 128, 2, 2, 3>(a, st);
     case 309: return launch_big<128, 64, 2, 2, 2>(a, st);
@@ -223,6 +228,12 @@ int launch_gemm(const GemmArgs& a, hipStream_t st) {
     case 512: return launch_stream32_auto<false>(a, nullptr, nullptr, st, 2);
     case 514: return launch_stream32_auto<false>(a, nullptr, nullptr, st, 4);
     case 518: return launch_stream32_auto<false>(a, nullptr, nullptr, st, 8);
+    case 411: return launch_persistent<128, 128, 2, 2, 2, true>(a, st, 2, 0);
+    case 412: return launch_persistent<128, 128, 2, 2, 2, true>(a, st, 2, 1);
+    case 413: return launch_persistent<128, 128, 2, 2, 2, true>(a, st, 2, 2);
+    case 414: return launch_persistent<128, 128, 2, 2, 2, true>(a, st, 2, 3);
+    case 415: return launch_persistent<128, 128, 2, 2, 2, true>(a, st, 1, 0);
+    case 416: return launch_persistent<128, 128, 2, 2, 4, true>(a, st, 1, 0);
     case 401: return launch_persistent<128, 128, 2, 2, 4>(a, st);
     case 402: return launch_persistent<128, 128, 2, 2, 3>(a, st);
     case 403: return launch_persistent<128, 128, 2, 2, 2>(a, st);
@@ -392,7 +403,8 @@ int marian_hip_int8_affine_f32(const float* A, int8_t* Aq, const int8_t* Bq, con
     GemmArgs a;
     a.Aq = Aq; a.Bq = Bq; a.bias = bias; a.idx = idx; a.out = out;
     a.M = (int)M; a.K = (int)K; a.N = (int)N; a.n_out = (int)n_out;
-    a.scale = scale; a.relu = relu ? 1 : 0; a.dump = 0; a.dbg = 0; a.prof = nullptr;
+    a.scale = scale; a.relu = relu ? 1 : 0; a.dump = 0; a.dbg = 0;
+    a.prof = g_prof.load(std::memory_order_relaxed);
     int kw = 0;
     if(which == 611) kw = 1;
     if(which == 612) kw = 2;

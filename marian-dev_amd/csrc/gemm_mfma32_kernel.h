@@ -19,6 +19,8 @@
 // Requires K % 128 == 0.
 #pragma once
 
+#include <type_traits>
+
 #include "int8_common.h"
 
 namespace marian_hip {
@@ -97,7 +99,11 @@ __device__ __forceinline__ void store_tile32_any(const v16i& acc, char* out, siz
   else store_tile32<false, false, false, GUARD>(acc, out, row_bytes, unquant, bias_v, rows_left, col_valid);
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int NSTAGE>
+// PAIRED: fragments of two K sub-steps are requested two sub-steps ahead (four fragment sets in
+// registers; needed when a sub-step has only a few MFMAs to cover the LDS latency).  Otherwise the
+// fragments of sub-step s+1 are requested during sub-step s (two sets; for large wave tiles, whose
+// accumulators leave no room for four).
+template <int BM, int BN, int WAVES_M, int WAVES_N, int NSTAGE, bool PAIRED = true>
 __global__ __launch_bounds__(WAVES_M * WAVES_N * kWave) void gemm_mfma32_kernel(
     GemmArgs args, int tiles_n, int tiles_m) {
   using Cfg = BigCfg<BM, BN, WAVES_M, WAVES_N, NSTAGE>;
@@ -105,6 +111,7 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * kWave) void gemm_mfma32_kernel(
   const unsigned lds_base = (unsigned)(size_t)lds;  // LDS byte address of the ring
 
   const long long t_start = clock64();
+  const long long w_start = wall_clock64();
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
   const int lane = tid % kWave;
@@ -146,14 +153,15 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * kWave) void gemm_mfma32_kernel(
     }
     goff[j] = src * K + chunk * 16;
   }
+  auto issue_one = [&](int kb, int stage, int j) {
+    const int8_t* base = (j < Cfg::kLoadsA) ? args.Aq : args.Bq;
+    const int8_t* src = base + (size_t)(unsigned)goff[j] + (size_t)kb * Cfg::BK;
+    global_load_lds16(src, lds_base + stage * Cfg::kStageBytes + (j * Cfg::kWaves + wave) * 1024);
+  };
   auto issue = [&](int kb) {
     const int stage = kb % NSTAGE;
 #pragma unroll
-    for(int j = 0; j < Cfg::kLoads; ++j) {
-      const int8_t* base = (j < Cfg::kLoadsA) ? args.Aq : args.Bq;
-      const int8_t* src = base + (size_t)(unsigned)goff[j] + (size_t)kb * Cfg::BK;
-      global_load_lds16(src, lds_base + stage * Cfg::kStageBytes + (j * Cfg::kWaves + wave) * 1024);
-    }
+    for(int j = 0; j < Cfg::kLoads; ++j) issue_one(kb, stage, j);
   };
 
   // ---- fragment addressing: lane (li, lg) reads row li of a 32-row tile, chunk kk*2 + lg ----
@@ -163,7 +171,7 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * kWave) void gemm_mfma32_kernel(
   const int a_row0 = wm * Cfg::WTM * 32;          // first activation row of this wave in a stage
   const int b_row0 = BM + wn * Cfg::WTN * 32;     // first weight row
 
-  v4i af[4][Cfg::WTM], bf[4][Cfg::WTN];
+  v4i af[PAIRED ? 4 : 2][Cfg::WTM], bf[PAIRED ? 4 : 2][Cfg::WTN];
   auto read_frags = [&](int stage, int kk, int set) {
     const int8_t* buf = lds + stage * Cfg::kStageBytes + frag_off[kk];
 #pragma unroll
@@ -174,6 +182,16 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * kWave) void gemm_mfma32_kernel(
       bf[set][b] = *reinterpret_cast<const v4i*>(buf + (b_row0 + b * 32) * 128);
   };
 
+  // fragment `idx` of the pair of sub-steps (0, 1): idx = set * (WTM + WTN) + f
+  auto read_one = [&](int stage, int idx) {
+    const int set = idx / (Cfg::WTM + Cfg::WTN), f = idx % (Cfg::WTM + Cfg::WTN);
+    const int8_t* buf = lds + stage * Cfg::kStageBytes + frag_off[set];
+    if(f < Cfg::WTM)
+      af[set][f] = *reinterpret_cast<const v4i*>(buf + (a_row0 + f * 32) * 128);
+    else
+      bf[set][f - Cfg::WTM] = *reinterpret_cast<const v4i*>(buf + (b_row0 + (f - Cfg::WTM) * 32) * 128);
+  };
+
   v16i acc[Cfg::WTM][Cfg::WTN];
 #pragma unroll
   for(int a = 0; a < Cfg::WTM; ++a)
@@ -181,6 +199,33 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * kWave) void gemm_mfma32_kernel(
     for(int b = 0; b < Cfg::WTN; ++b)
 #pragma unroll
       for(int v = 0; v < 16; ++v) acc[a][b][v] = 0;
+  // Sub-steps 2 and 3 of a block as 2 * WTM * WTN slots of one MFMA each.  Every slot first issues
+  // its share of the global->LDS loads of block kb + NSTAGE and of the LDS reads of the next
+  // block's sub-steps 0 and 1; their issue time then hides under the MFMA of the previous slot.
+  // (The loads are inline assembly, so the order is pinned slot by slot.)
+  auto second_half = [&](bool do_issue, int kb) {
+    constexpr int nM = Cfg::WTM * Cfg::WTN;
+    constexpr int LPS = (Cfg::kLoads + 2 * nM - 1) / (2 * nM);
+    constexpr int nR = 2 * (Cfg::WTM + Cfg::WTN);
+    constexpr int RPS = (nR + nM - 1) / nM;
+    const int ld_stage = (kb + NSTAGE) % NSTAGE, rd_stage = (kb + 1) % NSTAGE;
+#pragma unroll
+    for(int slot = 0; slot < 2 * nM; ++slot) {
+      if(do_issue) {   // wave-uniform: only the load is skipped, the MFMA code exists once
+#pragma unroll
+        for(int l = 0; l < LPS; ++l)
+          if(slot * LPS + l < Cfg::kLoads) issue_one(kb + NSTAGE, ld_stage, slot * LPS + l);
+      }
+      if(slot < nM) {
+#pragma unroll
+        for(int r = 0; r < RPS; ++r)
+          if(slot * RPS + r < nR) read_one(rd_stage, slot * RPS + r);
+      }
+      const int set = slot < nM ? 2 : 3, i = slot % nM, a = i / Cfg::WTN, b = i % Cfg::WTN;
+      acc[a][b] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[set][a], bf[set][b], acc[a][b], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
   auto multiply = [&](int set) {
 #pragma unroll
     for(int a = 0; a < Cfg::WTM; ++a)
@@ -212,45 +257,74 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * kWave) void gemm_mfma32_kernel(
   else wait_vmcnt<0>();
   __builtin_amdgcn_s_barrier();
   const long long t_prologue = clock64();
-  read_frags(0, 0, 0);
-  read_frags(0, 1, 1);
+  if constexpr(!PAIRED) {
+    auto spread = [&]() {   // one LDS read after each MFMA
+#pragma unroll
+      for(int i = 0; i < Cfg::WTM + Cfg::WTN; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      }
+    };
+    read_frags(0, 0, 0);
+    for(int kb = 0; kb < KB; ++kb) {
+      const int stage = kb % NSTAGE;
+      read_frags(stage, 1, 1);
+      multiply(0);
+      spread();
+      read_frags(stage, 2, 0);
+      multiply(1);
+      spread();
+      read_frags(stage, 3, 1);
+      multiply(0);
+      spread();
+      if(kb + 1 < KB) {
+        __builtin_amdgcn_sched_barrier(0);
+        wait_lgkmcnt0();
+        if(NSTAGE == 3 && kb + 2 < KB) wait_vmcnt<Cfg::kLoads>();
+        else wait_vmcnt<0>();
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+        if(kb + NSTAGE < KB && !(args.dbg & 1)) issue(kb + NSTAGE);
+        read_frags((kb + 1) % NSTAGE, 0, 0);
+      }
+      multiply(1);
+      spread();
+    }
+  } else {
+    read_frags(0, 0, 0);
+    read_frags(0, 1, 1);
 
-  for(int kb = 0; kb + 1 < KB; ++kb) {
-    const int stage = kb % NSTAGE;
-    read_frags(stage, 2, 2);
-    read_frags(stage, 3, 3);
-    multiply(0);
-    interleave();
-    multiply(1);
-    mfma_only();
-    // All reads of this block were issued one sub-step ago; once they have returned the stage
-    // is free.  Block kb+1 must have landed (this wave's share); later blocks may be in flight.
-    __builtin_amdgcn_sched_barrier(0);  // keep the MFMAs above on this side of the wait
-    wait_lgkmcnt0();
-    if(NSTAGE == 3 && kb + 2 < KB) wait_vmcnt<Cfg::kLoads>();
-    else wait_vmcnt<0>();
-    __builtin_amdgcn_s_barrier();
-    __builtin_amdgcn_sched_barrier(0);
-    if(kb + NSTAGE < KB && !(args.dbg & 1)) issue(kb + NSTAGE);
-    read_frags((kb + 1) % NSTAGE, 0, 0);
-    read_frags((kb + 1) % NSTAGE, 1, 1);
-    multiply(2);
-    interleave();
-    multiply(3);
-    mfma_only();
-  }
-  {
-    const int stage = (KB - 1) % NSTAGE;
-    read_frags(stage, 2, 2);
-    read_frags(stage, 3, 3);
-    multiply(0);
-    interleave();
-    multiply(1);
-    mfma_only();
-    multiply(2);
-    mfma_only();
-    multiply(3);
-    mfma_only();
+    for(int kb = 0; kb + 1 < KB; ++kb) {
+      const int stage = kb % NSTAGE;
+      read_frags(stage, 2, 2);
+      read_frags(stage, 3, 3);
+      multiply(0);
+      interleave();
+      multiply(1);
+      mfma_only();
+      // All reads of this block were issued one sub-step ago; once they have returned the stage
+      // is free.  Block kb+1 must have landed (this wave's share); later blocks may be in flight.
+      __builtin_amdgcn_sched_barrier(0);  // keep the MFMAs above on this side of the wait
+      wait_lgkmcnt0();
+      if(NSTAGE == 3 && kb + 2 < KB) wait_vmcnt<Cfg::kLoads>();
+      else wait_vmcnt<0>();
+      __builtin_amdgcn_s_barrier();
+      __builtin_amdgcn_sched_barrier(0);
+      second_half(kb + NSTAGE < KB && !(args.dbg & 1), kb);
+    }
+    {
+      const int stage = (KB - 1) % NSTAGE;
+      read_frags(stage, 2, 2);
+      read_frags(stage, 3, 3);
+      multiply(0);
+      interleave();
+      multiply(1);
+      mfma_only();
+      multiply(2);
+      mfma_only();
+      multiply(3);
+      mfma_only();
+    }
   }
 
   const long long t_main = clock64();
@@ -284,7 +358,7 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * kWave) void gemm_mfma32_kernel(
   }
   if(args.prof && tid == 0) {
     long long* p = args.prof + (size_t)blockIdx.x * 8;
-    p[0] = t_start; p[1] = t_prologue; p[2] = t_main; p[3] = clock64();
+    p[0] = t_start; p[1] = t_prologue; p[2] = t_main; p[3] = clock64(); p[6] = w_start; p[7] = wall_clock64();
   }
 }
 

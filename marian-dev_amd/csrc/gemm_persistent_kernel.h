@@ -23,7 +23,11 @@
 
 namespace marian_hip {
 
-template <int BM_, int BN_, int WAVES_M, int WAVES_N, int NSTAGE_>
+// DIRECT_: write accumulators straight from registers (4-byte stores, a half-wave covers 128 bytes
+// of an output row) instead of transposing through LDS; needs no LDS buffer, so two workgroups fit
+// on a CU, but its 16 stores per 32x32 tile are too many to count in vmcnt, so the loads of the
+// next tile are only confirmed after the stores have retired.
+template <int BM_, int BN_, int WAVES_M, int WAVES_N, int NSTAGE_, bool DIRECT_ = false>
 struct PersistCfg {
   static constexpr int BM = BM_, BN = BN_, BK = 128, NSTAGE = NSTAGE_;
   static constexpr int kWaves = WAVES_M * WAVES_N;
@@ -35,14 +39,15 @@ struct PersistCfg {
   static constexpr int kLoads = (kRows / 8) / kWaves;     // wave loads per K block
   static constexpr int kLoadsA = (BM / 8) / kWaves;
   static constexpr int kStoresPerTile = 4 * WTM * WTN;    // 16-byte stores per lane per tile
-  static constexpr int kEpiBytes = kWaves * 4096;         // one 32x32 fp32 tile per wave
+  static constexpr bool DIRECT = DIRECT_;
+  static constexpr int kEpiBytes = DIRECT ? 0 : kWaves * 4096;   // one 32x32 fp32 tile per wave
   static constexpr int kBiasBytes = 2 * 1024;              // bias of two consecutive tiles
   static constexpr int kLdsBytes = NSTAGE * kStageBytes + kEpiBytes + kBiasBytes;
   static_assert(BN <= 256, "one wave load stages the bias of a tile");
   static_assert((BM / 8) % kWaves == 0 && (BN / 8) % kWaves == 0, "tile rows vs waves");
   static_assert(BM % (WAVES_M * 32) == 0 && BN % (WAVES_N * 32) == 0, "tile vs wave grid");
   static_assert(NSTAGE >= 2 && NSTAGE <= 4, "two to four LDS stages");
-  static_assert((NSTAGE - 2) * kLoads + kStoresPerTile <= 63, "vmcnt is a 6-bit counter");
+  static_assert(DIRECT || (NSTAGE - 2) * kLoads + kStoresPerTile <= 63, "vmcnt is a 6-bit counter");
   static_assert(kLoads % 2 == 0 && kStoresPerTile % 2 == 0, "wait counts are even");
 };
 
@@ -78,13 +83,15 @@ __device__ __forceinline__ void persistent_tile_coords(int round, int block, int
 // GATHER selects the shortlist form (weight rows and bias picked through args.idx).  It is a
 // separate instantiation because its index and bias reads are ordinary vector loads inside the
 // tile loop; the dense form keeps every in-loop load under manual vmcnt control.
-template <int BM, int BN, int WAVES_M, int WAVES_N, int NSTAGE, bool GATHER>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int NSTAGE, bool GATHER, bool DIRECT = false>
 __global__ __launch_bounds__(WAVES_M * WAVES_N * kWave) void gemm_persistent_kernel(
-    GemmArgs args, int tiles_n, int tiles_m) {
-  using Cfg = PersistCfg<BM, BN, WAVES_M, WAVES_N, NSTAGE>;
+    GemmArgs args, int tiles_n, int tiles_m, int stagger) {
+  using Cfg = PersistCfg<BM, BN, WAVES_M, WAVES_N, NSTAGE, DIRECT>;
   extern __shared__ __attribute__((aligned(16))) int8_t lds[];
   const unsigned lds_base = (unsigned)(size_t)lds;  // LDS byte address of the ring
 
+  const long long t_start = clock64();
+  long long t_epi = 0;
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
   const int lane = tid % kWave;
@@ -209,6 +216,35 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * kWave) void gemm_persistent_ker
     persistent_tile_coords(round, blockIdx.x, grid, tiles_n, tiles_m, tn, tm);
     const int m0 = tm * BM, n0 = tn * BN;
     last_tile_interior = (m0 + BM <= M) && (n0 + BN <= args.n_out) && !(args.dbg & 2);
+    if(DIRECT) {
+      const bool interior = last_tile_interior;
+      const size_t row_bytes = (size_t)args.n_out * 4;
+#pragma unroll
+      for(int b = 0; b < Cfg::WTN; ++b) {
+        const int n = n0 + (wn * Cfg::WTN + b) * 32 + li;
+        const bool nvalid = n < args.n_out;
+        float bias_v = 0.0f;
+        if(has_bias) {
+          if(GATHER) {
+            bias_v = args.bias[args.idx[min(n, args.n_out - 1)]];
+          } else {
+            const float* staged = reinterpret_cast<const float*>(lds + NSTAGE * Cfg::kStageBytes + Cfg::kEpiBytes);
+            bias_v = staged[(round & 1) * 256 + (wn * Cfg::WTN + b) * 32 + li];
+          }
+        }
+#pragma unroll
+        for(int a = 0; a < Cfg::WTM; ++a) {
+          const int mbase = m0 + (wm * Cfg::WTM + a) * 32 + 4 * lg;
+          char* outp = reinterpret_cast<char*>(args.out) + ((size_t)mbase * (size_t)args.n_out + (size_t)n) * 4;
+          if(args.dbg & 2) continue;
+          if(interior)
+            store_tile32_any<false>(acc[a][b], outp, row_bytes, unquant, bias_v, 32, true, args.dump, has_bias, args.relu);
+          else
+            store_tile32_any<true>(acc[a][b], outp, row_bytes, unquant, bias_v, M - mbase, nvalid, args.dump, has_bias, args.relu);
+        }
+      }
+      return;
+    }
 #pragma unroll
     for(int b = 0; b < Cfg::WTN; ++b) {
       const int ncol0 = n0 + (wn * Cfg::WTN + b) * 32;
@@ -254,6 +290,10 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * kWave) void gemm_persistent_ker
 
   // ---------------- prologue ----------------
   if(n_my <= 0) return;
+  // Two workgroups share a CU; the second half of the grid starts late so that one of the two is
+  // in its main loop while the other loads its first blocks or writes a tile out.
+  if(stagger > 0 && blockIdx.x >= (unsigned)(grid / 2))
+    for(int i = 0; i < stagger; ++i) __builtin_amdgcn_s_sleep(127);
   load_tile_setup(0);
 #pragma unroll
   for(int s = 0; s < NSTAGE; ++s)
@@ -262,6 +302,7 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * kWave) void gemm_persistent_ker
   // block 0 has landed once at most the later blocks' loads are outstanding
   wait_vmcnt_dyn((min(total_blocks, NSTAGE) - 1) * Cfg::kLoads);
   __builtin_amdgcn_s_barrier();
+  const long long t_prologue = clock64();
   read_frags(0, 0, 0);
   read_frags(0, 1, 1);
 
@@ -271,7 +312,7 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * kWave) void gemm_persistent_ker
   // than them.  (With fewer K blocks per tile than stages several tiles could fall into that
   // window; then the stores are simply waited for.)
   int since_store = NSTAGE;
-  const bool count_stores = KB >= NSTAGE;
+  const bool count_stores = KB >= NSTAGE && !DIRECT;
   for(int g = 0; g < total_blocks; ++g) {
     const int stage = g % NSTAGE;
     read_frags(stage, 2, 2);
@@ -314,12 +355,19 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * kWave) void gemm_persistent_ker
         wait_vmcnt<0>();
         __builtin_amdgcn_s_barrier();
       }
+      long long te0 = 0;
+      if(args.prof) te0 = clock64();
       epilogue(round);
+      if(args.prof) t_epi += clock64() - te0;
       zero_acc();
       pos = 0;
       ++round;
       since_store = 0;
     }
+  }
+  if(args.prof && tid == 0) {
+    long long* p = args.prof + (size_t)blockIdx.x * 8;
+    p[0] = t_start; p[1] = t_prologue; p[2] = clock64() - t_epi; p[3] = clock64(); p[4] = t_epi; p[5] = total_blocks;
   }
 }
 

@@ -5,7 +5,9 @@
 // lane l of a wave loads 16 consecutive K bytes of weight row n0 + l % 32, which is the row
 // operand layout of v_mfma_i32_32x32x32_i8, so they need no LDS staging or transposition.  The
 // small quantized activations are the column operand; a workgroup keeps them in LDS in operand
-// order.  The 8 waves of a workgroup are arranged WN (different weight rows) x KW (different K
+// order (within a fragment the 32 rows of a K chunk are XOR-permuted by the chunk number, which
+// spreads the quantizer's 4-byte writes over the LDS banks and keeps the fragment reads
+// conflict free).  The 8 waves of a workgroup are arranged WN (different weight rows) x KW (different K
 // ranges of the same rows); the KW partial sums are added through LDS (exact in any order).
 //
 // FUSED: the workgroup reads the fp32 activations itself, takes their abs-max (every workgroup
@@ -24,7 +26,7 @@ typedef int v16i_s __attribute__((ext_vector_type(16)));
 constexpr int kStream32Waves = 8;
 constexpr int kStream32Threads = kStream32Waves * kWave;
 constexpr int kFusedMaxElems = 32768;   // fp32 activations a workgroup holds in registers
-constexpr int kFusedVecs = kFusedMaxElems / 4 / kStream32Threads;   // float4 per thread
+constexpr int kFusedGroups = kFusedMaxElems / 16 / kStream32Threads;   // 16-value groups per thread
 
 // MT32: 32-row activation tiles per workgroup (blockIdx.y walks M in steps of 32 * MT32; the
 // fused form needs all of M in one workgroup).  CS: 32-byte K sub-steps staged per chunk.
@@ -55,6 +57,8 @@ __global__ __launch_bounds__(kStream32Threads) void gemm_stream32_kernel(GemmArg
   extern __shared__ __attribute__((aligned(16))) int8_t lds[];
   __shared__ float red[kStream32Waves];
 
+  long long tp[6] = {0, 0, 0, 0, 0, 0};
+  if(args.prof) tp[0] = clock64();
   const int tid = threadIdx.x;
   const int wave = tid / kWave, lane = tid % kWave;
   const int wn = wave % WN, kw = wave / WN;
@@ -72,6 +76,27 @@ __global__ __launch_bounds__(kStream32Threads) void gemm_stream32_kernel(GemmArg
     if(n < args.n_out) wsrc = args.idx ? (int)args.idx[n] : n;
   }
   const int8_t* wrow = args.Bq + (size_t)wsrc * (size_t)K + lg * 16;
+
+  // FUSED: the fp32 activations are requested before anything else - they are needed first, and
+  // a wave's loads return in issue order, so behind the weight stream they would arrive last.
+  // A thread owns groups of 16 consecutive values of one activation row (one 16-byte LDS slot
+  // after quantization): group number gi = j * threads + tid is row gi / (K/16), chunk gi % (K/16).
+  v4f vals[FUSED ? kFusedGroups : 1][4];
+  float amax = 0.0f;
+  const int n16 = M * K / 16;
+  if(FUSED) {
+    const v4f* a4 = reinterpret_cast<const v4f*>(A);
+#pragma unroll
+    for(int j = 0; j < kFusedGroups; ++j) {
+      const int gi = j * kStream32Threads + tid;
+#pragma unroll
+      for(int e = 0; e < 4; ++e) {
+        v4f v = {0.0f, 0.0f, 0.0f, 0.0f};
+        if(gi < n16) v = a4[gi * 4 + e];
+        vals[j][e] = v;
+      }
+    }
+  }
 
   v4i w[Cfg::PW];
   auto load_weights = [&](int chunk) {
@@ -116,34 +141,47 @@ __global__ __launch_bounds__(kStream32Threads) void gemm_stream32_kernel(GemmArg
   float aqm = 0.0f;
   if(FUSED) {
     // whole A (M*K <= kFusedMaxElems floats) in registers: abs-max, then quantize into LDS
-    const v4f* a4 = reinterpret_cast<const v4f*>(A);
-    const int n4 = M * K / 4;
-    v4f vals[kFusedVecs];
-    float m = 0.0f;
 #pragma unroll
-    for(int j = 0; j < kFusedVecs; ++j) {
-      const int i = j * kStream32Threads + tid;
-      v4f v = {0.0f, 0.0f, 0.0f, 0.0f};
-      if(i < n4) v = a4[i];
-      vals[j] = v;
-      m = abs4max(v, m);
-    }
+    for(int j = 0; j < kFusedGroups; ++j)
+#pragma unroll
+      for(int e = 0; e < 4; ++e) amax = abs4max(vals[j][e], amax);
     // zero the rows between M and the next multiple of 32 (whole LDS stage, cheap)
     for(int i = tid; i < S * MT32 * 64; i += kStream32Threads)
       reinterpret_cast<v4i*>(lds)[i] = v4i{0, 0, 0, 0};
-    m = block_max(m, red);   // contains the barriers that order the zero fill before the writes
-    aqm = quant_mult_from_maxabs(m);
-    const int k4 = K / 4;    // float4 per activation row
+    amax = block_max(amax, red);   // its barriers also order the zero fill before the writes
+    if(args.prof) tp[1] = clock64();
+    aqm = quant_mult_from_maxabs(amax);
+    // with a finite non-zero abs-max no product can leave [-127.0001, 127.0001]
+    const bool finite = amax > 0.0f && amax < __builtin_inff();
+    const int k16n = K / 16;   // 16-byte chunks per activation row
+    int row = tid / k16n, c16 = tid % k16n;
+    const int drow = kStream32Threads / k16n, dc16 = kStream32Threads % k16n;
 #pragma unroll
-    for(int j = 0; j < kFusedVecs; ++j) {
-      const int i = j * kStream32Threads + tid;
-      if(i < n4) {
-        const int row = i / k4, k = (i % k4) * 4;
-        const uint32_t q = quantize_pack4(vals[j], aqm);
-        const int s = k / 32, g = (k % 32) / 16, b = k % 16;
-        const int slot = (s * MT32 + row / 32) * 64 + g * 32 + (row % 32);
-        *reinterpret_cast<uint32_t*>(lds + slot * 16 + b) = q;
-        if(aq_out && blockIdx.x == 0) *reinterpret_cast<uint32_t*>(aq_out + (size_t)row * K + k) = q;
+    for(int j = 0; j < kFusedGroups; ++j) {
+      const int gi = j * kStream32Threads + tid;
+      if(gi < n16) {
+        uint4 q;
+        if(finite) {
+          q.x = quantize_pack4_finite(vals[j][0], aqm);
+          q.y = quantize_pack4_finite(vals[j][1], aqm);
+          q.z = quantize_pack4_finite(vals[j][2], aqm);
+          q.w = quantize_pack4_finite(vals[j][3], aqm);
+        } else {
+          q.x = quantize_pack4(vals[j][0], aqm);
+          q.y = quantize_pack4(vals[j][1], aqm);
+          q.z = quantize_pack4(vals[j][2], aqm);
+          q.w = quantize_pack4(vals[j][3], aqm);
+        }
+        const int s = c16 / 2, g = c16 % 2;
+        const int slot = (s * MT32 + row / 32) * 64 + g * 32 + ((row % 32) ^ (c16 & 7));
+        *reinterpret_cast<uint4*>(lds + slot * 16) = q;
+        if(aq_out && blockIdx.x == 0) *reinterpret_cast<uint4*>(aq_out + (size_t)row * K + c16 * 16) = q;
+      }
+      row += drow;
+      c16 += dc16;
+      if(c16 >= k16n) {
+        c16 -= k16n;
+        row += 1;
       }
     }
     if(aq_out && blockIdx.x == 0 && tid == 0)
@@ -170,8 +208,12 @@ __global__ __launch_bounds__(kStream32Threads) void gemm_stream32_kernel(GemmArg
   };
   auto stage_store = [&]() {
 #pragma unroll
-    for(int j = 0; j < kStageVecs; ++j)
-      *reinterpret_cast<v4i*>(lds + (j * kStream32Threads + tid) * 16) = stage[j];
+    for(int j = 0; j < kStageVecs; ++j) {
+      const int slot = j * kStream32Threads + tid;
+      const int l = slot % 64, step = (slot / 64) / MT32;
+      const int sw = (slot & ~31) | ((l % 32) ^ ((2 * step + l / 32) & 7));
+      *reinterpret_cast<v4i*>(lds + sw * 16) = stage[j];
+    }
   };
   if(!FUSED) {
     stage_fetch(0);
@@ -179,6 +221,7 @@ __global__ __launch_bounds__(kStream32Threads) void gemm_stream32_kernel(GemmArg
     __syncthreads();
   }
 
+  if(args.prof) tp[2] = clock64();
   v16i_s acc[MT32];
 #pragma unroll
   for(int mt = 0; mt < MT32; ++mt)
@@ -206,7 +249,8 @@ __global__ __launch_bounds__(kStream32Threads) void gemm_stream32_kernel(GemmArg
       if(FUSED) step = min(c * Cfg::CS + step, S - 1);
 #pragma unroll
       for(int mt = 0; mt < MT32; ++mt) {
-        const v4i a = *reinterpret_cast<const v4i*>(lds + (step * MT32 + mt) * kFragBytes + lane * 16);
+        const v4i a = *reinterpret_cast<const v4i*>(
+            lds + (step * MT32 + mt) * kFragBytes + (lg * 32 + (li ^ ((2 * step + lg) & 7))) * 16);
         acc[mt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(w[p], a, acc[mt], 0, 0, 0);
       }
     }
@@ -221,6 +265,7 @@ __global__ __launch_bounds__(kStream32Threads) void gemm_stream32_kernel(GemmArg
     }
   }
 
+  if(args.prof) tp[3] = clock64();
   // ---- add the KW partial sums into the kw == 0 waves ----
   if(KW > 1) {
     __syncthreads();
@@ -252,6 +297,7 @@ __global__ __launch_bounds__(kStream32Threads) void gemm_stream32_kernel(GemmArg
 
   // ---- epilogue: element v of lane (li, lg) is weight row 8*(v/4) + 4*lg + v%4 of the tile,
   //      activation row li ----
+  if(args.prof) tp[4] = clock64();
   if(kw == 0) {
     const float unquant = unquant_mult(FUSED ? aqm : aqm_pre, bqm, args.scale);
     const bool has_bias = args.bias != nullptr;
@@ -289,6 +335,11 @@ __global__ __launch_bounds__(kStream32Threads) void gemm_stream32_kernel(GemmArg
         *reinterpret_cast<v4f*>(reinterpret_cast<float*>(args.out) + off) = y;
       }
     }
+  }
+  if(args.prof && tid == 0) {
+    long long* p = args.prof + ((size_t)blockIdx.y * gridDim.x + blockIdx.x) * 8;
+    p[0] = tp[0]; p[1] = tp[1]; p[2] = tp[2]; p[3] = tp[3]; p[4] = tp[4]; p[5] = clock64();
+    p[6] = wall_clock64();
   }
 }
 

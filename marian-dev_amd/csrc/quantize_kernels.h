@@ -33,6 +33,18 @@ __device__ __forceinline__ uint32_t quantize_low_byte(float x, float qm) {
   return __float_as_uint(c + 12582912.0f);
 }
 
+// Fast form for the usual case (finite, non-zero abs-max): every product lies within
+// [-127.0001, 127.0001], so the non-finite check of quantize_low_byte can never fire.
+__device__ __forceinline__ uint32_t quantize_pack4_finite(v4f x, float qm) {
+  const uint32_t b0 = __float_as_uint(__builtin_amdgcn_fmed3f(x.x * qm, -127.0f, 127.0f) + 12582912.0f);
+  const uint32_t b1 = __float_as_uint(__builtin_amdgcn_fmed3f(x.y * qm, -127.0f, 127.0f) + 12582912.0f);
+  const uint32_t b2 = __float_as_uint(__builtin_amdgcn_fmed3f(x.z * qm, -127.0f, 127.0f) + 12582912.0f);
+  const uint32_t b3 = __float_as_uint(__builtin_amdgcn_fmed3f(x.w * qm, -127.0f, 127.0f) + 12582912.0f);
+  const uint32_t lo = __builtin_amdgcn_perm(b1, b0, 0x0c0c0400u);
+  const uint32_t hi = __builtin_amdgcn_perm(b3, b2, 0x0c0c0400u);
+  return __builtin_amdgcn_perm(hi, lo, 0x05040100u);
+}
+
 __device__ __forceinline__ uint32_t quantize_pack4(v4f x, float qm) {
   const uint32_t b0 = quantize_low_byte(x.x, qm), b1 = quantize_low_byte(x.y, qm);
   const uint32_t b2 = quantize_low_byte(x.z, qm), b3 = quantize_low_byte(x.w, qm);

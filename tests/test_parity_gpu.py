@@ -87,7 +87,7 @@ def test_prepare_b_bit_exact(integer, orc, synth, K, N):
 
 # ---------------------------------------------------------------- multiply: int32 and fp32
 
-KERNELS = [0, 101, 102, 501, 511, 512, 514, 518, 521, 522, 524, 201, 202, 203, 204, 301, 302, 303, 304, 305, 306, 307, 308, 401, 402, 403, 404]
+KERNELS = [0, 101, 102, 501, 511, 512, 514, 518, 521, 522, 524, 201, 202, 203, 204, 301, 302, 303, 304, 305, 306, 307, 308, 401, 402, 403, 404, 411, 413, 416]
 
 
 def run_case(integer, orc, synth, seed, M, K, N, kernel, bias_on=True, relu=False, scale=1.0):
@@ -117,7 +117,7 @@ def test_multiply_all_kernels_small_m(integer, orc, synth, M, K, N, kernel):
     run_case(integer, orc, synth, 300 + M + N, M, K, N, kernel, bias_on=True, relu=(M % 2 == 0))
 
 
-@pytest.mark.parametrize("kernel", [0, 501, 512, 521, 522, 524, 201, 202, 203, 204, 301, 302, 303, 304, 305, 306, 307, 308, 401, 402, 403, 404])
+@pytest.mark.parametrize("kernel", [0, 501, 512, 521, 522, 524, 201, 202, 203, 204, 301, 302, 303, 304, 305, 306, 307, 308, 401, 402, 403, 404, 411, 413, 416])
 @pytest.mark.parametrize("M,K,N", [(129, 64, 8), (256, 1024, 504), (300, 320, 1000), (513, 128, 264)])
 def test_multiply_tile_kernels_ragged(integer, orc, synth, M, K, N, kernel):
     say("multiply ragged", M, K, N, "kernel", kernel)
