@@ -95,10 +95,10 @@ inline bool stream32_can_fuse(int64_t M, int64_t K) {
   return M <= 128 && M * K <= kFusedMaxElems && stream32_fused_lds_bytes(mt32, (int)K) <= 64 * 1024;
 }
 
-template <int MT32, int WN, int KW, bool FUSED>
+template <int MT32, int WN, int KW, int PW, bool FUSED>
 int launch_stream32(const GemmArgs& a, const float* A, int8_t* aq_out, hipStream_t st) {
-  using Cfg = Stream32Cfg<MT32, WN, KW>;
-  auto kernel = gemm_stream32_kernel<MT32, WN, KW, FUSED>;
+  using Cfg = Stream32Cfg<MT32, WN, KW, PW>;
+  auto kernel = gemm_stream32_kernel<MT32, WN, KW, PW, FUSED>;
   constexpr int kMaxLds = 64 * 1024 > Cfg::kLdsBytes ? 64 * 1024 : Cfg::kLdsBytes;
   static const int lds_status = allow_lds(kernel, kMaxLds);
   if(lds_status != MARIAN_HIP_OK) return lds_status;
@@ -111,13 +111,28 @@ int launch_stream32(const GemmArgs& a, const float* A, int8_t* aq_out, hipStream
   return MARIAN_HIP_OK;
 }
 
+// Picks the number of K sub-steps a wave holds per chunk: the smallest instantiated value that
+// covers K in one chunk, else the largest whose activations fit the 64 KB LDS stage
+// (MT32 * KW * PW <= 64).
 template <int MT32, bool FUSED>
 int launch_stream32_kw(const GemmArgs& a, const float* A, int8_t* aq_out, hipStream_t st, int kw) {
+  const int need = (a.K / 32 + kw - 1) / kw;   // sub-steps per wave if K is one chunk
   switch(kw) {
-    case 1: return launch_stream32<MT32, 8, 1, FUSED>(a, A, aq_out, st);
-    case 2: return launch_stream32<MT32, 4, 2, FUSED>(a, A, aq_out, st);
-    case 4: return launch_stream32<MT32, 2, 4, FUSED>(a, A, aq_out, st);
-    default: return launch_stream32<MT32, 1, 8, FUSED>(a, A, aq_out, st);
+    case 1: return launch_stream32<MT32, 8, 1, 8, FUSED>(a, A, aq_out, st);
+    case 2: return launch_stream32<MT32, 4, 2, 8, FUSED>(a, A, aq_out, st);
+    case 4:
+      if constexpr(MT32 <= 2) {
+        if(need > 4) return launch_stream32<MT32, 2, 4, 8, FUSED>(a, A, aq_out, st);
+      }
+      return launch_stream32<MT32, 2, 4, 4, FUSED>(a, A, aq_out, st);
+    default:
+      if constexpr(MT32 == 1) {
+        if(need > 4) return launch_stream32<MT32, 1, 8, 8, FUSED>(a, A, aq_out, st);
+      }
+      if constexpr(MT32 <= 2) {
+        if(need > 2) return launch_stream32<MT32, 1, 8, 4, FUSED>(a, A, aq_out, st);
+      }
+      return launch_stream32<MT32, 1, 8, 2, FUSED>(a, A, aq_out, st);
   }
 }
 

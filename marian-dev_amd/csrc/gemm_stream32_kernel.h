@@ -29,31 +29,30 @@ constexpr int kFusedMaxElems = 32768;   // fp32 activations a workgroup holds in
 constexpr int kFusedGroups = kFusedMaxElems / 16 / kStream32Threads;   // 16-value groups per thread
 
 // MT32: 32-row activation tiles per workgroup (blockIdx.y walks M in steps of 32 * MT32; the
-// fused form needs all of M in one workgroup).  CS: 32-byte K sub-steps staged per chunk.
-template <int MT32, int WN, int KW>
+// fused form needs all of M in one workgroup).  PW: 32-byte K sub-steps (weight loads in flight)
+// per wave and chunk; a chunk is CS = PW * KW sub-steps, and its activations fill at most 64 KB
+// of LDS.  The launcher picks the smallest PW that covers K in one chunk where there is one, so
+// that no wave is left with sub-steps past the end of K.
+template <int MT32, int WN, int KW, int PW_>
 struct Stream32Cfg {
   static_assert(WN * KW == kStream32Waves, "eight waves");
   static constexpr int kColsPerBlock = WN * 32;
-  // K sub-steps per chunk: activations of a chunk fill at most 64 KB of LDS, and each wave owns
-  // at most 8 sub-steps (8 weight loads in flight) of a chunk
-  static constexpr int kMaxChunkSteps = (64 * 1024) / (MT32 * kFragBytes) < 8 * KW
-                                            ? (64 * 1024) / (MT32 * kFragBytes)
-                                            : 8 * KW;
-  static constexpr int PW = kMaxChunkSteps / KW;      // sub-steps per wave per chunk
+  static constexpr int PW = PW_;
   static constexpr int CS = PW * KW;
   static constexpr int kStageBytes = MT32 * CS * kFragBytes;
   static constexpr int kReduceBytes = (KW - 1) * WN * MT32 * 4 * kFragBytes;  // v16i per lane
   static constexpr int kLdsBytes = kStageBytes > kReduceBytes ? kStageBytes : kReduceBytes;
-  static_assert(PW >= 1, "chunk too small");
+  static_assert(PW >= 1 && PW <= 8 && kStageBytes <= 64 * 1024, "chunk size");
+  static_assert(CS * MT32 * 64 % kStream32Threads == 0, "stage must divide over the threads");
 };
 
 // Dynamic LDS: FUSED holds all of K (32 * MT32 * K bytes); otherwise one chunk (kStageBytes);
 // both at least kReduceBytes.
-template <int MT32, int WN, int KW, bool FUSED>
+template <int MT32, int WN, int KW, int PW, bool FUSED>
 __global__ __launch_bounds__(kStream32Threads) void gemm_stream32_kernel(GemmArgs args,
                                                                         const float* A,
                                                                         int8_t* aq_out) {
-  using Cfg = Stream32Cfg<MT32, WN, KW>;
+  using Cfg = Stream32Cfg<MT32, WN, KW, PW>;
   extern __shared__ __attribute__((aligned(16))) int8_t lds[];
   __shared__ float red[kStream32Waves];
 
@@ -68,14 +67,45 @@ __global__ __launch_bounds__(kStream32Threads) void gemm_stream32_kernel(GemmArg
   const int n_chunks = (S + Cfg::CS - 1) / Cfg::CS;
   const int m_base = blockIdx.y * (MT32 * 32);            // activation rows of this workgroup
 
-  // ---- weight row of this lane ----
+  // Loads of a wave return in issue order and the compiler counts them: a value is waited for
+  // with "all but the N youngest loads".  A load inside a branch makes that count unknown, and
+  // everything older is then waited for with N = 0.  So the loads that may be skipped (shortlist
+  // ids, bias) come first, and the activation and weight loads after them are unconditional
+  // (out-of-range indices are clamped and the values replaced afterwards): the activations can
+  // then be waited for while the weight loads are still in flight.
+
+  // ---- weight row of this lane; bias of the columns this wave will write, through the
+  //      shortlist ids when there are any ----
   const int n0 = (blockIdx.x * WN + wn) * 32;
-  int wsrc = 0;
-  {
-    const int n = n0 + li;
-    if(n < args.n_out) wsrc = args.idx ? (int)args.idx[n] : n;
+  int wsrc = min(n0 + li, args.n_out - 1);
+  if(args.idx) wsrc = (int)args.idx[wsrc];
+  // (pins the wait for the id here, where nothing else is in flight; left to itself the compiler
+  // computes the weight address, and waits, after the activation loads)
+  asm volatile("" : "+v"(wsrc));
+  // Each wave finishes SL of a lane's 16 * MT32 accumulator values (see the reduction below):
+  // values kw * SL + c * CW .. + CW - 1 for chunk c, i.e. activation tile mt = value / 16 and
+  // weight rows n0 + 8 * q + 4 * lg + e with q = value % 16 / 4, e = value % 4.
+  constexpr int V = 16 * MT32;
+  constexpr int SL = V / KW;
+  constexpr int CW = SL >= 4 ? 4 : SL;   // values per store: 4, or 2 for MT32 = 1 with KW = 8
+  constexpr int NC = SL / CW;
+  static_assert(SL >= 2 && NC * CW == SL, "slice shape");
+  float bias_s[NC][CW];
+#pragma unroll
+  for(int c = 0; c < NC; ++c) {
+    const int v = (kw * SL + c * CW) % 16;
+    const int n = min(n0 + 8 * (v / 4) + 4 * lg + v % 4, args.n_out - CW);   // n_out % 8 == 0
+#pragma unroll
+    for(int e = 0; e < CW; ++e) {
+      bias_s[c][e] = 0.0f;
+      if(args.bias) bias_s[c][e] = args.bias[args.idx ? args.idx[n + e] : (uint32_t)(n + e)];
+    }
   }
+  const float bqm = tail_quant_mult(args.Bq, (size_t)K * (size_t)args.N);
+  float aqm_pre = 0.0f;
+  if(!FUSED) aqm_pre = tail_quant_mult(args.Aq, (size_t)M * (size_t)K);
   const int8_t* wrow = args.Bq + (size_t)wsrc * (size_t)K + lg * 16;
+  __builtin_amdgcn_sched_barrier(0);
 
   // FUSED: the fp32 activations are requested before anything else - they are needed first, and
   // a wave's loads return in issue order, so behind the weight stream they would arrive last.
@@ -91,9 +121,9 @@ __global__ __launch_bounds__(kStream32Threads) void gemm_stream32_kernel(GemmArg
       const int gi = j * kStream32Threads + tid;
 #pragma unroll
       for(int e = 0; e < 4; ++e) {
-        v4f v = {0.0f, 0.0f, 0.0f, 0.0f};
-        if(gi < n16) v = a4[gi * 4 + e];
-        vals[j][e] = v;
+        vals[j][e] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+        // (a wave whose 64 groups are all out of range skips the loads)
+        if(j * kStream32Threads + wave * kWave < n16) vals[j][e] = a4[min(gi, n16 - 1) * 4 + e];
       }
     }
   }
@@ -103,38 +133,16 @@ __global__ __launch_bounds__(kStream32Threads) void gemm_stream32_kernel(GemmArg
 #pragma unroll
     for(int p = 0; p < Cfg::PW; ++p) {
       const int s = chunk * Cfg::CS + kw * Cfg::PW + p;
-      v4i v = {0, 0, 0, 0};
-      if(s < S) v = load16(wrow + s * 32);
-      w[p] = v;
+      w[p] = load16(wrow + min(s, S - 1) * 32);
     }
   };
+  // sub-steps past the end of K multiply zero weights
+  auto mask_weights = [&](int chunk) {
+#pragma unroll
+    for(int p = 0; p < Cfg::PW; ++p)
+      if(chunk * Cfg::CS + kw * Cfg::PW + p >= S) w[p] = v4i{0, 0, 0, 0};
+  };
   load_weights(0);   // in flight while the activations are prepared
-
-  // Everything else the epilogue needs from global memory is requested now as well, so that all
-  // global latencies of this workgroup overlap: the weight quantMult, the bias of the lane's
-  // columns n0 + 8q + 4*lg .. +3 (q = 0..3), through the shortlist ids when there are any.
-  float bqm = 0.0f, aqm_pre = 0.0f;
-  v4f bias_v[4];
-#pragma unroll
-  for(int q = 0; q < 4; ++q) bias_v[q] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
-  if(!args.dump) {
-    bqm = tail_quant_mult(args.Bq, (size_t)K * (size_t)args.N);
-    if(!FUSED) aqm_pre = tail_quant_mult(args.Aq, (size_t)M * (size_t)K);
-    if(args.bias && kw == 0) {
-#pragma unroll
-      for(int q = 0; q < 4; ++q) {
-        const int n = n0 + 8 * q + 4 * lg;
-        if(n < args.n_out) {
-          if(args.idx) {
-            bias_v[q] = v4f{args.bias[args.idx[n]], args.bias[args.idx[n + 1]],
-                            args.bias[args.idx[n + 2]], args.bias[args.idx[n + 3]]};
-          } else {
-            bias_v[q] = v4f{args.bias[n], args.bias[n + 1], args.bias[n + 2], args.bias[n + 3]};
-          }
-        }
-      }
-    }
-  }
 
   // ---- activations into LDS, operand order: slot (sub-step, m-tile, lane) of 16 bytes holds
   //      Aq[mt*32 + lane%32][(s0+step)*32 + (lane/32)*16 .. +15]
@@ -144,7 +152,10 @@ __global__ __launch_bounds__(kStream32Threads) void gemm_stream32_kernel(GemmArg
 #pragma unroll
     for(int j = 0; j < kFusedGroups; ++j)
 #pragma unroll
-      for(int e = 0; e < 4; ++e) amax = abs4max(vals[j][e], amax);
+      for(int e = 0; e < 4; ++e) {
+        if(j * kStream32Threads + tid >= n16) vals[j][e] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+        amax = abs4max(vals[j][e], amax);
+      }
     // zero the rows between M and the next multiple of 32 (whole LDS stage, cheap)
     for(int i = tid; i < S * MT32 * 64; i += kStream32Threads)
       reinterpret_cast<v4i*>(lds)[i] = v4i{0, 0, 0, 0};
@@ -201,18 +212,19 @@ __global__ __launch_bounds__(kStream32Threads) void gemm_stream32_kernel(GemmArg
       const int mt = f % MT32, step = f / MT32;
       const int m = m_base + mt * 32 + (l % 32);
       const int s = s0 + step;
-      v4i v = {0, 0, 0, 0};
-      if(m < M && s < S) v = load16(args.Aq + (size_t)m * (size_t)K + s * 32 + (l / 32) * 16);
-      stage[j] = v;
+      stage[j] = load16(args.Aq + (size_t)min(m, M - 1) * (size_t)K + min(s, S - 1) * 32 + (l / 32) * 16);
     }
   };
   auto stage_store = [&]() {
 #pragma unroll
     for(int j = 0; j < kStageVecs; ++j) {
       const int slot = j * kStream32Threads + tid;
-      const int l = slot % 64, step = (slot / 64) / MT32;
+      const int l = slot % 64, f = slot / 64;
+      const int mt = f % MT32, step = f / MT32;
       const int sw = (slot & ~31) | ((l % 32) ^ ((2 * step + l / 32) & 7));
-      *reinterpret_cast<v4i*>(lds + sw * 16) = stage[j];
+      // rows past M hold zeros (sub-steps past K multiply zero weights, any value will do)
+      const bool live = m_base + mt * 32 + (l % 32) < M;
+      *reinterpret_cast<v4i*>(lds + sw * 16) = live ? stage[j] : v4i{0, 0, 0, 0};
     }
   };
   if(!FUSED) {
@@ -236,11 +248,10 @@ __global__ __launch_bounds__(kStream32Threads) void gemm_stream32_kernel(GemmArg
 #pragma unroll
       for(int p = 0; p < Cfg::PW; ++p) {
         const int s = (c + 1) * Cfg::CS + kw * Cfg::PW + p;
-        v4i v = {0, 0, 0, 0};
-        if(s < S) v = load16(wrow + s * 32);
-        wnext[p] = v;
+        wnext[p] = load16(wrow + min(s, S - 1) * 32);
       }
     }
+    mask_weights(c);
 #pragma unroll
     for(int p = 0; p < Cfg::PW; ++p) {
       // FUSED keeps every sub-step in LDS; otherwise LDS holds the current chunk only.  Sub-steps
@@ -266,74 +277,78 @@ __global__ __launch_bounds__(kStream32Threads) void gemm_stream32_kernel(GemmArg
   }
 
   if(args.prof) tp[3] = clock64();
-  // ---- add the KW partial sums into the kw == 0 waves ----
+  // ---- add the KW partial sums: wave r collects slice r (values r * SL .. + SL - 1 of every
+  //      lane) from the other waves of its column group, so that the additions and the stores
+  //      of the epilogue are spread over all waves.  Slot (r, t, wn, c, lane) of CW ints holds
+  //      what source wave t' (t = t' minus one if t' > r) contributes to chunk c of slice r. ----
+  int mine[NC][CW];
   if(KW > 1) {
-    __syncthreads();
-    v4i* redbuf = reinterpret_cast<v4i*>(lds);
-    if(kw > 0) {
+    __syncthreads();   // every wave is done reading activations from LDS
+    int* redbuf = reinterpret_cast<int*>(lds);
 #pragma unroll
-      for(int mt = 0; mt < MT32; ++mt)
+    for(int r = 0; r < KW; ++r) {
+      if(r == kw) {
 #pragma unroll
-        for(int q = 0; q < 4; ++q)
-          redbuf[((((kw - 1) * WN + wn) * MT32 + mt) * 4 + q) * 64 + lane] =
-              v4i{acc[mt][4 * q], acc[mt][4 * q + 1], acc[mt][4 * q + 2], acc[mt][4 * q + 3]};
+        for(int c = 0; c < NC; ++c)
+#pragma unroll
+          for(int e = 0; e < CW; ++e) mine[c][e] = acc[(r * SL + c * CW + e) / 16][(r * SL + c * CW + e) % 16];
+      } else {
+        const int t = kw < r ? kw : kw - 1;
+#pragma unroll
+        for(int c = 0; c < NC; ++c) {
+          int* dst = redbuf + (size_t)(((((r * (KW - 1) + t) * WN + wn) * NC + c) * 64 + lane) * CW);
+#pragma unroll
+          for(int e = 0; e < CW; ++e) dst[e] = acc[(r * SL + c * CW + e) / 16][(r * SL + c * CW + e) % 16];
+        }
+      }
     }
     __syncthreads();
-    if(kw == 0) {
-#pragma unroll 1   // one partial sum at a time keeps the register count down
-      for(int r = 1; r < KW; ++r)
 #pragma unroll
-        for(int mt = 0; mt < MT32; ++mt)
+    for(int t = 0; t < KW - 1; ++t)
 #pragma unroll
-          for(int q = 0; q < 4; ++q) {
-            const v4i t = redbuf[((((r - 1) * WN + wn) * MT32 + mt) * 4 + q) * 64 + lane];
-            acc[mt][4 * q] += t.x;
-            acc[mt][4 * q + 1] += t.y;
-            acc[mt][4 * q + 2] += t.z;
-            acc[mt][4 * q + 3] += t.w;
-          }
-    }
+      for(int c = 0; c < NC; ++c) {
+        const int* src = redbuf + (size_t)(((((kw * (KW - 1) + t) * WN + wn) * NC + c) * 64 + lane) * CW);
+#pragma unroll
+        for(int e = 0; e < CW; ++e) mine[c][e] += src[e];
+      }
+  } else {
+#pragma unroll
+    for(int c = 0; c < NC; ++c)
+#pragma unroll
+      for(int e = 0; e < CW; ++e) mine[c][e] = acc[(c * CW + e) / 16][(c * CW + e) % 16];
   }
 
-  // ---- epilogue: element v of lane (li, lg) is weight row 8*(v/4) + 4*lg + v%4 of the tile,
-  //      activation row li ----
+  // ---- epilogue: value v of tile mt in lane (li, lg) is activation row mt * 32 + li, weight
+  //      row 8 * (v / 4) + 4 * lg + v % 4 of the wave's 32 ----
   if(args.prof) tp[4] = clock64();
-  if(kw == 0) {
+  {
     const float unquant = unquant_mult(FUSED ? aqm : aqm_pre, bqm, args.scale);
     const bool has_bias = args.bias != nullptr;
 #pragma unroll
-    for(int mt = 0; mt < MT32; ++mt) {
-      const int m = m_base + mt * 32 + li;
-#pragma unroll
-      for(int q = 0; q < 4; ++q) {
-        const int n = n0 + 8 * q + 4 * lg;
-        if(m >= M || n >= args.n_out) continue;
-        const size_t off = (size_t)m * (size_t)args.n_out + (size_t)n;
-        const v4i a4 = v4i{acc[mt][4 * q], acc[mt][4 * q + 1], acc[mt][4 * q + 2], acc[mt][4 * q + 3]};
-        if(args.dump) {
-          *reinterpret_cast<v4i*>(reinterpret_cast<int32_t*>(args.out) + off) = a4;
-          continue;
-        }
-        // y = float(acc) * unquant (+ bias); relu: y > 0 ? y : 0; mul and add round separately
-        v4f y;
-        y.x = (float)a4.x * unquant;
-        y.y = (float)a4.y * unquant;
-        y.z = (float)a4.z * unquant;
-        y.w = (float)a4.w * unquant;
-        if(has_bias) {
-          y.x = y.x + bias_v[q].x;
-          y.y = y.y + bias_v[q].y;
-          y.z = y.z + bias_v[q].z;
-          y.w = y.w + bias_v[q].w;
-        }
-        if(args.relu) {
-          y.x = y.x > 0.0f ? y.x : 0.0f;
-          y.y = y.y > 0.0f ? y.y : 0.0f;
-          y.z = y.z > 0.0f ? y.z : 0.0f;
-          y.w = y.w > 0.0f ? y.w : 0.0f;
-        }
-        *reinterpret_cast<v4f*>(reinterpret_cast<float*>(args.out) + off) = y;
+    for(int c = 0; c < NC; ++c) {
+      const int vv = kw * SL + c * CW;
+      const int v = vv % 16;
+      const int m = m_base + (vv / 16) * 32 + li;
+      const int n = n0 + 8 * (v / 4) + 4 * lg + v % 4;
+      if(m >= M || n >= args.n_out) continue;
+      const size_t off = (size_t)m * (size_t)args.n_out + (size_t)n;
+      if(args.dump) {
+        int32_t* o = reinterpret_cast<int32_t*>(args.out) + off;
+        if(CW == 4) *reinterpret_cast<v4i*>(o) = v4i{mine[c][0], mine[c][1], mine[c][CW - 2], mine[c][CW - 1]};
+        else *reinterpret_cast<int2*>(o) = int2{mine[c][0], mine[c][1]};
+        continue;
       }
+      // y = float(acc) * unquant (+ bias); relu: y > 0 ? y : 0; mul and add round separately
+      float y[CW];
+#pragma unroll
+      for(int e = 0; e < CW; ++e) {
+        y[e] = (float)mine[c][e] * unquant;
+        if(has_bias) y[e] = y[e] + bias_s[c][e];
+        if(args.relu) y[e] = y[e] > 0.0f ? y[e] : 0.0f;
+      }
+      float* o = reinterpret_cast<float*>(args.out) + off;
+      if(CW == 4) *reinterpret_cast<v4f*>(o) = v4f{y[0], y[1], y[CW - 2], y[CW - 1]};
+      else *reinterpret_cast<float2*>(o) = float2{y[0], y[1]};
     }
   }
   if(args.prof && tid == 0) {

@@ -165,6 +165,38 @@ def test_fused_shortlist(integer, orc, synth):
     assert np.array_equal(Aq.numpy(), Aq_h) and np.array_equal(out.cpu().numpy(), want)
 
 
+@pytest.mark.parametrize("kernel", [0, 101, 102, 201, 301, 307, 401, 411, 501, 511, 512, 514, 518, 521,
+                                    522, 524, 600, 611, 612, 614, 618])
+@pytest.mark.parametrize("M", [8, 100])
+def test_shortlist_every_kernel_family(integer, orc, synth, M, kernel):
+    """The row gather of W^T and of the bias inside each kernel family (ids >= 600: fused call)."""
+    import torch
+    from conftest import load
+    lib = load("_lib").lib()
+    say("shortlist", M, "kernel", kernel)
+    K, N = 256, 2048
+    A, W, bias = inputs(synth, 707 + M, M, K, N)
+    Aq_h, Bq_h = orc.prepare_a(A), orc.prepare_b(W)
+    idx = synth.shortlist(707 + M, N, 100, 300)
+    want, want_acc = orc.affine_shortlist(Aq_h, Bq_h, bias, idx, M, K, N)
+    Bq = upload_q(integer, Bq_h, (K, N))
+    didx = torch.from_numpy(idx.view(np.int32)).cuda()
+    prev = lib.marian_hip_int8_set_kernel(kernel)
+    try:
+        if kernel >= 600:
+            out, Aq = integer.affine_f32(dev(A), Bq, dev(bias), shortlist=didx)
+            assert np.array_equal(Aq.numpy(), Aq_h)
+        else:
+            Aq = upload_q(integer, Aq_h, (M, K))
+            acc = integer.multiply_i32(Aq, Bq, shortlist=didx).cpu().numpy()
+            assert np.array_equal(acc, want_acc)
+            out = integer.multiply(Aq, Bq, dev(bias), shortlist=didx)
+        out = out.cpu().numpy()
+    finally:
+        lib.marian_hip_int8_set_kernel(prev)
+    assert np.array_equal(out, want)
+
+
 def test_config1_single_affine_end_to_end(integer, orc, synth):
     """BASELINE config 1: A[64x512] ~ N(0,1), W[512x2048] ~ N(0,0.02^2), bias ~ N(0,0.01^2), ReLU."""
     say("config1")
