@@ -95,68 +95,6 @@ inline bool stream32_can_fuse(int64_t M, int64_t K) {
   return M <= 128 && M * K <= kFusedMaxElems && stream32_fused_lds_bytes(mt32, (int)K) <= 64 * 1024;
 }
 
-template <int MT32, int WN, int KW, int PW, bool FUSED>
-int launch_stream32(const GemmArgs& a, const float* A, int8_t* aq_out, hipStream_t st) {
-  using Cfg = Stream32Cfg<MT32, WN, KW, PW>;
-  auto kernel = gemm_stream32_kernel<MT32, WN, KW, PW, FUSED>;
-  constexpr int kMaxLds = 64 * 1024 > Cfg::kLdsBytes ? 64 * 1024 : Cfg::kLdsBytes;
-  static const int lds_status = allow_lds(kernel, kMaxLds);
-  if(lds_status != MARIAN_HIP_OK) return lds_status;
-  int lds = FUSED ? stream32_fused_lds_bytes(MT32, a.K) : Cfg::kStageBytes;
-  if(lds < Cfg::kReduceBytes) lds = Cfg::kReduceBytes;
-  int blocks = (a.n_out + Cfg::kColsPerBlock - 1) / Cfg::kColsPerBlock;
-  int m_tiles = FUSED ? 1 : (a.M + MT32 * 32 - 1) / (MT32 * 32);
-  hipLaunchKernelGGL(kernel, dim3(blocks, m_tiles), dim3(kStream32Threads), lds, st, a, A, aq_out);
-  MH_HIP(hipGetLastError());
-  return MARIAN_HIP_OK;
-}
-
-// Picks the number of K sub-steps a wave holds per chunk: the smallest instantiated value that
-// covers K in one chunk, else the largest whose activations fit the 64 KB LDS stage
-// (MT32 * KW * PW <= 64).
-template <int MT32, bool FUSED>
-int launch_stream32_kw(const GemmArgs& a, const float* A, int8_t* aq_out, hipStream_t st, int kw) {
-  const int need = (a.K / 32 + kw - 1) / kw;   // sub-steps per wave if K is one chunk
-  switch(kw) {
-    case 1: return launch_stream32<MT32, 8, 1, 8, FUSED>(a, A, aq_out, st);
-    case 2: return launch_stream32<MT32, 4, 2, 8, FUSED>(a, A, aq_out, st);
-    case 4:
-      if constexpr(MT32 <= 2) {
-        if(need > 4) return launch_stream32<MT32, 2, 4, 8, FUSED>(a, A, aq_out, st);
-      }
-      return launch_stream32<MT32, 2, 4, 4, FUSED>(a, A, aq_out, st);
-    default:
-      if constexpr(MT32 == 1) {
-        if(need > 4) return launch_stream32<MT32, 1, 8, 8, FUSED>(a, A, aq_out, st);
-      }
-      if constexpr(MT32 <= 2) {
-        if(need > 2) return launch_stream32<MT32, 1, 8, 4, FUSED>(a, A, aq_out, st);
-      }
-      return launch_stream32<MT32, 1, 8, 2, FUSED>(a, A, aq_out, st);
-  }
-}
-
-// kw_override: 0 = pick the K split from the number of 32-column weight tiles.
-// mt_override: 0 = activation rows per workgroup chosen here (the fused form takes all of M).
-template <bool FUSED>
-int launch_stream32_auto(const GemmArgs& a, const float* A, int8_t* aq_out, hipStream_t st,
-                         int kw_override, int mt_override = 0) {
-  const int tiles = (a.n_out + 31) / 32;
-  int kw = tiles < 512 ? 8 : (tiles < 1000 ? 4 : (tiles < 4096 ? 2 : 1));
-  if(kw_override) kw = kw_override;
-  while(kw > 1 && a.K / 32 < kw) kw >>= 1;
-  int mt = a.M <= 32 ? 1 : (a.M <= 64 ? 2 : 4);
-  if(!FUSED) {
-    // few weight tiles: split M over workgroups as well, so that more CUs pull on the operands
-    // and each workgroup stages fewer activation rows
-    if(tiles < 256 && mt > 1) mt = 1;
-    if(mt_override) mt = mt_override;
-  }
-  if(mt == 1) return launch_stream32_kw<1, FUSED>(a, A, aq_out, st, kw);
-  if(mt == 2) return launch_stream32_kw<2, FUSED>(a, A, aq_out, st, kw);
-  return launch_stream32_kw<4, FUSED>(a, A, aq_out, st, kw);
-}
-
 int compute_units() {
   static const int cus = [] {
     int dev = 0, n = 0;
@@ -166,6 +104,98 @@ int compute_units() {
     return n;
   }();
   return cus;
+}
+
+struct FusedSrc {   // what the fused modes read and write besides GemmArgs
+  const float* A = nullptr;
+  int8_t* aq_out = nullptr;
+  const float* partials = nullptr;
+  int n_partials = 0;
+};
+
+template <int MT32, int WN, int KW, int PW, int MODE>
+int launch_stream32(const GemmArgs& a, const FusedSrc& f, hipStream_t st) {
+  using Cfg = Stream32Cfg<MT32, WN, KW, PW>;
+  auto kernel = gemm_stream32_kernel<MT32, WN, KW, PW, MODE>;
+  constexpr int kMaxLds = 64 * 1024 > Cfg::kLdsBytes ? 64 * 1024 : Cfg::kLdsBytes;
+  static const int lds_status = allow_lds(kernel, kMaxLds);
+  if(lds_status != MARIAN_HIP_OK) return lds_status;
+  int lds = MODE == kFusedAll ? stream32_fused_lds_bytes(MT32, a.K) : Cfg::kStageBytes;
+  if(lds < Cfg::kReduceBytes) lds = Cfg::kReduceBytes;
+  int blocks = (a.n_out + Cfg::kColsPerBlock - 1) / Cfg::kColsPerBlock;
+  int m_tiles = MODE == kFusedAll ? 1 : (a.M + MT32 * 32 - 1) / (MT32 * 32);
+  hipLaunchKernelGGL(kernel, dim3(blocks, m_tiles), dim3(kStream32Threads), lds, st, a, f.A,
+                     f.aq_out, f.partials, f.n_partials);
+  MH_HIP(hipGetLastError());
+  return MARIAN_HIP_OK;
+}
+
+// Picks the number of K sub-steps a wave holds per chunk: the smallest instantiated value that
+// covers K in one chunk, else the largest whose activations fit the 64 KB LDS stage
+// (MT32 * KW * PW <= 64).  kFusedTiled stages fp32 values in registers: at most 4 per wave (8 when K is not split).
+template <int MT32, int MODE>
+int launch_stream32_kw(const GemmArgs& a, const FusedSrc& f, hipStream_t st, int kw) {
+  const int need = (a.K / 32 + kw - 1) / kw;   // sub-steps per wave if K is one chunk
+  if constexpr(MODE == kFusedTiled) {
+    static_assert(MT32 == 1, "tiled fused form: 32 rows per workgroup");
+    switch(kw) {
+      case 1: return launch_stream32<1, 8, 1, 8, MODE>(a, f, st);
+      case 2: return launch_stream32<1, 4, 2, 4, MODE>(a, f, st);
+      case 4: return launch_stream32<1, 2, 4, 4, MODE>(a, f, st);
+      default:
+        if(need > 2) return launch_stream32<1, 1, 8, 4, MODE>(a, f, st);
+        return launch_stream32<1, 1, 8, 2, MODE>(a, f, st);
+    }
+  } else {
+    switch(kw) {
+      case 1: return launch_stream32<MT32, 8, 1, 8, MODE>(a, f, st);
+      case 2: return launch_stream32<MT32, 4, 2, 8, MODE>(a, f, st);
+      case 4:
+        if constexpr(MT32 <= 2) {
+          if(need > 4) return launch_stream32<MT32, 2, 4, 8, MODE>(a, f, st);
+        }
+        return launch_stream32<MT32, 2, 4, 4, MODE>(a, f, st);
+      default:
+        if constexpr(MT32 == 1) {
+          if(need > 4) return launch_stream32<MT32, 1, 8, 8, MODE>(a, f, st);
+        }
+        if constexpr(MT32 <= 2) {
+          if(need > 2) return launch_stream32<MT32, 1, 8, 4, MODE>(a, f, st);
+        }
+        return launch_stream32<MT32, 1, 8, 2, MODE>(a, f, st);
+    }
+  }
+}
+
+// kw_override: 0 = pick the K split from the number of workgroups it gives.
+// mt_override: 0 = activation rows per workgroup chosen here (kFusedAll takes all of M,
+// kFusedTiled 32).
+template <int MODE>
+int launch_stream32_auto(const GemmArgs& a, const FusedSrc& f, hipStream_t st, int kw_override,
+                         int mt_override = 0) {
+  const int tiles = (a.n_out + 31) / 32;
+  int mt = a.M <= 32 ? 1 : (a.M <= 64 ? 2 : 4);
+  if(MODE == kPrequant) {
+    // few weight tiles: split M over workgroups as well, so that more CUs pull on the operands
+    // and each workgroup stages fewer activation rows
+    if(tiles < 256 && mt > 1) mt = 1;
+    if(mt_override) mt = mt_override;
+  }
+  if(MODE == kFusedTiled) mt = 1;
+  const int m_tiles = MODE == kFusedAll ? 1 : (a.M + mt * 32 - 1) / (mt * 32);
+  // the widest K split (most loads in flight per weight row) that stays within one workgroup
+  // per CU; the narrowest if none does
+  int kw = 8;
+  while(kw > 1 && (long long)((tiles * kw + 7) / 8) * m_tiles > compute_units()) kw >>= 1;
+  if(kw_override) kw = kw_override;
+  while(kw > 1 && a.K / 32 < kw) kw >>= 1;
+  if constexpr(MODE == kFusedTiled) {
+    return launch_stream32_kw<1, MODE>(a, f, st, kw);
+  } else {
+    if(mt == 1) return launch_stream32_kw<1, MODE>(a, f, st, kw);
+    if(mt == 2) return launch_stream32_kw<2, MODE>(a, f, st, kw);
+    return launch_stream32_kw<4, MODE>(a, f, st, kw);
+  }
 }
 
 template <int BM, int BN, int WM, int WN, int NSTAGE, bool DIRECT = false>
@@ -235,14 +265,14 @@ int launch_gemm(const GemmArgs& a, hipStream_t st) {
     case 312: return launch_big<128, 128, 2, 4, 2>(a, st);
     case 313: return launch_big<128, 64, 2, 2, 3>(a, st);
     case 314: return launch_big<128, 64, 4, 2, 2>(a, st);
-    case 501: return launch_stream32_auto<false>(a, nullptr, nullptr, st, 0);
-    case 521: return launch_stream32_auto<false>(a, nullptr, nullptr, st, 0, 1);
-    case 522: return launch_stream32_auto<false>(a, nullptr, nullptr, st, 0, 2);
-    case 524: return launch_stream32_auto<false>(a, nullptr, nullptr, st, 0, 4);
-    case 511: return launch_stream32_auto<false>(a, nullptr, nullptr, st, 1);
-    case 512: return launch_stream32_auto<false>(a, nullptr, nullptr, st, 2);
-    case 514: return launch_stream32_auto<false>(a, nullptr, nullptr, st, 4);
-    case 518: return launch_stream32_auto<false>(a, nullptr, nullptr, st, 8);
+    case 501: return launch_stream32_auto<kPrequant>(a, FusedSrc(), st, 0);
+    case 521: return launch_stream32_auto<kPrequant>(a, FusedSrc(), st, 0, 1);
+    case 522: return launch_stream32_auto<kPrequant>(a, FusedSrc(), st, 0, 2);
+    case 524: return launch_stream32_auto<kPrequant>(a, FusedSrc(), st, 0, 4);
+    case 511: return launch_stream32_auto<kPrequant>(a, FusedSrc(), st, 1);
+    case 512: return launch_stream32_auto<kPrequant>(a, FusedSrc(), st, 2);
+    case 514: return launch_stream32_auto<kPrequant>(a, FusedSrc(), st, 4);
+    case 518: return launch_stream32_auto<kPrequant>(a, FusedSrc(), st, 8);
     case 411: return launch_persistent<128, 128, 2, 2, 2, true>(a, st, 2, 0);
     case 412: return launch_persistent<128, 128, 2, 2, 2, true>(a, st, 2, 1);
     case 413: return launch_persistent<128, 128, 2, 2, 2, true>(a, st, 2, 2);
@@ -256,14 +286,12 @@ int launch_gemm(const GemmArgs& a, hipStream_t st) {
     default: break;
   }
   // Small M (decode): the weights are streamed once, the activations sit in LDS.
-  //  - up to 16 rows, and the 32000-column vocabulary at up to 64 rows: 16x16x64 MFMA kernels
+  //  - up to 8 rows (16 for narrow outputs): the 16x16x64 MFMA kernel, one 16-row tile
   //  - otherwise the 32x32x32 MFMA kernel, which also tiles M (shortlisted output layer, M = 256)
   const int tiles32 = (a.n_out + 31) / 32;
-  if(a.M <= 16) return launch_stream_auto(a, st, 2);
-  if(a.M <= 64 && tiles32 >= 512) return launch_stream_auto(a, st, 1);
-  if(a.M <= 128 && tiles32 >= 512) return launch_stream_auto(a, st, 1);
+  if(a.M <= 8 || (a.M <= 16 && tiles32 < 512)) return launch_stream_auto(a, st, 2);
   if(a.M <= 128 || (a.M <= 512 && tiles32 < 128))
-    return launch_stream32_auto<false>(a, nullptr, nullptr, st, 0);
+    return launch_stream32_auto<kPrequant>(a, FusedSrc(), st, 0);
   if(a.K % 128 != 0) return launch_tile<4, 4>(a, st);
   // large outputs: 256x256 tiles (one per CU keeps operand traffic lowest); otherwise 128x128
   // tiles with a three-deep LDS ring so that enough loads are in flight per CU
@@ -413,19 +441,39 @@ int marian_hip_int8_affine_f32(const float* A, int8_t* Aq, const int8_t* Bq, con
   if(M == 0) return MARIAN_HIP_OK;
   if(!A) return MARIAN_HIP_ERR_NULL;
   if(!aligned(A, 16)) return MARIAN_HIP_ERR_ALIGN;
+  // Measurement ids: 600 = separate prepareA and GEMM launches; 611/612/614/618 = one fused
+  // kernel with that K split; 620 = abs-max launch + tiled fused kernel, 621/622/624/628 with
+  // that K split.
   const int which = g_kernel_override.load(std::memory_order_relaxed) % 1000;
-  if(n_out > 0 && stream32_can_fuse(M, K) && which != 600) {
-    GemmArgs a;
-    a.Aq = Aq; a.Bq = Bq; a.bias = bias; a.idx = idx; a.out = out;
-    a.M = (int)M; a.K = (int)K; a.N = (int)N; a.n_out = (int)n_out;
-    a.scale = scale; a.relu = relu ? 1 : 0; a.dump = 0; a.dbg = 0;
-    a.prof = g_prof.load(std::memory_order_relaxed);
+  hipStream_t hst = reinterpret_cast<hipStream_t>(stream);
+  GemmArgs a;
+  a.Aq = Aq; a.Bq = Bq; a.bias = bias; a.idx = idx; a.out = out;
+  a.M = (int)M; a.K = (int)K; a.N = (int)N; a.n_out = (int)n_out;
+  a.scale = scale; a.relu = relu ? 1 : 0; a.dump = 0; a.dbg = 0;
+  a.prof = g_prof.load(std::memory_order_relaxed);
+  FusedSrc f;
+  f.A = A; f.aq_out = Aq;
+  const bool want_tiled = which >= 620 && which <= 628;
+  if(n_out > 0 && stream32_can_fuse(M, K) && which != 600 && !want_tiled) {
     int kw = 0;
-    if(which == 611) kw = 1;
-    if(which == 612) kw = 2;
-    if(which == 614) kw = 4;
-    if(which == 618) kw = 8;
-    return launch_stream32_auto<true>(a, A, Aq, reinterpret_cast<hipStream_t>(stream), kw);
+    if(which >= 611 && which <= 618) kw = which - 610;
+    return launch_stream32_auto<kFusedAll>(a, f, hst, kw);
+  }
+  // Mid-size activations: every workgroup quantizes its own 32 rows, so the work is repeated
+  // once per 32..256 output columns; measured to pay (one launch fewer) only for short rows and
+  // moderate output widths.
+  const bool tiled_ok = n_out > 0 && workspace && workspace_bytes >= kWorkspaceBytes &&
+                        aligned(workspace, 4);
+  if(tiled_ok && which != 600 && (want_tiled || (M <= 256 && K <= 1024 && n_out <= 8192))) {
+    const size_t n = (size_t)M * (size_t)K;
+    float* partials = reinterpret_cast<float*>(workspace);
+    const int g = absmax_blocks(n / 4);
+    hipLaunchKernelGGL(absmax_partial_kernel, dim3(g), dim3(kQuantThreads), 0, hst, A, n / 4,
+                       partials);
+    MH_HIP(hipGetLastError());
+    f.partials = partials;
+    f.n_partials = g;
+    return launch_stream32_auto<kFusedTiled>(a, f, hst, want_tiled ? which - 620 : 0);
   }
   st = marian_hip_int8_prepare_a(A, Aq, M, K, workspace, workspace_bytes, stream);
   if(st != MARIAN_HIP_OK) return st;

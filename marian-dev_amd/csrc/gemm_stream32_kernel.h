@@ -10,10 +10,13 @@
 // conflict free).  The 8 waves of a workgroup are arranged WN (different weight rows) x KW (different K
 // ranges of the same rows); the KW partial sums are added through LDS (exact in any order).
 //
-// FUSED: the workgroup reads the fp32 activations itself, takes their abs-max (every workgroup
-// gets the same value: max is exact and order independent), quantizes them into LDS and so
-// replaces a separate prepareA launch.  Workgroup 0 also writes the quantized activations and
-// their quantMult to global memory, exactly what prepareA would have produced.
+// MODE kFusedAll: the workgroup reads the fp32 activations itself, takes their abs-max (every
+// workgroup gets the same value: max is exact and order independent), quantizes them into LDS
+// and so replaces a separate prepareA launch.  Workgroup 0 also writes the quantized activations
+// and their quantMult to global memory, exactly what prepareA would have produced.
+// MODE kFusedTiled: for activations too large for that.  A separate small kernel leaves per-
+// workgroup abs-max values; this kernel reduces them, and quantizes its own 32 * MT32 rows chunk
+// by chunk on the way into LDS (the workgroups of column 0 also write them out).
 #pragma once
 
 #include "int8_common.h"
@@ -27,6 +30,7 @@ constexpr int kStream32Waves = 8;
 constexpr int kStream32Threads = kStream32Waves * kWave;
 constexpr int kFusedMaxElems = 32768;   // fp32 activations a workgroup holds in registers
 constexpr int kFusedGroups = kFusedMaxElems / 16 / kStream32Threads;   // 16-value groups per thread
+constexpr int kPrequant = 0, kFusedAll = 1, kFusedTiled = 2;            // MODE
 
 // MT32: 32-row activation tiles per workgroup (blockIdx.y walks M in steps of 32 * MT32; the
 // fused form needs all of M in one workgroup).  PW: 32-byte K sub-steps (weight loads in flight)
@@ -46,13 +50,17 @@ struct Stream32Cfg {
   static_assert(CS * MT32 * 64 % kStream32Threads == 0, "stage must divide over the threads");
 };
 
-// Dynamic LDS: FUSED holds all of K (32 * MT32 * K bytes); otherwise one chunk (kStageBytes);
-// both at least kReduceBytes.
-template <int MT32, int WN, int KW, int PW, bool FUSED>
+// Dynamic LDS: kFusedAll holds all of K (32 * MT32 * K bytes); otherwise one chunk (kStageBytes);
+// both at least kReduceBytes.  partials: n_partials (1..1024) abs-max values (kFusedTiled only).
+template <int MT32, int WN, int KW, int PW, int MODE>
 __global__ __launch_bounds__(kStream32Threads) void gemm_stream32_kernel(GemmArgs args,
                                                                         const float* A,
-                                                                        int8_t* aq_out) {
+                                                                        int8_t* aq_out,
+                                                                        const float* partials,
+                                                                        int n_partials) {
   using Cfg = Stream32Cfg<MT32, WN, KW, PW>;
+  constexpr bool FUSED = MODE == kFusedAll;
+  constexpr bool TILED = MODE == kFusedTiled;
   extern __shared__ __attribute__((aligned(16))) int8_t lds[];
   __shared__ float red[kStream32Waves];
 
@@ -103,7 +111,12 @@ __global__ __launch_bounds__(kStream32Threads) void gemm_stream32_kernel(GemmArg
   }
   const float bqm = tail_quant_mult(args.Bq, (size_t)K * (size_t)args.N);
   float aqm_pre = 0.0f;
-  if(!FUSED) aqm_pre = tail_quant_mult(args.Aq, (size_t)M * (size_t)K);
+  if(MODE == kPrequant) aqm_pre = tail_quant_mult(args.Aq, (size_t)M * (size_t)K);
+  float amax = 0.0f;
+  if(TILED) {   // two (clamped) abs-max partials per thread cover all 1024
+    amax = fmaxf(partials[min(tid, n_partials - 1)],
+                 partials[min(tid + kStream32Threads, n_partials - 1)]);
+  }
   const int8_t* wrow = args.Bq + (size_t)wsrc * (size_t)K + lg * 16;
   __builtin_amdgcn_sched_barrier(0);
 
@@ -112,7 +125,6 @@ __global__ __launch_bounds__(kStream32Threads) void gemm_stream32_kernel(GemmArg
   // A thread owns groups of 16 consecutive values of one activation row (one 16-byte LDS slot
   // after quantization): group number gi = j * threads + tid is row gi / (K/16), chunk gi % (K/16).
   v4f vals[FUSED ? kFusedGroups : 1][4];
-  float amax = 0.0f;
   const int n16 = M * K / 16;
   if(FUSED) {
     const v4f* a4 = reinterpret_cast<const v4f*>(A);
@@ -127,6 +139,72 @@ __global__ __launch_bounds__(kStream32Threads) void gemm_stream32_kernel(GemmArg
       }
     }
   }
+
+  float aqm = 0.0f;        // quantMult of the activations (fused modes)
+  bool finite_t = false;   // kFusedTiled: abs-max finite and non-zero
+  // Otherwise a chunk of activations is fetched into registers (all loads in flight at once) and
+  // then dropped into LDS, so the fetch of chunk c+1 overlaps the multiplication of chunk c.
+  // Pre-quantized: thread slot (sub-step, m-tile, lane) in operand order.  kFusedTiled: fp32
+  // source; a thread takes 16 consecutive values of a row (slot = row * 2 * CS + 16-byte chunk,
+  // so that a wave reads whole rows), quantizes them and finds the operand slot from there.
+  constexpr int kStageVecs = Cfg::CS * MT32 * 64 / kStream32Threads;
+  v4i stage[TILED ? 1 : kStageVecs];
+  v4f stagef[TILED ? kStageVecs : 1][4];
+  auto stage_fetch = [&](int chunk) {
+    const int s0 = chunk * Cfg::CS;
+#pragma unroll
+    for(int j = 0; j < kStageVecs; ++j) {
+      const int slot = j * kStream32Threads + tid;
+      if(TILED) {
+        const int r = slot / (2 * Cfg::CS), c16 = slot % (2 * Cfg::CS);
+        const int m = min(m_base + r, M - 1), s = min(s0 + c16 / 2, S - 1);
+        const v4f* src = reinterpret_cast<const v4f*>(A + (size_t)m * (size_t)K + s * 32 + (c16 % 2) * 16);
+#pragma unroll
+        for(int e = 0; e < 4; ++e) stagef[j][e] = src[e];
+      } else {
+        const int l = slot % 64, f = slot / 64;
+        const int mt = f % MT32, step = f / MT32;
+        const int m = m_base + mt * 32 + (l % 32);
+        const int s = s0 + step;
+        stage[j] = load16(args.Aq + (size_t)min(m, M - 1) * (size_t)K + min(s, S - 1) * 32 + (l / 32) * 16);
+      }
+    }
+  };
+  auto stage_store = [&](int chunk) {
+#pragma unroll
+    for(int j = 0; j < kStageVecs; ++j) {
+      const int slot = j * kStream32Threads + tid;
+      if(TILED) {
+        const int r = slot / (2 * Cfg::CS), c16 = slot % (2 * Cfg::CS);
+        const int m = m_base + r, s = chunk * Cfg::CS + c16 / 2;
+        uint4 q;
+        if(finite_t) {
+          q.x = quantize_pack4_finite(stagef[j][0], aqm);
+          q.y = quantize_pack4_finite(stagef[j][1], aqm);
+          q.z = quantize_pack4_finite(stagef[j][2], aqm);
+          q.w = quantize_pack4_finite(stagef[j][3], aqm);
+        } else {
+          q.x = quantize_pack4(stagef[j][0], aqm);
+          q.y = quantize_pack4(stagef[j][1], aqm);
+          q.z = quantize_pack4(stagef[j][2], aqm);
+          q.w = quantize_pack4(stagef[j][3], aqm);
+        }
+        // rows past M hold zeros (sub-steps past K multiply zero weights, any value will do)
+        if(m >= M) q = uint4{0, 0, 0, 0};
+        const int sw = ((c16 / 2) * MT32 + r / 32) * 64 + (c16 % 2) * 32 + ((r % 32) ^ (c16 & 7));
+        *reinterpret_cast<uint4*>(lds + sw * 16) = q;
+        if(aq_out && blockIdx.x == 0 && m < M && s < S)
+          *reinterpret_cast<uint4*>(aq_out + (size_t)m * (size_t)K + s * 32 + (c16 % 2) * 16) = q;
+      } else {
+        const int l = slot % 64, f = slot / 64;
+        const int mt = f % MT32, step = f / MT32;
+        const int sw = (slot & ~31) | ((l % 32) ^ ((2 * step + l / 32) & 7));
+        const bool live = m_base + mt * 32 + (l % 32) < M;
+        *reinterpret_cast<v4i*>(lds + sw * 16) = live ? stage[j] : v4i{0, 0, 0, 0};
+      }
+    }
+  };
+  if(!FUSED) stage_fetch(0);   // ahead of the weights, like the fp32 activations above
 
   v4i w[Cfg::PW];
   auto load_weights = [&](int chunk) {
@@ -146,7 +224,13 @@ __global__ __launch_bounds__(kStream32Threads) void gemm_stream32_kernel(GemmArg
 
   // ---- activations into LDS, operand order: slot (sub-step, m-tile, lane) of 16 bytes holds
   //      Aq[mt*32 + lane%32][(s0+step)*32 + (lane/32)*16 .. +15]
-  float aqm = 0.0f;
+  if(TILED) {
+    amax = block_max(amax, red);
+    aqm = quant_mult_from_maxabs(amax);
+    finite_t = amax > 0.0f && amax < __builtin_inff();
+    if(aq_out && blockIdx.x == 0 && blockIdx.y == 0 && tid == 0)
+      *reinterpret_cast<float*>(aq_out + (size_t)M * K) = aqm;
+  }
   if(FUSED) {
     // whole A (M*K <= kFusedMaxElems floats) in registers: abs-max, then quantize into LDS
 #pragma unroll
@@ -199,37 +283,8 @@ __global__ __launch_bounds__(kStream32Threads) void gemm_stream32_kernel(GemmArg
       *reinterpret_cast<float*>(aq_out + (size_t)M * K) = aqm;
     __syncthreads();
   }
-  // Pre-quantized activations: a chunk is fetched into registers (all loads in flight at once)
-  // and then dropped into LDS, so the fetch of chunk c+1 overlaps the multiplication of chunk c.
-  constexpr int kStageVecs = Cfg::CS * MT32 * 64 / kStream32Threads;
-  v4i stage[kStageVecs];
-  auto stage_fetch = [&](int chunk) {
-    const int s0 = chunk * Cfg::CS;
-#pragma unroll
-    for(int j = 0; j < kStageVecs; ++j) {
-      const int slot = j * kStream32Threads + tid;
-      const int l = slot % 64, f = slot / 64;
-      const int mt = f % MT32, step = f / MT32;
-      const int m = m_base + mt * 32 + (l % 32);
-      const int s = s0 + step;
-      stage[j] = load16(args.Aq + (size_t)min(m, M - 1) * (size_t)K + min(s, S - 1) * 32 + (l / 32) * 16);
-    }
-  };
-  auto stage_store = [&]() {
-#pragma unroll
-    for(int j = 0; j < kStageVecs; ++j) {
-      const int slot = j * kStream32Threads + tid;
-      const int l = slot % 64, f = slot / 64;
-      const int mt = f % MT32, step = f / MT32;
-      const int sw = (slot & ~31) | ((l % 32) ^ ((2 * step + l / 32) & 7));
-      // rows past M hold zeros (sub-steps past K multiply zero weights, any value will do)
-      const bool live = m_base + mt * 32 + (l % 32) < M;
-      *reinterpret_cast<v4i*>(lds + sw * 16) = live ? stage[j] : v4i{0, 0, 0, 0};
-    }
-  };
   if(!FUSED) {
-    stage_fetch(0);
-    stage_store();
+    stage_store(0);
     __syncthreads();
   }
 
@@ -268,7 +323,7 @@ __global__ __launch_bounds__(kStream32Threads) void gemm_stream32_kernel(GemmArg
     if(more) {
       if(!FUSED) {
         __syncthreads();   // everyone is done reading chunk c
-        stage_store();
+        stage_store(c + 1);
         __syncthreads();
       }
 #pragma unroll
@@ -322,7 +377,7 @@ __global__ __launch_bounds__(kStream32Threads) void gemm_stream32_kernel(GemmArg
   //      row 8 * (v / 4) + 4 * lg + v % 4 of the wave's 32 ----
   if(args.prof) tp[4] = clock64();
   {
-    const float unquant = unquant_mult(FUSED ? aqm : aqm_pre, bqm, args.scale);
+    const float unquant = unquant_mult(MODE == kPrequant ? aqm_pre : aqm, bqm, args.scale);
     const bool has_bias = args.bias != nullptr;
 #pragma unroll
     for(int c = 0; c < NC; ++c) {
