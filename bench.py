@@ -35,8 +35,8 @@ INT8_PEAK_TOPS = 5000.0      # MI355X dense int8 MFMA, published (5.0 POP/s)
 # runs of `bench.py --pmc-probe` (KiB per dispatch, scaled by the same counters' reading for a
 # plain copy of known size); the runs are summarised under profiles/.  None = not measured.
 MEASURED_TRAFFIC = {
-    # (8700.2 KiB FETCH_SIZE x 1.9992 + 8032.1 KiB WRITE_SIZE) per dispatch
-    "stream32_fused_M64_K512_N32000": int((8700.2 * 1.9992 + 8032.1) * 1024),
+    # (8683.1 KiB FETCH_SIZE x 1.9992 + 8107.7 KiB WRITE_SIZE) per dispatch
+    "stream32_fused_M64_K512_N32000": int((8683.1 * 1.9992 + 8107.7) * 1024),
 }
 
 DECODE_SHAPES = [(512, 1536), (512, 512), (512, 2048), (2048, 512), (512, 32000)]
@@ -269,7 +269,7 @@ def main():
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                 "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                 "traffic": MEASURED_TRAFFIC.get("stream32_fused_M64_K512_N32000"),
-                "kernel": "gemm_stream32_kernel<2,4,2,fused> M=64 K=512 N=32000",
+                "kernel": "gemm_stream32_kernel<MT32=2,WN=4,KW=2,PW=8,fused> M=64 K=512 N=32000",
                 "bytes_per_launch": dom_bytes, "avg_launch_us": round(mean_ms * 1e3, 3),
                 "median_launch_us": round(med_ms * 1e3, 3),
                 "launches_timed": 12 * sets}
