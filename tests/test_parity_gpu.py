@@ -317,6 +317,49 @@ def test_config5_shortlist(integer, orc, synth, M):
     assert np.array_equal(dense_acc[rows], want_acc) and np.array_equal(dense[rows], want)
 
 
+# ---------------------------------------------------------------- random shapes
+
+def _random_cases(n):
+    """Seeded shapes over everything the dispatch distinguishes: M 1..600, K a multiple of 64 up
+    to 2048, N a multiple of 8 up to 5000, with and without bias / ReLU / scale / shortlist."""
+    rng = np.random.default_rng(20261125)
+    cases = []
+    for i in range(n):
+        M = int(rng.choice([1, 2, 7, 16, 17, 31, 33, 64, 65, 100, 128, 129, 200, 257, 384, 600]))
+        K = 64 * int(rng.integers(1, 33))
+        N = 8 * int(rng.integers(1, 626))
+        cases.append((i, M, K, N, bool(rng.integers(2)), bool(rng.integers(2)),
+                      float(rng.choice([1.0, 0.5, 0.125, 3.0])), bool(rng.integers(3) == 0)))
+    return cases
+
+
+@pytest.mark.parametrize("i,M,K,N,bias_on,relu,scale,short", _random_cases(48))
+def test_random_shapes_both_entry_points(integer, orc, synth, i, M, K, N, bias_on, relu, scale, short):
+    """Automatic kernel choice on seeded random shapes: the two-call form (prepareA, multiply) and
+    the single fused call give the checker's bits."""
+    import torch
+    say("random", i, M, K, N, bias_on, relu, scale, short)
+    A, W, bias = inputs(synth, 5000 + i, M, K, N)
+    Aq_h, Bq_h = orc.prepare_a(A), orc.prepare_b(W)
+    b = bias if bias_on else None
+    idx = didx = None
+    if short and N >= 64:
+        idx = synth.shortlist(5000 + i, N, 8, max(8, N // 2))
+        didx = torch.from_numpy(idx.view(np.int32)).cuda()
+        want, want_acc = orc.affine_shortlist(Aq_h, Bq_h, b, idx, M, K, N, scale, relu)
+    else:
+        want, want_acc = orc.affine(Aq_h, Bq_h, b, M, K, N, scale, relu)
+    Bq = upload_q(integer, Bq_h, (K, N))
+    db = dev(bias) if bias_on else None
+    Aq = integer.prepareA(dev(A))
+    assert np.array_equal(Aq.numpy(), Aq_h)
+    assert np.array_equal(integer.multiply_i32(Aq, Bq, shortlist=didx).cpu().numpy(), want_acc)
+    out2 = integer.multiply(Aq, Bq, db, scale=scale, relu=relu, shortlist=didx).cpu().numpy()
+    out1, Aq1 = integer.affine_f32(dev(A), Bq, db, scale=scale, relu=relu, shortlist=didx)
+    assert np.array_equal(Aq1.numpy(), Aq_h)
+    assert np.array_equal(out2, want) and np.array_equal(out1.cpu().numpy(), want)
+
+
 # ---------------------------------------------------------------- fixtures, contract, errors
 
 def test_golden_fixtures_on_gpu(integer):
