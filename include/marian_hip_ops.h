@@ -1,0 +1,74 @@
+/*
+ * marian_hip_ops.h - C ABI of the float32 operators that sit between the int8 GEMMs of a
+ * transformer decode step (same library and conventions as marian_hip_int8.h: device pointers,
+ * caller-owned buffers, nothing retained, work enqueued on `stream`, status codes, no
+ * synchronisation).  All tensors are dense row-major fp32; pointers need 4-byte alignment only
+ * (16-byte aligned rows take a vector path).  In-place operation (out == in) is allowed for
+ * layer_norm, softmax and logsoftmax.
+ */
+#ifndef MARIAN_HIP_OPS_H
+#define MARIAN_HIP_OPS_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/*
+ * Replaces LayerNormalization, reference src/tensors/gpu/tensor_operators.cu (gLNormalization)
+ * and src/tensors/cpu/tensor_operators.cpp:1087-1162, node LayerNormalizationOp
+ * (src/graph/expression_operators.cpp:901-913):
+ *   mean = sum(x) / cols; sigma = sqrt(sum((x - mean)^2) / cols + eps);
+ *   out = gamma * ((x - mean) / sigma) (+ beta)
+ * over the last dimension.  gamma_cols / beta_cols: `cols`, or 1 for a single broadcast value;
+ * beta may be NULL.  add != NULL fuses the skip connection that precedes the normalization in
+ * the transformer's post-processing (`output + prevInput`, src/models/transformer.h:192-193,207):
+ * x = in + add, else x = in.
+ */
+int marian_hip_layer_norm(const float* in, const float* add, const float* gamma,
+                          int64_t gamma_cols, const float* beta, int64_t beta_cols, float* out,
+                          int64_t rows, int64_t cols, float eps, void* stream);
+
+/*
+ * Replaces Softmax, reference src/tensors/gpu/tensor_operators.cu (gSoftmax) and
+ * src/tensors/cpu/tensor_operators.cpp:415-470, over the last dimension.  mask != NULL fuses the
+ * `z + mask` node in front of it (src/models/transformer.h:264): mask holds n_masks rows of
+ * `cols` values and row r of `in` uses mask row (r / rows_per_mask) % n_masks - a
+ * [batch, 1, 1, len] log-mask, repeated over the beam (src/models/transformer.h:772-774),
+ * against scores of shape [beam * batch, heads, tgt, len] has rows_per_mask = heads * tgt,
+ * n_masks = batch.
+ */
+int marian_hip_softmax(const float* in, const float* mask, int64_t n_masks, int64_t rows_per_mask,
+                       float* out, int64_t rows, int64_t cols, void* stream);
+
+/* Replaces LogSoftmax, reference src/tensors/gpu/tensor_operators.cu (gLogSoftmax) and
+ * src/tensors/cpu/tensor_operators.cpp:474-526. */
+int marian_hip_logsoftmax(const float* in, float* out, int64_t rows, int64_t cols, void* stream);
+
+/*
+ * Replaces TransposeND for the axes {0, 2, 1, 3} (Transpose0213, reference
+ * src/tensors/cpu/tensor_operators.cpp:220-246, gTranspose0213 on the GPU), the head split and
+ * join of src/models/transformer.h:145-170: in [d0, d1, d2, d3] -> out [d0, d2, d1, d3].
+ * out must not alias in.
+ */
+int marian_hip_transpose0213(const float* in, float* out, int64_t d0, int64_t d1, int64_t d2,
+                             int64_t d3, void* stream);
+
+/*
+ * Replaces ProdBatchedLegacy with beta = 0, reference src/tensors/cpu/prod.cpp:233-330 and
+ * src/tensors/gpu/prod.cpp:471-574 (node bdot_legacy, the attention products of
+ * src/models/transformer.h:261,277):
+ *   C[i] = scalar * op(A[i % batchA]) * op(B[i % batchB]),  i < max(batchA, batchB)
+ * A: [batchA, m, k] ([batchA, k, m] when transA), B: [batchB, k, n] ([batchB, n, k] when
+ * transB), C: [max(batchA, batchB), m, n].
+ */
+int marian_hip_bdot_legacy(const float* A, const float* B, float* C, int64_t batchA,
+                           int64_t batchB, int64_t m, int64_t n, int64_t k, int transA,
+                           int transB, float scalar, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MARIAN_HIP_OPS_H */

@@ -28,6 +28,12 @@ SIGNATURES = {
                                               _f, _i, _vp]),
     "marian_hip_int8_multiply_i32": (_i, [_vp, _vp, _vp, _i64, _vp, _i64, _i64, _i64, _vp]),
     "marian_hip_int8_set_kernel": (_i, [_i]),
+    # include/marian_hip_ops.h
+    "marian_hip_layer_norm": (_i, [_vp, _vp, _vp, _i64, _vp, _i64, _vp, _i64, _i64, _f, _vp]),
+    "marian_hip_softmax": (_i, [_vp, _vp, _i64, _i64, _vp, _i64, _i64, _vp]),
+    "marian_hip_logsoftmax": (_i, [_vp, _vp, _i64, _i64, _vp]),
+    "marian_hip_transpose0213": (_i, [_vp, _vp, _i64, _i64, _i64, _i64, _vp]),
+    "marian_hip_bdot_legacy": (_i, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i, _i, _f, _vp]),
 }
 
 _lib = None

@@ -6,6 +6,7 @@
 
 #include <atomic>
 
+#include "abi_common.h"
 #include "gemm_mfma32_kernel.h"
 #include "gemm_persistent_kernel.h"
 #include "gemm_stream32_kernel.h"
@@ -16,15 +17,20 @@
 using namespace marian_hip;
 
 namespace {
-
 thread_local int g_last_hip_error = 0;
+}
+
+int marian_hip::record_hip_error(int e) {
+  g_last_hip_error = e;
+  return MARIAN_HIP_ERR_HIP;
+}
+
+namespace {
+
 std::atomic<int> g_kernel_override{0};
 std::atomic<long long*> g_prof{nullptr};
 
-int hip_fail(hipError_t e) {
-  g_last_hip_error = (int)e;
-  return MARIAN_HIP_ERR_HIP;
-}
+int hip_fail(hipError_t e) { return marian_hip::record_hip_error((int)e); }
 
 #define MH_HIP(expr)                            \
   do {                                          \

@@ -1,0 +1,329 @@
+// Float32 operators between the int8 GEMMs of a transformer decode step: layer normalization
+// (with the skip connection in front of it), softmax (with the attention mask in front of it),
+// log-softmax, the 0213 transpose of the head split/join, and the batched attention products.
+// Declarations and the reference code each entry point replaces: include/marian_hip_ops.h
+//
+// All of them are memory- or latency-bound at decode sizes (a few hundred KB per call), so the
+// kernels are single-pass where the row fits in registers and use 64-lane wave reductions;
+// nothing here needs LDS tiling or MFMA.
+#include "../../include/marian_hip_ops.h"
+
+#include <hip/hip_runtime.h>
+
+#include "../../include/marian_hip_int8.h"
+#include "abi_common.h"
+#include "int8_common.h"
+
+using namespace marian_hip;
+
+namespace {
+
+constexpr int64_t kMaxElemsOps = 2147483647LL;
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for(int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+__device__ __forceinline__ float wave_maxf(float v) {
+#pragma unroll
+  for(int o = 32; o > 0; o >>= 1) {
+    const float t = __shfl_xor(v, o, 64);
+    v = t > v ? t : v;
+  }
+  return v;
+}
+
+// Reduction over the THREADS threads that share a row (64: one wave, no LDS; more: through LDS).
+// red: one float per wave of the workgroup.
+template <int THREADS, bool MAX>
+__device__ __forceinline__ float row_reduce(float v, float* red) {
+  v = MAX ? wave_maxf(v) : wave_sum(v);
+  if(THREADS > 64) {
+    const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+    __syncthreads();
+    if(lane == 0) red[wave] = v;
+    __syncthreads();
+    float r = red[0];
+#pragma unroll
+    for(int w = 1; w < THREADS / 64; ++w) r = MAX ? (red[w] > r ? red[w] : r) : r + red[w];
+    v = r;
+  }
+  return v;
+}
+
+// ---------------------------------------------------------------- layer normalization
+// One workgroup of 256 threads per row.  CACHE float4 vectors per thread hold the row in
+// registers (cols <= 1024 * CACHE, cols % 4 == 0, 16-byte aligned rows); CACHE == 0 is the
+// general form, which re-reads the row (it stays in L2).
+template <int CACHE>
+__global__ __launch_bounds__(256) void layer_norm_kernel(const float* in,
+                                                         const float* __restrict__ add,
+                                                         const float* __restrict__ gamma, int gamma_stride,
+                                                         const float* __restrict__ beta, int beta_stride,
+                                                         float* out, int cols, float eps) {
+  __shared__ float red[4];
+  const size_t row = blockIdx.x;
+  const float* x = in + row * cols;
+  const float* a = add ? add + row * cols : nullptr;
+  float* y = out + row * cols;
+  const int tid = threadIdx.x;
+  if(CACHE > 0) {
+    const int cols4 = cols / 4;
+    v4f v[CACHE > 0 ? CACHE : 1];
+    float sum = 0.0f;
+#pragma unroll
+    for(int j = 0; j < CACHE; ++j) {
+      const int i = j * 256 + tid;
+      v[j] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+      if(i < cols4) {
+        v[j] = reinterpret_cast<const v4f*>(x)[i];
+        if(a) {
+          const v4f t = reinterpret_cast<const v4f*>(a)[i];
+          v[j].x = v[j].x + t.x; v[j].y = v[j].y + t.y; v[j].z = v[j].z + t.z; v[j].w = v[j].w + t.w;
+        }
+        sum += (v[j].x + v[j].y) + (v[j].z + v[j].w);
+      }
+    }
+    const float mean = row_reduce<256, false>(sum, red) / (float)cols;
+    float sq = 0.0f;
+#pragma unroll
+    for(int j = 0; j < CACHE; ++j) {
+      if(j * 256 + tid < cols4) {
+        const float d0 = v[j].x - mean, d1 = v[j].y - mean, d2 = v[j].z - mean, d3 = v[j].w - mean;
+        sq += (d0 * d0 + d1 * d1) + (d2 * d2 + d3 * d3);
+      }
+    }
+    const float sigma = sqrtf(row_reduce<256, false>(sq, red) / (float)cols + eps);
+#pragma unroll
+    for(int j = 0; j < CACHE; ++j) {
+      const int i = j * 256 + tid;
+      if(i < cols4) {
+        float r[4] = {v[j].x, v[j].y, v[j].z, v[j].w};
+#pragma unroll
+        for(int e = 0; e < 4; ++e) {
+          float t = gamma[gamma_stride * (4 * i + e)] * ((r[e] - mean) / sigma);
+          if(beta) t = t + beta[beta_stride * (4 * i + e)];
+          r[e] = t;
+        }
+        reinterpret_cast<v4f*>(y)[i] = v4f{r[0], r[1], r[2], r[3]};
+      }
+    }
+  } else {
+    float sum = 0.0f;
+    for(int i = tid; i < cols; i += 256) sum += a ? x[i] + a[i] : x[i];
+    const float mean = row_reduce<256, false>(sum, red) / (float)cols;
+    float sq = 0.0f;
+    for(int i = tid; i < cols; i += 256) {
+      const float d = (a ? x[i] + a[i] : x[i]) - mean;
+      sq += d * d;
+    }
+    const float sigma = sqrtf(row_reduce<256, false>(sq, red) / (float)cols + eps);
+    for(int i = tid; i < cols; i += 256) {
+      float t = gamma[gamma_stride * i] * (((a ? x[i] + a[i] : x[i]) - mean) / sigma);
+      if(beta) t = t + beta[beta_stride * i];
+      y[i] = t;
+    }
+  }
+}
+
+// ---------------------------------------------------------------- softmax / log-softmax
+// THREADS threads per row, 256 / THREADS... rows per workgroup: 64 (a wave per row, four rows
+// per workgroup: attention scores) or 1024 (vocabulary-size rows).  Three passes over the row:
+// max, sum of exponentials, result; the row stays in L1/L2 between them.
+template <int THREADS, bool LOG>
+__global__ __launch_bounds__(THREADS < 256 ? 256 : THREADS) void softmax_kernel(
+    const float* in, const float* __restrict__ mask, long long n_masks,
+    long long rows_per_mask, float* out, long long rows, int cols) {
+  __shared__ float red[THREADS > 64 ? THREADS / 64 : 1];
+  constexpr int kRowsPerBlock = THREADS < 256 ? 256 / THREADS : 1;
+  const long long row = (long long)blockIdx.x * kRowsPerBlock + (THREADS < 256 ? threadIdx.x / THREADS : 0);
+  const int t = threadIdx.x % THREADS;
+  if(THREADS <= 64 && row >= rows) return;   // whole waves leave; no workgroup barrier is used
+  const float* x = in + (size_t)row * cols;
+  const float* m = mask ? mask + (size_t)((row / rows_per_mask) % n_masks) * cols : nullptr;
+  float* y = out + (size_t)row * cols;
+  float mx = -__builtin_inff();
+  for(int i = t; i < cols; i += THREADS) {
+    const float v = m ? x[i] + m[i] : x[i];
+    mx = v > mx ? v : mx;
+  }
+  mx = row_reduce<THREADS, true>(mx, red);
+  float sum = 0.0f;
+  for(int i = t; i < cols; i += THREADS) sum += expf((m ? x[i] + m[i] : x[i]) - mx);
+  sum = row_reduce<THREADS, false>(sum, red);
+  if(LOG) {
+    const float log_sum = logf(sum);
+    for(int i = t; i < cols; i += THREADS) y[i] = ((m ? x[i] + m[i] : x[i]) - mx) - log_sum;
+  } else {
+    for(int i = t; i < cols; i += THREADS) y[i] = expf((m ? x[i] + m[i] : x[i]) - mx) / sum;
+  }
+}
+
+// ---------------------------------------------------------------- transpose 0213
+// One element (VEC floats of the innermost dimension) per thread, indexed by the output.
+template <int VEC>
+__global__ __launch_bounds__(256) void transpose0213_kernel(const float* in,
+                                                            float* __restrict__ out, long long total,
+                                                            int d1, int d2, int d3v) {
+  const long long stride = (long long)gridDim.x * 256;
+  for(long long o = (long long)blockIdx.x * 256 + threadIdx.x; o < total; o += stride) {
+    const int i3 = (int)(o % d3v);
+    long long r = o / d3v;
+    const int i1 = (int)(r % d1);
+    r /= d1;
+    const int i2 = (int)(r % d2);
+    const long long i0 = r / d2;
+    const long long src = ((i0 * d1 + i1) * d2 + i2) * d3v + i3;
+    if(VEC == 4) reinterpret_cast<v4f*>(out)[o] = reinterpret_cast<const v4f*>(in)[src];
+    else out[o] = in[src];
+  }
+}
+
+// ---------------------------------------------------------------- batched product
+// One wave per output row (batch i, row r): lanes walk the n columns, every lane runs over k.
+// At decode sizes (m = 1, k or n = 64, a few thousand batch entries) a product is a matrix-vector
+// product of a few KB; the operands of a wave stay in L1 while it walks k.
+__global__ __launch_bounds__(256) void bdot_kernel(const float* __restrict__ A, const float* __restrict__ B,
+                                                   float* __restrict__ C, long long batchA,
+                                                   long long batchB, long long rows_total, int m, int n,
+                                                   int k, int transA, int transB, float scalar) {
+  const long long wr = (long long)blockIdx.x * 4 + threadIdx.x / 64;   // output row of this wave
+  if(wr >= rows_total) return;
+  const int lane = threadIdx.x % 64;
+  const long long i = wr / m;
+  const int r = (int)(wr % m);
+  const float* a = A + (size_t)(i % batchA) * m * k;
+  const float* b = B + (size_t)(i % batchB) * n * k;
+  float* c = C + (size_t)wr * n;
+  const int lda = transA ? m : k, ldb = transB ? k : n;
+  for(int q = lane; q < n; q += 64) {
+    float s = 0.0f;
+    if(!transA && transB && (k % 4) == 0 && ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b)) % 16) == 0) {
+      const v4f* ar = reinterpret_cast<const v4f*>(a + (size_t)r * lda);
+      const v4f* br = reinterpret_cast<const v4f*>(b + (size_t)q * ldb);
+      for(int p = 0; p < k / 4; ++p) {
+        const v4f av = ar[p], bv = br[p];
+        s = fmaf(av.x, bv.x, s);
+        s = fmaf(av.y, bv.y, s);
+        s = fmaf(av.z, bv.z, s);
+        s = fmaf(av.w, bv.w, s);
+      }
+    } else {
+      for(int p = 0; p < k; ++p) {
+        const float av = transA ? a[(size_t)p * lda + r] : a[(size_t)r * lda + p];
+        const float bv = transB ? b[(size_t)q * ldb + p] : b[(size_t)p * ldb + q];
+        s = fmaf(av, bv, s);
+      }
+    }
+    c[q] = scalar * s;
+  }
+}
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) % 16) == 0; }
+inline bool aligned4(const void* p) { return (reinterpret_cast<uintptr_t>(p) % 4) == 0; }
+
+#define MH_HIP(expr)                                      \
+  do {                                                    \
+    hipError_t e_ = (expr);                               \
+    if(e_ != hipSuccess) return record_hip_error((int)e_); \
+  } while(0)
+
+}  // namespace
+
+extern "C" {
+
+int marian_hip_layer_norm(const float* in, const float* add, const float* gamma, int64_t gamma_cols,
+                          const float* beta, int64_t beta_cols, float* out, int64_t rows,
+                          int64_t cols, float eps, void* stream) {
+  if(rows < 0 || cols <= 0) return MARIAN_HIP_ERR_SHAPE;
+  if((gamma_cols != cols && gamma_cols != 1) || (beta && beta_cols != cols && beta_cols != 1))
+    return MARIAN_HIP_ERR_SHAPE;
+  if(rows == 0) return MARIAN_HIP_OK;
+  if(!in || !gamma || !out) return MARIAN_HIP_ERR_NULL;
+  if(rows * cols > kMaxElemsOps) return MARIAN_HIP_ERR_RANGE;
+  if(!aligned4(in) || !aligned4(out) || !aligned4(gamma) || (add && !aligned4(add)) || (beta && !aligned4(beta)))
+    return MARIAN_HIP_ERR_ALIGN;
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  const int gs = gamma_cols > 1 ? 1 : 0, bs = (beta && beta_cols > 1) ? 1 : 0;
+  const bool vec = cols % 4 == 0 && aligned16(in) && aligned16(out) && (!add || aligned16(add));
+  if(vec && cols <= 1024)
+    hipLaunchKernelGGL(layer_norm_kernel<1>, dim3((unsigned)rows), dim3(256), 0, st, in, add, gamma, gs, beta, bs, out, (int)cols, eps);
+  else if(vec && cols <= 4096)
+    hipLaunchKernelGGL(layer_norm_kernel<4>, dim3((unsigned)rows), dim3(256), 0, st, in, add, gamma, gs, beta, bs, out, (int)cols, eps);
+  else
+    hipLaunchKernelGGL(layer_norm_kernel<0>, dim3((unsigned)rows), dim3(256), 0, st, in, add, gamma, gs, beta, bs, out, (int)cols, eps);
+  MH_HIP(hipGetLastError());
+  return MARIAN_HIP_OK;
+}
+
+static int softmax_common(const float* in, const float* mask, int64_t n_masks, int64_t rows_per_mask,
+                          float* out, int64_t rows, int64_t cols, bool log, void* stream) {
+  if(rows < 0 || cols <= 0) return MARIAN_HIP_ERR_SHAPE;
+  if(mask && (n_masks <= 0 || rows_per_mask <= 0)) return MARIAN_HIP_ERR_SHAPE;
+  if(rows == 0) return MARIAN_HIP_OK;
+  if(!in || !out) return MARIAN_HIP_ERR_NULL;
+  if(rows * cols > kMaxElemsOps) return MARIAN_HIP_ERR_RANGE;
+  if(!aligned4(in) || !aligned4(out) || (mask && !aligned4(mask))) return MARIAN_HIP_ERR_ALIGN;
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  if(!mask) { n_masks = 1; rows_per_mask = 1; }
+  if(cols <= 2048) {
+    const unsigned blocks = (unsigned)((rows + 3) / 4);
+    if(log) hipLaunchKernelGGL((softmax_kernel<64, true>), dim3(blocks), dim3(256), 0, st, in, mask, (long long)n_masks, (long long)rows_per_mask, out, (long long)rows, (int)cols);
+    else hipLaunchKernelGGL((softmax_kernel<64, false>), dim3(blocks), dim3(256), 0, st, in, mask, (long long)n_masks, (long long)rows_per_mask, out, (long long)rows, (int)cols);
+  } else {
+    if(log) hipLaunchKernelGGL((softmax_kernel<1024, true>), dim3((unsigned)rows), dim3(1024), 0, st, in, mask, (long long)n_masks, (long long)rows_per_mask, out, (long long)rows, (int)cols);
+    else hipLaunchKernelGGL((softmax_kernel<1024, false>), dim3((unsigned)rows), dim3(1024), 0, st, in, mask, (long long)n_masks, (long long)rows_per_mask, out, (long long)rows, (int)cols);
+  }
+  MH_HIP(hipGetLastError());
+  return MARIAN_HIP_OK;
+}
+
+int marian_hip_softmax(const float* in, const float* mask, int64_t n_masks, int64_t rows_per_mask,
+                       float* out, int64_t rows, int64_t cols, void* stream) {
+  return softmax_common(in, mask, n_masks, rows_per_mask, out, rows, cols, false, stream);
+}
+
+int marian_hip_logsoftmax(const float* in, float* out, int64_t rows, int64_t cols, void* stream) {
+  return softmax_common(in, nullptr, 1, 1, out, rows, cols, true, stream);
+}
+
+int marian_hip_transpose0213(const float* in, float* out, int64_t d0, int64_t d1, int64_t d2,
+                             int64_t d3, void* stream) {
+  if(d0 < 0 || d1 <= 0 || d2 <= 0 || d3 <= 0) return MARIAN_HIP_ERR_SHAPE;
+  if(d0 == 0) return MARIAN_HIP_OK;
+  if(!in || !out) return MARIAN_HIP_ERR_NULL;
+  if(in == out) return MARIAN_HIP_ERR_SHAPE;
+  if(d0 * d1 * d2 * d3 > kMaxElemsOps) return MARIAN_HIP_ERR_RANGE;
+  if(!aligned4(in) || !aligned4(out)) return MARIAN_HIP_ERR_ALIGN;
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  const bool vec = d3 % 4 == 0 && aligned16(in) && aligned16(out);
+  const long long total = d0 * d1 * d2 * (vec ? d3 / 4 : d3);
+  long long blocks = (total + 255) / 256;
+  if(blocks > 8192) blocks = 8192;
+  if(vec) hipLaunchKernelGGL(transpose0213_kernel<4>, dim3((unsigned)blocks), dim3(256), 0, st, in, out, total, (int)d1, (int)d2, (int)(d3 / 4));
+  else hipLaunchKernelGGL(transpose0213_kernel<1>, dim3((unsigned)blocks), dim3(256), 0, st, in, out, total, (int)d1, (int)d2, (int)d3);
+  MH_HIP(hipGetLastError());
+  return MARIAN_HIP_OK;
+}
+
+int marian_hip_bdot_legacy(const float* A, const float* B, float* C, int64_t batchA, int64_t batchB,
+                           int64_t m, int64_t n, int64_t k, int transA, int transB, float scalar,
+                           void* stream) {
+  if(batchA < 0 || batchB < 0 || m <= 0 || n <= 0 || k <= 0) return MARIAN_HIP_ERR_SHAPE;
+  if(batchA == 0 || batchB == 0) return MARIAN_HIP_OK;
+  if(!A || !B || !C) return MARIAN_HIP_ERR_NULL;
+  const int64_t batchC = batchA > batchB ? batchA : batchB;
+  if(batchA * m * k > kMaxElemsOps || batchB * n * k > kMaxElemsOps || batchC * m * n > kMaxElemsOps)
+    return MARIAN_HIP_ERR_RANGE;
+  if(!aligned4(A) || !aligned4(B) || !aligned4(C)) return MARIAN_HIP_ERR_ALIGN;
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  const long long rows_total = batchC * m;
+  hipLaunchKernelGGL(bdot_kernel, dim3((unsigned)((rows_total + 3) / 4)), dim3(256), 0, st, A, B, C,
+                     (long long)batchA, (long long)batchB, rows_total, (int)m, (int)n, (int)k,
+                     transA ? 1 : 0, transB ? 1 : 0, scalar);
+  MH_HIP(hipGetLastError());
+  return MARIAN_HIP_OK;
+}
+
+}  // extern "C"

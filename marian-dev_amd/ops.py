@@ -1,0 +1,122 @@
+"""Host mirror of the float operators between the int8 GEMMs of a transformer decode step,
+running on the HIP library (include/marian_hip_ops.h).
+
+Mirrors, name for name:
+  reference src/graph/expression_operators.cpp:901-913   layerNorm(x, gamma, beta, eps = 1e-9)
+  reference src/graph/expression_operators.cpp           softmax(a), logsoftmax(a),
+                                                         transpose(a, {0, 2, 1, 3}),
+                                                         bdot_legacy(a, b, transA, transB, scalar)
+  reference src/models/transformer.h:145-170             SplitHeads, JoinHeads
+
+Tensors are torch float32 tensors on the GPU (device memory and streams only); every arithmetic
+step is a call into the C ABI.  There is no CPU fallback.
+"""
+import torch
+
+from . import _lib
+from .integer import _abort_if, _backend_of
+
+
+def _f32c(x, what):
+    _abort_if(x.dtype != torch.float32, "{} expects float32, got {}", what, x.dtype)
+    return x.contiguous()
+
+
+def layerNorm(x, gamma, beta=None, eps=1e-9, add=None):
+    """reference src/graph/expression_operators.cpp:901-913; `add` fuses the skip connection in
+    front of it (out = layerNorm(x + add))."""
+    x = _f32c(x, "layerNorm")
+    be = _backend_of(x)
+    cols = x.shape[-1]
+    rows = x.numel() // cols if x.numel() else 0
+    gamma = _f32c(gamma, "layerNorm").reshape(-1)
+    _abort_if(gamma.numel() not in (1, cols), "layerNorm: gamma must have {} or 1 values", cols)
+    if beta is not None:
+        beta = _f32c(beta, "layerNorm").reshape(-1)
+        _abort_if(beta.numel() not in (1, cols), "layerNorm: beta must have {} or 1 values", cols)
+    if add is not None:
+        add = _f32c(add, "layerNorm")
+        _abort_if(tuple(add.shape) != tuple(x.shape), "layerNorm: skip input shape {} vs {}", tuple(add.shape), tuple(x.shape))
+    out = torch.empty_like(x)
+    st = be.lib.marian_hip_layer_norm(
+        x.data_ptr(), None if add is None else add.data_ptr(), gamma.data_ptr(), gamma.numel(),
+        None if beta is None else beta.data_ptr(), 0 if beta is None else beta.numel(),
+        out.data_ptr(), rows, cols, eps, be.stream())
+    _lib.check(st, "layerNorm")
+    return out
+
+
+def softmax(a, mask=None, rowsPerMask=1):
+    """softmax over the last axis; `mask` [n, cols] fuses the `a + mask` in front of it, row r of
+    `a` taking mask row (r / rowsPerMask) % n (reference src/models/transformer.h:264,772-774)."""
+    a = _f32c(a, "softmax")
+    be = _backend_of(a)
+    cols = a.shape[-1]
+    rows = a.numel() // cols if a.numel() else 0
+    n_masks = 0
+    if mask is not None:
+        mask = _f32c(mask, "softmax").reshape(-1, cols)
+        n_masks = mask.shape[0]
+    out = torch.empty_like(a)
+    st = be.lib.marian_hip_softmax(a.data_ptr(), None if mask is None else mask.data_ptr(), n_masks,
+                                   rowsPerMask, out.data_ptr(), rows, cols, be.stream())
+    _lib.check(st, "softmax")
+    return out
+
+
+def logsoftmax(a):
+    a = _f32c(a, "logsoftmax")
+    be = _backend_of(a)
+    cols = a.shape[-1]
+    rows = a.numel() // cols if a.numel() else 0
+    out = torch.empty_like(a)
+    _lib.check(be.lib.marian_hip_logsoftmax(a.data_ptr(), out.data_ptr(), rows, cols, be.stream()),
+               "logsoftmax")
+    return out
+
+
+def transpose0213(a):
+    """transpose(a, {0, 2, 1, 3}) of a 4-d tensor"""
+    a = _f32c(a, "transpose")
+    _abort_if(a.dim() != 4, "transpose0213 expects a 4-d tensor, got {} dimensions", a.dim())
+    be = _backend_of(a)
+    d0, d1, d2, d3 = a.shape
+    out = torch.empty((d0, d2, d1, d3), dtype=torch.float32, device=a.device)
+    _lib.check(be.lib.marian_hip_transpose0213(a.data_ptr(), out.data_ptr(), d0, d1, d2, d3, be.stream()),
+               "transpose")
+    return out
+
+
+def SplitHeads(input, dimHeads):
+    """reference src/models/transformer.h:145-156: [beam, batch, steps, model] ->
+    [batch * beam, heads, steps, depth]"""
+    dimBeam, dimBatch, dimSteps, dimModel = input.shape
+    return transpose0213(input.reshape(dimBatch * dimBeam, dimSteps, dimHeads, dimModel // dimHeads))
+
+
+def JoinHeads(input, dimBeam=1):
+    """reference src/models/transformer.h:158-170"""
+    dimBatchBeam, dimHeads, dimSteps, dimDepth = input.shape
+    out = transpose0213(input)
+    return out.reshape(dimBeam, dimBatchBeam // dimBeam, dimSteps, dimHeads * dimDepth)
+
+
+def bdot_legacy(a, b, transA=False, transB=False, scalar=1.0):
+    """reference src/tensors/cpu/prod.cpp:233-330: batch entry i uses a[i % batchA], b[i % batchB]"""
+    a, b = _f32c(a, "bdot"), _f32c(b, "bdot")
+    be = _backend_of(a)
+    batchA = a.numel() // (a.shape[-1] * a.shape[-2])
+    batchB = b.numel() // (b.shape[-1] * b.shape[-2])
+    m, k = a.shape[-2], a.shape[-1]
+    if transA:
+        m, k = k, m
+    l, n = b.shape[-2], b.shape[-1]
+    if transB:
+        l, n = n, l
+    _abort_if(l != k, "Matrix product requires inner dimensions to match: {} vs {}", k, l)
+    lead = tuple(a.shape[:-2]) if batchA >= batchB else tuple(b.shape[:-2])
+    out = torch.empty(lead + (m, n), dtype=torch.float32, device=a.device)
+    st = be.lib.marian_hip_bdot_legacy(a.data_ptr(), b.data_ptr(), out.data_ptr(), batchA, batchB,
+                                       m, n, k, int(transA), int(transB), scalar, be.stream())
+    _lib.check(st, "bdot")
+    return out

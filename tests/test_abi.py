@@ -8,20 +8,25 @@ import pytest
 
 from conftest import ROOT, load
 
-HEADER = os.path.join(ROOT, "include", "marian_hip_int8.h")
+HEADERS = [os.path.join(ROOT, "include", h) for h in ("marian_hip_int8.h", "marian_hip_ops.h")]
 
 
 def declared_functions():
-    text = open(HEADER).read()
-    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(marian_hip_\w+)\s*\(", text)))
+    names = set()
+    for header in HEADERS:
+        text = open(header).read()
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        names |= set(re.findall(r"\b(marian_hip_\w+)\s*\(", text))
+    return sorted(names)
 
 
 def test_header_declares_expected_entry_points():
     names = declared_functions()
     for must in ("marian_hip_int8_prepare_a", "marian_hip_int8_prepare_b",
                  "marian_hip_int8_prepare_b_quantized_transposed", "marian_hip_int8_affine",
-                 "marian_hip_int8_affine_shortlist", "marian_hip_int8_multiply_i32"):
+                 "marian_hip_int8_affine_shortlist", "marian_hip_int8_multiply_i32",
+                 "marian_hip_layer_norm", "marian_hip_softmax", "marian_hip_logsoftmax",
+                 "marian_hip_transpose0213", "marian_hip_bdot_legacy"):
         assert must in names
 
 
@@ -58,6 +63,18 @@ def test_argument_validation_returns_codes_not_aborts():
     assert lib.marian_hip_int8_affine(buf, buf, None, buf, 0, 64, 8, 1.0, 0, None) == L.OK  # empty batch
     assert lib.marian_hip_int8_affine_shortlist(buf, buf, None, None, 8, buf, 1, 64, 8, 1.0, 0, None) == L.ERR_NULL
     assert lib.marian_hip_int8_affine(None, None, None, None, 0, 64, 8, 1.0, 0, None) == L.OK
+    # float operators of include/marian_hip_ops.h
+    assert lib.marian_hip_layer_norm(buf, None, buf, 8, None, 0, buf, 2, 0, 1e-9, None) == L.ERR_SHAPE
+    assert lib.marian_hip_layer_norm(buf, None, buf, 7, None, 0, buf, 2, 8, 1e-9, None) == L.ERR_SHAPE
+    assert lib.marian_hip_layer_norm(None, None, buf, 8, None, 0, buf, 2, 8, 1e-9, None) == L.ERR_NULL
+    assert lib.marian_hip_layer_norm(buf, None, buf, 8, None, 0, buf, 0, 8, 1e-9, None) == L.OK
+    assert lib.marian_hip_softmax(buf, buf, 0, 1, buf, 2, 8, None) == L.ERR_SHAPE
+    assert lib.marian_hip_softmax(buf + 2, None, 0, 0, buf, 2, 8, None) == L.ERR_ALIGN
+    assert lib.marian_hip_logsoftmax(buf, None, 2, 8, None) == L.ERR_NULL
+    assert lib.marian_hip_transpose0213(buf, buf, 1, 2, 3, 4, None) == L.ERR_SHAPE   # aliasing
+    assert lib.marian_hip_transpose0213(buf, buf + 64, 0, 2, 3, 4, None) == L.OK
+    assert lib.marian_hip_bdot_legacy(buf, buf, buf, 2, 2, 0, 4, 4, 0, 0, 1.0, None) == L.ERR_SHAPE
+    assert lib.marian_hip_bdot_legacy(buf, None, buf, 2, 2, 1, 4, 4, 0, 0, 1.0, None) == L.ERR_NULL
     assert lib.marian_hip_int8_affine_shortlist(buf, buf, None, buf, 12, buf, 1, 64, 8, 1.0, 0, None) == L.ERR_SHAPE
     assert lib.marian_hip_int8_prepare_a(buf, buf, 4, 100, buf, 4096, None) == L.ERR_SHAPE
     assert lib.marian_hip_int8_prepare_a(buf, buf, 4096, 1024, buf, 16, None) == L.ERR_WORKSPACE

@@ -1,0 +1,163 @@
+"""GPU parity of the float operators of include/marian_hip_ops.h (through the C ABI, via the host
+mirror marian-dev_amd/ops.py) against the CPU checker and against float64 closed forms.
+
+Bar: 1e-5 relative plus a small absolute floor.  These are floating-point reductions whose
+summation order differs between the reference's own builds (SIMD width, fast-math), the checker
+(sequential) and the kernels (wave trees); the kernels are held to the float64 value within the
+bar, and to the checker within the bar widened by the checker's own sequential-sum error on long
+rows."""
+import numpy as np
+import pytest
+
+from conftest import load
+
+pytestmark = pytest.mark.gpu
+f64 = np.float64
+REL = 1e-5
+
+
+@pytest.fixture(scope="module")
+def ops(integer):
+    return load("ops")
+
+
+@pytest.fixture(scope="module")
+def chk():
+    from oracle import decode_ops
+    decode_ops.lib()
+    return decode_ops
+
+
+def dev(x):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(x)).cuda()
+
+
+def close(got, want, rel=REL, floor=1e-6):
+    got, want = np.asarray(got, f64), np.asarray(want, f64)
+    err = np.abs(got - want)
+    ok = err <= rel * np.abs(want) + floor
+    assert ok.all(), "max err %g (rel %g) at %s" % (err.max(), (err / (np.abs(want) + floor)).max(),
+                                                    np.argwhere(~ok)[:3].tolist())
+
+
+@pytest.mark.parametrize("rows,cols", [(1, 8), (5, 64), (128, 1024), (3, 1000), (7, 4096), (2, 5000),
+                                       (4, 1023)])
+@pytest.mark.parametrize("with_add,with_beta", [(False, True), (True, True), (True, False)])
+def test_layer_norm(ops, chk, synth, rows, cols, with_add, with_beta):
+    x = synth.normal(rows * 7 + cols, 0, (rows, cols), 2.0) + np.float32(0.3)
+    add = synth.normal(rows * 7 + cols, 1, (rows, cols), 1.0) if with_add else None
+    g = synth.normal(cols, 2, (cols,), 0.2) + np.float32(1.0)
+    b = synth.normal(cols, 3, (cols,), 0.5) if with_beta else None
+    for eps in (1e-9, 1e-6):
+        got = ops.layerNorm(dev(x), dev(g), None if b is None else dev(b), eps,
+                            None if add is None else dev(add)).cpu().numpy()
+        xs = (x if add is None else x + add).astype(f64)
+        mean = xs.mean(-1, keepdims=True)
+        var = ((xs - mean) ** 2).mean(-1, keepdims=True)
+        want = g.astype(f64) * (xs - mean) / np.sqrt(var + eps) + (0 if b is None else b.astype(f64))
+        close(got, want, REL, 2e-6)
+        close(got, chk.layer_norm(x, g, b, eps, add=add), 2 * REL, 4e-6)
+    # a single broadcast gamma/beta value (reference alphaStride/betaStride = 0)
+    got = ops.layerNorm(dev(x), dev(np.array([2.0], np.float32)), dev(np.array([-1.0], np.float32)), 1e-9).cpu().numpy()
+    close(got, chk.layer_norm(x, np.array([2.0], np.float32), np.array([-1.0], np.float32), 1e-9), 2 * REL, 4e-6)
+
+
+def test_layer_norm_4d_and_inplace_shapes(ops, chk, synth):
+    x = synth.normal(11, 0, (4, 32, 1, 1024), 1.0)
+    g = synth.normal(11, 2, (1, 1024), 0.1) + np.float32(1.0)
+    b = synth.normal(11, 3, (1, 1024), 0.1)
+    got = ops.layerNorm(dev(x), dev(g), dev(b), 1e-6, dev(x)).cpu().numpy()
+    assert got.shape == x.shape
+    close(got, chk.layer_norm(x, g, b, 1e-6, add=x), 2 * REL, 4e-6)
+
+
+@pytest.mark.parametrize("rows,cols", [(1, 1), (7, 5), (2048, 40), (4096, 64), (33, 2048), (5, 2049),
+                                       (128, 32000)])
+def test_softmax_and_logsoftmax(ops, chk, synth, rows, cols):
+    x = synth.normal(rows + cols, 0, (rows, cols), 3.0)
+    xs = x.astype(f64)
+    e = np.exp(xs - xs.max(-1, keepdims=True))
+    want = e / e.sum(-1, keepdims=True)
+    got = ops.softmax(dev(x)).cpu().numpy()
+    close(got, want, REL, 1e-10)
+    assert np.allclose(got.astype(f64).sum(-1), 1.0, atol=1e-5)
+    lwant = xs - xs.max(-1, keepdims=True) - np.log(e.sum(-1, keepdims=True))
+    lgot = ops.logsoftmax(dev(x)).cpu().numpy()
+    close(lgot, lwant, REL, 1e-5)
+    if rows * cols <= 1 << 20:   # against the checker, widened by its sequential-sum error
+        wide = REL * max(1.0, cols / 250.0)
+        close(got, chk.softmax(x), wide, 1e-10)
+        close(lgot, chk.logsoftmax(x), wide, 1e-5 * max(1.0, cols / 250.0))
+
+
+def test_softmax_with_attention_mask(ops, chk, synth):
+    """scores [beam*batch, heads, 1, len] + log-mask [batch, 1, 1, len] repeated over the beam"""
+    beam, batch, heads, L = 4, 8, 16, 37
+    z = synth.normal(21, 0, (beam * batch, heads, 1, L), 1.0)
+    lens = 1 + (np.arange(batch) * 5) % L
+    keep = (np.arange(L)[None, :] < lens[:, None])
+    mask = ((1 - keep) * -99999999.0).astype(np.float32)
+    got = ops.softmax(dev(z), dev(mask), rowsPerMask=heads).cpu().numpy()
+    close(got, chk.softmax(z, mask, rows_per_mask=heads), REL, 1e-10)
+    g4 = got.reshape(beam, batch, heads, L)
+    for bi in range(batch):
+        assert np.all(g4[:, bi, :, lens[bi]:] == 0) and np.allclose(g4[:, bi].sum(-1), 1.0, atol=1e-5)
+
+
+@pytest.mark.parametrize("shape", [(3, 5, 7, 4), (128, 1, 16, 64), (128, 16, 1, 64), (32, 40, 16, 64),
+                                   (2, 3, 4, 5), (1, 2, 2, 1)])
+def test_transpose0213(ops, chk, synth, shape):
+    x = synth.normal(sum(shape), 0, shape, 1.0)
+    y = ops.transpose0213(dev(x))
+    assert np.array_equal(y.cpu().numpy(), chk.transpose0213(x))
+    assert np.array_equal(ops.transpose0213(y).cpu().numpy(), x)
+
+
+def test_split_and_join_heads(ops, synth):
+    beam, batch, steps, heads, depth = 4, 8, 1, 16, 64
+    x = synth.normal(31, 0, (beam, batch, steps, heads * depth), 1.0)
+    q = ops.SplitHeads(dev(x), heads)
+    assert tuple(q.shape) == (beam * batch, heads, steps, depth)
+    want = x.reshape(beam * batch, steps, heads, depth).transpose(0, 2, 1, 3)
+    assert np.array_equal(q.cpu().numpy(), want)
+    assert np.array_equal(ops.JoinHeads(q, beam).cpu().numpy(), x)
+
+
+@pytest.mark.parametrize("tA,tB", [(False, False), (False, True), (True, False), (True, True)])
+@pytest.mark.parametrize("batch,m,n,k", [(6, 3, 5, 8), (2048, 1, 40, 64), (2048, 1, 64, 40), (8, 33, 70, 65)])
+def test_bdot_legacy(ops, chk, synth, tA, tB, batch, m, n, k):
+    a = synth.normal(batch + m, 0, (batch, k, m) if tA else (batch, m, k), 1.0)
+    b = synth.normal(batch + n, 1, (batch, n, k) if tB else (batch, k, n), 1.0)
+    got = ops.bdot_legacy(dev(a), dev(b), tA, tB, 0.125).cpu().numpy()
+    A = a.transpose(0, 2, 1) if tA else a
+    B = b.transpose(0, 2, 1) if tB else b
+    want = 0.125 * np.matmul(A.astype(f64), B.astype(f64))
+    floor = 2e-6 * np.sqrt(k)   # cancellation in sums of k products of unit-variance values
+    close(got, want, REL, floor)
+    if batch * m * n * k <= 1 << 22:
+        close(got, chk.bdot_legacy(a, b, tA, tB, 0.125), REL, 2 * floor)
+    # batch broadcast i % batchB
+    b2 = np.ascontiguousarray(b[:2])
+    got2 = ops.bdot_legacy(dev(a), dev(b2), tA, tB, 1.0).cpu().numpy()
+    B2 = b2.transpose(0, 2, 1) if tB else b2
+    want2 = np.stack([A[i].astype(f64) @ B2[i % 2].astype(f64) for i in range(batch)])
+    close(got2, want2, REL, 8 * floor)
+
+
+def test_attention_products_of_a_decode_step(ops, chk, synth):
+    """q [B*H, 1, dk] . k^T [B*H, len, dk] * 1/sqrt(dk), softmax, . v [B*H, len, dk]
+    (reference src/models/transformer.h:258-277) against the checker, op by op."""
+    BH, L, dk = 128 * 16, 40, 64
+    q = synth.normal(41, 0, (BH, 1, dk), 1.0)
+    k = synth.normal(41, 1, (BH, L, dk), 1.0)
+    v = synth.normal(41, 2, (BH, L, dk), 1.0)
+    z = ops.bdot_legacy(dev(q), dev(k), False, True, 1.0 / np.sqrt(dk))
+    w = ops.softmax(z)
+    o = ops.bdot_legacy(w, dev(v))
+    zc = chk.bdot_legacy(q, k, False, True, 1.0 / np.sqrt(dk))
+    wc = chk.softmax(zc)
+    oc = chk.bdot_legacy(wc, v)
+    close(z.cpu().numpy(), zc, REL, 1e-5)
+    close(w.cpu().numpy(), wc, 4 * REL, 1e-8)
+    close(o.cpu().numpy(), oc, 4 * REL, 1e-5)

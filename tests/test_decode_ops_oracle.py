@@ -1,0 +1,119 @@
+"""Pins the CPU checker of the decode-step float operators (oracle/decode_ops_oracle.c) against
+float64 closed forms and against invariants that a dropped term, a wrong sign or a wrong index
+would break.  No GPU."""
+import numpy as np
+import pytest
+
+f64 = np.float64
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from oracle import decode_ops
+    decode_ops.lib()
+    return decode_ops
+
+
+def close(a, b, rel=2e-6, floor=2e-6):
+    a, b = np.asarray(a, f64), np.asarray(b, f64)
+    return np.all(np.abs(a - b) <= rel * np.abs(b) + floor)
+
+
+@pytest.mark.parametrize("rows,cols", [(1, 8), (5, 64), (128, 1024), (3, 1000)])
+def test_layer_norm_closed_form(ops, rows, cols):
+    rng = np.random.default_rng(rows * cols)
+    x = rng.normal(0.3, 2.0, (rows, cols)).astype(np.float32)
+    g = rng.normal(1.0, 0.2, cols).astype(np.float32)
+    b = rng.normal(0.0, 0.5, cols).astype(np.float32)
+    add = rng.normal(0, 1, (rows, cols)).astype(np.float32)
+    for eps in (1e-9, 1e-6, 1e-3):
+        for a in (None, add):
+            xs = x.astype(f64) if a is None else (x + a).astype(f64)   # the skip add is an fp32 add
+            mean = xs.mean(-1, keepdims=True)
+            var = ((xs - mean) ** 2).mean(-1, keepdims=True)
+            want = g.astype(f64) * (xs - mean) / np.sqrt(var + eps) + b.astype(f64)
+            assert close(ops.layer_norm(x, g, b, eps, add=a), want, 5e-6, 5e-6)
+    # no beta; broadcast gamma (a single value)
+    xs = x.astype(f64)
+    mean = xs.mean(-1, keepdims=True)
+    var = ((xs - mean) ** 2).mean(-1, keepdims=True)
+    assert close(ops.layer_norm(x, np.array([2.0], np.float32), None, 1e-9),
+                 2.0 * (xs - mean) / np.sqrt(var + 1e-9), 5e-6, 5e-6)
+
+
+def test_layer_norm_invariants(ops):
+    rng = np.random.default_rng(1)
+    x = rng.normal(5.0, 3.0, (16, 512)).astype(np.float32)
+    y = ops.layer_norm(x, np.full(512, 3.0, np.float32), np.full(512, -1.0, np.float32), 1e-9)
+    assert np.allclose(y.mean(-1), -1.0, atol=1e-4) and np.allclose(y.std(-1), 3.0, atol=1e-3)
+    # shift of the input leaves the output unchanged (a wrong mean term would not)
+    y2 = ops.layer_norm(x + np.float32(8.0), np.full(512, 3.0, np.float32), np.full(512, -1.0, np.float32), 1e-9)
+    assert np.allclose(y, y2, atol=2e-5)
+
+
+@pytest.mark.parametrize("rows,cols", [(1, 1), (7, 5), (64, 40), (4, 32000)])
+def test_softmax_and_logsoftmax(ops, rows, cols):
+    rng = np.random.default_rng(rows + cols)
+    x = rng.normal(0, 3.0, (rows, cols)).astype(np.float32)
+    xs = x.astype(f64)
+    e = np.exp(xs - xs.max(-1, keepdims=True))
+    want = e / e.sum(-1, keepdims=True)
+    # the checker sums sequentially in float like the reference loop: its error grows with cols
+    rel = 5e-6 * max(1.0, cols / 500.0)
+    got = ops.softmax(x)
+    assert close(got, want, rel, 1e-9)
+    assert np.allclose(got.astype(f64).sum(-1), 1.0, atol=2 * rel)
+    assert close(ops.softmax(x + np.float32(11.0)), want, 4 * rel, 1e-9)      # shift invariance
+    lwant = xs - xs.max(-1, keepdims=True) - np.log(e.sum(-1, keepdims=True))
+    assert close(ops.logsoftmax(x), lwant, rel, 5e-6 * max(1.0, cols / 500.0))
+    assert close(np.exp(ops.logsoftmax(x).astype(f64)), want, 4 * rel, 1e-9)
+
+
+def test_softmax_mask_rows(ops):
+    """mask row = (row / rows_per_mask) % n_masks: scores [beam*batch, heads, 1, len] against a
+    [batch, 1, 1, len] mask repeated over the beam."""
+    beam, batch, heads, L = 2, 3, 4, 9
+    rng = np.random.default_rng(3)
+    z = rng.normal(0, 1, (beam * batch, heads, 1, L)).astype(np.float32)
+    keep = (rng.random((batch, L)) > 0.3)
+    keep[:, 0] = True
+    mask = ((1 - keep) * -99999999.0).astype(np.float32)
+    got = ops.softmax(z, mask, rows_per_mask=heads)
+    zz = z.astype(f64) + np.tile(mask.astype(np.float32), (beam, 1))[:, None, None, :]
+    e = np.exp(zz - zz.max(-1, keepdims=True))
+    want = e / e.sum(-1, keepdims=True)
+    assert close(got, want, 5e-6, 1e-9)
+    assert np.all(got.reshape(beam, batch, heads, L).transpose(1, 3, 0, 2)[~keep] == 0)
+
+
+def test_transpose0213(ops):
+    rng = np.random.default_rng(4)
+    x = rng.normal(0, 1, (3, 5, 7, 4)).astype(np.float32)
+    y = ops.transpose0213(x)
+    assert np.array_equal(y, x.transpose(0, 2, 1, 3))
+    assert np.array_equal(ops.transpose0213(y), x)
+    # split heads then join heads (reference src/models/transformer.h:145-170) is the identity
+    q = rng.normal(0, 1, (6, 1, 8, 16)).astype(np.float32)
+    assert np.array_equal(ops.transpose0213(ops.transpose0213(q)), q)
+
+
+@pytest.mark.parametrize("tA,tB", [(False, False), (False, True), (True, False), (True, True)])
+def test_bdot_legacy(ops, tA, tB):
+    rng = np.random.default_rng(5 + tA + 2 * tB)
+    batch, m, n, k = 6, 3, 5, 8
+    a = rng.normal(0, 1, (batch, k, m) if tA else (batch, m, k)).astype(np.float32)
+    b = rng.normal(0, 1, (batch, n, k) if tB else (batch, k, n)).astype(np.float32)
+    A = a.transpose(0, 2, 1) if tA else a
+    B = b.transpose(0, 2, 1) if tB else b
+    want = 0.125 * np.matmul(A.astype(f64), B.astype(f64))
+    assert close(ops.bdot_legacy(a, b, tA, tB, 0.125), want, 1e-5, 1e-6)
+    # batch broadcast: B has two batch entries, used as i % 2
+    b2 = b[:2]
+    B2 = b2.transpose(0, 2, 1) if tB else b2
+    want2 = np.stack([A[i].astype(f64) @ B2[i % 2].astype(f64) for i in range(batch)])
+    assert close(ops.bdot_legacy(a, b2, tA, tB, 1.0), want2, 1e-5, 1e-6)
+    # a single A against all B
+    a1 = a[:1]
+    A1 = a1.transpose(0, 2, 1) if tA else a1
+    want3 = np.stack([A1[0].astype(f64) @ B[i].astype(f64) for i in range(batch)])
+    assert close(ops.bdot_legacy(a1, b, tA, tB, 1.0), want3, 1e-5, 1e-6)
