@@ -68,6 +68,20 @@ int marian_hip_bdot_legacy(const float* A, const float* B, float* C, int64_t bat
                            int64_t batchB, int64_t m, int64_t n, int64_t k, int transA,
                            int transB, float scalar, void* stream);
 
+/*
+ * The attention of one decoding step in one launch: the nodes bdot_legacy(q, k, false, true,
+ * scale), `+ mask`, softmax and bdot_legacy(weights, v) of Attention(), reference
+ * src/models/transformer.h:241-280.  The arithmetic is that of the three separate entry points
+ * above, operation for operation, so the result equals theirs bit for bit.
+ *   q: [batchQ, m, dk], k and v: [batchKV, len, dk] (entry i uses k, v of i % batchKV: encoder
+ *   keys shared by the beam), out: [batchQ, m, dk]; mask as in marian_hip_softmax for score rows
+ *   [batchQ * m, len], or NULL.  len <= 4096.
+ */
+int marian_hip_attention(const float* q, const float* k, const float* v, const float* mask,
+                         int64_t n_masks, int64_t rows_per_mask, float* out, int64_t batchQ,
+                         int64_t batchKV, int64_t m, int64_t len, int64_t dk, float scale,
+                         void* stream);
+
 #ifdef __cplusplus
 }
 #endif

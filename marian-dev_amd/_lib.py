@@ -34,6 +34,8 @@ SIGNATURES = {
     "marian_hip_logsoftmax": (_i, [_vp, _vp, _i64, _i64, _vp]),
     "marian_hip_transpose0213": (_i, [_vp, _vp, _i64, _i64, _i64, _i64, _vp]),
     "marian_hip_bdot_legacy": (_i, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i, _i, _f, _vp]),
+    "marian_hip_attention": (_i, [_vp, _vp, _vp, _vp, _i64, _i64, _vp, _i64, _i64, _i64, _i64, _i64,
+                                  _f, _vp]),
 }
 
 _lib = None

@@ -220,6 +220,63 @@ __global__ __launch_bounds__(256) void bdot_kernel(const float* __restrict__ A, 
   }
 }
 
+// ---------------------------------------------------------------- one-launch attention
+// One wave per query row (entry i, row r): scores over the key positions (a lane per position,
+// the query row and a key row are walked with the same fused multiply-adds, in the same order,
+// as bdot_kernel walks them), softmax over them exactly as softmax_kernel<64> computes it, then
+// the weighted sum of the value rows (a lane per output column, positions in ascending order,
+// as bdot_kernel does).  The scores of a row live in LDS: `len` floats per wave.
+__global__ __launch_bounds__(256) void attention_kernel(const float* __restrict__ Q, const float* __restrict__ Kt,
+                                                        const float* __restrict__ V, const float* __restrict__ mask,
+                                                        long long n_masks, long long rows_per_mask,
+                                                        float* __restrict__ out, long long rows_total,
+                                                        long long batchKV, int m, int len, int dk,
+                                                        float scale) {
+  extern __shared__ float att_lds[];
+  const long long wr = (long long)blockIdx.x * 4 + threadIdx.x / 64;
+  if(wr >= rows_total) return;   // whole waves leave; no workgroup barrier is used
+  float* sc = att_lds + (threadIdx.x / 64) * len;
+  const int lane = threadIdx.x % 64;
+  const long long i = wr / m;
+  const float* q = Q + (size_t)wr * dk;
+  const float* kb = Kt + (size_t)(i % batchKV) * len * dk;
+  const float* vb = V + (size_t)(i % batchKV) * len * dk;
+  const float* mk = mask ? mask + (size_t)((wr / rows_per_mask) % n_masks) * len : nullptr;
+  const bool vec = (dk % 4) == 0 && ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(kb)) % 16) == 0;
+  float mx = -__builtin_inff();
+  for(int pos = lane; pos < len; pos += 64) {
+    float s = 0.0f;
+    if(vec) {
+      const v4f* ar = reinterpret_cast<const v4f*>(q);
+      const v4f* br = reinterpret_cast<const v4f*>(kb + (size_t)pos * dk);
+      for(int p = 0; p < dk / 4; ++p) {
+        const v4f av = ar[p], bv = br[p];
+        s = fmaf(av.x, bv.x, s);
+        s = fmaf(av.y, bv.y, s);
+        s = fmaf(av.z, bv.z, s);
+        s = fmaf(av.w, bv.w, s);
+      }
+    } else {
+      for(int p = 0; p < dk; ++p) s = fmaf(q[p], kb[(size_t)pos * dk + p], s);
+    }
+    float z = scale * s;
+    if(mk) z = z + mk[pos];
+    sc[pos] = z;
+    mx = z > mx ? z : mx;
+  }
+  mx = wave_maxf(mx);
+  float sum = 0.0f;
+  for(int pos = lane; pos < len; pos += 64) sum += expf(sc[pos] - mx);
+  sum = wave_sum(sum);
+  for(int pos = lane; pos < len; pos += 64) sc[pos] = expf(sc[pos] - mx) / sum;
+  // (a wave's LDS writes are visible to its own later reads: same wave, program order)
+  for(int d = lane; d < dk; d += 64) {
+    float o = 0.0f;
+    for(int pos = 0; pos < len; ++pos) o = fmaf(sc[pos], vb[(size_t)pos * dk + d], o);
+    out[(size_t)wr * dk + d] = 1.0f * o;
+  }
+}
+
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) % 16) == 0; }
 inline bool aligned4(const void* p) { return (reinterpret_cast<uintptr_t>(p) % 4) == 0; }
 
@@ -322,6 +379,35 @@ int marian_hip_bdot_legacy(const float* A, const float* B, float* C, int64_t bat
   hipLaunchKernelGGL(bdot_kernel, dim3((unsigned)((rows_total + 3) / 4)), dim3(256), 0, st, A, B, C,
                      (long long)batchA, (long long)batchB, rows_total, (int)m, (int)n, (int)k,
                      transA ? 1 : 0, transB ? 1 : 0, scalar);
+  MH_HIP(hipGetLastError());
+  return MARIAN_HIP_OK;
+}
+
+int marian_hip_attention(const float* q, const float* k, const float* v, const float* mask,
+                         int64_t n_masks, int64_t rows_per_mask, float* out, int64_t batchQ,
+                         int64_t batchKV, int64_t m, int64_t len, int64_t dk, float scale,
+                         void* stream) {
+  if(batchQ < 0 || batchKV <= 0 || m <= 0 || len <= 0 || dk <= 0) return MARIAN_HIP_ERR_SHAPE;
+  if(mask && (n_masks <= 0 || rows_per_mask <= 0)) return MARIAN_HIP_ERR_SHAPE;
+  if(len > 4096) return MARIAN_HIP_ERR_RANGE;
+  if(batchQ == 0) return MARIAN_HIP_OK;
+  if(!q || !k || !v || !out) return MARIAN_HIP_ERR_NULL;
+  if(batchQ * m * dk > kMaxElemsOps || batchKV * len * dk > kMaxElemsOps) return MARIAN_HIP_ERR_RANGE;
+  if(!aligned4(q) || !aligned4(k) || !aligned4(v) || !aligned4(out) || (mask && !aligned4(mask)))
+    return MARIAN_HIP_ERR_ALIGN;
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  if(!mask) { n_masks = 1; rows_per_mask = 1; }
+  const long long rows_total = batchQ * m;
+  const size_t lds = (size_t)4 * (size_t)len * sizeof(float);
+  static const int lds_status = [] {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(attention_kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024);
+    return e == hipSuccess ? 0 : (int)e;
+  }();
+  if(lds_status != 0) return record_hip_error(lds_status);
+  hipLaunchKernelGGL(attention_kernel, dim3((unsigned)((rows_total + 3) / 4)), dim3(256), lds, st, q, k, v,
+                     mask, (long long)n_masks, (long long)rows_per_mask, out, rows_total,
+                     (long long)batchKV, (int)m, (int)len, (int)dk, scale);
   MH_HIP(hipGetLastError());
   return MARIAN_HIP_OK;
 }

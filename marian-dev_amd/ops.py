@@ -76,11 +76,15 @@ def logsoftmax(a):
 
 
 def transpose0213(a):
-    """transpose(a, {0, 2, 1, 3}) of a 4-d tensor"""
+    """transpose(a, {0, 2, 1, 3}) of a 4-d tensor.  With a middle dimension of 1 (the single
+    target position of a decoding step) the transposed tensor has the same memory image, so it
+    is returned as a view and no kernel runs."""
     a = _f32c(a, "transpose")
     _abort_if(a.dim() != 4, "transpose0213 expects a 4-d tensor, got {} dimensions", a.dim())
     be = _backend_of(a)
     d0, d1, d2, d3 = a.shape
+    if d1 == 1 or d2 == 1:
+        return a.reshape(d0, d2, d1, d3)
     out = torch.empty((d0, d2, d1, d3), dtype=torch.float32, device=a.device)
     _lib.check(be.lib.marian_hip_transpose0213(a.data_ptr(), out.data_ptr(), d0, d1, d2, d3, be.stream()),
                "transpose")
@@ -119,4 +123,28 @@ def bdot_legacy(a, b, transA=False, transB=False, scalar=1.0):
     st = be.lib.marian_hip_bdot_legacy(a.data_ptr(), b.data_ptr(), out.data_ptr(), batchA, batchB,
                                        m, n, k, int(transA), int(transB), scalar, be.stream())
     _lib.check(st, "bdot")
+    return out
+
+
+def Attention(q, k, v, mask=None, rowsPerMask=1):
+    """reference src/models/transformer.h:241-280 (inference: no dropout, weights not kept):
+    softmax(bdot_legacy(q, k, false, true, 1/sqrt(dk)) + mask) then bdot_legacy(weights, v), in
+    one launch.  q: [batch*beam, heads, tgt, dk]; k, v: [batch(*beam), heads, len, dk]."""
+    q, k, v = _f32c(q, "Attention"), _f32c(k, "Attention"), _f32c(v, "Attention")
+    be = _backend_of(q)
+    dk, m, L = q.shape[-1], q.shape[-2], k.shape[-2]
+    _abort_if(k.shape[-1] != dk or tuple(v.shape) != tuple(k.shape), "Attention: key/value shapes {} {} vs dk {}",
+              tuple(k.shape), tuple(v.shape), dk)
+    batchQ = q.numel() // (m * dk)
+    batchKV = k.numel() // (L * dk)
+    n_masks = 0
+    if mask is not None:
+        mask = _f32c(mask, "Attention").reshape(-1, L)
+        n_masks = mask.shape[0]
+    out = torch.empty_like(q)
+    st = be.lib.marian_hip_attention(q.data_ptr(), k.data_ptr(), v.data_ptr(),
+                                     None if mask is None else mask.data_ptr(), n_masks, rowsPerMask,
+                                     out.data_ptr(), batchQ, batchKV, m, L, dk, 1.0 / float(dk) ** 0.5,
+                                     be.stream())
+    _lib.check(st, "Attention")
     return out

@@ -26,7 +26,7 @@ def test_header_declares_expected_entry_points():
                  "marian_hip_int8_prepare_b_quantized_transposed", "marian_hip_int8_affine",
                  "marian_hip_int8_affine_shortlist", "marian_hip_int8_multiply_i32",
                  "marian_hip_layer_norm", "marian_hip_softmax", "marian_hip_logsoftmax",
-                 "marian_hip_transpose0213", "marian_hip_bdot_legacy"):
+                 "marian_hip_transpose0213", "marian_hip_bdot_legacy", "marian_hip_attention"):
         assert must in names
 
 
@@ -75,6 +75,8 @@ def test_argument_validation_returns_codes_not_aborts():
     assert lib.marian_hip_transpose0213(buf, buf + 64, 0, 2, 3, 4, None) == L.OK
     assert lib.marian_hip_bdot_legacy(buf, buf, buf, 2, 2, 0, 4, 4, 0, 0, 1.0, None) == L.ERR_SHAPE
     assert lib.marian_hip_bdot_legacy(buf, None, buf, 2, 2, 1, 4, 4, 0, 0, 1.0, None) == L.ERR_NULL
+    assert lib.marian_hip_attention(buf, buf, buf, None, 0, 0, buf, 2, 2, 1, 5000, 64, 0.125, None) == L.ERR_RANGE
+    assert lib.marian_hip_attention(buf, buf, None, None, 0, 0, buf, 2, 2, 1, 40, 64, 0.125, None) == L.ERR_NULL
     assert lib.marian_hip_int8_affine_shortlist(buf, buf, None, buf, 12, buf, 1, 64, 8, 1.0, 0, None) == L.ERR_SHAPE
     assert lib.marian_hip_int8_prepare_a(buf, buf, 4, 100, buf, 4096, None) == L.ERR_SHAPE
     assert lib.marian_hip_int8_prepare_a(buf, buf, 4096, 1024, buf, 16, None) == L.ERR_WORKSPACE

@@ -161,3 +161,31 @@ def test_attention_products_of_a_decode_step(ops, chk, synth):
     close(z.cpu().numpy(), zc, REL, 1e-5)
     close(w.cpu().numpy(), wc, 4 * REL, 1e-8)
     close(o.cpu().numpy(), oc, 4 * REL, 1e-5)
+
+
+@pytest.mark.parametrize("BQ,BKV,m,L,dk,masked", [(2048, 2048, 1, 21, 64, False), (2048, 512, 1, 40, 64, True),
+                                                  (24, 24, 3, 130, 64, False), (8, 4, 2, 7, 20, True),
+                                                  (16, 16, 1, 1, 64, False)])
+def test_one_launch_attention_equals_the_three_operators(ops, chk, synth, BQ, BKV, m, L, dk, masked):
+    """marian_hip_attention against bdot_legacy + (mask) softmax + bdot_legacy of the same library:
+    bit for bit; and against the checker within the bar."""
+    heads = 4
+    q = synth.normal(BQ + L, 0, (BQ, m, dk), 1.0)
+    k = synth.normal(BQ + L, 1, (BKV, L, dk), 1.0)
+    v = synth.normal(BQ + L, 2, (BKV, L, dk), 1.0)
+    mask = None
+    rpm = 1
+    if masked:
+        n_masks = BKV // heads
+        lens = 1 + (np.arange(n_masks) * 3) % L
+        mask = ((np.arange(L)[None, :] >= lens[:, None]) * -99999999.0).astype(np.float32)
+        rpm = heads * m
+    scale = 1.0 / float(dk) ** 0.5
+    z = ops.bdot_legacy(dev(q), dev(k), False, True, scale)
+    w = ops.softmax(z, None if mask is None else dev(mask), rpm)
+    want = ops.bdot_legacy(w, dev(v)).cpu().numpy()
+    got = ops.Attention(dev(q), dev(k), dev(v), None if mask is None else dev(mask), rpm).cpu().numpy()
+    assert np.array_equal(got, want)
+    zc = chk.bdot_legacy(q, k, False, True, scale)
+    wc = chk.softmax(zc, mask, rows_per_mask=rpm)
+    close(got, chk.bdot_legacy(wc, v), 4 * REL, 2e-5)
