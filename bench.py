@@ -102,6 +102,92 @@ class Op:
             assert r == 0, r
 
 
+class BigDecoder:
+    """Transformer-big decoder (6 layers, d = 1024, ffn = 4096, 16 heads, tied 32000-word output
+    layer) with random-init weights, driven through the host mirrors of the library: one full
+    decoding step at beam 4 x batch 32 (reference src/models/transformer.h:603-760 for the layer
+    structure, post-processing "dan", inference).  Self-attention keys/values of `t_past` earlier
+    positions and encoder keys/values of `src_len` positions are resident; K/V projections are
+    taken for the new position only.  Beam search itself (top-k, hypothesis bookkeeping) is not
+    part of the step."""
+
+    def __init__(self, torch, integer, ops, sets, t_past=20, src_len=40, seed=300):
+        self.torch, self.integer, self.ops = torch, integer, ops
+        self.d, self.ffn, self.V, self.H = 1024, 4096, 32000, 16
+        self.beam, self.batch = 4, 32
+        self.M = self.beam * self.batch
+        self.T, self.L = t_past + 1, src_len
+        g = torch.Generator(device="cuda")
+        g.manual_seed(seed)
+        d, ffn, V, H, M = self.d, self.ffn, self.V, self.H, self.M
+
+        def qw(K, N):
+            return integer.prepareB(torch.randn(K, N, device="cuda", generator=g) * 0.02)
+
+        def vec(n, scale=0.01, shift=0.0):
+            return torch.randn(n, device="cuda", generator=g) * scale + shift
+
+        first = {"layers": [], "out": (qw(d, V), vec(V))}
+        for _ in range(6):
+            ly = {}
+            for name, (K, N) in {"Wq": (d, d), "Wk": (d, d), "Wv": (d, d), "Wo": (d, d), "cWq": (d, d),
+                                 "cWo": (d, d), "W1": (d, ffn), "W2": (ffn, d)}.items():
+                ly[name] = (qw(K, N), vec(N))
+            for name in ("ln1", "ln2", "ln3"):
+                ly[name] = (vec(d, 0.1, 1.0), vec(d, 0.1))
+            first["layers"].append(ly)
+
+        def clone(x):
+            if isinstance(x, dict):
+                return {k: clone(v) for k, v in x.items()}
+            if isinstance(x, (list, tuple)):
+                return type(x)(clone(v) for v in x)
+            if isinstance(x, integer.QTensor):
+                return integer.QTensor(x.data.clone(), x.shape, x.type)
+            return x   # small fp32 vectors are shared
+        self.sets = [first] + [clone(first) for _ in range(sets - 1)]
+        self.weight_bytes = 6 * (6 * d * d + 2 * d * ffn) + d * V
+        self.gemm_ops = 2 * M * self.weight_bytes
+        # resident state
+        self.x = torch.randn(M, d, device="cuda", generator=g)
+        self.Kself = [torch.randn(M * H, self.T, d // H, device="cuda", generator=g) for _ in range(6)]
+        self.Vself = [torch.randn(M * H, self.T, d // H, device="cuda", generator=g) for _ in range(6)]
+        self.Kenc = [torch.randn(self.batch * H, self.L, d // H, device="cuda", generator=g) for _ in range(6)]
+        self.Venc = [torch.randn(self.batch * H, self.L, d // H, device="cuda", generator=g) for _ in range(6)]
+        lens = torch.randint(20, self.L + 1, (self.batch,), device="cuda", generator=g)
+        self.mask = (torch.arange(self.L, device="cuda")[None, :] >= lens[:, None]).float() * -99999999.0
+
+    def step(self, s, gemm_only=False):
+        integer, ops = self.integer, self.ops
+        W = self.sets[s % len(self.sets)]
+        H, M, d = self.H, self.M, self.d
+        dk = d // H
+        x = self.x
+        for li, ly in enumerate(W["layers"]):
+            q, _ = integer.affine_f32(x, *ly["Wq"])
+            k, _ = integer.affine_f32(x, *ly["Wk"])
+            v, _ = integer.affine_f32(x, *ly["Wv"])
+            if gemm_only:
+                o = q
+            else:
+                # head split of a single position is a view; append the new key/value, attend
+                self.Kself[li][:, self.T - 1, :].copy_(k.view(M * H, dk))
+                self.Vself[li][:, self.T - 1, :].copy_(v.view(M * H, dk))
+                o = ops.Attention(q.view(M * H, 1, dk), self.Kself[li], self.Vself[li]).view(M, d)
+            a, _ = integer.affine_f32(o, *ly["Wo"])
+            x1 = a if gemm_only else ops.layerNorm(a, *ly["ln1"], eps=1e-6, add=x)
+            cq, _ = integer.affine_f32(x1, *ly["cWq"])
+            co = cq if gemm_only else ops.Attention(cq.view(M * H, 1, dk), self.Kenc[li], self.Venc[li],
+                                                    self.mask, rowsPerMask=H).view(M, d)
+            ca, _ = integer.affine_f32(co, *ly["cWo"])
+            x2 = ca if gemm_only else ops.layerNorm(ca, *ly["ln2"], eps=1e-6, add=x1)
+            f1, _ = integer.affine_f32(x2, *ly["W1"], relu=True)
+            f2, _ = integer.affine_f32(f1, *ly["W2"])
+            x = f2 if gemm_only else ops.layerNorm(f2, *ly["ln3"], eps=1e-6, add=x2)
+        logits, _ = integer.affine_f32(x, *W["out"])
+        return logits if gemm_only else ops.logsoftmax(logits)
+
+
 def capture(torch, fn):
     """Record fn's launches into a HIP graph (no memset nodes: the path has none)."""
     s = torch.cuda.Stream()
@@ -378,6 +464,25 @@ def main():
             "weight_sets": bsets}
         del bgraphs
         del ops_big
+
+        # the same step with everything between the GEMMs (N3 operators) through the host mirrors
+        ops_mod = importlib.import_module(PKG + ".ops")
+        dec = BigDecoder(torch, integer, ops_mod, bsets)
+        full = [capture(torch, (lambda c=c: dec.step(c))) for c in range(bsets)]
+        fdt = time_graphs(torch, full, n, max(4, args.warmup // 2))
+        gonly = [capture(torch, (lambda c=c: dec.step(c, gemm_only=True))) for c in range(bsets)]
+        gdt = time_graphs(torch, gonly, n, max(4, args.warmup // 2))
+        out["transformer_big_decode_full"] = {
+            "what": "full decoder step through the host mirrors: 49 int8 affine calls + per layer "
+                    "2 cache appends, 2 one-launch attentions (20 cached positions; 40 source "
+                    "positions with mask), 3 skip-add+layer-norm; log-softmax over 32000; no beam "
+                    "search bookkeeping",
+            "ms_per_step": round(fdt / n * 1e3, 4),
+            "hyp_tokens_per_s": round(dec.M * n / fdt, 1),
+            "output_tokens_per_s": round(dec.batch * n / fdt, 1),
+            "gemm_only_ms_per_step_same_harness": round(gdt / n * 1e3, 4),
+            "non_gemm_share": round(1.0 - gdt / fdt, 3)}
+        del full, gonly, dec
 
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline()

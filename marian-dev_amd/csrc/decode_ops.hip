@@ -160,6 +160,55 @@ __global__ __launch_bounds__(THREADS < 256 ? 256 : THREADS) void softmax_kernel(
   }
 }
 
+// Vocabulary-size rows (cols % 4 == 0, cols <= 32768, 16-byte aligned rows, no mask): 1024
+// threads per row keep the row in registers (eight float4 each), so it is read once.  Same
+// operations per element as softmax_kernel.
+template <bool LOG>
+__global__ __launch_bounds__(1024) void softmax_wide_kernel(const float* in, float* out, int cols) {
+  __shared__ float red[16];
+  const size_t row = blockIdx.x;
+  const v4f* x = reinterpret_cast<const v4f*>(in + row * cols);
+  v4f* y = reinterpret_cast<v4f*>(out + row * cols);
+  const int cols4 = cols / 4, t = threadIdx.x;
+  v4f v[8];
+  float mx = -__builtin_inff();
+#pragma unroll
+  for(int j = 0; j < 8; ++j) {
+    const int i = j * 1024 + t;
+    if(i < cols4) {
+      v[j] = x[i];
+      const float a = v[j].x > v[j].y ? v[j].x : v[j].y, b = v[j].z > v[j].w ? v[j].z : v[j].w;
+      const float c = a > b ? a : b;
+      mx = c > mx ? c : mx;
+    }
+  }
+  mx = row_reduce<1024, true>(mx, red);
+  float sum = 0.0f;
+#pragma unroll
+  for(int j = 0; j < 8; ++j) {
+    if(j * 1024 + t < cols4) {
+      if(LOG) {
+        v[j].x = v[j].x - mx; v[j].y = v[j].y - mx; v[j].z = v[j].z - mx; v[j].w = v[j].w - mx;
+        sum += (expf(v[j].x) + expf(v[j].y)) + (expf(v[j].z) + expf(v[j].w));
+      } else {
+        v[j].x = expf(v[j].x - mx); v[j].y = expf(v[j].y - mx);
+        v[j].z = expf(v[j].z - mx); v[j].w = expf(v[j].w - mx);
+        sum += (v[j].x + v[j].y) + (v[j].z + v[j].w);
+      }
+    }
+  }
+  sum = row_reduce<1024, false>(sum, red);
+  const float log_sum = logf(sum);
+#pragma unroll
+  for(int j = 0; j < 8; ++j) {
+    const int i = j * 1024 + t;
+    if(i < cols4) {
+      if(LOG) y[i] = v4f{v[j].x - log_sum, v[j].y - log_sum, v[j].z - log_sum, v[j].w - log_sum};
+      else y[i] = v4f{v[j].x / sum, v[j].y / sum, v[j].z / sum, v[j].w / sum};
+    }
+  }
+}
+
 // ---------------------------------------------------------------- transpose 0213
 // One element (VEC floats of the innermost dimension) per thread, indexed by the output.
 template <int VEC>
@@ -246,7 +295,21 @@ __global__ __launch_bounds__(256) void attention_kernel(const float* __restrict_
   float mx = -__builtin_inff();
   for(int pos = lane; pos < len; pos += 64) {
     float s = 0.0f;
-    if(vec) {
+    if(vec && dk == 64) {   // the usual head size: all sixteen loads of the key row in flight at once
+      const v4f* ar = reinterpret_cast<const v4f*>(q);
+      const v4f* br = reinterpret_cast<const v4f*>(kb + (size_t)pos * dk);
+      v4f kr[16];
+#pragma unroll
+      for(int p = 0; p < 16; ++p) kr[p] = br[p];
+#pragma unroll
+      for(int p = 0; p < 16; ++p) {
+        const v4f av = ar[p];
+        s = fmaf(av.x, kr[p].x, s);
+        s = fmaf(av.y, kr[p].y, s);
+        s = fmaf(av.z, kr[p].z, s);
+        s = fmaf(av.w, kr[p].w, s);
+      }
+    } else if(vec) {
       const v4f* ar = reinterpret_cast<const v4f*>(q);
       const v4f* br = reinterpret_cast<const v4f*>(kb + (size_t)pos * dk);
       for(int p = 0; p < dk / 4; ++p) {
@@ -272,7 +335,15 @@ __global__ __launch_bounds__(256) void attention_kernel(const float* __restrict_
   // (a wave's LDS writes are visible to its own later reads: same wave, program order)
   for(int d = lane; d < dk; d += 64) {
     float o = 0.0f;
-    for(int pos = 0; pos < len; ++pos) o = fmaf(sc[pos], vb[(size_t)pos * dk + d], o);
+    int pos = 0;
+    for(; pos + 8 <= len; pos += 8) {   // eight value loads in flight, same summation order
+      float vr[8];
+#pragma unroll
+      for(int u = 0; u < 8; ++u) vr[u] = vb[(size_t)(pos + u) * dk + d];
+#pragma unroll
+      for(int u = 0; u < 8; ++u) o = fmaf(sc[pos + u], vr[u], o);
+    }
+    for(; pos < len; ++pos) o = fmaf(sc[pos], vb[(size_t)pos * dk + d], o);
     out[(size_t)wr * dk + d] = 1.0f * o;
   }
 }
@@ -328,6 +399,9 @@ static int softmax_common(const float* in, const float* mask, int64_t n_masks, i
     const unsigned blocks = (unsigned)((rows + 3) / 4);
     if(log) hipLaunchKernelGGL((softmax_kernel<64, true>), dim3(blocks), dim3(256), 0, st, in, mask, (long long)n_masks, (long long)rows_per_mask, out, (long long)rows, (int)cols);
     else hipLaunchKernelGGL((softmax_kernel<64, false>), dim3(blocks), dim3(256), 0, st, in, mask, (long long)n_masks, (long long)rows_per_mask, out, (long long)rows, (int)cols);
+  } else if(!mask && cols % 4 == 0 && cols <= 32768 && aligned16(in) && aligned16(out)) {
+    if(log) hipLaunchKernelGGL(softmax_wide_kernel<true>, dim3((unsigned)rows), dim3(1024), 0, st, in, out, (int)cols);
+    else hipLaunchKernelGGL(softmax_wide_kernel<false>, dim3((unsigned)rows), dim3(1024), 0, st, in, out, (int)cols);
   } else {
     if(log) hipLaunchKernelGGL((softmax_kernel<1024, true>), dim3((unsigned)rows), dim3(1024), 0, st, in, mask, (long long)n_masks, (long long)rows_per_mask, out, (long long)rows, (int)cols);
     else hipLaunchKernelGGL((softmax_kernel<1024, false>), dim3((unsigned)rows), dim3(1024), 0, st, in, mask, (long long)n_masks, (long long)rows_per_mask, out, (long long)rows, (int)cols);

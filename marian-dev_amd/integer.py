@@ -42,7 +42,8 @@ class QTensor:
     @staticmethod
     def empty(shape, type_, device):
         nbytes = _align256(requiredBytes(shape, type_))
-        return QTensor(torch.zeros(nbytes, dtype=torch.int8, device=device), shape, type_)
+        # (the bytes past elements + 4 are allocation padding and are never read)
+        return QTensor(torch.empty(nbytes, dtype=torch.int8, device=device), shape, type_)
 
     @staticmethod
     def from_numpy(flat_int8, shape, type_, device):

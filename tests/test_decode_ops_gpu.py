@@ -73,7 +73,7 @@ def test_layer_norm_4d_and_inplace_shapes(ops, chk, synth):
 
 
 @pytest.mark.parametrize("rows,cols", [(1, 1), (7, 5), (2048, 40), (4096, 64), (33, 2048), (5, 2049),
-                                       (128, 32000)])
+                                       (128, 32000), (3, 32768), (2, 32772), (3, 8190), (4, 4100)])
 def test_softmax_and_logsoftmax(ops, chk, synth, rows, cols):
     x = synth.normal(rows + cols, 0, (rows, cols), 3.0)
     xs = x.astype(f64)
