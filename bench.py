@@ -157,34 +157,66 @@ class BigDecoder:
         lens = torch.randint(20, self.L + 1, (self.batch,), device="cuda", generator=g)
         self.mask = (torch.arange(self.L, device="cuda")[None, :] >= lens[:, None]).float() * -99999999.0
 
-    def step(self, s, gemm_only=False):
+    def step(self, s, gemm_only=False, chained=True):
+        """chained: every tensor that feeds an affine call leaves its abs-max where it is
+        produced (layer norm, attention, the ReLU GEMM), so those calls skip their abs-max pass."""
         integer, ops = self.integer, self.ops
         W = self.sets[s % len(self.sets)]
         H, M, d = self.H, self.M, self.d
         dk = d // H
-        x = self.x
+        x, xmax = self.x, None
+        ch = chained and not gemm_only
         for li, ly in enumerate(W["layers"]):
-            q, _ = integer.affine_f32(x, *ly["Wq"])
-            k, _ = integer.affine_f32(x, *ly["Wk"])
-            v, _ = integer.affine_f32(x, *ly["Wv"])
+            q, _ = integer.affine_f32(x, *ly["Wq"], absmax=xmax)
+            k, _ = integer.affine_f32(x, *ly["Wk"], absmax=xmax)
+            v, _ = integer.affine_f32(x, *ly["Wv"], absmax=xmax)
+            omax = x1max = comax = x2max = f1max = None
             if gemm_only:
                 o = q
             else:
                 # head split of a single position is a view; append the new key/value, attend
                 self.Kself[li][:, self.T - 1, :].copy_(k.view(M * H, dk))
                 self.Vself[li][:, self.T - 1, :].copy_(v.view(M * H, dk))
-                o = ops.Attention(q.view(M * H, 1, dk), self.Kself[li], self.Vself[li]).view(M, d)
-            a, _ = integer.affine_f32(o, *ly["Wo"])
-            x1 = a if gemm_only else ops.layerNorm(a, *ly["ln1"], eps=1e-6, add=x)
-            cq, _ = integer.affine_f32(x1, *ly["cWq"])
-            co = cq if gemm_only else ops.Attention(cq.view(M * H, 1, dk), self.Kenc[li], self.Venc[li],
-                                                    self.mask, rowsPerMask=H).view(M, d)
-            ca, _ = integer.affine_f32(co, *ly["cWo"])
-            x2 = ca if gemm_only else ops.layerNorm(ca, *ly["ln2"], eps=1e-6, add=x1)
-            f1, _ = integer.affine_f32(x2, *ly["W1"], relu=True)
-            f2, _ = integer.affine_f32(f1, *ly["W2"])
-            x = f2 if gemm_only else ops.layerNorm(f2, *ly["ln3"], eps=1e-6, add=x2)
-        logits, _ = integer.affine_f32(x, *W["out"])
+                o = ops.Attention(q.view(M * H, 1, dk), self.Kself[li], self.Vself[li], want_absmax=ch)
+                if ch:
+                    o, omax = o
+                o = o.view(M, d)
+            a, _ = integer.affine_f32(o, *ly["Wo"], absmax=omax)
+            if gemm_only:
+                x1 = a
+            else:
+                x1 = ops.layerNorm(a, *ly["ln1"], eps=1e-6, add=x, want_absmax=ch)
+                if ch:
+                    x1, x1max = x1
+            cq, _ = integer.affine_f32(x1, *ly["cWq"], absmax=x1max)
+            if gemm_only:
+                co = cq
+            else:
+                co = ops.Attention(cq.view(M * H, 1, dk), self.Kenc[li], self.Venc[li], self.mask,
+                                   rowsPerMask=H, want_absmax=ch)
+                if ch:
+                    co, comax = co
+                co = co.view(M, d)
+            ca, _ = integer.affine_f32(co, *ly["cWo"], absmax=comax)
+            if gemm_only:
+                x2 = ca
+            else:
+                x2 = ops.layerNorm(ca, *ly["ln2"], eps=1e-6, add=x1, want_absmax=ch)
+                if ch:
+                    x2, x2max = x2
+            f1 = integer.affine_f32(x2, *ly["W1"], relu=True, absmax=x2max, want_absmax=ch)
+            if ch:
+                f1, _, f1max = f1
+            else:
+                f1 = f1[0]
+            f2, _ = integer.affine_f32(f1, *ly["W2"], absmax=f1max)
+            if gemm_only:
+                x = f2
+            else:
+                x = ops.layerNorm(f2, *ly["ln3"], eps=1e-6, add=x2, want_absmax=ch)
+                if ch:
+                    x, xmax = x
+        logits, _ = integer.affine_f32(x, *W["out"], absmax=xmax)
         return logits if gemm_only else ops.logsoftmax(logits)
 
 
@@ -468,6 +500,11 @@ def main():
         # the same step with everything between the GEMMs (N3 operators) through the host mirrors
         ops_mod = importlib.import_module(PKG + ".ops")
         dec = BigDecoder(torch, integer, ops_mod, bsets)
+        # chained and unchained steps give the same bits
+        same = bool(torch.equal(dec.step(0, chained=True), dec.step(0, chained=False)))
+        unch = [capture(torch, (lambda c=c: dec.step(c, chained=False))) for c in range(bsets)]
+        udt = time_graphs(torch, unch, n, max(4, args.warmup // 2))
+        del unch
         full = [capture(torch, (lambda c=c: dec.step(c))) for c in range(bsets)]
         fdt = time_graphs(torch, full, n, max(4, args.warmup // 2))
         gonly = [capture(torch, (lambda c=c: dec.step(c, gemm_only=True))) for c in range(bsets)]
@@ -476,8 +513,11 @@ def main():
             "what": "full decoder step through the host mirrors: 49 int8 affine calls + per layer "
                     "2 cache appends, 2 one-launch attentions (20 cached positions; 40 source "
                     "positions with mask), 3 skip-add+layer-norm; log-softmax over 32000; no beam "
-                    "search bookkeeping",
+                    "search bookkeeping; the abs-max of every GEMM input is left by the kernel that "
+                    "produced it",
             "ms_per_step": round(fdt / n * 1e3, 4),
+            "ms_per_step_unchained": round(udt / n * 1e3, 4),
+            "chained_equals_unchained": same,
             "hyp_tokens_per_s": round(dec.M * n / fdt, 1),
             "output_tokens_per_s": round(dec.batch * n / fdt, 1),
             "gemm_only_ms_per_step_same_harness": round(gdt / n * 1e3, 4),

@@ -112,6 +112,25 @@ int marian_hip_int8_affine_f32(const float* A, int8_t* Aq, const int8_t* Bq, con
                                size_t workspace_bytes, void* stream);
 
 /*
+ * marian_hip_int8_affine_f32 with the activations' abs-max handed from the call that produced
+ * them to the call that consumes them.  The reference recomputes max|A| in every prepareA node
+ * (src/tensors/cpu/intgemm_interface.h:23); here the kernel that writes a tensor can leave values
+ * whose maximum is that abs-max, and the next call takes them instead of scanning the tensor
+ * again (one launch fewer per call in a decoder step).  Results are those of
+ * marian_hip_int8_affine_f32, bit for bit (a maximum is exact in any grouping).
+ *   absmax_in:  NULL, or MARIAN_HIP_ABSMAX_SLOTS floats whose maximum is max|A| - the absmax_out
+ *               of the call that wrote A (this one, marian_hip_layer_norm or marian_hip_attention).
+ *   absmax_out: NULL, or MARIAN_HIP_ABSMAX_SLOTS floats that receive values whose maximum is
+ *               max|out|.
+ */
+#define MARIAN_HIP_ABSMAX_SLOTS 2048
+int marian_hip_int8_affine_f32_chained(const float* A, int8_t* Aq, const int8_t* Bq,
+                                       const float* bias, const uint32_t* idx, int64_t n_idx,
+                                       float* out, int64_t M, int64_t K, int64_t N, float scale,
+                                       int relu, const float* absmax_in, float* absmax_out,
+                                       void* workspace, size_t workspace_bytes, void* stream);
+
+/*
  * Shortlisted output layer.  Reference (fp32): index_select(Wt, 0, idx), index_select(b, -1,
  * idx), then dot/affine with transB (src/data/shortlist.cpp:62-79,
  * src/layers/output.cpp:335-350).  Here rows idx[j] of the [N x K] payload and bias[idx[j]]

@@ -26,10 +26,12 @@ extern "C" {
  * beta may be NULL.  add != NULL fuses the skip connection that precedes the normalization in
  * the transformer's post-processing (`output + prevInput`, src/models/transformer.h:192-193,207):
  * x = in + add, else x = in.
+ * absmax_out: NULL, or MARIAN_HIP_ABSMAX_SLOTS (2048) floats that receive values whose maximum is
+ * max|out|, for marian_hip_int8_affine_f32_chained (needs rows <= 2048).
  */
 int marian_hip_layer_norm(const float* in, const float* add, const float* gamma,
                           int64_t gamma_cols, const float* beta, int64_t beta_cols, float* out,
-                          int64_t rows, int64_t cols, float eps, void* stream);
+                          int64_t rows, int64_t cols, float eps, float* absmax_out, void* stream);
 
 /*
  * Replaces Softmax, reference src/tensors/gpu/tensor_operators.cu (gSoftmax) and
@@ -76,11 +78,12 @@ int marian_hip_bdot_legacy(const float* A, const float* B, float* C, int64_t bat
  *   q: [batchQ, m, dk], k and v: [batchKV, len, dk] (entry i uses k, v of i % batchKV: encoder
  *   keys shared by the beam), out: [batchQ, m, dk]; mask as in marian_hip_softmax for score rows
  *   [batchQ * m, len], or NULL.  len <= 4096.
+ *   absmax_out: as for marian_hip_layer_norm (needs batchQ * m <= 2048).
  */
 int marian_hip_attention(const float* q, const float* k, const float* v, const float* mask,
                          int64_t n_masks, int64_t rows_per_mask, float* out, int64_t batchQ,
                          int64_t batchKV, int64_t m, int64_t len, int64_t dk, float scale,
-                         void* stream);
+                         float* absmax_out, void* stream);
 
 #ifdef __cplusplus
 }

@@ -24,19 +24,23 @@ SIGNATURES = {
     "marian_hip_int8_affine": (_i, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _f, _i, _vp]),
     "marian_hip_int8_affine_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _i64, _vp, _i64, _i64, _i64, _f, _i,
                                         _vp, _sz, _vp]),
+    "marian_hip_int8_affine_f32_chained": (_i, [_vp, _vp, _vp, _vp, _vp, _i64, _vp, _i64, _i64, _i64, _f,
+                                                _i, _vp, _vp, _vp, _sz, _vp]),
     "marian_hip_int8_affine_shortlist": (_i, [_vp, _vp, _vp, _vp, _i64, _vp, _i64, _i64, _i64,
                                               _f, _i, _vp]),
     "marian_hip_int8_multiply_i32": (_i, [_vp, _vp, _vp, _i64, _vp, _i64, _i64, _i64, _vp]),
     "marian_hip_int8_set_kernel": (_i, [_i]),
     # include/marian_hip_ops.h
-    "marian_hip_layer_norm": (_i, [_vp, _vp, _vp, _i64, _vp, _i64, _vp, _i64, _i64, _f, _vp]),
+    "marian_hip_layer_norm": (_i, [_vp, _vp, _vp, _i64, _vp, _i64, _vp, _i64, _i64, _f, _vp, _vp]),
     "marian_hip_softmax": (_i, [_vp, _vp, _i64, _i64, _vp, _i64, _i64, _vp]),
     "marian_hip_logsoftmax": (_i, [_vp, _vp, _i64, _i64, _vp]),
     "marian_hip_transpose0213": (_i, [_vp, _vp, _i64, _i64, _i64, _i64, _vp]),
     "marian_hip_bdot_legacy": (_i, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i, _i, _f, _vp]),
     "marian_hip_attention": (_i, [_vp, _vp, _vp, _vp, _i64, _i64, _vp, _i64, _i64, _i64, _i64, _i64,
-                                  _f, _vp]),
+                                  _f, _vp, _vp]),
 }
+
+ABSMAX_SLOTS = 2048   # MARIAN_HIP_ABSMAX_SLOTS
 
 _lib = None
 

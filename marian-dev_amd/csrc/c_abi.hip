@@ -18,6 +18,8 @@ using namespace marian_hip;
 
 namespace {
 thread_local int g_last_hip_error = 0;
+// set by the launcher whose kernel fills GemmArgs::absmax_out itself
+thread_local bool t_absmax_written = false;
 }
 
 int marian_hip::record_hip_error(int e) {
@@ -130,7 +132,12 @@ int launch_stream32(const GemmArgs& a, const FusedSrc& f, hipStream_t st) {
   if(lds < Cfg::kReduceBytes) lds = Cfg::kReduceBytes;
   int blocks = (a.n_out + Cfg::kColsPerBlock - 1) / Cfg::kColsPerBlock;
   int m_tiles = MODE == kFusedAll ? 1 : (a.M + MT32 * 32 - 1) / (MT32 * 32);
-  hipLaunchKernelGGL(kernel, dim3(blocks, m_tiles), dim3(kStream32Threads), lds, st, a, f.A,
+  GemmArgs a2 = a;
+  if(a.absmax_out) {   // eight slots per workgroup, one per wave
+    if((long long)blocks * m_tiles * kStream32Waves <= kAbsmaxSlots) t_absmax_written = true;
+    else a2.absmax_out = nullptr;
+  }
+  hipLaunchKernelGGL(kernel, dim3(blocks, m_tiles), dim3(kStream32Threads), lds, st, a2, f.A,
                      f.aq_out, f.partials, f.n_partials);
   MH_HIP(hipGetLastError());
   return MARIAN_HIP_OK;
@@ -321,7 +328,7 @@ int check_gemm(const int8_t* Aq, const int8_t* Bq, const void* out, const float*
 
 int run_gemm(const int8_t* Aq, const int8_t* Bq, const float* bias, const uint32_t* idx,
              int64_t n_idx, void* out, int64_t M, int64_t K, int64_t N, float scale, int relu,
-             int dump, void* stream) {
+             int dump, void* stream, float* absmax_out = nullptr) {
   int st = check_gemm(Aq, Bq, out, bias, idx, n_idx, M, K, N);
   if(st != MARIAN_HIP_OK) return st;
   const int64_t n_out = idx ? n_idx : N;
@@ -332,6 +339,7 @@ int run_gemm(const int8_t* Aq, const int8_t* Bq, const float* bias, const uint32
   a.scale = scale; a.relu = relu ? 1 : 0; a.dump = dump;
   a.dbg = g_kernel_override.load(std::memory_order_relaxed) / 1000;
   a.prof = g_prof.load(std::memory_order_relaxed);
+  a.absmax_out = absmax_out;
   return launch_gemm(a, reinterpret_cast<hipStream_t>(stream));
 }
 
@@ -437,10 +445,11 @@ int marian_hip_int8_affine(const int8_t* Aq, const int8_t* Bq, const float* bias
   return run_gemm(Aq, Bq, bias, nullptr, 0, out, M, K, N, scale, relu, 0, stream);
 }
 
-int marian_hip_int8_affine_f32(const float* A, int8_t* Aq, const int8_t* Bq, const float* bias,
-                               const uint32_t* idx, int64_t n_idx, float* out, int64_t M,
-                               int64_t K, int64_t N, float scale, int relu, void* workspace,
-                               size_t workspace_bytes, void* stream) {
+static int affine_f32_impl(const float* A, int8_t* Aq, const int8_t* Bq, const float* bias,
+                           const uint32_t* idx, int64_t n_idx, float* out, int64_t M, int64_t K,
+                           int64_t N, float scale, int relu, const float* absmax_in,
+                           float* absmax_out, void* workspace, size_t workspace_bytes,
+                           void* stream) {
   int st = check_gemm(Aq, Bq, out, bias, idx, n_idx, M, K, N);
   if(st != MARIAN_HIP_OK) return st;
   const int64_t n_out = idx ? n_idx : N;
@@ -457,6 +466,7 @@ int marian_hip_int8_affine_f32(const float* A, int8_t* Aq, const int8_t* Bq, con
   a.M = (int)M; a.K = (int)K; a.N = (int)N; a.n_out = (int)n_out;
   a.scale = scale; a.relu = relu ? 1 : 0; a.dump = 0; a.dbg = 0;
   a.prof = g_prof.load(std::memory_order_relaxed);
+  a.absmax_out = absmax_out;
   FusedSrc f;
   f.A = A; f.aq_out = Aq;
   const bool want_tiled = which >= 620 && which <= 628;
@@ -471,20 +481,69 @@ int marian_hip_int8_affine_f32(const float* A, int8_t* Aq, const int8_t* Bq, con
   const bool tiled_ok = n_out > 0 && workspace && workspace_bytes >= kWorkspaceBytes &&
                         aligned(workspace, 4);
   if(tiled_ok && which != 600 && (want_tiled || (M <= 256 && K <= 1024 && n_out <= 8192))) {
-    const size_t n = (size_t)M * (size_t)K;
-    float* partials = reinterpret_cast<float*>(workspace);
-    const int g = absmax_blocks(n / 4);
-    hipLaunchKernelGGL(absmax_partial_kernel, dim3(g), dim3(kQuantThreads), 0, hst, A, n / 4,
-                       partials);
-    MH_HIP(hipGetLastError());
-    f.partials = partials;
-    f.n_partials = g;
+    if(absmax_in) {   // the producer of A left its abs-max: no launch for it
+      f.partials = absmax_in;
+      f.n_partials = kAbsmaxSlots;
+    } else {
+      const size_t n = (size_t)M * (size_t)K;
+      float* partials = reinterpret_cast<float*>(workspace);
+      const int g = absmax_blocks(n / 4);
+      hipLaunchKernelGGL(absmax_partial_kernel, dim3(g), dim3(kQuantThreads), 0, hst, A, n / 4,
+                         partials);
+      MH_HIP(hipGetLastError());
+      f.partials = partials;
+      f.n_partials = g;
+    }
     return launch_stream32_auto<kFusedTiled>(a, f, hst, want_tiled ? which - 620 : 0);
   }
-  st = marian_hip_int8_prepare_a(A, Aq, M, K, workspace, workspace_bytes, stream);
-  if(st != MARIAN_HIP_OK) return st;
-  return run_gemm(Aq, Bq, bias, idx, n_idx, out, M, K, N, scale, relu, 0, stream);
+  if(absmax_in) {   // quantize with the abs-max the producer left, then the GEMM
+    const size_t n = (size_t)M * (size_t)K;
+    size_t qblocks = (n / 16 + kQuantThreads - 1) / kQuantThreads;
+    if(qblocks > 4096) qblocks = 4096;
+    hipLaunchKernelGGL(quantize_a_kernel, dim3((int)qblocks), dim3(kQuantThreads), 0, hst, A, n / 16,
+                       absmax_in, (int)kAbsmaxSlots, Aq);
+    MH_HIP(hipGetLastError());
+  } else {
+    st = marian_hip_int8_prepare_a(A, Aq, M, K, workspace, workspace_bytes, stream);
+    if(st != MARIAN_HIP_OK) return st;
+  }
+  return run_gemm(Aq, Bq, bias, idx, n_idx, out, M, K, N, scale, relu, 0, stream, absmax_out);
 }
+
+// abs-max of a finished output for the next call, when the kernel that wrote it did not leave it
+static int absmax_after(const float* out, int64_t M, int64_t n_out, float* absmax_out, hipStream_t st) {
+  const size_t n = (size_t)M * (size_t)n_out;
+  const int g = absmax_blocks(n / 4);   // n_out % 8 == 0; g <= 1024 partials
+  hipLaunchKernelGGL(zero_floats_kernel, dim3(2), dim3(kQuantThreads), 0, st, absmax_out + g, kAbsmaxSlots - g);
+  hipLaunchKernelGGL(absmax_partial_kernel, dim3(g), dim3(kQuantThreads), 0, st, out, n / 4, absmax_out);
+  MH_HIP(hipGetLastError());
+  return MARIAN_HIP_OK;
+}
+
+int marian_hip_int8_affine_f32(const float* A, int8_t* Aq, const int8_t* Bq, const float* bias,
+                               const uint32_t* idx, int64_t n_idx, float* out, int64_t M,
+                               int64_t K, int64_t N, float scale, int relu, void* workspace,
+                               size_t workspace_bytes, void* stream) {
+  return affine_f32_impl(A, Aq, Bq, bias, idx, n_idx, out, M, K, N, scale, relu, nullptr, nullptr,
+                         workspace, workspace_bytes, stream);
+}
+
+int marian_hip_int8_affine_f32_chained(const float* A, int8_t* Aq, const int8_t* Bq,
+                                       const float* bias, const uint32_t* idx, int64_t n_idx,
+                                       float* out, int64_t M, int64_t K, int64_t N, float scale,
+                                       int relu, const float* absmax_in, float* absmax_out,
+                                       void* workspace, size_t workspace_bytes, void* stream) {
+  if((absmax_in && !aligned(absmax_in, 4)) || (absmax_out && !aligned(absmax_out, 4)))
+    return MARIAN_HIP_ERR_ALIGN;
+  t_absmax_written = false;
+  int st = affine_f32_impl(A, Aq, Bq, bias, idx, n_idx, out, M, K, N, scale, relu, absmax_in,
+                           absmax_out, workspace, workspace_bytes, stream);
+  if(st != MARIAN_HIP_OK || !absmax_out || t_absmax_written) return st;
+  const int64_t n_out = idx ? n_idx : N;
+  if(M == 0 || n_out == 0) return MARIAN_HIP_OK;
+  return absmax_after(out, M, n_out, absmax_out, reinterpret_cast<hipStream_t>(stream));
+}
+
 
 int marian_hip_int8_affine_shortlist(const int8_t* Aq, const int8_t* Bq, const float* bias,
                                      const uint32_t* idx, int64_t n_idx, float* out, int64_t M,

@@ -61,8 +61,10 @@ __global__ __launch_bounds__(256) void layer_norm_kernel(const float* in,
                                                          const float* __restrict__ add,
                                                          const float* __restrict__ gamma, int gamma_stride,
                                                          const float* __restrict__ beta, int beta_stride,
-                                                         float* out, int cols, float eps) {
+                                                         float* out, int cols, float eps,
+                                                         float* __restrict__ absmax_out) {
   __shared__ float red[4];
+  float omax = 0.0f;   // max |y| over what this thread writes
   const size_t row = blockIdx.x;
   const float* x = in + row * cols;
   const float* a = add ? add + row * cols : nullptr;
@@ -105,6 +107,7 @@ __global__ __launch_bounds__(256) void layer_norm_kernel(const float* in,
           float t = gamma[gamma_stride * (4 * i + e)] * ((r[e] - mean) / sigma);
           if(beta) t = t + beta[beta_stride * (4 * i + e)];
           r[e] = t;
+          omax = fmaxf(omax, fabsf(t));
         }
         reinterpret_cast<v4f*>(y)[i] = v4f{r[0], r[1], r[2], r[3]};
       }
@@ -123,7 +126,14 @@ __global__ __launch_bounds__(256) void layer_norm_kernel(const float* in,
       float t = gamma[gamma_stride * i] * (((a ? x[i] + a[i] : x[i]) - mean) / sigma);
       if(beta) t = t + beta[beta_stride * i];
       y[i] = t;
+      omax = fmaxf(omax, fabsf(t));
     }
+  }
+  if(absmax_out) {   // slot `row`; workgroup 0 zeroes the slots past the last row
+    omax = row_reduce<256, true>(omax, red);
+    if(tid == 0) absmax_out[row] = omax;
+    if(row == 0)
+      for(int sl = gridDim.x + tid; sl < kAbsmaxSlots; sl += 256) absmax_out[sl] = 0.0f;
   }
 }
 
@@ -280,9 +290,11 @@ __global__ __launch_bounds__(256) void attention_kernel(const float* __restrict_
                                                         long long n_masks, long long rows_per_mask,
                                                         float* __restrict__ out, long long rows_total,
                                                         long long batchKV, int m, int len, int dk,
-                                                        float scale) {
+                                                        float scale, float* __restrict__ absmax_out) {
   extern __shared__ float att_lds[];
   const long long wr = (long long)blockIdx.x * 4 + threadIdx.x / 64;
+  if(absmax_out && blockIdx.x == 0)   // slots past the last query row
+    for(int sl = (int)rows_total + threadIdx.x; sl < kAbsmaxSlots; sl += 256) absmax_out[sl] = 0.0f;
   if(wr >= rows_total) return;   // whole waves leave; no workgroup barrier is used
   float* sc = att_lds + (threadIdx.x / 64) * len;
   const int lane = threadIdx.x % 64;
@@ -293,6 +305,7 @@ __global__ __launch_bounds__(256) void attention_kernel(const float* __restrict_
   const float* mk = mask ? mask + (size_t)((wr / rows_per_mask) % n_masks) * len : nullptr;
   const bool vec = (dk % 4) == 0 && ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(kb)) % 16) == 0;
   float mx = -__builtin_inff();
+  float omax = 0.0f;   // max |out| of this query row
   for(int pos = lane; pos < len; pos += 64) {
     float s = 0.0f;
     if(vec && dk == 64) {   // the usual head size: all sixteen loads of the key row in flight at once
@@ -345,6 +358,11 @@ __global__ __launch_bounds__(256) void attention_kernel(const float* __restrict_
     }
     for(; pos < len; ++pos) o = fmaf(sc[pos], vb[(size_t)pos * dk + d], o);
     out[(size_t)wr * dk + d] = 1.0f * o;
+    omax = fmaxf(omax, fabsf(1.0f * o));
+  }
+  if(absmax_out) {   // slot = query row
+    omax = wave_maxf(omax);
+    if(lane == 0) absmax_out[wr] = omax;
   }
 }
 
@@ -363,7 +381,9 @@ extern "C" {
 
 int marian_hip_layer_norm(const float* in, const float* add, const float* gamma, int64_t gamma_cols,
                           const float* beta, int64_t beta_cols, float* out, int64_t rows,
-                          int64_t cols, float eps, void* stream) {
+                          int64_t cols, float eps, float* absmax_out, void* stream) {
+  if(absmax_out && rows > kAbsmaxSlots) return MARIAN_HIP_ERR_RANGE;
+  if(absmax_out && !aligned4(absmax_out)) return MARIAN_HIP_ERR_ALIGN;
   if(rows < 0 || cols <= 0) return MARIAN_HIP_ERR_SHAPE;
   if((gamma_cols != cols && gamma_cols != 1) || (beta && beta_cols != cols && beta_cols != 1))
     return MARIAN_HIP_ERR_SHAPE;
@@ -376,11 +396,11 @@ int marian_hip_layer_norm(const float* in, const float* add, const float* gamma,
   const int gs = gamma_cols > 1 ? 1 : 0, bs = (beta && beta_cols > 1) ? 1 : 0;
   const bool vec = cols % 4 == 0 && aligned16(in) && aligned16(out) && (!add || aligned16(add));
   if(vec && cols <= 1024)
-    hipLaunchKernelGGL(layer_norm_kernel<1>, dim3((unsigned)rows), dim3(256), 0, st, in, add, gamma, gs, beta, bs, out, (int)cols, eps);
+    hipLaunchKernelGGL(layer_norm_kernel<1>, dim3((unsigned)rows), dim3(256), 0, st, in, add, gamma, gs, beta, bs, out, (int)cols, eps, absmax_out);
   else if(vec && cols <= 4096)
-    hipLaunchKernelGGL(layer_norm_kernel<4>, dim3((unsigned)rows), dim3(256), 0, st, in, add, gamma, gs, beta, bs, out, (int)cols, eps);
+    hipLaunchKernelGGL(layer_norm_kernel<4>, dim3((unsigned)rows), dim3(256), 0, st, in, add, gamma, gs, beta, bs, out, (int)cols, eps, absmax_out);
   else
-    hipLaunchKernelGGL(layer_norm_kernel<0>, dim3((unsigned)rows), dim3(256), 0, st, in, add, gamma, gs, beta, bs, out, (int)cols, eps);
+    hipLaunchKernelGGL(layer_norm_kernel<0>, dim3((unsigned)rows), dim3(256), 0, st, in, add, gamma, gs, beta, bs, out, (int)cols, eps, absmax_out);
   MH_HIP(hipGetLastError());
   return MARIAN_HIP_OK;
 }
@@ -460,7 +480,9 @@ int marian_hip_bdot_legacy(const float* A, const float* B, float* C, int64_t bat
 int marian_hip_attention(const float* q, const float* k, const float* v, const float* mask,
                          int64_t n_masks, int64_t rows_per_mask, float* out, int64_t batchQ,
                          int64_t batchKV, int64_t m, int64_t len, int64_t dk, float scale,
-                         void* stream) {
+                         float* absmax_out, void* stream) {
+  if(absmax_out && batchQ * m > kAbsmaxSlots) return MARIAN_HIP_ERR_RANGE;
+  if(absmax_out && !aligned4(absmax_out)) return MARIAN_HIP_ERR_ALIGN;
   if(batchQ < 0 || batchKV <= 0 || m <= 0 || len <= 0 || dk <= 0) return MARIAN_HIP_ERR_SHAPE;
   if(mask && (n_masks <= 0 || rows_per_mask <= 0)) return MARIAN_HIP_ERR_SHAPE;
   if(len > 4096) return MARIAN_HIP_ERR_RANGE;
@@ -481,7 +503,7 @@ int marian_hip_attention(const float* q, const float* k, const float* v, const f
   if(lds_status != 0) return record_hip_error(lds_status);
   hipLaunchKernelGGL(attention_kernel, dim3((unsigned)((rows_total + 3) / 4)), dim3(256), lds, st, q, k, v,
                      mask, (long long)n_masks, (long long)rows_per_mask, out, rows_total,
-                     (long long)batchKV, (int)m, (int)len, (int)dk, scale);
+                     (long long)batchKV, (int)m, (int)len, (int)dk, scale, absmax_out);
   MH_HIP(hipGetLastError());
   return MARIAN_HIP_OK;
 }

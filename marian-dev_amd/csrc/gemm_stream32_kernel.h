@@ -51,7 +51,7 @@ struct Stream32Cfg {
 };
 
 // Dynamic LDS: kFusedAll holds all of K (32 * MT32 * K bytes); otherwise one chunk (kStageBytes);
-// both at least kReduceBytes.  partials: n_partials (1..1024) abs-max values (kFusedTiled only).
+// both at least kReduceBytes.  partials: n_partials (1..2048) abs-max values (kFusedTiled only).
 template <int MT32, int WN, int KW, int PW, int MODE>
 __global__ __launch_bounds__(kStream32Threads) void gemm_stream32_kernel(GemmArgs args,
                                                                         const float* A,
@@ -114,8 +114,10 @@ __global__ __launch_bounds__(kStream32Threads) void gemm_stream32_kernel(GemmArg
   if(MODE == kPrequant) aqm_pre = tail_quant_mult(args.Aq, (size_t)M * (size_t)K);
   float amax = 0.0f;
   if(TILED) {   // two (clamped) abs-max partials per thread cover all 1024
-    amax = fmaxf(partials[min(tid, n_partials - 1)],
-                 partials[min(tid + kStream32Threads, n_partials - 1)]);
+    amax = fmaxf(fmaxf(partials[min(tid, n_partials - 1)],
+                       partials[min(tid + kStream32Threads, n_partials - 1)]),
+                 fmaxf(partials[min(tid + 2 * kStream32Threads, n_partials - 1)],
+                       partials[min(tid + 3 * kStream32Threads, n_partials - 1)]));
   }
   const int8_t* wrow = args.Bq + (size_t)wsrc * (size_t)K + lg * 16;
   __builtin_amdgcn_sched_barrier(0);
@@ -376,6 +378,7 @@ __global__ __launch_bounds__(kStream32Threads) void gemm_stream32_kernel(GemmArg
   // ---- epilogue: value v of tile mt in lane (li, lg) is activation row mt * 32 + li, weight
   //      row 8 * (v / 4) + 4 * lg + v % 4 of the wave's 32 ----
   if(args.prof) tp[4] = clock64();
+  float omax = 0.0f;   // max |y| over what this wave stores
   {
     const float unquant = unquant_mult(MODE == kPrequant ? aqm_pre : aqm, bqm, args.scale);
     const bool has_bias = args.bias != nullptr;
@@ -400,11 +403,21 @@ __global__ __launch_bounds__(kStream32Threads) void gemm_stream32_kernel(GemmArg
         y[e] = (float)mine[c][e] * unquant;
         if(has_bias) y[e] = y[e] + bias_s[c][e];
         if(args.relu) y[e] = y[e] > 0.0f ? y[e] : 0.0f;
+        omax = fmaxf(omax, fabsf(y[e]));
       }
       float* o = reinterpret_cast<float*>(args.out) + off;
       if(CW == 4) *reinterpret_cast<v4f*>(o) = v4f{y[0], y[1], y[CW - 2], y[CW - 1]};
       else *reinterpret_cast<float2*>(o) = float2{y[0], y[1]};
     }
+  }
+  if(args.absmax_out && !args.dump) {
+    // slot (workgroup, wave) takes this wave's maximum; workgroup 0 zeroes the slots nobody owns
+    // (the launcher made sure that 8 slots per workgroup fit)
+    const int block = blockIdx.y * gridDim.x + blockIdx.x, used = gridDim.x * gridDim.y * kStream32Waves;
+    omax = wave_max(omax);
+    if(lane == 0) args.absmax_out[block * kStream32Waves + wave] = omax;
+    if(block == 0)
+      for(int sl = used + tid; sl < kAbsmaxSlots; sl += kStream32Threads) args.absmax_out[sl] = 0.0f;
   }
   if(args.prof && tid == 0) {
     long long* p = args.prof + ((size_t)blockIdx.y * gridDim.x + blockIdx.x) * 8;

@@ -100,7 +100,12 @@ struct GemmArgs {
   int relu, dump;
   int dbg;  // measurement switches (bit 0: no refetch, bit 1: no stores); 0 in normal use
   long long* prof;  // per-workgroup phase clocks for tuning runs, null in normal use
+  // kAbsmaxSlots floats that receive values whose maximum is max|out| (the next call's abs-max,
+  // taken where the tensor is produced), or null
+  float* absmax_out = nullptr;
 };
+
+constexpr int kAbsmaxSlots = 2048;
 
 __device__ __forceinline__ Epilogue make_epilogue(const GemmArgs& a) {
   Epilogue e;

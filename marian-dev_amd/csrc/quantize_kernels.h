@@ -102,6 +102,11 @@ __global__ __launch_bounds__(kQuantThreads) void absmax_partial_kernel(
   if(threadIdx.x == 0) partials[blockIdx.x] = m;
 }
 
+// Clears n floats (a kernel rather than a memset node, so callers may capture the call in a graph).
+__global__ __launch_bounds__(kQuantThreads) void zero_floats_kernel(float* __restrict__ p, int n) {
+  for(int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) p[i] = 0.0f;
+}
+
 // Pass 2 of prepareA: reduce the partials, quantize 16 values per thread per step, block 0
 // writes the quantMult tail at byte n.
 __global__ __launch_bounds__(kQuantThreads) void quantize_a_kernel(

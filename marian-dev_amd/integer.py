@@ -172,10 +172,24 @@ def affineOrDot(a, bQuant, bias=None, transA=False, transB=False, scale=1.0, rel
     return out
 
 
-def affine_f32(a, bQuant, bias=None, scale=1.0, relu=False, shortlist=None):
+class AbsMax:
+    """Values whose maximum is max|x| of the tensor they were produced with (2048 floats on the
+    device): handed from the call that writes a tensor to the affine call that reads it, in place
+    of the abs-max pass of prepareA (reference src/tensors/cpu/intgemm_interface.h:23)."""
+
+    def __init__(self, device):
+        self.data = torch.empty(_lib.ABSMAX_SLOTS, dtype=torch.float32, device=device)
+
+    def data_ptr(self):
+        return self.data.data_ptr()
+
+
+def affine_f32(a, bQuant, bias=None, scale=1.0, relu=False, shortlist=None, absmax=None,
+               want_absmax=False):
     """prepareA node + multiply node through the single C-ABI call marian_hip_int8_affine_f32
     (one fused kernel for small activations).  Returns (out, aQuant): aQuant is what the
-    prepareA node would have produced."""
+    prepareA node would have produced.  absmax: the AbsMax left by the call that produced `a`;
+    want_absmax: also return an AbsMax of `out` as a third value."""
     a = a.contiguous()
     be = _backend_of(a)
     aQuant = QTensor.empty(a.shape, Type.intgemm8, a.device)
@@ -191,13 +205,23 @@ def affine_f32(a, bQuant, bias=None, scale=1.0, relu=False, shortlist=None):
         bias_ptr = bias.data_ptr()
     if shortlist is not None:
         _abort_if(shortlist.dtype not in (torch.int32, torch.uint32), "shortlist ids must be uint32, got {}", shortlist.dtype)
-    st = be.lib.marian_hip_int8_affine_f32(
-        a.data_ptr(), aQuant.data_ptr(), bQuant.data_ptr(), bias_ptr,
-        None if shortlist is None else shortlist.data_ptr(), n_out if shortlist is not None else 0,
-        out.data_ptr(), M, K, N, scale, int(relu), be.workspace.data_ptr(), be.workspace_bytes,
+    idx_ptr = None if shortlist is None else shortlist.data_ptr()
+    n_idx = n_out if shortlist is not None else 0
+    if absmax is None and not want_absmax:
+        st = be.lib.marian_hip_int8_affine_f32(
+            a.data_ptr(), aQuant.data_ptr(), bQuant.data_ptr(), bias_ptr, idx_ptr, n_idx,
+            out.data_ptr(), M, K, N, scale, int(relu), be.workspace.data_ptr(), be.workspace_bytes,
+            be.stream())
+        _lib.check(st, "affineOrDot")
+        return out, aQuant
+    omax = AbsMax(a.device) if want_absmax else None
+    st = be.lib.marian_hip_int8_affine_f32_chained(
+        a.data_ptr(), aQuant.data_ptr(), bQuant.data_ptr(), bias_ptr, idx_ptr, n_idx,
+        out.data_ptr(), M, K, N, scale, int(relu), None if absmax is None else absmax.data_ptr(),
+        None if omax is None else omax.data_ptr(), be.workspace.data_ptr(), be.workspace_bytes,
         be.stream())
     _lib.check(st, "affineOrDot")
-    return out, aQuant
+    return (out, aQuant, omax) if want_absmax else (out, aQuant)
 
 
 def multiply(aQuant, bQuant, bias=None, scale=1.0, relu=False, shortlist=None):

@@ -14,7 +14,7 @@ step is a call into the C ABI.  There is no CPU fallback.
 import torch
 
 from . import _lib
-from .integer import _abort_if, _backend_of
+from .integer import AbsMax, _abort_if, _backend_of
 
 
 def _f32c(x, what):
@@ -22,9 +22,10 @@ def _f32c(x, what):
     return x.contiguous()
 
 
-def layerNorm(x, gamma, beta=None, eps=1e-9, add=None):
+def layerNorm(x, gamma, beta=None, eps=1e-9, add=None, want_absmax=False):
     """reference src/graph/expression_operators.cpp:901-913; `add` fuses the skip connection in
-    front of it (out = layerNorm(x + add))."""
+    front of it (out = layerNorm(x + add)).  want_absmax: also return the AbsMax of the output
+    for the affine calls that read it."""
     x = _f32c(x, "layerNorm")
     be = _backend_of(x)
     cols = x.shape[-1]
@@ -38,12 +39,13 @@ def layerNorm(x, gamma, beta=None, eps=1e-9, add=None):
         add = _f32c(add, "layerNorm")
         _abort_if(tuple(add.shape) != tuple(x.shape), "layerNorm: skip input shape {} vs {}", tuple(add.shape), tuple(x.shape))
     out = torch.empty_like(x)
+    omax = AbsMax(x.device) if want_absmax else None
     st = be.lib.marian_hip_layer_norm(
         x.data_ptr(), None if add is None else add.data_ptr(), gamma.data_ptr(), gamma.numel(),
         None if beta is None else beta.data_ptr(), 0 if beta is None else beta.numel(),
-        out.data_ptr(), rows, cols, eps, be.stream())
+        out.data_ptr(), rows, cols, eps, None if omax is None else omax.data_ptr(), be.stream())
     _lib.check(st, "layerNorm")
-    return out
+    return (out, omax) if want_absmax else out
 
 
 def softmax(a, mask=None, rowsPerMask=1):
@@ -126,7 +128,7 @@ def bdot_legacy(a, b, transA=False, transB=False, scalar=1.0):
     return out
 
 
-def Attention(q, k, v, mask=None, rowsPerMask=1):
+def Attention(q, k, v, mask=None, rowsPerMask=1, want_absmax=False):
     """reference src/models/transformer.h:241-280 (inference: no dropout, weights not kept):
     softmax(bdot_legacy(q, k, false, true, 1/sqrt(dk)) + mask) then bdot_legacy(weights, v), in
     one launch.  q: [batch*beam, heads, tgt, dk]; k, v: [batch(*beam), heads, len, dk]."""
@@ -142,9 +144,10 @@ def Attention(q, k, v, mask=None, rowsPerMask=1):
         mask = _f32c(mask, "Attention").reshape(-1, L)
         n_masks = mask.shape[0]
     out = torch.empty_like(q)
+    omax = AbsMax(q.device) if want_absmax else None
     st = be.lib.marian_hip_attention(q.data_ptr(), k.data_ptr(), v.data_ptr(),
                                      None if mask is None else mask.data_ptr(), n_masks, rowsPerMask,
                                      out.data_ptr(), batchQ, batchKV, m, L, dk, 1.0 / float(dk) ** 0.5,
-                                     be.stream())
+                                     None if omax is None else omax.data_ptr(), be.stream())
     _lib.check(st, "Attention")
-    return out
+    return (out, omax) if want_absmax else out

@@ -189,3 +189,27 @@ def test_one_launch_attention_equals_the_three_operators(ops, chk, synth, BQ, BK
     zc = chk.bdot_legacy(q, k, False, True, scale)
     wc = chk.softmax(zc, mask, rows_per_mask=rpm)
     close(got, chk.bdot_legacy(wc, v), 4 * REL, 2e-5)
+
+
+def test_absmax_outputs_of_layer_norm_and_attention(ops, integer, synth):
+    """The abs-max slots a producer leaves have max|out| as their maximum, and an affine call that
+    takes them gives the bits of the call that scans the tensor itself."""
+    x = synth.normal(51, 0, (128, 1024), 1.0)
+    g = synth.normal(51, 2, (1024,), 0.1) + np.float32(1.0)
+    b = synth.normal(51, 3, (1024,), 0.1)
+    y, ymax = ops.layerNorm(dev(x), dev(g), dev(b), 1e-6, dev(x), want_absmax=True)
+    assert np.array_equal(y.cpu().numpy(), ops.layerNorm(dev(x), dev(g), dev(b), 1e-6, dev(x)).cpu().numpy())
+    assert float(ymax.data.max()) == float(y.abs().max())
+    q = synth.normal(52, 0, (2048, 1, 64), 1.0)
+    k = synth.normal(52, 1, (2048, 21, 64), 1.0)
+    v = synth.normal(52, 2, (2048, 21, 64), 1.0)
+    o, omax = ops.Attention(dev(q), dev(k), dev(v), want_absmax=True)
+    assert np.array_equal(o.cpu().numpy(), ops.Attention(dev(q), dev(k), dev(v)).cpu().numpy())
+    assert float(omax.data.max()) == float(o.abs().max())
+    import torch
+    W = torch.randn(1024, 1024, device="cuda") * 0.02
+    Bq = integer.prepareB(W)
+    for t, tmax in ((y, ymax), (o.view(128, 1024), omax)):
+        got, aq = integer.affine_f32(t, Bq, None, absmax=tmax)
+        want, aq_ref = integer.affine_f32(t, Bq, None)
+        assert np.array_equal(aq.numpy(), aq_ref.numpy()) and np.array_equal(got.cpu().numpy(), want.cpu().numpy())

@@ -317,6 +317,33 @@ def test_config5_shortlist(integer, orc, synth, M):
     assert np.array_equal(dense_acc[rows], want_acc) and np.array_equal(dense[rows], want)
 
 
+# ---------------------------------------------------------------- abs-max handed between calls
+
+@pytest.mark.parametrize("M,K,N,N2", [(128, 1024, 1024, 1024), (128, 1024, 4096, 1024), (128, 4096, 1024, 512),
+                                      (16, 512, 512, 64), (64, 2048, 512, 2048), (200, 1024, 504, 1000),
+                                      (300, 1024, 32000, 64), (600, 512, 2048, 512), (33, 192, 136, 24)])
+def test_absmax_chaining_equals_recomputation(integer, orc, synth, M, K, N, N2):
+    """A first affine call leaves the abs-max of its output; a second one, reading that output,
+    takes it instead of scanning the tensor: outputs and quantized activations are bit-identical to
+    the unchained calls, and the slots' maximum is max|out| exactly - whichever kernel ran."""
+    say("chain", M, K, N, N2)
+    A, W, bias = inputs(synth, 8000 + M + N, M, K, N)
+    W2 = synth.normal(8001 + M, synth.STREAM_W, (N, N2), 0.02) if N % 64 == 0 else None
+    Bq = upload_q(integer, orc.prepare_b(W), (K, N))
+    relu = (N % 16 == 0)
+    out, Aq, omax = integer.affine_f32(dev(A), Bq, dev(bias), relu=relu, want_absmax=True)
+    ref, Aq_ref = integer.affine_f32(dev(A), Bq, dev(bias), relu=relu)
+    assert np.array_equal(out.cpu().numpy(), ref.cpu().numpy()) and np.array_equal(Aq.numpy(), Aq_ref.numpy())
+    slots = omax.data.cpu().numpy()
+    assert slots.shape == (2048,) and float(slots.max()) == float(np.abs(ref.cpu().numpy()).max())
+    if W2 is None:
+        return
+    Bq2 = upload_q(integer, orc.prepare_b(W2), (N, N2))
+    got, Aq2 = integer.affine_f32(out, Bq2, None, absmax=omax)
+    want, Aq2_ref = integer.affine_f32(ref, Bq2, None)
+    assert np.array_equal(Aq2.numpy(), Aq2_ref.numpy()) and np.array_equal(got.cpu().numpy(), want.cpu().numpy())
+
+
 # ---------------------------------------------------------------- random shapes
 
 def _random_cases(n):
