@@ -79,11 +79,16 @@ int marian_hip_bdot_legacy(const float* A, const float* B, float* C, int64_t bat
  *   keys shared by the beam), out: [batchQ, m, dk]; mask as in marian_hip_softmax for score rows
  *   [batchQ * m, len], or NULL.  len <= 4096.
  *   absmax_out: as for marian_hip_layer_norm (needs batchQ * m <= 2048).
+ *   k_new, v_new: NULL, or [batchQ, dk] keys and values of the newest position (self-attention of
+ *   a decoding step: m == 1, batchKV == batchQ).  They take the place of position len - 1 of k and
+ *   v, and the call also stores them there, which is the concatenation of the new position onto
+ *   the cached ones (decoder state of src/models/transformer.h:683-700) without a copy launch; k
+ *   and v are written in that case.
  */
-int marian_hip_attention(const float* q, const float* k, const float* v, const float* mask,
-                         int64_t n_masks, int64_t rows_per_mask, float* out, int64_t batchQ,
-                         int64_t batchKV, int64_t m, int64_t len, int64_t dk, float scale,
-                         float* absmax_out, void* stream);
+int marian_hip_attention(const float* q, float* k, float* v, const float* mask, int64_t n_masks,
+                         int64_t rows_per_mask, float* out, int64_t batchQ, int64_t batchKV,
+                         int64_t m, int64_t len, int64_t dk, float scale, float* absmax_out,
+                         const float* k_new, const float* v_new, void* stream);
 
 #ifdef __cplusplus
 }

@@ -37,7 +37,7 @@ SIGNATURES = {
     "marian_hip_transpose0213": (_i, [_vp, _vp, _i64, _i64, _i64, _i64, _vp]),
     "marian_hip_bdot_legacy": (_i, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i, _i, _f, _vp]),
     "marian_hip_attention": (_i, [_vp, _vp, _vp, _vp, _i64, _i64, _vp, _i64, _i64, _i64, _i64, _i64,
-                                  _f, _vp, _vp]),
+                                  _f, _vp, _vp, _vp, _vp]),
 }
 
 ABSMAX_SLOTS = 2048   # MARIAN_HIP_ABSMAX_SLOTS

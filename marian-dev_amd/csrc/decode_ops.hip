@@ -285,8 +285,10 @@ __global__ __launch_bounds__(256) void bdot_kernel(const float* __restrict__ A, 
 // as bdot_kernel walks them), softmax over them exactly as softmax_kernel<64> computes it, then
 // the weighted sum of the value rows (a lane per output column, positions in ascending order,
 // as bdot_kernel does).  The scores of a row live in LDS: `len` floats per wave.
-__global__ __launch_bounds__(256) void attention_kernel(const float* __restrict__ Q, const float* __restrict__ Kt,
-                                                        const float* __restrict__ V, const float* __restrict__ mask,
+__global__ __launch_bounds__(256) void attention_kernel(const float* __restrict__ Q, float* Kt, float* V,
+                                                        const float* __restrict__ k_new,
+                                                        const float* __restrict__ v_new,
+                                                        const float* __restrict__ mask,
                                                         long long n_masks, long long rows_per_mask,
                                                         float* __restrict__ out, long long rows_total,
                                                         long long batchKV, int m, int len, int dk,
@@ -300,17 +302,29 @@ __global__ __launch_bounds__(256) void attention_kernel(const float* __restrict_
   const int lane = threadIdx.x % 64;
   const long long i = wr / m;
   const float* q = Q + (size_t)wr * dk;
-  const float* kb = Kt + (size_t)(i % batchKV) * len * dk;
-  const float* vb = V + (size_t)(i % batchKV) * len * dk;
+  float* kb = Kt + (size_t)(i % batchKV) * len * dk;
+  float* vb = V + (size_t)(i % batchKV) * len * dk;
+  if(k_new) {
+    // Newest position (m == 1, one wave per cache entry): its key and value rows go into the
+    // cache for the following steps; this step reads them from k_new / v_new directly.
+    for(int d = lane; d < dk; d += 64) {
+      kb[(size_t)(len - 1) * dk + d] = k_new[(size_t)wr * dk + d];
+      vb[(size_t)(len - 1) * dk + d] = v_new[(size_t)wr * dk + d];
+    }
+  }
+  const float* k_last = k_new ? k_new + (size_t)wr * dk : kb + (size_t)(len - 1) * dk;
+  const float* v_last = v_new ? v_new + (size_t)wr * dk : vb + (size_t)(len - 1) * dk;
   const float* mk = mask ? mask + (size_t)((wr / rows_per_mask) % n_masks) * len : nullptr;
-  const bool vec = (dk % 4) == 0 && ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(kb)) % 16) == 0;
+  const bool vec = (dk % 4) == 0 && ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(kb) |
+                                     reinterpret_cast<uintptr_t>(k_last)) % 16) == 0;
   float mx = -__builtin_inff();
   float omax = 0.0f;   // max |out| of this query row
   for(int pos = lane; pos < len; pos += 64) {
     float s = 0.0f;
+    const float* krow = pos == len - 1 ? k_last : kb + (size_t)pos * dk;
     if(vec && dk == 64) {   // the usual head size: all sixteen loads of the key row in flight at once
       const v4f* ar = reinterpret_cast<const v4f*>(q);
-      const v4f* br = reinterpret_cast<const v4f*>(kb + (size_t)pos * dk);
+      const v4f* br = reinterpret_cast<const v4f*>(krow);
       v4f kr[16];
 #pragma unroll
       for(int p = 0; p < 16; ++p) kr[p] = br[p];
@@ -324,7 +338,7 @@ __global__ __launch_bounds__(256) void attention_kernel(const float* __restrict_
       }
     } else if(vec) {
       const v4f* ar = reinterpret_cast<const v4f*>(q);
-      const v4f* br = reinterpret_cast<const v4f*>(kb + (size_t)pos * dk);
+      const v4f* br = reinterpret_cast<const v4f*>(krow);
       for(int p = 0; p < dk / 4; ++p) {
         const v4f av = ar[p], bv = br[p];
         s = fmaf(av.x, bv.x, s);
@@ -333,7 +347,7 @@ __global__ __launch_bounds__(256) void attention_kernel(const float* __restrict_
         s = fmaf(av.w, bv.w, s);
       }
     } else {
-      for(int p = 0; p < dk; ++p) s = fmaf(q[p], kb[(size_t)pos * dk + p], s);
+      for(int p = 0; p < dk; ++p) s = fmaf(q[p], krow[p], s);
     }
     float z = scale * s;
     if(mk) z = z + mk[pos];
@@ -352,11 +366,11 @@ __global__ __launch_bounds__(256) void attention_kernel(const float* __restrict_
     for(; pos + 8 <= len; pos += 8) {   // eight value loads in flight, same summation order
       float vr[8];
 #pragma unroll
-      for(int u = 0; u < 8; ++u) vr[u] = vb[(size_t)(pos + u) * dk + d];
+      for(int u = 0; u < 8; ++u) vr[u] = pos + u == len - 1 ? v_last[d] : vb[(size_t)(pos + u) * dk + d];
 #pragma unroll
       for(int u = 0; u < 8; ++u) o = fmaf(sc[pos + u], vr[u], o);
     }
-    for(; pos < len; ++pos) o = fmaf(sc[pos], vb[(size_t)pos * dk + d], o);
+    for(; pos < len; ++pos) o = fmaf(sc[pos], pos == len - 1 ? v_last[d] : vb[(size_t)pos * dk + d], o);
     out[(size_t)wr * dk + d] = 1.0f * o;
     omax = fmaxf(omax, fabsf(1.0f * o));
   }
@@ -477,10 +491,13 @@ int marian_hip_bdot_legacy(const float* A, const float* B, float* C, int64_t bat
   return MARIAN_HIP_OK;
 }
 
-int marian_hip_attention(const float* q, const float* k, const float* v, const float* mask,
-                         int64_t n_masks, int64_t rows_per_mask, float* out, int64_t batchQ,
-                         int64_t batchKV, int64_t m, int64_t len, int64_t dk, float scale,
-                         float* absmax_out, void* stream) {
+int marian_hip_attention(const float* q, float* k, float* v, const float* mask, int64_t n_masks,
+                         int64_t rows_per_mask, float* out, int64_t batchQ, int64_t batchKV,
+                         int64_t m, int64_t len, int64_t dk, float scale, float* absmax_out,
+                         const float* k_new, const float* v_new, void* stream) {
+  if((k_new != nullptr) != (v_new != nullptr)) return MARIAN_HIP_ERR_NULL;
+  if(k_new && (m != 1 || batchKV != batchQ)) return MARIAN_HIP_ERR_SHAPE;
+  if(k_new && (!aligned4(k_new) || !aligned4(v_new))) return MARIAN_HIP_ERR_ALIGN;
   if(absmax_out && batchQ * m > kAbsmaxSlots) return MARIAN_HIP_ERR_RANGE;
   if(absmax_out && !aligned4(absmax_out)) return MARIAN_HIP_ERR_ALIGN;
   if(batchQ < 0 || batchKV <= 0 || m <= 0 || len <= 0 || dk <= 0) return MARIAN_HIP_ERR_SHAPE;
@@ -502,7 +519,7 @@ int marian_hip_attention(const float* q, const float* k, const float* v, const f
   }();
   if(lds_status != 0) return record_hip_error(lds_status);
   hipLaunchKernelGGL(attention_kernel, dim3((unsigned)((rows_total + 3) / 4)), dim3(256), lds, st, q, k, v,
-                     mask, (long long)n_masks, (long long)rows_per_mask, out, rows_total,
+                     k_new, v_new, mask, (long long)n_masks, (long long)rows_per_mask, out, rows_total,
                      (long long)batchKV, (int)m, (int)len, (int)dk, scale, absmax_out);
   MH_HIP(hipGetLastError());
   return MARIAN_HIP_OK;

@@ -128,11 +128,20 @@ def bdot_legacy(a, b, transA=False, transB=False, scalar=1.0):
     return out
 
 
-def Attention(q, k, v, mask=None, rowsPerMask=1, want_absmax=False):
+def Attention(q, k, v, mask=None, rowsPerMask=1, want_absmax=False, kNew=None, vNew=None):
     """reference src/models/transformer.h:241-280 (inference: no dropout, weights not kept):
     softmax(bdot_legacy(q, k, false, true, 1/sqrt(dk)) + mask) then bdot_legacy(weights, v), in
-    one launch.  q: [batch*beam, heads, tgt, dk]; k, v: [batch(*beam), heads, len, dk]."""
-    q, k, v = _f32c(q, "Attention"), _f32c(k, "Attention"), _f32c(v, "Attention")
+    one launch.  q: [batch*beam, heads, tgt, dk]; k, v: [batch(*beam), heads, len, dk].
+    kNew, vNew [batch*beam*heads, dk]: key and value of the newest position of a decoding step;
+    they stand for position len - 1 and are also stored there in k and v (the concatenation onto
+    the cached positions, src/models/transformer.h:683-700)."""
+    q = _f32c(q, "Attention")
+    _abort_if(k.dtype != torch.float32 or v.dtype != torch.float32, "Attention expects float32, got {}", k.dtype)
+    if kNew is None:
+        k, v = k.contiguous(), v.contiguous()
+    else:
+        _abort_if(not (k.is_contiguous() and v.is_contiguous()), "Attention: the key/value cache must be contiguous{}", "")
+        kNew, vNew = _f32c(kNew, "Attention"), _f32c(vNew, "Attention")
     be = _backend_of(q)
     dk, m, L = q.shape[-1], q.shape[-2], k.shape[-2]
     _abort_if(k.shape[-1] != dk or tuple(v.shape) != tuple(k.shape), "Attention: key/value shapes {} {} vs dk {}",
@@ -148,6 +157,8 @@ def Attention(q, k, v, mask=None, rowsPerMask=1, want_absmax=False):
     st = be.lib.marian_hip_attention(q.data_ptr(), k.data_ptr(), v.data_ptr(),
                                      None if mask is None else mask.data_ptr(), n_masks, rowsPerMask,
                                      out.data_ptr(), batchQ, batchKV, m, L, dk, 1.0 / float(dk) ** 0.5,
-                                     None if omax is None else omax.data_ptr(), be.stream())
+                                     None if omax is None else omax.data_ptr(),
+                                     None if kNew is None else kNew.data_ptr(),
+                                     None if vNew is None else vNew.data_ptr(), be.stream())
     _lib.check(st, "Attention")
     return (out, omax) if want_absmax else out

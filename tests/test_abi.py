@@ -76,8 +76,9 @@ def test_argument_validation_returns_codes_not_aborts():
     assert lib.marian_hip_transpose0213(buf, buf + 64, 0, 2, 3, 4, None) == L.OK
     assert lib.marian_hip_bdot_legacy(buf, buf, buf, 2, 2, 0, 4, 4, 0, 0, 1.0, None) == L.ERR_SHAPE
     assert lib.marian_hip_bdot_legacy(buf, None, buf, 2, 2, 1, 4, 4, 0, 0, 1.0, None) == L.ERR_NULL
-    assert lib.marian_hip_attention(buf, buf, buf, None, 0, 0, buf, 2, 2, 1, 5000, 64, 0.125, None, None) == L.ERR_RANGE
-    assert lib.marian_hip_attention(buf, buf, None, None, 0, 0, buf, 2, 2, 1, 40, 64, 0.125, None, None) == L.ERR_NULL
+    assert lib.marian_hip_attention(buf, buf, buf, None, 0, 0, buf, 2, 2, 1, 5000, 64, 0.125, None, None, None, None) == L.ERR_RANGE
+    assert lib.marian_hip_attention(buf, buf, None, None, 0, 0, buf, 2, 2, 1, 40, 64, 0.125, None, None, None, None) == L.ERR_NULL
+    assert lib.marian_hip_attention(buf, buf, buf, None, 0, 0, buf, 4, 2, 1, 40, 64, 0.125, None, buf, buf, None) == L.ERR_SHAPE
     assert lib.marian_hip_int8_affine_shortlist(buf, buf, None, buf, 12, buf, 1, 64, 8, 1.0, 0, None) == L.ERR_SHAPE
     assert lib.marian_hip_int8_prepare_a(buf, buf, 4, 100, buf, 4096, None) == L.ERR_SHAPE
     assert lib.marian_hip_int8_prepare_a(buf, buf, 4096, 1024, buf, 16, None) == L.ERR_WORKSPACE

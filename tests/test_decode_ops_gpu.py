@@ -213,3 +213,22 @@ def test_absmax_outputs_of_layer_norm_and_attention(ops, integer, synth):
         got, aq = integer.affine_f32(t, Bq, None, absmax=tmax)
         want, aq_ref = integer.affine_f32(t, Bq, None)
         assert np.array_equal(aq.numpy(), aq_ref.numpy()) and np.array_equal(got.cpu().numpy(), want.cpu().numpy())
+
+
+@pytest.mark.parametrize("BH,T,dk", [(2048, 21, 64), (64, 1, 64), (48, 70, 20), (16, 9, 64)])
+def test_attention_with_cache_append(ops, synth, BH, T, dk):
+    """kNew / vNew stand for the last cached position and are stored there: same output bits as
+    appending by hand first, and the cache ends up holding the new rows."""
+    q = synth.normal(61 + T, 0, (BH, 1, dk), 1.0)
+    k = synth.normal(61 + T, 1, (BH, T, dk), 1.0)
+    v = synth.normal(61 + T, 2, (BH, T, dk), 1.0)
+    kn = synth.normal(61 + T, 3, (BH, dk), 1.0)
+    vn = synth.normal(61 + T, 4, (BH, dk), 1.0)
+    k2, v2 = k.copy(), v.copy()
+    k2[:, T - 1, :] = kn
+    v2[:, T - 1, :] = vn
+    want = ops.Attention(dev(q), dev(k2), dev(v2)).cpu().numpy()
+    kc, vc = dev(k), dev(v)
+    got = ops.Attention(dev(q), kc, vc, kNew=dev(kn), vNew=dev(vn)).cpu().numpy()
+    assert np.array_equal(got, want)
+    assert np.array_equal(kc.cpu().numpy(), k2) and np.array_equal(vc.cpu().numpy(), v2)
