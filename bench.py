@@ -409,7 +409,8 @@ def main():
         "metric": "int8 affine TOPS & % roofline; transformer-big int8 decode tokens/sec",
         "value": round(tops, 4), "unit": "TOPS", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5), "higher_is_better": True,
-        "scaling": "weak", "vs_baseline": None, "dtype": "int8 x int8 -> int32, fp32 epilogue",
+        "scaling": "weak", "vs_baseline": None, "dtype": "int8",
+        "dtype_detail": "int8 x int8 -> int32 accumulate, fp32 quantize and epilogue",
         "data": "synthetic",
         "config": {"workload": "transformer-base decode GEMM sweep: M in {1,4,16,64} x "
                                "{512x1536, 512x512, 512x2048, 2048x512, 512x32000}, "
