@@ -99,6 +99,25 @@ class Backend:
         self.lib = _lib.lib()
         self.workspace_bytes = int(self.lib.marian_hip_int8_workspace_bytes())
         self.workspace = torch.empty(self.workspace_bytes, dtype=torch.uint8, device=self.device)
+        # float32 weights are quantized on first use and remembered when this is Type.intgemm8:
+        # the counterpart of getGemmType() (reference src/tensors/backend.h:36-40) with the
+        # memoized packing of src/graph/expression_operators.cpp:564-598 (its FBGEMM branch
+        # packs a memoized float B the same way)
+        self.gemmType = None
+        self._memo = {}
+
+    def setGemmType(self, type_):
+        _abort_if(type_ not in (None, Type.intgemm8), "Unsupported type {} for Intgemm type??", type_)
+        self.gemmType = type_
+
+    def memoizedPrepareB(self, w):
+        """prepareB of a float32 parameter, once per (storage, shape, version)."""
+        key = (w.data_ptr(), tuple(w.shape), w._version)
+        hit = self._memo.get(key)
+        if hit is None:
+            hit = prepareB(w)
+            self._memo[key] = hit
+        return hit
 
     @classmethod
     def get(cls, device):
@@ -266,6 +285,15 @@ def multiply_i32(aQuant, bQuant, shortlist=None):
 
 # ---- graph-operator surface (reference src/graph/expression_operators.cpp) --------------------
 
+def _maybe_quantize_b(a, b):
+    """float32 B with the backend's gemm type set to intgemm8: quantize on first use, remembered"""
+    if isinstance(b, torch.Tensor) and b.dtype == torch.float32 and b.dim() == 2:
+        be = _backend_of(a)
+        if be.gemmType == Type.intgemm8:
+            return be.memoizedPrepareB(b)
+    return b
+
+
 def _float_b_unsupported(b):
     raise MarianRuntimeError(
         -2, "GPU-based GEMM only supports float types in the reference; this backend implements "
@@ -274,6 +302,7 @@ def _float_b_unsupported(b):
 
 def dot(a, b, transA=False, transB=False, scale=1.0):
     """reference src/graph/expression_operators.cpp:554-619: isIntgemm(b) selects the int8 path."""
+    b = _maybe_quantize_b(a, b)
     if isinstance(b, QTensor) and isIntgemm(b.type):
         return affineOrDot(a, b, None, transA, transB, scale)
     _float_b_unsupported(b)
@@ -281,6 +310,7 @@ def dot(a, b, transA=False, transB=False, scale=1.0):
 
 def affine(a, b, bias, transA=False, transB=False, scale=1.0):
     """reference src/graph/expression_operators.cpp:647-718."""
+    b = _maybe_quantize_b(a, b)
     if isinstance(b, QTensor) and isIntgemm(b.type):
         return affineOrDot(a, b, bias, transA, transB, scale)
     _float_b_unsupported(b)
@@ -290,6 +320,7 @@ def affineWithReluDropout(x, W, bias, dropProb=0.0):
     """reference src/graph/expression_operators.cpp:721-731 at inference (dropProb == 0): the
     reference runs affine() and then an in-place ReLU node; here the ReLU is the GEMM epilogue."""
     _abort_if(dropProb != 0.0, "dropout is a training feature; inference path expects dropProb == 0, got {}", dropProb)
+    W = _maybe_quantize_b(x, W)
     if isinstance(W, QTensor) and isIntgemm(W.type):
         return affineOrDot(x, W, bias, False, False, 1.0, relu=True)
     _float_b_unsupported(W)

@@ -460,6 +460,33 @@ def test_repeatable_and_input_untouched(integer, synth):
     assert np.array_equal(r1, r2) and np.array_equal(a.cpu().numpy(), A)
 
 
+def test_float_weights_are_quantized_once_when_the_gemm_type_is_intgemm8(integer, orc, synth):
+    """On-line quantization of a float32 model: with the backend's gemm type set, dot/affine take
+    float32 weights, quantize them on first use (same bytes as the offline packer) and reuse the
+    result; without it they refuse, as before."""
+    import torch
+    M, K, N = 9, 128, 72
+    A, W, bias = inputs(synth, 911, M, K, N)
+    be = integer.Backend.get("cuda:0")
+    dW = dev(W)
+    with pytest.raises(integer.MarianRuntimeError):
+        integer.affine(dev(A), dW, dev(bias))
+    be.setGemmType(integer.Type.intgemm8)
+    try:
+        out = integer.affine(dev(A), dW, dev(bias)).cpu().numpy()
+        q1 = be.memoizedPrepareB(dW)
+        assert np.array_equal(q1.numpy(), orc.prepare_b(W))
+        assert be.memoizedPrepareB(dW) is q1                      # remembered
+        want, _ = orc.affine(orc.prepare_a(A), orc.prepare_b(W), bias, M, K, N)
+        assert np.array_equal(out, want)
+        assert np.array_equal(integer.dot(dev(A), dW).cpu().numpy(),
+                              orc.affine(orc.prepare_a(A), orc.prepare_b(W), None, M, K, N)[0])
+        dW.mul_(2.0)                                               # a changed parameter is re-quantized
+        assert be.memoizedPrepareB(dW) is not q1
+    finally:
+        be.setGemmType(None)
+
+
 def test_type_errors_like_the_reference(integer):
     import torch
     from conftest import load
