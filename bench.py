@@ -217,7 +217,13 @@ class BigDecoder:
                 if ch:
                     x, xmax = x
         logits, _ = integer.affine_f32(x, *W["out"], absmax=xmax)
-        return logits if gemm_only else ops.logsoftmax(logits)
+        if gemm_only:
+            return logits
+        # log-probabilities, then the beam's n-best per sentence over beam x vocabulary
+        lp = ops.logsoftmax(logits)
+        ops.getNBestList(lp.view(self.beam, self.batch, self.V).transpose(0, 1).reshape(self.batch, 1, self.beam, self.V),
+                         self.beam)
+        return lp
 
 
 def capture(torch, fn):
@@ -513,8 +519,8 @@ def main():
         out["transformer_big_decode_full"] = {
             "what": "full decoder step through the host mirrors: 49 int8 affine calls + per layer "
                     "2 one-launch attentions (20 cached positions + the new one, appended by the call; "
-                    "40 source positions with mask), 3 skip-add+layer-norm; log-softmax over 32000; no beam "
-                    "search bookkeeping; the abs-max of every GEMM input is left by the kernel that "
+                    "40 source positions with mask), 3 skip-add+layer-norm; log-softmax over 32000 and n-best per "
+                    "sentence; no hypothesis bookkeeping; the abs-max of every GEMM input is left by the kernel that "
                     "produced it",
             "ms_per_step": round(fdt / n * 1e3, 4),
             "ms_per_step_unchained": round(udt / n * 1e3, 4),

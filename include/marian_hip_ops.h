@@ -90,6 +90,17 @@ int marian_hip_attention(const float* q, float* k, float* v, const float* mask, 
                          int64_t m, int64_t len, int64_t dk, float scale, float* absmax_out,
                          const float* k_new, const float* v_new, void* stream);
 
+/*
+ * Replaces NthElement::getNBestList, reference src/translator/nth_element.cpp:26-67 (CPU) and
+ * src/translator/nth_element.cu (GPU): for each of dimBatch rows of rowLen = beam * vocabulary
+ * scores, the N best scores in descending order and their keys = absolute positions
+ * row * rowLen + index (uint32).  Equal scores come out lowest index first (the reference's
+ * partial_sort leaves that order unspecified).  1 <= N <= 16, N <= rowLen.
+ * outScores, outKeys: dimBatch * N values each, on the device.
+ */
+int marian_hip_nbest(const float* scores, int64_t dimBatch, int64_t rowLen, int64_t N,
+                     float* outScores, uint32_t* outKeys, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

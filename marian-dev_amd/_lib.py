@@ -36,6 +36,7 @@ SIGNATURES = {
     "marian_hip_logsoftmax": (_i, [_vp, _vp, _i64, _i64, _vp]),
     "marian_hip_transpose0213": (_i, [_vp, _vp, _i64, _i64, _i64, _i64, _vp]),
     "marian_hip_bdot_legacy": (_i, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i, _i, _f, _vp]),
+    "marian_hip_nbest": (_i, [_vp, _i64, _i64, _i64, _vp, _vp, _vp]),
     "marian_hip_attention": (_i, [_vp, _vp, _vp, _vp, _i64, _i64, _vp, _i64, _i64, _i64, _i64, _i64,
                                   _f, _vp, _vp, _vp, _vp]),
 }

@@ -380,6 +380,341 @@ __global__ __launch_bounds__(256) void attention_kernel(const float* __restrict_
   }
 }
 
+// ---------------------------------------------------------------- n-best
+// One workgroup of 1024 threads per row; a thread looks at every 1024th element (or group of
+// four).  Scores are ordered by (value descending, index ascending).
+//   1. every thread finds the best of its elements, every wave the best of its threads'; the N-th
+//      best of these 16 is a bound T: at least N elements of the row are at or before T, so
+//      nothing after T can be among the N best;
+//   2. the row is read again (from cache) and the elements at or before T - usually little more
+//      than N of them - are collected in LDS, one per thread at most;
+//   3. the N best of the collected ones are drawn one at a time.
+// If more than 1024 elements pass the bound (large values concentrated in a few threads, or
+// massive ties) every thread instead keeps the KEEP >= N best of its elements in registers and
+// the draw pops them one by one.
+constexpr int kNbestMax = 16;
+
+__device__ __forceinline__ bool nbest_before(float v, unsigned i, float w, unsigned j) {
+  return v > w || (v == w && i < j);
+}
+
+struct NbestShared {
+  float val[16];
+  unsigned idx[16];
+  int who[16];
+  int winner;
+  int count;
+  float cand_val[1024];
+  unsigned cand_idx[1024];
+};
+
+// Workgroup-wide best of one (value, index) per thread; every thread gets the result and the id of
+// the thread that held it.
+__device__ __forceinline__ void nbest_arg_best(float v, unsigned i, NbestShared& sh, float& gv, unsigned& gi,
+                                               int& gw) {
+  const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
+  float bv = v;
+  unsigned bi = i;
+  int bw = tid;
+#pragma unroll
+  for(int o = 32; o > 0; o >>= 1) {
+    const float ov = __shfl_xor(bv, o, 64);
+    const unsigned oi = (unsigned)__shfl_xor((int)bi, o, 64);
+    const int ow = __shfl_xor(bw, o, 64);
+    if(nbest_before(ov, oi, bv, bi)) {
+      bv = ov; bi = oi; bw = ow;
+    }
+  }
+  __syncthreads();   // the previous round's results have been read
+  if(lane == 0) {
+    sh.val[wave] = bv; sh.idx[wave] = bi; sh.who[wave] = bw;
+  }
+  __syncthreads();
+  gv = sh.val[0]; gi = sh.idx[0]; gw = sh.who[0];
+#pragma unroll
+  for(int w = 1; w < 16; ++w)
+    if(nbest_before(sh.val[w], sh.idx[w], gv, gi)) {
+      gv = sh.val[w]; gi = sh.idx[w]; gw = sh.who[w];
+    }
+}
+
+// Wave 0 only: draws the n best of the `count` <= 1024 (value, index) pairs in lv/li (LDS),
+// sixteen per lane, without workgroup barriers.  emit(n, value, index) is called by lane 0.
+template <typename Emit>
+__device__ __forceinline__ void nbest_wave_draw(const float* lv, const unsigned* li, int count, int n,
+                                                Emit emit) {
+  const int lane = threadIdx.x % 64;
+  const float ninf = -__builtin_inff();
+  const unsigned none = 0xFFFFFFFFu;
+  float v[16];
+  unsigned ix[16];
+#pragma unroll
+  for(int j = 0; j < 16; ++j) {
+    const int e = j * 64 + lane;
+    v[j] = e < count ? lv[e] : ninf;
+    ix[j] = e < count ? li[e] : none;
+  }
+  for(int r = 0; r < n; ++r) {
+    float bv = v[0];
+    unsigned bi = ix[0];
+#pragma unroll
+    for(int j = 1; j < 16; ++j)
+      if(nbest_before(v[j], ix[j], bv, bi)) {
+        bv = v[j]; bi = ix[j];
+      }
+    float gv = bv;
+    unsigned gi = bi;
+#pragma unroll
+    for(int o = 32; o > 0; o >>= 1) {
+      const float ov = __shfl_xor(gv, o, 64);
+      const unsigned oi = (unsigned)__shfl_xor((int)gi, o, 64);
+      if(nbest_before(ov, oi, gv, gi)) {
+        gv = ov; gi = oi;
+      }
+    }
+    if(lane == 0) emit(r, gv, gi);
+    // the holder drops it (indices are unique, so at most one entry matches)
+#pragma unroll
+    for(int j = 0; j < 16; ++j)
+      if(ix[j] == gi && gi != none) {
+        v[j] = ninf; ix[j] = none;
+      }
+  }
+}
+
+template <int KEEP>
+__global__ __launch_bounds__(1024) void nbest_kernel(const float* __restrict__ scores, long long rowLen, int N,
+                                                     float* __restrict__ outScores,
+                                                     unsigned* __restrict__ outKeys) {
+  __shared__ NbestShared sh;
+  const long long row = blockIdx.x;
+  const float* x = scores + row * rowLen;
+  const int tid = threadIdx.x;
+  const float ninf = -__builtin_inff();
+  const unsigned none = 0xFFFFFFFFu;
+
+  // 1. best element of this thread, then the N-th best of those
+  // (both scans keep sixteen loads in flight per thread; one load per dependent step would
+  // cost a memory latency per element)
+  float mv = ninf;
+  unsigned mi = none;
+  const bool vec = (rowLen % 4) == 0 && (reinterpret_cast<uintptr_t>(x) % 16) == 0;
+  const long long n4 = rowLen / 4;
+  if(vec) {   // 16-byte loads, eight in flight: elements 4 * (t + 1024 * j) .. + 3, in index order
+    const v4f* x4 = reinterpret_cast<const v4f*>(x);
+    auto take = [&](float v, unsigned i) {
+      if(nbest_before(v, i, mv, mi)) {
+        mv = v; mi = i;
+      }
+    };
+    long long i = tid;
+    for(; i + 7 * 1024 < n4; i += 8 * 1024) {
+      v4f v[8];
+#pragma unroll
+      for(int u = 0; u < 8; ++u) v[u] = x4[i + u * 1024];
+#pragma unroll
+      for(int u = 0; u < 8; ++u) {
+        const unsigned b = (unsigned)(4 * (i + u * 1024));
+        take(v[u].x, b); take(v[u].y, b + 1); take(v[u].z, b + 2); take(v[u].w, b + 3);
+      }
+    }
+    for(; i < n4; i += 1024) {
+      const v4f v = x4[i];
+      const unsigned b = (unsigned)(4 * i);
+      take(v.x, b); take(v.y, b + 1); take(v.z, b + 2); take(v.w, b + 3);
+    }
+  } else {
+    long long i = tid;
+    for(; i + 15 * 1024 < rowLen; i += 16 * 1024) {
+      float v[16];
+#pragma unroll
+      for(int u = 0; u < 16; ++u) v[u] = x[i + u * 1024];
+#pragma unroll
+      for(int u = 0; u < 16; ++u)
+        if(nbest_before(v[u], (unsigned)(i + u * 1024), mv, mi)) {
+          mv = v[u]; mi = (unsigned)(i + u * 1024);
+        }
+    }
+    for(; i < rowLen; i += 1024) {
+      const float v = x[i];
+      if(nbest_before(v, (unsigned)i, mv, mi)) {
+        mv = v; mi = (unsigned)i;
+      }
+    }
+  }
+  float tv = ninf;
+  unsigned ti = none;
+  if(N <= 4) {
+    // Bound for short lists: the N-th best of the 16 per-wave bests (16 distinct elements, so at
+    // least N elements of the row are at or before it).  Every thread derives it from the 16
+    // values itself; a wave without elements contributes "none", which sorts last.
+    float wv = mv;
+    unsigned wi = mi;
+#pragma unroll
+    for(int o = 32; o > 0; o >>= 1) {
+      const float ov = __shfl_xor(wv, o, 64);
+      const unsigned oi = (unsigned)__shfl_xor((int)wi, o, 64);
+      if(nbest_before(ov, oi, wv, wi)) {
+        wv = ov; wi = oi;
+      }
+    }
+    if(tid % 64 == 0) {
+      sh.val[tid / 64] = wv; sh.idx[tid / 64] = wi;
+    }
+    __syncthreads();
+    float lv[16];
+    unsigned li[16];
+#pragma unroll
+    for(int w = 0; w < 16; ++w) {
+      lv[w] = sh.val[w]; li[w] = sh.idx[w];
+    }
+    for(int n = 0; n < N; ++n) {
+      tv = lv[0]; ti = li[0];
+#pragma unroll
+      for(int w = 1; w < 16; ++w)
+        if(nbest_before(lv[w], li[w], tv, ti)) {
+          tv = lv[w]; ti = li[w];
+        }
+#pragma unroll
+      for(int w = 0; w < 16; ++w)
+        if(li[w] == ti) {
+          lv[w] = ninf; li[w] = none;
+        }
+    }
+  } else {
+    // Bound for longer lists: the N-th best of the 1024 per-thread bests, found by wave 0 (the
+    // per-wave bests would leave too many candidates).
+    sh.cand_val[tid] = mv;
+    sh.cand_idx[tid] = mi;
+    __syncthreads();
+    if(tid < 64)
+      nbest_wave_draw(sh.cand_val, sh.cand_idx, 1024, N, [&](int r, float v, unsigned i) {
+        if(r == N - 1) {
+          sh.val[0] = v; sh.idx[0] = i;
+        }
+      });
+    __syncthreads();
+    tv = sh.val[0];
+    ti = sh.idx[0];
+    __syncthreads();   // before the candidate list is reused below
+  }
+  // (with fewer than N holders of an element the bound is "none" and everything passes)
+
+  // 2. collect what is at or before the bound
+  if(tid == 0) sh.count = 0;
+  __syncthreads();
+  auto collect = [&](float v, unsigned i) {
+    if(!nbest_before(tv, ti, v, i)) {
+      const int slot = atomicAdd(&sh.count, 1);
+      if(slot < 1024) {
+        sh.cand_val[slot] = v; sh.cand_idx[slot] = i;
+      }
+    }
+  };
+  if(vec) {
+    const v4f* x4 = reinterpret_cast<const v4f*>(x);
+    long long i = tid;
+    for(; i + 7 * 1024 < n4; i += 8 * 1024) {
+      v4f v[8];
+#pragma unroll
+      for(int u = 0; u < 8; ++u) v[u] = x4[i + u * 1024];
+#pragma unroll
+      for(int u = 0; u < 8; ++u) {
+        const unsigned b = (unsigned)(4 * (i + u * 1024));
+        collect(v[u].x, b); collect(v[u].y, b + 1); collect(v[u].z, b + 2); collect(v[u].w, b + 3);
+      }
+    }
+    for(; i < n4; i += 1024) {
+      const v4f v = x4[i];
+      const unsigned b = (unsigned)(4 * i);
+      collect(v.x, b); collect(v.y, b + 1); collect(v.z, b + 2); collect(v.w, b + 3);
+    }
+  } else {
+    long long i = tid;
+    for(; i + 15 * 1024 < rowLen; i += 16 * 1024) {
+      float v[16];
+#pragma unroll
+      for(int u = 0; u < 16; ++u) v[u] = x[i + u * 1024];
+#pragma unroll
+      for(int u = 0; u < 16; ++u) collect(v[u], (unsigned)(i + u * 1024));
+    }
+    for(; i < rowLen; i += 1024) collect(x[i], (unsigned)i);
+  }
+  __syncthreads();
+  const int count = sh.count;
+
+  if(count <= 1024) {
+    // 3. the N best of the collected elements: a handful, drawn by one thread; more, by wave 0
+    if(count <= 64) {
+      if(tid == 0) {
+        float pv = __builtin_inff();
+        unsigned pi = 0;
+        for(int r = 0; r < N; ++r) {   // best of those strictly after the previous pick
+          float bv = ninf;
+          unsigned bi = none;
+          for(int c = 0; c < count; ++c) {
+            const float v = sh.cand_val[c];
+            const unsigned i = sh.cand_idx[c];
+            const bool after_prev = r == 0 || nbest_before(pv, pi, v, i);
+            if(after_prev && nbest_before(v, i, bv, bi)) {
+              bv = v; bi = i;
+            }
+          }
+          outScores[row * N + r] = bv;
+          outKeys[row * N + r] = (unsigned)(row * rowLen) + bi;
+          pv = bv; pi = bi;
+        }
+      }
+    } else if(tid < 64) {
+      nbest_wave_draw(sh.cand_val, sh.cand_idx, count, N, [&](int r, float v, unsigned i) {
+        outScores[row * N + r] = v;
+        outKeys[row * N + r] = (unsigned)(row * rowLen) + i;
+      });
+    }
+    return;
+  }
+
+  // too many at or before the bound: per-thread sorted lists of the KEEP best, popped by the draw
+  float val[KEEP];
+  unsigned idx[KEEP];
+#pragma unroll
+  for(int j = 0; j < KEEP; ++j) {
+    val[j] = ninf;
+    idx[j] = none;
+  }
+  for(long long i = tid; i < rowLen; i += 1024) {
+    const float v = x[i];
+    if(nbest_before(v, (unsigned)i, val[KEEP - 1], idx[KEEP - 1])) {
+      val[KEEP - 1] = v;
+      idx[KEEP - 1] = (unsigned)i;
+#pragma unroll
+      for(int j = KEEP - 1; j > 0; --j) {
+        if(nbest_before(val[j], idx[j], val[j - 1], idx[j - 1])) {
+          const float sv = val[j]; val[j] = val[j - 1]; val[j - 1] = sv;
+          const unsigned si = idx[j]; idx[j] = idx[j - 1]; idx[j - 1] = si;
+        }
+      }
+    }
+  }
+  for(int n = 0; n < N; ++n) {
+    float gv; unsigned gi; int who;
+    nbest_arg_best(val[0], idx[0], sh, gv, gi, who);
+    if(tid == 0) {
+      outScores[row * N + n] = gv;
+      outKeys[row * N + n] = (unsigned)(row * rowLen) + gi;
+    }
+    if(tid == who) {   // pop the head
+#pragma unroll
+      for(int j = 0; j < KEEP - 1; ++j) {
+        val[j] = val[j + 1];
+        idx[j] = idx[j + 1];
+      }
+      val[KEEP - 1] = ninf;
+      idx[KEEP - 1] = none;
+    }
+  }
+}
+
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) % 16) == 0; }
 inline bool aligned4(const void* p) { return (reinterpret_cast<uintptr_t>(p) % 4) == 0; }
 
@@ -521,6 +856,24 @@ int marian_hip_attention(const float* q, float* k, float* v, const float* mask, 
   hipLaunchKernelGGL(attention_kernel, dim3((unsigned)((rows_total + 3) / 4)), dim3(256), lds, st, q, k, v,
                      k_new, v_new, mask, (long long)n_masks, (long long)rows_per_mask, out, rows_total,
                      (long long)batchKV, (int)m, (int)len, (int)dk, scale, absmax_out);
+  MH_HIP(hipGetLastError());
+  return MARIAN_HIP_OK;
+}
+
+int marian_hip_nbest(const float* scores, int64_t dimBatch, int64_t rowLen, int64_t N,
+                     float* outScores, uint32_t* outKeys, void* stream) {
+  if(dimBatch < 0 || rowLen <= 0 || N <= 0 || N > kNbestMax || N > rowLen) return MARIAN_HIP_ERR_SHAPE;
+  if(dimBatch == 0) return MARIAN_HIP_OK;
+  if(!scores || !outScores || !outKeys) return MARIAN_HIP_ERR_NULL;
+  if(dimBatch * rowLen > 4294967295LL) return MARIAN_HIP_ERR_RANGE;   // keys are uint32
+  if(!aligned4(scores) || !aligned4(outScores) || !aligned4(outKeys)) return MARIAN_HIP_ERR_ALIGN;
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  if(N <= 4)
+    hipLaunchKernelGGL(nbest_kernel<4>, dim3((unsigned)dimBatch), dim3(1024), 0, st, scores, (long long)rowLen, (int)N, outScores, outKeys);
+  else if(N <= 8)
+    hipLaunchKernelGGL(nbest_kernel<8>, dim3((unsigned)dimBatch), dim3(1024), 0, st, scores, (long long)rowLen, (int)N, outScores, outKeys);
+  else
+    hipLaunchKernelGGL(nbest_kernel<16>, dim3((unsigned)dimBatch), dim3(1024), 0, st, scores, (long long)rowLen, (int)N, outScores, outKeys);
   MH_HIP(hipGetLastError());
   return MARIAN_HIP_OK;
 }

@@ -162,3 +162,18 @@ def Attention(q, k, v, mask=None, rowsPerMask=1, want_absmax=False, kNew=None, v
                                      None if vNew is None else vNew.data_ptr(), be.stream())
     _lib.check(st, "Attention")
     return (out, omax) if want_absmax else out
+
+
+def getNBestList(scores, N):
+    """reference src/translator/nth_element.cpp:26-67: scores [dimBatch, 1, beam, vocab]; returns
+    (pathScores, keys) of dimBatch * N entries, keys = position in the flattened tensor."""
+    scores = _f32c(scores, "getNBestList")
+    be = _backend_of(scores)
+    dimBatch = scores.shape[0]
+    rowLen = scores.numel() // dimBatch if dimBatch else 0
+    vals = torch.empty(dimBatch * N, dtype=torch.float32, device=scores.device)
+    keys = torch.empty(dimBatch * N, dtype=torch.int32, device=scores.device)
+    st = be.lib.marian_hip_nbest(scores.data_ptr(), dimBatch, rowLen, N, vals.data_ptr(), keys.data_ptr(),
+                                 be.stream())
+    _lib.check(st, "getNBestList")
+    return vals, keys

@@ -112,10 +112,15 @@ class Output:
         return out
 
     def bestWords(self, input, k=1):
-        """top-k per row, returned as (scores, vocabulary ids): shortlist coordinates are mapped
-        back like Shortlist::reverseMap does for the beam search (src/translator/beam_search.cpp)"""
+        """the k best words per row (k <= 16), returned as (scores, vocabulary ids): shortlist
+        coordinates are mapped back like Shortlist::reverseMap does for the beam search
+        (src/translator/beam_search.cpp); selection by the n-best kernel of the library"""
+        from . import ops
         logits = self.applyAsLogits(input)
-        scores, pos = torch.topk(logits.reshape(-1, logits.shape[-1]), k, dim=-1)
+        rows, cols = logits.numel() // logits.shape[-1], logits.shape[-1]
+        scores, keys = ops.getNBestList(logits.reshape(rows, 1, 1, cols), k)   # one "batch" entry per row
+        scores = scores.reshape(rows, k)
+        pos = keys.reshape(rows, k).to(torch.int64) - torch.arange(rows, device=logits.device)[:, None] * cols
         if self.shortlist_ is not None:
             pos = self.shortlist_.getIndicesExpr(input.device).to(torch.int64)[pos]
         return scores, pos

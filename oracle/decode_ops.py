@@ -38,6 +38,8 @@ def lib():
         L.oracle_bdot_legacy.restype = None
         L.oracle_bdot_legacy.argtypes = [fp, fp, fp, i64, i64, i64, i64, i64, c.c_int, c.c_int,
                                          c.c_float]
+        L.oracle_nbest.restype = None
+        L.oracle_nbest.argtypes = [fp, i64, i64, i64, fp, c.POINTER(c.c_uint32)]
         _lib = L
     return _lib
 
@@ -110,3 +112,14 @@ def bdot_legacy(a, b, transA=False, transB=False, scalar=1.0):
     lib().oracle_bdot_legacy(_p(out), _p(a), _p(b), batchA, batchB, m, n, k, int(transA),
                              int(transB), np.float32(scalar))
     return out
+
+
+def nbest(scores, N):
+    scores = _f32(scores)
+    dimBatch = scores.shape[0]
+    rowLen = scores.size // dimBatch
+    vals = np.empty(dimBatch * N, dtype=np.float32)
+    keys = np.empty(dimBatch * N, dtype=np.uint32)
+    lib().oracle_nbest(_p(scores), dimBatch, rowLen, N, _p(vals),
+                       keys.ctypes.data_as(ctypes.POINTER(ctypes.c_uint32)))
+    return vals, keys

@@ -14,12 +14,14 @@
  *   oracle_logsoftmax      reference src/tensors/cpu/tensor_operators.cpp:474-509
  *   oracle_transpose0213   reference src/tensors/cpu/tensor_operators.cpp:220-246
  *   oracle_bdot_legacy     reference src/tensors/cpu/prod.cpp:233-330 (ProdBatchedLegacy, beta = 0)
+ *   oracle_nbest           reference src/translator/nth_element.cpp:26-67 (getNBestList)
  *
  * Pinning status (tests/test_decode_ops.py): every function is checked against float64 closed
  * forms in numpy and against invariants that a dropped term or a wrong index would break
  * (softmax rows sum to one and are shift invariant; layer-norm output has mean beta and
  * variance gamma^2 for constant gamma/beta; transposing twice is the identity; the batched
- * product against numpy matmul including the batch broadcast i % batchA, i % batchB): pinned.
+ * product against numpy matmul including the batch broadcast i % batchA, i % batchB; the n-best
+ * list against a full numpy sort): pinned.
  */
 #include <math.h>
 #include <stddef.h>
@@ -133,5 +135,27 @@ void oracle_bdot_legacy(float* C, const float* A, const float* B, int64_t batchA
         }
         c[r * n + q] = scalar * s;
       }
+  }
+}
+
+/* For each of dimBatch rows of rowLen scores: the N best in descending order (selection by
+ * repeated maximum; equal scores lowest index first, an order the reference's partial_sort leaves
+ * open) and their keys = row * rowLen + index. */
+void oracle_nbest(const float* scores, int64_t dimBatch, int64_t rowLen, int64_t N,
+                  float* outScores, uint32_t* outKeys) {
+  for(int64_t b = 0; b < dimBatch; ++b) {
+    const float* x = scores + b * rowLen;
+    for(int64_t n = 0; n < N; ++n) {
+      int64_t best = -1;
+      for(int64_t i = 0; i < rowLen; ++i) {
+        int taken = 0;
+        for(int64_t p = 0; p < n; ++p)
+          if(outKeys[b * N + p] == (uint32_t)(b * rowLen + i)) taken = 1;
+        if(taken) continue;
+        if(best < 0 || x[i] > x[best]) best = i;
+      }
+      outScores[b * N + n] = x[best];
+      outKeys[b * N + n] = (uint32_t)(b * rowLen + best);
+    }
   }
 }

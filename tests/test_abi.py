@@ -26,7 +26,8 @@ def test_header_declares_expected_entry_points():
                  "marian_hip_int8_prepare_b_quantized_transposed", "marian_hip_int8_affine",
                  "marian_hip_int8_affine_shortlist", "marian_hip_int8_multiply_i32",
                  "marian_hip_layer_norm", "marian_hip_softmax", "marian_hip_logsoftmax",
-                 "marian_hip_transpose0213", "marian_hip_bdot_legacy", "marian_hip_attention"):
+                 "marian_hip_transpose0213", "marian_hip_bdot_legacy", "marian_hip_attention",
+                 "marian_hip_nbest"):
         assert must in names
 
 
@@ -77,6 +78,8 @@ def test_argument_validation_returns_codes_not_aborts():
     assert lib.marian_hip_bdot_legacy(buf, buf, buf, 2, 2, 0, 4, 4, 0, 0, 1.0, None) == L.ERR_SHAPE
     assert lib.marian_hip_bdot_legacy(buf, None, buf, 2, 2, 1, 4, 4, 0, 0, 1.0, None) == L.ERR_NULL
     assert lib.marian_hip_attention(buf, buf, buf, None, 0, 0, buf, 2, 2, 1, 5000, 64, 0.125, None, None, None, None) == L.ERR_RANGE
+    assert lib.marian_hip_nbest(buf, 2, 100, 17, buf, buf, None) == L.ERR_SHAPE
+    assert lib.marian_hip_nbest(buf, 2, 100, 4, None, buf, None) == L.ERR_NULL
     assert lib.marian_hip_attention(buf, buf, None, None, 0, 0, buf, 2, 2, 1, 40, 64, 0.125, None, None, None, None) == L.ERR_NULL
     assert lib.marian_hip_attention(buf, buf, buf, None, 0, 0, buf, 4, 2, 1, 40, 64, 0.125, None, buf, buf, None) == L.ERR_SHAPE
     assert lib.marian_hip_int8_affine_shortlist(buf, buf, None, buf, 12, buf, 1, 64, 8, 1.0, 0, None) == L.ERR_SHAPE

@@ -232,3 +232,44 @@ def test_attention_with_cache_append(ops, synth, BH, T, dk):
     got = ops.Attention(dev(q), kc, vc, kNew=dev(kn), vNew=dev(vn)).cpu().numpy()
     assert np.array_equal(got, want)
     assert np.array_equal(kc.cpu().numpy(), k2) and np.array_equal(vc.cpu().numpy(), v2)
+
+
+@pytest.mark.parametrize("batch,beam,V,N", [(32, 4, 32000, 4), (1, 1, 32000, 12), (7, 6, 1000, 6), (3, 1, 20, 16),
+                                            (2, 2, 8, 16), (5, 4, 3000, 1)])
+def test_nbest(ops, chk, synth, batch, beam, V, N):
+    x = synth.normal(71 + V, 0, (batch, 1, beam, V), 2.0)
+    vals, keys = ops.getNBestList(dev(x), N)
+    flat = x.reshape(batch, -1)
+    order = np.argsort(-flat, axis=1, kind="stable")[:, :N]
+    assert np.array_equal(vals.cpu().numpy().reshape(batch, N), np.take_along_axis(flat, order, 1))
+    want_keys = order + np.arange(batch)[:, None] * flat.shape[1]
+    assert np.array_equal(keys.cpu().numpy().view(np.uint32).reshape(batch, N).astype(np.int64), want_keys)
+    if batch * beam * V <= 20000:
+        cv, ck = chk.nbest(x, N)
+        assert np.array_equal(vals.cpu().numpy(), cv) and np.array_equal(keys.cpu().numpy().view(np.uint32), ck)
+
+
+def test_nbest_ties_lowest_index_first(ops):
+    t = np.zeros((2, 5000), np.float32)
+    t[0, [4000, 17, 2048]] = 3.0
+    t[1, :] = -1.0
+    vals, keys = ops.getNBestList(dev(t), 4)
+    k = keys.cpu().numpy().view(np.uint32).reshape(2, 4)
+    assert k[0].tolist() == [17, 2048, 4000, 0] and k[1].tolist() == [5000, 5001, 5002, 5003]
+
+
+@pytest.mark.parametrize("N", [3, 8, 16])
+def test_nbest_when_one_thread_holds_the_best_elements(ops, synth, N):
+    """Every 1024th element is large (the kernel gives those to one thread), so the bound taken
+    from per-thread bests is loose and many candidates pass; and a row of equal scores, where all
+    elements pass.  Results still equal a full sort."""
+    x = synth.normal(81, 0, (3, 1, 1, 40000), 1.0)
+    x[0, 0, 0, ::1024] += np.float32(50.0)
+    x[1, 0, 0, 5::1024] += np.float32(50.0)
+    x[2] = np.float32(0.25)
+    vals, keys = ops.getNBestList(dev(x), N)
+    flat = x.reshape(3, -1)
+    order = np.argsort(-flat, axis=1, kind="stable")[:, :N]
+    assert np.array_equal(vals.cpu().numpy().reshape(3, N), np.take_along_axis(flat, order, 1))
+    assert np.array_equal(keys.cpu().numpy().view(np.uint32).reshape(3, N).astype(np.int64),
+                          order + np.arange(3)[:, None] * flat.shape[1])

@@ -117,3 +117,18 @@ def test_bdot_legacy(ops, tA, tB):
     A1 = a1.transpose(0, 2, 1) if tA else a1
     want3 = np.stack([A1[0].astype(f64) @ B[i].astype(f64) for i in range(batch)])
     assert close(ops.bdot_legacy(a1, b, tA, tB, 1.0), want3, 1e-5, 1e-6)
+
+
+def test_nbest_against_full_sort(ops):
+    rng = np.random.default_rng(9)
+    x = rng.normal(0, 1, (5, 1, 3, 400)).astype(np.float32)
+    vals, keys = ops.nbest(x, 6)
+    flat = x.reshape(5, -1)
+    order = np.argsort(-flat, axis=1, kind="stable")[:, :6]
+    assert np.array_equal(vals.reshape(5, 6), np.take_along_axis(flat, order, 1))
+    assert np.array_equal(keys.reshape(5, 6).astype(np.int64), order + np.arange(5)[:, None] * flat.shape[1])
+    # equal scores: lowest index first
+    t = np.zeros((1, 10), np.float32)
+    t[0, [7, 2, 5]] = 1.0
+    v, k = ops.nbest(t, 4)
+    assert k.tolist() == [2, 5, 7, 0] and v.tolist() == [1.0, 1.0, 1.0, 0.0]
