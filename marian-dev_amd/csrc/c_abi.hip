@@ -134,10 +134,10 @@ int launch_stream32(const GemmArgs& a, const FusedSrc& f, hipStream_t st) {
   int m_tiles = MODE == kFusedAll ? 1 : (a.M + MT32 * 32 - 1) / (MT32 * 32);
   GemmArgs a2 = a;
   if(a.absmax_out) {   // eight slots per workgroup, one per wave
-    if((long long)blocks * m_tiles * kStream32Waves <= kAbsmaxSlots) t_absmax_written = true;
+    if((long long)blocks * m_tiles * Cfg::kWaves <= kAbsmaxSlots) t_absmax_written = true;
     else a2.absmax_out = nullptr;
   }
-  hipLaunchKernelGGL(kernel, dim3(blocks, m_tiles), dim3(kStream32Threads), lds, st, a2, f.A,
+  hipLaunchKernelGGL(kernel, dim3(blocks, m_tiles), dim3(Cfg::kThreads), lds, st, a2, f.A,
                      f.aq_out, f.partials, f.n_partials);
   MH_HIP(hipGetLastError());
   return MARIAN_HIP_OK;

@@ -5,8 +5,8 @@
 // lane l of a wave loads 16 consecutive K bytes of weight row n0 + l % 32, which is the row
 // operand layout of v_mfma_i32_32x32x32_i8, so they need no LDS staging or transposition.  The
 // small quantized activations are the column operand; a workgroup keeps them in LDS in operand
-// order (within a fragment the 32 rows of a K chunk are XOR-permuted by the chunk number, which
-// spreads the quantizer's 4-byte writes over the LDS banks and keeps the fragment reads
+// order (within a fragment the 32 rows of a K chunk are XOR-permuted by a key of the chunk number,
+// which spreads the quantizer's 4-byte writes over the LDS banks and keeps the fragment reads
 // conflict free).  The 8 waves of a workgroup are arranged WN (different weight rows) x KW (different K
 // ranges of the same rows); the KW partial sums are added through LDS (exact in any order).
 //
@@ -26,11 +26,14 @@ namespace marian_hip {
 
 typedef int v16i_s __attribute__((ext_vector_type(16)));
 
-constexpr int kStream32Waves = 8;
-constexpr int kStream32Threads = kStream32Waves * kWave;
 constexpr int kFusedMaxElems = 32768;   // fp32 activations a workgroup holds in registers
-constexpr int kFusedGroups = kFusedMaxElems / 16 / kStream32Threads;   // 16-value groups per thread
 constexpr int kPrequant = 0, kFusedAll = 1, kFusedTiled = 2;            // MODE
+
+// The 32 rows of 16-byte chunk c16 of the activations are stored XOR-permuted by this key.  Any key
+// leaves a fragment read (32 consecutive slots, permuted) free of bank conflicts; this one makes
+// the quantizer's dword writes hit eight different slots (mod 8) for the eight quads that cover
+// 32 consecutive chunks of one row, and for quads in neighbouring rows at the same chunk.
+__device__ __forceinline__ int stream32_row_key(int c16) { return (c16 ^ (c16 >> 2)) & 7; }
 
 // MT32: 32-row activation tiles per workgroup (blockIdx.y walks M in steps of 32 * MT32; the
 // fused form needs all of M in one workgroup).  PW: 32-byte K sub-steps (weight loads in flight)
@@ -39,7 +42,9 @@ constexpr int kPrequant = 0, kFusedAll = 1, kFusedTiled = 2;            // MODE
 // that no wave is left with sub-steps past the end of K.
 template <int MT32, int WN, int KW, int PW_>
 struct Stream32Cfg {
-  static_assert(WN * KW == kStream32Waves, "eight waves");
+  static constexpr int kWaves = WN * KW;
+  static constexpr int kThreads = kWaves * kWave;
+  static_assert(kWaves == 8, "eight waves");
   static constexpr int kColsPerBlock = WN * 32;
   static constexpr int PW = PW_;
   static constexpr int CS = PW * KW;
@@ -47,18 +52,21 @@ struct Stream32Cfg {
   static constexpr int kReduceBytes = (KW - 1) * WN * MT32 * 4 * kFragBytes;  // v16i per lane
   static constexpr int kLdsBytes = kStageBytes > kReduceBytes ? kStageBytes : kReduceBytes;
   static_assert(PW >= 1 && PW <= 8 && kStageBytes <= 64 * 1024, "chunk size");
-  static_assert(CS * MT32 * 64 % kStream32Threads == 0, "stage must divide over the threads");
+  static_assert(CS * MT32 * 64 % kThreads == 0, "stage must divide over the threads");
+  static_assert(CS % 2 == 0, "a quad of lanes quantizes four 16-byte chunks of one row");
 };
 
 // Dynamic LDS: kFusedAll holds all of K (32 * MT32 * K bytes); otherwise one chunk (kStageBytes);
 // both at least kReduceBytes.  partials: n_partials (1..2048) abs-max values (kFusedTiled only).
 template <int MT32, int WN, int KW, int PW, int MODE>
-__global__ __launch_bounds__(kStream32Threads) void gemm_stream32_kernel(GemmArgs args,
+__global__ __launch_bounds__(WN * KW * kWave) void gemm_stream32_kernel(GemmArgs args,
                                                                         const float* A,
                                                                         int8_t* aq_out,
                                                                         const float* partials,
                                                                         int n_partials) {
   using Cfg = Stream32Cfg<MT32, WN, KW, PW>;
+  constexpr int kStream32Waves = Cfg::kWaves, kStream32Threads = Cfg::kThreads;
+  constexpr int kFusedGroups = kFusedMaxElems / 16 / kStream32Threads;   // 16-value groups per thread
   constexpr bool FUSED = MODE == kFusedAll;
   constexpr bool TILED = MODE == kFusedTiled;
   extern __shared__ __attribute__((aligned(16))) int8_t lds[];
@@ -76,20 +84,13 @@ __global__ __launch_bounds__(kStream32Threads) void gemm_stream32_kernel(GemmArg
   const int m_base = blockIdx.y * (MT32 * 32);            // activation rows of this workgroup
 
   // Loads of a wave return in issue order and the compiler counts them: a value is waited for
-  // with "all but the N youngest loads".  A load inside a branch makes that count unknown, and
-  // everything older is then waited for with N = 0.  So the loads that may be skipped (shortlist
-  // ids, bias) come first, and the activation and weight loads after them are unconditional
-  // (out-of-range indices are clamped and the values replaced afterwards): the activations can
-  // then be waited for while the weight loads are still in flight.
+  // with "all but the N youngest loads", and N can only count loads that are certain to have been
+  // issued.  The order below follows from that: first the shortlist ids (one round trip, waited
+  // for at once - they are addresses), then the activations, then the weights, last the bias
+  // (needed last); the activation, weight and bias loads are unconditional (out-of-range indices
+  // are clamped and the values replaced afterwards), so the activations are waited for with
+  // exactly the weight and bias loads still in flight.
 
-  // ---- weight row of this lane; bias of the columns this wave will write, through the
-  //      shortlist ids when there are any ----
-  const int n0 = (blockIdx.x * WN + wn) * 32;
-  int wsrc = min(n0 + li, args.n_out - 1);
-  if(args.idx) wsrc = (int)args.idx[wsrc];
-  // (pins the wait for the id here, where nothing else is in flight; left to itself the compiler
-  // computes the weight address, and waits, after the activation loads)
-  asm volatile("" : "+v"(wsrc));
   // Each wave finishes SL of a lane's 16 * MT32 accumulator values (see the reduction below):
   // values kw * SL + c * CW .. + CW - 1 for chunk c, i.e. activation tile mt = value / 16 and
   // weight rows n0 + 8 * q + 4 * lg + e with q = value % 16 / 4, e = value % 4.
@@ -98,17 +99,31 @@ __global__ __launch_bounds__(kStream32Threads) void gemm_stream32_kernel(GemmArg
   constexpr int CW = SL >= 4 ? 4 : SL;   // values per store: 4, or 2 for MT32 = 1 with KW = 8
   constexpr int NC = SL / CW;
   static_assert(SL >= 2 && NC * CW == SL, "slice shape");
-  float bias_s[NC][CW];
+
+  // ---- weight row of this lane and where the bias of the columns this wave will write sits,
+  //      both through the shortlist ids when there are any ----
+  const int n0 = (blockIdx.x * WN + wn) * 32;
+  int wsrc = min(n0 + li, args.n_out - 1);
+  uint32_t bias_at[NC][CW];
 #pragma unroll
   for(int c = 0; c < NC; ++c) {
     const int v = (kw * SL + c * CW) % 16;
     const int n = min(n0 + 8 * (v / 4) + 4 * lg + v % 4, args.n_out - CW);   // n_out % 8 == 0
 #pragma unroll
-    for(int e = 0; e < CW; ++e) {
-      bias_s[c][e] = 0.0f;
-      if(args.bias) bias_s[c][e] = args.bias[args.idx ? args.idx[n + e] : (uint32_t)(n + e)];
-    }
+    for(int e = 0; e < CW; ++e) bias_at[c][e] = (uint32_t)(n + e);
   }
+  if(args.idx) {
+    if(args.bias) {
+#pragma unroll
+      for(int c = 0; c < NC; ++c)
+#pragma unroll
+        for(int e = 0; e < CW; ++e) bias_at[c][e] = args.idx[bias_at[c][e]];
+    }
+    wsrc = (int)args.idx[wsrc];
+  }
+  // (pins the wait for the ids here, where nothing else is in flight; left to itself the compiler
+  // computes the weight address, and waits, after the activation loads)
+  asm volatile("" : "+v"(wsrc));
   const float bqm = tail_quant_mult(args.Bq, (size_t)K * (size_t)args.N);
   float aqm_pre = 0.0f;
   if(MODE == kPrequant) aqm_pre = tail_quant_mult(args.Aq, (size_t)M * (size_t)K);
@@ -124,20 +139,26 @@ __global__ __launch_bounds__(kStream32Threads) void gemm_stream32_kernel(GemmArg
 
   // FUSED: the fp32 activations are requested before anything else - they are needed first, and
   // a wave's loads return in issue order, so behind the weight stream they would arrive last.
-  // A thread owns groups of 16 consecutive values of one activation row (one 16-byte LDS slot
-  // after quantization): group number gi = j * threads + tid is row gi / (K/16), chunk gi % (K/16).
+  // Four neighbouring lanes (a quad) own four consecutive groups of 16 values of one activation
+  // row (K % 64 == 0 keeps them in one row); load e brings lane i of the quad the i-th four values
+  // of group e, so a quad reads 64 contiguous bytes per load (one cache line per quad, the rate
+  // the address unit works at) and, after quantization, holds dword i of four 16-byte LDS slots.
+  // Quad number qi = j * threads / 4 + tid / 4 covers groups 4 * qi .. 4 * qi + 3; group g is row
+  // g / (K/16), 16-byte chunk g % (K/16).
   v4f vals[FUSED ? kFusedGroups : 1][4];
-  const int n16 = M * K / 16;
+  const int n16 = M * K / 16;   // groups; a multiple of four
+  const int quad = tid / 4, qlane = tid % 4;
+  const int wave_s = __builtin_amdgcn_readfirstlane(wave);   // (a scalar for the compiler)
   if(FUSED) {
     const v4f* a4 = reinterpret_cast<const v4f*>(A);
 #pragma unroll
     for(int j = 0; j < kFusedGroups; ++j) {
-      const int gi = j * kStream32Threads + tid;
+      const int g0 = min(4 * (j * (kStream32Threads / 4) + quad), n16 - 4);
 #pragma unroll
       for(int e = 0; e < 4; ++e) {
         vals[j][e] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
         // (a wave whose 64 groups are all out of range skips the loads)
-        if(j * kStream32Threads + wave * kWave < n16) vals[j][e] = a4[min(gi, n16 - 1) * 4 + e];
+        if(j * kStream32Threads + wave_s * kWave < n16) vals[j][e] = a4[(g0 + e) * 4 + qlane];
       }
     }
   }
@@ -147,8 +168,8 @@ __global__ __launch_bounds__(kStream32Threads) void gemm_stream32_kernel(GemmArg
   // Otherwise a chunk of activations is fetched into registers (all loads in flight at once) and
   // then dropped into LDS, so the fetch of chunk c+1 overlaps the multiplication of chunk c.
   // Pre-quantized: thread slot (sub-step, m-tile, lane) in operand order.  kFusedTiled: fp32
-  // source; a thread takes 16 consecutive values of a row (slot = row * 2 * CS + 16-byte chunk,
-  // so that a wave reads whole rows), quantizes them and finds the operand slot from there.
+  // source; group = row * 2 * CS + 16-byte chunk, a quad of lanes takes four consecutive groups
+  // (a wave reads whole rows), quantizes them and finds the operand slots from there.
   constexpr int kStageVecs = Cfg::CS * MT32 * 64 / kStream32Threads;
   v4i stage[TILED ? 1 : kStageVecs];
   v4f stagef[TILED ? kStageVecs : 1][4];
@@ -158,11 +179,15 @@ __global__ __launch_bounds__(kStream32Threads) void gemm_stream32_kernel(GemmArg
     for(int j = 0; j < kStageVecs; ++j) {
       const int slot = j * kStream32Threads + tid;
       if(TILED) {
-        const int r = slot / (2 * Cfg::CS), c16 = slot % (2 * Cfg::CS);
-        const int m = min(m_base + r, M - 1), s = min(s0 + c16 / 2, S - 1);
-        const v4f* src = reinterpret_cast<const v4f*>(A + (size_t)m * (size_t)K + s * 32 + (c16 % 2) * 16);
+        // quad slot / 4 takes chunks c16 .. c16 + 3 of row r, lane i of the quad the i-th four
+        // values of each (64 contiguous bytes per quad and load, as in the fused form)
+        const int g = (slot / 4) * 4, r = g / (2 * Cfg::CS), c16 = g % (2 * Cfg::CS);
+        const int m = min(m_base + r, M - 1);
 #pragma unroll
-        for(int e = 0; e < 4; ++e) stagef[j][e] = src[e];
+        for(int e = 0; e < 4; ++e) {
+          const int s = min(s0 + (c16 + e) / 2, S - 1);
+          stagef[j][e] = *reinterpret_cast<const v4f*>(A + (size_t)m * (size_t)K + s * 32 + (e % 2) * 16 + (slot % 4) * 4);
+        }
       } else {
         const int l = slot % 64, f = slot / 64;
         const int mt = f % MT32, step = f / MT32;
@@ -177,30 +202,31 @@ __global__ __launch_bounds__(kStream32Threads) void gemm_stream32_kernel(GemmArg
     for(int j = 0; j < kStageVecs; ++j) {
       const int slot = j * kStream32Threads + tid;
       if(TILED) {
-        const int r = slot / (2 * Cfg::CS), c16 = slot % (2 * Cfg::CS);
-        const int m = m_base + r, s = chunk * Cfg::CS + c16 / 2;
-        uint4 q;
+        const int g = (slot / 4) * 4, r = g / (2 * Cfg::CS), c16 = g % (2 * Cfg::CS);
+        const int m = m_base + r;
+        uint32_t q[4];
         if(finite_t) {
-          q.x = quantize_pack4_finite(stagef[j][0], aqm);
-          q.y = quantize_pack4_finite(stagef[j][1], aqm);
-          q.z = quantize_pack4_finite(stagef[j][2], aqm);
-          q.w = quantize_pack4_finite(stagef[j][3], aqm);
+#pragma unroll
+          for(int e = 0; e < 4; ++e) q[e] = quantize_pack4_finite(stagef[j][e], aqm);
         } else {
-          q.x = quantize_pack4(stagef[j][0], aqm);
-          q.y = quantize_pack4(stagef[j][1], aqm);
-          q.z = quantize_pack4(stagef[j][2], aqm);
-          q.w = quantize_pack4(stagef[j][3], aqm);
+#pragma unroll
+          for(int e = 0; e < 4; ++e) q[e] = quantize_pack4(stagef[j][e], aqm);
         }
-        // rows past M hold zeros (sub-steps past K multiply zero weights, any value will do)
-        if(m >= M) q = uint4{0, 0, 0, 0};
-        const int sw = ((c16 / 2) * MT32 + r / 32) * 64 + (c16 % 2) * 32 + ((r % 32) ^ (c16 & 7));
-        *reinterpret_cast<uint4*>(lds + sw * 16) = q;
-        if(aq_out && blockIdx.x == 0 && m < M && s < S)
-          *reinterpret_cast<uint4*>(aq_out + (size_t)m * (size_t)K + s * 32 + (c16 % 2) * 16) = q;
+        const int slot0 = ((c16 / 2) * MT32 + r / 32) * 64, x = (r % 32) ^ stream32_row_key(c16);
+#pragma unroll
+        for(int e = 0; e < 4; ++e) {
+          // rows past M hold zeros (sub-steps past K multiply zero weights, any value will do)
+          if(m >= M) q[e] = 0;
+          const int s = chunk * Cfg::CS + (c16 + e) / 2;
+          const int sw = slot0 + (e / 2) * MT32 * 64 + (e % 2) * 32 + (x ^ e);
+          *reinterpret_cast<uint32_t*>(lds + sw * 16 + (slot % 4) * 4) = q[e];
+          if(aq_out && blockIdx.x == 0 && m < M && s < S)
+            *reinterpret_cast<uint32_t*>(aq_out + (size_t)m * (size_t)K + s * 32 + (e % 2) * 16 + (slot % 4) * 4) = q[e];
+        }
       } else {
         const int l = slot % 64, f = slot / 64;
         const int mt = f % MT32, step = f / MT32;
-        const int sw = (slot & ~31) | ((l % 32) ^ ((2 * step + l / 32) & 7));
+        const int sw = (slot & ~31) | ((l % 32) ^ stream32_row_key(2 * step + l / 32));
         const bool live = m_base + mt * 32 + (l % 32) < M;
         *reinterpret_cast<v4i*>(lds + sw * 16) = live ? stage[j] : v4i{0, 0, 0, 0};
       }
@@ -222,7 +248,23 @@ __global__ __launch_bounds__(kStream32Threads) void gemm_stream32_kernel(GemmArg
     for(int p = 0; p < Cfg::PW; ++p)
       if(chunk * Cfg::CS + kw * Cfg::PW + p >= S) w[p] = v4i{0, 0, 0, 0};
   };
+  // A CU's vector memory pipeline answers in request order, across its waves too: activation
+  // requests (cache hits) queued behind another wave's weight requests (HBM) would wait for those.
+  // The barrier puts every activation request of the workgroup ahead of every weight request.
+  __builtin_amdgcn_sched_barrier(0);
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_sched_barrier(0);
   load_weights(0);   // in flight while the activations are prepared
+  __builtin_amdgcn_sched_barrier(0);
+  // (unconditional as well: without a bias the weights stand in - 4 * N readable bytes - and the
+  // values are dropped in the epilogue)
+  float bias_s[NC][CW];
+  const float* bias_src = args.bias ? args.bias : reinterpret_cast<const float*>(args.Bq);
+#pragma unroll
+  for(int c = 0; c < NC; ++c)
+#pragma unroll
+    for(int e = 0; e < CW; ++e) bias_s[c][e] = bias_src[bias_at[c][e]];
+  __builtin_amdgcn_sched_barrier(0);
 
   // ---- activations into LDS, operand order: slot (sub-step, m-tile, lane) of 16 bytes holds
   //      Aq[mt*32 + lane%32][(s0+step)*32 + (lane/32)*16 .. +15]
@@ -239,7 +281,7 @@ __global__ __launch_bounds__(kStream32Threads) void gemm_stream32_kernel(GemmArg
     for(int j = 0; j < kFusedGroups; ++j)
 #pragma unroll
       for(int e = 0; e < 4; ++e) {
-        if(j * kStream32Threads + tid >= n16) vals[j][e] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+        if(4 * (j * (kStream32Threads / 4) + quad) >= n16) vals[j][e] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
         amax = abs4max(vals[j][e], amax);
       }
     // zero the rows between M and the next multiple of 32 (whole LDS stage, cheap)
@@ -250,35 +292,45 @@ __global__ __launch_bounds__(kStream32Threads) void gemm_stream32_kernel(GemmArg
     aqm = quant_mult_from_maxabs(amax);
     // with a finite non-zero abs-max no product can leave [-127.0001, 127.0001]
     const bool finite = amax > 0.0f && amax < __builtin_inff();
-    const int k16n = K / 16;   // 16-byte chunks per activation row
-    int row = tid / k16n, c16 = tid % k16n;
-    const int drow = kStream32Threads / k16n, dc16 = kStream32Threads % k16n;
+    const unsigned k16n = K / 16;   // 16-byte chunks per activation row (a multiple of four)
+    unsigned row = 4 * quad / k16n, c16 = 4 * quad % k16n;   // of the quad's first group
+    const unsigned drow = kStream32Threads / k16n, dc16 = kStream32Threads % k16n;
+    uint32_t q[kFusedGroups][4];
 #pragma unroll
     for(int j = 0; j < kFusedGroups; ++j) {
-      const int gi = j * kStream32Threads + tid;
-      if(gi < n16) {
-        uint4 q;
+      if(4 * (j * (kStream32Threads / 4) + quad) < n16) {
         if(finite) {
-          q.x = quantize_pack4_finite(vals[j][0], aqm);
-          q.y = quantize_pack4_finite(vals[j][1], aqm);
-          q.z = quantize_pack4_finite(vals[j][2], aqm);
-          q.w = quantize_pack4_finite(vals[j][3], aqm);
+#pragma unroll
+          for(int e = 0; e < 4; ++e) q[j][e] = quantize_pack4_finite(vals[j][e], aqm);
         } else {
-          q.x = quantize_pack4(vals[j][0], aqm);
-          q.y = quantize_pack4(vals[j][1], aqm);
-          q.z = quantize_pack4(vals[j][2], aqm);
-          q.w = quantize_pack4(vals[j][3], aqm);
+#pragma unroll
+          for(int e = 0; e < 4; ++e) q[j][e] = quantize_pack4(vals[j][e], aqm);
         }
-        const int s = c16 / 2, g = c16 % 2;
-        const int slot = (s * MT32 + row / 32) * 64 + g * 32 + ((row % 32) ^ (c16 & 7));
-        *reinterpret_cast<uint4*>(lds + slot * 16) = q;
-        if(aq_out && blockIdx.x == 0) *reinterpret_cast<uint4*>(aq_out + (size_t)row * K + c16 * 16) = q;
+        // slot of group e: chunk c16 + e, i.e. sub-step (c16 + e) / 2, half (c16 + e) % 2, and
+        // the row permuted by the key of chunk c16 + e, which is the key of c16 (c16 % 4 == 0) ^ e
+        const unsigned slot0 = ((c16 >> 1) * MT32 + (row >> 5)) * 64, x = (row & 31) ^ stream32_row_key(c16);
+#pragma unroll
+        for(int e = 0; e < 4; ++e) {
+          const unsigned slot = slot0 + (e / 2) * MT32 * 64 + (e % 2) * 32 + (x ^ e);
+          *reinterpret_cast<uint32_t*>(lds + slot * 16 + qlane * 4) = q[j][e];
+        }
       }
       row += drow;
       c16 += dc16;
       if(c16 >= k16n) {
         c16 -= k16n;
         row += 1;
+      }
+    }
+    if(aq_out && blockIdx.x == 0) {   // the quad's four groups are 64 consecutive bytes of Aq
+#pragma unroll
+      for(int j = 0; j < kFusedGroups; ++j) {
+        const int g = 4 * (j * (kStream32Threads / 4) + quad);
+        if(g < n16) {
+#pragma unroll
+          for(int e = 0; e < 4; ++e)
+            *reinterpret_cast<uint32_t*>(aq_out + (size_t)(g + e) * 16 + qlane * 4) = q[j][e];
+        }
       }
     }
     if(aq_out && blockIdx.x == 0 && tid == 0)
@@ -318,7 +370,7 @@ __global__ __launch_bounds__(kStream32Threads) void gemm_stream32_kernel(GemmArg
 #pragma unroll
       for(int mt = 0; mt < MT32; ++mt) {
         const v4i a = *reinterpret_cast<const v4i*>(
-            lds + (step * MT32 + mt) * kFragBytes + (lg * 32 + (li ^ ((2 * step + lg) & 7))) * 16);
+            lds + (step * MT32 + mt) * kFragBytes + (lg * 32 + (li ^ stream32_row_key(2 * step + lg))) * 16);
         acc[mt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(w[p], a, acc[mt], 0, 0, 0);
       }
     }
