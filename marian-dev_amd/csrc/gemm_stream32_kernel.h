@@ -49,7 +49,7 @@ struct Stream32Cfg {
   static constexpr int PW = PW_;
   static constexpr int CS = PW * KW;
   static constexpr int kStageBytes = MT32 * CS * kFragBytes;
-  static constexpr int kReduceBytes = (KW - 1) * WN * MT32 * 4 * kFragBytes;  // v16i per lane
+  static constexpr int kReduceBytes = KW * WN * MT32 * 4 * kFragBytes;  // every wave's 32 * MT32 x 32 int32 tile
   static constexpr int kLdsBytes = kStageBytes > kReduceBytes ? kStageBytes : kReduceBytes;
   static_assert(PW >= 1 && PW <= 8 && kStageBytes <= 64 * 1024, "chunk size");
   static_assert(CS * MT32 * 64 % kThreads == 0, "stage must divide over the threads");
@@ -91,33 +91,17 @@ __global__ __launch_bounds__(WN * KW * kWave) void gemm_stream32_kernel(GemmArgs
   // are clamped and the values replaced afterwards), so the activations are waited for with
   // exactly the weight and bias loads still in flight.
 
-  // Each wave finishes SL of a lane's 16 * MT32 accumulator values (see the reduction below):
-  // values kw * SL + c * CW .. + CW - 1 for chunk c, i.e. activation tile mt = value / 16 and
-  // weight rows n0 + 8 * q + 4 * lg + e with q = value % 16 / 4, e = value % 4.
-  constexpr int V = 16 * MT32;
-  constexpr int SL = V / KW;
-  constexpr int CW = SL >= 4 ? 4 : SL;   // values per store: 4, or 2 for MT32 = 1 with KW = 8
-  constexpr int NC = SL / CW;
-  static_assert(SL >= 2 && NC * CW == SL, "slice shape");
-
-  // ---- weight row of this lane and where the bias of the columns this wave will write sits,
-  //      both through the shortlist ids when there are any ----
+  // ---- weight row of this lane and where the bias of the four columns this lane will write
+  //      sits (see the epilogue), both through the shortlist ids when there are any ----
   const int n0 = (blockIdx.x * WN + wn) * 32;
   int wsrc = min(n0 + li, args.n_out - 1);
-  uint32_t bias_at[NC][CW];
+  uint32_t bias_at[4];
 #pragma unroll
-  for(int c = 0; c < NC; ++c) {
-    const int v = (kw * SL + c * CW) % 16;
-    const int n = min(n0 + 8 * (v / 4) + 4 * lg + v % 4, args.n_out - CW);   // n_out % 8 == 0
-#pragma unroll
-    for(int e = 0; e < CW; ++e) bias_at[c][e] = (uint32_t)(n + e);
-  }
+  for(int e = 0; e < 4; ++e) bias_at[e] = (uint32_t)min(n0 + 4 * (lane % 8) + e, args.n_out - 1);
   if(args.idx) {
     if(args.bias) {
 #pragma unroll
-      for(int c = 0; c < NC; ++c)
-#pragma unroll
-        for(int e = 0; e < CW; ++e) bias_at[c][e] = args.idx[bias_at[c][e]];
+      for(int e = 0; e < 4; ++e) bias_at[e] = args.idx[bias_at[e]];
     }
     wsrc = (int)args.idx[wsrc];
   }
@@ -258,12 +242,10 @@ __global__ __launch_bounds__(WN * KW * kWave) void gemm_stream32_kernel(GemmArgs
   __builtin_amdgcn_sched_barrier(0);
   // (unconditional as well: without a bias the weights stand in - 4 * N readable bytes - and the
   // values are dropped in the epilogue)
-  float bias_s[NC][CW];
+  float bias_s[4];
   const float* bias_src = args.bias ? args.bias : reinterpret_cast<const float*>(args.Bq);
 #pragma unroll
-  for(int c = 0; c < NC; ++c)
-#pragma unroll
-    for(int e = 0; e < CW; ++e) bias_s[c][e] = bias_src[bias_at[c][e]];
+  for(int e = 0; e < 4; ++e) bias_s[e] = bias_src[bias_at[e]];
   __builtin_amdgcn_sched_barrier(0);
 
   // ---- activations into LDS, operand order: slot (sub-step, m-tile, lane) of 16 bytes holds
@@ -386,80 +368,63 @@ __global__ __launch_bounds__(WN * KW * kWave) void gemm_stream32_kernel(GemmArgs
   }
 
   if(args.prof) tp[3] = clock64();
-  // ---- add the KW partial sums: wave r collects slice r (values r * SL .. + SL - 1 of every
-  //      lane) from the other waves of its column group, so that the additions and the stores
-  //      of the epilogue are spread over all waves.  Slot (r, t, wn, c, lane) of CW ints holds
-  //      what source wave t' (t = t' minus one if t' > r) contributes to chunk c of slice r. ----
-  int mine[NC][CW];
-  if(KW > 1) {
-    __syncthreads();   // every wave is done reading activations from LDS
-    int* redbuf = reinterpret_cast<int*>(lds);
+  // ---- every wave drops its 32 * MT32 x 32 tile of int32 partial sums into LDS as a row-major
+  //      matrix [activation row][32 weight rows] (128 bytes per row; the eight 16-byte pieces of
+  //      a row XOR-permuted by the row number, which keeps both sides free of bank conflicts),
+  //      and finishes 1/KW of the rows of its column group: it adds the KW partial tiles (exact in
+  //      any order) and stores whole 128-byte output rows, eight lanes per row.  Accumulator
+  //      value v of tile mt in lane (li, lg) is activation row mt * 32 + li, weight row
+  //      8 * (v / 4) + 4 * lg + v % 4, i.e. piece 2 * (v / 4) + lg of that row. ----
+  constexpr int R = MT32 * 32;                 // activation rows of the workgroup
+  constexpr int kTileBytes = R * 128;
+  __syncthreads();   // every wave is done reading activations from LDS
+  {
+    int8_t* mine = lds + (size_t)(wn * KW + kw) * kTileBytes;
 #pragma unroll
-    for(int r = 0; r < KW; ++r) {
-      if(r == kw) {
+    for(int mt = 0; mt < MT32; ++mt)
 #pragma unroll
-        for(int c = 0; c < NC; ++c)
-#pragma unroll
-          for(int e = 0; e < CW; ++e) mine[c][e] = acc[(r * SL + c * CW + e) / 16][(r * SL + c * CW + e) % 16];
-      } else {
-        const int t = kw < r ? kw : kw - 1;
-#pragma unroll
-        for(int c = 0; c < NC; ++c) {
-          int* dst = redbuf + (size_t)(((((r * (KW - 1) + t) * WN + wn) * NC + c) * 64 + lane) * CW);
-#pragma unroll
-          for(int e = 0; e < CW; ++e) dst[e] = acc[(r * SL + c * CW + e) / 16][(r * SL + c * CW + e) % 16];
-        }
+      for(int q = 0; q < 4; ++q) {
+        const int m = mt * 32 + li, piece = (2 * q + lg) ^ (li & 7);
+        *reinterpret_cast<v4i*>(mine + m * 128 + piece * 16) =
+            v4i{acc[mt][4 * q], acc[mt][4 * q + 1], acc[mt][4 * q + 2], acc[mt][4 * q + 3]};
       }
-    }
-    __syncthreads();
-#pragma unroll
-    for(int t = 0; t < KW - 1; ++t)
-#pragma unroll
-      for(int c = 0; c < NC; ++c) {
-        const int* src = redbuf + (size_t)(((((kw * (KW - 1) + t) * WN + wn) * NC + c) * 64 + lane) * CW);
-#pragma unroll
-        for(int e = 0; e < CW; ++e) mine[c][e] += src[e];
-      }
-  } else {
-#pragma unroll
-    for(int c = 0; c < NC; ++c)
-#pragma unroll
-      for(int e = 0; e < CW; ++e) mine[c][e] = acc[(c * CW + e) / 16][(c * CW + e) % 16];
   }
+  __syncthreads();
 
-  // ---- epilogue: value v of tile mt in lane (li, lg) is activation row mt * 32 + li, weight
-  //      row 8 * (v / 4) + 4 * lg + v % 4 of the wave's 32 ----
   if(args.prof) tp[4] = clock64();
   float omax = 0.0f;   // max |y| over what this wave stores
   {
+    constexpr int kPieces = R * 8 / KW;        // 16-byte pieces this wave finishes (32 .. 1024)
     const float unquant = unquant_mult(MODE == kPrequant ? aqm_pre : aqm, bqm, args.scale);
     const bool has_bias = args.bias != nullptr;
+    const int n = n0 + 4 * (lane % 8);
+    const int8_t* tiles = lds + (size_t)(wn * KW) * kTileBytes;
 #pragma unroll
-    for(int c = 0; c < NC; ++c) {
-      const int vv = kw * SL + c * CW;
-      const int v = vv % 16;
-      const int m = m_base + (vv / 16) * 32 + li;
-      const int n = n0 + 8 * (v / 4) + 4 * lg + v % 4;
+    for(int it = 0; it < (kPieces + 63) / 64; ++it) {
+      const int pc = it * 64 + lane;
+      const int mrow = kw * (R / KW) + pc / 8;              // row within the workgroup's tile
+      if(kPieces % 64 != 0 && pc >= kPieces) continue;
+      const int8_t* src = tiles + mrow * 128 + (((lane % 8) ^ (mrow & 7)) * 16);
+      v4i sum = *reinterpret_cast<const v4i*>(src);
+#pragma unroll
+      for(int t = 1; t < KW; ++t) sum += *reinterpret_cast<const v4i*>(src + t * kTileBytes);
+      const int m = m_base + mrow;
       if(m >= M || n >= args.n_out) continue;
       const size_t off = (size_t)m * (size_t)args.n_out + (size_t)n;
       if(args.dump) {
-        int32_t* o = reinterpret_cast<int32_t*>(args.out) + off;
-        if(CW == 4) *reinterpret_cast<v4i*>(o) = v4i{mine[c][0], mine[c][1], mine[c][CW - 2], mine[c][CW - 1]};
-        else *reinterpret_cast<int2*>(o) = int2{mine[c][0], mine[c][1]};
+        *reinterpret_cast<v4i*>(reinterpret_cast<int32_t*>(args.out) + off) = sum;
         continue;
       }
       // y = float(acc) * unquant (+ bias); relu: y > 0 ? y : 0; mul and add round separately
-      float y[CW];
+      float y[4];
 #pragma unroll
-      for(int e = 0; e < CW; ++e) {
-        y[e] = (float)mine[c][e] * unquant;
-        if(has_bias) y[e] = y[e] + bias_s[c][e];
+      for(int e = 0; e < 4; ++e) {
+        y[e] = (float)sum[e] * unquant;
+        if(has_bias) y[e] = y[e] + bias_s[e];
         if(args.relu) y[e] = y[e] > 0.0f ? y[e] : 0.0f;
         omax = fmaxf(omax, fabsf(y[e]));
       }
-      float* o = reinterpret_cast<float*>(args.out) + off;
-      if(CW == 4) *reinterpret_cast<v4f*>(o) = v4f{y[0], y[1], y[CW - 2], y[CW - 1]};
-      else *reinterpret_cast<float2*>(o) = float2{y[0], y[1]};
+      *reinterpret_cast<v4f*>(reinterpret_cast<float*>(args.out) + off) = v4f{y[0], y[1], y[2], y[3]};
     }
   }
   if(args.absmax_out && !args.dump) {
