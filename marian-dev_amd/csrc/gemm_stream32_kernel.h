@@ -72,8 +72,11 @@ __global__ __launch_bounds__(WN * KW * kWave) void gemm_stream32_kernel(GemmArgs
   extern __shared__ __attribute__((aligned(16))) int8_t lds[];
   __shared__ float red[kStream32Waves];
 
-  long long tp[6] = {0, 0, 0, 0, 0, 0};
-  if(args.prof) tp[0] = clock64();
+  long long tp[6] = {0, 0, 0, 0, 0, 0}, wall0 = 0;
+  if(args.prof) {
+    tp[0] = clock64();
+    wall0 = wall_clock64();
+  }
   const int tid = threadIdx.x;
   const int wave = tid / kWave, lane = tid % kWave;
   const int wn = wave % WN, kw = wave / WN;
@@ -440,6 +443,7 @@ __global__ __launch_bounds__(WN * KW * kWave) void gemm_stream32_kernel(GemmArgs
     long long* p = args.prof + ((size_t)blockIdx.y * gridDim.x + blockIdx.x) * 8;
     p[0] = tp[0]; p[1] = tp[1]; p[2] = tp[2]; p[3] = tp[3]; p[4] = tp[4]; p[5] = clock64();
     p[6] = wall_clock64();
+    p[7] = wall0;
   }
 }
 

@@ -21,36 +21,45 @@ __device__ __forceinline__ int quantize_one(float x, float qm) {
   return (fabsf(v) < 2147483648.0f) ? q : -127;
 }
 
-// Same result as quantize_one in the low byte of the returned word, in five VALU operations:
-// clamping to [-127, 127] first commutes with rounding (the bounds are integers; med3 returns
-// -127 for NaN), and adding 1.5 * 2^23 rounds to nearest-even with the integer landing in the
-// low mantissa bits (two's complement in the low byte).  Products >= 2^31 (only possible for
-// non-finite inputs) follow the x86 conversion and give -127.
-__device__ __forceinline__ uint32_t quantize_low_byte(float x, float qm) {
-  float v = x * qm;
-  float c = __builtin_amdgcn_fmed3f(v, -127.0f, 127.0f);
-  c = (v >= 2147483648.0f) ? -127.0f : c;
-  return __float_as_uint(c + 12582912.0f);
+// The value whose rounding to nearest-even is quantize_one(x, qm): clamping to [-127, 127] first
+// commutes with rounding (the bounds are integers; med3 returns -127 for NaN).  Products >= 2^31
+// (only possible for non-finite inputs) follow the x86 conversion and give -127.
+__device__ __forceinline__ float quantize_clamped(float x, float qm) {
+  const float v = x * qm;
+  const float c = __builtin_amdgcn_fmed3f(v, -127.0f, 127.0f);
+  return (v >= 2147483648.0f) ? -127.0f : c;
+}
+
+// Four clamped products -> four int8 in one word.  Adding 1.5 * 2^23 rounds to nearest-even and
+// leaves the integer in the low byte of the sum; the SDWA form of the add writes that low byte
+// straight into byte 0..3 of the destination, so no byte shuffles are needed afterwards.
+__device__ __forceinline__ uint32_t round_pack4(float c0, float c1, float c2, float c3) {
+  const float magic = 12582912.0f;
+  uint32_t q;
+  asm("v_add_f32_sdwa %0, %1, %2 dst_sel:BYTE_0 dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:DWORD"
+      : "=v"(q) : "v"(c0), "v"(magic));
+  asm("v_add_f32_sdwa %0, %1, %2 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD"
+      : "+v"(q) : "v"(c1), "v"(magic));
+  asm("v_add_f32_sdwa %0, %1, %2 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD"
+      : "+v"(q) : "v"(c2), "v"(magic));
+  asm("v_add_f32_sdwa %0, %1, %2 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD"
+      : "+v"(q) : "v"(c3), "v"(magic));
+  return q;
 }
 
 // Fast form for the usual case (finite, non-zero abs-max): every product lies within
-// [-127.0001, 127.0001], so the non-finite check of quantize_low_byte can never fire.
+// [-127.0001, 127.0001], so the out-of-range check of quantize_clamped can never fire (med3
+// still maps a NaN among the values to -127).
 __device__ __forceinline__ uint32_t quantize_pack4_finite(v4f x, float qm) {
-  const uint32_t b0 = __float_as_uint(__builtin_amdgcn_fmed3f(x.x * qm, -127.0f, 127.0f) + 12582912.0f);
-  const uint32_t b1 = __float_as_uint(__builtin_amdgcn_fmed3f(x.y * qm, -127.0f, 127.0f) + 12582912.0f);
-  const uint32_t b2 = __float_as_uint(__builtin_amdgcn_fmed3f(x.z * qm, -127.0f, 127.0f) + 12582912.0f);
-  const uint32_t b3 = __float_as_uint(__builtin_amdgcn_fmed3f(x.w * qm, -127.0f, 127.0f) + 12582912.0f);
-  const uint32_t lo = __builtin_amdgcn_perm(b1, b0, 0x0c0c0400u);
-  const uint32_t hi = __builtin_amdgcn_perm(b3, b2, 0x0c0c0400u);
-  return __builtin_amdgcn_perm(hi, lo, 0x05040100u);
+  return round_pack4(__builtin_amdgcn_fmed3f(x.x * qm, -127.0f, 127.0f),
+                     __builtin_amdgcn_fmed3f(x.y * qm, -127.0f, 127.0f),
+                     __builtin_amdgcn_fmed3f(x.z * qm, -127.0f, 127.0f),
+                     __builtin_amdgcn_fmed3f(x.w * qm, -127.0f, 127.0f));
 }
 
 __device__ __forceinline__ uint32_t quantize_pack4(v4f x, float qm) {
-  const uint32_t b0 = quantize_low_byte(x.x, qm), b1 = quantize_low_byte(x.y, qm);
-  const uint32_t b2 = quantize_low_byte(x.z, qm), b3 = quantize_low_byte(x.w, qm);
-  const uint32_t lo = __builtin_amdgcn_perm(b1, b0, 0x0c0c0400u);  // [b0.0, b1.0, 0, 0]
-  const uint32_t hi = __builtin_amdgcn_perm(b3, b2, 0x0c0c0400u);
-  return __builtin_amdgcn_perm(hi, lo, 0x05040100u);               // [lo.0, lo.1, hi.0, hi.1]
+  return round_pack4(quantize_clamped(x.x, qm), quantize_clamped(x.y, qm), quantize_clamped(x.z, qm),
+                     quantize_clamped(x.w, qm));
 }
 
 __device__ __forceinline__ float abs4max(v4f x, float m) {
