@@ -121,10 +121,13 @@ struct FusedSrc {   // what the fused modes read and write besides GemmArgs
   int n_partials = 0;
 };
 
-template <int MT32, int WN, int KW, int PW, int MODE>
+template <int MT32, int WN, int KW, int PW, int MODE, int NG = 4>
 int launch_stream32(const GemmArgs& a, const FusedSrc& f, hipStream_t st) {
+  if constexpr(MODE == kFusedAll && NG == 4) {   // at most two groups of 16 values per thread
+    if((long long)a.M * a.K <= kFusedMaxElems / 2) return launch_stream32<MT32, WN, KW, PW, MODE, 2>(a, f, st);
+  }
   using Cfg = Stream32Cfg<MT32, WN, KW, PW>;
-  auto kernel = gemm_stream32_kernel<MT32, WN, KW, PW, MODE>;
+  auto kernel = gemm_stream32_kernel<MT32, WN, KW, PW, MODE, NG>;
   constexpr int kMaxLds = 64 * 1024 > Cfg::kLdsBytes ? 64 * 1024 : Cfg::kLdsBytes;
   static const int lds_status = allow_lds(kernel, kMaxLds);
   if(lds_status != MARIAN_HIP_OK) return lds_status;

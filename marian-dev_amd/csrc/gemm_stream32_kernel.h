@@ -58,7 +58,10 @@ struct Stream32Cfg {
 
 // Dynamic LDS: kFusedAll holds all of K (32 * MT32 * K bytes); otherwise one chunk (kStageBytes);
 // both at least kReduceBytes.  partials: n_partials (1..2048) abs-max values (kFusedTiled only).
-template <int MT32, int WN, int KW, int PW, int MODE>
+// NG (kFusedAll only): 16-value groups per thread that are compiled in, 2 or 4; all but the last
+// two are complete (the launcher picks NG = 2 for M * K <= 16384), so their loads, abs-max and
+// quantization carry no range checks.
+template <int MT32, int WN, int KW, int PW, int MODE, int NG = 4>
 __global__ __launch_bounds__(WN * KW * kWave) void gemm_stream32_kernel(GemmArgs args,
                                                                         const float* A,
                                                                         int8_t* aq_out,
@@ -66,7 +69,9 @@ __global__ __launch_bounds__(WN * KW * kWave) void gemm_stream32_kernel(GemmArgs
                                                                         int n_partials) {
   using Cfg = Stream32Cfg<MT32, WN, KW, PW>;
   constexpr int kStream32Waves = Cfg::kWaves, kStream32Threads = Cfg::kThreads;
-  constexpr int kFusedGroups = kFusedMaxElems / 16 / kStream32Threads;   // 16-value groups per thread
+  constexpr int kFusedGroups = NG, kFullGroups = NG - 2;
+  static_assert(NG == 2 || NG == 4, "groups per thread");
+  static_assert(kFusedMaxElems == 4 * 16 * Cfg::kThreads, "four groups per thread hold the largest fused input");
   constexpr bool FUSED = MODE == kFusedAll;
   constexpr bool TILED = MODE == kFusedTiled;
   extern __shared__ __attribute__((aligned(16))) int8_t lds[];
@@ -136,16 +141,26 @@ __global__ __launch_bounds__(WN * KW * kWave) void gemm_stream32_kernel(GemmArgs
   const int n16 = M * K / 16;   // groups; a multiple of four
   const int quad = tid / 4, qlane = tid % 4;
   const int wave_s = __builtin_amdgcn_readfirstlane(wave);   // (a scalar for the compiler)
+  // does group set j reach into this thread's / this wave's range?  (complete sets: always)
+  auto in_range = [&](int j) { return j < kFullGroups || 4 * (j * (kStream32Threads / 4) + quad) < n16; };
   if(FUSED) {
+    // a quad's four groups are 256 consecutive bytes; group set j starts 32 KB after set j - 1
+    const char* a_quad = reinterpret_cast<const char*>(A) + quad * 256 + qlane * 16;
     const v4f* a4 = reinterpret_cast<const v4f*>(A);
 #pragma unroll
     for(int j = 0; j < kFusedGroups; ++j) {
-      const int g0 = min(4 * (j * (kStream32Threads / 4) + quad), n16 - 4);
+      if(j < kFullGroups) {
 #pragma unroll
-      for(int e = 0; e < 4; ++e) {
-        vals[j][e] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
-        // (a wave whose 64 groups are all out of range skips the loads)
-        if(j * kStream32Threads + wave_s * kWave < n16) vals[j][e] = a4[(g0 + e) * 4 + qlane];
+        for(int e = 0; e < 4; ++e)
+          vals[j][e] = *reinterpret_cast<const v4f*>(a_quad + j * (kStream32Threads * 64) + e * 64);
+      } else {
+        const int g0 = min(4 * (j * (kStream32Threads / 4) + quad), n16 - 4);
+#pragma unroll
+        for(int e = 0; e < 4; ++e) {
+          vals[j][e] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+          // (a wave whose 64 groups are all out of range skips the loads)
+          if(j * kStream32Threads + wave_s * kWave < n16) vals[j][e] = a4[(g0 + e) * 4 + qlane];
+        }
       }
     }
   }
@@ -257,6 +272,7 @@ __global__ __launch_bounds__(WN * KW * kWave) void gemm_stream32_kernel(GemmArgs
     amax = block_max(amax, red);
     aqm = quant_mult_from_maxabs(amax);
     finite_t = amax > 0.0f && amax < __builtin_inff();
+    if(args.prof) tp[1] = clock64();
     if(aq_out && blockIdx.x == 0 && blockIdx.y == 0 && tid == 0)
       *reinterpret_cast<float*>(aq_out + (size_t)M * K) = aqm;
   }
@@ -266,12 +282,14 @@ __global__ __launch_bounds__(WN * KW * kWave) void gemm_stream32_kernel(GemmArgs
     for(int j = 0; j < kFusedGroups; ++j)
 #pragma unroll
       for(int e = 0; e < 4; ++e) {
-        if(4 * (j * (kStream32Threads / 4) + quad) >= n16) vals[j][e] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+        if(!in_range(j)) vals[j][e] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
         amax = abs4max(vals[j][e], amax);
       }
-    // zero the rows between M and the next multiple of 32 (whole LDS stage, cheap)
-    for(int i = tid; i < S * MT32 * 64; i += kStream32Threads)
-      reinterpret_cast<v4i*>(lds)[i] = v4i{0, 0, 0, 0};
+    // zero the rows between M and the end of the last 32-row tile (whole LDS stage, cheap)
+    if(M < MT32 * 32) {
+      for(int i = tid; i < S * MT32 * 64; i += kStream32Threads)
+        reinterpret_cast<v4i*>(lds)[i] = v4i{0, 0, 0, 0};
+    }
     amax = block_max(amax, red);   // its barriers also order the zero fill before the writes
     if(args.prof) tp[1] = clock64();
     aqm = quant_mult_from_maxabs(amax);
@@ -283,7 +301,7 @@ __global__ __launch_bounds__(WN * KW * kWave) void gemm_stream32_kernel(GemmArgs
     uint32_t q[kFusedGroups][4];
 #pragma unroll
     for(int j = 0; j < kFusedGroups; ++j) {
-      if(4 * (j * (kStream32Threads / 4) + quad) < n16) {
+      if(in_range(j)) {
         if(finite) {
 #pragma unroll
           for(int e = 0; e < 4; ++e) q[j][e] = quantize_pack4_finite(vals[j][e], aqm);
@@ -311,7 +329,7 @@ __global__ __launch_bounds__(WN * KW * kWave) void gemm_stream32_kernel(GemmArgs
 #pragma unroll
       for(int j = 0; j < kFusedGroups; ++j) {
         const int g = 4 * (j * (kStream32Threads / 4) + quad);
-        if(g < n16) {
+        if(in_range(j)) {
 #pragma unroll
           for(int e = 0; e < 4; ++e)
             *reinterpret_cast<uint32_t*>(aq_out + (size_t)(g + e) * 16 + qlane * 4) = q[j][e];
