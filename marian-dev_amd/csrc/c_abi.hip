@@ -131,7 +131,9 @@ int launch_stream32(const GemmArgs& a, const FusedSrc& f, hipStream_t st) {
   constexpr int kMaxLds = 64 * 1024 > Cfg::kLdsBytes ? 64 * 1024 : Cfg::kLdsBytes;
   static const int lds_status = allow_lds(kernel, kMaxLds);
   if(lds_status != MARIAN_HIP_OK) return lds_status;
-  int lds = MODE == kFusedAll ? stream32_fused_lds_bytes(MT32, a.K) : Cfg::kStageBytes;
+  // (kFusedAll: all of K, and at least one whole chunk so that the first chunk needs no bounds)
+  int lds = Cfg::kStageBytes;
+  if(MODE == kFusedAll && lds < stream32_fused_lds_bytes(MT32, a.K)) lds = stream32_fused_lds_bytes(MT32, a.K);
   if(lds < Cfg::kReduceBytes) lds = Cfg::kReduceBytes;
   int blocks = (a.n_out + Cfg::kColsPerBlock - 1) / Cfg::kColsPerBlock;
   int m_tiles = MODE == kFusedAll ? 1 : (a.M + MT32 * 32 - 1) / (MT32 * 32);

@@ -19,6 +19,8 @@
 // by chunk on the way into LDS (the workgroups of column 0 also write them out).
 #pragma once
 
+#include <type_traits>
+
 #include "int8_common.h"
 #include "quantize_kernels.h"
 
@@ -56,8 +58,8 @@ struct Stream32Cfg {
   static_assert(CS % 2 == 0, "a quad of lanes quantizes four 16-byte chunks of one row");
 };
 
-// Dynamic LDS: kFusedAll holds all of K (32 * MT32 * K bytes); otherwise one chunk (kStageBytes);
-// both at least kReduceBytes.  partials: n_partials (1..2048) abs-max values (kFusedTiled only).
+// Dynamic LDS: one chunk (kStageBytes), for kFusedAll all of K (32 * MT32 * K bytes) if that is
+// more; at least kReduceBytes.  partials: n_partials (1..2048) abs-max values (kFusedTiled only).
 // NG (kFusedAll only): 16-value groups per thread that are compiled in, 2 or 4; all but the last
 // two are complete (the launcher picks NG = 2 for M * K <= 16384), so their loads, abs-max and
 // quantization carry no range checks.
@@ -175,7 +177,7 @@ __global__ __launch_bounds__(WN * KW * kWave) void gemm_stream32_kernel(GemmArgs
   constexpr int kStageVecs = Cfg::CS * MT32 * 64 / kStream32Threads;
   v4i stage[TILED ? 1 : kStageVecs];
   v4f stagef[TILED ? kStageVecs : 1][4];
-  auto stage_fetch = [&](int chunk) {
+  auto stage_fetch = [&](int chunk) __attribute__((always_inline)) {
     const int s0 = chunk * Cfg::CS;
 #pragma unroll
     for(int j = 0; j < kStageVecs; ++j) {
@@ -199,7 +201,7 @@ __global__ __launch_bounds__(WN * KW * kWave) void gemm_stream32_kernel(GemmArgs
       }
     }
   };
-  auto stage_store = [&](int chunk) {
+  auto stage_store = [&](int chunk) __attribute__((always_inline)) {
 #pragma unroll
     for(int j = 0; j < kStageVecs; ++j) {
       const int slot = j * kStream32Threads + tid;
@@ -237,15 +239,25 @@ __global__ __launch_bounds__(WN * KW * kWave) void gemm_stream32_kernel(GemmArgs
   if(!FUSED) stage_fetch(0);   // ahead of the weights, like the fp32 activations above
 
   v4i w[Cfg::PW];
-  auto load_weights = [&](int chunk) {
+  const int kw_s = __builtin_amdgcn_readfirstlane(kw);   // (a scalar for the compiler)
+  const int step0 = kw * Cfg::PW;                        // this wave's first sub-step within a chunk
+  // weights of a chunk: 32 * PW consecutive bytes of the lane's weight row, one pointer and
+  // constant offsets when the wave's sub-steps all lie within K, clamped one by one otherwise
+  auto load_weights = [&](int chunk, v4i (&dst)[Cfg::PW]) __attribute__((always_inline)) {
+    if(chunk * Cfg::CS + (kw_s + 1) * Cfg::PW <= S) {
+      const int8_t* wp = wrow + (chunk * Cfg::CS + step0) * 32;
 #pragma unroll
-    for(int p = 0; p < Cfg::PW; ++p) {
-      const int s = chunk * Cfg::CS + kw * Cfg::PW + p;
-      w[p] = load16(wrow + min(s, S - 1) * 32);
+      for(int p = 0; p < Cfg::PW; ++p) dst[p] = load16(wp + p * 32);
+    } else {
+#pragma unroll
+      for(int p = 0; p < Cfg::PW; ++p) {
+        const int s = chunk * Cfg::CS + step0 + p;
+        dst[p] = load16(wrow + min(s, S - 1) * 32);
+      }
     }
   };
   // sub-steps past the end of K multiply zero weights
-  auto mask_weights = [&](int chunk) {
+  auto mask_weights = [&](int chunk) __attribute__((always_inline)) {
 #pragma unroll
     for(int p = 0; p < Cfg::PW; ++p)
       if(chunk * Cfg::CS + kw * Cfg::PW + p >= S) w[p] = v4i{0, 0, 0, 0};
@@ -256,7 +268,7 @@ __global__ __launch_bounds__(WN * KW * kWave) void gemm_stream32_kernel(GemmArgs
   __builtin_amdgcn_sched_barrier(0);
   __builtin_amdgcn_s_barrier();
   __builtin_amdgcn_sched_barrier(0);
-  load_weights(0);   // in flight while the activations are prepared
+  load_weights(0, w);   // in flight while the activations are prepared
   __builtin_amdgcn_sched_barrier(0);
   // (unconditional as well: without a bias the weights stand in - 4 * N readable bytes - and the
   // values are dropped in the epilogue)
@@ -346,35 +358,43 @@ __global__ __launch_bounds__(WN * KW * kWave) void gemm_stream32_kernel(GemmArgs
   }
 
   if(args.prof) tp[2] = clock64();
+  // The first chunk is peeled off the loop: its first product starts from a literal zero and its
+  // fragment addresses are this wave's base plus constants (slot of sub-step step0 + p, half lg,
+  // row li: the row key of chunk number 2 * (step0 + p) + lg is key(2 * step0) ^ key(2 * p) ^ lg,
+  // the three parts occupy different bits).  In the fused form LDS holds every sub-step of K, so
+  // later chunks address it by the global sub-step, clamped (sub-steps past the end of K multiply
+  // zero weights; for the first chunk the allocation covers a whole chunk).
   v16i_s acc[MT32];
-#pragma unroll
-  for(int mt = 0; mt < MT32; ++mt)
-#pragma unroll
-    for(int v = 0; v < 16; ++v) acc[mt][v] = 0;
-
   v4i wnext[Cfg::PW];
-  for(int c = 0; c < n_chunks; ++c) {
+  const int8_t* frag0 = lds + step0 * MT32 * kFragBytes + lg * 512;
+  const int akey = li ^ lg ^ stream32_row_key(2 * step0);
+  auto multiply_chunk = [&](int c, auto first_tag) __attribute__((always_inline)) {
+    constexpr bool kFirst = decltype(first_tag)::value;
     const bool more = c + 1 < n_chunks;
     if(more) {
       if(!FUSED) stage_fetch(c + 1);
-#pragma unroll
-      for(int p = 0; p < Cfg::PW; ++p) {
-        const int s = (c + 1) * Cfg::CS + kw * Cfg::PW + p;
-        wnext[p] = load16(wrow + min(s, S - 1) * 32);
-      }
+      load_weights(c + 1, wnext);
     }
-    mask_weights(c);
+    if((c + 1) * Cfg::CS > S) mask_weights(c);
 #pragma unroll
     for(int p = 0; p < Cfg::PW; ++p) {
-      // FUSED keeps every sub-step in LDS; otherwise LDS holds the current chunk only.  Sub-steps
-      // past the end of K multiply zero weights; their LDS slot is clamped to a valid one.
-      int step = kw * Cfg::PW + p;
-      if(FUSED) step = min(c * Cfg::CS + step, S - 1);
 #pragma unroll
       for(int mt = 0; mt < MT32; ++mt) {
-        const v4i a = *reinterpret_cast<const v4i*>(
-            lds + (step * MT32 + mt) * kFragBytes + (lg * 32 + (li ^ stream32_row_key(2 * step + lg))) * 16);
-        acc[mt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(w[p], a, acc[mt], 0, 0, 0);
+        v4i a;
+        if(FUSED && !kFirst) {
+          const int step = min(c * Cfg::CS + step0 + p, S - 1);
+          a = *reinterpret_cast<const v4i*>(
+              lds + (step * MT32 + mt) * kFragBytes + (lg * 32 + (li ^ stream32_row_key(2 * step + lg))) * 16);
+        } else {
+          a = *reinterpret_cast<const v4i*>(frag0 + (p * MT32 + mt) * kFragBytes +
+                                            (akey ^ stream32_row_key(2 * p)) * 16);
+        }
+        if(kFirst && p == 0) {
+          const v16i_s zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+          acc[mt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(w[p], a, zero, 0, 0, 0);
+        } else {
+          acc[mt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(w[p], a, acc[mt], 0, 0, 0);
+        }
       }
     }
     if(more) {
@@ -386,7 +406,9 @@ __global__ __launch_bounds__(WN * KW * kWave) void gemm_stream32_kernel(GemmArgs
 #pragma unroll
       for(int p = 0; p < Cfg::PW; ++p) w[p] = wnext[p];
     }
-  }
+  };
+  multiply_chunk(0, std::true_type());
+  for(int c = 1; c < n_chunks; ++c) multiply_chunk(c, std::false_type());
 
   if(args.prof) tp[3] = clock64();
   // ---- every wave drops its 32 * MT32 x 32 tile of int32 partial sums into LDS as a row-major
