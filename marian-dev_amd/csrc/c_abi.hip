@@ -136,7 +136,8 @@ int launch_stream32(const GemmArgs& a, const FusedSrc& f, hipStream_t st) {
   if(MODE == kFusedAll && lds < stream32_fused_lds_bytes(MT32, a.K)) lds = stream32_fused_lds_bytes(MT32, a.K);
   if(lds < Cfg::kReduceBytes) lds = Cfg::kReduceBytes;
   int blocks = (a.n_out + Cfg::kColsPerBlock - 1) / Cfg::kColsPerBlock;
-  int m_tiles = MODE == kFusedAll ? 1 : (a.M + MT32 * 32 - 1) / (MT32 * 32);
+  constexpr int kRows = (MODE == kFusedTiled && NG == 2) ? 16 : MT32 * 32;   // activation rows per workgroup
+  int m_tiles = MODE == kFusedAll ? 1 : (a.M + kRows - 1) / kRows;
   GemmArgs a2 = a;
   if(a.absmax_out) {   // eight slots per workgroup, one per wave
     if((long long)blocks * m_tiles * Cfg::kWaves <= kAbsmaxSlots) t_absmax_written = true;
@@ -152,16 +153,22 @@ int launch_stream32(const GemmArgs& a, const FusedSrc& f, hipStream_t st) {
 // covers K in one chunk, else the largest whose activations fit the 64 KB LDS stage
 // (MT32 * KW * PW <= 64).  kFusedTiled stages fp32 values in registers: at most 4 per wave (8 when K is not split).
 template <int MT32, int MODE>
-int launch_stream32_kw(const GemmArgs& a, const FusedSrc& f, hipStream_t st, int kw) {
+int launch_stream32_kw(const GemmArgs& a, const FusedSrc& f, hipStream_t st, int kw, bool half_rows = false) {
   const int need = (a.K / 32 + kw - 1) / kw;   // sub-steps per wave if K is one chunk
   if constexpr(MODE == kFusedTiled) {
-    static_assert(MT32 == 1, "tiled fused form: 32 rows per workgroup");
+    static_assert(MT32 == 1, "tiled fused form: 32 (or 16) rows per workgroup");
     switch(kw) {
       case 1: return launch_stream32<1, 8, 1, 8, MODE>(a, f, st);
       case 2: return launch_stream32<1, 4, 2, 4, MODE>(a, f, st);
-      case 4: return launch_stream32<1, 2, 4, 4, MODE>(a, f, st);
+      case 4:
+        if(half_rows) return launch_stream32<1, 2, 4, 4, MODE, 2>(a, f, st);
+        return launch_stream32<1, 2, 4, 4, MODE>(a, f, st);
       default:
-        if(need > 2) return launch_stream32<1, 1, 8, 4, MODE>(a, f, st);
+        if(need > 2) {
+          if(half_rows) return launch_stream32<1, 1, 8, 4, MODE, 2>(a, f, st);
+          return launch_stream32<1, 1, 8, 4, MODE>(a, f, st);
+        }
+        if(half_rows) return launch_stream32<1, 1, 8, 2, MODE, 2>(a, f, st);
         return launch_stream32<1, 1, 8, 2, MODE>(a, f, st);
     }
   } else {
@@ -208,7 +215,14 @@ int launch_stream32_auto(const GemmArgs& a, const FusedSrc& f, hipStream_t st, i
   if(kw_override) kw = kw_override;
   while(kw > 1 && a.K / 32 < kw) kw >>= 1;
   if constexpr(MODE == kFusedTiled) {
-    return launch_stream32_kw<1, MODE>(a, f, st, kw);
+    // Every workgroup quantizes the activation rows it multiplies.  With 16 rows instead of 32
+    // that work halves and the workgroups double: taken when they still fit one per CU.
+    // (measurement ids 640 / 641 force 32 / 16 rows)
+    const int ov = g_kernel_override.load(std::memory_order_relaxed) % 1000;
+    const long long blocks32 = (long long)((tiles * kw + 7) / 8) * m_tiles;
+    const bool half_rows = kw >= 4 && ov != 640 &&
+                           (ov == 641 || (a.M > 16 && 2 * blocks32 <= compute_units()));
+    return launch_stream32_kw<1, MODE>(a, f, st, kw, half_rows);
   } else {
     if(mt == 1) return launch_stream32_kw<1, MODE>(a, f, st, kw);
     if(mt == 2) return launch_stream32_kw<2, MODE>(a, f, st, kw);

@@ -60,9 +60,11 @@ struct Stream32Cfg {
 
 // Dynamic LDS: one chunk (kStageBytes), for kFusedAll all of K (32 * MT32 * K bytes) if that is
 // more; at least kReduceBytes.  partials: n_partials (1..2048) abs-max values (kFusedTiled only).
-// NG (kFusedAll only): 16-value groups per thread that are compiled in, 2 or 4; all but the last
-// two are complete (the launcher picks NG = 2 for M * K <= 16384), so their loads, abs-max and
-// quantization carry no range checks.
+// NG, kFusedAll: 16-value groups per thread that are compiled in, 2 or 4; all but the last two are
+// complete (the launcher picks NG = 2 for M * K <= 16384), so their loads, abs-max and
+// quantization carry no range checks.  NG, kFusedTiled: 2 = a workgroup takes 16 activation rows
+// instead of 32 (MT32 = 1; half the quantizing per workgroup, twice the workgroups - for calls
+// that would otherwise leave half of the CUs idle), 4 = 32 rows.
 template <int MT32, int WN, int KW, int PW, int MODE, int NG = 4>
 __global__ __launch_bounds__(WN * KW * kWave) void gemm_stream32_kernel(GemmArgs args,
                                                                         const float* A,
@@ -91,7 +93,9 @@ __global__ __launch_bounds__(WN * KW * kWave) void gemm_stream32_kernel(GemmArgs
   const int K = args.K, M = args.M;
   const int S = K / 32;                                   // K sub-steps
   const int n_chunks = (S + Cfg::CS - 1) / Cfg::CS;
-  const int m_base = blockIdx.y * (MT32 * 32);            // activation rows of this workgroup
+  constexpr int R = (TILED && NG == 2) ? 16 : MT32 * 32;   // activation rows of this workgroup
+  static_assert(R == MT32 * 32 || (MT32 == 1 && Cfg::CS % 16 == 0), "half-height tiles");
+  const int m_base = blockIdx.y * R;
 
   // Loads of a wave return in issue order and the compiler counts them: a value is waited for
   // with "all but the N youngest loads", and N can only count loads that are certain to have been
@@ -174,7 +178,7 @@ __global__ __launch_bounds__(WN * KW * kWave) void gemm_stream32_kernel(GemmArgs
   // Pre-quantized: thread slot (sub-step, m-tile, lane) in operand order.  kFusedTiled: fp32
   // source; group = row * 2 * CS + 16-byte chunk, a quad of lanes takes four consecutive groups
   // (a wave reads whole rows), quantizes them and finds the operand slots from there.
-  constexpr int kStageVecs = Cfg::CS * MT32 * 64 / kStream32Threads;
+  constexpr int kStageVecs = Cfg::CS * R * 2 / kStream32Threads;
   v4i stage[TILED ? 1 : kStageVecs];
   v4f stagef[TILED ? kStageVecs : 1][4];
   auto stage_fetch = [&](int chunk) __attribute__((always_inline)) {
@@ -219,8 +223,6 @@ __global__ __launch_bounds__(WN * KW * kWave) void gemm_stream32_kernel(GemmArgs
         const int slot0 = ((c16 / 2) * MT32 + r / 32) * 64, x = (r % 32) ^ stream32_row_key(c16);
 #pragma unroll
         for(int e = 0; e < 4; ++e) {
-          // rows past M hold zeros (sub-steps past K multiply zero weights, any value will do)
-          if(m >= M) q[e] = 0;
           const int s = chunk * Cfg::CS + (c16 + e) / 2;
           const int sw = slot0 + (e / 2) * MT32 * 64 + (e % 2) * 32 + (x ^ e);
           *reinterpret_cast<uint32_t*>(lds + sw * 16 + (slot % 4) * 4) = q[e];
@@ -229,10 +231,9 @@ __global__ __launch_bounds__(WN * KW * kWave) void gemm_stream32_kernel(GemmArgs
         }
       } else {
         const int l = slot % 64, f = slot / 64;
-        const int mt = f % MT32, step = f / MT32;
+        const int step = f / MT32;
         const int sw = (slot & ~31) | ((l % 32) ^ stream32_row_key(2 * step + l / 32));
-        const bool live = m_base + mt * 32 + (l % 32) < M;
-        *reinterpret_cast<v4i*>(lds + sw * 16) = live ? stage[j] : v4i{0, 0, 0, 0};
+        *reinterpret_cast<v4i*>(lds + sw * 16) = stage[j];   // (rows past M: a copy of row M - 1, never stored)
       }
     }
   };
@@ -297,12 +298,10 @@ __global__ __launch_bounds__(WN * KW * kWave) void gemm_stream32_kernel(GemmArgs
         if(!in_range(j)) vals[j][e] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
         amax = abs4max(vals[j][e], amax);
       }
-    // zero the rows between M and the end of the last 32-row tile (whole LDS stage, cheap)
-    if(M < MT32 * 32) {
-      for(int i = tid; i < S * MT32 * 64; i += kStream32Threads)
-        reinterpret_cast<v4i*>(lds)[i] = v4i{0, 0, 0, 0};
-    }
-    amax = block_max(amax, red);   // its barriers also order the zero fill before the writes
+    // (activation rows between M and the end of the last 32-row tile stay whatever LDS holds: a
+    // row only feeds its own output row, integer products cannot trap, and rows past M are never
+    // stored)
+    amax = block_max(amax, red);
     if(args.prof) tp[1] = clock64();
     aqm = quant_mult_from_maxabs(amax);
     // with a finite non-zero abs-max no product can leave [-127.0001, 127.0001]
@@ -418,7 +417,6 @@ __global__ __launch_bounds__(WN * KW * kWave) void gemm_stream32_kernel(GemmArgs
   //      any order) and stores whole 128-byte output rows, eight lanes per row.  Accumulator
   //      value v of tile mt in lane (li, lg) is activation row mt * 32 + li, weight row
   //      8 * (v / 4) + 4 * lg + v % 4, i.e. piece 2 * (v / 4) + lg of that row. ----
-  constexpr int R = MT32 * 32;                 // activation rows of the workgroup
   constexpr int kTileBytes = R * 128;
   __syncthreads();   // every wave is done reading activations from LDS
   {
@@ -428,6 +426,7 @@ __global__ __launch_bounds__(WN * KW * kWave) void gemm_stream32_kernel(GemmArgs
 #pragma unroll
       for(int q = 0; q < 4; ++q) {
         const int m = mt * 32 + li, piece = (2 * q + lg) ^ (li & 7);
+        if(R < 32 && li >= R) continue;
         *reinterpret_cast<v4i*>(mine + m * 128 + piece * 16) =
             v4i{acc[mt][4 * q], acc[mt][4 * q + 1], acc[mt][4 * q + 2], acc[mt][4 * q + 3]};
       }
