@@ -192,6 +192,26 @@ int launch_stream32_kw(const GemmArgs& a, const FusedSrc& f, hipStream_t st, int
   }
 }
 
+// The K split and the tile height of the tiled fused form for a call.  K split: the widest (most
+// loads in flight per weight row) that stays within one workgroup per CU, the narrowest if none
+// does.  Every workgroup quantizes the activation rows it multiplies; with 16 rows instead of 32
+// that work halves and the workgroups double - taken when they still fit one per CU.
+struct TiledPlan {
+  int kw;
+  bool half_rows;
+};
+TiledPlan plan_tiled(int M, int K, int n_out, int kw_override) {
+  const int tiles = (n_out + 31) / 32, m_tiles = (M + 31) / 32;
+  int kw = 8;
+  while(kw > 1 && (long long)((tiles * kw + 7) / 8) * m_tiles > compute_units()) kw >>= 1;
+  if(kw_override) kw = kw_override;
+  while(kw > 1 && K / 32 < kw) kw >>= 1;
+  const int ov = g_kernel_override.load(std::memory_order_relaxed) % 1000;   // 640 / 641: force 32 / 16 rows
+  const long long blocks32 = (long long)((tiles * kw + 7) / 8) * m_tiles;
+  const bool half_rows = kw >= 4 && ov != 640 && (ov == 641 || (M > 16 && 2 * blocks32 <= compute_units()));
+  return TiledPlan{kw, half_rows};
+}
+
 // kw_override: 0 = pick the K split from the number of workgroups it gives.
 // mt_override: 0 = activation rows per workgroup chosen here (kFusedAll takes all of M,
 // kFusedTiled 32).
@@ -215,14 +235,8 @@ int launch_stream32_auto(const GemmArgs& a, const FusedSrc& f, hipStream_t st, i
   if(kw_override) kw = kw_override;
   while(kw > 1 && a.K / 32 < kw) kw >>= 1;
   if constexpr(MODE == kFusedTiled) {
-    // Every workgroup quantizes the activation rows it multiplies.  With 16 rows instead of 32
-    // that work halves and the workgroups double: taken when they still fit one per CU.
-    // (measurement ids 640 / 641 force 32 / 16 rows)
-    const int ov = g_kernel_override.load(std::memory_order_relaxed) % 1000;
-    const long long blocks32 = (long long)((tiles * kw + 7) / 8) * m_tiles;
-    const bool half_rows = kw >= 4 && ov != 640 &&
-                           (ov == 641 || (a.M > 16 && 2 * blocks32 <= compute_units()));
-    return launch_stream32_kw<1, MODE>(a, f, st, kw, half_rows);
+    const TiledPlan plan = plan_tiled(a.M, a.K, a.n_out, kw_override);
+    return launch_stream32_kw<1, MODE>(a, f, st, plan.kw, plan.half_rows);
   } else {
     if(mt == 1) return launch_stream32_kw<1, MODE>(a, f, st, kw);
     if(mt == 2) return launch_stream32_kw<2, MODE>(a, f, st, kw);
@@ -494,12 +508,19 @@ static int affine_f32_impl(const float* A, int8_t* Aq, const int8_t* Bq, const f
     if(which >= 611 && which <= 618) kw = which - 610;
     return launch_stream32_auto<kFusedAll>(a, f, hst, kw);
   }
-  // Mid-size activations: every workgroup quantizes its own 32 rows, so the work is repeated
-  // once per 32..256 output columns; measured to pay (one launch fewer) only for short rows and
-  // moderate output widths.
+  // Mid-size activations: every workgroup quantizes its own 16 or 32 rows, so the work is
+  // repeated once per 32..256 output columns; measured to pay (one launch fewer) for short rows
+  // and moderate output widths, and for longer rows when few columns leave room for 16-row
+  // workgroups with an eight-way K split (at most 64 K values per workgroup).
   const bool tiled_ok = n_out > 0 && workspace && workspace_bytes >= kWorkspaceBytes &&
                         aligned(workspace, 4);
-  if(tiled_ok && which != 600 && (want_tiled || (M <= 256 && K <= 1024 && n_out <= 8192))) {
+  bool tiled = want_tiled;
+  if(tiled_ok && !tiled && M <= 256 && n_out <= 8192) {
+    const TiledPlan plan = plan_tiled((int)M, (int)K, (int)n_out, 0);
+    tiled = K <= 1024 ||
+            (K <= 4096 && plan.kw == 8 && (long long)(plan.half_rows ? 16 : 32) * K <= 65536);
+  }
+  if(tiled_ok && which != 600 && tiled) {
     if(absmax_in) {   // the producer of A left its abs-max: no launch for it
       f.partials = absmax_in;
       f.n_partials = kAbsmaxSlots;
