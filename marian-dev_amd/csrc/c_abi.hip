@@ -121,13 +121,14 @@ struct FusedSrc {   // what the fused modes read and write besides GemmArgs
   int n_partials = 0;
 };
 
-template <int MT32, int WN, int KW, int PW, int MODE, int NG = 4>
+template <int MT32, int WN, int KW, int PW, int MODE, int ROWS = 32 * MT32, int NG = 4>
 int launch_stream32(const GemmArgs& a, const FusedSrc& f, hipStream_t st) {
   if constexpr(MODE == kFusedAll && NG == 4) {   // at most two groups of 16 values per thread
-    if((long long)a.M * a.K <= kFusedMaxElems / 2) return launch_stream32<MT32, WN, KW, PW, MODE, 2>(a, f, st);
+    if((long long)a.M * a.K <= kFusedMaxElems / 2)
+      return launch_stream32<MT32, WN, KW, PW, MODE, ROWS, 2>(a, f, st);
   }
   using Cfg = Stream32Cfg<MT32, WN, KW, PW>;
-  auto kernel = gemm_stream32_kernel<MT32, WN, KW, PW, MODE, NG>;
+  auto kernel = gemm_stream32_kernel<MT32, WN, KW, PW, MODE, NG, ROWS>;
   constexpr int kMaxLds = 64 * 1024 > Cfg::kLdsBytes ? 64 * 1024 : Cfg::kLdsBytes;
   static const int lds_status = allow_lds(kernel, kMaxLds);
   if(lds_status != MARIAN_HIP_OK) return lds_status;
@@ -136,8 +137,7 @@ int launch_stream32(const GemmArgs& a, const FusedSrc& f, hipStream_t st) {
   if(MODE == kFusedAll && lds < stream32_fused_lds_bytes(MT32, a.K)) lds = stream32_fused_lds_bytes(MT32, a.K);
   if(lds < Cfg::kReduceBytes) lds = Cfg::kReduceBytes;
   int blocks = (a.n_out + Cfg::kColsPerBlock - 1) / Cfg::kColsPerBlock;
-  constexpr int kRows = (MODE == kFusedTiled && NG == 2) ? 16 : MT32 * 32;   // activation rows per workgroup
-  int m_tiles = MODE == kFusedAll ? 1 : (a.M + kRows - 1) / kRows;
+  int m_tiles = (a.M + ROWS - 1) / ROWS;   // (kFusedAll with full-height tiles: M <= ROWS)
   GemmArgs a2 = a;
   if(a.absmax_out) {   // eight slots per workgroup, one per wave
     if((long long)blocks * m_tiles * Cfg::kWaves <= kAbsmaxSlots) t_absmax_written = true;
@@ -161,14 +161,14 @@ int launch_stream32_kw(const GemmArgs& a, const FusedSrc& f, hipStream_t st, int
       case 1: return launch_stream32<1, 8, 1, 8, MODE>(a, f, st);
       case 2: return launch_stream32<1, 4, 2, 4, MODE>(a, f, st);
       case 4:
-        if(half_rows) return launch_stream32<1, 2, 4, 4, MODE, 2>(a, f, st);
+        if(half_rows) return launch_stream32<1, 2, 4, 4, MODE, 16>(a, f, st);
         return launch_stream32<1, 2, 4, 4, MODE>(a, f, st);
       default:
         if(need > 2) {
-          if(half_rows) return launch_stream32<1, 1, 8, 4, MODE, 2>(a, f, st);
+          if(half_rows) return launch_stream32<1, 1, 8, 4, MODE, 16>(a, f, st);
           return launch_stream32<1, 1, 8, 4, MODE>(a, f, st);
         }
-        if(half_rows) return launch_stream32<1, 1, 8, 2, MODE, 2>(a, f, st);
+        if(half_rows) return launch_stream32<1, 1, 8, 2, MODE, 16>(a, f, st);
         return launch_stream32<1, 1, 8, 2, MODE>(a, f, st);
     }
   } else {
@@ -181,6 +181,13 @@ int launch_stream32_kw(const GemmArgs& a, const FusedSrc& f, hipStream_t st, int
         }
         return launch_stream32<MT32, 2, 4, 4, MODE>(a, f, st);
       default:
+        if constexpr(MT32 == 1 && MODE == kFusedAll) {
+          if(half_rows) {
+            if(need > 4) return launch_stream32<1, 1, 8, 8, MODE, 16>(a, f, st);
+            if(need > 2) return launch_stream32<1, 1, 8, 4, MODE, 16>(a, f, st);
+            return launch_stream32<1, 1, 8, 2, MODE, 16>(a, f, st);
+          }
+        }
         if constexpr(MT32 == 1) {
           if(need > 4) return launch_stream32<MT32, 1, 8, 8, MODE>(a, f, st);
         }
@@ -238,6 +245,15 @@ int launch_stream32_auto(const GemmArgs& a, const FusedSrc& f, hipStream_t st, i
     const TiledPlan plan = plan_tiled(a.M, a.K, a.n_out, kw_override);
     return launch_stream32_kw<1, MODE>(a, f, st, plan.kw, plan.half_rows);
   } else {
+    if constexpr(MODE == kFusedAll) {
+      // Few weight tiles: 16-row workgroups (all of them take the abs-max over the whole input,
+      // each quantizes and multiplies its own rows), if they fit one per CU with the widest K
+      // split.  (measurement ids 650 / 651 force full-height / 16-row workgroups)
+      const int ov = g_kernel_override.load(std::memory_order_relaxed) % 1000;
+      const bool rows16 = a.K / 32 >= 8 && !kw_override && ov != 650 &&
+                          (ov == 651 || (a.M > 16 && (long long)tiles * ((a.M + 15) / 16) <= compute_units()));
+      if(rows16) return launch_stream32_kw<1, MODE>(a, f, st, 8, true);
+    }
     if(mt == 1) return launch_stream32_kw<1, MODE>(a, f, st, kw);
     if(mt == 2) return launch_stream32_kw<2, MODE>(a, f, st, kw);
     return launch_stream32_kw<4, MODE>(a, f, st, kw);

@@ -60,12 +60,14 @@ struct Stream32Cfg {
 
 // Dynamic LDS: one chunk (kStageBytes), for kFusedAll all of K (32 * MT32 * K bytes) if that is
 // more; at least kReduceBytes.  partials: n_partials (1..2048) abs-max values (kFusedTiled only).
-// NG, kFusedAll: 16-value groups per thread that are compiled in, 2 or 4; all but the last two are
+// NG (kFusedAll): 16-value groups per thread that are compiled in, 2 or 4; all but the last two are
 // complete (the launcher picks NG = 2 for M * K <= 16384), so their loads, abs-max and
-// quantization carry no range checks.  NG, kFusedTiled: 2 = a workgroup takes 16 activation rows
-// instead of 32 (MT32 = 1; half the quantizing per workgroup, twice the workgroups - for calls
-// that would otherwise leave half of the CUs idle), 4 = 32 rows.
-template <int MT32, int WN, int KW, int PW, int MODE, int NG = 4>
+// quantization carry no range checks.
+// ROWS: activation rows a workgroup multiplies, 32 * MT32 or (fused forms, MT32 = 1) 16: half the
+// quantizing per workgroup and twice the workgroups, for calls that would otherwise leave most
+// CUs idle.  With ROWS < M the kFusedAll form still takes the abs-max over all of A in every
+// workgroup and quantizes only its own rows.
+template <int MT32, int WN, int KW, int PW, int MODE, int NG = 4, int ROWS = 32 * MT32>
 __global__ __launch_bounds__(WN * KW * kWave) void gemm_stream32_kernel(GemmArgs args,
                                                                         const float* A,
                                                                         int8_t* aq_out,
@@ -93,8 +95,9 @@ __global__ __launch_bounds__(WN * KW * kWave) void gemm_stream32_kernel(GemmArgs
   const int K = args.K, M = args.M;
   const int S = K / 32;                                   // K sub-steps
   const int n_chunks = (S + Cfg::CS - 1) / Cfg::CS;
-  constexpr int R = (TILED && NG == 2) ? 16 : MT32 * 32;   // activation rows of this workgroup
-  static_assert(R == MT32 * 32 || (MT32 == 1 && Cfg::CS % 16 == 0), "half-height tiles");
+  constexpr int R = ROWS;   // activation rows of this workgroup
+  static_assert(R == MT32 * 32 || (R == 16 && MT32 == 1 && MODE != kPrequant && (FUSED || Cfg::CS % 16 == 0)),
+                "half-height tiles");
   const int m_base = blockIdx.y * R;
 
   // Loads of a wave return in issue order and the compiler counts them: a value is waited for
@@ -312,7 +315,8 @@ __global__ __launch_bounds__(WN * KW * kWave) void gemm_stream32_kernel(GemmArgs
     uint32_t q[kFusedGroups][4];
 #pragma unroll
     for(int j = 0; j < kFusedGroups; ++j) {
-      if(in_range(j)) {
+      const unsigned rr = row - m_base;   // row within this workgroup's tile
+      if(in_range(j) && rr < (unsigned)R) {
         if(finite) {
 #pragma unroll
           for(int e = 0; e < 4; ++e) q[j][e] = quantize_pack4_finite(vals[j][e], aqm);
@@ -322,7 +326,7 @@ __global__ __launch_bounds__(WN * KW * kWave) void gemm_stream32_kernel(GemmArgs
         }
         // slot of group e: chunk c16 + e, i.e. sub-step (c16 + e) / 2, half (c16 + e) % 2, and
         // the row permuted by the key of chunk c16 + e, which is the key of c16 (c16 % 4 == 0) ^ e
-        const unsigned slot0 = ((c16 >> 1) * MT32 + (row >> 5)) * 64, x = (row & 31) ^ stream32_row_key(c16);
+        const unsigned slot0 = ((c16 >> 1) * MT32 + (rr >> 5)) * 64, x = (rr & 31) ^ stream32_row_key(c16);
 #pragma unroll
         for(int e = 0; e < 4; ++e) {
           const unsigned slot = slot0 + (e / 2) * MT32 * 64 + (e % 2) * 32 + (x ^ e);
@@ -340,14 +344,14 @@ __global__ __launch_bounds__(WN * KW * kWave) void gemm_stream32_kernel(GemmArgs
 #pragma unroll
       for(int j = 0; j < kFusedGroups; ++j) {
         const int g = 4 * (j * (kStream32Threads / 4) + quad);
-        if(in_range(j)) {
+        if(in_range(j) && (unsigned)(g / (int)k16n - m_base) < (unsigned)R) {
 #pragma unroll
           for(int e = 0; e < 4; ++e)
             *reinterpret_cast<uint32_t*>(aq_out + (size_t)(g + e) * 16 + qlane * 4) = q[j][e];
         }
       }
     }
-    if(aq_out && blockIdx.x == 0 && tid == 0)
+    if(aq_out && blockIdx.x == 0 && blockIdx.y == 0 && tid == 0)
       *reinterpret_cast<float*>(aq_out + (size_t)M * K) = aqm;
     __syncthreads();
   }
