@@ -266,11 +266,6 @@ __global__ __launch_bounds__(WN * KW * kWave) void gemm_stream32_kernel(GemmArgs
     for(int p = 0; p < Cfg::PW; ++p)
       if(chunk * Cfg::CS + kw * Cfg::PW + p >= S) w[p] = v4i{0, 0, 0, 0};
   };
-  // A CU's vector memory pipeline answers in request order, across its waves too: activation
-  // requests (cache hits) queued behind another wave's weight requests (HBM) would wait for those.
-  // The barrier puts every activation request of the workgroup ahead of every weight request.
-  __builtin_amdgcn_sched_barrier(0);
-  __builtin_amdgcn_s_barrier();
   __builtin_amdgcn_sched_barrier(0);
   load_weights(0, w);   // in flight while the activations are prepared
   __builtin_amdgcn_sched_barrier(0);
