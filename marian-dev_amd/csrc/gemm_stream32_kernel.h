@@ -112,9 +112,10 @@ __global__ __launch_bounds__(WN * KW * kWave) void gemm_stream32_kernel(GemmArgs
   //      sits (see the epilogue), both through the shortlist ids when there are any ----
   const int n0 = (blockIdx.x * WN + wn) * 32;
   int wsrc = min(n0 + li, args.n_out - 1);
+  const int bias_n = min(n0 + 4 * (lane % 8), args.n_out - 4);   // n_out % 8 == 0: four valid columns
   uint32_t bias_at[4];
 #pragma unroll
-  for(int e = 0; e < 4; ++e) bias_at[e] = (uint32_t)min(n0 + 4 * (lane % 8) + e, args.n_out - 1);
+  for(int e = 0; e < 4; ++e) bias_at[e] = (uint32_t)(bias_n + e);
   if(args.idx) {
     if(args.bias) {
 #pragma unroll
@@ -155,7 +156,6 @@ __global__ __launch_bounds__(WN * KW * kWave) void gemm_stream32_kernel(GemmArgs
   if(FUSED) {
     // a quad's four groups are 256 consecutive bytes; group set j starts 32 KB after set j - 1
     const char* a_quad = reinterpret_cast<const char*>(A) + quad * 256 + qlane * 16;
-    const v4f* a4 = reinterpret_cast<const v4f*>(A);
 #pragma unroll
     for(int j = 0; j < kFusedGroups; ++j) {
       if(j < kFullGroups) {
@@ -163,12 +163,18 @@ __global__ __launch_bounds__(WN * KW * kWave) void gemm_stream32_kernel(GemmArgs
         for(int e = 0; e < 4; ++e)
           vals[j][e] = *reinterpret_cast<const v4f*>(a_quad + j * (kStream32Threads * 64) + e * 64);
       } else {
+        // (a wave whose 64 groups are all out of range skips the loads; a thread past the end
+        // reads a copy of the last groups, which is never looked at)
         const int g0 = min(4 * (j * (kStream32Threads / 4) + quad), n16 - 4);
+        const char* a_part = reinterpret_cast<const char*>(A) + (size_t)g0 * 64 + qlane * 16;
 #pragma unroll
         for(int e = 0; e < 4; ++e) {
-          vals[j][e] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
-          // (a wave whose 64 groups are all out of range skips the loads)
-          if(j * kStream32Threads + wave_s * kWave < n16) vals[j][e] = a4[(g0 + e) * 4 + qlane];
+          // (any value: never looked at.  Not zero - the compiler would share the register of an
+          // existing zero constant with one component and then has to copy the loaded value into
+          // it, waiting for the load right after issuing it)
+          vals[j][e] = v4f{1.0f, 1.0f, 1.0f, 1.0f};
+          if(j * kStream32Threads + wave_s * kWave < n16)
+            vals[j][e] = *reinterpret_cast<const v4f*>(a_part + e * 64);
         }
       }
     }
@@ -290,12 +296,12 @@ __global__ __launch_bounds__(WN * KW * kWave) void gemm_stream32_kernel(GemmArgs
   if(FUSED) {
     // whole A (M*K <= kFusedMaxElems floats) in registers: abs-max, then quantize into LDS
 #pragma unroll
-    for(int j = 0; j < kFusedGroups; ++j)
+    for(int j = 0; j < kFusedGroups; ++j) {
+      if(in_range(j)) {
 #pragma unroll
-      for(int e = 0; e < 4; ++e) {
-        if(!in_range(j)) vals[j][e] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
-        amax = abs4max(vals[j][e], amax);
+        for(int e = 0; e < 4; ++e) amax = abs4max(vals[j][e], amax);
       }
+    }
     // (activation rows between M and the end of the last 32-row tile stay whatever LDS holds: a
     // row only feeds its own output row, integer products cannot trap, and rows past M are never
     // stored)

@@ -1,0 +1,70 @@
+"""The small-M kernel relies on a property of the generated code: between the wait for the shortlist
+ids and the last load of the prologue there is no other wait on vector loads, so activations,
+weights and bias are all requested before the wave blocks for the first time (a single early wait
+costs a memory round trip per call).  The compiler decides where waits go, and small source changes
+have moved them; this test compiles the device code to assembly and checks every fully fused
+instantiation (MODE 1) and every pre-quantized one (MODE 0)."""
+import os
+import re
+import shutil
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+CSRC = os.path.join(ROOT, "marian-dev_amd", "csrc")
+HIPCC = "/opt/rocm/bin/hipcc"
+
+
+@pytest.fixture(scope="module")
+def assembly(tmp_path_factory):
+    if not os.path.exists(HIPCC):
+        pytest.skip("hipcc not available")
+    flags = None
+    for line in open(os.path.join(CSRC, "Makefile")).read().replace("\\\n", " ").splitlines():
+        if line.startswith("HIPFLAGS"):
+            flags = line.split("=", 1)[1].replace("$(ARCH)", "gfx950").split()
+    assert flags, "HIPFLAGS not found in the Makefile"
+    flags = [f for f in flags if f not in ("-fPIC", "-shared")]
+    out = tmp_path_factory.mktemp("asm") / "c_abi.s"
+    cmd = [HIPCC] + flags + ["-S", "--cuda-device-only", "-o", str(out), "c_abi.hip"]
+    r = subprocess.run(cmd, cwd=CSRC, capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr[-2000:]
+    return open(out).read().split("\n")
+
+
+def kernels(lines):
+    for i, l in enumerate(lines):
+        m = re.match(r"^(_ZN10marian_hip20gemm_stream32_kernelILi(\d)ELi(\d)ELi(\d)ELi(\d)ELi(\d)ELi(\d)ELi(\d+)E\w*):", l)
+        if m:
+            end = next(j for j in range(i, len(lines)) if "s_endpgm" in lines[j])
+            yield m.group(1), tuple(int(x) for x in m.groups()[1:]), lines[i:end]
+
+
+def test_no_wait_between_ids_and_last_prologue_load(assembly):
+    checked = 0
+    for name, (mt32, wn, kw, pw, mode, ng, rows), body in kernels(assembly):
+        if mode == 2:      # quantize-on-stage: the abs-max partials are waited for first, by design
+            continue
+        first_barrier = next(i for i, l in enumerate(body) if "s_barrier" in l)
+        loads = [i for i, l in enumerate(body[:first_barrier]) if "global_load" in l]
+        waits = [i for i, l in enumerate(body[:first_barrier]) if re.search(r"s_waitcnt.*vmcnt", l)]
+        assert loads and waits, name
+        # waits[0] is the one for the shortlist ids (vmcnt(0) with nothing else in flight)
+        early = [w for w in waits[1:] if w < loads[-1]]
+        assert not early, "%s: wait on vector loads at line %d, before the last prologue load at %d" % (
+            name, early[0], loads[-1])
+        checked += 1
+    assert checked >= 30, "expected the fused and pre-quantized instantiations, found %d" % checked
+
+
+def test_no_scratch_memory_in_stream32_kernels(assembly):
+    """Register arrays indexed through a lambda that is not inlined end up in scratch memory (a
+    forty-fold slowdown was measured); every instantiation must report a zero private segment."""
+    text = "\n".join(assembly)
+    found = 0
+    for m in re.finditer(r"\.name:\s+(_ZN10marian_hip20gemm_stream32_kernel\w+)\n(.*?)\.wavefront_size", text, re.S):
+        meta = dict(re.findall(r"\.(vgpr_spill_count|private_segment_fixed_size):\s+(\d+)", m.group(2)))
+        assert int(meta["private_segment_fixed_size"]) == 0 and int(meta["vgpr_spill_count"]) == 0, (m.group(1), meta)
+        found += 1
+    assert found >= 40
