@@ -246,6 +246,23 @@ int launch_stream32_auto(const GemmArgs& a, const FusedSrc& f, hipStream_t st, i
     return launch_stream32_kw<1, MODE>(a, f, st, plan.kw, plan.half_rows);
   } else {
     if constexpr(MODE == kFusedAll) {
+      // The smallest inputs (at most two 16-value groups per thread of four waves): one wave per
+      // SIMD.  The kernel is a chain of short dependent phases there, bound by instruction issue,
+      // and a wave that has its SIMD to itself issues twice as fast.  (K up to 1024: one chunk.)
+      // (measurement ids 660 / 661 force eight / four waves)
+      {
+        const int ov = g_kernel_override.load(std::memory_order_relaxed) % 1000;
+        const int S = a.K / 32;
+        const bool four = !kw_override && ov != 660 && ov != 650 && ov != 651 && S >= 8 && S <= 32 &&
+                          (long long)a.M * a.K <= 2 * 16 * 256 && a.M <= 32 &&
+                          (ov == 661 || tiles <= compute_units());
+        if(four) {
+          const int need = (S + 3) / 4;
+          if(need > 4) return launch_stream32<1, 1, 4, 8, MODE, 32, 2>(a, f, st);
+          if(need > 2) return launch_stream32<1, 1, 4, 4, MODE, 32, 2>(a, f, st);
+          return launch_stream32<1, 1, 4, 2, MODE, 32, 2>(a, f, st);
+        }
+      }
       // Few weight tiles: 16-row workgroups (all of them take the abs-max over the whole input,
       // each quantizes and multiplies its own rows), if they fit one per CU with the widest K
       // split.  (measurement ids 650 / 651 force full-height / 16-row workgroups)

@@ -7,7 +7,8 @@
 // small quantized activations are the column operand; a workgroup keeps them in LDS in operand
 // order (within a fragment the 32 rows of a K chunk are XOR-permuted by a key of the chunk number,
 // which spreads the quantizer's 4-byte writes over the LDS banks and keeps the fragment reads
-// conflict free).  The 8 waves of a workgroup are arranged WN (different weight rows) x KW (different K
+// conflict free).  The 8 waves of a workgroup (4 for the smallest inputs: a wave then has its SIMD
+// to itself and issues an instruction every 4 clocks instead of every 8) are arranged WN (different weight rows) x KW (different K
 // ranges of the same rows); the KW partial sums are added through LDS (exact in any order).
 //
 // MODE kFusedAll: the workgroup reads the fp32 activations itself, takes their abs-max (every
@@ -46,7 +47,7 @@ template <int MT32, int WN, int KW, int PW_>
 struct Stream32Cfg {
   static constexpr int kWaves = WN * KW;
   static constexpr int kThreads = kWaves * kWave;
-  static_assert(kWaves == 8, "eight waves");
+  static_assert(kWaves == 8 || kWaves == 4, "eight waves, or four (one per SIMD) for the smallest inputs");
   static constexpr int kColsPerBlock = WN * 32;
   static constexpr int PW = PW_;
   static constexpr int CS = PW * KW;
@@ -75,9 +76,11 @@ __global__ __launch_bounds__(WN * KW * kWave) void gemm_stream32_kernel(GemmArgs
                                                                         int n_partials) {
   using Cfg = Stream32Cfg<MT32, WN, KW, PW>;
   constexpr int kStream32Waves = Cfg::kWaves, kStream32Threads = Cfg::kThreads;
+  constexpr bool TILED_ = MODE == kFusedTiled;
   constexpr int kFusedGroups = NG, kFullGroups = NG - 2;
   static_assert(NG == 2 || NG == 4, "groups per thread");
-  static_assert(kFusedMaxElems == 4 * 16 * Cfg::kThreads, "four groups per thread hold the largest fused input");
+  static_assert(kFusedMaxElems == 4 * 16 * kWave * 8, "four groups per thread of eight waves hold the largest fused input");
+  static_assert(!TILED_ || Cfg::kWaves == 8, "the abs-max partials are read by 512 threads");
   constexpr bool FUSED = MODE == kFusedAll;
   constexpr bool TILED = MODE == kFusedTiled;
   extern __shared__ __attribute__((aligned(16))) int8_t lds[];
