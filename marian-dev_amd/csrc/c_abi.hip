@@ -78,11 +78,11 @@ int launch_tile(const GemmArgs& a, hipStream_t st) {
   return MARIAN_HIP_OK;
 }
 
-template <int BM, int BN, int WM, int WN, int NSTAGE, bool PAIRED = true>
+template <int BM, int BN, int WM, int WN, int NSTAGE, bool PAIRED = true, bool NT = false>
 int launch_big(const GemmArgs& a, hipStream_t st) {
   using Cfg = BigCfg<BM, BN, WM, WN, NSTAGE>;
   if(a.K % Cfg::BK != 0) return launch_tile<4, 4>(a, st);  // this family needs K % 128 == 0
-  auto kernel = gemm_mfma32_kernel<BM, BN, WM, WN, NSTAGE, PAIRED>;
+  auto kernel = gemm_mfma32_kernel<BM, BN, WM, WN, NSTAGE, PAIRED, NT>;
   static const int lds_status = allow_lds(kernel, Cfg::kLdsBytes);
   if(lds_status != MARIAN_HIP_OK) return lds_status;
   int tiles_n = (a.n_out + BN - 1) / BN;
@@ -375,7 +375,13 @@ int launch_gemm(const GemmArgs& a, hipStream_t st) {
   // large outputs: 256x256 tiles (one per CU keeps operand traffic lowest); otherwise 128x128
   // tiles with a three-deep LDS ring so that enough loads are in flight per CU
   const long long tiles256 = ((a.M + 255) / 256) * (long long)((a.n_out + 255) / 256);
-  if(tiles256 >= 192) return launch_big<256, 256, 2, 4, 2>(a, st);
+  // an output that would fit the L2 caches (8 x 4 MB) is streamed out with non-temporal stores
+  const bool stream_out = (long long)a.M * a.n_out * 4 <= (32ll << 20) && !a.dump;
+  if(tiles256 >= 192) {
+    if(stream_out) return launch_big<256, 256, 2, 4, 2, true, true>(a, st);
+    return launch_big<256, 256, 2, 4, 2>(a, st);
+  }
+  if(stream_out) return launch_big<128, 128, 2, 2, 3, true, true>(a, st);
   return launch_big<128, 128, 2, 2, 3>(a, st);
 }
 
