@@ -474,7 +474,12 @@ __global__ __launch_bounds__(WN * KW * kWave) void gemm_stream32_kernel(GemmArgs
         if(args.relu) y[e] = y[e] > 0.0f ? y[e] : 0.0f;
         omax = fmaxf(omax, fabsf(y[e]));
       }
-      *reinterpret_cast<v4f*>(reinterpret_cast<float*>(args.out) + off) = v4f{y[0], y[1], y[2], y[3]};
+      v4f* dst = reinterpret_cast<v4f*>(reinterpret_cast<float*>(args.out) + off);
+      const v4f yv = v4f{y[0], y[1], y[2], y[3]};
+      // (written out: behind a branch the compiler merges a non-temporal builtin store and a plain
+      // one into one plain store)
+      if(args.stream_out) asm volatile("global_store_dwordx4 %0, %1, off nt" : : "v"(dst), "v"(yv) : "memory");
+      else *dst = yv;
     }
   }
   if(args.absmax_out && !args.dump) {

@@ -103,6 +103,9 @@ struct GemmArgs {
   // kAbsmaxSlots floats that receive values whose maximum is max|out| (the next call's abs-max,
   // taken where the tensor is produced), or null
   float* absmax_out = nullptr;
+  // write the output with non-temporal stores (set by the launchers for outputs of several MB,
+  // which would otherwise sit dirty in L2 until the kernel ends and be written back then)
+  int stream_out = 0;
 };
 
 constexpr int kAbsmaxSlots = 2048;
