@@ -139,8 +139,10 @@ int launch_stream32(const GemmArgs& a, const FusedSrc& f, hipStream_t st) {
   int blocks = (a.n_out + Cfg::kColsPerBlock - 1) / Cfg::kColsPerBlock;
   int m_tiles = (a.M + ROWS - 1) / ROWS;   // (kFusedAll with full-height tiles: M <= ROWS)
   GemmArgs a2 = a;
-  // (measured: 10.1 instead of 11.1 us for the 8 MB output of the 64 x 32000 call; outputs of
-  // less than a MB are up to 0.5 us slower with them)
+  // (measured: 10.0 instead of 11.1 us for the 8 MB output of the 64 x 32000 call; outputs of
+  // less than a MB are up to 0.5 us slower with them.  The next kernel then finds the output in
+  // HBM rather than in the memory-side cache: a log-softmax over 16 MB of logits takes 14.1
+  // instead of 12.0 us, which is why the limit sits above the layer outputs of a decoder.)
   a2.stream_out = (long long)a.M * a.n_out * 4 >= (4ll << 20) ? 1 : 0;
   if(a.absmax_out) {   // one slot per wave
     if((long long)blocks * m_tiles * Cfg::kWaves <= kAbsmaxSlots) t_absmax_written = true;
