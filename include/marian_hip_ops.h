@@ -74,7 +74,9 @@ int marian_hip_bdot_legacy(const float* A, const float* B, float* C, int64_t bat
  * The attention of one decoding step in one launch: the nodes bdot_legacy(q, k, false, true,
  * scale), `+ mask`, softmax and bdot_legacy(weights, v) of Attention(), reference
  * src/models/transformer.h:241-280.  The arithmetic is that of the three separate entry points
- * above, operation for operation, so the result equals theirs bit for bit.
+ * above; for head sizes other than 64 operation for operation (the result equals theirs bit for
+ * bit), for dk == 64 with the dot products summed sixteen lanes wide and the weighted values four
+ * positions wide (equal within the 1e-5 relative bar of the float operators).
  *   q: [batchQ, m, dk], k and v: [batchKV, len, dk] (entry i uses k, v of i % batchKV: encoder
  *   keys shared by the beam), out: [batchQ, m, dk]; mask as in marian_hip_softmax for score rows
  *   [batchQ * m, len], or NULL.  len <= 4096.

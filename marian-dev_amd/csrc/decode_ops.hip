@@ -25,6 +25,15 @@ __device__ __forceinline__ float wave_sum(float v) {
   for(int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
   return v;
 }
+// Sum over each group of 16 consecutive lanes, left in all 16 of them (four DPP steps: the two
+// lane swaps within a quad, then the mirror within half a row and within the row).
+__device__ __forceinline__ float row16_sum(float v) {
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, false));   // quad_perm [1,0,3,2]
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, false));   // quad_perm [2,3,0,1]
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xF, 0xF, false));  // row_half_mirror
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xF, 0xF, false));  // row_mirror
+  return v;
+}
 __device__ __forceinline__ float wave_maxf(float v) {
 #pragma unroll
   for(int o = 32; o > 0; o >>= 1) {
@@ -298,7 +307,8 @@ __global__ __launch_bounds__(256) void attention_kernel(const float* __restrict_
   if(absmax_out && blockIdx.x == 0)   // slots past the last query row
     for(int sl = (int)rows_total + threadIdx.x; sl < kAbsmaxSlots; sl += 256) absmax_out[sl] = 0.0f;
   if(wr >= rows_total) return;   // whole waves leave; no workgroup barrier is used
-  float* sc = att_lds + (threadIdx.x / 64) * len;
+  float* sc = att_lds + (threadIdx.x / 64) * (len + 256);   // scores, then 4 x 64 partial outputs
+  float* part = sc + len;
   const int lane = threadIdx.x % 64;
   const long long i = wr / m;
   const float* q = Q + (size_t)wr * dk;
@@ -319,7 +329,39 @@ __global__ __launch_bounds__(256) void attention_kernel(const float* __restrict_
                                      reinterpret_cast<uintptr_t>(k_last)) % 16) == 0;
   float mx = -__builtin_inff();
   float omax = 0.0f;   // max |out| of this query row
-  for(int pos = lane; pos < len; pos += 64) {
+  const bool fast = vec && dk == 64 && ((reinterpret_cast<uintptr_t>(vb) | reinterpret_cast<uintptr_t>(v_last)) % 16) == 0;
+  if(fast) {
+    // The usual head size.  Sixteen lanes cover the 64 values of a key or value row with 16 bytes
+    // each and the four groups of sixteen take four consecutive positions, so one load of the wave
+    // moves 1 KB of contiguous cache (every lane busy, whatever the number of positions).
+    const int g = lane / 16, c = lane % 16;
+    const v4f q4 = reinterpret_cast<const v4f*>(q)[c];
+    for(int base = 0; base < len; base += 32) {   // eight loads in flight
+      v4f kr[8];
+#pragma unroll
+      for(int u = 0; u < 8; ++u) {
+        const int pos = min(base + 4 * u + g, len - 1);
+        const float* krow = pos == len - 1 ? k_last : kb + (size_t)pos * dk;
+        kr[u] = reinterpret_cast<const v4f*>(krow)[c];
+      }
+#pragma unroll
+      for(int u = 0; u < 8; ++u) {
+        const int pos = base + 4 * u + g;
+        float s = q4.x * kr[u].x;
+        s = fmaf(q4.y, kr[u].y, s);
+        s = fmaf(q4.z, kr[u].z, s);
+        s = fmaf(q4.w, kr[u].w, s);
+        s = row16_sum(s);
+        if(c == 0 && pos < len) {
+          float z = scale * s;
+          if(mk) z = z + mk[pos];
+          sc[pos] = z;
+        }
+      }
+    }
+    for(int pos = lane; pos < len; pos += 64) mx = fmaxf(mx, sc[pos]);
+  }
+  for(int pos = lane; pos < len && !fast; pos += 64) {
     float s = 0.0f;
     const float* krow = pos == len - 1 ? k_last : kb + (size_t)pos * dk;
     if(vec && dk == 64) {   // the usual head size: all sixteen loads of the key row in flight at once
@@ -360,7 +402,33 @@ __global__ __launch_bounds__(256) void attention_kernel(const float* __restrict_
   sum = wave_sum(sum);
   for(int pos = lane; pos < len; pos += 64) sc[pos] = expf(sc[pos] - mx) / sum;
   // (a wave's LDS writes are visible to its own later reads: same wave, program order)
-  for(int d = lane; d < dk; d += 64) {
+  if(fast) {
+    const int g = lane / 16, c = lane % 16;
+    v4f o4 = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+    for(int base = 0; base < len; base += 32) {
+      v4f vr[8];
+#pragma unroll
+      for(int u = 0; u < 8; ++u) {
+        const int pos = min(base + 4 * u + g, len - 1);
+        const float* vrow = pos == len - 1 ? v_last : vb + (size_t)pos * dk;
+        vr[u] = reinterpret_cast<const v4f*>(vrow)[c];
+      }
+#pragma unroll
+      for(int u = 0; u < 8; ++u) {
+        const int pos = base + 4 * u + g;
+        const float w = pos < len ? sc[pos] : 0.0f;
+        o4.x = fmaf(w, vr[u].x, o4.x);
+        o4.y = fmaf(w, vr[u].y, o4.y);
+        o4.z = fmaf(w, vr[u].z, o4.z);
+        o4.w = fmaf(w, vr[u].w, o4.w);
+      }
+    }
+    reinterpret_cast<v4f*>(part)[g * 16 + c] = o4;   // partial sums of the positions g, g + 4, ...
+    const float o = ((part[lane] + part[64 + lane]) + part[128 + lane]) + part[192 + lane];
+    out[(size_t)wr * dk + lane] = o;
+    omax = fabsf(o);
+  }
+  for(int d = lane; d < dk && !fast; d += 64) {
     float o = 0.0f;
     int pos = 0;
     for(; pos + 8 <= len; pos += 8) {   // eight value loads in flight, same summation order
@@ -846,10 +914,10 @@ int marian_hip_attention(const float* q, float* k, float* v, const float* mask, 
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   if(!mask) { n_masks = 1; rows_per_mask = 1; }
   const long long rows_total = batchQ * m;
-  const size_t lds = (size_t)4 * (size_t)len * sizeof(float);
+  const size_t lds = (size_t)4 * (size_t)(len + 256) * sizeof(float);   // per wave: scores + partial outputs
   static const int lds_status = [] {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(attention_kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024);
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, 72 * 1024);
     return e == hipSuccess ? 0 : (int)e;
   }();
   if(lds_status != 0) return record_hip_error(lds_status);

@@ -168,7 +168,9 @@ def test_attention_products_of_a_decode_step(ops, chk, synth):
                                                   (16, 16, 1, 1, 64, False)])
 def test_one_launch_attention_equals_the_three_operators(ops, chk, synth, BQ, BKV, m, L, dk, masked):
     """marian_hip_attention against bdot_legacy + (mask) softmax + bdot_legacy of the same library:
-    bit for bit; and against the checker within the bar."""
+    bit for bit where it sums in their order (head sizes other than 64), within the bar for the
+    head size 64, whose dot products are summed sixteen lanes wide and whose weighted values four
+    positions wide; and against the checker within the bar."""
     heads = 4
     q = synth.normal(BQ + L, 0, (BQ, m, dk), 1.0)
     k = synth.normal(BQ + L, 1, (BKV, L, dk), 1.0)
@@ -185,7 +187,10 @@ def test_one_launch_attention_equals_the_three_operators(ops, chk, synth, BQ, BK
     w = ops.softmax(z, None if mask is None else dev(mask), rpm)
     want = ops.bdot_legacy(w, dev(v)).cpu().numpy()
     got = ops.Attention(dev(q), dev(k), dev(v), None if mask is None else dev(mask), rpm).cpu().numpy()
-    assert np.array_equal(got, want)
+    if dk == 64:
+        close(got, want, 4 * REL, 2e-5)
+    else:
+        assert np.array_equal(got, want)
     zc = chk.bdot_legacy(q, k, False, True, scale)
     wc = chk.softmax(zc, mask, rows_per_mask=rpm)
     close(got, chk.bdot_legacy(wc, v), 4 * REL, 2e-5)
