@@ -169,6 +169,8 @@ int launch_stream32_kw(const GemmArgs& a, const FusedSrc& f, hipStream_t st, int
         if(half_rows) return launch_stream32<1, 2, 4, 4, MODE, 16>(a, f, st);
         return launch_stream32<1, 2, 4, 4, MODE>(a, f, st);
       default:
+        if(need > 4 && half_rows && g_kernel_override.load(std::memory_order_relaxed) % 1000 != 670)
+          return launch_stream32<1, 1, 8, 8, MODE, 16>(a, f, st);   // long rows: half as many chunks (measurement id 670 keeps the shorter ones)
         if(need > 2) {
           if(half_rows) return launch_stream32<1, 1, 8, 4, MODE, 16>(a, f, st);
           return launch_stream32<1, 1, 8, 4, MODE>(a, f, st);
