@@ -8,6 +8,7 @@
 
 #include "abi_common.h"
 #include "gemm_mfma32_kernel.h"
+#include "gemm_pair_kernel.h"
 #include "gemm_persistent_kernel.h"
 #include "gemm_stream32_kernel.h"
 #include "gemm_stream_kernel.h"
@@ -89,6 +90,27 @@ int launch_big(const GemmArgs& a, hipStream_t st) {
   int tiles_m = (a.M + BM - 1) / BM;
   hipLaunchKernelGGL(kernel, dim3(tiles_n * tiles_m), dim3(Cfg::kThreads), Cfg::kLdsBytes, st, a,
                      tiles_n, tiles_m);
+  MH_HIP(hipGetLastError());
+  return MARIAN_HIP_OK;
+}
+
+// Two side-by-side 256x128 tiles per workgroup, the first written out while the second is multiplied.
+inline bool pair_kernel_fits(const GemmArgs& a) {
+  return !a.dump && !a.idx && a.M % PairCfg::BM == 0 && a.n_out % (2 * PairCfg::BN) == 0 &&
+         a.K % PairCfg::BK == 0 && a.K / PairCfg::BK >= PairCfg::kSideBlocks &&
+         (!a.bias || aligned(a.bias, 16));
+}
+
+template <bool NT>
+int launch_pair(const GemmArgs& a, hipStream_t st) {
+  if(!pair_kernel_fits(a)) return launch_big<256, 256, 2, 4, 2>(a, st);
+  auto kernel = gemm_pair_kernel<NT>;
+  static const int lds_status = allow_lds(kernel, PairCfg::kLdsBytes);
+  if(lds_status != MARIAN_HIP_OK) return lds_status;
+  int pairs_n = a.n_out / (2 * PairCfg::BN);
+  int tiles_m = a.M / PairCfg::BM;
+  hipLaunchKernelGGL(kernel, dim3(pairs_n * tiles_m), dim3(PairCfg::kThreads), PairCfg::kLdsBytes, st, a,
+                     pairs_n, tiles_m);
   MH_HIP(hipGetLastError());
   return MARIAN_HIP_OK;
 }
@@ -343,6 +365,8 @@ int launch_gemm(const GemmArgs& a, hipStream_t st) {
     case 315: return launch_big<256, 256, 2, 4, 2, false>(a, st);
     case 316: return launch_big<256, 128, 2, 2, 2, false>(a, st);
     case 317: return launch_big<128, 256, 2, 2, 2, false>(a, st);
+    case 330: return launch_pair<false>(a, st);
+    case 331: return launch_pair<true>(a, st);
     case 307: return launch_big<128, 128, 2, 2, 3>(a, st);
     case 308: return launch_big<256, 128, 2, 2, 3>(a, st);
     case 309: return launch_big<128, 64, 2, 2, 2>(a, st);
@@ -385,8 +409,18 @@ int launch_gemm(const GemmArgs& a, hipStream_t st) {
   // an output that would fit the L2 caches (8 x 4 MB) is streamed out with non-temporal stores
   const bool stream_out = (long long)a.M * a.n_out * 4 <= (32ll << 20) && !a.dump;
   if(tiles256 >= 192) {
+    // short K: the fp32 output is most of the bytes; write one tile out while the next is multiplied
+    if(pair_kernel_fits(a) && a.K <= 1536 && g_kernel_override.load(std::memory_order_relaxed) % 1000 != 332)
+      return launch_pair<true>(a, st);
     if(stream_out) return launch_big<256, 256, 2, 4, 2, true, true>(a, st);
     return launch_big<256, 256, 2, 4, 2>(a, st);
+  }
+  // two or more 128x128 tiles per CU: eight waves and two LDS stages, so that two workgroups share
+  // a CU and one multiplies while the other writes its tile out; otherwise four waves, three stages
+  const long long tiles128 = ((a.M + 127) / 128) * (long long)((a.n_out + 127) / 128);
+  if(tiles128 >= 2 * compute_units()) {
+    if(stream_out) return launch_big<128, 128, 2, 4, 2, true, true>(a, st);
+    return launch_big<128, 128, 2, 4, 2>(a, st);
   }
   if(stream_out) return launch_big<128, 128, 2, 2, 3, true, true>(a, st);
   return launch_big<128, 128, 2, 2, 3>(a, st);

@@ -64,6 +64,14 @@ __device__ __forceinline__ void global_load_lds16(const void* gptr, unsigned lds
                : "memory", "m0");
 }
 
+// The same with the address as a wave-uniform 64-bit base (scalar registers) plus a 32-bit unsigned
+// per-lane offset: advancing along K then changes only the scalar base, no vector arithmetic per load.
+__device__ __forceinline__ void global_load_lds16(const void* sbase, unsigned voff, unsigned lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+               :
+               : "s"(lds_addr), "v"(voff), "s"(sbase)
+               : "memory", "m0");
+}
 
 // Writes one 32x32 accumulator tile.  Element v of the tile is row 8*(v/4) + 4*(lane/32) + v%4,
 // column lane%32; `out` points at this lane's element of tile row 4*(lane/32).
@@ -202,8 +210,8 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * kWave) void gemm_mfma32_kernel(
   }
   auto issue_one = [&](int kb, int stage, int j) {
     const int8_t* base = (j < Cfg::kLoadsA) ? args.Aq : args.Bq;
-    const int8_t* src = base + (size_t)(unsigned)goff[j] + (size_t)kb * Cfg::BK;
-    global_load_lds16(src, lds_base + stage * Cfg::kStageBytes + (j * Cfg::kWaves + wave) * 1024);
+    global_load_lds16(base + (size_t)kb * Cfg::BK, (unsigned)goff[j],
+                      lds_base + stage * Cfg::kStageBytes + (j * Cfg::kWaves + wave) * 1024);
   };
   auto issue = [&](int kb) {
     const int stage = kb % NSTAGE;
@@ -250,7 +258,9 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * kWave) void gemm_mfma32_kernel(
   // its share of the global->LDS loads of block kb + NSTAGE and of the LDS reads of the next
   // block's sub-steps 0 and 1; their issue time then hides under the MFMA of the previous slot.
   // (The loads are inline assembly, so the order is pinned slot by slot.)
-  auto second_half = [&](bool do_issue, int kb) {
+  auto second_half = [&](auto steady_c, bool may_issue, int kb) __attribute__((always_inline)) {
+    // steady: block kb + NSTAGE exists, its loads are issued without a branch between the MFMAs
+    const bool do_issue = decltype(steady_c)::value || may_issue;
     constexpr int nM = Cfg::WTM * Cfg::WTN;
     constexpr int LPS = (Cfg::kLoads + 2 * nM - 1) / (2 * nM);
     constexpr int nR = 2 * (Cfg::WTM + Cfg::WTN);
@@ -341,7 +351,7 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * kWave) void gemm_mfma32_kernel(
     read_frags(0, 0, 0);
     read_frags(0, 1, 1);
 
-    for(int kb = 0; kb + 1 < KB; ++kb) {
+    auto one_block = [&](int kb, auto steady_c) __attribute__((always_inline)) {
       const int stage = kb % NSTAGE;
       read_frags(stage, 2, 2);
       read_frags(stage, 3, 3);
@@ -353,12 +363,16 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * kWave) void gemm_mfma32_kernel(
       // is free.  Block kb+1 must have landed (this wave's share); later blocks may be in flight.
       __builtin_amdgcn_sched_barrier(0);  // keep the MFMAs above on this side of the wait
       wait_lgkmcnt0();
-      if(NSTAGE == 3 && kb + 2 < KB) wait_vmcnt<Cfg::kLoads>();
+      if(NSTAGE == 3 && (decltype(steady_c)::value || kb + 2 < KB)) wait_vmcnt<Cfg::kLoads>();
       else wait_vmcnt<0>();
       __builtin_amdgcn_s_barrier();
       __builtin_amdgcn_sched_barrier(0);
-      second_half(kb + NSTAGE < KB && !(args.dbg & 1), kb);
-    }
+      second_half(steady_c, kb + NSTAGE < KB && !(args.dbg & 1), kb);
+    };
+    int kb = 0;
+    if(!(args.dbg & 1))
+      for(; kb + NSTAGE < KB; ++kb) one_block(kb, std::true_type());
+    for(; kb + 1 < KB; ++kb) one_block(kb, std::false_type());
     {
       const int stage = (KB - 1) % NSTAGE;
       read_frags(stage, 2, 2);

@@ -117,12 +117,24 @@ def test_multiply_all_kernels_small_m(integer, orc, synth, M, K, N, kernel):
     run_case(integer, orc, synth, 300 + M + N, M, K, N, kernel, bias_on=True, relu=(M % 2 == 0))
 
 
-@pytest.mark.parametrize("kernel", [0, 501, 512, 521, 522, 524, 201, 202, 203, 204, 301, 302, 303, 304, 305, 306, 307, 308, 401, 402, 403, 404, 411, 413, 416])
+@pytest.mark.parametrize("kernel", [0, 501, 512, 521, 522, 524, 201, 202, 203, 204, 301, 302, 303, 304, 305, 306, 307, 308, 311, 312, 330, 401, 402, 403, 404, 411, 413, 416])
 @pytest.mark.parametrize("M,K,N", [(129, 64, 8), (256, 1024, 504), (300, 320, 1000), (513, 128, 264)])
 def test_multiply_tile_kernels_ragged(integer, orc, synth, M, K, N, kernel):
     say("multiply ragged", M, K, N, "kernel", kernel)
     run_case(integer, orc, synth, 400 + M + N, M, K, N, kernel, bias_on=(N % 16 == 8), relu=True,
              scale=0.5)
+
+
+@pytest.mark.parametrize("kernel", [330, 331])
+@pytest.mark.parametrize("M,K,N,bias_on,relu", [(256, 1024, 256, True, True), (512, 1024, 512, False, False),
+                                                (256, 1152, 256, True, False), (256, 1280, 512, False, True),
+                                                (512, 2048, 256, True, True), (768, 1024, 1024, True, False)])
+def test_multiply_tile_pair_kernel(integer, orc, synth, M, K, N, bias_on, relu, kernel):
+    """The large-M kernel that writes one tile out while it multiplies the next: eight K blocks
+    per tile (the write-out starts with the second tile) and more (it starts later), several
+    workgroups, with and without bias and ReLU, plain and non-temporal stores."""
+    say("multiply tile pair", M, K, N, "kernel", kernel)
+    run_case(integer, orc, synth, 460 + M + N, M, K, N, kernel, bias_on=bias_on, relu=relu, scale=0.25)
 
 
 @pytest.mark.parametrize("kernel", [0, 600, 611, 612, 614, 618, 620, 621, 622, 624, 628, 640, 641, 650, 651, 660, 661, 670])
@@ -166,7 +178,7 @@ def test_fused_shortlist(integer, orc, synth):
     assert np.array_equal(Aq.numpy(), Aq_h) and np.array_equal(out.cpu().numpy(), want)
 
 
-@pytest.mark.parametrize("kernel", [0, 101, 102, 201, 301, 307, 401, 411, 501, 511, 512, 514, 518, 521,
+@pytest.mark.parametrize("kernel", [0, 101, 102, 201, 301, 307, 312, 401, 411, 501, 511, 512, 514, 518, 521,
                                     522, 524, 600, 611, 612, 614, 618, 620, 621, 624, 628, 641, 651, 661, 670])
 @pytest.mark.parametrize("M", [8, 100])
 def test_shortlist_every_kernel_family(integer, orc, synth, M, kernel):
