@@ -31,7 +31,8 @@ struct PairCfg {
   static constexpr int kLoads = (BM + BN) / 8 / kWaves;   // 12 wave loads per K block
   static constexpr int kLoadsA = BM / 8 / kWaves;         // the first 8 are activation rows
   static constexpr int kRingBytes = NSTAGE * kStageBytes;
-  static constexpr int kLdsBytes = kRingBytes + kWaves * 1024;   // + the pair's 256 bias values, once per wave
+  // + per wave: the pair's 256 bias values (1 KB) and the two quantization multipliers (2 x 256 B)
+  static constexpr int kLdsBytes = kRingBytes + kWaves * (1024 + 512);
   static constexpr int kSideBlocks = 8;                   // K blocks that carry the first tile's write-out
   static constexpr int kStoresPerBlock = WTM * WTN * 16 / kSideBlocks;   // 16, on the odd MFMA slots
 };
@@ -41,6 +42,14 @@ template <bool NT>
 __device__ __forceinline__ void global_store_f32(const void* sbase, unsigned voff, float y) {
   if(NT) asm volatile("global_store_dword %0, %1, %2 nt" : : "v"(voff), "v"(y), "s"(sbase) : "memory");
   else asm volatile("global_store_dword %0, %1, %2" : : "v"(voff), "v"(y), "s"(sbase) : "memory");
+}
+
+// 4 bytes per lane from global memory straight into LDS: lane l writes LDS bytes lds_addr + 4*l .. +3.
+__device__ __forceinline__ void global_load_lds4(const void* sbase, unsigned voff, unsigned lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2"
+               :
+               : "s"(lds_addr), "v"(voff), "s"(sbase)
+               : "memory", "m0");
 }
 
 // Vector-memory operations of this wave that are younger than its loads of K block g + 1 when
@@ -75,11 +84,6 @@ __global__ __launch_bounds__(PairCfg::kThreads) void gemm_pair_kernel(GemmArgs a
   const int KB = K / Cfg::BK;
   const int total_blocks = 2 * KB;
 
-  // Read first, while nothing else is in flight: ordinary loads later on would be waited for with
-  // a count that does not know the hand-issued global->LDS loads.
-  const float aqm = tail_quant_mult(args.Aq, (size_t)args.M * (size_t)K);
-  const float bqm = tail_quant_mult(args.Bq, (size_t)K * (size_t)args.N);
-  float unquant = unquant_mult(aqm, bqm, args.scale);
 
   int tn, tm;
   {
@@ -140,6 +144,7 @@ __global__ __launch_bounds__(PairCfg::kThreads) void gemm_pair_kernel(GemmArgs a
 
   v16i acc[2][Cfg::WTM][Cfg::WTN];
   float bias0[Cfg::WTN], bias1[Cfg::WTN];   // this lane's columns of the first and of the second tile
+  float unquant;
 
   // value v (0..127) of the first tile, row by row across the two side-by-side accumulator tiles
   auto side_store = [&](int v) __attribute__((always_inline)) {
@@ -201,7 +206,10 @@ __global__ __launch_bounds__(PairCfg::kThreads) void gemm_pair_kernel(GemmArgs a
   // oldest load of the wave, so the first wait covers it; needs a 16-byte aligned bias).
   if(has_bias)
     global_load_lds16(args.bias + n0, (unsigned)lane * 16u, lds_base + Cfg::kRingBytes + wave * 1024);
-  asm volatile("" : "+v"(unquant));   // the two tail reads are waited for here, before the stream starts
+  // The two quantization multipliers travel the same way (every lane fetches the same 4 bytes):
+  // an ordinary load here would be waited for with a count that does not know the hand-issued loads.
+  global_load_lds4(args.Aq + (size_t)args.M * (size_t)K, 0u, lds_base + Cfg::kRingBytes + Cfg::kWaves * 1024 + wave * 512);
+  global_load_lds4(args.Bq + (size_t)K * (size_t)args.N, 0u, lds_base + Cfg::kRingBytes + Cfg::kWaves * 1024 + wave * 512 + 256);
 #pragma unroll
   for(int s = 0; s < NSTAGE; ++s)
 #pragma unroll
@@ -211,6 +219,10 @@ __global__ __launch_bounds__(PairCfg::kThreads) void gemm_pair_kernel(GemmArgs a
   const long long t_prologue = clock64();
 #pragma unroll
   for(int f = 0; f < 12; ++f) read_one(0, f / 6, f % 6);
+  {
+    const float* tails = reinterpret_cast<const float*>(lds + Cfg::kRingBytes + Cfg::kWaves * 1024 + wave * 512);
+    unquant = unquant_mult(tails[0], tails[64], args.scale);
+  }
   {
     const float* staged = reinterpret_cast<const float*>(lds + Cfg::kRingBytes + wave * 1024) + wn * Cfg::WTN * 32 + li;
 #pragma unroll

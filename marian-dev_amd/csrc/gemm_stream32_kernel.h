@@ -80,7 +80,7 @@ __global__ __launch_bounds__(WN * KW * kWave) void gemm_stream32_kernel(GemmArgs
   constexpr int kFusedGroups = NG, kFullGroups = NG - 2;
   static_assert(NG == 2 || NG == 4, "groups per thread");
   static_assert(kFusedMaxElems == 4 * 16 * kWave * 8, "four groups per thread of eight waves hold the largest fused input");
-  static_assert(!TILED_ || Cfg::kWaves == 8, "the abs-max partials are read by 512 threads");
+  static_assert(!TILED_ || kAbsmaxSlots % Cfg::kThreads == 0, "the abs-max partials are split evenly over the threads");
   constexpr bool FUSED = MODE == kFusedAll;
   constexpr bool TILED = MODE == kFusedTiled;
   extern __shared__ __attribute__((aligned(16))) int8_t lds[];
@@ -133,11 +133,13 @@ __global__ __launch_bounds__(WN * KW * kWave) void gemm_stream32_kernel(GemmArgs
   float aqm_pre = 0.0f;
   if(MODE == kPrequant) aqm_pre = tail_quant_mult(args.Aq, (size_t)M * (size_t)K);
   float amax = 0.0f;
-  if(TILED) {   // two (clamped) abs-max partials per thread cover all 1024
-    amax = fmaxf(fmaxf(partials[min(tid, n_partials - 1)],
-                       partials[min(tid + kStream32Threads, n_partials - 1)]),
-                 fmaxf(partials[min(tid + 2 * kStream32Threads, n_partials - 1)],
-                       partials[min(tid + 3 * kStream32Threads, n_partials - 1)]));
+  if(TILED) {   // a few (clamped) abs-max partials per thread cover all kAbsmaxSlots
+    float pm[kAbsmaxSlots / kStream32Threads];
+#pragma unroll
+    for(int i = 0; i < kAbsmaxSlots / kStream32Threads; ++i)
+      pm[i] = partials[min(tid + i * kStream32Threads, n_partials - 1)];
+#pragma unroll
+    for(int i = 0; i < kAbsmaxSlots / kStream32Threads; ++i) amax = fmaxf(amax, pm[i]);
   }
   const int8_t* wrow = args.Bq + (size_t)wsrc * (size_t)K + lg * 16;
   __builtin_amdgcn_sched_barrier(0);
