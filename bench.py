@@ -35,8 +35,8 @@ INT8_PEAK_TOPS = 5000.0      # MI355X dense int8 MFMA, published (5.0 POP/s)
 # runs of `bench.py --pmc-probe` (KiB per dispatch, scaled by the same counters' reading for a
 # plain copy of known size); the runs are summarised under profiles/.  None = not measured.
 MEASURED_TRAFFIC = {
-    # (8676.2 KiB FETCH_SIZE x 1.9992 + 8035.2 KiB WRITE_SIZE) per dispatch
-    "stream32_fused_M64_K512_N32000": int((8676.2 * 1.9992 + 8035.2) * 1024),
+    # (8677.6 KiB FETCH_SIZE x 1.9992 + 8033.8 KiB WRITE_SIZE) per dispatch
+    "stream32_fused_M64_K512_N32000": int((8677.6 * 1.9992 + 8033.8) * 1024),
 }
 
 DECODE_SHAPES = [(512, 1536), (512, 512), (512, 2048), (2048, 512), (512, 32000)]
