@@ -221,8 +221,8 @@ class BigDecoder:
             return logits
         # log-probabilities, then the beam's n-best per sentence over beam x vocabulary
         lp = ops.logsoftmax(logits)
-        ops.getNBestList(lp.view(self.beam, self.batch, self.V).transpose(0, 1).reshape(self.batch, 1, self.beam, self.V),
-                         self.beam)
+        # (the transposition to [batch, beam * V] of beam_search.cpp:472 happens inside the call)
+        ops.getNBestListOfBeams(lp.view(self.beam, 1, self.batch, self.V), self.beam)
         return lp
 
 
@@ -519,7 +519,7 @@ def main():
         out["transformer_big_decode_full"] = {
             "what": "full decoder step through the host mirrors: 49 int8 affine calls + per layer "
                     "2 one-launch attentions (20 cached positions + the new one, appended by the call; "
-                    "40 source positions with mask), 3 skip-add+layer-norm; log-softmax over 32000 and n-best per "
+                    "40 source positions with mask), 3 skip-add+layer-norm; log-softmax over 32000, beam/batch transposition + n-best per "
                     "sentence; no hypothesis bookkeeping; the abs-max of every GEMM input is left by the kernel that "
                     "produced it",
             "ms_per_step": round(fdt / n * 1e3, 4),

@@ -103,6 +103,27 @@ int marian_hip_attention(const float* q, float* k, float* v, const float* mask, 
 int marian_hip_nbest(const float* scores, int64_t dimBatch, int64_t rowLen, int64_t N,
                      float* outScores, uint32_t* outKeys, void* stream);
 
+/*
+ * The transposition and the n-best selection of a beam-search step in one call: reference
+ * src/translator/beam_search.cpp:472 (swapAxes(expandedPathScores, 0, 2)) followed by :492
+ * (getNBestList).  scores: [beam, dimBatch, vocab], the layout in which the step's scores leave the
+ * decoder.  The result is that of marian_hip_nbest on the transposed tensor [dimBatch, beam * vocab]
+ * - the same scores, the same keys b * beam * vocab + k * vocab + v, the same order - without
+ * writing that tensor, and with the row of a batch entry split over several workgroups (the N best
+ * of every part, then the N best of those, in one launch).  1 <= N <= 16, beam * N <= 1024, dimBatch <= 4096.
+ *   workspace: device memory of at least marian_hip_nbest_beams_workspace_bytes(...) bytes (the
+ *   reference's NthElement holds such buffers itself, src/translator/nth_element.cu): the
+ *   candidates of the parts, and one counter per batch entry by which the workgroup that finishes an
+ *   entry last knows that it is to draw the final list.  The counters are zero between calls:
+ *   marian_hip_nbest_beams_workspace_init clears a freshly allocated workspace once (a kernel, so it
+ *   may be captured in a graph); calls that share a workspace must not overlap.
+ */
+size_t marian_hip_nbest_beams_workspace_bytes(int64_t beam, int64_t dimBatch, int64_t vocab, int64_t N);
+int marian_hip_nbest_beams_workspace_init(void* workspace, size_t workspace_bytes, void* stream);
+int marian_hip_nbest_beams(const float* scores, int64_t beam, int64_t dimBatch, int64_t vocab, int64_t N,
+                           float* outScores, uint32_t* outKeys, void* workspace, size_t workspace_bytes,
+                           void* stream);
+
 #ifdef __cplusplus
 }
 #endif

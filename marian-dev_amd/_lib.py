@@ -37,6 +37,9 @@ SIGNATURES = {
     "marian_hip_transpose0213": (_i, [_vp, _vp, _i64, _i64, _i64, _i64, _vp]),
     "marian_hip_bdot_legacy": (_i, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i, _i, _f, _vp]),
     "marian_hip_nbest": (_i, [_vp, _i64, _i64, _i64, _vp, _vp, _vp]),
+    "marian_hip_nbest_beams_workspace_bytes": (_sz, [_i64, _i64, _i64, _i64]),
+    "marian_hip_nbest_beams_workspace_init": (_i, [_vp, _sz, _vp]),
+    "marian_hip_nbest_beams": (_i, [_vp, _i64, _i64, _i64, _i64, _vp, _vp, _vp, _sz, _vp]),
     "marian_hip_attention": (_i, [_vp, _vp, _vp, _vp, _i64, _i64, _vp, _i64, _i64, _i64, _i64, _i64,
                                   _f, _vp, _vp, _vp, _vp]),
 }

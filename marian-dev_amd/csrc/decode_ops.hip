@@ -461,6 +461,11 @@ __global__ __launch_bounds__(256) void attention_kernel(const float* __restrict_
 // massive ties) every thread instead keeps the KEEP >= N best of its elements in registers and
 // the draw pops them one by one.
 constexpr int kNbestMax = 16;
+constexpr long long kNbestMaxBatch = 4096;     // batch entries of the beam-major form
+// Its counters, 256 bytes apart: atomics on one cache line are served one after the other
+// (measured: the 256 arrivals of 32 entries on one line cost 7 us).
+constexpr int kNbestCounterStride = 64;
+constexpr size_t kNbestCounterBytes = kNbestMaxBatch * kNbestCounterStride * 4;
 
 __device__ __forceinline__ bool nbest_before(float v, unsigned i, float w, unsigned j) {
   return v > w || (v == w && i < j);
@@ -506,6 +511,24 @@ __device__ __forceinline__ void nbest_arg_best(float v, unsigned i, NbestShared&
     }
 }
 
+// One wave: the n best of `count` <= 64 (value, index) pairs, one per lane.
+// A lane counts the pairs that come before its own; the lanes of rank < n call emit(rank, ...)
+// themselves, and ranks that no pair fills (count < n) are emitted as (-inf, none) by lane 0.
+template <typename Emit>
+__device__ __forceinline__ void nbest_small_draw(const float* lv, const unsigned* li, int count, int n,
+                                                 Emit emit) {
+  const int lane = threadIdx.x % 64;
+  const int e = min(lane, count - 1);
+  const float v = lv[e];
+  const unsigned ix = li[e];
+  int rank = 0;
+  for(int c = 0; c < count; ++c)   // (equal pairs - fillers (-inf, none) - rank in lane order)
+    rank += (nbest_before(lv[c], li[c], v, ix) || (lv[c] == v && li[c] == ix && c < lane)) ? 1 : 0;
+  if(lane < count && rank < n) emit(rank, v, ix);
+  if(lane == 0)
+    for(int r = count; r < n; ++r) emit(r, -__builtin_inff(), 0xFFFFFFFFu);
+}
+
 // Wave 0 only: draws the n best of the `count` <= 1024 (value, index) pairs in lv/li (LDS),
 // sixteen per lane, without workgroup barriers.  emit(n, value, index) is called by lane 0.
 template <typename Emit>
@@ -517,11 +540,16 @@ __device__ __forceinline__ void nbest_wave_draw(const float* lv, const unsigned*
   float v[16];
   unsigned ix[16];
 #pragma unroll
-  for(int j = 0; j < 16; ++j) {
-    const int e = j * 64 + lane;
-    v[j] = e < count ? lv[e] : ninf;
-    ix[j] = e < count ? li[e] : none;
+  for(int j = 0; j < 16; ++j) {   // (clamped positions, dropped afterwards: all 32 loads in flight at once)
+    const int e = min(j * 64 + lane, count - 1);
+    v[j] = lv[e];
+    ix[j] = li[e];
   }
+#pragma unroll
+  for(int j = 0; j < 16; ++j)
+    if(j * 64 + lane >= count) {
+      v[j] = ninf; ix[j] = none;
+    }
   for(int r = 0; r < n; ++r) {
     float bv = v[0];
     unsigned bi = ix[0];
@@ -550,13 +578,11 @@ __device__ __forceinline__ void nbest_wave_draw(const float* lv, const unsigned*
   }
 }
 
-template <int KEEP>
-__global__ __launch_bounds__(1024) void nbest_kernel(const float* __restrict__ scores, long long rowLen, int N,
-                                                     float* __restrict__ outScores,
-                                                     unsigned* __restrict__ outKeys) {
-  __shared__ NbestShared sh;
-  const long long row = blockIdx.x;
-  const float* x = scores + row * rowLen;
+// The N best of x[0 .. rowLen), by the whole workgroup (1024 threads).  emit(r, value, index) is
+// called once for r = 0 .. N-1 (best first) by one thread each; index is the position within x.
+template <int KEEP, typename Emit>
+__device__ __forceinline__ void nbest_of_row(const float* __restrict__ x, long long rowLen, int N,
+                                             NbestShared& sh, Emit emit) {
   const int tid = threadIdx.x;
   const float ninf = -__builtin_inff();
   const unsigned none = 0xFFFFFFFFu;
@@ -570,44 +596,36 @@ __global__ __launch_bounds__(1024) void nbest_kernel(const float* __restrict__ s
   const long long n4 = rowLen / 4;
   if(vec) {   // 16-byte loads, eight in flight: elements 4 * (t + 1024 * j) .. + 3, in index order
     const v4f* x4 = reinterpret_cast<const v4f*>(x);
+    // (a thread meets its elements in index order, so "strictly greater, or the first" keeps the
+    // lowest index among equal scores)
     auto take = [&](float v, unsigned i) {
-      if(nbest_before(v, i, mv, mi)) {
+      if(v > mv || mi == none) {
         mv = v; mi = i;
       }
     };
-    long long i = tid;
-    for(; i + 7 * 1024 < n4; i += 8 * 1024) {
+    // (the last round reads clamped positions unconditionally and drops them afterwards: loads
+    // behind a range check would be waited for one by one)
+    for(long long i = tid; i < n4; i += 8 * 1024) {
       v4f v[8];
 #pragma unroll
-      for(int u = 0; u < 8; ++u) v[u] = x4[i + u * 1024];
+      for(int u = 0; u < 8; ++u) v[u] = x4[min(i + u * 1024, n4 - 1)];
 #pragma unroll
       for(int u = 0; u < 8; ++u) {
+        if(i + u * 1024 >= n4) break;
         const unsigned b = (unsigned)(4 * (i + u * 1024));
         take(v[u].x, b); take(v[u].y, b + 1); take(v[u].z, b + 2); take(v[u].w, b + 3);
       }
     }
-    for(; i < n4; i += 1024) {
-      const v4f v = x4[i];
-      const unsigned b = (unsigned)(4 * i);
-      take(v.x, b); take(v.y, b + 1); take(v.z, b + 2); take(v.w, b + 3);
-    }
   } else {
-    long long i = tid;
-    for(; i + 15 * 1024 < rowLen; i += 16 * 1024) {
+    for(long long i = tid; i < rowLen; i += 16 * 1024) {
       float v[16];
 #pragma unroll
-      for(int u = 0; u < 16; ++u) v[u] = x[i + u * 1024];
+      for(int u = 0; u < 16; ++u) v[u] = x[min(i + u * 1024, rowLen - 1)];
 #pragma unroll
       for(int u = 0; u < 16; ++u)
-        if(nbest_before(v[u], (unsigned)(i + u * 1024), mv, mi)) {
+        if(i + u * 1024 < rowLen && nbest_before(v[u], (unsigned)(i + u * 1024), mv, mi)) {
           mv = v[u]; mi = (unsigned)(i + u * 1024);
         }
-    }
-    for(; i < rowLen; i += 1024) {
-      const float v = x[i];
-      if(nbest_before(v, (unsigned)i, mv, mi)) {
-        mv = v; mi = (unsigned)i;
-      }
     }
   }
   float tv = ninf;
@@ -630,24 +648,18 @@ __global__ __launch_bounds__(1024) void nbest_kernel(const float* __restrict__ s
       sh.val[tid / 64] = wv; sh.idx[tid / 64] = wi;
     }
     __syncthreads();
-    float lv[16];
-    unsigned li[16];
+    // lane l % 16 ranks wave-best l % 16: the number of wave-bests before it; the one of rank
+    // N - 1 is the bound (the cost does not grow with N)
+    const float cvv = sh.val[tid % 16];
+    const unsigned cii = sh.idx[tid % 16];
+    int rank = 0;
 #pragma unroll
-    for(int w = 0; w < 16; ++w) {
-      lv[w] = sh.val[w]; li[w] = sh.idx[w];
-    }
-    for(int n = 0; n < N; ++n) {
-      tv = lv[0]; ti = li[0];
-#pragma unroll
-      for(int w = 1; w < 16; ++w)
-        if(nbest_before(lv[w], li[w], tv, ti)) {
-          tv = lv[w]; ti = li[w];
-        }
-#pragma unroll
-      for(int w = 0; w < 16; ++w)
-        if(li[w] == ti) {
-          lv[w] = ninf; li[w] = none;
-        }
+    for(int w = 0; w < 16; ++w) rank += nbest_before(sh.val[w], sh.idx[w], cvv, cii) ? 1 : 0;
+    const unsigned long long holders = __ballot(rank == N - 1) & 0xFFFFull;
+    if(holders) {
+      const int l = __ffsll((long long)holders) - 1;
+      tv = __shfl(cvv, l, 64);
+      ti = (unsigned)__shfl((int)cii, l, 64);
     }
   } else {
     // Bound for longer lists: the N-th best of the 1024 per-thread bests, found by wave 0 (the
@@ -681,63 +693,37 @@ __global__ __launch_bounds__(1024) void nbest_kernel(const float* __restrict__ s
   };
   if(vec) {
     const v4f* x4 = reinterpret_cast<const v4f*>(x);
-    long long i = tid;
-    for(; i + 7 * 1024 < n4; i += 8 * 1024) {
+    for(long long i = tid; i < n4; i += 8 * 1024) {
       v4f v[8];
 #pragma unroll
-      for(int u = 0; u < 8; ++u) v[u] = x4[i + u * 1024];
+      for(int u = 0; u < 8; ++u) v[u] = x4[min(i + u * 1024, n4 - 1)];
 #pragma unroll
       for(int u = 0; u < 8; ++u) {
+        if(i + u * 1024 >= n4) break;
         const unsigned b = (unsigned)(4 * (i + u * 1024));
         collect(v[u].x, b); collect(v[u].y, b + 1); collect(v[u].z, b + 2); collect(v[u].w, b + 3);
       }
     }
-    for(; i < n4; i += 1024) {
-      const v4f v = x4[i];
-      const unsigned b = (unsigned)(4 * i);
-      collect(v.x, b); collect(v.y, b + 1); collect(v.z, b + 2); collect(v.w, b + 3);
-    }
   } else {
-    long long i = tid;
-    for(; i + 15 * 1024 < rowLen; i += 16 * 1024) {
+    for(long long i = tid; i < rowLen; i += 16 * 1024) {
       float v[16];
 #pragma unroll
-      for(int u = 0; u < 16; ++u) v[u] = x[i + u * 1024];
+      for(int u = 0; u < 16; ++u) v[u] = x[min(i + u * 1024, rowLen - 1)];
 #pragma unroll
-      for(int u = 0; u < 16; ++u) collect(v[u], (unsigned)(i + u * 1024));
+      for(int u = 0; u < 16; ++u)
+        if(i + u * 1024 < rowLen) collect(v[u], (unsigned)(i + u * 1024));
     }
-    for(; i < rowLen; i += 1024) collect(x[i], (unsigned)i);
   }
   __syncthreads();
   const int count = sh.count;
 
   if(count <= 1024) {
-    // 3. the N best of the collected elements: a handful, drawn by one thread; more, by wave 0
+    // 3. the N best of the collected elements, drawn by wave 0: up to 64, one per lane; more,
+    //    sixteen per lane
     if(count <= 64) {
-      if(tid == 0) {
-        float pv = __builtin_inff();
-        unsigned pi = 0;
-        for(int r = 0; r < N; ++r) {   // best of those strictly after the previous pick
-          float bv = ninf;
-          unsigned bi = none;
-          for(int c = 0; c < count; ++c) {
-            const float v = sh.cand_val[c];
-            const unsigned i = sh.cand_idx[c];
-            const bool after_prev = r == 0 || nbest_before(pv, pi, v, i);
-            if(after_prev && nbest_before(v, i, bv, bi)) {
-              bv = v; bi = i;
-            }
-          }
-          outScores[row * N + r] = bv;
-          outKeys[row * N + r] = (unsigned)(row * rowLen) + bi;
-          pv = bv; pi = bi;
-        }
-      }
+      if(tid < 64) nbest_small_draw(sh.cand_val, sh.cand_idx, count, N, emit);
     } else if(tid < 64) {
-      nbest_wave_draw(sh.cand_val, sh.cand_idx, count, N, [&](int r, float v, unsigned i) {
-        outScores[row * N + r] = v;
-        outKeys[row * N + r] = (unsigned)(row * rowLen) + i;
-      });
+      nbest_wave_draw(sh.cand_val, sh.cand_idx, count, N, emit);
     }
     return;
   }
@@ -767,10 +753,7 @@ __global__ __launch_bounds__(1024) void nbest_kernel(const float* __restrict__ s
   for(int n = 0; n < N; ++n) {
     float gv; unsigned gi; int who;
     nbest_arg_best(val[0], idx[0], sh, gv, gi, who);
-    if(tid == 0) {
-      outScores[row * N + n] = gv;
-      outKeys[row * N + n] = (unsigned)(row * rowLen) + gi;
-    }
+    if(tid == 0) emit(n, gv, gi);
     if(tid == who) {   // pop the head
 #pragma unroll
       for(int j = 0; j < KEEP - 1; ++j) {
@@ -781,6 +764,119 @@ __global__ __launch_bounds__(1024) void nbest_kernel(const float* __restrict__ s
       idx[KEEP - 1] = none;
     }
   }
+}
+
+template <int KEEP>
+__global__ __launch_bounds__(1024) void nbest_kernel(const float* __restrict__ scores, long long rowLen, int N,
+                                                     float* __restrict__ outScores,
+                                                     unsigned* __restrict__ outKeys) {
+  __shared__ NbestShared sh;
+  const long long row = blockIdx.x;
+  nbest_of_row<KEEP>(scores + row * rowLen, rowLen, N, sh, [&](int r, float v, unsigned i) {
+    outScores[row * N + r] = v;
+    outKeys[row * N + r] = (unsigned)(row * rowLen) + i;
+  });
+}
+
+// Beam-major scores [beam, dimBatch, vocab]; the row of batch entry b is the beam's `beam` segments
+// of `vocab` scores, element (k, v) at logical position k * vocab + v.  Workgroup (part, b) takes
+// slice part % perSeg of segment part / perSeg and leaves the N best of it, with their logical
+// positions, in cand*[(b * parts + part) * N ..]; a slice shorter than N fills up with
+// (-inf, none), which sorts last.  The workgroup that finishes last for a batch entry (a counter per
+// entry, zero between calls) draws the N best of all the entry's candidates.  No workgroup waits
+// for another.
+template <int KEEP>
+__global__ __launch_bounds__(1024) void nbest_part_kernel(const float* __restrict__ scores, long long dimBatch,
+                                                          long long vocab, int perSeg, long long sliceLen,
+                                                          int N, float* candVal, unsigned* candIdx,
+                                                          unsigned* counters, float* __restrict__ outScores,
+                                                          unsigned* __restrict__ outKeys) {
+  __shared__ NbestShared sh;
+  __shared__ int is_last;
+  const int part = blockIdx.x, parts = gridDim.x;
+  const long long b = blockIdx.y;
+  const long long k = part / perSeg, v0 = (long long)(part % perSeg) * sliceLen;
+  const long long len = min(sliceLen, vocab - v0);
+  float* cv = candVal + ((size_t)b * parts + part) * N;
+  unsigned* ci = candIdx + ((size_t)b * parts + part) * N;
+  // Every path below publishes the candidates from wave 0, with stores that go through to memory
+  // (device scope), so that whichever workgroup turns out to be the last can read them without a
+  // cache write-back and invalidation around the counter (a fence pair costs ~8 us here).
+  auto publish = [&](int r, float v, unsigned i) {
+    __hip_atomic_store(cv + r, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(ci + r, i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  };
+  if(len < N) {   // (only a ragged last slice can be this short: one thread sorts it)
+    if(threadIdx.x == 0) {
+      const float* x = scores + ((size_t)k * dimBatch + b) * vocab + v0;
+      float pv = __builtin_inff();
+      long long pi = -1;
+      for(int r = 0; r < N; ++r) {
+        float bv = -__builtin_inff();
+        long long bi = -1;
+        for(long long c = 0; c < len; ++c) {
+          const float v = x[c];
+          const bool after_prev = r == 0 || v < pv || (v == pv && c > pi);
+          if(after_prev && (bi < 0 || v > bv)) {
+            bv = v; bi = c;
+          }
+        }
+        publish(r, bi < 0 ? -__builtin_inff() : bv, bi < 0 ? 0xFFFFFFFFu : (unsigned)(k * vocab + v0 + bi));
+        if(bi >= 0) { pv = bv; pi = bi; }
+      }
+    }
+  } else {
+    const unsigned base = (unsigned)(k * vocab + v0);
+    nbest_of_row<KEEP>(scores + ((size_t)k * dimBatch + b) * vocab + v0, len, N, sh,
+                       [&](int r, float v, unsigned i) { publish(r, v, base + i); });
+  }
+  if(threadIdx.x < 64) {   // (wave 0 wrote the candidates)
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // its stores have reached memory before the count goes up
+    if(threadIdx.x == 0)
+      is_last = __hip_atomic_fetch_add(&counters[b * kNbestCounterStride], 1u, __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT) == (unsigned)(parts - 1);
+  }
+  __syncthreads();
+  if(!is_last) return;
+  // the entry's candidates (at most 1024 pairs), read past this XCD's caches, into LDS
+  const int total = parts * N;
+  for(int e = threadIdx.x; e < total; e += 1024) {
+    sh.cand_val[e] = __hip_atomic_load(candVal + (size_t)b * total + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    sh.cand_idx[e] = __hip_atomic_load(candIdx + (size_t)b * total + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  __syncthreads();
+  if(threadIdx.x < 64) {
+    const long long rowLen = (long long)(parts / perSeg) * vocab;
+    auto result = [&](int r, float v, unsigned i) {
+      outScores[b * N + r] = v;
+      outKeys[b * N + r] = (unsigned)(b * rowLen) + i;
+    };
+    if(total <= 64) nbest_small_draw(sh.cand_val, sh.cand_idx, total, N, result);
+    else nbest_wave_draw(sh.cand_val, sh.cand_idx, total, N, result);
+    if(threadIdx.x == 0) counters[b * kNbestCounterStride] = 0;   // for the next call
+  }
+}
+
+__global__ __launch_bounds__(256) void zero_words_kernel(unsigned* __restrict__ p, long long n) {
+  for(long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long long)gridDim.x * blockDim.x)
+    p[i] = 0u;
+}
+
+// Slices per beam segment: enough workgroups for every CU (256 and up) as long as a slice keeps
+// 4096 scores, a multiple of four so that slices start 16-byte aligned when the rows do.
+struct NbestPlan {
+  int perSeg;
+  long long sliceLen;
+  int parts;
+};
+inline NbestPlan nbest_plan(int64_t beam, int64_t dimBatch, int64_t vocab, int64_t N) {
+  long long perSeg = (256 + beam * dimBatch - 1) / (beam * dimBatch);
+  const long long most = vocab / 4096 > 0 ? vocab / 4096 : 1;
+  if(perSeg > most) perSeg = most;
+  while(perSeg > 1 && beam * perSeg * N > 1024) --perSeg;   // the merge draws from at most 1024
+  long long sliceLen = ((vocab + perSeg - 1) / perSeg + 3) / 4 * 4;
+  perSeg = (vocab + sliceLen - 1) / sliceLen;
+  return NbestPlan{(int)perSeg, sliceLen, (int)(beam * perSeg)};
 }
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) % 16) == 0; }
@@ -942,6 +1038,57 @@ int marian_hip_nbest(const float* scores, int64_t dimBatch, int64_t rowLen, int6
     hipLaunchKernelGGL(nbest_kernel<8>, dim3((unsigned)dimBatch), dim3(1024), 0, st, scores, (long long)rowLen, (int)N, outScores, outKeys);
   else
     hipLaunchKernelGGL(nbest_kernel<16>, dim3((unsigned)dimBatch), dim3(1024), 0, st, scores, (long long)rowLen, (int)N, outScores, outKeys);
+  MH_HIP(hipGetLastError());
+  return MARIAN_HIP_OK;
+}
+
+size_t marian_hip_nbest_beams_workspace_bytes(int64_t beam, int64_t dimBatch, int64_t vocab, int64_t N) {
+  if(beam <= 0 || dimBatch <= 0 || vocab <= 0 || N <= 0 || N > kNbestMax) return 0;
+  const NbestPlan plan = nbest_plan(beam, dimBatch, vocab, N);
+  return kNbestCounterBytes + (size_t)dimBatch * plan.parts * N * 8;
+}
+
+int marian_hip_nbest_beams_workspace_init(void* workspace, size_t workspace_bytes, void* stream) {
+  if(workspace_bytes == 0) return MARIAN_HIP_OK;
+  if(!workspace) return MARIAN_HIP_ERR_NULL;
+  if(!aligned4(workspace)) return MARIAN_HIP_ERR_ALIGN;
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  const long long words = (long long)(workspace_bytes / 4);
+  const unsigned blocks = (unsigned)((words + 255) / 256 < 1024 ? (words + 255) / 256 : 1024);
+  if(words > 0)
+    hipLaunchKernelGGL(zero_words_kernel, dim3(blocks), dim3(256), 0, st, reinterpret_cast<unsigned*>(workspace), words);
+  MH_HIP(hipGetLastError());
+  return MARIAN_HIP_OK;
+}
+
+int marian_hip_nbest_beams(const float* scores, int64_t beam, int64_t dimBatch, int64_t vocab, int64_t N,
+                           float* outScores, uint32_t* outKeys, void* workspace, size_t workspace_bytes,
+                           void* stream) {
+  if(beam <= 0 || dimBatch < 0 || vocab <= 0 || N <= 0 || N > kNbestMax || N > beam * vocab)
+    return MARIAN_HIP_ERR_SHAPE;
+  if(beam * N > 1024) return MARIAN_HIP_ERR_SHAPE;
+  if(dimBatch == 0) return MARIAN_HIP_OK;
+  if(!scores || !outScores || !outKeys || !workspace) return MARIAN_HIP_ERR_NULL;
+  if(dimBatch * beam * vocab > 4294967295LL || dimBatch > kNbestMaxBatch) return MARIAN_HIP_ERR_RANGE;   // keys are uint32
+  if(!aligned4(scores) || !aligned4(outScores) || !aligned4(outKeys) || !aligned4(workspace))
+    return MARIAN_HIP_ERR_ALIGN;
+  const NbestPlan plan = nbest_plan(beam, dimBatch, vocab, N);
+  const size_t entries = (size_t)dimBatch * plan.parts * N;
+  if(workspace_bytes < kNbestCounterBytes + entries * 8) return MARIAN_HIP_ERR_WORKSPACE;
+  // layout: the counters (one per batch entry, zero between calls) in a region of fixed size, so
+  // that no call's candidates ever land on another call's counters; then candidate scores and
+  // candidate positions
+  unsigned* counters = reinterpret_cast<unsigned*>(workspace);
+  float* candVal = reinterpret_cast<float*>(counters + kNbestMaxBatch * kNbestCounterStride);
+  unsigned* candIdx = reinterpret_cast<unsigned*>(candVal + entries);
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  const dim3 grid((unsigned)plan.parts, (unsigned)dimBatch);
+  if(N <= 4)
+    hipLaunchKernelGGL(nbest_part_kernel<4>, grid, dim3(1024), 0, st, scores, (long long)dimBatch, (long long)vocab, plan.perSeg, plan.sliceLen, (int)N, candVal, candIdx, counters, outScores, outKeys);
+  else if(N <= 8)
+    hipLaunchKernelGGL(nbest_part_kernel<8>, grid, dim3(1024), 0, st, scores, (long long)dimBatch, (long long)vocab, plan.perSeg, plan.sliceLen, (int)N, candVal, candIdx, counters, outScores, outKeys);
+  else
+    hipLaunchKernelGGL(nbest_part_kernel<16>, grid, dim3(1024), 0, st, scores, (long long)dimBatch, (long long)vocab, plan.perSeg, plan.sliceLen, (int)N, candVal, candIdx, counters, outScores, outKeys);
   MH_HIP(hipGetLastError());
   return MARIAN_HIP_OK;
 }

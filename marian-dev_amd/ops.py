@@ -177,3 +177,29 @@ def getNBestList(scores, N):
                                  be.stream())
     _lib.check(st, "getNBestList")
     return vals, keys
+
+
+_nbest_workspaces = {}   # device -> uint8 tensor, grown on demand (the reference's NthElement owns its buffers too)
+
+
+def getNBestListOfBeams(scores, N):
+    """reference src/translator/beam_search.cpp:472 + :492: swapAxes(expandedPathScores, 0, 2)
+    followed by getNBestList, without the transposed copy.  scores [beam, 1, dimBatch, vocab] (or
+    [beam, dimBatch, vocab]); returns what getNBestList returns for the transposed tensor."""
+    scores = _f32c(scores, "getNBestListOfBeams")
+    be = _backend_of(scores)
+    beam, vocab = scores.shape[0], scores.shape[-1]
+    dimBatch = scores.numel() // (beam * vocab) if beam * vocab else 0
+    vals = torch.empty(dimBatch * N, dtype=torch.float32, device=scores.device)
+    keys = torch.empty(dimBatch * N, dtype=torch.int32, device=scores.device)
+    need = be.lib.marian_hip_nbest_beams_workspace_bytes(beam, dimBatch, vocab, N)
+    ws = _nbest_workspaces.get(scores.device)
+    if ws is None or ws.numel() < need:
+        ws = torch.empty(max(int(need), 4), dtype=torch.uint8, device=scores.device)
+        _lib.check(be.lib.marian_hip_nbest_beams_workspace_init(ws.data_ptr(), ws.numel(), be.stream()),
+                   "getNBestListOfBeams")
+        _nbest_workspaces[scores.device] = ws
+    st = be.lib.marian_hip_nbest_beams(scores.data_ptr(), beam, dimBatch, vocab, N, vals.data_ptr(),
+                                       keys.data_ptr(), ws.data_ptr(), ws.numel(), be.stream())
+    _lib.check(st, "getNBestListOfBeams")
+    return vals, keys

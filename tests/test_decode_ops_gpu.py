@@ -254,6 +254,56 @@ def test_nbest(ops, chk, synth, batch, beam, V, N):
         assert np.array_equal(vals.cpu().numpy(), cv) and np.array_equal(keys.cpu().numpy().view(np.uint32), ck)
 
 
+@pytest.mark.parametrize("batch,beam,V,N", [(32, 4, 32000, 4), (1, 1, 32000, 12), (7, 6, 1000, 6), (3, 1, 20, 16),
+                                            (2, 2, 8, 16), (5, 4, 3000, 1), (2, 3, 8195, 5), (300, 2, 4099, 2),
+                                            (1, 12, 50001, 16), (4, 64, 512, 16)])
+def test_nbest_of_beams(ops, chk, synth, batch, beam, V, N):
+    """Beam-major scores [beam, 1, batch, V] in one call = the transposition followed by the n-best
+    of the rows (the separate entry point and a stable sort), several slices per beam entry, ragged
+    last slices, rows not 16-byte aligned (odd V), slices shorter than N, equal scores across
+    slices and beam entries."""
+    x = synth.normal(91 + V, 0, (beam, 1, batch, V), 2.0)
+    if V >= 4099:
+        x[:, 0, 0, ::997] = np.float32(7.5)       # ties across slices and beam entries
+        x[0, 0, -1, :] = np.float32(-np.inf)
+    vals, keys = ops.getNBestListOfBeams(dev(x), N)
+    swapped = np.ascontiguousarray(np.swapaxes(x, 0, 2))       # [batch, 1, beam, V]
+    flat = swapped.reshape(batch, -1)
+    order = np.argsort(-flat, axis=1, kind="stable")[:, :N]
+    assert np.array_equal(vals.cpu().numpy().reshape(batch, N), np.take_along_axis(flat, order, 1))
+    want_keys = order + np.arange(batch)[:, None] * flat.shape[1]
+    assert np.array_equal(keys.cpu().numpy().view(np.uint32).reshape(batch, N).astype(np.int64), want_keys)
+    v1, k1 = ops.getNBestList(dev(swapped), N)
+    assert np.array_equal(vals.cpu().numpy(), v1.cpu().numpy()) and np.array_equal(keys.cpu().numpy(), k1.cpu().numpy())
+    if batch * beam * V <= 20000:
+        cv, ck = chk.nbest(swapped, N)
+        assert np.array_equal(vals.cpu().numpy(), cv) and np.array_equal(keys.cpu().numpy().view(np.uint32), ck)
+
+
+def test_nbest_of_beams_argument_checks(ops):
+    import torch
+    from conftest import load
+    lib = load("_lib").lib()
+    x = torch.zeros(4, 2, 100, device="cuda")
+    out = torch.zeros(8, device="cuda")
+    keys = torch.zeros(8, dtype=torch.int32, device="cuda")
+    need = lib.marian_hip_nbest_beams_workspace_bytes(4, 2, 100, 4)
+    assert need == 4096 * 256 + 2 * 4 * 4 * 8
+    ws = torch.full((need,), 255, dtype=torch.uint8, device="cuda")
+    assert lib.marian_hip_nbest_beams_workspace_init(ws.data_ptr(), need, None) == 0
+    torch.cuda.synchronize()
+    assert int(ws.to(torch.int64).sum()) == 0
+    call = lambda beam, batch, V, N, w, wb: lib.marian_hip_nbest_beams(x.data_ptr(), beam, batch, V, N, out.data_ptr(),
+                                                                       keys.data_ptr(), w, wb, None)
+    assert call(4, 2, 100, 4, ws.data_ptr(), need) == 0
+    assert call(4, 2, 100, 4, ws.data_ptr(), need - 1) == 4        # workspace too small
+    assert call(4, 2, 100, 4, None, need) == 1                     # null workspace
+    assert call(4, 2, 100, 17, ws.data_ptr(), need) == 2           # N > 16
+    assert call(0, 2, 100, 4, ws.data_ptr(), need) == 2
+    assert call(4, 0, 100, 4, ws.data_ptr(), need) == 0            # empty batch: nothing is touched
+    torch.cuda.synchronize()
+
+
 def test_nbest_ties_lowest_index_first(ops):
     t = np.zeros((2, 5000), np.float32)
     t[0, [4000, 17, 2048]] = 3.0
