@@ -456,7 +456,8 @@ __global__ __launch_bounds__(256) void attention_kernel(const float* __restrict_
 //      nothing after T can be among the N best;
 //   2. the row is read again (from cache) and the elements at or before T - usually little more
 //      than N of them - are collected in LDS, one per thread at most;
-//   3. the N best of the collected ones are drawn one at a time.
+//   3. the N best of the collected ones are found by rank (each candidate counts the candidates
+//      before it), or drawn one at a time when there are more than 256.
 // If more than 1024 elements pass the bound (large values concentrated in a few threads, or
 // massive ties) every thread instead keeps the KEEP >= N best of its elements in registers and
 // the draw pops them one by one.
@@ -630,10 +631,10 @@ __device__ __forceinline__ void nbest_of_row(const float* __restrict__ x, long l
   }
   float tv = ninf;
   unsigned ti = none;
-  if(N <= 4) {
-    // Bound for short lists: the N-th best of the 16 per-wave bests (16 distinct elements, so at
-    // least N elements of the row are at or before it).  Every thread derives it from the 16
-    // values itself; a wave without elements contributes "none", which sorts last.
+  {
+    // Bound: the N-th best of the 16 per-wave bests (16 distinct elements and N <= 16, so at least
+    // N elements of the row are at or before it; for N = 16 and scores without structure that
+    // leaves some 50 candidates).  A wave without elements contributes "none", which sorts last.
     float wv = mv;
     unsigned wi = mi;
 #pragma unroll
@@ -661,22 +662,6 @@ __device__ __forceinline__ void nbest_of_row(const float* __restrict__ x, long l
       tv = __shfl(cvv, l, 64);
       ti = (unsigned)__shfl((int)cii, l, 64);
     }
-  } else {
-    // Bound for longer lists: the N-th best of the 1024 per-thread bests, found by wave 0 (the
-    // per-wave bests would leave too many candidates).
-    sh.cand_val[tid] = mv;
-    sh.cand_idx[tid] = mi;
-    __syncthreads();
-    if(tid < 64)
-      nbest_wave_draw(sh.cand_val, sh.cand_idx, 1024, N, [&](int r, float v, unsigned i) {
-        if(r == N - 1) {
-          sh.val[0] = v; sh.idx[0] = i;
-        }
-      });
-    __syncthreads();
-    tv = sh.val[0];
-    ti = sh.idx[0];
-    __syncthreads();   // before the candidate list is reused below
   }
   // (with fewer than N holders of an element the bound is "none" and everything passes)
 
@@ -722,6 +707,15 @@ __device__ __forceinline__ void nbest_of_row(const float* __restrict__ x, long l
     //    sixteen per lane
     if(count <= 64) {
       if(tid < 64) nbest_small_draw(sh.cand_val, sh.cand_idx, count, N, emit);
+    } else if(count <= 256) {
+      // up to 256 (long lists): thread t ranks candidate t among all of them (distinct elements)
+      if(tid < count) {
+        const float v = sh.cand_val[tid];
+        const unsigned ix = sh.cand_idx[tid];
+        int rank = 0;
+        for(int c = 0; c < count; ++c) rank += nbest_before(sh.cand_val[c], sh.cand_idx[c], v, ix) ? 1 : 0;
+        if(rank < N) emit(rank, v, ix);
+      }
     } else if(tid < 64) {
       nbest_wave_draw(sh.cand_val, sh.cand_idx, count, N, emit);
     }
@@ -799,7 +793,7 @@ __global__ __launch_bounds__(1024) void nbest_part_kernel(const float* __restric
   const long long len = min(sliceLen, vocab - v0);
   float* cv = candVal + ((size_t)b * parts + part) * N;
   unsigned* ci = candIdx + ((size_t)b * parts + part) * N;
-  // Every path below publishes the candidates from wave 0, with stores that go through to memory
+  // Every path below publishes the candidates with stores that go through to memory
   // (device scope), so that whichever workgroup turns out to be the last can read them without a
   // cache write-back and invalidation around the counter (a fence pair costs ~8 us here).
   auto publish = [&](int r, float v, unsigned i) {
@@ -830,12 +824,11 @@ __global__ __launch_bounds__(1024) void nbest_part_kernel(const float* __restric
     nbest_of_row<KEEP>(scores + ((size_t)k * dimBatch + b) * vocab + v0, len, N, sh,
                        [&](int r, float v, unsigned i) { publish(r, v, base + i); });
   }
-  if(threadIdx.x < 64) {   // (wave 0 wrote the candidates)
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // its stores have reached memory before the count goes up
-    if(threadIdx.x == 0)
-      is_last = __hip_atomic_fetch_add(&counters[b * kNbestCounterStride], 1u, __ATOMIC_RELAXED,
-                                       __HIP_MEMORY_SCOPE_AGENT) == (unsigned)(parts - 1);
-  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // every wave's stores have reached memory ...
+  __syncthreads();
+  if(threadIdx.x == 0)                               // ... before the count goes up
+    is_last = __hip_atomic_fetch_add(&counters[b * kNbestCounterStride], 1u, __ATOMIC_RELAXED,
+                                     __HIP_MEMORY_SCOPE_AGENT) == (unsigned)(parts - 1);
   __syncthreads();
   if(!is_last) return;
   // the entry's candidates (at most 1024 pairs), read past this XCD's caches, into LDS
