@@ -1,0 +1,64 @@
+"""The library's calls recorded into a HIP graph: every replay gives the eager result.
+
+The calls allocate nothing and clear what must start from zero with kernels (abs-max slots, the
+counters of the split n-best), so a captured sequence is replayable as often as wanted.  The graph
+is replayed several times with eager work of the same library and synchronisations in between,
+and every replay is compared with the eager results, bit for bit."""
+import numpy as np
+import pytest
+
+from conftest import load
+
+pytestmark = pytest.mark.gpu
+
+
+def test_decoder_tail_replays(integer, synth):
+    import torch
+    ops = load("ops")
+    M, K, V, beam, batch = 32, 512, 4096, 4, 8
+    g = torch.Generator(device="cuda")
+    g.manual_seed(5)
+    x = torch.randn(M, K, device="cuda", generator=g)
+    skip = torch.randn(M, K, device="cuda", generator=g)
+    gamma = torch.randn(K, device="cuda", generator=g) * 0.1 + 1.0
+    beta = torch.randn(K, device="cuda", generator=g) * 0.1
+    W1 = integer.prepareB(torch.randn(K, K, device="cuda", generator=g) * 0.02)
+    b1 = torch.randn(K, device="cuda", generator=g) * 0.01
+    Wv = integer.prepareB(torch.randn(K, V, device="cuda", generator=g) * 0.02)
+    bv = torch.randn(V, device="cuda", generator=g) * 0.01
+
+    def step():
+        # layer norm (leaves the abs-max of its output) -> chained affine + ReLU -> affine over the
+        # vocabulary -> log-softmax -> transposition + n-best of the beam
+        h, hmax = ops.layerNorm(x, gamma, beta, 1e-6, skip, want_absmax=True)
+        h1, _, h1max = integer.affine_f32(h, W1, b1, relu=True, absmax=hmax, want_absmax=True)
+        logits, _ = integer.affine_f32(h1, Wv, bv, absmax=h1max)
+        lp = ops.logsoftmax(logits)
+        vals, keys = ops.getNBestListOfBeams(lp.view(beam, 1, batch, V), beam)
+        return lp, vals, keys
+
+    want = [t.clone() for t in step()]
+    torch.cuda.synchronize()
+
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        step()   # warm up on the capture stream (module load, workspaces)
+    torch.cuda.current_stream().wait_stream(s)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        outs = step()
+    for replay in range(4):
+        for t in outs:
+            t.fill_(float("nan")) if t.is_floating_point() else t.fill_(-1)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for got, w in zip(outs, want):
+            assert torch.equal(got, w), "replay %d differs from the eager result" % replay
+        # eager work of the same kind between the replays (shares the n-best workspace)
+        other = step()
+        torch.cuda.synchronize()
+        for got, w in zip(other, want):
+            assert torch.equal(got, w)
