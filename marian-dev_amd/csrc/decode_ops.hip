@@ -451,11 +451,11 @@ __global__ __launch_bounds__(256) void attention_kernel(const float* __restrict_
 // ---------------------------------------------------------------- n-best
 // One workgroup of 1024 threads per row; a thread looks at every 1024th element (or group of
 // four).  Scores are ordered by (value descending, index ascending).
-//   1. every thread finds the best of its elements, every wave the best of its threads'; the N-th
-//      best of these 16 is a bound T: at least N elements of the row are at or before T, so
-//      nothing after T can be among the N best;
-//   2. the row is read again (from cache) and the elements at or before T - usually little more
-//      than N of them - are collected in LDS, one per thread at most;
+//   1. every thread finds the largest of its scores, every wave the largest of its threads'; the
+//      N-th largest of these 16 is a bound T: at least N elements of the row are >= T, so nothing
+//      below T can be among the N best;
+//   2. the row is read again (from cache) and the elements >= T - usually little more than N of
+//      them - are collected in LDS with their positions;
 //   3. the N best of the collected ones are found by rank (each candidate counts the candidates
 //      before it), or drawn one at a time when there are more than 256.
 // If more than 1024 elements pass the bound (large values concentrated in a few threads, or
@@ -588,24 +588,17 @@ __device__ __forceinline__ void nbest_of_row(const float* __restrict__ x, long l
   const float ninf = -__builtin_inff();
   const unsigned none = 0xFFFFFFFFu;
 
-  // 1. best element of this thread, then the N-th best of those
-  // (both scans keep sixteen loads in flight per thread; one load per dependent step would
-  // cost a memory latency per element)
+  // 1. largest score of this thread, of its wave, and the N-th largest of the 16 wave maxima: the
+  //    bound T.  The maxima belong to 16 distinct elements and N <= 16, so at least N elements of the
+  //    row are >= T; for N = 16 and scores without structure some 50 are.  (Values only: one
+  //    instruction per element.  Both scans keep eight 16-byte loads in flight per thread; the last
+  //    round reads clamped positions unconditionally and drops them afterwards, because loads
+  //    behind a range check would be waited for one by one.)
   float mv = ninf;
-  unsigned mi = none;
   const bool vec = (rowLen % 4) == 0 && (reinterpret_cast<uintptr_t>(x) % 16) == 0;
   const long long n4 = rowLen / 4;
-  if(vec) {   // 16-byte loads, eight in flight: elements 4 * (t + 1024 * j) .. + 3, in index order
+  if(vec) {   // elements 4 * (t + 1024 * j) .. + 3
     const v4f* x4 = reinterpret_cast<const v4f*>(x);
-    // (a thread meets its elements in index order, so "strictly greater, or the first" keeps the
-    // lowest index among equal scores)
-    auto take = [&](float v, unsigned i) {
-      if(v > mv || mi == none) {
-        mv = v; mi = i;
-      }
-    };
-    // (the last round reads clamped positions unconditionally and drops them afterwards: loads
-    // behind a range check would be waited for one by one)
     for(long long i = tid; i < n4; i += 8 * 1024) {
       v4f v[8];
 #pragma unroll
@@ -613,8 +606,7 @@ __device__ __forceinline__ void nbest_of_row(const float* __restrict__ x, long l
 #pragma unroll
       for(int u = 0; u < 8; ++u) {
         if(i + u * 1024 >= n4) break;
-        const unsigned b = (unsigned)(4 * (i + u * 1024));
-        take(v[u].x, b); take(v[u].y, b + 1); take(v[u].z, b + 2); take(v[u].w, b + 3);
+        mv = fmaxf(fmaxf(mv, fmaxf(v[u].x, v[u].y)), fmaxf(v[u].z, v[u].w));
       }
     }
   } else {
@@ -624,52 +616,33 @@ __device__ __forceinline__ void nbest_of_row(const float* __restrict__ x, long l
       for(int u = 0; u < 16; ++u) v[u] = x[min(i + u * 1024, rowLen - 1)];
 #pragma unroll
       for(int u = 0; u < 16; ++u)
-        if(i + u * 1024 < rowLen && nbest_before(v[u], (unsigned)(i + u * 1024), mv, mi)) {
-          mv = v[u]; mi = (unsigned)(i + u * 1024);
-        }
+        if(i + u * 1024 < rowLen) mv = fmaxf(mv, v[u]);
     }
   }
-  float tv = ninf;
-  unsigned ti = none;
+  float tv = ninf;   // (a wave without elements contributes -inf; with fewer than N waves that hold
+                     // elements the bound is -inf and everything passes)
   {
-    // Bound: the N-th best of the 16 per-wave bests (16 distinct elements and N <= 16, so at least
-    // N elements of the row are at or before it; for N = 16 and scores without structure that
-    // leaves some 50 candidates).  A wave without elements contributes "none", which sorts last.
     float wv = mv;
-    unsigned wi = mi;
 #pragma unroll
-    for(int o = 32; o > 0; o >>= 1) {
-      const float ov = __shfl_xor(wv, o, 64);
-      const unsigned oi = (unsigned)__shfl_xor((int)wi, o, 64);
-      if(nbest_before(ov, oi, wv, wi)) {
-        wv = ov; wi = oi;
-      }
-    }
-    if(tid % 64 == 0) {
-      sh.val[tid / 64] = wv; sh.idx[tid / 64] = wi;
-    }
+    for(int o = 32; o > 0; o >>= 1) wv = fmaxf(wv, __shfl_xor(wv, o, 64));
+    if(tid % 64 == 0) sh.val[tid / 64] = wv;
     __syncthreads();
-    // lane l % 16 ranks wave-best l % 16: the number of wave-bests before it; the one of rank
-    // N - 1 is the bound (the cost does not grow with N)
-    const float cvv = sh.val[tid % 16];
-    const unsigned cii = sh.idx[tid % 16];
+    // lane l % 16 ranks wave maximum l % 16 (equal values in wave order); the one of rank N - 1
+    // is the bound (the cost does not grow with N)
+    const int c = tid % 16;
+    const float cvv = sh.val[c];
     int rank = 0;
 #pragma unroll
-    for(int w = 0; w < 16; ++w) rank += nbest_before(sh.val[w], sh.idx[w], cvv, cii) ? 1 : 0;
+    for(int w = 0; w < 16; ++w) rank += (sh.val[w] > cvv || (sh.val[w] == cvv && w < c)) ? 1 : 0;
     const unsigned long long holders = __ballot(rank == N - 1) & 0xFFFFull;
-    if(holders) {
-      const int l = __ffsll((long long)holders) - 1;
-      tv = __shfl(cvv, l, 64);
-      ti = (unsigned)__shfl((int)cii, l, 64);
-    }
+    tv = __shfl(cvv, __ffsll((long long)holders) - 1, 64);   // (ranks 0..15 are all taken: one holder)
   }
-  // (with fewer than N holders of an element the bound is "none" and everything passes)
 
-  // 2. collect what is at or before the bound
+  // 2. collect what is >= the bound
   if(tid == 0) sh.count = 0;
   __syncthreads();
   auto collect = [&](float v, unsigned i) {
-    if(!nbest_before(tv, ti, v, i)) {
+    if(v >= tv) {
       const int slot = atomicAdd(&sh.count, 1);
       if(slot < 1024) {
         sh.cand_val[slot] = v; sh.cand_idx[slot] = i;
