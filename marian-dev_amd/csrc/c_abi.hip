@@ -189,6 +189,8 @@ int launch_stream32_kw(const GemmArgs& a, const FusedSrc& f, hipStream_t st, int
       case 2: return launch_stream32<1, 4, 2, 4, MODE>(a, f, st);
       case 4:
         if(half_rows) return launch_stream32<1, 2, 4, 4, MODE, 16>(a, f, st);
+        if(need > 4 && g_kernel_override.load(std::memory_order_relaxed) % 1000 != 690)
+          return launch_stream32<1, 2, 4, 8, MODE>(a, f, st);   // long rows: half as many chunks (measurement id 690 keeps the shorter ones)
         return launch_stream32<1, 2, 4, 4, MODE>(a, f, st);
       default:
         if(need > 4 && half_rows && g_kernel_override.load(std::memory_order_relaxed) % 1000 != 670)

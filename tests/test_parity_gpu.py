@@ -137,7 +137,7 @@ def test_multiply_tile_pair_kernel(integer, orc, synth, M, K, N, bias_on, relu, 
     run_case(integer, orc, synth, 460 + M + N, M, K, N, kernel, bias_on=bias_on, relu=relu, scale=0.25)
 
 
-@pytest.mark.parametrize("kernel", [0, 600, 611, 612, 614, 618, 620, 621, 622, 624, 628, 640, 641, 650, 651, 660, 661, 670])
+@pytest.mark.parametrize("kernel", [0, 600, 611, 612, 614, 618, 620, 621, 622, 624, 628, 640, 641, 650, 651, 660, 661, 670, 690])
 @pytest.mark.parametrize("M,K,N", [(1, 64, 8), (1, 512, 512), (4, 2048, 512), (16, 512, 1536),
                                    (33, 192, 136), (64, 512, 2048), (100, 256, 1000), (128, 256, 64),
                                    (16, 1024, 32000), (7, 4096, 64), (128, 1024, 1024),
@@ -179,7 +179,7 @@ def test_fused_shortlist(integer, orc, synth):
 
 
 @pytest.mark.parametrize("kernel", [0, 101, 102, 201, 301, 307, 312, 401, 411, 501, 511, 512, 514, 518, 521,
-                                    522, 524, 600, 611, 612, 614, 618, 620, 621, 624, 628, 641, 651, 661, 670])
+                                    522, 524, 600, 611, 612, 614, 618, 620, 621, 624, 628, 641, 651, 661, 670, 690])
 @pytest.mark.parametrize("M", [8, 100])
 def test_shortlist_every_kernel_family(integer, orc, synth, M, kernel):
     """The row gather of W^T and of the bias inside each kernel family (ids >= 600: fused call)."""
