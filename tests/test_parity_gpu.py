@@ -211,7 +211,7 @@ def test_shortlist_every_kernel_family(integer, orc, synth, M, kernel):
 
 
 def test_config1_single_affine_end_to_end(integer, orc, synth):
-    """BASELINE config 1: A[64x512] ~ N(0,1), W[512x2048] ~ N(0,0.02^2), bias ~ N(0,0.01^2), ReLU."""
+    """Benchmark configuration 1: A[64x512] ~ N(0,1), W[512x2048] ~ N(0,0.02^2), bias ~ N(0,0.01^2), ReLU."""
     say("config1")
     M, K, N = 64, 512, 2048
     A, W, bias = inputs(synth, 1001, M, K, N)
@@ -233,7 +233,7 @@ def test_config1_single_affine_end_to_end(integer, orc, synth):
 @pytest.mark.parametrize("K,N", [(512, 1536), (512, 512), (512, 2048), (2048, 512), (512, 32000)])
 @pytest.mark.parametrize("M", [1, 4, 16, 64])
 def test_config2_decode_sweep(integer, orc, synth, M, K, N):
-    """BASELINE config 2: transformer-base decode shapes."""
+    """Benchmark configuration 2: transformer-base decode shapes."""
     say("config2", M, K, N)
     A, W, bias = inputs(synth, 1002, M, K, N)
     Bq_h, Aq_h = orc.prepare_b(W), orc.prepare_a(A)
@@ -247,7 +247,7 @@ def test_config2_decode_sweep(integer, orc, synth, M, K, N):
 
 
 def test_config3_transformer_big_step_shapes(integer, orc, synth):
-    """BASELINE config 3 GEMM shapes at M = 128 (beam 4 x batch 32), d = 1024, ffn = 4096."""
+    """Benchmark configuration 3, GEMM shapes at M = 128 (beam 4 x batch 32), d = 1024, ffn = 4096."""
     M = 128
     for K, N, relu in [(1024, 1024, False), (1024, 4096, True), (4096, 1024, False)]:
         say("config3", M, K, N)
@@ -264,7 +264,7 @@ def test_config3_transformer_big_step_shapes(integer, orc, synth):
 
 @pytest.mark.parametrize("K,N", [(1024, 4096), (4096, 1024)])
 def test_config4_large_m_full_size(integer, orc, synth, K, N):
-    """BASELINE config 4 at full size (M = 4096).  The checker runs on 96 sampled rows (rows are
+    """Benchmark configuration 4 at full size (M = 4096).  The checker runs on 96 sampled rows (rows are
     independent once A is quantized); the rest is covered by a column-sum identity in int64:
     sum_m acc[m, n] == (sum_m Aq[m, :]) . Bt[n, :]."""
     M = 4096
@@ -295,7 +295,7 @@ def test_config4_large_m_full_size(integer, orc, synth, K, N):
 
 @pytest.mark.parametrize("M", [4, 64, 256])
 def test_config5_shortlist(integer, orc, synth, M):
-    """BASELINE config 5: W int8 [32000 x 1024], shortlist of 500-2000 sorted unique ids.
+    """Benchmark configuration 5: W int8 [32000 x 1024], shortlist of 500-2000 sorted unique ids.
     gather-GEMM == column pick of the dense GEMM, bit-exactly, and matches the checker."""
     import torch
     K, N = 1024, 32000
