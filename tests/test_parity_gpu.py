@@ -141,7 +141,8 @@ def test_multiply_tile_pair_kernel(integer, orc, synth, M, K, N, bias_on, relu, 
 @pytest.mark.parametrize("M,K,N", [(1, 64, 8), (1, 512, 512), (4, 2048, 512), (16, 512, 1536),
                                    (33, 192, 136), (64, 512, 2048), (100, 256, 1000), (128, 256, 64),
                                    (16, 1024, 32000), (7, 4096, 64), (128, 1024, 1024),
-                                   (100, 2048, 512), (200, 1024, 504), (128, 4096, 1024)])
+                                   (100, 2048, 512), (200, 1024, 504), (128, 4096, 1024),
+                                   (128, 1024, 4096), (96, 1024, 2048)])
 def test_fused_affine_f32(integer, orc, synth, M, K, N, kernel):
     """prepareA + multiply in one call (one fused kernel where the activations are small):
     output, quantized activations and quantMult equal those of the two separate steps."""
