@@ -261,6 +261,23 @@ def test_config3_transformer_big_step_shapes(integer, orc, synth):
         assert np.array_equal(integer.multiply_i32(Aq, Bq).cpu().numpy(), want_acc)
         got = integer.multiply(Aq, Bq, dev(bias), relu=relu).cpu().numpy()
         assert np.array_equal(got, want)
+        # and as the decoder calls it: one call from the fp32 activations
+        got = integer.affine(dev(A), Bq, dev(bias)).cpu().numpy() if not relu else \
+            integer.affineWithReluDropout(dev(A), Bq, dev(bias)).cpu().numpy()
+        assert np.array_equal(got, want)
+
+
+def test_config3_vocabulary_projection_from_fp32(integer, orc, synth):
+    """The 32000-word output layer of configuration 3 at M = 128, through the operator (abs-max,
+    quantize and GEMM behind one call)."""
+    M, K, N = 128, 1024, 32000
+    say("config3 vocabulary", M, K, N)
+    A, W, bias = inputs(synth, 1013, M, K, N)
+    Bq_h, Aq_h = orc.prepare_b(W), orc.prepare_a(A)
+    want, _ = orc.affine(Aq_h, Bq_h, bias, M, K, N, 1.0, False)
+    Bq = upload_q(integer, Bq_h, (K, N))
+    got = integer.affine(dev(A), Bq, dev(bias)).cpu().numpy()
+    assert np.array_equal(got, want)
 
 
 @pytest.mark.parametrize("K,N", [(1024, 4096), (4096, 1024)])
