@@ -170,26 +170,34 @@ __global__ __launch_bounds__(256) void quantize_b_transpose_kernel(
     const float* __restrict__ W, int K, int N, const float* __restrict__ partials,
     int n_partials, int8_t* __restrict__ out) {
   __shared__ float red[256 / kWave];
-  __shared__ __attribute__((aligned(16))) int8_t tile[64][64 + 16];  // [n][k], padded rows
+  // [n][k / 4] as packed dwords, 17 dwords per row: the 64 lanes of a wave (consecutive n, one k
+  // group) hit every bank twice, the minimum for 64 lanes on 32 banks
+  __shared__ uint32_t tile[64][17];
   float m = 0.0f;
   for(int p = threadIdx.x; p < n_partials; p += blockDim.x) m = fmaxf(m, partials[p]);
   m = block_max(m, red);
   const float qm = quant_mult_from_maxabs(m);
 
   const int n0 = blockIdx.x * 64, k0 = blockIdx.y * 64;
-  const int tn = threadIdx.x % 64, tk = threadIdx.x / 64;  // 4 k rows per pass
-#pragma unroll 4
-  for(int kk = tk; kk < 64; kk += 4) {
-    int k = k0 + kk, n = n0 + tn;
-    float v = (k < K && n < N) ? W[(size_t)k * N + n] : 0.0f;
-    tile[tn][kk] = (int8_t)quantize_one(v, qm);
+  const int tn = threadIdx.x % 64, tk = threadIdx.x / 64;  // wave tk takes k rows 16*tk .. 16*tk+15
+  const int n_in = n0 + tn;
+#pragma unroll
+  for(int g = 0; g < 4; ++g) {
+    const int kk = tk * 16 + g * 4;   // four consecutive k of column n: one packed dword
+    v4f v = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+    if(n_in < N) {   // (K % 64 == 0: the k rows of a tile are all inside)
+      const float* w = W + (size_t)(k0 + kk) * N + n_in;
+      v = v4f{w[0], w[(size_t)N], w[2 * (size_t)N], w[3 * (size_t)N]};
+    }
+    tile[tn][kk / 4] = quantize_pack4(v, qm);
   }
   __syncthreads();
   // 64 rows (n) x 64 bytes (k): 4 threads per row, 16 bytes each
   const int rn = threadIdx.x / 4, ck = (threadIdx.x % 4) * 16;
   int n = n0 + rn, k = k0 + ck;
   if(n < N && k < K) {  // K % 64 == 0, so a 16-byte run is inside or outside as a whole
-    uint4 v = *reinterpret_cast<const uint4*>(&tile[rn][ck]);
+    uint4 v;
+    v.x = tile[rn][ck / 4]; v.y = tile[rn][ck / 4 + 1]; v.z = tile[rn][ck / 4 + 2]; v.w = tile[rn][ck / 4 + 3];
     *reinterpret_cast<uint4*>(out + (size_t)n * K + k) = v;
   }
   if(blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0)
