@@ -179,36 +179,37 @@ __global__ __launch_bounds__(THREADS < 256 ? 256 : THREADS) void softmax_kernel(
   }
 }
 
-// Vocabulary-size rows (cols % 4 == 0, cols <= 32768, 16-byte aligned rows, no mask): 1024
-// threads per row keep the row in registers (eight float4 each), so it is read once.  Same
+// Rows kept in registers (cols % 4 == 0, 16-byte aligned rows, no mask), so that they are read
+// once: 1024 threads with eight float4 each for vocabulary-size rows (up to 32768), 256 threads
+// with four for rows up to 4096.  Same
 // operations per element as softmax_kernel.
-template <bool LOG>
-__global__ __launch_bounds__(1024) void softmax_wide_kernel(const float* in, float* out, int cols) {
-  __shared__ float red[16];
+template <bool LOG, int THREADS, int VPT>
+__global__ __launch_bounds__(THREADS) void softmax_wide_kernel(const float* in, float* out, int cols) {
+  __shared__ float red[THREADS / 64];
   const size_t row = blockIdx.x;
   const v4f* x = reinterpret_cast<const v4f*>(in + row * cols);
   v4f* y = reinterpret_cast<v4f*>(out + row * cols);
   const int cols4 = cols / 4, t = threadIdx.x;
-  v4f v[8];
+  v4f v[VPT];
   float mx = -__builtin_inff();
-  // (all eight loads at once, positions past the row clamped and dropped afterwards: a load behind a
+  // (all loads at once, positions past the row clamped and dropped afterwards: a load behind a
   // range check is waited for inside its branch, one memory latency per load)
 #pragma unroll
-  for(int j = 0; j < 8; ++j) v[j] = x[min(j * 1024 + t, cols4 - 1)];
+  for(int j = 0; j < VPT; ++j) v[j] = x[min(j * THREADS + t, cols4 - 1)];
 #pragma unroll
-  for(int j = 0; j < 8; ++j) {
-    const int i = j * 1024 + t;
+  for(int j = 0; j < VPT; ++j) {
+    const int i = j * THREADS + t;
     if(i < cols4) {
       const float a = v[j].x > v[j].y ? v[j].x : v[j].y, b = v[j].z > v[j].w ? v[j].z : v[j].w;
       const float c = a > b ? a : b;
       mx = c > mx ? c : mx;
     }
   }
-  mx = row_reduce<1024, true>(mx, red);
+  mx = row_reduce<THREADS, true>(mx, red);
   float sum = 0.0f;
 #pragma unroll
-  for(int j = 0; j < 8; ++j) {
-    if(j * 1024 + t < cols4) {
+  for(int j = 0; j < VPT; ++j) {
+    if(j * THREADS + t < cols4) {
       if(LOG) {
         v[j].x = v[j].x - mx; v[j].y = v[j].y - mx; v[j].z = v[j].z - mx; v[j].w = v[j].w - mx;
         // (the exponentials only enter the logarithm of their sum: the hardware exp2 form, about
@@ -222,11 +223,11 @@ __global__ __launch_bounds__(1024) void softmax_wide_kernel(const float* in, flo
       }
     }
   }
-  sum = row_reduce<1024, false>(sum, red);
+  sum = row_reduce<THREADS, false>(sum, red);
   const float log_sum = logf(sum);
 #pragma unroll
-  for(int j = 0; j < 8; ++j) {
-    const int i = j * 1024 + t;
+  for(int j = 0; j < VPT; ++j) {
+    const int i = j * THREADS + t;
     if(i < cols4) {
       if(LOG) y[i] = v4f{v[j].x - log_sum, v[j].y - log_sum, v[j].z - log_sum, v[j].w - log_sum};
       else y[i] = v4f{v[j].x / sum, v[j].y / sum, v[j].z / sum, v[j].w / sum};
@@ -900,13 +901,19 @@ static int softmax_common(const float* in, const float* mask, int64_t n_masks, i
   if(!aligned4(in) || !aligned4(out) || (mask && !aligned4(mask))) return MARIAN_HIP_ERR_ALIGN;
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   if(!mask) { n_masks = 1; rows_per_mask = 1; }
-  if(cols <= 2048) {
+  // rows that fit registers of one workgroup and need no mask: read once (a wave per row walks a
+  // 1024-value row in 16 dependent steps per pass: 10 us for 128 rows against 4)
+  const bool wide_ok = !mask && cols % 4 == 0 && cols <= 32768 && aligned16(in) && aligned16(out);
+  if(cols <= 2048 && !(wide_ok && cols > 256)) {
     const unsigned blocks = (unsigned)((rows + 3) / 4);
     if(log) hipLaunchKernelGGL((softmax_kernel<64, true>), dim3(blocks), dim3(256), 0, st, in, mask, (long long)n_masks, (long long)rows_per_mask, out, (long long)rows, (int)cols);
     else hipLaunchKernelGGL((softmax_kernel<64, false>), dim3(blocks), dim3(256), 0, st, in, mask, (long long)n_masks, (long long)rows_per_mask, out, (long long)rows, (int)cols);
-  } else if(!mask && cols % 4 == 0 && cols <= 32768 && aligned16(in) && aligned16(out)) {
-    if(log) hipLaunchKernelGGL(softmax_wide_kernel<true>, dim3((unsigned)rows), dim3(1024), 0, st, in, out, (int)cols);
-    else hipLaunchKernelGGL(softmax_wide_kernel<false>, dim3((unsigned)rows), dim3(1024), 0, st, in, out, (int)cols);
+  } else if(wide_ok && cols <= 4096) {
+    if(log) hipLaunchKernelGGL((softmax_wide_kernel<true, 256, 4>), dim3((unsigned)rows), dim3(256), 0, st, in, out, (int)cols);
+    else hipLaunchKernelGGL((softmax_wide_kernel<false, 256, 4>), dim3((unsigned)rows), dim3(256), 0, st, in, out, (int)cols);
+  } else if(wide_ok) {
+    if(log) hipLaunchKernelGGL((softmax_wide_kernel<true, 1024, 8>), dim3((unsigned)rows), dim3(1024), 0, st, in, out, (int)cols);
+    else hipLaunchKernelGGL((softmax_wide_kernel<false, 1024, 8>), dim3((unsigned)rows), dim3(1024), 0, st, in, out, (int)cols);
   } else {
     if(log) hipLaunchKernelGGL((softmax_kernel<1024, true>), dim3((unsigned)rows), dim3(1024), 0, st, in, mask, (long long)n_masks, (long long)rows_per_mask, out, (long long)rows, (int)cols);
     else hipLaunchKernelGGL((softmax_kernel<1024, false>), dim3((unsigned)rows), dim3(1024), 0, st, in, mask, (long long)n_masks, (long long)rows_per_mask, out, (long long)rows, (int)cols);
