@@ -295,6 +295,79 @@ __global__ __launch_bounds__(256) void bdot_kernel(const float* __restrict__ A, 
   }
 }
 
+// The same products for matrices with many rows (encoder-size attention: m = n = 64 per head):
+// a workgroup takes a 64 x 64 tile of one batch entry, K in chunks of 32 through LDS, a thread a
+// 4 x 4 patch.  Every output is still summed over p = 0 .. k-1 in ascending order with one fma per
+// term, so the result equals bdot_kernel's bit for bit.  A not transposed, k % 4 == 0 (TRANSB:
+// B is [n x k]) or n % 4 == 0 (B is [k x n]), 16-byte aligned matrices.
+template <bool TRANSB>
+__global__ __launch_bounds__(256) void bdot_tile_kernel(const float* __restrict__ A, const float* __restrict__ B,
+                                                        float* __restrict__ C, long long batchA,
+                                                        long long batchB, int m, int n, int k, float scalar) {
+  constexpr int KC = 32, LD = 64 + 4;
+  __shared__ __attribute__((aligned(16))) float As[KC][LD];   // [p][row]
+  __shared__ __attribute__((aligned(16))) float Bs[KC][LD];   // [p][col]
+  const long long i = blockIdx.z;
+  const float* a = A + (size_t)(i % batchA) * m * k;
+  const float* b = B + (size_t)(i % batchB) * n * k;
+  float* c = C + (size_t)i * m * n;
+  const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
+  const int tid = threadIdx.x, ty = tid / 16, tx = tid % 16;
+  float acc[4][4];
+#pragma unroll
+  for(int y = 0; y < 4; ++y)
+#pragma unroll
+    for(int x = 0; x < 4; ++x) acc[y][x] = 0.0f;
+  for(int p0 = 0; p0 < k; p0 += KC) {
+    const int pc = min(KC, k - p0);   // a multiple of four
+    __syncthreads();                  // the previous chunk has been read
+    // rows of A (and of a transposed B): lane = row, so that the transposing LDS writes of a wave
+    // fall into consecutive banks; four consecutive p per load
+#pragma unroll
+    for(int h = 0; h < 2; ++h) {
+      const int idx = h * 256 + tid, row = idx % 64, p4 = idx / 64;   // p4 = 0 .. 7
+      if(p4 * 4 < pc) {
+        const v4f v = *reinterpret_cast<const v4f*>(a + (size_t)min(r0 + row, m - 1) * k + p0 + p4 * 4);
+        As[p4 * 4][row] = v.x; As[p4 * 4 + 1][row] = v.y; As[p4 * 4 + 2][row] = v.z; As[p4 * 4 + 3][row] = v.w;
+        if(TRANSB) {
+          const v4f w = *reinterpret_cast<const v4f*>(b + (size_t)min(c0 + row, n - 1) * k + p0 + p4 * 4);
+          Bs[p4 * 4][row] = w.x; Bs[p4 * 4 + 1][row] = w.y; Bs[p4 * 4 + 2][row] = w.z; Bs[p4 * 4 + 3][row] = w.w;
+        }
+      }
+    }
+    if(!TRANSB) {   // B is [k x n]: rows p, four consecutive columns per load
+#pragma unroll
+      for(int h = 0; h < 2; ++h) {
+        const int idx = h * 256 + tid, col4 = idx % 16, p = idx / 16;   // p = 0 .. 31
+        if(p < pc) {
+          const int col = min(c0 + col4 * 4, n - 4);   // (n % 4 == 0; columns past n are never stored)
+          *reinterpret_cast<v4f*>(&Bs[p][col4 * 4]) = *reinterpret_cast<const v4f*>(b + (size_t)(p0 + p) * n + col);
+        }
+      }
+    }
+    __syncthreads();
+    for(int p = 0; p < pc; ++p) {
+      const v4f av = *reinterpret_cast<const v4f*>(&As[p][ty * 4]);
+      const v4f bv = *reinterpret_cast<const v4f*>(&Bs[p][tx * 4]);
+      const float ar[4] = {av.x, av.y, av.z, av.w}, br[4] = {bv.x, bv.y, bv.z, bv.w};
+#pragma unroll
+      for(int y = 0; y < 4; ++y)
+#pragma unroll
+        for(int x = 0; x < 4; ++x) acc[y][x] = fmaf(ar[y], br[x], acc[y][x]);
+    }
+  }
+#pragma unroll
+  for(int y = 0; y < 4; ++y) {
+    const int r = r0 + ty * 4 + y;
+    if(r >= m) continue;
+#pragma unroll
+    for(int x = 0; x < 4; ++x) {
+      const int q = c0 + tx * 4 + x;
+      if(q < n) c[(size_t)r * n + q] = scalar * acc[y][x];
+    }
+  }
+}
+
 // ---------------------------------------------------------------- one-launch attention
 // One wave per query row (entry i, row r): scores over the key positions (a lane per position,
 // the query row and a key row are walked with the same fused multiply-adds, in the same order,
@@ -962,6 +1035,19 @@ int marian_hip_bdot_legacy(const float* A, const float* B, float* C, int64_t bat
   if(!aligned4(A) || !aligned4(B) || !aligned4(C)) return MARIAN_HIP_ERR_ALIGN;
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   const long long rows_total = batchC * m;
+  const bool tile_ok = !transA && m >= 8 && batchC <= 65535 && aligned16(A) && aligned16(B) &&
+                       (transB ? k % 4 == 0 : (k % 4 == 0 && n % 4 == 0));
+  if(tile_ok) {
+    const dim3 grid((unsigned)((n + 63) / 64), (unsigned)((m + 63) / 64), (unsigned)batchC);
+    if(transB)
+      hipLaunchKernelGGL(bdot_tile_kernel<true>, grid, dim3(256), 0, st, A, B, C, (long long)batchA,
+                         (long long)batchB, (int)m, (int)n, (int)k, scalar);
+    else
+      hipLaunchKernelGGL(bdot_tile_kernel<false>, grid, dim3(256), 0, st, A, B, C, (long long)batchA,
+                         (long long)batchB, (int)m, (int)n, (int)k, scalar);
+    MH_HIP(hipGetLastError());
+    return MARIAN_HIP_OK;
+  }
   hipLaunchKernelGGL(bdot_kernel, dim3((unsigned)((rows_total + 3) / 4)), dim3(256), 0, st, A, B, C,
                      (long long)batchA, (long long)batchB, rows_total, (int)m, (int)n, (int)k,
                      transA ? 1 : 0, transB ? 1 : 0, scalar);

@@ -125,7 +125,9 @@ def test_split_and_join_heads(ops, synth):
 
 
 @pytest.mark.parametrize("tA,tB", [(False, False), (False, True), (True, False), (True, True)])
-@pytest.mark.parametrize("batch,m,n,k", [(6, 3, 5, 8), (2048, 1, 40, 64), (2048, 1, 64, 40), (8, 33, 70, 65)])
+@pytest.mark.parametrize("batch,m,n,k", [(6, 3, 5, 8), (2048, 1, 40, 64), (2048, 1, 64, 40), (8, 33, 70, 65),
+                                         (4, 64, 64, 64), (3, 70, 100, 36), (2, 9, 8, 8), (16, 40, 44, 64),
+                                         (64, 64, 64, 64)])
 def test_bdot_legacy(ops, chk, synth, tA, tB, batch, m, n, k):
     a = synth.normal(batch + m, 0, (batch, k, m) if tA else (batch, m, k), 1.0)
     b = synth.normal(batch + n, 1, (batch, n, k) if tB else (batch, k, n), 1.0)
