@@ -80,6 +80,10 @@ int marian_hip_bdot_legacy(const float* A, const float* B, float* C, int64_t bat
  *   q: [batchQ, m, dk], k and v: [batchKV, len, dk] (entry i uses k, v of i % batchKV: encoder
  *   keys shared by the beam), out: [batchQ, m, dk]; mask as in marian_hip_softmax for score rows
  *   [batchQ * m, len], or NULL.  len <= 4096.
+ *   Built for decoding steps (m = 1 or a few query positions per head): every query row gets a
+ *   wave that walks the head's keys and values itself.  With eight or more positions per head
+ *   (encoder layers) the three separate entry points, which share a head's keys and values
+ *   through LDS tiles, are about twice as fast; the host mirror switches over by itself.
  *   absmax_out: as for marian_hip_layer_norm (needs batchQ * m <= 2048).
  *   k_new, v_new: NULL, or [batchQ, dk] keys and values of the newest position (self-attention of
  *   a decoding step: m == 1, batchKV == batchQ).  They take the place of position len - 1 of k and

@@ -148,6 +148,13 @@ def Attention(q, k, v, mask=None, rowsPerMask=1, want_absmax=False, kNew=None, v
               tuple(k.shape), tuple(v.shape), dk)
     batchQ = q.numel() // (m * dk)
     batchKV = k.numel() // (L * dk)
+    if m >= 8 and kNew is None and not want_absmax:
+        # Many query positions per head (encoder layers, whole target sentences): the one-launch
+        # form gives every query row a wave that walks the head's keys and values on its own; the
+        # three operators share them through LDS tiles (1024 heads of 64 x 64 x 64: 57 us against 105).
+        scores = bdot_legacy(q.reshape(batchQ, m, dk), k.reshape(batchKV, L, dk), False, True, 1.0 / float(dk) ** 0.5)
+        weights = softmax(scores, mask, rowsPerMask)
+        return bdot_legacy(weights, v.reshape(batchKV, L, dk)).reshape(q.shape)
     n_masks = 0
     if mask is not None:
         mask = _f32c(mask, "Attention").reshape(-1, L)

@@ -222,6 +222,28 @@ def test_absmax_outputs_of_layer_norm_and_attention(ops, integer, synth):
         assert np.array_equal(aq.numpy(), aq_ref.numpy()) and np.array_equal(got.cpu().numpy(), want.cpu().numpy())
 
 
+@pytest.mark.parametrize("BQ,BKV,m,L,dk,masked", [(24, 24, 40, 40, 64, True), (16, 8, 9, 33, 32, False)])
+def test_attention_with_many_query_positions(ops, synth, BQ, BKV, m, L, dk, masked):
+    """Encoder-size use (many query positions per head; the host mirror runs the three operators):
+    against the float64 closed form."""
+    q = synth.normal(BQ + m, 0, (BQ, m, dk), 1.0)
+    k = synth.normal(BQ + m, 1, (BKV, L, dk), 1.0)
+    v = synth.normal(BQ + m, 2, (BKV, L, dk), 1.0)
+    mask = None
+    heads = 4
+    if masked:   # one mask row per sentence, shared by its heads and query positions
+        mask = np.zeros((BQ // heads, L), np.float32)
+        mask[:, L - 5:] = -np.inf
+    got = ops.Attention(dev(q), dev(k), dev(v), None if mask is None else dev(mask), heads * m).cpu().numpy()
+    z = np.einsum("bmd,bld->bml", q.astype(f64), k.astype(f64)[np.arange(BQ) % BKV]) / np.sqrt(dk)
+    if masked:
+        z = z + mask.astype(f64)[np.arange(BQ) // heads][:, None, :]
+    w = np.exp(z - z.max(-1, keepdims=True))
+    w = w / w.sum(-1, keepdims=True)
+    want = np.einsum("bml,bld->bmd", w, v.astype(f64)[np.arange(BQ) % BKV])
+    close(got, want, 4 * REL, 2e-5)
+
+
 @pytest.mark.parametrize("BH,T,dk", [(2048, 21, 64), (64, 1, 64), (48, 70, 20), (16, 9, 64)])
 def test_attention_with_cache_append(ops, synth, BH, T, dk):
     """kNew / vNew stand for the last cached position and are stored there: same output bits as
