@@ -402,7 +402,10 @@ int launch_gemm(const GemmArgs& a, hipStream_t st) {
   //  - otherwise the 32x32x32 MFMA kernel, which also tiles M (shortlisted output layer, M = 256)
   const int tiles32 = (a.n_out + 31) / 32;
   if(a.M <= 8 || (a.M <= 16 && tiles32 < 512)) return launch_stream_auto(a, st, 2);
-  if(a.M <= 128 || (a.M <= 512 && tiles32 < 128))
+  //    (few columns, M up to 512; beyond 256 rows with K >= 2048 and 1024 or more columns the
+  //    128x64-tile kernel below is 20 % faster)
+  if(a.M <= 128 || (a.M <= 512 && tiles32 < 128 &&
+                    (a.M <= 256 || a.K < 2048 || tiles32 < 32 || a.K % 128 != 0)))
     return launch_stream32_auto<kPrequant>(a, FusedSrc(), st, 0);
   if(a.K % 128 != 0) return launch_tile<4, 4>(a, st);
   // large outputs: 256x256 tiles (one per CU keeps operand traffic lowest); otherwise 128x128
@@ -423,6 +426,12 @@ int launch_gemm(const GemmArgs& a, hipStream_t st) {
   if(tiles128 >= 2 * compute_units()) {
     if(stream_out) return launch_big<128, 128, 2, 4, 2, true, true>(a, st);
     return launch_big<128, 128, 2, 4, 2>(a, st);
+  }
+  // so few 128x128 tiles that half the CUs would idle: 128x64 tiles (measured -20 % to -25 % for
+  // M = 512 .. 1024, K = 4096, N = 1024; measurement id 340 keeps the square tiles)
+  if(2 * tiles128 <= compute_units() && g_kernel_override.load(std::memory_order_relaxed) % 1000 != 340) {
+    if(stream_out) return launch_big<128, 64, 2, 2, 3, true, true>(a, st);
+    return launch_big<128, 64, 2, 2, 3>(a, st);
   }
   if(stream_out) return launch_big<128, 128, 2, 2, 3, true, true>(a, st);
   return launch_big<128, 128, 2, 2, 3>(a, st);

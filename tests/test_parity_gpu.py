@@ -117,12 +117,21 @@ def test_multiply_all_kernels_small_m(integer, orc, synth, M, K, N, kernel):
     run_case(integer, orc, synth, 300 + M + N, M, K, N, kernel, bias_on=True, relu=(M % 2 == 0))
 
 
-@pytest.mark.parametrize("kernel", [0, 501, 512, 521, 522, 524, 201, 202, 203, 204, 301, 302, 303, 304, 305, 306, 307, 308, 311, 312, 330, 401, 402, 403, 404, 411, 413, 416])
+@pytest.mark.parametrize("kernel", [0, 501, 512, 521, 522, 524, 201, 202, 203, 204, 301, 302, 303, 304, 305, 306, 307, 308, 311, 312, 313, 330, 340, 401, 402, 403, 404, 411, 413, 416])
 @pytest.mark.parametrize("M,K,N", [(129, 64, 8), (256, 1024, 504), (300, 320, 1000), (513, 128, 264)])
 def test_multiply_tile_kernels_ragged(integer, orc, synth, M, K, N, kernel):
     say("multiply ragged", M, K, N, "kernel", kernel)
     run_case(integer, orc, synth, 400 + M + N, M, K, N, kernel, bias_on=(N % 16 == 8), relu=True,
              scale=0.5)
+
+
+@pytest.mark.parametrize("M,K,N", [(384, 4096, 1024), (512, 2048, 1024), (640, 1024, 1024), (520, 2048, 1000),
+                                   (300, 4096, 512), (512, 2048, 512), (384, 2112, 1024)])
+def test_multiply_mid_size_dispatch(integer, orc, synth, M, K, N):
+    """Between the decode and the encoder sizes: the shapes around the switch from the
+    weight-streaming kernels to 128x64 tiles (few tiles, long K), both sides of it."""
+    say("multiply mid size", M, K, N)
+    run_case(integer, orc, synth, 470 + M + N, M, K, N, 0, bias_on=True, relu=(M % 128 == 0), scale=1.5)
 
 
 @pytest.mark.parametrize("kernel", [330, 331])
