@@ -179,15 +179,18 @@ __global__ __launch_bounds__(THREADS < 256 ? 256 : THREADS) void softmax_kernel(
   }
 }
 
-// Rows kept in registers (cols % 4 == 0, 16-byte aligned rows, no mask), so that they are read
-// once: 1024 threads with eight float4 each for vocabulary-size rows (up to 32768), 256 threads
-// with four for rows up to 4096.  Same
+// Rows kept in registers (cols % 4 == 0, 16-byte aligned rows and mask), so that they are read
+// once: 256 threads with four float4 each for rows up to 4096 values, 1024 threads with eight or
+// sixteen for vocabulary-size rows (up to 32768 / 65536).  Same
 // operations per element as softmax_kernel.
 template <bool LOG, int THREADS, int VPT>
-__global__ __launch_bounds__(THREADS) void softmax_wide_kernel(const float* in, float* out, int cols) {
+__global__ __launch_bounds__(THREADS) void softmax_wide_kernel(const float* in, const float* __restrict__ mask,
+                                                                long long n_masks, long long rows_per_mask,
+                                                                float* out, int cols) {
   __shared__ float red[THREADS / 64];
   const size_t row = blockIdx.x;
   const v4f* x = reinterpret_cast<const v4f*>(in + row * cols);
+  const v4f* mk = mask ? reinterpret_cast<const v4f*>(mask + (size_t)((row / rows_per_mask) % n_masks) * cols) : nullptr;
   v4f* y = reinterpret_cast<v4f*>(out + row * cols);
   const int cols4 = cols / 4, t = threadIdx.x;
   v4f v[VPT];
@@ -196,6 +199,15 @@ __global__ __launch_bounds__(THREADS) void softmax_wide_kernel(const float* in, 
   // range check is waited for inside its branch, one memory latency per load)
 #pragma unroll
   for(int j = 0; j < VPT; ++j) v[j] = x[min(j * THREADS + t, cols4 - 1)];
+  if(mk) {   // (wave-uniform: the whole row has a mask or none)
+    v4f mv[VPT];
+#pragma unroll
+    for(int j = 0; j < VPT; ++j) mv[j] = mk[min(j * THREADS + t, cols4 - 1)];
+#pragma unroll
+    for(int j = 0; j < VPT; ++j) {
+      v[j].x = v[j].x + mv[j].x; v[j].y = v[j].y + mv[j].y; v[j].z = v[j].z + mv[j].z; v[j].w = v[j].w + mv[j].w;
+    }
+  }
 #pragma unroll
   for(int j = 0; j < VPT; ++j) {
     const int i = j * THREADS + t;
@@ -958,6 +970,8 @@ int marian_hip_layer_norm(const float* in, const float* add, const float* gamma,
     hipLaunchKernelGGL(layer_norm_kernel<1>, dim3((unsigned)rows), dim3(256), 0, st, in, add, gamma, gs, beta, bs, out, (int)cols, eps, absmax_out);
   else if(vec && cols <= 4096)
     hipLaunchKernelGGL(layer_norm_kernel<4>, dim3((unsigned)rows), dim3(256), 0, st, in, add, gamma, gs, beta, bs, out, (int)cols, eps, absmax_out);
+  else if(vec && cols <= 8192)
+    hipLaunchKernelGGL(layer_norm_kernel<8>, dim3((unsigned)rows), dim3(256), 0, st, in, add, gamma, gs, beta, bs, out, (int)cols, eps, absmax_out);
   else
     hipLaunchKernelGGL(layer_norm_kernel<0>, dim3((unsigned)rows), dim3(256), 0, st, in, add, gamma, gs, beta, bs, out, (int)cols, eps, absmax_out);
   MH_HIP(hipGetLastError());
@@ -974,19 +988,22 @@ static int softmax_common(const float* in, const float* mask, int64_t n_masks, i
   if(!aligned4(in) || !aligned4(out) || (mask && !aligned4(mask))) return MARIAN_HIP_ERR_ALIGN;
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   if(!mask) { n_masks = 1; rows_per_mask = 1; }
-  // rows that fit registers of one workgroup and need no mask: read once (a wave per row walks a
-  // 1024-value row in 16 dependent steps per pass: 10 us for 128 rows against 4)
-  const bool wide_ok = !mask && cols % 4 == 0 && cols <= 32768 && aligned16(in) && aligned16(out);
+  // rows of more than 256 values that fit the registers of one workgroup: read once (a wave per row
+  // walks a 1024-value row in 16 dependent steps per pass: 10 us for 128 rows against 4)
+  const bool wide_ok = cols % 4 == 0 && cols <= 65536 && aligned16(in) && aligned16(out) && (!mask || aligned16(mask));
   if(cols <= 2048 && !(wide_ok && cols > 256)) {
     const unsigned blocks = (unsigned)((rows + 3) / 4);
     if(log) hipLaunchKernelGGL((softmax_kernel<64, true>), dim3(blocks), dim3(256), 0, st, in, mask, (long long)n_masks, (long long)rows_per_mask, out, (long long)rows, (int)cols);
     else hipLaunchKernelGGL((softmax_kernel<64, false>), dim3(blocks), dim3(256), 0, st, in, mask, (long long)n_masks, (long long)rows_per_mask, out, (long long)rows, (int)cols);
   } else if(wide_ok && cols <= 4096) {
-    if(log) hipLaunchKernelGGL((softmax_wide_kernel<true, 256, 4>), dim3((unsigned)rows), dim3(256), 0, st, in, out, (int)cols);
-    else hipLaunchKernelGGL((softmax_wide_kernel<false, 256, 4>), dim3((unsigned)rows), dim3(256), 0, st, in, out, (int)cols);
+    if(log) hipLaunchKernelGGL((softmax_wide_kernel<true, 256, 4>), dim3((unsigned)rows), dim3(256), 0, st, in, mask, (long long)n_masks, (long long)rows_per_mask, out, (int)cols);
+    else hipLaunchKernelGGL((softmax_wide_kernel<false, 256, 4>), dim3((unsigned)rows), dim3(256), 0, st, in, mask, (long long)n_masks, (long long)rows_per_mask, out, (int)cols);
+  } else if(wide_ok && cols <= 32768) {
+    if(log) hipLaunchKernelGGL((softmax_wide_kernel<true, 1024, 8>), dim3((unsigned)rows), dim3(1024), 0, st, in, mask, (long long)n_masks, (long long)rows_per_mask, out, (int)cols);
+    else hipLaunchKernelGGL((softmax_wide_kernel<false, 1024, 8>), dim3((unsigned)rows), dim3(1024), 0, st, in, mask, (long long)n_masks, (long long)rows_per_mask, out, (int)cols);
   } else if(wide_ok) {
-    if(log) hipLaunchKernelGGL((softmax_wide_kernel<true, 1024, 8>), dim3((unsigned)rows), dim3(1024), 0, st, in, out, (int)cols);
-    else hipLaunchKernelGGL((softmax_wide_kernel<false, 1024, 8>), dim3((unsigned)rows), dim3(1024), 0, st, in, out, (int)cols);
+    if(log) hipLaunchKernelGGL((softmax_wide_kernel<true, 1024, 16>), dim3((unsigned)rows), dim3(1024), 0, st, in, mask, (long long)n_masks, (long long)rows_per_mask, out, (int)cols);
+    else hipLaunchKernelGGL((softmax_wide_kernel<false, 1024, 16>), dim3((unsigned)rows), dim3(1024), 0, st, in, mask, (long long)n_masks, (long long)rows_per_mask, out, (int)cols);
   } else {
     if(log) hipLaunchKernelGGL((softmax_kernel<1024, true>), dim3((unsigned)rows), dim3(1024), 0, st, in, mask, (long long)n_masks, (long long)rows_per_mask, out, (long long)rows, (int)cols);
     else hipLaunchKernelGGL((softmax_kernel<1024, false>), dim3((unsigned)rows), dim3(1024), 0, st, in, mask, (long long)n_masks, (long long)rows_per_mask, out, (long long)rows, (int)cols);

@@ -42,7 +42,7 @@ def close(got, want, rel=REL, floor=1e-6):
 
 
 @pytest.mark.parametrize("rows,cols", [(1, 8), (5, 64), (128, 1024), (3, 1000), (7, 4096), (2, 5000),
-                                       (4, 1023)])
+                                       (4, 1023), (3, 8192), (2, 8196)])
 @pytest.mark.parametrize("with_add,with_beta", [(False, True), (True, True), (True, False)])
 def test_layer_norm(ops, chk, synth, rows, cols, with_add, with_beta):
     x = synth.normal(rows * 7 + cols, 0, (rows, cols), 2.0) + np.float32(0.3)
@@ -73,7 +73,8 @@ def test_layer_norm_4d_and_inplace_shapes(ops, chk, synth):
 
 
 @pytest.mark.parametrize("rows,cols", [(1, 1), (7, 5), (2048, 40), (4096, 64), (33, 2048), (5, 2049),
-                                       (128, 32000), (3, 32768), (2, 32772), (3, 8190), (4, 4100)])
+                                       (128, 32000), (3, 32768), (2, 32772), (3, 8190), (4, 4100),
+                                       (5, 50000), (2, 65536), (2, 65540), (300, 512)])
 def test_softmax_and_logsoftmax(ops, chk, synth, rows, cols):
     x = synth.normal(rows + cols, 0, (rows, cols), 3.0)
     xs = x.astype(f64)
@@ -103,6 +104,21 @@ def test_softmax_with_attention_mask(ops, chk, synth):
     g4 = got.reshape(beam, batch, heads, L)
     for bi in range(batch):
         assert np.all(g4[:, bi, :, lens[bi]:] == 0) and np.allclose(g4[:, bi].sum(-1), 1.0, atol=1e-5)
+
+
+@pytest.mark.parametrize("L", [300, 1000, 4100, 258])
+def test_softmax_with_mask_on_long_rows(ops, chk, synth, L):
+    """Masked rows of more than 256 scores (long source sentences): the register-resident kernels
+    add the mask row as they load."""
+    batch, heads = 6, 4
+    z = synth.normal(22 + L, 0, (batch, heads, 3, L), 1.0)
+    lens = 1 + (np.arange(batch) * 97) % L
+    mask = ((np.arange(L)[None, :] >= lens[:, None]) * -99999999.0).astype(np.float32)
+    got = ops.softmax(dev(z), dev(mask), rowsPerMask=heads * 3).cpu().numpy()
+    zs = z.astype(f64) + mask.astype(f64)[:, None, None, :]
+    e = np.exp(zs - zs.max(-1, keepdims=True))
+    close(got, e / e.sum(-1, keepdims=True), REL, 1e-10)
+    close(got, chk.softmax(z, mask, rows_per_mask=heads * 3), REL * max(1.0, L / 250.0), 1e-10)
 
 
 @pytest.mark.parametrize("shape", [(3, 5, 7, 4), (128, 1, 16, 64), (128, 16, 1, 64), (32, 40, 16, 64),
