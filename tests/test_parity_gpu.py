@@ -426,6 +426,53 @@ def test_random_shapes_both_entry_points(integer, orc, synth, i, M, K, N, bias_o
     assert np.array_equal(out2, want) and np.array_equal(out1.cpu().numpy(), want)
 
 
+def _random_large_cases(n):
+    """Seeded shapes above the decode sizes: M 601..4500, K a multiple of 64 up to 4096, N a
+    multiple of 8 up to 4096 - whole and ragged tiles of every large-M kernel under the automatic
+    choice.  Sizes are bounded so that the checker needs at most a few seconds per case."""
+    rng = np.random.default_rng(20261126)
+    cases = []
+    while len(cases) < n:
+        M = int(rng.choice([640, 768, 1000, 1024, 1280, 1536, 2048, 2050, 2560, 3000, 4096, 4500]))
+        K = 64 * int(rng.integers(1, 65))
+        N = 8 * int(rng.integers(1, 513))
+        if len(cases) % 3 == 0:   # whole tiles: the shapes the 256-wide kernels take
+            K = 128 * int(rng.integers(4, 33))
+            N = 256 * int(rng.integers(1, 17))
+            M = 256 * int(rng.integers(3, 17))
+        if M * K * N > 2.5e10:
+            continue
+        cases.append((len(cases), M, K, N, bool(rng.integers(2)), bool(rng.integers(2)),
+                      float(rng.choice([1.0, 0.5, 3.0])), bool(rng.integers(4) == 0)))
+    return cases
+
+
+@pytest.mark.parametrize("i,M,K,N,bias_on,relu,scale,short", _random_large_cases(24))
+def test_random_large_shapes_both_entry_points(integer, orc, synth, i, M, K, N, bias_on, relu, scale, short):
+    """Automatic kernel choice on seeded random shapes of encoder size, both call forms."""
+    import torch
+    say("random large", i, M, K, N, bias_on, relu, scale, short)
+    A, W, bias = inputs(synth, 7000 + i, M, K, N)
+    Aq_h, Bq_h = orc.prepare_a(A), orc.prepare_b(W)
+    b = bias if bias_on else None
+    didx = None
+    if short and N >= 64:
+        idx = synth.shortlist(7000 + i, N, 8, max(8, N // 2))
+        didx = torch.from_numpy(idx.view(np.int32)).cuda()
+        want, want_acc = orc.affine_shortlist(Aq_h, Bq_h, b, idx, M, K, N, scale, relu)
+    else:
+        want, want_acc = orc.affine(Aq_h, Bq_h, b, M, K, N, scale, relu)
+    Bq = upload_q(integer, Bq_h, (K, N))
+    db = dev(bias) if bias_on else None
+    Aq = integer.prepareA(dev(A))
+    assert np.array_equal(Aq.numpy(), Aq_h)
+    assert np.array_equal(integer.multiply_i32(Aq, Bq, shortlist=didx).cpu().numpy(), want_acc)
+    out2 = integer.multiply(Aq, Bq, db, scale=scale, relu=relu, shortlist=didx).cpu().numpy()
+    out1, Aq1 = integer.affine_f32(dev(A), Bq, db, scale=scale, relu=relu, shortlist=didx)
+    assert np.array_equal(Aq1.numpy(), Aq_h)
+    assert np.array_equal(out2, want) and np.array_equal(out1.cpu().numpy(), want)
+
+
 # ---------------------------------------------------------------- fixtures, contract, errors
 
 def test_golden_fixtures_on_gpu(integer):
