@@ -163,6 +163,66 @@ def test_bdot_legacy(ops, chk, synth, tA, tB, batch, m, n, k):
     close(got2, want2, REL, 8 * floor)
 
 
+def _random_row_cases(n):
+    rng = np.random.default_rng(20261128)
+    cases = []
+    for i in range(n):
+        cols = int(rng.choice([1, 3, 64, 100, 255, 256, 260, 1024, 2047, 2052, 4096, 4104, 8192, 9000,
+                               32768, 40000, 65536, 66000]))
+        rows = int(rng.integers(1, 600)) if cols <= 4104 else int(rng.integers(1, 12))
+        cases.append((i, rows, cols))
+    return cases
+
+
+@pytest.mark.parametrize("i,rows,cols", _random_row_cases(28))
+def test_row_operators_random_shapes(ops, synth, i, rows, cols):
+    """Seeded random shapes through softmax (plain and with a mask per group of rows), log-softmax
+    and layer norm (with the skip input), against float64: every column-count range of the
+    kernel choice, aligned and unaligned row lengths."""
+    x = synth.normal(9500 + i, 0, (rows, cols), 2.5)
+    xs = x.astype(f64)
+    e = np.exp(xs - xs.max(-1, keepdims=True))
+    close(ops.softmax(dev(x)).cpu().numpy(), e / e.sum(-1, keepdims=True), REL, 1e-10)
+    close(ops.logsoftmax(dev(x)).cpu().numpy(), xs - xs.max(-1, keepdims=True) - np.log(e.sum(-1, keepdims=True)),
+          REL, 1e-5)
+    # mask rows shared by rpm consecutive score rows
+    rpm = [r for r in (1, 2, 3, 4, 5) if rows % r == 0][-1]
+    lens = 1 + (np.arange(rows // rpm) * 37) % cols
+    mask = ((np.arange(cols)[None, :] >= lens[:, None]) * -99999999.0).astype(np.float32)
+    zs = xs.reshape(rows // rpm, rpm, cols) + mask.astype(f64)[:, None, :]
+    em = np.exp(zs - zs.max(-1, keepdims=True))
+    got = ops.softmax(dev(x.reshape(rows // rpm, rpm, 1, cols)), dev(mask), rowsPerMask=rpm).cpu().numpy()
+    close(got.reshape(rows // rpm, rpm, cols), em / em.sum(-1, keepdims=True), REL, 1e-10)
+    g = synth.normal(9500 + i, 2, (cols,), 0.2) + np.float32(1.0)
+    b = synth.normal(9500 + i, 3, (cols,), 0.5)
+    add = synth.normal(9500 + i, 1, (rows, cols), 1.0)
+    ys = xs + add.astype(f64)
+    mean = ys.mean(-1, keepdims=True)
+    var = ((ys - mean) ** 2).mean(-1, keepdims=True)
+    want = g.astype(f64) * (ys - mean) / np.sqrt(var + 1e-6) + b.astype(f64)
+    # x + add is rounded to float32 before the mean is taken off: rows whose values nearly coincide
+    # amplify that rounding by max|y| / sigma, in any float32 implementation
+    floor = 2e-6 + 4 * 2.0 ** -24 * np.abs(ys).max(-1, keepdims=True) / np.sqrt(var + 1e-6) * np.abs(g).max()
+    close(ops.layerNorm(dev(x), dev(g), dev(b), 1e-6, dev(add)).cpu().numpy(), want, REL, floor)
+
+
+def _random_bdot_cases(n):
+    rng = np.random.default_rng(20261129)
+    return [(i, int(rng.integers(1, 40)), int(rng.integers(1, 100)), int(rng.integers(1, 100)),
+             int(rng.choice([1, 4, 8, 20, 36, 64, 65, 128])), bool(rng.integers(2)), bool(rng.integers(2)))
+            for i in range(n)]
+
+
+@pytest.mark.parametrize("i,batch,m,n,k,tA,tB", _random_bdot_cases(24))
+def test_bdot_random_shapes(ops, synth, i, batch, m, n, k, tA, tB):
+    a = synth.normal(9700 + i, 0, (batch, k, m) if tA else (batch, m, k), 1.0)
+    b = synth.normal(9700 + i, 1, (batch, n, k) if tB else (batch, k, n), 1.0)
+    got = ops.bdot_legacy(dev(a), dev(b), tA, tB, 0.5).cpu().numpy()
+    A = a.transpose(0, 2, 1) if tA else a
+    B = b.transpose(0, 2, 1) if tB else b
+    close(got, 0.5 * np.matmul(A.astype(f64), B.astype(f64)), REL, 2e-6 * np.sqrt(k))
+
+
 def test_attention_products_of_a_decode_step(ops, chk, synth):
     """q [B*H, 1, dk] . k^T [B*H, len, dk] * 1/sqrt(dk), softmax, . v [B*H, len, dk]
     (reference src/models/transformer.h:258-277) against the checker, op by op."""
@@ -318,6 +378,35 @@ def test_nbest_of_beams(ops, chk, synth, batch, beam, V, N):
     if batch * beam * V <= 20000:
         cv, ck = chk.nbest(swapped, N)
         assert np.array_equal(vals.cpu().numpy(), cv) and np.array_equal(keys.cpu().numpy().view(np.uint32), ck)
+
+
+def _random_nbest_cases(n):
+    rng = np.random.default_rng(20261127)
+    cases = []
+    for i in range(n):
+        V = int(rng.choice([8, 20, 63, 64, 65, 257, 1000, 4096, 8191, 32000, 50001, 70003]))
+        beam = int(rng.integers(1, 13))
+        batch = int(rng.integers(1, 41)) if V <= 8191 else int(rng.integers(1, 9))
+        N = int(min(rng.integers(1, 17), beam * V))
+        cases.append((i, batch, beam, V, N, bool(rng.integers(2))))
+    return cases
+
+
+@pytest.mark.parametrize("i,batch,beam,V,N,coarse", _random_nbest_cases(32))
+def test_nbest_random_shapes(ops, synth, i, batch, beam, V, N, coarse):
+    """Seeded random shapes through both n-best entry points against a stable sort; 'coarse' rounds
+    the scores to one decimal, so that equal scores are everywhere (lowest index first)."""
+    x = synth.normal(9000 + i, 0, (beam, 1, batch, V), 2.0)
+    if coarse:
+        x = np.round(x, 1).astype(np.float32)
+    swapped = np.ascontiguousarray(np.swapaxes(x, 0, 2))
+    flat = swapped.reshape(batch, -1)
+    order = np.argsort(-flat, axis=1, kind="stable")[:, :N]
+    want_vals = np.take_along_axis(flat, order, 1)
+    want_keys = order + np.arange(batch)[:, None] * flat.shape[1]
+    for vals, keys in (ops.getNBestListOfBeams(dev(x), N), ops.getNBestList(dev(swapped), N)):
+        assert np.array_equal(vals.cpu().numpy().reshape(batch, N), want_vals)
+        assert np.array_equal(keys.cpu().numpy().view(np.uint32).reshape(batch, N).astype(np.int64), want_keys)
 
 
 def test_nbest_of_beams_argument_checks(ops):
