@@ -320,6 +320,42 @@ def test_attention_with_many_query_positions(ops, synth, BQ, BKV, m, L, dk, mask
     close(got, want, 4 * REL, 2e-5)
 
 
+def _random_attention_cases(n):
+    rng = np.random.default_rng(20261130)
+    cases = []
+    for i in range(n):
+        heads = int(rng.choice([1, 2, 4, 8]))
+        batch = int(rng.integers(1, 7))
+        beam = int(rng.integers(1, 5))
+        cases.append((i, beam, batch, heads, int(rng.choice([1, 1, 1, 2, 7, 8, 9, 20])),
+                      int(rng.choice([1, 2, 15, 16, 17, 40, 63, 64, 65, 130, 300, 1000])),
+                      int(rng.choice([8, 20, 32, 64, 64, 128])), bool(rng.integers(2)), bool(rng.integers(2))))
+    return cases
+
+
+@pytest.mark.parametrize("i,beam,batch,heads,m,L,dk,masked,shared", _random_attention_cases(32))
+def test_attention_random_shapes(ops, synth, i, beam, batch, heads, m, L, dk, masked, shared):
+    """Seeded random shapes against the float64 closed form: one and many query positions, keys and
+    values per beam entry or shared by the beam (i % batchKV), a mask row per sentence."""
+    BQ = beam * batch * heads
+    BKV = batch * heads if shared else BQ
+    q = synth.normal(9800 + i, 0, (BQ, m, dk), 1.0)
+    k = synth.normal(9800 + i, 1, (BKV, L, dk), 1.0)
+    v = synth.normal(9800 + i, 2, (BKV, L, dk), 1.0)
+    mask = None
+    if masked:
+        lens = 1 + (np.arange(batch) * 7 + i) % L
+        mask = ((np.arange(L)[None, :] >= lens[:, None]) * -99999999.0).astype(np.float32)
+    got = ops.Attention(dev(q), dev(k), dev(v), None if mask is None else dev(mask), heads * m).cpu().numpy()
+    z = np.einsum("bmd,bld->bml", q.astype(f64), k.astype(f64)[np.arange(BQ) % BKV]) / np.sqrt(dk)
+    if masked:
+        z = z + mask.astype(f64)[(np.arange(BQ) // heads) % batch][:, None, :]
+    w = np.exp(z - z.max(-1, keepdims=True))
+    w = w / w.sum(-1, keepdims=True)
+    want = np.einsum("bml,bld->bmd", w, v.astype(f64)[np.arange(BQ) % BKV])
+    close(got, want, 4 * REL, 2e-5)
+
+
 @pytest.mark.parametrize("BH,T,dk", [(2048, 21, 64), (64, 1, 64), (48, 70, 20), (16, 9, 64)])
 def test_attention_with_cache_append(ops, synth, BH, T, dk):
     """kNew / vNew stand for the last cached position and are stored there: same output bits as
