@@ -85,6 +85,33 @@ def test_prepare_b_bit_exact(integer, orc, synth, K, N):
     assert np.array_equal(q.numpy(), want)
 
 
+def _random_prepare_cases(n):
+    rng = np.random.default_rng(20261131)
+    return [(i, int(rng.choice([1, 2, 5, 31, 64, 100, 511, 512, 513, 1500, 4099])), 64 * int(rng.integers(1, 65)),
+             8 * int(rng.integers(1, 600)), float(rng.choice([1e-3, 0.02, 1.0, 300.0])))
+            for i in range(n)]
+
+
+@pytest.mark.parametrize("i,M,K,N,sigma", _random_prepare_cases(20))
+def test_prepare_a_and_b_random_shapes(integer, orc, synth, i, M, K, N, sigma):
+    """Seeded random shapes and magnitudes through both quantizers; the extreme value sits at a
+    random place with a random sign, and exact .5 multiples of the step make ties to round."""
+    say("prepare random", i, M, K, N, sigma)
+    rng = np.random.default_rng(8000 + i)
+    A = synth.normal(8000 + i, synth.STREAM_A, (M, K), sigma)
+    peak = np.float32(127.0 * 2.0 ** int(rng.integers(-9, 6)))       # quantMult is a power of two
+    A = np.clip(A, -peak, peak)
+    A.flat[int(rng.integers(A.size))] = peak if rng.integers(2) else -peak
+    ties = rng.integers(A.size, size=min(64, A.size))
+    A.flat[ties] = (rng.integers(-126, 126, size=ties.size) + 0.5).astype(f32) * (peak / np.float32(127.0))
+    A.flat[int(rng.integers(A.size))] = peak
+    got = integer.prepareA(dev(A)).numpy()
+    assert np.array_equal(got, orc.prepare_a(A))
+    W = synth.normal(8000 + i, synth.STREAM_W, (K, N), sigma)
+    W.flat[int(rng.integers(W.size))] *= np.float32(-3.0)
+    assert np.array_equal(integer.prepareB(dev(W)).numpy(), orc.prepare_b(W))
+
+
 # ---------------------------------------------------------------- multiply: int32 and fp32
 
 KERNELS = [0, 101, 102, 501, 511, 512, 514, 518, 521, 522, 524, 201, 202, 203, 204, 301, 302, 303, 304, 305, 306, 307, 308, 401, 402, 403, 404, 411, 413, 416]
