@@ -82,12 +82,28 @@ int launch_tile(const GemmArgs& a, hipStream_t st) {
 template <int BM, int BN, int WM, int WN, int NSTAGE, bool PAIRED = true, bool NT = false>
 int launch_big(const GemmArgs& a, hipStream_t st) {
   using Cfg = BigCfg<BM, BN, WM, WN, NSTAGE>;
-  if(a.K % Cfg::BK != 0) return launch_tile<4, 4>(a, st);  // this family needs K % 128 == 0
+  // whole 128-column K blocks, or (paired-fragment form) a last block of 64 columns; measurement id
+  // 350 keeps the 16x16x64 tile kernel for such K
+  const int tiles_n = (a.n_out + BN - 1) / BN;
+  const int tiles_m = (a.M + BM - 1) / BM;
+  if(a.K % Cfg::BK != 0) {
+    if(!PAIRED || a.K % 64 != 0 || g_kernel_override.load(std::memory_order_relaxed) % 1000 == 350)
+      return launch_tile<4, 4>(a, st);
+    if constexpr(!Cfg::kHalfTailOk || !PAIRED) {
+      return launch_big<128, 128, 2, 4, 2, true, NT>(a, st);
+    } else {
+      auto half = gemm_mfma32_kernel<BM, BN, WM, WN, NSTAGE, true, NT, true>;
+      static const int half_lds_status = allow_lds(half, Cfg::kLdsBytes);
+      if(half_lds_status != MARIAN_HIP_OK) return half_lds_status;
+      hipLaunchKernelGGL(half, dim3(tiles_n * tiles_m), dim3(Cfg::kThreads), Cfg::kLdsBytes, st, a,
+                         tiles_n, tiles_m);
+      MH_HIP(hipGetLastError());
+      return MARIAN_HIP_OK;
+    }
+  }
   auto kernel = gemm_mfma32_kernel<BM, BN, WM, WN, NSTAGE, PAIRED, NT>;
   static const int lds_status = allow_lds(kernel, Cfg::kLdsBytes);
   if(lds_status != MARIAN_HIP_OK) return lds_status;
-  int tiles_n = (a.n_out + BN - 1) / BN;
-  int tiles_m = (a.M + BM - 1) / BM;
   hipLaunchKernelGGL(kernel, dim3(tiles_n * tiles_m), dim3(Cfg::kThreads), Cfg::kLdsBytes, st, a,
                      tiles_n, tiles_m);
   MH_HIP(hipGetLastError());
@@ -405,9 +421,8 @@ int launch_gemm(const GemmArgs& a, hipStream_t st) {
   //    (few columns, M up to 512; beyond 256 rows with K >= 2048 and 1024 or more columns the
   //    128x64-tile kernel below is 20 % faster)
   if(a.M <= 128 || (a.M <= 512 && tiles32 < 128 &&
-                    (a.M <= 256 || a.K < 2048 || tiles32 < 32 || a.K % 128 != 0)))
+                    (a.M <= 256 || a.K < 2048 || tiles32 < 32)))
     return launch_stream32_auto<kPrequant>(a, FusedSrc(), st, 0);
-  if(a.K % 128 != 0) return launch_tile<4, 4>(a, st);
   // large outputs: 256x256 tiles (one per CU keeps operand traffic lowest); otherwise 128x128
   // tiles with a three-deep LDS ring so that enough loads are in flight per CU
   const long long tiles256 = ((a.M + 255) / 256) * (long long)((a.n_out + 255) / 256);

@@ -40,6 +40,9 @@ struct BigCfg {
   static constexpr int kLoads = kGroups / kWaves;      // loads per wave per K block
   static constexpr int kLoadsA = (BM / 8) / kWaves;    // the first of them are activation rows
   static constexpr int kLdsBytes = NSTAGE * kStageBytes;
+  // A last K block of 64 columns is supported unless the eight-wave 256x256 tile is chosen: that
+  // one uses 242 of its 256 registers and the few more that the half block needs made it spill.
+  static constexpr bool kHalfTailOk = !(BM == 256 && BN == 256 && kWaves == 8);
   static_assert((BM / 8) % kWaves == 0 && (BN / 8) % kWaves == 0, "tile rows vs waves");
   static_assert(BM % (WAVES_M * 32) == 0 && BN % (WAVES_N * 32) == 0, "tile vs wave grid");
   static_assert(NSTAGE == 2 || NSTAGE == 3, "two or three LDS stages");
@@ -158,7 +161,10 @@ __device__ __forceinline__ void store_tile32_any(const v16i& acc, char* out, siz
 // otherwise sit there dirty until the end of the kernel and be written back then, after the last
 // workgroup, in one piece (measured: 24.1 instead of 25.6 us for a 16 MB output; a 64 MB output
 // does not fit anyway and is 2 % slower with them).
-template <int BM, int BN, int WAVES_M, int WAVES_N, int NSTAGE, bool PAIRED = true, bool NT = false>
+// HALF: K is a multiple of 64 but not of 128, the last block holds 64 columns (an instantiation of
+// its own, so that whole-block calls run code without the checks).
+template <int BM, int BN, int WAVES_M, int WAVES_N, int NSTAGE, bool PAIRED = true, bool NT = false,
+          bool HALF = false>
 __global__ __launch_bounds__(WAVES_M * WAVES_N * kWave) void gemm_mfma32_kernel(
     GemmArgs args, int tiles_n, int tiles_m) {
   using Cfg = BigCfg<BM, BN, WAVES_M, WAVES_N, NSTAGE>;
@@ -173,7 +179,11 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * kWave) void gemm_mfma32_kernel(
   const int wm = wave / WAVES_N, wn = wave % WAVES_N;
   const int li = lane % 32, lg = lane / 32;
   const int K = args.K, M = args.M;
-  const int KB = K / Cfg::BK;
+  // K is a multiple of 64: the last block may hold 64 columns only (PAIRED form; the launcher sends
+  // other K to the plain form only as whole blocks).  Its loads stay inside the rows, see tail_adj.
+  static_assert(!HALF || (PAIRED && Cfg::kHalfTailOk), "no half last block in this form");
+  const int KB = HALF ? (K + Cfg::BK - 1) / Cfg::BK : K / Cfg::BK;
+  constexpr bool half_tail = HALF;
 
   int tn, tm;
   {
@@ -208,15 +218,23 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * kWave) void gemm_mfma32_kernel(
     }
     goff[j] = src * K + chunk * 16;
   }
-  auto issue_one = [&](int kb, int stage, int j) {
+  // A half last block: the lanes of the upper four 16-byte chunks of a row would read past the
+  // row (past the buffer, for the last row), so they re-read the lower half instead; what they
+  // stage is never multiplied.  The chunk of a lane is the same for all its loads (the number of
+  // waves is even, so (row >> 1) & 7 does not depend on j).
+  static_assert(Cfg::kWaves % 2 == 0, "the chunk of a lane must not depend on the load index");
+  const int tail_adj = (((lane % 8) ^ ((((wave * 8 + lane / 8) >> 1)) & 7)) >= 4) ? 64 : 0;
+  auto issue_one = [&](int kb, int stage, int j, auto check_tail) __attribute__((always_inline)) {
     const int8_t* base = (j < Cfg::kLoadsA) ? args.Aq : args.Bq;
-    global_load_lds16(base + (size_t)kb * Cfg::BK, (unsigned)goff[j],
+    int voff = goff[j];
+    if(decltype(check_tail)::value && half_tail && kb == KB - 1) voff -= tail_adj;
+    global_load_lds16(base + (size_t)kb * Cfg::BK, (unsigned)voff,
                       lds_base + stage * Cfg::kStageBytes + (j * Cfg::kWaves + wave) * 1024);
   };
   auto issue = [&](int kb) {
     const int stage = kb % NSTAGE;
 #pragma unroll
-    for(int j = 0; j < Cfg::kLoads; ++j) issue_one(kb, stage, j);
+    for(int j = 0; j < Cfg::kLoads; ++j) issue_one(kb, stage, j, std::true_type());
   };
 
   // ---- fragment addressing: lane (li, lg) reads row li of a 32-row tile, chunk kk*2 + lg ----
@@ -271,7 +289,8 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * kWave) void gemm_mfma32_kernel(
       if(do_issue) {   // wave-uniform: only the load is skipped, the MFMA code exists once
 #pragma unroll
         for(int l = 0; l < LPS; ++l)
-          if(slot * LPS + l < Cfg::kLoads) issue_one(kb + NSTAGE, ld_stage, slot * LPS + l);
+          if(slot * LPS + l < Cfg::kLoads)
+            issue_one(kb + NSTAGE, ld_stage, slot * LPS + l, std::integral_constant<bool, !decltype(steady_c)::value>());
       }
       if(slot < nM) {
 #pragma unroll
@@ -370,10 +389,14 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * kWave) void gemm_mfma32_kernel(
       second_half(steady_c, kb + NSTAGE < KB && !(args.dbg & 1), kb);
     };
     int kb = 0;
+    const int KBsteady = half_tail ? KB - 1 : KB;   // the steady body issues whole blocks only
     if(!(args.dbg & 1))
-      for(; kb + NSTAGE < KB; ++kb) one_block(kb, std::true_type());
+      for(; kb + NSTAGE < KBsteady; ++kb) one_block(kb, std::true_type());
     for(; kb + 1 < KB; ++kb) one_block(kb, std::false_type());
-    {
+    if(half_tail) {   // 64 columns: sub-steps 0 and 1 only
+      multiply(0);
+      multiply(1);
+    } else {
       const int stage = (KB - 1) % NSTAGE;
       read_frags(stage, 2, 2);
       read_frags(stage, 3, 3);

@@ -68,3 +68,16 @@ def test_no_scratch_memory_in_stream32_kernels(assembly):
         assert int(meta["private_segment_fixed_size"]) == 0 and int(meta["vgpr_spill_count"]) == 0, (m.group(1), meta)
         found += 1
     assert found >= 40
+
+
+def test_no_scratch_memory_in_the_large_m_kernels_the_dispatch_picks(assembly):
+    """The eight-wave 256x256 tile uses nearly all of its registers: a few more and it spills (a
+    three-fold slowdown was measured).  Every paired-fragment instantiation and the tile-pair
+    kernel must report a zero private segment."""
+    text = "\n".join(assembly)
+    found = 0
+    for m in re.finditer(r"\.name:\s+(_ZN10marian_hip(?:18gemm_mfma32_kernelILi\d+ELi\d+ELi\dELi\dELi\dELb1E|16gemm_pair_kernel)\w+)\n(.*?)\.wavefront_size", text, re.S):
+        meta = dict(re.findall(r"\.(vgpr_spill_count|private_segment_fixed_size):\s+(\d+)", m.group(2)))
+        assert int(meta["private_segment_fixed_size"]) == 0 and int(meta["vgpr_spill_count"]) == 0, (m.group(1), meta)
+        found += 1
+    assert found >= 14

@@ -161,6 +161,16 @@ def test_multiply_mid_size_dispatch(integer, orc, synth, M, K, N):
     run_case(integer, orc, synth, 470 + M + N, M, K, N, 0, bias_on=True, relu=(M % 128 == 0), scale=1.5)
 
 
+@pytest.mark.parametrize("kernel", [0, 301, 302, 303, 307, 308, 309, 311, 312, 313, 330, 350])
+@pytest.mark.parametrize("M,K,N", [(512, 192, 512), (1024, 1088, 1024), (640, 448, 264), (2048, 64, 2048),
+                                   (1300, 2112, 776)])
+def test_multiply_half_last_k_block(integer, orc, synth, M, K, N, kernel):
+    """K a multiple of 64 but not of 128 at encoder sizes: the large-M kernels take a last block of
+    64 columns (one, two and many blocks; 350 keeps the 16x16x64 tile kernel for comparison)."""
+    say("multiply half last block", M, K, N, "kernel", kernel)
+    run_case(integer, orc, synth, 480 + M + N, M, K, N, kernel, bias_on=True, relu=(K % 256 == 64), scale=0.75)
+
+
 @pytest.mark.parametrize("kernel", [330, 331])
 @pytest.mark.parametrize("M,K,N,bias_on,relu", [(256, 1024, 256, True, True), (512, 1024, 512, False, False),
                                                 (256, 1152, 256, True, False), (256, 1280, 512, False, True),
