@@ -433,6 +433,13 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * kWave) void gemm_mfma32_kernel(
       bias_v[b] = 0.0f;
       if(has_bias && nvalid[b] && !args.dump) bias_v[b] = args.bias[args.idx ? args.idx[n] : (uint32_t)n];
     }
+    // Use the loaded values once here, ahead of the stores: the compiler then waits for them here.
+    // Otherwise, in the edge form, it re-inserts a wait for all vector memory operations behind the
+    // lane-wise branches, i.e. every store waits for the one before (measured on the edge
+    // workgroups of a 4096 x 4000 output: 41 k instead of 17 k clocks for the write-out).
+#pragma unroll
+    for(int b = 0; b < Cfg::WTN; ++b) asm volatile("" ::"v"(bias_v[b]));
+    asm volatile("" ::"v"(unquant));
 #pragma unroll
     for(int a = 0; a < Cfg::WTM; ++a) {
       const int mbase = m0 + (wm * Cfg::WTM + a) * 32 + 4 * lg;
