@@ -451,6 +451,11 @@ __global__ __launch_bounds__(WN * KW * kWave) void gemm_stream32_kernel(GemmArgs
     const bool has_bias = args.bias != nullptr;
     const int n = n0 + 4 * (lane % 8);
     const int8_t* tiles = lds + (size_t)(wn * KW) * kTileBytes;
+    // Use the bias values once ahead of the stores, so that the compiler waits for their loads here
+    // (they arrived long ago).  Otherwise it waits inside the loop, behind the branches, for all
+    // vector memory operations before each use - and every store then waits for the one before.
+#pragma unroll
+    for(int e = 0; e < 4; ++e) asm volatile("" ::"v"(bias_s[e]));
 #pragma unroll
     for(int it = 0; it < (kPieces + 63) / 64; ++it) {
       const int pc = it * 64 + lane;
