@@ -41,7 +41,8 @@ enum {
   MARIAN_HIP_ERR_ALIGN = 3,     /* pointer alignment violated */
   MARIAN_HIP_ERR_WORKSPACE = 4, /* workspace too small */
   MARIAN_HIP_ERR_HIP = 5,       /* HIP runtime error, see marian_hip_last_hip_error() */
-  MARIAN_HIP_ERR_RANGE = 6      /* size exceeds what the kernels index (2^31 - 1 elements) */
+  MARIAN_HIP_ERR_RANGE = 6,     /* size exceeds what the kernels index (2^31 - 1 elements) */
+  MARIAN_HIP_ERR_STATIC_LIMIT = 7 /* M * K exceeds MARIAN_HIP_STATIC_MAX_ELEMS (static-scratch entry point) */
 };
 
 /* Human-readable text for a status code (host pointer, static storage). */
@@ -129,6 +130,26 @@ int marian_hip_int8_affine_f32_chained(const float* A, int8_t* Aq, const int8_t*
                                        float* out, int64_t M, int64_t K, int64_t N, float scale,
                                        int relu, const float* absmax_in, float* absmax_out,
                                        void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * marian_hip_int8_affine_f32 for callers that cannot allocate and have no workspace to pass: code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no
+ * counterpart in the reference (there the prepareA node's output and every temporary come from the
+ * graph's allocator).  The caller passes inputs and the output only; the quantized activations
+ * (M*K + 4 bytes) and the abs-max partials live in an array of
+ * MARIAN_HIP_STATIC_MAX_ELEMS + 256 + marian_hip_int8_workspace_bytes() bytes that the library
+ * holds on every GPU it runs on until the process ends.  The call makes no hipMalloc / hipFree
+ * and no allocating library call.  `out` is what marian_hip_int8_affine_f32 writes, bit for bit.
+ *   M * K > MARIAN_HIP_STATIC_MAX_ELEMS returns MARIAN_HIP_ERR_STATIC_LIMIT (checked first).
+ *   The device must be current and `stream` must belong to it.  The first call on a device looks
+ *   up the array's address (make that call outside a graph capture).
+ *   All calls on one GPU share the array: calls that overlap on one GPU (two streams, two
+ *   threads) race; serialise them or use marian_hip_int8_affine_f32 with buffers of your own.
+ */
+#define MARIAN_HIP_STATIC_MAX_ELEMS (16 * 1024 * 1024)
+int marian_hip_int8_affine_f32_static(const float* A, const int8_t* Bq, const float* bias,
+                                      const uint32_t* idx, int64_t n_idx, float* out, int64_t M,
+                                      int64_t K, int64_t N, float scale, int relu, void* stream);
 
 /*
  * Shortlisted output layer.  Reference (fp32): index_select(Wt, 0, idx), index_select(b, -1,

@@ -8,7 +8,7 @@ import subprocess
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libmarian_hip_int8.so")
 
-OK, ERR_NULL, ERR_SHAPE, ERR_ALIGN, ERR_WORKSPACE, ERR_HIP, ERR_RANGE = range(7)
+OK, ERR_NULL, ERR_SHAPE, ERR_ALIGN, ERR_WORKSPACE, ERR_HIP, ERR_RANGE, ERR_STATIC_LIMIT = range(8)
 
 # name -> (restype, argtypes); the single place the Python side states the ABI
 _c = ctypes
@@ -26,6 +26,7 @@ SIGNATURES = {
                                         _vp, _sz, _vp]),
     "marian_hip_int8_affine_f32_chained": (_i, [_vp, _vp, _vp, _vp, _vp, _i64, _vp, _i64, _i64, _i64, _f,
                                                 _i, _vp, _vp, _vp, _sz, _vp]),
+    "marian_hip_int8_affine_f32_static": (_i, [_vp, _vp, _vp, _vp, _i64, _vp, _i64, _i64, _i64, _f, _i, _vp]),
     "marian_hip_int8_affine_shortlist": (_i, [_vp, _vp, _vp, _vp, _i64, _vp, _i64, _i64, _i64,
                                               _f, _i, _vp]),
     "marian_hip_int8_multiply_i32": (_i, [_vp, _vp, _vp, _i64, _vp, _i64, _i64, _i64, _vp]),
@@ -45,6 +46,7 @@ SIGNATURES = {
 }
 
 ABSMAX_SLOTS = 2048   # MARIAN_HIP_ABSMAX_SLOTS
+STATIC_MAX_ELEMS = 16 * 1024 * 1024   # MARIAN_HIP_STATIC_MAX_ELEMS
 
 _lib = None
 

@@ -503,13 +503,15 @@ const char* marian_hip_status_string(int status) {
     case MARIAN_HIP_ERR_WORKSPACE: return "workspace too small";
     case MARIAN_HIP_ERR_HIP: return "HIP runtime error";
     case MARIAN_HIP_ERR_RANGE: return "tensor too large for 32-bit element indices";
+    case MARIAN_HIP_ERR_STATIC_LIMIT:
+      return "activations exceed MARIAN_HIP_STATIC_MAX_ELEMS, the capacity of the library's static scratch";
     default: return "unknown status";
   }
 }
 
 int marian_hip_last_hip_error(void) { return g_last_hip_error; }
 
-int marian_hip_int8_abi_version(void) { return 1; }
+int marian_hip_int8_abi_version(void) { return 2; }
 
 size_t marian_hip_int8_workspace_bytes(void) { return kWorkspaceBytes; }
 
@@ -690,6 +692,57 @@ int marian_hip_int8_affine_f32_chained(const float* A, int8_t* Aq, const int8_t*
   return absmax_after(out, M, n_out, absmax_out, reinterpret_cast<hipStream_t>(stream));
 }
 
+
+// ---- the entry point that allocates nothing -------------------------------------------------
+// Device memory the call needs besides its inputs and outputs - the quantized activations with
+// their quantMult tail, and the abs-max partials - lives in one file-scope array per GPU.  In host
+// code the array's name is only a handle: its device address comes from hipGetSymbolAddress, once
+// per device, and only that address is handed to kernels.
+namespace {
+constexpr size_t kStaticMaxElems = MARIAN_HIP_STATIC_MAX_ELEMS;
+constexpr size_t kStaticAqBytes = kStaticMaxElems + 256;   // payload, tail, padding to 256
+constexpr size_t kStaticBytes = kStaticAqBytes + kWorkspaceBytes;
+}  // namespace
+static __device__ __align__(256) unsigned char scratch[kStaticBytes];
+namespace {
+constexpr int kMaxDevices = 64;
+std::atomic<unsigned char*> g_scratch_ptr[kMaxDevices];
+
+// Address of the current device's copy of `scratch` (looked up on the first call per device).
+int static_scratch(unsigned char** out) {
+  int dev = 0;
+  MH_HIP(hipGetDevice(&dev));
+  if(dev < 0 || dev >= kMaxDevices) return MARIAN_HIP_ERR_RANGE;
+  unsigned char* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if(!p) {
+    void* sym = nullptr;
+    MH_HIP(hipGetSymbolAddress(&sym, HIP_SYMBOL(scratch)));
+    if(!sym) return MARIAN_HIP_ERR_NULL;
+    p = static_cast<unsigned char*>(sym);
+    g_scratch_ptr[dev].store(p, std::memory_order_release);   // (every thread finds the same address)
+  }
+  *out = p;
+  return MARIAN_HIP_OK;
+}
+}  // namespace
+
+int marian_hip_int8_affine_f32_static(const float* A, const int8_t* Bq, const float* bias,
+                                      const uint32_t* idx, int64_t n_idx, float* out, int64_t M,
+                                      int64_t K, int64_t N, float scale, int relu, void* stream) {
+  // sizes first, so that an oversized call is refused before anything touches the device
+  if(M < 0 || K <= 0 || N < 0 || (K % 64) != 0 || (N % 8) != 0) return MARIAN_HIP_ERR_SHAPE;
+  if(M > 0 && (uint64_t)M * (uint64_t)K > (uint64_t)kStaticMaxElems) return MARIAN_HIP_ERR_STATIC_LIMIT;
+  if(M == 0) return MARIAN_HIP_OK;
+  unsigned char* base = nullptr;
+  int st = static_scratch(&base);
+  if(st != MARIAN_HIP_OK) return st;
+  int8_t* Aq = reinterpret_cast<int8_t*>(base);
+  void* workspace = base + kStaticAqBytes;
+  // every byte the kernels read from the array was written earlier in the same call (the
+  // activations by the quantizer, the partials by the abs-max pass): nothing has to start at zero
+  return affine_f32_impl(A, Aq, Bq, bias, idx, n_idx, out, M, K, N, scale, relu, nullptr, nullptr,
+                         workspace, kWorkspaceBytes, stream);
+}
 
 int marian_hip_int8_affine_shortlist(const int8_t* Aq, const int8_t* Bq, const float* bias,
                                      const uint32_t* idx, int64_t n_idx, float* out, int64_t M,

@@ -44,10 +44,10 @@ def test_library_exports_every_declared_symbol():
 def test_status_strings_and_version():
     L = load("_lib")
     lib = L.lib()
-    assert lib.marian_hip_int8_abi_version() == 1
+    assert lib.marian_hip_int8_abi_version() == 2
     assert lib.marian_hip_int8_workspace_bytes() >= 4096
-    seen = {lib.marian_hip_status_string(i) for i in range(7)}
-    assert len(seen) == 7 and lib.marian_hip_status_string(0) == b"ok"
+    seen = {lib.marian_hip_status_string(i) for i in range(8)}
+    assert len(seen) == 8 and lib.marian_hip_status_string(0) == b"ok"
 
 
 def test_argument_validation_returns_codes_not_aborts():
