@@ -172,13 +172,6 @@ int marian_hip_int8_multiply_i32(const int8_t* Aq, const int8_t* Bq, const uint3
                                  int64_t n_idx, int32_t* acc, int64_t M, int64_t K, int64_t N,
                                  void* stream);
 
-/*
- * Kernel selection override for measurements: 0 = automatic (default), other values pin one
- * kernel family for subsequent affine/multiply calls of the calling process.  Returns the
- * previous value.  Not needed for normal use.
- */
-int marian_hip_int8_set_kernel(int which);
-
 #ifdef __cplusplus
 }
 #endif

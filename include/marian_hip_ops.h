@@ -120,7 +120,9 @@ int marian_hip_nbest(const float* scores, int64_t dimBatch, int64_t rowLen, int6
  *   candidates of the parts, and one counter per batch entry by which the workgroup that finishes an
  *   entry last knows that it is to draw the final list.  The counters are zero between calls:
  *   marian_hip_nbest_beams_workspace_init clears a freshly allocated workspace once (a kernel, so it
- *   may be captured in a graph); calls that share a workspace must not overlap.
+ *   may be captured in a graph).  One workspace serves one stream: calls that share a workspace must
+ *   not overlap (two streams, or two threads, need a workspace each), and a workspace whose address a
+ *   recorded graph holds must stay allocated as long as that graph is replayed.
  */
 size_t marian_hip_nbest_beams_workspace_bytes(int64_t beam, int64_t dimBatch, int64_t vocab, int64_t N);
 int marian_hip_nbest_beams_workspace_init(void* workspace, size_t workspace_bytes, void* stream);

@@ -10,13 +10,18 @@ What differs from the reference loader (:88-114): a `Type::intgemm8` item is kep
 int8 W^T row-major [N, K] followed by the fp32 quantMult at byte K*N - because that is the layout the
 GPU kernels consume; the reference re-tiles it for the CPU it runs on (prepareAndTransposeB,
 src/tensors/cpu/integer_common.h:189-216).  Items whose type is one of the CPU-tiled variants
-(intgemm8ssse3/avx2/avx512/avx512vnni) cannot be used on a GPU and are refused.
+(intgemm8ssse3/avx2/avx512/avx512vnni) cannot be used on a GPU and are refused.  So are the 16-bit
+intgemm types: their arithmetic (int16 operands, quantMult fixed at 1024,
+src/tensors/cpu/integer_common.h:174-175) exists for CPUs without 8-bit dot products and has no
+matrix-core form on gfx950; this backend implements the 8-bit path only and says so with the text
+of the reference's own dispatch (src/tensors/cpu/intgemm_interface.h:126).  A type id outside
+Marian's enum is reported with the item's name.
 """
 import struct
 
 import numpy as np
 
-from .types import Type, elements, isHardwareSpecific, isIntgemm, requiredBytes
+from .types import Type, elements, isHardwareSpecific, isIntgemm, isPacked, requiredBytes, sizeOf
 
 BINARY_FILE_VERSION = 1
 _HEADER = struct.Struct("<QQQQ")
@@ -110,7 +115,18 @@ def load_items(path):
     pos += 8 + offset
     items = []
     for h, name, shape in zip(headers, names, shapes):
-        type_ = Type(h[1])
+        try:
+            type_ = Type(h[1])
+        except ValueError:
+            raise ValueError("Item {} has the unsupported item type 0x{:x} (this loader knows: {})".format(
+                name, h[1], ", ".join(t.name for t in Type))) from None
+        if isIntgemm(type_) and sizeOf(type_) != 1:
+            raise ValueError("Item {}: Unsupported type {} for Intgemm type?? (the HIP backend implements "
+                             "intgemm8 only; convert the model with marian-conv --gemm-type intgemm8)".format(
+                                 name, type_.name))
+        if isPacked(type_):
+            raise ValueError("Item {} has the FBGEMM-packed type {}: a CPU cache layout that a GPU backend "
+                             "cannot consume (reference src/tensors/cpu/fbgemm/packed_gemm.h)".format(name, type_.name))
         if isHardwareSpecific(type_):
             raise ValueError(
                 "Item {} has the CPU-tiled type {}; a GPU backend needs the hardware-agnostic "

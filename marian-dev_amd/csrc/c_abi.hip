@@ -9,11 +9,15 @@
 #include "abi_common.h"
 #include "gemm_mfma32_kernel.h"
 #include "gemm_pair_kernel.h"
-#include "gemm_persistent_kernel.h"
 #include "gemm_stream32_kernel.h"
 #include "gemm_stream_kernel.h"
-#include "gemm_tile_kernel.h"
 #include "quantize_kernels.h"
+#ifdef MARIAN_HIP_TUNING
+// kernel families that only measurements select, and the switches that select them
+#include "../../include/marian_hip_int8_tuning.h"
+#include "gemm_persistent_kernel.h"
+#include "gemm_tile_kernel.h"
+#endif
 
 using namespace marian_hip;
 
@@ -30,8 +34,15 @@ int marian_hip::record_hip_error(int e) {
 
 namespace {
 
+// The shipped library has no switches: kernel_override() is the constant 0 there and the
+// measurement ids named in the comments below exist in the tuning build only.
+#ifdef MARIAN_HIP_TUNING
 std::atomic<int> g_kernel_override{0};
 std::atomic<long long*> g_prof{nullptr};
+inline int kernel_override() { return g_kernel_override.load(std::memory_order_relaxed); }
+#else
+constexpr int kernel_override() { return 0; }
+#endif
 
 int hip_fail(hipError_t e) { return marian_hip::record_hip_error((int)e); }
 
@@ -45,11 +56,27 @@ inline bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_
 
 constexpr int64_t kMaxElems = 2147483647LL;
 
+constexpr int kMaxDevices = 64;
+
+// The current device, as an index into the per-device caches below.
+inline int current_device(int* dev) {
+  MH_HIP(hipGetDevice(dev));
+  if(*dev < 0 || *dev >= kMaxDevices) return MARIAN_HIP_ERR_RANGE;
+  return MARIAN_HIP_OK;
+}
+
+// Raises a kernel's dynamic LDS limit, once per kernel and device (`done`: one bit per device).
 template <typename KernelT>
-int allow_lds(KernelT kernel, int bytes) {
-  if(bytes > 48 * 1024)
-    MH_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                               hipFuncAttributeMaxDynamicSharedMemorySize, bytes));
+int allow_lds(KernelT kernel, int bytes, std::atomic<uint64_t>& done) {
+  if(bytes <= 48 * 1024) return MARIAN_HIP_OK;
+  int dev = 0;
+  int st = current_device(&dev);
+  if(st != MARIAN_HIP_OK) return st;
+  const uint64_t bit = 1ull << dev;
+  if(done.load(std::memory_order_acquire) & bit) return MARIAN_HIP_OK;
+  MH_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                             hipFuncAttributeMaxDynamicSharedMemorySize, bytes));
+  done.fetch_or(bit, std::memory_order_release);
   return MARIAN_HIP_OK;
 }
 
@@ -57,7 +84,8 @@ template <int MT, int NT, int WN, int KW, int PF>
 int launch_stream(const GemmArgs& a, hipStream_t st) {
   using Cfg = StreamCfg<MT, NT, WN, KW, PF>;
   auto kernel = gemm_stream_kernel<MT, NT, WN, KW, PF>;
-  static const int lds_status = allow_lds(kernel, Cfg::kLdsBytes);
+  static std::atomic<uint64_t> lds_done{0};
+  const int lds_status = allow_lds(kernel, Cfg::kLdsBytes, lds_done);
   if(lds_status != MARIAN_HIP_OK) return lds_status;
   int blocks = (a.n_out + Cfg::kColsPerBlock - 1) / Cfg::kColsPerBlock;
   hipLaunchKernelGGL(kernel, dim3(blocks), dim3(Cfg::kThreads), Cfg::kLdsBytes, st, a);
@@ -65,11 +93,13 @@ int launch_stream(const GemmArgs& a, hipStream_t st) {
   return MARIAN_HIP_OK;
 }
 
+#ifdef MARIAN_HIP_TUNING
 template <int WNT, int WMT>
 int launch_tile(const GemmArgs& a, hipStream_t st) {
   using Cfg = TileCfg<WNT, WMT>;
   auto kernel = gemm_tile_kernel<WNT, WMT>;
-  static const int lds_status = allow_lds(kernel, Cfg::kLdsBytes);
+  static std::atomic<uint64_t> lds_done{0};
+  const int lds_status = allow_lds(kernel, Cfg::kLdsBytes, lds_done);
   if(lds_status != MARIAN_HIP_OK) return lds_status;
   int tiles_n = (a.n_out + Cfg::BN - 1) / Cfg::BN;
   int tiles_m = (a.M + Cfg::BM - 1) / Cfg::BM;
@@ -78,6 +108,7 @@ int launch_tile(const GemmArgs& a, hipStream_t st) {
   MH_HIP(hipGetLastError());
   return MARIAN_HIP_OK;
 }
+#endif
 
 template <int BM, int BN, int WM, int WN, int NSTAGE, bool PAIRED = true, bool NT = false>
 int launch_big(const GemmArgs& a, hipStream_t st) {
@@ -87,13 +118,19 @@ int launch_big(const GemmArgs& a, hipStream_t st) {
   const int tiles_n = (a.n_out + BN - 1) / BN;
   const int tiles_m = (a.M + BM - 1) / BM;
   if(a.K % Cfg::BK != 0) {
-    if(!PAIRED || a.K % 64 != 0 || g_kernel_override.load(std::memory_order_relaxed) % 1000 == 350)
+#ifdef MARIAN_HIP_TUNING
+    if(!PAIRED || a.K % 64 != 0 || kernel_override() % 1000 == 350)
       return launch_tile<4, 4>(a, st);
+#else
+    static_assert(PAIRED, "the shipped dispatch uses the paired-fragment form only");
+    if(a.K % 64 != 0) return MARIAN_HIP_ERR_SHAPE;   // (refused by the argument checks already)
+#endif
     if constexpr(!Cfg::kHalfTailOk || !PAIRED) {
       return launch_big<128, 128, 2, 4, 2, true, NT>(a, st);
     } else {
       auto half = gemm_mfma32_kernel<BM, BN, WM, WN, NSTAGE, true, NT, true>;
-      static const int half_lds_status = allow_lds(half, Cfg::kLdsBytes);
+      static std::atomic<uint64_t> half_lds_done{0};
+      const int half_lds_status = allow_lds(half, Cfg::kLdsBytes, half_lds_done);
       if(half_lds_status != MARIAN_HIP_OK) return half_lds_status;
       hipLaunchKernelGGL(half, dim3(tiles_n * tiles_m), dim3(Cfg::kThreads), Cfg::kLdsBytes, st, a,
                          tiles_n, tiles_m);
@@ -102,7 +139,8 @@ int launch_big(const GemmArgs& a, hipStream_t st) {
     }
   }
   auto kernel = gemm_mfma32_kernel<BM, BN, WM, WN, NSTAGE, PAIRED, NT>;
-  static const int lds_status = allow_lds(kernel, Cfg::kLdsBytes);
+  static std::atomic<uint64_t> lds_done{0};
+  const int lds_status = allow_lds(kernel, Cfg::kLdsBytes, lds_done);
   if(lds_status != MARIAN_HIP_OK) return lds_status;
   hipLaunchKernelGGL(kernel, dim3(tiles_n * tiles_m), dim3(Cfg::kThreads), Cfg::kLdsBytes, st, a,
                      tiles_n, tiles_m);
@@ -121,7 +159,8 @@ template <bool NT>
 int launch_pair(const GemmArgs& a, hipStream_t st) {
   if(!pair_kernel_fits(a)) return launch_big<256, 256, 2, 4, 2>(a, st);
   auto kernel = gemm_pair_kernel<NT>;
-  static const int lds_status = allow_lds(kernel, PairCfg::kLdsBytes);
+  static std::atomic<uint64_t> lds_done{0};
+  const int lds_status = allow_lds(kernel, PairCfg::kLdsBytes, lds_done);
   if(lds_status != MARIAN_HIP_OK) return lds_status;
   int pairs_n = a.n_out / (2 * PairCfg::BN);
   int tiles_m = a.M / PairCfg::BM;
@@ -141,15 +180,17 @@ inline bool stream32_can_fuse(int64_t M, int64_t K) {
   return M <= 128 && M * K <= kFusedMaxElems && stream32_fused_lds_bytes(mt32, (int)K) <= 64 * 1024;
 }
 
+// Compute units of the current device (looked up once per device; 256 if the query fails).
 int compute_units() {
-  static const int cus = [] {
-    int dev = 0, n = 0;
-    if(hipGetDevice(&dev) != hipSuccess) return 256;
-    if(hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
-      return 256;
-    return n;
-  }();
-  return cus;
+  static std::atomic<int> cus[kMaxDevices];
+  int dev = 0;
+  if(hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 256;
+  int n = cus[dev].load(std::memory_order_relaxed);
+  if(n > 0) return n;
+  if(hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+    n = 256;
+  cus[dev].store(n, std::memory_order_relaxed);
+  return n;
 }
 
 struct FusedSrc {   // what the fused modes read and write besides GemmArgs
@@ -168,7 +209,8 @@ int launch_stream32(const GemmArgs& a, const FusedSrc& f, hipStream_t st) {
   using Cfg = Stream32Cfg<MT32, WN, KW, PW>;
   auto kernel = gemm_stream32_kernel<MT32, WN, KW, PW, MODE, NG, ROWS>;
   constexpr int kMaxLds = 64 * 1024 > Cfg::kLdsBytes ? 64 * 1024 : Cfg::kLdsBytes;
-  static const int lds_status = allow_lds(kernel, kMaxLds);
+  static std::atomic<uint64_t> lds_done{0};
+  const int lds_status = allow_lds(kernel, kMaxLds, lds_done);
   if(lds_status != MARIAN_HIP_OK) return lds_status;
   // (kFusedAll: all of K, and at least one whole chunk so that the first chunk needs no bounds)
   int lds = Cfg::kStageBytes;
@@ -205,11 +247,11 @@ int launch_stream32_kw(const GemmArgs& a, const FusedSrc& f, hipStream_t st, int
       case 2: return launch_stream32<1, 4, 2, 4, MODE>(a, f, st);
       case 4:
         if(half_rows) return launch_stream32<1, 2, 4, 4, MODE, 16>(a, f, st);
-        if(need > 4 && g_kernel_override.load(std::memory_order_relaxed) % 1000 != 690)
+        if(need > 4 && kernel_override() % 1000 != 690)
           return launch_stream32<1, 2, 4, 8, MODE>(a, f, st);   // long rows: half as many chunks (measurement id 690 keeps the shorter ones)
         return launch_stream32<1, 2, 4, 4, MODE>(a, f, st);
       default:
-        if(need > 4 && half_rows && g_kernel_override.load(std::memory_order_relaxed) % 1000 != 670)
+        if(need > 4 && half_rows && kernel_override() % 1000 != 670)
           return launch_stream32<1, 1, 8, 8, MODE, 16>(a, f, st);   // long rows: half as many chunks (measurement id 670 keeps the shorter ones)
         if(need > 2) {
           if(half_rows) return launch_stream32<1, 1, 8, 4, MODE, 16>(a, f, st);
@@ -260,7 +302,7 @@ TiledPlan plan_tiled(int M, int K, int n_out, int kw_override) {
   while(kw > 1 && (long long)((tiles * kw + 7) / 8) * m_tiles > compute_units()) kw >>= 1;
   if(kw_override) kw = kw_override;
   while(kw > 1 && K / 32 < kw) kw >>= 1;
-  const int ov = g_kernel_override.load(std::memory_order_relaxed) % 1000;   // 640 / 641: force 32 / 16 rows
+  const int ov = kernel_override() % 1000;   // 640 / 641: force 32 / 16 rows
   const long long blocks32 = (long long)((tiles * kw + 7) / 8) * m_tiles;
   const bool half_rows = kw >= 4 && ov != 640 && (ov == 641 || (M > 16 && 2 * blocks32 <= compute_units()));
   return TiledPlan{kw, half_rows};
@@ -298,7 +340,7 @@ int launch_stream32_auto(const GemmArgs& a, const FusedSrc& f, hipStream_t st, i
       // and a wave that has its SIMD to itself issues twice as fast.  (K up to 1024: one chunk.)
       // (measurement ids 660 / 661 force eight / four waves)
       {
-        const int ov = g_kernel_override.load(std::memory_order_relaxed) % 1000;
+        const int ov = kernel_override() % 1000;
         const int S = a.K / 32;
         const bool four = !kw_override && ov != 660 && ov != 650 && ov != 651 && S >= 8 && S <= 32 &&
                           (long long)a.M * a.K <= 2 * 16 * 256 && a.M <= 32 &&
@@ -313,7 +355,7 @@ int launch_stream32_auto(const GemmArgs& a, const FusedSrc& f, hipStream_t st, i
       // Few weight tiles: 16-row workgroups (all of them take the abs-max over the whole input,
       // each quantizes and multiplies its own rows), if they fit one per CU with the widest K
       // split.  (measurement ids 650 / 651 force full-height / 16-row workgroups)
-      const int ov = g_kernel_override.load(std::memory_order_relaxed) % 1000;
+      const int ov = kernel_override() % 1000;
       const bool rows16 = a.K / 32 >= 8 && !kw_override && ov != 650 &&
                           (ov == 651 || (a.M > 16 && (long long)tiles * ((a.M + 15) / 16) <= compute_units()));
       if(rows16) return launch_stream32_kw<1, MODE>(a, f, st, 8, true);
@@ -324,6 +366,7 @@ int launch_stream32_auto(const GemmArgs& a, const FusedSrc& f, hipStream_t st, i
   }
 }
 
+#ifdef MARIAN_HIP_TUNING
 template <int BM, int BN, int WM, int WN, int NSTAGE, bool DIRECT = false>
 int launch_persistent(const GemmArgs& a, hipStream_t st, int per_cu = 1, int stagger = 0) {
   using Cfg = PersistCfg<BM, BN, WM, WN, NSTAGE, DIRECT>;
@@ -332,7 +375,8 @@ int launch_persistent(const GemmArgs& a, hipStream_t st, int per_cu = 1, int sta
     return launch_big<BM, BN, WM, WN, 2>(a, st);
   auto dense = gemm_persistent_kernel<BM, BN, WM, WN, NSTAGE, false, DIRECT>;
   auto gather = gemm_persistent_kernel<BM, BN, WM, WN, NSTAGE, true, DIRECT>;
-  static const int lds_status = allow_lds(dense, Cfg::kLdsBytes) | allow_lds(gather, Cfg::kLdsBytes);
+  static std::atomic<uint64_t> dense_done{0}, gather_done{0};
+  const int lds_status = allow_lds(dense, Cfg::kLdsBytes, dense_done) | allow_lds(gather, Cfg::kLdsBytes, gather_done);
   if(lds_status != MARIAN_HIP_OK) return lds_status;
   int tiles_n = (a.n_out + BN - 1) / BN;
   int tiles_m = (a.M + BM - 1) / BM;
@@ -345,6 +389,7 @@ int launch_persistent(const GemmArgs& a, hipStream_t st, int per_cu = 1, int sta
   MH_HIP(hipGetLastError());
   return MARIAN_HIP_OK;
 }
+#endif
 
 // wide: many weight rows, every wave streams its own rows over the whole K
 // narrow: few weight rows, the four waves split K and reduce
@@ -366,7 +411,8 @@ int launch_stream_auto(const GemmArgs& a, hipStream_t st, int force_wide) {
 }
 
 int launch_gemm(const GemmArgs& a, hipStream_t st) {
-  const int which = g_kernel_override.load(std::memory_order_relaxed) % 1000;
+#ifdef MARIAN_HIP_TUNING
+  const int which = kernel_override() % 1000;
   switch(which) {
     case 101: if(a.M <= 128) return launch_stream_auto(a, st, 1); break;
     case 102: if(a.M <= 128) return launch_stream_auto(a, st, 2); break;
@@ -413,6 +459,7 @@ int launch_gemm(const GemmArgs& a, hipStream_t st) {
     case 404: return launch_persistent<256, 128, 2, 2, 2>(a, st);
     default: break;
   }
+#endif
   // Small M (decode): the weights are streamed once, the activations sit in LDS.
   //  - up to 8 rows (16 for narrow outputs): the 16x16x64 MFMA kernel, one 16-row tile
   //  - otherwise the 32x32x32 MFMA kernel, which also tiles M (shortlisted output layer, M = 256)
@@ -430,7 +477,7 @@ int launch_gemm(const GemmArgs& a, hipStream_t st) {
   const bool stream_out = (long long)a.M * a.n_out * 4 <= (32ll << 20) && !a.dump;
   if(tiles256 >= 192) {
     // short K: the fp32 output is most of the bytes; write one tile out while the next is multiplied
-    if(pair_kernel_fits(a) && a.K <= 1536 && g_kernel_override.load(std::memory_order_relaxed) % 1000 != 332)
+    if(pair_kernel_fits(a) && a.K <= 1536 && kernel_override() % 1000 != 332)
       return launch_pair<true>(a, st);
     if(stream_out) return launch_big<256, 256, 2, 4, 2, true, true>(a, st);
     return launch_big<256, 256, 2, 4, 2>(a, st);
@@ -444,7 +491,7 @@ int launch_gemm(const GemmArgs& a, hipStream_t st) {
   }
   // so few 128x128 tiles that half the CUs would idle: 128x64 tiles (measured -20 % to -25 % for
   // M = 512 .. 1024, K = 4096, N = 1024; measurement id 340 keeps the square tiles)
-  if(2 * tiles128 <= compute_units() && g_kernel_override.load(std::memory_order_relaxed) % 1000 != 340) {
+  if(2 * tiles128 <= compute_units() && kernel_override() % 1000 != 340) {
     if(stream_out) return launch_big<128, 64, 2, 2, 3, true, true>(a, st);
     return launch_big<128, 64, 2, 2, 3>(a, st);
   }
@@ -476,8 +523,10 @@ int run_gemm(const int8_t* Aq, const int8_t* Bq, const float* bias, const uint32
   a.Aq = Aq; a.Bq = Bq; a.bias = bias; a.idx = idx; a.out = out;
   a.M = (int)M; a.K = (int)K; a.N = (int)N; a.n_out = (int)n_out;
   a.scale = scale; a.relu = relu ? 1 : 0; a.dump = dump;
-  a.dbg = g_kernel_override.load(std::memory_order_relaxed) / 1000;
+#ifdef MARIAN_HIP_TUNING
+  a.dbg = kernel_override() / 1000;
   a.prof = g_prof.load(std::memory_order_relaxed);
+#endif
   a.absmax_out = absmax_out;
   return launch_gemm(a, reinterpret_cast<hipStream_t>(stream));
 }
@@ -515,9 +564,11 @@ int marian_hip_int8_abi_version(void) { return 2; }
 
 size_t marian_hip_int8_workspace_bytes(void) { return kWorkspaceBytes; }
 
+#ifdef MARIAN_HIP_TUNING
 int marian_hip_int8_set_kernel(int which) { return g_kernel_override.exchange(which); }
 
 void marian_hip_int8_debug_profile(long long* p) { g_prof.store(p); }
+#endif
 
 int marian_hip_int8_prepare_a(const float* A, int8_t* Aq, int64_t M, int64_t K, void* workspace,
                               size_t workspace_bytes, void* stream) {
@@ -600,13 +651,15 @@ static int affine_f32_impl(const float* A, int8_t* Aq, const int8_t* Bq, const f
   // Measurement ids: 600 = separate prepareA and GEMM launches; 611/612/614/618 = one fused
   // kernel with that K split; 620 = abs-max launch + tiled fused kernel, 621/622/624/628 with
   // that K split.
-  const int which = g_kernel_override.load(std::memory_order_relaxed) % 1000;
+  const int which = kernel_override() % 1000;
   hipStream_t hst = reinterpret_cast<hipStream_t>(stream);
   GemmArgs a;
   a.Aq = Aq; a.Bq = Bq; a.bias = bias; a.idx = idx; a.out = out;
   a.M = (int)M; a.K = (int)K; a.N = (int)N; a.n_out = (int)n_out;
-  a.scale = scale; a.relu = relu ? 1 : 0; a.dump = 0; a.dbg = 0;
+  a.scale = scale; a.relu = relu ? 1 : 0; a.dump = 0;
+#ifdef MARIAN_HIP_TUNING
   a.prof = g_prof.load(std::memory_order_relaxed);
+#endif
   a.absmax_out = absmax_out;
   FusedSrc f;
   f.A = A; f.aq_out = Aq;
@@ -705,14 +758,13 @@ constexpr size_t kStaticBytes = kStaticAqBytes + kWorkspaceBytes;
 }  // namespace
 static __device__ __align__(256) unsigned char scratch[kStaticBytes];
 namespace {
-constexpr int kMaxDevices = 64;
 std::atomic<unsigned char*> g_scratch_ptr[kMaxDevices];
 
 // Address of the current device's copy of `scratch` (looked up on the first call per device).
-int static_scratch(unsigned char** out) {
+static int static_scratch(unsigned char** out) {
   int dev = 0;
-  MH_HIP(hipGetDevice(&dev));
-  if(dev < 0 || dev >= kMaxDevices) return MARIAN_HIP_ERR_RANGE;
+  const int dst = current_device(&dev);
+  if(dst != MARIAN_HIP_OK) return dst;
   unsigned char* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
   if(!p) {
     void* sym = nullptr;

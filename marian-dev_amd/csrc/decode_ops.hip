@@ -10,9 +10,12 @@
 
 #include <hip/hip_runtime.h>
 
+#include <atomic>
+
 #include "../../include/marian_hip_int8.h"
 #include "abi_common.h"
 #include "int8_common.h"
+#include "nbest_plan.h"
 
 using namespace marian_hip;
 
@@ -394,13 +397,16 @@ __global__ __launch_bounds__(256) void attention_kernel(const float* __restrict_
                                                         float* __restrict__ out, long long rows_total,
                                                         long long batchKV, int m, int len, int dk,
                                                         float scale, float* __restrict__ absmax_out) {
-  extern __shared__ float att_lds[];
+  extern __shared__ __attribute__((aligned(16))) float att_lds[];
   const long long wr = (long long)blockIdx.x * 4 + threadIdx.x / 64;
   if(absmax_out && blockIdx.x == 0)   // slots past the last query row
     for(int sl = (int)rows_total + threadIdx.x; sl < kAbsmaxSlots; sl += 256) absmax_out[sl] = 0.0f;
   if(wr >= rows_total) return;   // whole waves leave; no workgroup barrier is used
-  float* sc = att_lds + (threadIdx.x / 64) * (len + 256);   // scores, then 4 x 64 partial outputs
-  float* part = sc + len;
+  // per wave: the scores (rounded up to whole 16-byte units, so that the partial outputs behind
+  // them are 16-byte aligned for the v4f stores), then 4 x 64 partial outputs
+  const int len4 = (len + 3) & ~3;
+  float* sc = att_lds + (threadIdx.x / 64) * (len4 + 256);
+  float* part = sc + len4;
   const int lane = threadIdx.x % 64;
   const long long i = wr / m;
   const float* q = Q + (size_t)wr * dk;
@@ -889,10 +895,25 @@ __global__ __launch_bounds__(1024) void nbest_part_kernel(const float* __restric
     nbest_of_row<KEEP>(scores + ((size_t)k * dimBatch + b) * vocab + v0, len, N, sh,
                        [&](int r, float v, unsigned i) { publish(r, v, base + i); });
   }
+  // Hand-over without fences.  What it relies on (gfx942/gfx950 memory model as the AMDGPU backend
+  // documents it): an agent-scope store or atomic bypasses the XCD-local L2 and is performed at the
+  // memory side, where all XCDs see it; a wave's vmcnt reaches zero only once each of its stores
+  // has been acknowledged from there; an agent-scope load reads from there too.  So: candidates
+  // stored (agent scope) -> vmcnt(0) in every wave -> workgroup barrier -> counter incremented; the
+  // workgroup that reads parts - 1 from the counter then loads (agent scope) candidates that are all
+  // in memory already.  Building with -DMARIAN_HIP_NBEST_FENCED makes the counter update an
+  // acquire-release operation instead (the compiler then adds the cache write-back / invalidate
+  // the language-level memory model asks for; ~8 us slower): if results ever differ between the
+  // two builds, the hand-over is at fault and not the selection.
+#ifdef MARIAN_HIP_NBEST_FENCED
+  constexpr int kCounterOrder = __ATOMIC_ACQ_REL;
+#else
+  constexpr int kCounterOrder = __ATOMIC_RELAXED;
+#endif
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // every wave's stores have reached memory ...
   __syncthreads();
   if(threadIdx.x == 0)                               // ... before the count goes up
-    is_last = __hip_atomic_fetch_add(&counters[b * kNbestCounterStride], 1u, __ATOMIC_RELAXED,
+    is_last = __hip_atomic_fetch_add(&counters[b * kNbestCounterStride], 1u, kCounterOrder,
                                      __HIP_MEMORY_SCOPE_AGENT) == (unsigned)(parts - 1);
   __syncthreads();
   if(!is_last) return;
@@ -911,30 +932,14 @@ __global__ __launch_bounds__(1024) void nbest_part_kernel(const float* __restric
     };
     if(total <= 64) nbest_small_draw(sh.cand_val, sh.cand_idx, total, N, result);
     else nbest_wave_draw(sh.cand_val, sh.cand_idx, total, N, result);
-    if(threadIdx.x == 0) counters[b * kNbestCounterStride] = 0;   // for the next call
+    if(threadIdx.x == 0)   // for the next call (every part of this entry has arrived: nobody else touches it)
+      __hip_atomic_store(&counters[b * kNbestCounterStride], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
 }
 
 __global__ __launch_bounds__(256) void zero_words_kernel(unsigned* __restrict__ p, long long n) {
   for(long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long long)gridDim.x * blockDim.x)
     p[i] = 0u;
-}
-
-// Slices per beam segment: enough workgroups for every CU (256 and up) as long as a slice keeps
-// 4096 scores, a multiple of four so that slices start 16-byte aligned when the rows do.
-struct NbestPlan {
-  int perSeg;
-  long long sliceLen;
-  int parts;
-};
-inline NbestPlan nbest_plan(int64_t beam, int64_t dimBatch, int64_t vocab, int64_t N) {
-  long long perSeg = (256 + beam * dimBatch - 1) / (beam * dimBatch);
-  const long long most = vocab / 4096 > 0 ? vocab / 4096 : 1;
-  if(perSeg > most) perSeg = most;
-  while(perSeg > 1 && beam * perSeg * N > 1024) --perSeg;   // the merge draws from at most 1024
-  long long sliceLen = ((vocab + perSeg - 1) / perSeg + 3) / 4 * 4;
-  perSeg = (vocab + sliceLen - 1) / sliceLen;
-  return NbestPlan{(int)perSeg, sliceLen, (int)(beam * perSeg)};
 }
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) % 16) == 0; }
@@ -1092,13 +1097,18 @@ int marian_hip_attention(const float* q, float* k, float* v, const float* mask, 
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   if(!mask) { n_masks = 1; rows_per_mask = 1; }
   const long long rows_total = batchQ * m;
-  const size_t lds = (size_t)4 * (size_t)(len + 256) * sizeof(float);   // per wave: scores + partial outputs
-  static const int lds_status = [] {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(attention_kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, 72 * 1024);
-    return e == hipSuccess ? 0 : (int)e;
-  }();
-  if(lds_status != 0) return record_hip_error(lds_status);
+  const size_t lds = (size_t)4 * (size_t)(((len + 3) & ~(int64_t)3) + 256) * sizeof(float);   // per wave: scores (whole 16-byte units) + partial outputs
+  {   // the kernel's dynamic LDS limit, raised once per device (one bit per device)
+    static std::atomic<uint64_t> lds_done{0};
+    int dev = 0;
+    MH_HIP(hipGetDevice(&dev));
+    if(dev < 0 || dev >= 64) return MARIAN_HIP_ERR_RANGE;
+    if(!(lds_done.load(std::memory_order_acquire) & (1ull << dev))) {
+      MH_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(attention_kernel),
+                                 hipFuncAttributeMaxDynamicSharedMemorySize, 72 * 1024));
+      lds_done.fetch_or(1ull << dev, std::memory_order_release);
+    }
+  }
   hipLaunchKernelGGL(attention_kernel, dim3((unsigned)((rows_total + 3) / 4)), dim3(256), lds, st, q, k, v,
                      k_new, v_new, mask, (long long)n_masks, (long long)rows_per_mask, out, rows_total,
                      (long long)batchKV, (int)m, (int)len, (int)dk, scale, absmax_out);

@@ -171,8 +171,8 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * kWave) void gemm_mfma32_kernel(
   extern __shared__ __attribute__((aligned(16))) int8_t lds[];
   const unsigned lds_base = (unsigned)(size_t)lds;  // LDS byte address of the ring
 
-  const long long t_start = clock64();
-  const long long w_start = wall_clock64();
+  const long long t_start = MH_CLOCK();
+  const long long w_start = MH_WALL();
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
   const int lane = tid % kWave;
@@ -332,7 +332,7 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * kWave) void gemm_mfma32_kernel(
   else if(KB >= 2) wait_vmcnt<Cfg::kLoads>();
   else wait_vmcnt<0>();
   __builtin_amdgcn_s_barrier();
-  const long long t_prologue = clock64();
+  const long long t_prologue = MH_CLOCK();
   if constexpr(!PAIRED) {
     auto spread = [&]() {   // one LDS read after each MFMA
 #pragma unroll
@@ -360,7 +360,7 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * kWave) void gemm_mfma32_kernel(
         else wait_vmcnt<0>();
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
-        if(kb + NSTAGE < KB && !(args.dbg & 1)) issue(kb + NSTAGE);
+        if(kb + NSTAGE < KB && !(MH_DBG(args, 1))) issue(kb + NSTAGE);
         read_frags((kb + 1) % NSTAGE, 0, 0);
       }
       multiply(1);
@@ -386,11 +386,11 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * kWave) void gemm_mfma32_kernel(
       else wait_vmcnt<0>();
       __builtin_amdgcn_s_barrier();
       __builtin_amdgcn_sched_barrier(0);
-      second_half(steady_c, kb + NSTAGE < KB && !(args.dbg & 1), kb);
+      second_half(steady_c, kb + NSTAGE < KB && !(MH_DBG(args, 1)), kb);
     };
     int kb = 0;
     const int KBsteady = half_tail ? KB - 1 : KB;   // the steady body issues whole blocks only
-    if(!(args.dbg & 1))
+    if(!(MH_DBG(args, 1)))
       for(; kb + NSTAGE < KBsteady; ++kb) one_block(kb, std::true_type());
     for(; kb + 1 < KB; ++kb) one_block(kb, std::false_type());
     if(half_tail) {   // 64 columns: sub-steps 0 and 1 only
@@ -411,7 +411,7 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * kWave) void gemm_mfma32_kernel(
     }
   }
 
-  const long long t_main = clock64();
+  const long long t_main = MH_CLOCK();
   // ---- epilogue: element v of a 32x32 tile is row 8*(v/4) + 4*lg + v%4, column li ----
   float unquant = 0.0f;
   if(!args.dump) {
@@ -422,7 +422,7 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * kWave) void gemm_mfma32_kernel(
   const bool interior = (m0 + BM <= M) && (n0 + BN <= args.n_out);
   const size_t row_bytes = (size_t)args.n_out * 4;
   const bool has_bias = args.bias != nullptr;
-  if(!(args.dbg & 2)) {
+  if(!(MH_DBG(args, 2))) {
     const int nw = n0 + wn * Cfg::WTN * 32 + li;   // this lane's column in the first of the wave's tiles
     float bias_v[Cfg::WTN];
     bool nvalid[Cfg::WTN];
@@ -450,9 +450,9 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * kWave) void gemm_mfma32_kernel(
         store_tiles32_rowwise_any<Cfg::WTN, true, NT>(acc[a], outp, row_bytes, unquant, bias_v, M - mbase, nvalid, args.dump, has_bias, args.relu);
     }
   }
-  if(args.prof && tid == 0) {
-    long long* p = args.prof + (size_t)blockIdx.x * 8;
-    p[0] = t_start; p[1] = t_prologue; p[2] = t_main; p[3] = clock64(); p[6] = w_start; p[7] = wall_clock64();
+  if(MH_PROF(args) && tid == 0) {
+    long long* p = MH_PROF(args) + (size_t)blockIdx.x * 8;
+    p[0] = t_start; p[1] = t_prologue; p[2] = t_main; p[3] = MH_CLOCK(); p[6] = w_start; p[7] = MH_WALL();
   }
 }
 

@@ -73,8 +73,8 @@ __global__ __launch_bounds__(PairCfg::kThreads) void gemm_pair_kernel(GemmArgs a
   extern __shared__ __attribute__((aligned(16))) int8_t lds[];
   const unsigned lds_base = (unsigned)(size_t)lds;
 
-  const long long t_start = clock64();
-  const long long w_start = wall_clock64();
+  const long long t_start = MH_CLOCK();
+  const long long w_start = MH_WALL();
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
   const int lane = tid % kWave;
@@ -135,7 +135,8 @@ __global__ __launch_bounds__(PairCfg::kThreads) void gemm_pair_kernel(GemmArgs a
 
   // ---- dequantization constants and the write-out addresses of the first tile ----
   const bool has_bias = args.bias != nullptr;
-  const float relu_floor = args.relu ? 0.0f : -__builtin_inff();   // max(y, -inf) = y
+  // max(y, NaN) = y for every y, a NaN included; max(NaN, 0) = 0 like the CPU path's y > 0 ? y : 0
+  const float relu_floor = args.relu ? 0.0f : __builtin_nanf("");
   // element e of accumulator tile (a, b): row 32*a + 8*(e/4) + 4*lg + e%4, column 32*b + li
   const unsigned out_voff = ((unsigned)(4 * lg) * (unsigned)args.n_out + (unsigned)li) * 4u;
   const char* const out_base0 = reinterpret_cast<const char*>(args.out) +
@@ -216,7 +217,7 @@ __global__ __launch_bounds__(PairCfg::kThreads) void gemm_pair_kernel(GemmArgs a
     for(int j = 0; j < Cfg::kLoads; ++j) issue_one(s, s, j);
   wait_vmcnt<(NSTAGE - 1) * Cfg::kLoads>();
   __builtin_amdgcn_s_barrier();
-  const long long t_prologue = clock64();
+  const long long t_prologue = MH_CLOCK();
 #pragma unroll
   for(int f = 0; f < 12; ++f) read_one(0, f / 6, f % 6);
   {
@@ -249,7 +250,7 @@ __global__ __launch_bounds__(PairCfg::kThreads) void gemm_pair_kernel(GemmArgs a
   } else {
     block(g, stage, set1, std::true_type(), I()); advance();
   }
-  const long long t_side = clock64();
+  const long long t_side = MH_CLOCK();
   block(g + 1, stage, set1, std::false_type(), std::integral_constant<int, 1>()); advance();
   block(g + 2, stage, set1, std::false_type(), std::integral_constant<int, 2>()); advance();
   block(g + 3, stage, set1, std::false_type(), std::integral_constant<int, 3>()); advance();
@@ -257,7 +258,7 @@ __global__ __launch_bounds__(PairCfg::kThreads) void gemm_pair_kernel(GemmArgs a
   block(g + 5, stage, set1, std::false_type(), std::integral_constant<int, 5>()); advance();
   block(g + 6, stage, set1, std::false_type(), std::integral_constant<int, 6>()); advance();
   block(g + 7, stage, set1, std::false_type(), std::integral_constant<int, 7>());
-  const long long t_main = clock64();
+  const long long t_main = MH_CLOCK();
 
   // ---- the second tile's write-out: the same store form, four values in flight ----
   {
@@ -272,9 +273,9 @@ __global__ __launch_bounds__(PairCfg::kThreads) void gemm_pair_kernel(GemmArgs a
       global_store_f32<NT>(out_base1 + (size_t)r * row_bytes + b * 128, out_voff, y);
     }
   }
-  if(args.prof && tid == 0) {
-    long long* p = args.prof + (size_t)blockIdx.x * 8;
-    p[0] = t_start; p[1] = t_prologue; p[2] = t_main; p[3] = clock64(); p[4] = t_main; p[5] = t_side; p[6] = w_start; p[7] = wall_clock64();
+  if(MH_PROF(args) && tid == 0) {
+    long long* p = MH_PROF(args) + (size_t)blockIdx.x * 8;
+    p[0] = t_start; p[1] = t_prologue; p[2] = t_main; p[3] = MH_CLOCK(); p[4] = t_main; p[5] = t_side; p[6] = w_start; p[7] = MH_WALL();
   }
 }
 

@@ -90,7 +90,7 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * kWave) void gemm_persistent_ker
   extern __shared__ __attribute__((aligned(16))) int8_t lds[];
   const unsigned lds_base = (unsigned)(size_t)lds;  // LDS byte address of the ring
 
-  const long long t_start = clock64();
+  const long long t_start = MH_CLOCK();
   long long t_epi = 0;
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
@@ -215,7 +215,7 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * kWave) void gemm_persistent_ker
     int tn, tm;
     persistent_tile_coords(round, blockIdx.x, grid, tiles_n, tiles_m, tn, tm);
     const int m0 = tm * BM, n0 = tn * BN;
-    last_tile_interior = (m0 + BM <= M) && (n0 + BN <= args.n_out) && !(args.dbg & 2);
+    last_tile_interior = (m0 + BM <= M) && (n0 + BN <= args.n_out) && !(MH_DBG(args, 2));
     if(DIRECT) {
       const bool interior = last_tile_interior;
       const size_t row_bytes = (size_t)args.n_out * 4;
@@ -236,7 +236,7 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * kWave) void gemm_persistent_ker
         for(int a = 0; a < Cfg::WTM; ++a) {
           const int mbase = m0 + (wm * Cfg::WTM + a) * 32 + 4 * lg;
           char* outp = reinterpret_cast<char*>(args.out) + ((size_t)mbase * (size_t)args.n_out + (size_t)n) * 4;
-          if(args.dbg & 2) continue;
+          if(MH_DBG(args, 2)) continue;
           if(interior)
             store_tile32_any<false>(acc[a][b], outp, row_bytes, unquant, bias_v, 32, true, args.dump, has_bias, args.relu);
           else
@@ -280,7 +280,7 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * kWave) void gemm_persistent_ker
           const int r = q * 8 + lane / 8, c = (lane % 8) * 4;
           v4f y = *reinterpret_cast<const v4f*>(epi + r * 32 + c);
           const int m = mrow0 + r, n = ncol0 + c;
-          if(m < M && n < args.n_out && !(args.dbg & 2))
+          if(m < M && n < args.n_out && !(MH_DBG(args, 2)))
             *reinterpret_cast<v4f*>(reinterpret_cast<float*>(args.out) + (size_t)m * (size_t)args.n_out + n) = y;
         }
         wait_lgkmcnt0();   // the buffer is rewritten by the next tile
@@ -302,7 +302,7 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * kWave) void gemm_persistent_ker
   // block 0 has landed once at most the later blocks' loads are outstanding
   wait_vmcnt_dyn((min(total_blocks, NSTAGE) - 1) * Cfg::kLoads);
   __builtin_amdgcn_s_barrier();
-  const long long t_prologue = clock64();
+  const long long t_prologue = MH_CLOCK();
   read_frags(0, 0, 0);
   read_frags(0, 1, 1);
 
@@ -340,7 +340,7 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * kWave) void gemm_persistent_ker
       __builtin_amdgcn_s_barrier();
       __builtin_amdgcn_sched_barrier(0);
       // block g + NSTAGE takes the ring slot of block g, which every wave has finished reading
-      if(ld_count < total_blocks && !(args.dbg & 1)) issue_next();
+      if(ld_count < total_blocks && !(MH_DBG(args, 1))) issue_next();
       read_frags((g + 1) % NSTAGE, 0, 0);
       read_frags((g + 1) % NSTAGE, 1, 1);
     }
@@ -356,18 +356,18 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * kWave) void gemm_persistent_ker
         __builtin_amdgcn_s_barrier();
       }
       long long te0 = 0;
-      if(args.prof) te0 = clock64();
+      if(MH_PROF(args)) te0 = MH_CLOCK();
       epilogue(round);
-      if(args.prof) t_epi += clock64() - te0;
+      if(MH_PROF(args)) t_epi += MH_CLOCK() - te0;
       zero_acc();
       pos = 0;
       ++round;
       since_store = 0;
     }
   }
-  if(args.prof && tid == 0) {
-    long long* p = args.prof + (size_t)blockIdx.x * 8;
-    p[0] = t_start; p[1] = t_prologue; p[2] = clock64() - t_epi; p[3] = clock64(); p[4] = t_epi; p[5] = total_blocks;
+  if(MH_PROF(args) && tid == 0) {
+    long long* p = MH_PROF(args) + (size_t)blockIdx.x * 8;
+    p[0] = t_start; p[1] = t_prologue; p[2] = MH_CLOCK() - t_epi; p[3] = MH_CLOCK(); p[4] = t_epi; p[5] = total_blocks;
   }
 }
 

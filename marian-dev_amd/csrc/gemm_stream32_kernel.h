@@ -87,9 +87,9 @@ __global__ __launch_bounds__(WN * KW * kWave) void gemm_stream32_kernel(GemmArgs
   __shared__ float red[kStream32Waves];
 
   long long tp[6] = {0, 0, 0, 0, 0, 0}, wall0 = 0;
-  if(args.prof) {
-    tp[0] = clock64();
-    wall0 = wall_clock64();
+  if(MH_PROF(args)) {
+    tp[0] = MH_CLOCK();
+    wall0 = MH_WALL();
   }
   const int tid = threadIdx.x;
   const int wave = tid / kWave, lane = tid % kWave;
@@ -186,7 +186,7 @@ __global__ __launch_bounds__(WN * KW * kWave) void gemm_stream32_kernel(GemmArgs
   }
 
   float aqm = 0.0f;        // quantMult of the activations (fused modes)
-  bool finite_t = false;   // kFusedTiled: abs-max finite and non-zero
+  bool finite_t = false;   // kFusedTiled: the quantMult is finite
   // Otherwise a chunk of activations is fetched into registers (all loads in flight at once) and
   // then dropped into LDS, so the fetch of chunk c+1 overlaps the multiplication of chunk c.
   // Pre-quantized: thread slot (sub-step, m-tile, lane) in operand order.  kFusedTiled: fp32
@@ -293,8 +293,8 @@ __global__ __launch_bounds__(WN * KW * kWave) void gemm_stream32_kernel(GemmArgs
   if(TILED) {
     amax = block_max(amax, red);
     aqm = quant_mult_from_maxabs(amax);
-    finite_t = amax > 0.0f && amax < __builtin_inff();
-    if(args.prof) tp[1] = clock64();
+    finite_t = aqm < __builtin_inff();   // (see the fused form below)
+    if(MH_PROF(args)) tp[1] = MH_CLOCK();
     if(aq_out && blockIdx.x == 0 && blockIdx.y == 0 && tid == 0)
       *reinterpret_cast<float*>(aq_out + (size_t)M * K) = aqm;
   }
@@ -311,10 +311,13 @@ __global__ __launch_bounds__(WN * KW * kWave) void gemm_stream32_kernel(GemmArgs
     // row only feeds its own output row, integer products cannot trap, and rows past M are never
     // stored)
     amax = block_max(amax, red);
-    if(args.prof) tp[1] = clock64();
+    if(MH_PROF(args)) tp[1] = MH_CLOCK();
     aqm = quant_mult_from_maxabs(amax);
-    // with a finite non-zero abs-max no product can leave [-127.0001, 127.0001]
-    const bool finite = amax > 0.0f && amax < __builtin_inff();
+    // With a finite quantMult no product can leave [-127.0001, 127.0001]: finite values are at
+    // most the abs-max in magnitude, and an infinite value makes the quantMult 0 and its product
+    // NaN.  (An abs-max of zero, or one below 127 / FLT_MAX, gives an infinite quantMult, and then
+    // infinite products, which the conversion of the CPU path turns into -127, not +127.)
+    const bool finite = aqm < __builtin_inff();
     const unsigned k16n = K / 16;   // 16-byte chunks per activation row (a multiple of four)
     unsigned row = 4 * quad / k16n, c16 = 4 * quad % k16n;   // of the quad's first group
     const unsigned drow = kStream32Threads / k16n, dc16 = kStream32Threads % k16n;
@@ -366,7 +369,7 @@ __global__ __launch_bounds__(WN * KW * kWave) void gemm_stream32_kernel(GemmArgs
     __syncthreads();
   }
 
-  if(args.prof) tp[2] = clock64();
+  if(MH_PROF(args)) tp[2] = MH_CLOCK();
   // The first chunk is peeled off the loop: its first product starts from a literal zero and its
   // fragment addresses are this wave's base plus constants (slot of sub-step step0 + p, half lg,
   // row li: the row key of chunk number 2 * (step0 + p) + lg is key(2 * step0) ^ key(2 * p) ^ lg,
@@ -419,7 +422,7 @@ __global__ __launch_bounds__(WN * KW * kWave) void gemm_stream32_kernel(GemmArgs
   multiply_chunk(0, std::true_type());
   for(int c = 1; c < n_chunks; ++c) multiply_chunk(c, std::false_type());
 
-  if(args.prof) tp[3] = clock64();
+  if(MH_PROF(args)) tp[3] = MH_CLOCK();
   // ---- every wave drops its 32 * MT32 x 32 tile of int32 partial sums into LDS as a row-major
   //      matrix [activation row][32 weight rows] (128 bytes per row; the eight 16-byte pieces of
   //      a row XOR-permuted by the row number, which keeps both sides free of bank conflicts),
@@ -443,7 +446,7 @@ __global__ __launch_bounds__(WN * KW * kWave) void gemm_stream32_kernel(GemmArgs
   }
   __syncthreads();
 
-  if(args.prof) tp[4] = clock64();
+  if(MH_PROF(args)) tp[4] = MH_CLOCK();
   float omax = 0.0f;   // max |y| over what this wave stores
   {
     constexpr int kPieces = R * 8 / KW;        // 16-byte pieces this wave finishes (32 .. 1024)
@@ -498,10 +501,10 @@ __global__ __launch_bounds__(WN * KW * kWave) void gemm_stream32_kernel(GemmArgs
     if(block == 0)
       for(int sl = used + tid; sl < kAbsmaxSlots; sl += kStream32Threads) args.absmax_out[sl] = 0.0f;
   }
-  if(args.prof && tid == 0) {
-    long long* p = args.prof + ((size_t)blockIdx.y * gridDim.x + blockIdx.x) * 8;
-    p[0] = tp[0]; p[1] = tp[1]; p[2] = tp[2]; p[3] = tp[3]; p[4] = tp[4]; p[5] = clock64();
-    p[6] = wall_clock64();
+  if(MH_PROF(args) && tid == 0) {
+    long long* p = MH_PROF(args) + ((size_t)blockIdx.y * gridDim.x + blockIdx.x) * 8;
+    p[0] = tp[0]; p[1] = tp[1]; p[2] = tp[2]; p[3] = tp[3]; p[4] = tp[4]; p[5] = MH_CLOCK();
+    p[6] = MH_WALL();
     p[7] = wall0;
   }
 }

@@ -98,8 +98,10 @@ struct GemmArgs {
   int M, K, N, n_out;
   float scale;
   int relu, dump;
-  int dbg;  // measurement switches (bit 0: no refetch, bit 1: no stores); 0 in normal use
-  long long* prof;  // per-workgroup phase clocks for tuning runs, null in normal use
+#ifdef MARIAN_HIP_TUNING
+  int dbg = 0;  // measurement switches (bit 0: no refetch, bit 1: no stores)
+  long long* prof = nullptr;  // per-workgroup phase clocks
+#endif
   // kAbsmaxSlots floats that receive values whose maximum is max|out| (the next call's abs-max,
   // taken where the tensor is produced), or null
   float* absmax_out = nullptr;
@@ -109,6 +111,20 @@ struct GemmArgs {
 };
 
 constexpr int kAbsmaxSlots = 2048;
+
+// The tuning build (-DMARIAN_HIP_TUNING, libmarian_hip_int8_tuning.so) carries measurement switches
+// and per-workgroup phase clocks in the kernels; the shipped library compiles them out.
+#ifdef MARIAN_HIP_TUNING
+#define MH_DBG(args, bit) ((args).dbg & (bit))
+#define MH_PROF(args) ((args).prof)
+#define MH_CLOCK() clock64()
+#define MH_WALL() wall_clock64()
+#else
+#define MH_DBG(args, bit) 0
+#define MH_PROF(args) (static_cast<long long*>(nullptr))
+#define MH_CLOCK() 0ll
+#define MH_WALL() 0ll
+#endif
 
 __device__ __forceinline__ Epilogue make_epilogue(const GemmArgs& a) {
   Epilogue e;

@@ -47,7 +47,7 @@ __device__ __forceinline__ uint32_t round_pack4(float c0, float c1, float c2, fl
   return q;
 }
 
-// Fast form for the usual case (finite, non-zero abs-max): every product lies within
+// Fast form for the usual case (finite quantMult): every product lies within
 // [-127.0001, 127.0001], so the out-of-range check of quantize_clamped can never fire (med3
 // still maps a NaN among the values to -127).
 __device__ __forceinline__ uint32_t quantize_pack4_finite(v4f x, float qm) {

@@ -11,6 +11,8 @@ Tensors are torch tensors on the GPU (device memory and streams only); every ari
 is a call into the C ABI.  Quantized tensors are `QTensor`: a flat int8 buffer holding the
 payload plus the fp32 quantMult tail, with Marian's logical shape and element type.
 """
+import weakref
+
 import numpy as np
 import torch
 
@@ -96,7 +98,6 @@ class Backend:
 
     def __init__(self, device):
         self.device = torch.device(device)
-        self.lib = _lib.lib()
         self.workspace_bytes = int(self.lib.marian_hip_int8_workspace_bytes())
         self.workspace = torch.empty(self.workspace_bytes, dtype=torch.uint8, device=self.device)
         # float32 weights are quantized on first use and remembered when this is Type.intgemm8:
@@ -106,18 +107,39 @@ class Backend:
         self.gemmType = None
         self._memo = {}
 
+    @property
+    def lib(self):
+        return _lib.lib()
+
     def setGemmType(self, type_):
         _abort_if(type_ not in (None, Type.intgemm8), "Unsupported type {} for Intgemm type??", type_)
         self.gemmType = type_
 
+    @staticmethod
+    def _memo_key(w):
+        return (w.data_ptr(), tuple(w.shape), w._version)
+
     def memoizedPrepareB(self, w):
-        """prepareB of a float32 parameter, once per (storage, shape, version)."""
-        key = (w.data_ptr(), tuple(w.shape), w._version)
+        """prepareB of a float32 parameter, once per parameter and version.  The reference
+        memoizes per parameter node (src/graph/expression_operators.cpp:564-598); here an entry
+        belongs to one tensor object: it holds a weak reference to it, a hit requires that very
+        object to be alive and to be the one asked for (an address can be handed to a new tensor of
+        the same shape once the old one is freed), and the entry goes when the tensor does."""
+        key = self._memo_key(w)
         hit = self._memo.get(key)
-        if hit is None:
-            hit = prepareB(w)
-            self._memo[key] = hit
-        return hit
+        if hit is not None and hit[0]() is w:
+            return hit[1]
+        q = prepareB(w)
+        memo = self._memo
+        for k in [k for k, (ref, _) in memo.items() if ref() is None or ref() is w]:
+            del memo[k]   # dead owners, and earlier versions of this parameter
+
+        def evict(_ref, key=key, memo=memo):
+            ent = memo.get(key)
+            if ent is not None and ent[0] is _ref:
+                del memo[key]
+        memo[key] = (weakref.ref(w, evict), q)
+        return q
 
     @classmethod
     def get(cls, device):

@@ -186,7 +186,12 @@ def getNBestList(scores, N):
     return vals, keys
 
 
-_nbest_workspaces = {}   # device -> uint8 tensor, grown on demand (the reference's NthElement owns its buffers too)
+# (device, stream) -> list of uint8 tensors, the last one the largest.  The reference's NthElement
+# owns its buffers too (src/translator/nth_element.cu).  A workspace holds arrival counters that
+# every call leaves at zero, so calls on one stream share it; two streams never do.  A workspace
+# that has been handed out is kept for good (a HIP graph may have recorded its address): a larger
+# call gets an additional one.
+_nbest_workspaces = {}
 
 
 def getNBestListOfBeams(scores, N):
@@ -200,12 +205,13 @@ def getNBestListOfBeams(scores, N):
     vals = torch.empty(dimBatch * N, dtype=torch.float32, device=scores.device)
     keys = torch.empty(dimBatch * N, dtype=torch.int32, device=scores.device)
     need = be.lib.marian_hip_nbest_beams_workspace_bytes(beam, dimBatch, vocab, N)
-    ws = _nbest_workspaces.get(scores.device)
-    if ws is None or ws.numel() < need:
+    held = _nbest_workspaces.setdefault((scores.device, be.stream()), [])
+    if not held or held[-1].numel() < need:
         ws = torch.empty(max(int(need), 4), dtype=torch.uint8, device=scores.device)
         _lib.check(be.lib.marian_hip_nbest_beams_workspace_init(ws.data_ptr(), ws.numel(), be.stream()),
                    "getNBestListOfBeams")
-        _nbest_workspaces[scores.device] = ws
+        held.append(ws)
+    ws = held[-1]
     st = be.lib.marian_hip_nbest_beams(scores.data_ptr(), beam, dimBatch, vocab, N, vals.data_ptr(),
                                        keys.data_ptr(), ws.data_ptr(), ws.numel(), be.stream())
     _lib.check(st, "getNBestListOfBeams")

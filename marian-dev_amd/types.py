@@ -19,10 +19,19 @@ class TypeClass(enum.IntEnum):
 
 class Type(enum.IntEnum):
     int8 = TypeClass.signed_type + 1
+    int16 = TypeClass.signed_type + 2
     int32 = TypeClass.signed_type + 4
+    int64 = TypeClass.signed_type + 8
+    uint8 = TypeClass.unsigned_type + 1
+    uint16 = TypeClass.unsigned_type + 2
     uint32 = TypeClass.unsigned_type + 4
+    uint64 = TypeClass.unsigned_type + 8
     float16 = TypeClass.float_type + 2
     float32 = TypeClass.float_type + 4
+    float64 = TypeClass.float_type + 8
+    packed16 = TypeClass.packed_type + 2
+    packed8avx2 = TypeClass.packed_type + 1 + TypeClass.avx2_type
+    packed8avx512 = TypeClass.packed_type + 1 + TypeClass.avx512_type
     intgemm8 = TypeClass.intgemm_type + 1
     intgemm16 = TypeClass.intgemm_type + 2
     intgemm8ssse3 = TypeClass.intgemm_type + 1 + TypeClass.ssse3_type
@@ -32,6 +41,13 @@ class Type(enum.IntEnum):
     intgemm16sse2 = TypeClass.intgemm_type + 2 + TypeClass.sse2_type
     intgemm16avx2 = TypeClass.intgemm_type + 2 + TypeClass.avx2_type
     intgemm16avx512 = TypeClass.intgemm_type + 2 + TypeClass.avx512_type
+
+    # messages print a type by name, like operator<< of reference src/common/types.h:419-456
+    def __str__(self):
+        return self.name
+
+    def __format__(self, spec):
+        return format(self.name, spec)
 
 
 def sizeOf(t):
@@ -46,6 +62,11 @@ def isFloat(t):
 def isIntgemm(t):
     """reference src/common/types.h:378-380"""
     return (int(t) & TypeClass.intgemm_type) != 0
+
+
+def isPacked(t):
+    """reference src/common/types.h:358-360"""
+    return (int(t) & TypeClass.packed_type) != 0
 
 
 def isHardwareSpecific(t):

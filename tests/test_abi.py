@@ -3,17 +3,24 @@ validation (which runs before any HIP call) behaves as documented.  No compute w
 import ctypes
 import os
 import re
+import subprocess
 
 import pytest
 
 from conftest import ROOT, load
 
 HEADERS = [os.path.join(ROOT, "include", h) for h in ("marian_hip_int8.h", "marian_hip_ops.h")]
+TUNING_HEADER = os.path.join(ROOT, "include", "marian_hip_int8_tuning.h")
 
 
-def declared_functions():
+def exported_symbols(path):
+    out = subprocess.run(["nm", "-D", "--defined-only", path], check=True, capture_output=True, text=True).stdout
+    return sorted(line.split()[-1] for line in out.splitlines() if line.strip())
+
+
+def declared_functions(headers=HEADERS):
     names = set()
-    for header in HEADERS:
+    for header in headers:
         text = open(header).read()
         text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
         names |= set(re.findall(r"\b(marian_hip_\w+)\s*\(", text))
@@ -39,6 +46,18 @@ def test_library_exports_every_declared_symbol():
         assert hasattr(lib, name), name
     # and the Python binding covers the same set
     assert sorted(L.SIGNATURES) == declared_functions()
+
+
+def test_shipped_library_exports_exactly_what_the_headers_declare():
+    """No measurement switch, no undeclared hook and no C++ symbol leaves the shipped library; the
+    tuning build adds exactly the two functions of its own header."""
+    L = load("_lib")
+    assert exported_symbols(L.LIB_PATH) == declared_functions()
+    assert os.path.exists(L.TUNING_LIB_PATH), "build the library first (__graft_entry__.build())"
+    tuning = declared_functions([TUNING_HEADER])
+    assert tuning == ["marian_hip_int8_debug_profile", "marian_hip_int8_set_kernel"]
+    assert exported_symbols(L.TUNING_LIB_PATH) == sorted(declared_functions() + tuning)
+    assert sorted(L.TUNING_SIGNATURES) == tuning
 
 
 def test_status_strings_and_version():

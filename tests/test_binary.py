@@ -62,3 +62,51 @@ def test_unaligned_item_is_refused_on_save(tmp_path):
     with pytest.raises(ValueError, match="not 256-byte aligned"):
         B.save_items(os.path.join(tmp_path, "x.bin"),
                      [B.Item("a", (3,), T.Type.float32, np.zeros(12, np.uint8))])
+
+
+@pytest.mark.parametrize("name", ["intgemm16", "intgemm16sse2", "intgemm16avx2", "intgemm16avx512"])
+def test_sixteen_bit_intgemm_items_are_refused_with_the_reference_text(tmp_path, name):
+    """The HIP backend implements the 8-bit path; a 16-bit item (int16 payload, quantMult 1024,
+    reference src/tensors/cpu/integer_common.h:174-175) is refused at load with the text of the
+    reference's dispatch (src/tensors/cpu/intgemm_interface.h:126), naming the item."""
+    B = load("binary")
+    T = load("types")
+    raw = np.zeros(64 * 8 * 2 + 4, np.uint8)
+    raw[-4:] = np.frombuffer(f32(1024.0).tobytes(), np.uint8)
+    it = B.Item("decoder_l1_ffn_W1", (64, 8), T.Type[name], np.frombuffer(B._pad256(raw.tobytes()), np.uint8))
+    path = os.path.join(tmp_path, "w16.bin")
+    B.save_items(path, [it])
+    with pytest.raises(ValueError, match=r"decoder_l1_ffn_W1: Unsupported type %s for Intgemm type\?\?" % name):
+        B.load_items(path)
+
+
+def test_unknown_item_type_is_reported_with_the_item_name(tmp_path):
+    B = load("binary")
+    T = load("types")
+    it = B.float_item("special:model.yml", np.zeros(64, f32))
+    path = os.path.join(tmp_path, "u.bin")
+    B.save_items(path, [it])
+    raw = bytearray(open(path, "rb").read())
+    struct.pack_into("<Q", raw, 16 + 8, 0x20000 + 1)         # no such id in Marian's enum
+    open(path, "wb").write(raw)
+    with pytest.raises(ValueError, match=r"special:model.yml has the unsupported item type 0x20001"):
+        B.load_items(path)
+    struct.pack_into("<Q", raw, 16 + 8, int(T.Type.packed8avx2))
+    open(path, "wb").write(raw)
+    with pytest.raises(ValueError, match=r"special:model.yml has the FBGEMM-packed type packed8avx2"):
+        B.load_items(path)
+
+
+def test_operator_refuses_sixteen_bit_weights_with_the_reference_text():
+    """affineOrDot's type switch (reference src/tensors/cpu/intgemm_interface.h:104-127): anything
+    but an 8-bit hardware-agnostic intgemm weight ends in its default branch."""
+    import torch
+    integer = load("integer")
+    T = load("types")
+    a = torch.zeros(2, 64)
+    for t in (T.Type.intgemm16, T.Type.intgemm16avx2, T.Type.intgemm8avx2):
+        w = integer.QTensor(torch.zeros(64 * 8 * 2 + 4, dtype=torch.int8), (64, 8), t)
+        with pytest.raises(integer.MarianRuntimeError, match=r"Unsupported type .*%s.* for Intgemm type\?\?" % t.name):
+            integer.affineOrDot(a, w)
+    with pytest.raises(integer.MarianRuntimeError, match="Intgemm expects type of B to be a variant of intgemm"):
+        integer.affineOrDot(a, integer.QTensor(torch.zeros(64 * 8 * 4, dtype=torch.int8), (64, 8), T.Type.float32))

@@ -18,6 +18,14 @@ GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "int
 REL_TOL = 1e-5
 
 
+def forced(kernel):
+    """kernel == 0: the shipped library and its automatic selection.  Other ids pin a kernel
+    family, which only the tuning build of the library can do."""
+    import contextlib
+    from conftest import load
+    return load("_lib").forced_kernel(kernel) if kernel else contextlib.nullcontext()
+
+
 def say(*a):
     print(*a, flush=True)
     sys.stdout.flush()
@@ -118,18 +126,13 @@ KERNELS = [0, 101, 102, 501, 511, 512, 514, 518, 521, 522, 524, 201, 202, 203, 2
 
 
 def run_case(integer, orc, synth, seed, M, K, N, kernel, bias_on=True, relu=False, scale=1.0):
-    from conftest import load
-    lib = load("_lib").lib()
     A, W, bias = inputs(synth, seed, M, K, N)
     Aq_h, Bq_h = orc.prepare_a(A), orc.prepare_b(W)
     want_out, want_acc = orc.affine(Aq_h, Bq_h, bias if bias_on else None, M, K, N, scale, relu)
     Aq, Bq = upload_q(integer, Aq_h, (M, K)), upload_q(integer, Bq_h, (K, N))
-    prev = lib.marian_hip_int8_set_kernel(kernel)
-    try:
+    with forced(kernel):
         acc = integer.multiply_i32(Aq, Bq).cpu().numpy()
         out = integer.multiply(Aq, Bq, dev(bias) if bias_on else None, scale=scale, relu=relu).cpu().numpy()
-    finally:
-        lib.marian_hip_int8_set_kernel(prev)
     assert np.array_equal(acc, want_acc), "int32 accumulators differ (kernel %d)" % kernel
     unquant = orc.unquant_mult(orc.tail(Aq_h, M * K), orc.tail(Bq_h, K * N), scale)
     assert_close_fp32(out, want_out, unquant, K)
@@ -192,21 +195,16 @@ def test_multiply_tile_pair_kernel(integer, orc, synth, M, K, N, bias_on, relu, 
 def test_fused_affine_f32(integer, orc, synth, M, K, N, kernel):
     """prepareA + multiply in one call (one fused kernel where the activations are small):
     output, quantized activations and quantMult equal those of the two separate steps."""
-    from conftest import load
-    lib = load("_lib").lib()
     say("fused", M, K, N, "kernel", kernel)
     A, W, bias = inputs(synth, 500 + M + N, M, K, N)
     Aq_h, Bq_h = orc.prepare_a(A), orc.prepare_b(W)
     relu = (M % 2 == 1)
     want, _ = orc.affine(Aq_h, Bq_h, bias, M, K, N, 0.5, relu)
     Bq = upload_q(integer, Bq_h, (K, N))
-    prev = lib.marian_hip_int8_set_kernel(kernel)
-    try:
+    with forced(kernel):
         out, Aq = integer.affine_f32(dev(A), Bq, dev(bias), scale=0.5, relu=relu)
         out = out.cpu().numpy()
         got_aq = Aq.numpy()
-    finally:
-        lib.marian_hip_int8_set_kernel(prev)
     assert np.array_equal(got_aq, Aq_h), "quantized activations / quantMult of the fused call"
     assert np.array_equal(out, want)
 
@@ -231,8 +229,6 @@ def test_fused_shortlist(integer, orc, synth):
 def test_shortlist_every_kernel_family(integer, orc, synth, M, kernel):
     """The row gather of W^T and of the bias inside each kernel family (ids >= 600: fused call)."""
     import torch
-    from conftest import load
-    lib = load("_lib").lib()
     say("shortlist", M, "kernel", kernel)
     K, N = 256, 2048
     A, W, bias = inputs(synth, 707 + M, M, K, N)
@@ -241,8 +237,7 @@ def test_shortlist_every_kernel_family(integer, orc, synth, M, kernel):
     want, want_acc = orc.affine_shortlist(Aq_h, Bq_h, bias, idx, M, K, N)
     Bq = upload_q(integer, Bq_h, (K, N))
     didx = torch.from_numpy(idx.view(np.int32)).cuda()
-    prev = lib.marian_hip_int8_set_kernel(kernel)
-    try:
+    with forced(kernel):
         if kernel >= 600:
             out, Aq = integer.affine_f32(dev(A), Bq, dev(bias), shortlist=didx)
             assert np.array_equal(Aq.numpy(), Aq_h)
@@ -252,8 +247,6 @@ def test_shortlist_every_kernel_family(integer, orc, synth, M, kernel):
             assert np.array_equal(acc, want_acc)
             out = integer.multiply(Aq, Bq, dev(bias), shortlist=didx)
         out = out.cpu().numpy()
-    finally:
-        lib.marian_hip_int8_set_kernel(prev)
     assert np.array_equal(out, want)
 
 
