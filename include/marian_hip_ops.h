@@ -130,6 +130,15 @@ int marian_hip_nbest_beams(const float* scores, int64_t beam, int64_t dimBatch, 
                            float* outScores, uint32_t* outKeys, void* workspace, size_t workspace_bytes,
                            void* stream);
 
+/*
+ * Replaces gpu::fill, reference src/tensors/gpu/algorithm.cu:37-60 (gFill): `count` elements of
+ * elem_bytes (1, 2, 4 or 8) bytes each, starting at `begin` (aligned to elem_bytes), receive the
+ * low elem_bytes bytes of `pattern` - the bit pattern of the value, so one entry point serves
+ * every element type.  A kernel, not a memset: it may be recorded into a HIP graph.  Like every
+ * function here it does not synchronise; the C++ wrapper adds the reference's stream synchronisation.
+ */
+int marian_hip_fill(void* begin, int64_t count, int elem_bytes, uint64_t pattern, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

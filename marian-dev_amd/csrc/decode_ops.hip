@@ -937,6 +937,26 @@ __global__ __launch_bounds__(1024) void nbest_part_kernel(const float* __restric
   }
 }
 
+// Fill: the 16-byte aligned middle of the range with 16-byte stores of the repeated pattern, the
+// bytes before and after it one by one (byte i of the range holds byte i % elem_bytes of the
+// pattern; the middle starts on an element boundary because the range does).
+__global__ __launch_bounds__(256) void fill_kernel(unsigned char* __restrict__ p, long long bytes, long long head,
+                                                   long long vecs, int elem_bytes, unsigned long long pattern) {
+  const long long tid = (long long)blockIdx.x * blockDim.x + threadIdx.x, nthreads = (long long)gridDim.x * blockDim.x;
+  unsigned long long rep = pattern;
+  if(elem_bytes == 1) rep = (pattern & 0xFFull) * 0x0101010101010101ull;
+  else if(elem_bytes == 2) rep = (pattern & 0xFFFFull) * 0x0001000100010001ull;
+  else if(elem_bytes == 4) rep = (pattern & 0xFFFFFFFFull) * 0x0000000100000001ull;
+  typedef unsigned long long v2u64 __attribute__((ext_vector_type(2)));
+  v2u64* mid = reinterpret_cast<v2u64*>(p + head);
+  for(long long i = tid; i < vecs; i += nthreads) mid[i] = v2u64{rep, rep};
+  const long long tail0 = head + vecs * 16;
+  for(long long i = tid; i < head + (bytes - tail0); i += nthreads) {
+    const long long at = i < head ? i : tail0 + (i - head);
+    p[at] = (unsigned char)(pattern >> (8 * (at % elem_bytes)));
+  }
+}
+
 __global__ __launch_bounds__(256) void zero_words_kernel(unsigned* __restrict__ p, long long n) {
   for(long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long long)gridDim.x * blockDim.x)
     p[i] = 0u;
@@ -1130,6 +1150,27 @@ int marian_hip_nbest(const float* scores, int64_t dimBatch, int64_t rowLen, int6
     hipLaunchKernelGGL(nbest_kernel<8>, dim3((unsigned)dimBatch), dim3(1024), 0, st, scores, (long long)rowLen, (int)N, outScores, outKeys);
   else
     hipLaunchKernelGGL(nbest_kernel<16>, dim3((unsigned)dimBatch), dim3(1024), 0, st, scores, (long long)rowLen, (int)N, outScores, outKeys);
+  MH_HIP(hipGetLastError());
+  return MARIAN_HIP_OK;
+}
+
+int marian_hip_fill(void* begin, int64_t count, int elem_bytes, uint64_t pattern, void* stream) {
+  if(count < 0 || (elem_bytes != 1 && elem_bytes != 2 && elem_bytes != 4 && elem_bytes != 8))
+    return MARIAN_HIP_ERR_SHAPE;
+  if(count == 0) return MARIAN_HIP_OK;
+  if(!begin) return MARIAN_HIP_ERR_NULL;
+  if(reinterpret_cast<uintptr_t>(begin) % (uintptr_t)elem_bytes != 0) return MARIAN_HIP_ERR_ALIGN;
+  if(count > (int64_t)(0x7FFFFFFFFFFFFFFFll / 8)) return MARIAN_HIP_ERR_RANGE;
+  const long long bytes = (long long)count * elem_bytes;
+  long long head = (long long)((16 - reinterpret_cast<uintptr_t>(begin) % 16) % 16);
+  if(head > bytes) head = bytes;
+  const long long vecs = (bytes - head) / 16;
+  long long blocks = (vecs + 255) / 256;
+  if(blocks < 1) blocks = 1;
+  if(blocks > 4096) blocks = 4096;
+  hipLaunchKernelGGL(fill_kernel, dim3((unsigned)blocks), dim3(256), 0, reinterpret_cast<hipStream_t>(stream),
+                     reinterpret_cast<unsigned char*>(begin), bytes, head, vecs, elem_bytes,
+                     (unsigned long long)pattern);
   MH_HIP(hipGetLastError());
   return MARIAN_HIP_OK;
 }

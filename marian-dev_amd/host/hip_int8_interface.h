@@ -7,33 +7,26 @@
 //   src/tensors/cpu/intgemm_interface.h:17-32  prepareA()
 //   src/tensors/cpu/intgemm_interface.h:46-99  affineOrDotTyped()  -> affineOrDot()
 //   src/tensors/gpu/backend.h:23-110           Backend (stream, synchronize), reduced to this path
+//   src/tensors/tensor_allocator.h:12-93       TensorAllocator (tensors carved from hip_device.h's Allocator)
 //   src/tensors/gpu/cuda_helpers.h:15-19       CUDA_CHECK -> MARIAN_HIP_CHECK (status code -> abort)
+//
+// Tensors hold a MemoryPiece handle, not a pointer: the allocator may move its slab whenever
+// something is allocated, and every wrapper below reads the pointers at the moment of the call.
+// The library retains nothing between calls, so a move between two calls is harmless.
 #pragma once
 
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
-#include <cstdio>
-#include <cstdlib>
-#include <stdexcept>
 #include <string>
 #include <vector>
 
 #include "../../include/marian_hip_int8.h"
+#include "hip_device.h"
 
 namespace marian {
 namespace hip {
 
-// ABORT of src/common/logging.h:100-116: throws when asked to (setThrowExceptionOnAbort), else aborts.
-inline bool& throwOnAbort() {
-  static bool flag = true;
-  return flag;
-}
-[[noreturn]] inline void abortWith(const std::string& msg) {
-  if(throwOnAbort()) throw std::runtime_error(msg);
-  std::fprintf(stderr, "Error: %s\n", msg.c_str());
-  std::abort();
-}
 #define MARIAN_HIP_CHECK(expr)                                                              \
   do {                                                                                      \
     int st_ = (expr);                                                                       \
@@ -43,71 +36,119 @@ inline bool& throwOnAbort() {
                                     ? " (hipError " + std::to_string(marian_hip_last_hip_error()) + ")" \
                                     : std::string()));                                      \
   } while(0)
-#define HIP_CHECK(expr)                                                                     \
-  do {                                                                                      \
-    hipError_t e_ = (expr);                                                                 \
-    if(e_ != hipSuccess) ::marian::hip::abortWith(std::string(#expr) + ": " + hipGetErrorString(e_)); \
-  } while(0)
 
 // Element types with Marian's numeric values (src/common/types.h:270-328).
 enum class Type : size_t {
+  int8 = 0x100 + 1,
+  int32 = 0x100 + 4,
+  uint32 = 0x200 + 4,
   float32 = 0x400 + 4,
   intgemm8 = 0x10000 + 1,
+  intgemm16 = 0x10000 + 2,
   intgemm8ssse3 = 0x10000 + 1 + 0x8000,
   intgemm8avx2 = 0x10000 + 1 + 0x1000,
   intgemm8avx512 = 0x10000 + 1 + 0x2000,
   intgemm8avx512vnni = 0x10000 + 1 + 0x2000 + 4096,
+  intgemm16sse2 = 0x10000 + 2 + 0x4000,
+  intgemm16avx2 = 0x10000 + 2 + 0x1000,
+  intgemm16avx512 = 0x10000 + 2 + 0x2000,
 };
+inline size_t sizeOf(Type t) { return (size_t)t & 0xFF; }
 inline bool isIntgemm(Type t) { return ((size_t)t & 0x10000) != 0; }
 inline bool isFloat(Type t) { return ((size_t)t & 0x400) != 0; }
 inline bool isHardwareSpecific(Type t) { return isIntgemm(t) && ((size_t)t & 0xF000) != 0; }
 
-// A device tensor view: the caller (Marian's allocator) owns the memory.
+typedef std::vector<int> Shape;
+inline size_t elements(const Shape& shape) {
+  size_t n = 1;
+  for(int d : shape) n *= (size_t)d;
+  return n;
+}
+// src/common/types.cpp:32-34: intgemm tensors carry one extra fp32, the quantMult
+inline size_t requiredBytes(const Shape& shape, Type type) {
+  return elements(shape) * sizeOf(type) + (isIntgemm(type) ? sizeof(float) : 0);
+}
+
+// A device tensor: a piece of the allocator's slab with a shape and an element type.
 struct Tensor {
-  void* data = nullptr;
-  std::vector<int> shape;
+  MemoryPiece::PtrType memory;
+  Shape shape;
   Type type = Type::float32;
-  size_t elements() const {
-    size_t n = 1;
-    for(int d : shape) n *= (size_t)d;
-    return n;
-  }
+  size_t elements() const { return ::marian::hip::elements(shape); }
+  template <typename T>
+  T* data() const { return memory ? memory->data<T>() : nullptr; }
+  explicit operator bool() const { return memory && memory->data(); }
 };
 inline int cols(const Tensor& t) { return t.shape.back(); }
 inline int rows(const Tensor& t) { return (int)(t.elements() / (size_t)cols(t)); }
-// src/common/types.cpp:32-34
-inline size_t requiredBytes(const std::vector<int>& shape, Type type) {
-  size_t n = 1;
-  for(int d : shape) n *= (size_t)d;
-  return isIntgemm(type) ? n + sizeof(float) : n * sizeof(float);
-}
 
-// Per-device state of the path: one stream and the abs-max workspace.
+// Per-device state of the path: the device number and one stream.
 class Backend {
 public:
   explicit Backend(int device) : device_(device) {
     HIP_CHECK(hipSetDevice(device_));
     HIP_CHECK(hipStreamCreateWithFlags(&stream_, hipStreamNonBlocking));
-    workspaceBytes_ = marian_hip_int8_workspace_bytes();
-    HIP_CHECK(hipMalloc(&workspace_, workspaceBytes_));
   }
-  ~Backend() {
-    (void)hipFree(workspace_);
-    (void)hipStreamDestroy(stream_);
-  }
+  ~Backend() { (void)hipStreamDestroy(stream_); }
   Backend(const Backend&) = delete;
   Backend& operator=(const Backend&) = delete;
   void setDevice() { HIP_CHECK(hipSetDevice(device_)); }
   void synchronize() { HIP_CHECK(hipStreamSynchronize(stream_)); }
   hipStream_t stream() const { return stream_; }
-  void* workspace() const { return workspace_; }
-  size_t workspaceBytes() const { return workspaceBytes_; }
+  int deviceNo() const { return device_; }
 
 private:
   int device_;
   hipStream_t stream_ = nullptr;
-  void* workspace_ = nullptr;
-  size_t workspaceBytes_ = 0;
+};
+
+// Tensors out of an Allocator (reference src/tensors/tensor_allocator.h:12-93).  It also owns the
+// abs-max workspace of the int8 calls, a piece like any other (it moves with the slab).
+class TensorAllocator {
+public:
+  static constexpr size_t kGrow = 128ull << 20, kAlign = 256;
+  explicit TensorAllocator(Backend& backend, size_t step = kGrow, size_t limit = 0)
+      : backend_(backend),
+        device_(std::make_shared<Device>(backend.deviceNo(), kAlign)),
+        allocator_(std::make_shared<Allocator>(device_, 0, step, kAlign, limit, backend.stream())) {}
+
+  void throwAtReallocation(bool flag) { allocator_->throwAtReallocation(flag); }
+  void reserveExact(size_t bytes) {
+    allocator_->reserve(bytes);
+    workspace_.reset();
+  }
+  void clear() {
+    allocator_->clear();
+    workspace_.reset();
+  }
+  size_t capacity(const Shape& shape, Type type = Type::float32) const {
+    return allocator_->alignedSize(requiredBytes(shape, type));
+  }
+  void allocate(Tensor& t, const Shape& shape, Type type = Type::float32) {
+    if(!t || t.shape != shape || t.type != type) {
+      t.memory = allocator_->alloc(requiredBytes(shape, type));
+      t.shape = shape;
+      t.type = type;
+    }
+  }
+  void free(Tensor& t) {
+    if(t.memory) allocator_->free(t.memory);
+    t.memory.reset();
+  }
+  // the abs-max workspace of marian_hip_int8_prepare_a / _prepare_b / _affine_f32
+  void* workspace() {
+    if(!workspace_ || !workspace_->data()) workspace_ = allocator_->alloc(workspaceBytes());
+    return workspace_->data();
+  }
+  size_t workspaceBytes() const { return marian_hip_int8_workspace_bytes(); }
+  const std::shared_ptr<Allocator>& allocator() const { return allocator_; }
+  Backend& backend() const { return backend_; }
+
+private:
+  Backend& backend_;
+  std::shared_ptr<Device> device_;
+  std::shared_ptr<Allocator> allocator_;
+  MemoryPiece::PtrType workspace_;
 };
 
 namespace integer {
@@ -116,47 +157,96 @@ namespace integer {
 inline float getQuantMult(Backend& be, const Tensor& t) {
   if(!isIntgemm(t.type)) abortWith("getQuantMult does not work for this type");
   float qm = 0.f;
-  HIP_CHECK(hipMemcpyAsync(&qm, (const int8_t*)t.data + t.elements(), sizeof(float),
-                           hipMemcpyDeviceToHost, be.stream()));
-  be.synchronize();
+  copy(be.stream(), reinterpret_cast<const float*>(t.data<int8_t>() + t.elements()),
+       reinterpret_cast<const float*>(t.data<int8_t>() + t.elements()) + 1, &qm);
   return qm;
 }
 
 // Forward body of the prepareA node: out has shape of a, type intgemm8, requiredBytes(shape) bytes.
-inline void prepareA(Backend& be, const Tensor& a, Tensor& out) {
+inline void prepareA(TensorAllocator& ta, const Tensor& a, Tensor& out) {
   if(!isFloat(a.type)) abortWith("Intgemm expects type of A to be float32");
-  MARIAN_HIP_CHECK(marian_hip_int8_prepare_a((const float*)a.data, (int8_t*)out.data, rows(a), cols(a),
-                                             be.workspace(), be.workspaceBytes(), be.stream()));
+  void* ws = ta.workspace();   // (may allocate: before any pointer is read)
+  MARIAN_HIP_CHECK(marian_hip_int8_prepare_a(a.data<float>(), out.data<int8_t>(), rows(a), cols(a), ws,
+                                             ta.workspaceBytes(), ta.backend().stream()));
 }
 
 // Offline quantizer body (marian-conv): w float32 [K, N] -> out intgemm8 [K, N] (payload W^T).
-inline void prepareB(Backend& be, const Tensor& w, Tensor& out) {
-  MARIAN_HIP_CHECK(marian_hip_int8_prepare_b((const float*)w.data, (int8_t*)out.data, w.shape[0],
-                                             w.shape[1], be.workspace(), be.workspaceBytes(),
-                                             be.stream()));
+inline void prepareB(TensorAllocator& ta, const Tensor& w, Tensor& out) {
+  void* ws = ta.workspace();
+  MARIAN_HIP_CHECK(marian_hip_int8_prepare_b(w.data<float>(), out.data<int8_t>(), w.shape[0], w.shape[1],
+                                             ws, ta.workspaceBytes(), ta.backend().stream()));
+}
+
+inline void checkB(const Tensor& bQuant) {
+  if(!isIntgemm(bQuant.type)) abortWith("Intgemm expects type of B to be a variant of intgemm");
+  if(isHardwareSpecific(bQuant.type) || sizeOf(bQuant.type) != 1) abortWith("Unsupported type for Intgemm type??");
 }
 
 // Forward body of the multiply node; bias may be null (dot).  relu fuses the in-place ReLU node.
-inline void multiply(Backend& be, const Tensor& aQuant, const Tensor& bQuant, const Tensor* bias,
-                     Tensor& out, float scale, bool relu) {
-  MARIAN_HIP_CHECK(marian_hip_int8_affine((const int8_t*)aQuant.data, (const int8_t*)bQuant.data,
-                                          bias ? (const float*)bias->data : nullptr,
-                                          (float*)out.data, rows(aQuant), cols(aQuant), cols(bQuant),
-                                          scale, relu ? 1 : 0, be.stream()));
+// shortlist: device ids (sorted, unique, a multiple of eight many) or null.
+inline void multiply(Backend& be, const Tensor& aQuant, const Tensor& bQuant, const Tensor* bias, Tensor& out,
+                     float scale, bool relu, const Tensor* shortlist = nullptr) {
+  checkB(bQuant);
+  if(shortlist)
+    MARIAN_HIP_CHECK(marian_hip_int8_affine_shortlist(
+        aQuant.data<int8_t>(), bQuant.data<int8_t>(), bias ? bias->data<float>() : nullptr,
+        shortlist->data<uint32_t>(), (int64_t)shortlist->elements(), out.data<float>(), rows(aQuant),
+        cols(aQuant), cols(bQuant), scale, relu ? 1 : 0, be.stream()));
+  else
+    MARIAN_HIP_CHECK(marian_hip_int8_affine(aQuant.data<int8_t>(), bQuant.data<int8_t>(),
+                                            bias ? bias->data<float>() : nullptr, out.data<float>(),
+                                            rows(aQuant), cols(aQuant), cols(bQuant), scale, relu ? 1 : 0,
+                                            be.stream()));
+}
+
+// The int32 accumulators Kernels8::Multiply hands to its callback (parity hook).
+inline void multiplyInt32(Backend& be, const Tensor& aQuant, const Tensor& bQuant, Tensor& acc,
+                          const Tensor* shortlist = nullptr) {
+  checkB(bQuant);
+  MARIAN_HIP_CHECK(marian_hip_int8_multiply_i32(
+      aQuant.data<int8_t>(), bQuant.data<int8_t>(), shortlist ? shortlist->data<uint32_t>() : nullptr,
+      shortlist ? (int64_t)shortlist->elements() : 0, acc.data<int32_t>(), rows(aQuant), cols(aQuant),
+      cols(bQuant), be.stream()));
 }
 
 // affineOrDot: type guards as in the reference, then both node bodies in one call.  aQuant is the
 // prepareA node's output tensor (it is filled exactly as prepareA would fill it).
-inline void affineOrDot(Backend& be, const Tensor& a, Tensor& aQuant, const Tensor& bQuant,
+// absmaxIn / absmaxOut: optional tensors of MARIAN_HIP_ABSMAX_SLOTS floats; absmaxIn is what the
+// call that produced `a` left (then the abs-max pass over `a` is skipped), absmaxOut receives the
+// same for `out`.
+inline void affineOrDot(TensorAllocator& ta, const Tensor& a, Tensor& aQuant, const Tensor& bQuant,
                         const Tensor* bias, Tensor& out, float scale = 1.f, bool relu = false,
-                        const uint32_t* shortlist = nullptr, int nShortlist = 0) {
+                        const Tensor* shortlist = nullptr, const Tensor* absmaxIn = nullptr,
+                        Tensor* absmaxOut = nullptr) {
   if(!isFloat(a.type)) abortWith("Intgemm expects type of A to be float32");
-  if(!isIntgemm(bQuant.type)) abortWith("Intgemm expects type of B to be a variant of intgemm");
-  if(isHardwareSpecific(bQuant.type)) abortWith("Unsupported type for Intgemm type??");
-  MARIAN_HIP_CHECK(marian_hip_int8_affine_f32(
-      (const float*)a.data, (int8_t*)aQuant.data, (const int8_t*)bQuant.data,
-      bias ? (const float*)bias->data : nullptr, shortlist, nShortlist, (float*)out.data, rows(a),
-      cols(a), cols(bQuant), scale, relu ? 1 : 0, be.workspace(), be.workspaceBytes(), be.stream()));
+  checkB(bQuant);
+  void* ws = ta.workspace();   // (may allocate and move the slab: before any pointer is read)
+  const uint32_t* idx = shortlist ? shortlist->data<uint32_t>() : nullptr;
+  const int64_t nIdx = shortlist ? (int64_t)shortlist->elements() : 0;
+  if(absmaxIn || absmaxOut)
+    MARIAN_HIP_CHECK(marian_hip_int8_affine_f32_chained(
+        a.data<float>(), aQuant.data<int8_t>(), bQuant.data<int8_t>(), bias ? bias->data<float>() : nullptr,
+        idx, nIdx, out.data<float>(), rows(a), cols(a), cols(bQuant), scale, relu ? 1 : 0,
+        absmaxIn ? absmaxIn->data<float>() : nullptr, absmaxOut ? absmaxOut->data<float>() : nullptr, ws,
+        ta.workspaceBytes(), ta.backend().stream()));
+  else
+    MARIAN_HIP_CHECK(marian_hip_int8_affine_f32(
+        a.data<float>(), aQuant.data<int8_t>(), bQuant.data<int8_t>(), bias ? bias->data<float>() : nullptr,
+        idx, nIdx, out.data<float>(), rows(a), cols(a), cols(bQuant), scale, relu ? 1 : 0, ws,
+        ta.workspaceBytes(), ta.backend().stream()));
+}
+
+// The same for callers that cannot allocate: no aQuant tensor, no workspace (the library's static
+// scratch holds both; rows(a) * cols(a) <= MARIAN_HIP_STATIC_MAX_ELEMS).
+inline void affineOrDotStatic(Backend& be, const Tensor& a, const Tensor& bQuant, const Tensor* bias,
+                              Tensor& out, float scale = 1.f, bool relu = false,
+                              const Tensor* shortlist = nullptr) {
+  if(!isFloat(a.type)) abortWith("Intgemm expects type of A to be float32");
+  checkB(bQuant);
+  MARIAN_HIP_CHECK(marian_hip_int8_affine_f32_static(
+      a.data<float>(), bQuant.data<int8_t>(), bias ? bias->data<float>() : nullptr,
+      shortlist ? shortlist->data<uint32_t>() : nullptr, shortlist ? (int64_t)shortlist->elements() : 0,
+      out.data<float>(), rows(a), cols(a), cols(bQuant), scale, relu ? 1 : 0, be.stream()));
 }
 
 }  // namespace integer

@@ -1,0 +1,112 @@
+// C++ host side of the float operators between the int8 GEMMs (include/marian_hip_ops.h), with the
+// names and argument meaning of the tensor-level functions a HIP backend of Marian has to provide.
+//
+// Mirrors (reference file:line):
+//   src/tensors/tensor_operators.h (gpu:: declarations)                LayerNormalization, Softmax, LogSoftmax
+//   src/tensors/cpu/tensor_operators.cpp:220-246,415-526,1087-1162     their CPU bodies
+//   src/tensors/gpu/prod.cpp:471-574                                   ProdBatchedLegacy
+//   src/models/transformer.h:241-280                                   Attention()
+//   src/translator/nth_element.cpp:26-67, nth_element.cu               NthElement::getNBestList
+#pragma once
+
+#include "../../include/marian_hip_ops.h"
+#include "hip_int8_interface.h"
+
+namespace marian {
+namespace hip {
+
+// out = gamma * ((x - mean) / sigma) (+ beta) over the last dimension, x = in (+ add).
+// absmaxOut: optional tensor of MARIAN_HIP_ABSMAX_SLOTS floats for the affine call that reads `out`.
+inline void LayerNormalization(Backend& be, Tensor& out, const Tensor& in, const Tensor& gamma,
+                               const Tensor* beta, float eps, const Tensor* add = nullptr,
+                               Tensor* absmaxOut = nullptr) {
+  MARIAN_HIP_CHECK(marian_hip_layer_norm(
+      in.data<float>(), add ? add->data<float>() : nullptr, gamma.data<float>(), (int64_t)gamma.elements(),
+      beta ? beta->data<float>() : nullptr, beta ? (int64_t)beta->elements() : 0, out.data<float>(), rows(in),
+      cols(in), eps, absmaxOut ? absmaxOut->data<float>() : nullptr, be.stream()));
+}
+
+// mask: optional [nMasks, cols] log-mask; row r of `in` uses mask row (r / rowsPerMask) % nMasks.
+inline void Softmax(Backend& be, Tensor& out, const Tensor& in, const Tensor* mask = nullptr,
+                    int64_t rowsPerMask = 1) {
+  MARIAN_HIP_CHECK(marian_hip_softmax(in.data<float>(), mask ? mask->data<float>() : nullptr,
+                                      mask ? (int64_t)rows(*mask) : 0, rowsPerMask, out.data<float>(), rows(in),
+                                      cols(in), be.stream()));
+}
+
+inline void LogSoftmax(Backend& be, Tensor& out, const Tensor& in) {
+  MARIAN_HIP_CHECK(marian_hip_logsoftmax(in.data<float>(), out.data<float>(), rows(in), cols(in), be.stream()));
+}
+
+// in [d0, d1, d2, d3] -> out [d0, d2, d1, d3] (head split and join)
+inline void Transpose0213(Backend& be, Tensor& out, const Tensor& in) {
+  if(in.shape.size() != 4) abortWith("Transpose0213 expects a 4-d tensor");
+  MARIAN_HIP_CHECK(marian_hip_transpose0213(in.data<float>(), out.data<float>(), in.shape[0], in.shape[1],
+                                            in.shape[2], in.shape[3], be.stream()));
+}
+
+// C[i] = scalar * op(A[i % batchA]) * op(B[i % batchB]); the last two dimensions are the matrices.
+inline void ProdBatchedLegacy(Backend& be, Tensor& C, const Tensor& A, const Tensor& B, bool transA, bool transB,
+                              float scalar) {
+  const int64_t ra = A.shape[A.shape.size() - 2], ca = A.shape.back();
+  const int64_t rb = B.shape[B.shape.size() - 2], cb = B.shape.back();
+  const int64_t m = transA ? ca : ra, k = transA ? ra : ca, l = transB ? cb : rb, n = transB ? rb : cb;
+  if(l != k) abortWith("Matrix product requires inner dimensions to match");
+  MARIAN_HIP_CHECK(marian_hip_bdot_legacy(A.data<float>(), B.data<float>(), C.data<float>(),
+                                          (int64_t)(A.elements() / (size_t)(ra * ca)),
+                                          (int64_t)(B.elements() / (size_t)(rb * cb)), m, n, k, transA ? 1 : 0,
+                                          transB ? 1 : 0, scalar, be.stream()));
+}
+
+// q [batchQ, m, dk]; k, v [batchKV, len, dk]; out [batchQ, m, dk].  kNew / vNew [batchQ, dk]: the
+// newest position of a decoding step, appended to k and v by the call.
+inline void Attention(Backend& be, Tensor& out, const Tensor& q, Tensor& k, Tensor& v, float scale,
+                      const Tensor* mask = nullptr, int64_t rowsPerMask = 1, Tensor* absmaxOut = nullptr,
+                      const Tensor* kNew = nullptr, const Tensor* vNew = nullptr) {
+  if(q.shape.size() != 3 || k.shape.size() != 3) abortWith("Attention expects [batch, positions, dk] tensors");
+  MARIAN_HIP_CHECK(marian_hip_attention(
+      q.data<float>(), k.data<float>(), v.data<float>(), mask ? mask->data<float>() : nullptr,
+      mask ? (int64_t)rows(*mask) : 0, rowsPerMask, out.data<float>(), q.shape[0], k.shape[0], q.shape[1],
+      k.shape[1], q.shape[2], scale, absmaxOut ? absmaxOut->data<float>() : nullptr,
+      kNew ? kNew->data<float>() : nullptr, vNew ? vNew->data<float>() : nullptr, be.stream()));
+}
+
+// The beam search's n-best selection; it owns its device buffers like the reference's NthElement.
+class NthElement {
+public:
+  explicit NthElement(TensorAllocator& ta) : ta_(ta) {}
+
+  // scores [dimBatch, beam * vocab] -> the N best scores and keys of every row (device tensors)
+  void getNBestList(const Tensor& scores, int64_t N, Tensor& outScores, Tensor& outKeys) {
+    const int64_t dimBatch = scores.shape[0], rowLen = (int64_t)scores.elements() / dimBatch;
+    ta_.allocate(outScores, {(int)(dimBatch * N)}, Type::float32);
+    ta_.allocate(outKeys, {(int)(dimBatch * N)}, Type::uint32);
+    MARIAN_HIP_CHECK(marian_hip_nbest(scores.data<float>(), dimBatch, rowLen, N, outScores.data<float>(),
+                                      outKeys.data<uint32_t>(), ta_.backend().stream()));
+  }
+
+  // scores [beam, dimBatch, vocab] as they leave the decoder: transposition + n-best in one call
+  void getNBestListOfBeams(const Tensor& scores, int64_t N, Tensor& outScores, Tensor& outKeys) {
+    if(scores.shape.size() != 3) abortWith("getNBestListOfBeams expects [beam, batch, vocab]");
+    const int64_t beam = scores.shape[0], dimBatch = scores.shape[1], vocab = scores.shape[2];
+    ta_.allocate(outScores, {(int)(dimBatch * N)}, Type::float32);
+    ta_.allocate(outKeys, {(int)(dimBatch * N)}, Type::uint32);
+    const size_t need = marian_hip_nbest_beams_workspace_bytes(beam, dimBatch, vocab, N);
+    if(!workspace_ || workspace_.elements() < need) {
+      // (a larger one replaces the old one; its counters are cleared once, by a kernel)
+      if(workspace_) ta_.free(workspace_);
+      ta_.allocate(workspace_, {(int)need}, Type::int8);
+      MARIAN_HIP_CHECK(marian_hip_nbest_beams_workspace_init(workspace_.data<void>(), need, ta_.backend().stream()));
+    }
+    MARIAN_HIP_CHECK(marian_hip_nbest_beams(scores.data<float>(), beam, dimBatch, vocab, N, outScores.data<float>(),
+                                            outKeys.data<uint32_t>(), workspace_.data<void>(), workspace_.elements(),
+                                            ta_.backend().stream()));
+  }
+
+private:
+  TensorAllocator& ta_;
+  Tensor workspace_;
+};
+
+}  // namespace hip
+}  // namespace marian

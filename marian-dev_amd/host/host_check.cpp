@@ -1,79 +1,302 @@
-// Host-side check of the C++ wrappers: quantizes a small weight matrix on the GPU, runs
-// affineOrDot with bias and ReLU, and compares with a plain CPU restatement written out here
-// (max-abs, round-half-even quantize, exact integer dot product, two-step unquantize).
+// Check program for the C++ host side: Device / Allocator / TensorAllocator and the operator
+// wrappers, on the GPU, against expected values computed elsewhere.
+//
+//   host_check <fixture file>
+//
+// The fixture (written by the test that runs this program) holds the inputs and, for every step,
+// the values the CPU checker of the test suite computed from them; nothing is recomputed here.
+// Every buffer - inputs, quantized operands, outputs, the abs-max workspace - is carved from one
+// allocator whose slab is forced to grow, i.e. to MOVE, between prepareA and multiply, between two
+// affineOrDot calls and in the middle of a chained pair, so the "nothing is retained between
+// calls" contract of the library is exercised, not assumed.
+//
+// Fixture layout (little endian): "MHC2", int32 M, K, N, N2, nIdx, R, C, nbestN; then
+//   float A[M*K], W[K*N], bias[N], W2[N*N2]; uint32 idx[nIdx];
+//   int8 Aq[M*K+4], Bq[K*N+4], Bq2[N*N2+4]; int32 acc[M*N];
+//   float outRelu[M*N]      affine(A, W, bias), ReLU, scale 1
+//   float outSl[M*nIdx]     affine over the shortlist idx, no ReLU, scale 0.5
+//   float out2[M*N2]        affine(outRelu, W2), no bias
+//   float X[R*C], gamma[C], beta[C], ln[R*C] (eps 1e-6, skip input = X reversed), sm[R*C], lsm[R*C];
+//   float nbVal[R*nbestN]; uint32 nbKey[R*nbestN]     n-best of lsm
 #include <cmath>
 #include <cstring>
-#include <random>
+#include <fstream>
 
 #include "hip_int8_interface.h"
+#include "hip_ops_interface.h"
 
 using namespace marian::hip;
 
-static int8_t q1(float x, float qm) {
-  float v = x * qm;
-  float r = std::nearbyint(v);
-  r = std::fmin(std::fmax(r, -127.f), 127.f);
-  return (int8_t)r;
+namespace {
+
+struct Reader {
+  std::ifstream in;
+  explicit Reader(const char* path) : in(path, std::ios::binary) {
+    if(!in) abortWith(std::string("cannot open fixture ") + path);
+  }
+  template <typename T>
+  std::vector<T> take(size_t n) {
+    std::vector<T> v(n);
+    in.read(reinterpret_cast<char*>(v.data()), (std::streamsize)(n * sizeof(T)));
+    if(!in) abortWith("fixture is too short");
+    return v;
+  }
+};
+
+int failures = 0;
+void expect(bool ok, const char* what) {
+  std::printf("  %-74s %s\n", what, ok ? "ok" : "FAILED");
+  std::fflush(stdout);
+  if(!ok) ++failures;
 }
 
-int main() {
-  const int M = 24, K = 192, N = 72;
-  std::mt19937 gen(7);
-  std::normal_distribution<float> da(0.f, 1.f), dw(0.f, 0.02f), db(0.f, 0.01f);
-  std::vector<float> A(M * K), W(K * N), bias(N), out(M * N), want(M * N);
-  for(auto& v : A) v = da(gen);
-  for(auto& v : W) v = dw(gen);
-  for(auto& v : bias) v = db(gen);
+template <typename T>
+Tensor upload(TensorAllocator& ta, const std::vector<T>& host, const Shape& shape, Type type) {
+  Tensor t;
+  ta.allocate(t, shape, type);
+  copy(ta.backend().stream(), reinterpret_cast<const uint8_t*>(host.data()),
+       reinterpret_cast<const uint8_t*>(host.data()) + host.size() * sizeof(T), t.data<uint8_t>());
+  return t;
+}
 
-  Backend be(0);
-  Tensor a{nullptr, {M, K}, Type::float32}, w{nullptr, {K, N}, Type::float32};
-  Tensor aq{nullptr, {M, K}, Type::intgemm8}, bq{nullptr, {K, N}, Type::intgemm8};
-  Tensor b{nullptr, {1, N}, Type::float32}, o{nullptr, {M, N}, Type::float32};
-  HIP_CHECK(hipMalloc(&a.data, A.size() * 4));
-  HIP_CHECK(hipMalloc(&w.data, W.size() * 4));
-  HIP_CHECK(hipMalloc(&b.data, bias.size() * 4));
-  HIP_CHECK(hipMalloc(&o.data, out.size() * 4));
-  HIP_CHECK(hipMalloc(&aq.data, (requiredBytes(aq.shape, aq.type) + 255) / 256 * 256));
-  HIP_CHECK(hipMalloc(&bq.data, (requiredBytes(bq.shape, bq.type) + 255) / 256 * 256));
-  HIP_CHECK(hipMemcpy(a.data, A.data(), A.size() * 4, hipMemcpyHostToDevice));
-  HIP_CHECK(hipMemcpy(w.data, W.data(), W.size() * 4, hipMemcpyHostToDevice));
-  HIP_CHECK(hipMemcpy(b.data, bias.data(), bias.size() * 4, hipMemcpyHostToDevice));
-
-  integer::prepareB(be, w, bq);
-  integer::affineOrDot(be, a, aq, bq, &b, o, 1.0f, /*relu=*/true);
+template <typename T>
+std::vector<T> download(Backend& be, const Tensor& t, size_t n) {
+  std::vector<T> host(n);
   be.synchronize();
-  HIP_CHECK(hipMemcpy(out.data(), o.data, out.size() * 4, hipMemcpyDeviceToHost));
-  float aqm = integer::getQuantMult(be, aq), bqm = integer::getQuantMult(be, bq);
+  copy(be.stream(), t.data<T>(), t.data<T>() + n, host.data());
+  return host;
+}
 
-  float ma = 0.f, mw = 0.f;
-  for(float v : A) ma = std::fmax(ma, std::fabs(v));
-  for(float v : W) mw = std::fmax(mw, std::fabs(v));
-  const float qa = 127.0f / ma, qb = 127.0f / mw;
-  volatile float prod = qa * qb;
-  volatile float unq = 1.0f / prod;
-  int bad = 0;
-  for(int m = 0; m < M; ++m)
-    for(int n = 0; n < N; ++n) {
-      int32_t acc = 0;
-      for(int k = 0; k < K; ++k) acc += (int32_t)q1(A[m * K + k], qa) * (int32_t)q1(W[k * N + n], qb);
-      volatile float y = (float)acc * unq;
-      y = y + bias[n];
-      float r = y > 0.f ? y : 0.f;
-      if(r != out[m * N + n]) ++bad;
-    }
-  bool ok = bad == 0 && aqm == qa && bqm == qb;
+template <typename T>
+bool sameBits(const std::vector<T>& a, const std::vector<T>& b) {
+  return a.size() == b.size() && std::memcmp(a.data(), b.data(), a.size() * sizeof(T)) == 0;
+}
 
-  // error path: a CPU-tiled weight type must be refused with the reference's message
-  bool refused = false;
-  try {
-    Tensor tiled = bq;
-    tiled.type = Type::intgemm8avx512;
-    integer::affineOrDot(be, a, aq, tiled, &b, o);
-  } catch(const std::runtime_error& e) {
-    refused = std::strstr(e.what(), "Unsupported type") != nullptr;
+bool closeTo(const std::vector<float>& got, const std::vector<float>& want, double rel, double floor) {
+  if(got.size() != want.size()) return false;
+  for(size_t i = 0; i < got.size(); ++i)
+    if(!(std::fabs((double)got[i] - (double)want[i]) <= rel * std::fabs((double)want[i]) + floor)) return false;
+  return true;
+}
+
+// Allocates `bytes` more than the slab has free, so that the allocator must grow; returns whether
+// the slab moved.
+bool forceMove(TensorAllocator& ta, std::vector<Tensor>& ballast) {
+  const size_t before = ta.allocator()->device()->moves();
+  const uint8_t* base = ta.allocator()->device()->data();
+  Tensor t;
+  ta.allocate(t, {(int)(ta.allocator()->available() + 4096)}, Type::int8);
+  ballast.push_back(t);
+  return ta.allocator()->device()->moves() > before && ta.allocator()->device()->data() != base;
+}
+
+}  // namespace
+
+int main(int argc, char** argv) {
+  if(argc < 2) {
+    std::fprintf(stderr, "usage: host_check <fixture file>\n");
+    return 2;
   }
-  std::printf("host_check: mismatches %d, quantMult A %s B %s, tiled type refused %s -> %s\n", bad,
-              aqm == qa ? "ok" : "BAD", bqm == qb ? "ok" : "BAD", refused ? "yes" : "NO",
-              (ok && refused) ? "OK" : "FAILED");
-  return (ok && refused) ? 0 : 1;
+  try {
+    Reader rd(argv[1]);
+    auto magic = rd.take<char>(4);
+    if(std::memcmp(magic.data(), "MHC2", 4) != 0) abortWith("not a host_check fixture");
+    auto dims = rd.take<int32_t>(8);
+    const int M = dims[0], K = dims[1], N = dims[2], N2 = dims[3], nIdx = dims[4], R = dims[5], C = dims[6],
+              nbestN = dims[7];
+    auto A = rd.take<float>((size_t)M * K), W = rd.take<float>((size_t)K * N), bias = rd.take<float>(N),
+         W2 = rd.take<float>((size_t)N * N2);
+    auto idx = rd.take<uint32_t>(nIdx);
+    auto wantAq = rd.take<int8_t>((size_t)M * K + 4), wantBq = rd.take<int8_t>((size_t)K * N + 4),
+         wantBq2 = rd.take<int8_t>((size_t)N * N2 + 4);
+    auto wantAcc = rd.take<int32_t>((size_t)M * N);
+    auto wantRelu = rd.take<float>((size_t)M * N), wantSl = rd.take<float>((size_t)M * nIdx),
+         want2 = rd.take<float>((size_t)M * N2);
+    auto X = rd.take<float>((size_t)R * C), gamma = rd.take<float>(C), beta = rd.take<float>(C),
+         wantLn = rd.take<float>((size_t)R * C), wantSm = rd.take<float>((size_t)R * C),
+         wantLsm = rd.take<float>((size_t)R * C);
+    auto wantNbVal = rd.take<float>((size_t)R * nbestN);
+    auto wantNbKey = rd.take<uint32_t>((size_t)R * nbestN);
+
+    Backend be(0);
+    // a small step and a limit: growth happens often, and exhaustion can be provoked
+    const size_t kStep = 1u << 20, kLimit = 256u << 20;
+    TensorAllocator ta(be, kStep, kLimit);
+    std::vector<Tensor> ballast;
+    std::printf("host_check: M=%d K=%d N=%d N2=%d shortlist=%d, operators on %dx%d\n", M, K, N, N2, nIdx, R, C);
+
+    // ---- allocator on its own ----
+    {
+      Allocator& al = *ta.allocator();
+      expect(al.size() == 0 && al.available() == 0, "empty allocator: no slab yet");
+      auto p1 = al.alloc(100), p2 = al.alloc(256), p3 = al.alloc(257);
+      expect(al.size() == kStep && p1->size() == 256 && p2->size() == 256 && p3->size() == 512,
+             "first allocation grows the slab by one step; sizes round up to 256");
+      expect(((uintptr_t)p1->data() % 256) == 0 && p2->data() == p1->data() + 256 && p3->data() == p2->data() + 256,
+             "pieces are 256-byte aligned and packed");
+      expect(al.available() == kStep - 1024 && al.gaps() == 1, "one gap behind the pieces");
+      al.free(p2);
+      expect(al.gaps() == 2 && !p2->data(), "free leaves a gap and empties the handle");
+      auto p4 = al.alloc(200);
+      expect(p4->data() == p1->data() + 256 && al.gaps() == 1, "best fit: the freed 256 bytes are taken again");
+      al.free(p1);
+      al.free(p4);
+      expect(al.gaps() == 2, "neighbouring gaps merge (front)");
+      al.free(p3);
+      expect(al.gaps() == 1 && al.available() == al.size(), "all free: one gap, the whole slab");
+      auto q1 = al.alloc(1000);
+      const uint8_t* before = q1->data();
+      fill(be.stream(), q1->data<uint8_t>(), q1->data<uint8_t>() + 1000, (uint8_t)0x5A);
+      auto q2 = al.alloc(kStep);   // does not fit: grow = new slab + copy + free
+      std::vector<uint8_t> back(1000);
+      copy(be.stream(), (const uint8_t*)q1->data(), (const uint8_t*)q1->data() + 1000, back.data());
+      bool kept = true;
+      for(uint8_t b : back) kept = kept && b == 0x5A;
+      expect(al.device()->moves() == 1 && q1->data() != before && kept,
+             "grow moves the slab, re-points the pieces, keeps their bytes");
+      expect(al.size() == 2 * kStep && q2->size() == kStep, "grow adds max(step, request)");
+      al.throwAtReallocation(true);
+      bool threw = false;
+      try {
+        al.alloc(64u << 20);
+      } catch(const AllocationException&) {
+        threw = true;
+      }
+      al.throwAtReallocation(false);
+      expect(threw, "throwAtReallocation: AllocationException instead of growing");
+      bool refused = false;
+      try {
+        al.alloc(kLimit + 1);
+      } catch(const std::runtime_error& e) {
+        refused = std::strstr(e.what(), "Out of memory") != nullptr;
+      }
+      copy(be.stream(), (const uint8_t*)q1->data(), (const uint8_t*)q1->data() + 1000, back.data());
+      expect(refused && back[999] == 0x5A && al.size() == 2 * kStep,
+             "exhaustion is an error; slab and pieces survive it");
+      ta.clear();
+      expect(al.available() == al.size() && al.pieces() == 0 && !q1->data(), "clear forgets every piece");
+    }
+
+    // ---- fill and copy ----
+    {
+      Tensor f;
+      ta.allocate(f, {1031}, Type::float32);
+      fill(be.stream(), f.data<float>(), f.data<float>() + 1031, -1.0f);
+      fill(be.stream(), f.data<float>() + 3, f.data<float>() + 1030, 1.5f);   // unaligned start, ragged end
+      auto got = download<float>(be, f, 1031);
+      bool ok = got[0] == -1.0f && got[2] == -1.0f && got[1030] == -1.0f;
+      for(int i = 3; i < 1030; ++i) ok = ok && got[i] == 1.5f;
+      fill(be.stream(), f.data<int8_t>() + 1, f.data<int8_t>() + 38, (int8_t)-7);
+      fill(be.stream(), reinterpret_cast<uint16_t*>(f.data<int8_t>() + 40), reinterpret_cast<uint16_t*>(f.data<int8_t>() + 40) + 9, (uint16_t)0xBEEF);
+      fill(be.stream(), reinterpret_cast<uint64_t*>(f.data<int8_t>() + 64), reinterpret_cast<uint64_t*>(f.data<int8_t>() + 64) + 5, (uint64_t)0x0123456789ABCDEFull);
+      auto raw = download<uint8_t>(be, f, 128);
+      for(int i = 1; i < 38; ++i) ok = ok && raw[i] == (uint8_t)-7;
+      ok = ok && raw[0] == 0x00 && raw[38] == 0xC0;   // the bytes on either side (of -1.0f, of 1.5f) are untouched
+      for(int i = 0; i < 9; ++i) ok = ok && raw[40 + 2 * i] == 0xEF && raw[41 + 2 * i] == 0xBE;
+      for(int i = 0; i < 5; ++i) ok = ok && raw[64 + 8 * i] == 0xEF && raw[71 + 8 * i] == 0x01;
+      expect(ok, "fill: 1-, 2-, 4- and 8-byte elements, unaligned starts, ragged ends");
+      ta.free(f);
+    }
+
+    // ---- the int8 path, with the slab moving between the calls ----
+    Tensor a = upload(ta, A, {M, K}, Type::float32), w = upload(ta, W, {K, N}, Type::float32);
+    Tensor b = upload(ta, bias, {1, N}, Type::float32), w2 = upload(ta, W2, {N, N2}, Type::float32);
+    Tensor sl = upload(ta, idx, {nIdx}, Type::uint32);
+    Tensor aq, bq, bq2, acc, o, oSl, o2, aq2, omax;
+    ta.allocate(aq, {M, K}, Type::intgemm8);
+    ta.allocate(bq, {K, N}, Type::intgemm8);
+    ta.allocate(bq2, {N, N2}, Type::intgemm8);
+    ta.allocate(acc, {M, N}, Type::int32);
+    ta.allocate(o, {M, N}, Type::float32);
+    ta.allocate(oSl, {M, nIdx}, Type::float32);
+    ta.allocate(o2, {M, N2}, Type::float32);
+    ta.allocate(aq2, {M, N}, Type::intgemm8);
+    ta.allocate(omax, {MARIAN_HIP_ABSMAX_SLOTS}, Type::float32);
+
+    integer::prepareB(ta, w, bq);
+    integer::prepareB(ta, w2, bq2);
+    expect(sameBits(download<int8_t>(be, bq, wantBq.size()), wantBq) &&
+               sameBits(download<int8_t>(be, bq2, wantBq2.size()), wantBq2),
+           "prepareB: payload and quantMult as the checker's");
+    integer::prepareA(ta, a, aq);
+    const void* aqBefore = aq.data<void>();
+    expect(forceMove(ta, ballast) && aq.data<void>() != aqBefore, "slab moved between prepareA and multiply");
+    expect(sameBits(download<int8_t>(be, aq, wantAq.size()), wantAq), "prepareA: payload and quantMult, after the move");
+    integer::multiplyInt32(be, aq, bq, acc);
+    integer::multiply(be, aq, bq, &b, o, 1.0f, /*relu=*/true);
+    expect(sameBits(download<int32_t>(be, acc, wantAcc.size()), wantAcc), "multiply: int32 accumulators");
+    expect(sameBits(download<float>(be, o, wantRelu.size()), wantRelu), "multiply: bias + ReLU output, bit for bit");
+    float aqm = integer::getQuantMult(be, aq), wantAqm;
+    std::memcpy(&wantAqm, wantAq.data() + (size_t)M * K, 4);
+    expect(aqm == wantAqm, "getQuantMult reads the tail on the device");
+
+    fill(be.stream(), o.data<float>(), o.data<float>() + (size_t)M * N, 0.0f);
+    integer::affineOrDot(ta, a, aq, bq, &b, o, 1.0f, /*relu=*/true);
+    expect(sameBits(download<float>(be, o, wantRelu.size()), wantRelu), "affineOrDot: bias + ReLU output");
+    expect(forceMove(ta, ballast), "slab moved between two affineOrDot calls");
+    integer::affineOrDot(ta, a, aq, bq, &b, oSl, 0.5f, /*relu=*/false, &sl);
+    expect(sameBits(download<float>(be, oSl, wantSl.size()), wantSl), "affineOrDot over a shortlist, scale 0.5");
+    integer::multiply(be, aq, bq, &b, oSl, 0.5f, false, &sl);
+    expect(sameBits(download<float>(be, oSl, wantSl.size()), wantSl), "multiply over a shortlist");
+
+    // chained pair: the first call leaves the abs-max of its output, the second one takes it
+    integer::affineOrDot(ta, a, aq, bq, &b, o, 1.0f, true, nullptr, nullptr, &omax);
+    expect(forceMove(ta, ballast), "slab moved inside a chained pair");
+    integer::affineOrDot(ta, o, aq2, bq2, nullptr, o2, 1.0f, false, nullptr, &omax, nullptr);
+    expect(sameBits(download<float>(be, o2, want2.size()), want2), "chained affineOrDot (abs-max handed over)");
+    Tensor oStatic;
+    ta.allocate(oStatic, {M, N}, Type::float32);
+    integer::affineOrDotStatic(be, a, bq, &b, oStatic, 1.0f, true);
+    expect(sameBits(download<float>(be, oStatic, wantRelu.size()), wantRelu), "affineOrDotStatic (no Aq, no workspace)");
+
+    // error paths: the reference's messages, as exceptions
+    {
+      bool tiled = false, sixteen = false, notq = false;
+      Tensor t = bq;
+      t.type = Type::intgemm8avx512;
+      try { integer::affineOrDot(ta, a, aq, t, &b, o); } catch(const std::runtime_error& e) { tiled = std::strstr(e.what(), "Unsupported type") != nullptr; }
+      t.type = Type::intgemm16;
+      try { integer::affineOrDot(ta, a, aq, t, &b, o); } catch(const std::runtime_error& e) { sixteen = std::strstr(e.what(), "Unsupported type") != nullptr; }
+      t.type = Type::float32;
+      try { integer::affineOrDot(ta, a, aq, t, &b, o); } catch(const std::runtime_error& e) { notq = std::strstr(e.what(), "variant of intgemm") != nullptr; }
+      expect(tiled && sixteen && notq, "CPU-tiled, 16-bit and float weights are refused with the reference's texts");
+    }
+
+    // ---- float operators through their wrappers ----
+    {
+      std::vector<float> Xrev(X.rbegin(), X.rend());
+      Tensor x = upload(ta, X, {R, C}, Type::float32), xr = upload(ta, Xrev, {R, C}, Type::float32);
+      Tensor g = upload(ta, gamma, {C}, Type::float32), bt = upload(ta, beta, {C}, Type::float32);
+      Tensor ln, sm, lsm, nbV, nbK, nbV2, nbK2;
+      ta.allocate(ln, {R, C}, Type::float32);
+      ta.allocate(sm, {R, C}, Type::float32);
+      ta.allocate(lsm, {R, C}, Type::float32);
+      LayerNormalization(be, ln, x, g, &bt, 1e-6f, &xr);
+      Softmax(be, sm, x);
+      LogSoftmax(be, lsm, x);
+      expect(closeTo(download<float>(be, ln, wantLn.size()), wantLn, 2e-5, 4e-6), "LayerNormalization with skip input");
+      expect(closeTo(download<float>(be, sm, wantSm.size()), wantSm, 2e-5, 1e-7), "Softmax");
+      expect(closeTo(download<float>(be, lsm, wantLsm.size()), wantLsm, 2e-5, 4e-6), "LogSoftmax");
+      // n-best of the checker's log-probabilities (so that equal inputs decide, not rounding)
+      Tensor lsmRef = upload(ta, wantLsm, {R, C}, Type::float32);
+      NthElement nth(ta);
+      nth.getNBestList(lsmRef, nbestN, nbV, nbK);
+      expect(sameBits(download<float>(be, nbV, wantNbVal.size()), wantNbVal) &&
+                 sameBits(download<uint32_t>(be, nbK, wantNbKey.size()), wantNbKey),
+             "NthElement::getNBestList: scores and keys");
+      Tensor asBeams = lsmRef;   // the same rows seen as [beam 1, batch R, vocab C]
+      asBeams.shape = {1, R, C};
+      nth.getNBestListOfBeams(asBeams, nbestN, nbV2, nbK2);
+      expect(sameBits(download<float>(be, nbV2, wantNbVal.size()), wantNbVal) &&
+                 sameBits(download<uint32_t>(be, nbK2, wantNbKey.size()), wantNbKey),
+             "NthElement::getNBestListOfBeams: the same list");
+    }
+    be.synchronize();
+    std::printf("host_check: %d failure(s), slab moved %zu times -> %s\n", failures,
+                ta.allocator()->device()->moves(), failures == 0 ? "OK" : "FAILED");
+    return failures == 0 ? 0 : 1;
+  } catch(const std::exception& e) {
+    std::printf("host_check: exception: %s -> FAILED\n", e.what());
+    return 1;
+  }
 }

@@ -493,3 +493,63 @@ def test_nbest_when_one_thread_holds_the_best_elements(ops, synth, N):
     assert np.array_equal(vals.cpu().numpy().reshape(3, N), np.take_along_axis(flat, order, 1))
     assert np.array_equal(keys.cpu().numpy().view(np.uint32).reshape(3, N).astype(np.int64),
                           order + np.arange(3)[:, None] * flat.shape[1])
+
+
+# ---- the reference's own operator-test vectors (tests/golden/operator_vectors.json): at the
+#      margin the reference test allows, and at this file's own bar against float64 ----------------
+
+def reference_vectors():
+    import json
+    import os
+    return json.load(open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "operator_vectors.json")))
+
+
+def test_reference_softmax_logsoftmax_vectors(ops):
+    v = reference_vectors()["softmax_logsoftmax"]
+    x = np.array(v["in"], np.float32).reshape(v["shape"])
+    sm = ops.softmax(dev(x)).cpu().numpy()
+    lsm = ops.logsoftmax(dev(x)).cpu().numpy()
+    assert sm.shape == tuple(v["shape"]) and lsm.shape == tuple(v["shape"])
+    assert np.all(np.abs(sm.ravel() - np.array(v["softmax"])) <= v["margin"])
+    assert np.all(np.abs(lsm.ravel() - np.array(v["logsoftmax"])) <= v["margin"])
+    xs = x.astype(f64)
+    e = np.exp(xs - xs.max(-1, keepdims=True))
+    close(sm, e / e.sum(-1, keepdims=True), REL, 1e-7)
+    close(lsm, xs - xs.max(-1, keepdims=True) - np.log(e.sum(-1, keepdims=True)), REL, 1e-6)
+
+
+def test_reference_layer_norm_vector(ops):
+    v = reference_vectors()["layer_norm"]
+    x = np.array(v["in"], np.float32).reshape(v["shape"])
+    g, b = np.array(v["gamma"], np.float32), np.array(v["beta"], np.float32)
+    xs = x.astype(f64)
+    num = xs - xs.mean(-1, keepdims=True)
+    want = g.astype(f64) * (num / np.sqrt((num ** 2).mean(-1, keepdims=True) + v["eps"])) + b.astype(f64)
+    got = ops.layerNorm(dev(x), dev(g), dev(b), v["eps"]).cpu().numpy()
+    assert got.shape == tuple(v["shape"])
+    assert np.all(np.abs(got - want) <= v["margin"])
+    close(got, want, REL, 2e-6)
+
+
+def test_reference_bdot_vectors(ops):
+    v = reference_vectors()["bdot"]
+    A = np.array(v["A"], np.float32).reshape(v["A_shape"])
+    B = np.array(v["B"], np.float32).reshape(v["B_shape"])
+    C = np.array(v["C"], np.float32).reshape(v["C_shape"])
+    Ct = np.array(v["C_transB"], np.float32).reshape(v["C_shape"])
+    for i in range(2):   # (the legacy product pairs batch entries by modulo: entry i of A meets all of B)
+        assert np.array_equal(ops.bdot_legacy(dev(A[i]), dev(B[0])).cpu().numpy(), C[i])
+        assert np.array_equal(ops.bdot_legacy(dev(A[i]), dev(B[0]), transB=True).cpu().numpy(), Ct[i])
+
+
+def test_reference_topk_vectors(ops):
+    v = reference_vectors()["topk"]
+    x = np.array(v["in"], np.float32).reshape(-1, v["shape"][-1])
+    vals, keys = ops.getNBestList(dev(x), v["k"])
+    assert np.array_equal(vals.cpu().numpy(), np.array(v["values"], np.float32))
+    rows = np.repeat(np.arange(x.shape[0]), v["k"])
+    assert np.array_equal(keys.cpu().numpy().astype(np.int64) - rows * x.shape[1], np.array(v["indices"]))
+    # the same rows as the beam-major form sees them: beam 1, batch 4, vocabulary 3
+    vals2, keys2 = ops.getNBestListOfBeams(dev(x.reshape(1, 1, 4, 3)), v["k"])
+    assert np.array_equal(vals2.cpu().numpy(), vals.cpu().numpy())
+    assert np.array_equal(keys2.cpu().numpy(), keys.cpu().numpy())

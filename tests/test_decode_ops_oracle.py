@@ -132,3 +132,51 @@ def test_nbest_against_full_sort(ops):
     t[0, [7, 2, 5]] = 1.0
     v, k = ops.nbest(t, 4)
     assert k.tolist() == [2, 5, 7, 0] and v.tolist() == [1.0, 1.0, 1.0, 0.0]
+
+
+# ---- the reference's own operator-test vectors (tests/golden/operator_vectors.json) -------------
+
+def reference_vectors():
+    import json
+    import os
+    return json.load(open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "operator_vectors.json")))
+
+
+def test_reference_softmax_logsoftmax_vectors(ops):
+    v = reference_vectors()["softmax_logsoftmax"]
+    x = np.array(v["in"], np.float32).reshape(v["shape"])
+    assert np.all(np.abs(ops.softmax(x).ravel() - np.array(v["softmax"])) <= v["margin"])
+    assert np.all(np.abs(ops.logsoftmax(x).ravel() - np.array(v["logsoftmax"])) <= v["margin"])
+
+
+def test_reference_layer_norm_vector(ops):
+    v = reference_vectors()["layer_norm"]
+    x = np.array(v["in"], np.float32).reshape(v["shape"])
+    g, b = np.array(v["gamma"], np.float32), np.array(v["beta"], np.float32)
+    xs = x.astype(f64)
+    num = xs - xs.mean(-1, keepdims=True)
+    want = g.astype(f64) * (num / np.sqrt((num ** 2).mean(-1, keepdims=True) + v["eps"])) + b.astype(f64)
+    got = ops.layer_norm(x, g, b, v["eps"])
+    assert np.all(np.abs(got - want) <= v["margin"]) and close(got, want, 5e-6, 5e-6)
+
+
+def test_reference_bdot_vectors(ops):
+    """bdot broadcasts [2,1] x [1,3] batches; the legacy batched product pairs batch entries by
+    modulo (reference src/tensors/cpu/prod.cpp:233-330), so entry i of A meets all of B in a call."""
+    v = reference_vectors()["bdot"]
+    A = np.array(v["A"], np.float32).reshape(v["A_shape"])
+    B = np.array(v["B"], np.float32).reshape(v["B_shape"])
+    C = np.array(v["C"], np.float32).reshape(v["C_shape"])
+    Ct = np.array(v["C_transB"], np.float32).reshape(v["C_shape"])
+    for i in range(2):
+        assert np.array_equal(ops.bdot_legacy(A[i], B[0]), C[i])
+        assert np.array_equal(ops.bdot_legacy(A[i], B[0], transB=True), Ct[i])
+
+
+def test_reference_topk_vectors(ops):
+    v = reference_vectors()["topk"]
+    x = np.array(v["in"], np.float32).reshape(-1, v["shape"][-1])
+    vals, keys = ops.nbest(x, v["k"])
+    assert np.array_equal(vals, np.array(v["values"], np.float32))
+    rows = np.repeat(np.arange(x.shape[0]), v["k"])
+    assert np.array_equal(keys - rows * x.shape[1], np.array(v["indices"], np.uint32))

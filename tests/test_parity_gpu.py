@@ -639,14 +639,50 @@ def test_model_file_weights_run_verbatim(integer, orc, synth, tmp_path):
     assert np.array_equal(got, want)
 
 
-def test_cpp_host_wrappers(integer):
-    """The C++ mirror of the intgemm glue (host/hip_int8_interface.h) against its own CPU
-    restatement; built by __graft_entry__.build()."""
+def write_host_check_fixture(path, orc, synth):
+    """Inputs and the CPU checker's expected values for marian-dev_amd/host/host_check.cpp (layout in
+    that file's header)."""
+    from oracle import decode_ops
+    M, K, N, N2, R, C, nbestN = 24, 192, 128, 40, 6, 520, 4   # (N is the K of the chained second call)
+    A = synth.normal(7, synth.STREAM_A, (M, K), 1.0)
+    W = synth.normal(7, synth.STREAM_W, (K, N), 0.02)
+    bias = synth.normal(7, synth.STREAM_BIAS, (N,), 0.01)
+    W2 = synth.normal(8, synth.STREAM_W, (N, N2), 0.02)
+    idx = np.sort(np.random.default_rng(7).choice(N, size=16, replace=False)).astype(np.uint32)
+    Aq, Bq, Bq2 = orc.prepare_a(A), orc.prepare_b(W), orc.prepare_b(W2)
+    out_relu, acc = orc.affine(Aq, Bq, bias, M, K, N, 1.0, True)
+    out_sl, _ = orc.affine_shortlist(Aq, Bq, bias, idx, M, K, N, 0.5, False)
+    out2, _ = orc.affine(orc.prepare_a(out_relu), Bq2, None, M, N, N2, 1.0, False)
+    X = synth.normal(9, synth.STREAM_A, (R, C), 2.0)
+    gamma = synth.normal(9, synth.STREAM_W, (C,), 0.2) + f32(1.0)
+    beta = synth.normal(9, synth.STREAM_BIAS, (C,), 0.5)
+    Xrev = np.ascontiguousarray(X.ravel()[::-1].reshape(R, C))
+    ln = decode_ops.layer_norm(X, gamma, beta, 1e-6, add=Xrev)
+    sm, lsm = decode_ops.softmax(X), decode_ops.logsoftmax(X)
+    nb_val, nb_key = decode_ops.nbest(lsm, nbestN)
+    with open(path, "wb") as f:
+        f.write(b"MHC2")
+        f.write(np.array([M, K, N, N2, idx.size, R, C, nbestN], np.int32).tobytes())
+        for arr, ty in [(A, f32), (W, f32), (bias, f32), (W2, f32), (idx, np.uint32), (Aq, np.int8), (Bq, np.int8),
+                        (Bq2, np.int8), (acc, np.int32), (out_relu, f32), (out_sl, f32), (out2, f32), (X, f32),
+                        (gamma, f32), (beta, f32), (ln, f32), (sm, f32), (lsm, f32), (nb_val, f32),
+                        (nb_key, np.uint32)]:
+            f.write(np.ascontiguousarray(arr, dtype=ty).tobytes())
+
+
+def test_cpp_host_side(integer, orc, synth, tmp_path):
+    """The C++ host side (host/hip_device.h: Device, Allocator, TensorAllocator, copy, fill;
+    host/hip_int8_interface.h and host/hip_ops_interface.h: the operator wrappers) on the GPU, every
+    buffer carved from the allocator, whose slab is forced to move between prepareA and multiply,
+    between two affineOrDot calls and inside a chained pair; results against the CPU checker's
+    values handed over in a fixture file.  Built by __graft_entry__.build()."""
     import subprocess
     from conftest import ROOT
     exe = os.path.join(ROOT, "marian-dev_amd", "host", "host_check")
     assert os.path.exists(exe), "host_check not built"
     say("host_check")
-    r = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=120)
+    fixture = os.path.join(tmp_path, "host_check.fixture")
+    write_host_check_fixture(fixture, orc, synth)
+    r = subprocess.run([exe, fixture], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=120)
     print(r.stdout)
-    assert r.returncode == 0 and "-> OK" in r.stdout, r.stdout
+    assert r.returncode == 0 and "-> OK" in r.stdout and "FAILED" not in r.stdout, r.stdout
