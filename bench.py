@@ -157,9 +157,11 @@ class BigDecoder:
         lens = torch.randint(20, self.L + 1, (self.batch,), device="cuda", generator=g)
         self.mask = (torch.arange(self.L, device="cuda")[None, :] >= lens[:, None]).float() * -99999999.0
 
-    def step(self, s, gemm_only=False, chained=True):
+    def step(self, s, gemm_only=False, chained=True, grouped=True):
         """chained: every tensor that feeds an affine call leaves its abs-max where it is
-        produced (layer norm, attention, the ReLU GEMM), so those calls skip their abs-max pass."""
+        produced (layer norm, attention, the ReLU GEMM), so those calls skip their abs-max pass.
+        grouped: the self-attention projections Wq, Wk, Wv (one input, three weight matrices,
+        reference src/models/transformer.h:290-325) go through one call."""
         integer, ops = self.integer, self.ops
         W = self.sets[s % len(self.sets)]
         H, M, d = self.H, self.M, self.d
@@ -167,9 +169,12 @@ class BigDecoder:
         x, xmax = self.x, None
         ch = chained and not gemm_only
         for li, ly in enumerate(W["layers"]):
-            q, _ = integer.affine_f32(x, *ly["Wq"], absmax=xmax)
-            k, _ = integer.affine_f32(x, *ly["Wk"], absmax=xmax)
-            v, _ = integer.affine_f32(x, *ly["Wv"], absmax=xmax)
+            if grouped:   # one abs-max, one quantization, one launch for the three projections
+                (q, k, v), _ = integer.affine_f32_grouped(x, [ly["Wq"], ly["Wk"], ly["Wv"]], absmax=xmax)
+            else:
+                q, _ = integer.affine_f32(x, *ly["Wq"], absmax=xmax)
+                k, _ = integer.affine_f32(x, *ly["Wk"], absmax=xmax)
+                v, _ = integer.affine_f32(x, *ly["Wv"], absmax=xmax)
             omax = x1max = comax = x2max = f1max = None
             if gemm_only:
                 o = q

@@ -132,6 +132,25 @@ int marian_hip_int8_affine_f32_chained(const float* A, int8_t* Aq, const int8_t*
                                        void* workspace, size_t workspace_bytes, void* stream);
 
 /*
+ * One activation tensor, several weight matrices, one call: the self-attention projections of a
+ * transformer layer read the same input through three separate weight matrices with three
+ * quantMults (reference src/models/transformer.h:290-325: Wq, Wk, Wv), which in the reference is
+ * three affine nodes, each with its own prepareA node over the same tensor
+ * (src/tensors/cpu/intgemm_interface.h:52).  Here max|A| is taken once, A is quantized once (Aq and
+ * its tail are written once) and, for decode-size activations, one kernel multiplies it by all the
+ * matrices.  out[g] is what marian_hip_int8_affine_f32(A, Aq, Bq[g], bias[g], NULL, 0, out[g], M, K,
+ * N[g], scale, relu, ...) writes, bit for bit.
+ *   Bq, bias, out, N: HOST arrays of n_groups (1 .. 4) entries, read during the call; their
+ *   entries are device pointers / column counts.  bias may be NULL, and so may any bias[g].
+ *   absmax_in: as for marian_hip_int8_affine_f32_chained, or NULL.
+ */
+int marian_hip_int8_affine_f32_grouped(const float* A, int8_t* Aq, int64_t n_groups,
+                                       const int8_t* const* Bq, const float* const* bias,
+                                       float* const* out, const int64_t* N, int64_t M, int64_t K,
+                                       float scale, int relu, const float* absmax_in, void* workspace,
+                                       size_t workspace_bytes, void* stream);
+
+/*
  * marian_hip_int8_affine_f32 for callers that cannot allocate and have no workspace to pass: code
  * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no
  * counterpart in the reference (there the prepareA node's output and every temporary come from the

@@ -200,8 +200,15 @@ struct FusedSrc {   // what the fused modes read and write besides GemmArgs
   int n_partials = 0;
 };
 
+// Several weight matrices behind one activation tensor: the table the kernel reads, built for
+// `cols` output columns per workgroup.
+struct GroupLaunch {
+  GroupTable table;
+  int cols;
+};
+
 template <int MT32, int WN, int KW, int PW, int MODE, int ROWS = 32 * MT32, int NG = 4>
-int launch_stream32(const GemmArgs& a, const FusedSrc& f, hipStream_t st) {
+int launch_stream32(const GemmArgs& a, const FusedSrc& f, hipStream_t st, const GroupLaunch* groups = nullptr) {
   if constexpr(MODE == kFusedAll && NG == 4) {   // at most two groups of 16 values per thread
     if((long long)a.M * a.K <= kFusedMaxElems / 2)
       return launch_stream32<MT32, WN, KW, PW, MODE, ROWS, 2>(a, f, st);
@@ -219,6 +226,21 @@ int launch_stream32(const GemmArgs& a, const FusedSrc& f, hipStream_t st) {
   int blocks = (a.n_out + Cfg::kColsPerBlock - 1) / Cfg::kColsPerBlock;
   int m_tiles = (a.M + ROWS - 1) / ROWS;   // (kFusedAll with full-height tiles: M <= ROWS)
   GemmArgs a2 = a;
+  if constexpr(MODE == kFusedTiled) {
+    if(groups) {
+      if(groups->cols != Cfg::kColsPerBlock) return MARIAN_HIP_ERR_SHAPE;   // (table built for another kernel)
+      auto gkernel = gemm_stream32_kernel<MT32, WN, KW, PW, MODE, NG, ROWS, GroupTable>;
+      static std::atomic<uint64_t> glds_done{0};
+      const int glds_status = allow_lds(gkernel, kMaxLds, glds_done);
+      if(glds_status != MARIAN_HIP_OK) return glds_status;
+      a2.stream_out = 0;
+      a2.absmax_out = nullptr;
+      hipLaunchKernelGGL(gkernel, dim3(groups->table.block0[groups->table.n], m_tiles), dim3(Cfg::kThreads), lds, st,
+                         a2, f.A, f.aq_out, f.partials, f.n_partials, groups->table);
+      MH_HIP(hipGetLastError());
+      return MARIAN_HIP_OK;
+    }
+  }
   // (measured: 10.0 instead of 11.1 us for the 8 MB output of the 64 x 32000 call; outputs of
   // less than a MB are up to 0.5 us slower with them.  The next kernel then finds the output in
   // HBM rather than in the memory-side cache: a log-softmax over 16 MB of logits takes 14.1
@@ -229,7 +251,7 @@ int launch_stream32(const GemmArgs& a, const FusedSrc& f, hipStream_t st) {
     else a2.absmax_out = nullptr;
   }
   hipLaunchKernelGGL(kernel, dim3(blocks, m_tiles), dim3(Cfg::kThreads), lds, st, a2, f.A,
-                     f.aq_out, f.partials, f.n_partials);
+                     f.aq_out, f.partials, f.n_partials, NoGroups());
   MH_HIP(hipGetLastError());
   return MARIAN_HIP_OK;
 }
@@ -238,27 +260,28 @@ int launch_stream32(const GemmArgs& a, const FusedSrc& f, hipStream_t st) {
 // covers K in one chunk, else the largest whose activations fit the 64 KB LDS stage
 // (MT32 * KW * PW <= 64).  kFusedTiled stages fp32 values in registers: at most 4 per wave (8 when K is not split).
 template <int MT32, int MODE>
-int launch_stream32_kw(const GemmArgs& a, const FusedSrc& f, hipStream_t st, int kw, bool half_rows = false) {
+int launch_stream32_kw(const GemmArgs& a, const FusedSrc& f, hipStream_t st, int kw, bool half_rows = false,
+                       const GroupLaunch* g = nullptr) {
   const int need = (a.K / 32 + kw - 1) / kw;   // sub-steps per wave if K is one chunk
   if constexpr(MODE == kFusedTiled) {
     static_assert(MT32 == 1, "tiled fused form: 32 (or 16) rows per workgroup");
     switch(kw) {
-      case 1: return launch_stream32<1, 8, 1, 8, MODE>(a, f, st);
-      case 2: return launch_stream32<1, 4, 2, 4, MODE>(a, f, st);
+      case 1: return launch_stream32<1, 8, 1, 8, MODE>(a, f, st, g);
+      case 2: return launch_stream32<1, 4, 2, 4, MODE>(a, f, st, g);
       case 4:
-        if(half_rows) return launch_stream32<1, 2, 4, 4, MODE, 16>(a, f, st);
+        if(half_rows) return launch_stream32<1, 2, 4, 4, MODE, 16>(a, f, st, g);
         if(need > 4 && kernel_override() % 1000 != 690)
-          return launch_stream32<1, 2, 4, 8, MODE>(a, f, st);   // long rows: half as many chunks (measurement id 690 keeps the shorter ones)
-        return launch_stream32<1, 2, 4, 4, MODE>(a, f, st);
+          return launch_stream32<1, 2, 4, 8, MODE>(a, f, st, g);   // long rows: half as many chunks (measurement id 690 keeps the shorter ones)
+        return launch_stream32<1, 2, 4, 4, MODE>(a, f, st, g);
       default:
         if(need > 4 && half_rows && kernel_override() % 1000 != 670)
-          return launch_stream32<1, 1, 8, 8, MODE, 16>(a, f, st);   // long rows: half as many chunks (measurement id 670 keeps the shorter ones)
+          return launch_stream32<1, 1, 8, 8, MODE, 16>(a, f, st, g);   // long rows: half as many chunks (measurement id 670 keeps the shorter ones)
         if(need > 2) {
-          if(half_rows) return launch_stream32<1, 1, 8, 4, MODE, 16>(a, f, st);
-          return launch_stream32<1, 1, 8, 4, MODE>(a, f, st);
+          if(half_rows) return launch_stream32<1, 1, 8, 4, MODE, 16>(a, f, st, g);
+          return launch_stream32<1, 1, 8, 4, MODE>(a, f, st, g);
         }
-        if(half_rows) return launch_stream32<1, 1, 8, 2, MODE, 16>(a, f, st);
-        return launch_stream32<1, 1, 8, 2, MODE>(a, f, st);
+        if(half_rows) return launch_stream32<1, 1, 8, 2, MODE, 16>(a, f, st, g);
+        return launch_stream32<1, 1, 8, 2, MODE>(a, f, st, g);
     }
   } else {
     switch(kw) {
@@ -745,6 +768,93 @@ int marian_hip_int8_affine_f32_chained(const float* A, int8_t* Aq, const int8_t*
   return absmax_after(out, M, n_out, absmax_out, reinterpret_cast<hipStream_t>(stream));
 }
 
+
+int marian_hip_int8_affine_f32_grouped(const float* A, int8_t* Aq, int64_t n_groups,
+                                       const int8_t* const* Bq, const float* const* bias,
+                                       float* const* out, const int64_t* N, int64_t M, int64_t K,
+                                       float scale, int relu, const float* absmax_in, void* workspace,
+                                       size_t workspace_bytes, void* stream) {
+  if(n_groups < 1 || n_groups > kMaxGroups) return MARIAN_HIP_ERR_SHAPE;
+  if(!Bq || !out || !N) return MARIAN_HIP_ERR_NULL;
+  int64_t total_blocks32 = 0;
+  for(int64_t g = 0; g < n_groups; ++g) {
+    int st = check_gemm(Aq, Bq[g], out[g], bias ? bias[g] : nullptr, nullptr, 0, M, K, N[g]);
+    if(st != MARIAN_HIP_OK) return st;
+    total_blocks32 += (N[g] + 31) / 32;
+  }
+  if(absmax_in && !aligned(absmax_in, 4)) return MARIAN_HIP_ERR_ALIGN;
+  if(M == 0) return MARIAN_HIP_OK;
+  if(!A || !Aq) return MARIAN_HIP_ERR_NULL;
+  if(!aligned(A, 16)) return MARIAN_HIP_ERR_ALIGN;
+  hipStream_t hst = reinterpret_cast<hipStream_t>(stream);
+  const bool have_ws = workspace && workspace_bytes >= kWorkspaceBytes && aligned(workspace, 4);
+  // One launch for all matrices where the quantize-on-stage kernel takes the call (the same limits
+  // as for a single matrix of the summed width).
+  bool one_launch = false;
+  TiledPlan plan{1, false};
+  if(total_blocks32 > 0 && (absmax_in || have_ws) && M <= 256 && total_blocks32 * 32 <= 8192) {
+    plan = plan_tiled((int)M, (int)K, (int)(total_blocks32 * 32), 0);
+    one_launch = K <= 1024 || (K <= 4096 && plan.kw == 8 && (long long)(plan.half_rows ? 16 : 32) * K <= 65536);
+  }
+  if(one_launch) {
+    GroupLaunch gl;
+    gl.cols = 32 * (8 / plan.kw);
+    gl.table.n = 0;
+    gl.table.block0[0] = 0;
+    for(int64_t g = 0; g < n_groups; ++g) {
+      if(N[g] == 0) continue;
+      const int i = gl.table.n++;
+      gl.table.Bq[i] = Bq[g];
+      gl.table.bias[i] = bias ? bias[g] : nullptr;
+      gl.table.out[i] = out[g];
+      gl.table.N[i] = (int)N[g];
+      gl.table.block0[i + 1] = gl.table.block0[i] + (int)((N[g] + gl.cols - 1) / gl.cols);
+    }
+    for(int i = gl.table.n; i < kMaxGroups; ++i) {   // unused entries: never selected
+      gl.table.Bq[i] = nullptr; gl.table.bias[i] = nullptr; gl.table.out[i] = nullptr; gl.table.N[i] = 0;
+      gl.table.block0[i + 1] = gl.table.block0[gl.table.n];
+    }
+    GemmArgs a;
+    a.Aq = Aq; a.Bq = gl.table.Bq[0]; a.bias = gl.table.bias[0]; a.idx = nullptr; a.out = gl.table.out[0];
+    a.M = (int)M; a.K = (int)K; a.N = gl.table.N[0]; a.n_out = gl.table.N[0];
+    a.scale = scale; a.relu = relu ? 1 : 0; a.dump = 0;
+#ifdef MARIAN_HIP_TUNING
+    a.prof = g_prof.load(std::memory_order_relaxed);
+#endif
+    FusedSrc f;
+    f.A = A; f.aq_out = Aq;
+    if(absmax_in) {
+      f.partials = absmax_in;
+      f.n_partials = kAbsmaxSlots;
+    } else {
+      const size_t n = (size_t)M * (size_t)K;
+      float* partials = reinterpret_cast<float*>(workspace);
+      const int g = absmax_blocks(n / 4);
+      hipLaunchKernelGGL(absmax_partial_kernel, dim3(g), dim3(kQuantThreads), 0, hst, A, n / 4, partials);
+      MH_HIP(hipGetLastError());
+      f.partials = partials;
+      f.n_partials = g;
+    }
+    return launch_stream32_kw<1, kFusedTiled>(a, f, hst, plan.kw, plan.half_rows, &gl);
+  }
+  // Otherwise the activations are quantized once and every matrix gets its own multiplication.
+  if(absmax_in) {
+    const size_t n = (size_t)M * (size_t)K;
+    size_t qblocks = (n / 16 + kQuantThreads - 1) / kQuantThreads;
+    if(qblocks > 4096) qblocks = 4096;
+    hipLaunchKernelGGL(quantize_a_kernel, dim3((int)qblocks), dim3(kQuantThreads), 0, hst, A, n / 16, absmax_in,
+                       (int)kAbsmaxSlots, Aq);
+    MH_HIP(hipGetLastError());
+  } else {
+    int st = marian_hip_int8_prepare_a(A, Aq, M, K, workspace, workspace_bytes, stream);
+    if(st != MARIAN_HIP_OK) return st;
+  }
+  for(int64_t g = 0; g < n_groups; ++g) {
+    int st = run_gemm(Aq, Bq[g], bias ? bias[g] : nullptr, nullptr, 0, out[g], M, K, N[g], scale, relu, 0, stream);
+    if(st != MARIAN_HIP_OK) return st;
+  }
+  return MARIAN_HIP_OK;
+}
 
 // ---- the entry point that allocates nothing -------------------------------------------------
 // Device memory the call needs besides its inputs and outputs - the quantized activations with

@@ -59,6 +59,20 @@ struct Stream32Cfg {
   static_assert(CS % 2 == 0, "a quad of lanes quantizes four 16-byte chunks of one row");
 };
 
+// Several weight matrices behind one activation tensor (kFusedTiled only): the grid's columns are
+// the matrices' column blocks one after the other, and a workgroup takes weights, bias, output and
+// width from the entry its block index falls into (block0[g] <= blockIdx.x < block0[g + 1]).
+constexpr int kMaxGroups = 4;
+struct GroupTable {
+  const int8_t* Bq[kMaxGroups];
+  const float* bias[kMaxGroups];
+  void* out[kMaxGroups];
+  int N[kMaxGroups];
+  int block0[kMaxGroups + 1];
+  int n;
+};
+struct NoGroups {};
+
 // Dynamic LDS: one chunk (kStageBytes), for kFusedAll all of K (32 * MT32 * K bytes) if that is
 // more; at least kReduceBytes.  partials: n_partials (1..2048) abs-max values (kFusedTiled only).
 // NG (kFusedAll): 16-value groups per thread that are compiled in, 2 or 4; all but the last two are
@@ -68,13 +82,28 @@ struct Stream32Cfg {
 // quantizing per workgroup and twice the workgroups, for calls that would otherwise leave most
 // CUs idle.  With ROWS < M the kFusedAll form still takes the abs-max over all of A in every
 // workgroup and quantizes only its own rows.
-template <int MT32, int WN, int KW, int PW, int MODE, int NG = 4, int ROWS = 32 * MT32>
+template <int MT32, int WN, int KW, int PW, int MODE, int NG = 4, int ROWS = 32 * MT32, typename GROUPS = NoGroups>
 __global__ __launch_bounds__(WN * KW * kWave) void gemm_stream32_kernel(GemmArgs args,
                                                                         const float* A,
                                                                         int8_t* aq_out,
                                                                         const float* partials,
-                                                                        int n_partials) {
+                                                                        int n_partials, GROUPS groups) {
   using Cfg = Stream32Cfg<MT32, WN, KW, PW>;
+  constexpr bool GROUPED = std::is_same<GROUPS, GroupTable>::value;
+  static_assert(!GROUPED || MODE == kFusedTiled, "several weight matrices: quantize-on-stage form only");
+  int bx = blockIdx.x, gx = gridDim.x;   // column block within this workgroup's matrix, and how many it has
+  if constexpr(GROUPED) {
+    int g = 0;
+#pragma unroll
+    for(int i = 1; i < kMaxGroups; ++i)
+      if(i < groups.n && bx >= groups.block0[i]) g = i;
+    args.Bq = groups.Bq[g];
+    args.bias = groups.bias[g];
+    args.out = groups.out[g];
+    args.N = args.n_out = groups.N[g];
+    gx = groups.block0[g + 1] - groups.block0[g];
+    bx -= groups.block0[g];
+  }
   constexpr int kStream32Waves = Cfg::kWaves, kStream32Threads = Cfg::kThreads;
   constexpr bool TILED_ = MODE == kFusedTiled;
   constexpr int kFusedGroups = NG, kFullGroups = NG - 2;
@@ -113,7 +142,7 @@ __global__ __launch_bounds__(WN * KW * kWave) void gemm_stream32_kernel(GemmArgs
 
   // ---- weight row of this lane and where the bias of the four columns this lane will write
   //      sits (see the epilogue), both through the shortlist ids when there are any ----
-  const int n0 = (blockIdx.x * WN + wn) * 32;
+  const int n0 = (bx * WN + wn) * 32;
   int wsrc = min(n0 + li, args.n_out - 1);
   const int bias_n = min(n0 + 4 * (lane % 8), args.n_out - 4);   // n_out % 8 == 0: four valid columns
   uint32_t bias_at[4];
@@ -495,7 +524,7 @@ __global__ __launch_bounds__(WN * KW * kWave) void gemm_stream32_kernel(GemmArgs
   if(args.absmax_out && !args.dump) {
     // slot (workgroup, wave) takes this wave's maximum; workgroup 0 zeroes the slots nobody owns
     // (the launcher made sure that 8 slots per workgroup fit)
-    const int block = blockIdx.y * gridDim.x + blockIdx.x, used = gridDim.x * gridDim.y * kStream32Waves;
+    const int block = blockIdx.y * gx + bx, used = gx * gridDim.y * kStream32Waves;
     omax = wave_max(omax);
     if(lane == 0) args.absmax_out[block * kStream32Waves + wave] = omax;
     if(block == 0)

@@ -236,6 +236,35 @@ inline void affineOrDot(TensorAllocator& ta, const Tensor& a, Tensor& aQuant, co
         ta.workspaceBytes(), ta.backend().stream()));
 }
 
+// One activation tensor through several weight matrices (the self-attention projections Wq, Wk, Wv
+// of src/models/transformer.h:290-325): one abs-max, one quantization, for decode sizes one launch.
+// outs[g] is what affineOrDot(a, aQuant, *bQuants[g], biases[g], *outs[g], scale, relu) writes.
+inline void affineOrDotGrouped(TensorAllocator& ta, const Tensor& a, Tensor& aQuant,
+                               const std::vector<const Tensor*>& bQuants, const std::vector<const Tensor*>& biases,
+                               const std::vector<Tensor*>& outs, float scale = 1.f, bool relu = false,
+                               const Tensor* absmaxIn = nullptr) {
+  if(!isFloat(a.type)) abortWith("Intgemm expects type of A to be float32");
+  if(bQuants.empty() || bQuants.size() > 4 || outs.size() != bQuants.size() ||
+     (!biases.empty() && biases.size() != bQuants.size()))
+    abortWith("affineOrDotGrouped: between one and four weight matrices, one output (and bias entry) each");
+  void* ws = ta.workspace();   // (may allocate and move the slab: before any pointer is read)
+  std::vector<const int8_t*> bq(bQuants.size());
+  std::vector<const float*> bi(bQuants.size(), nullptr);
+  std::vector<float*> o(bQuants.size());
+  std::vector<int64_t> n(bQuants.size());
+  for(size_t g = 0; g < bQuants.size(); ++g) {
+    checkB(*bQuants[g]);
+    bq[g] = bQuants[g]->data<int8_t>();
+    if(!biases.empty() && biases[g]) bi[g] = biases[g]->data<float>();
+    o[g] = outs[g]->data<float>();
+    n[g] = cols(*bQuants[g]);
+  }
+  MARIAN_HIP_CHECK(marian_hip_int8_affine_f32_grouped(
+      a.data<float>(), aQuant.data<int8_t>(), (int64_t)bq.size(), bq.data(), bi.data(), o.data(), n.data(), rows(a),
+      cols(a), scale, relu ? 1 : 0, absmaxIn ? absmaxIn->data<float>() : nullptr, ws, ta.workspaceBytes(),
+      ta.backend().stream()));
+}
+
 // The same for callers that cannot allocate: no aQuant tensor, no workspace (the library's static
 // scratch holds both; rows(a) * cols(a) <= MARIAN_HIP_STATIC_MAX_ELEMS).
 inline void affineOrDotStatic(Backend& be, const Tensor& a, const Tensor& bQuant, const Tensor* bias,

@@ -244,6 +244,16 @@ int main(int argc, char** argv) {
     expect(forceMove(ta, ballast), "slab moved inside a chained pair");
     integer::affineOrDot(ta, o, aq2, bq2, nullptr, o2, 1.0f, false, nullptr, &omax, nullptr);
     expect(sameBits(download<float>(be, o2, want2.size()), want2), "chained affineOrDot (abs-max handed over)");
+    {   // two matrices behind one input in one call: the outputs of the separate calls
+      Tensor g1, g2;
+      ta.allocate(g1, {M, N}, Type::float32);
+      ta.allocate(g2, {M, N}, Type::float32);
+      integer::affineOrDotGrouped(ta, a, aq, {&bq, &bq}, {&b, nullptr}, {&g1, &g2}, 1.0f, true);
+      integer::multiply(be, aq, bq, nullptr, o, 1.0f, true);
+      expect(sameBits(download<float>(be, g1, wantRelu.size()), wantRelu) &&
+                 sameBits(download<float>(be, g2, wantRelu.size()), download<float>(be, o, wantRelu.size())),
+             "affineOrDotGrouped: both outputs as the separate calls'");
+    }
     Tensor oStatic;
     ta.allocate(oStatic, {M, N}, Type::float32);
     integer::affineOrDotStatic(be, a, bq, &b, oStatic, 1.0f, true);

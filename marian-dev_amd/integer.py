@@ -265,6 +265,44 @@ def affine_f32(a, bQuant, bias=None, scale=1.0, relu=False, shortlist=None, absm
     return (out, aQuant, omax) if want_absmax else (out, aQuant)
 
 
+def affine_f32_grouped(a, weights, scale=1.0, relu=False, absmax=None):
+    """One activation tensor through several weight matrices in one call
+    (marian_hip_int8_affine_f32_grouped): the self-attention projections Wq, Wk, Wv of reference
+    src/models/transformer.h:290-325 read the same input.  weights: list of (bQuant, bias or None).
+    Returns ([out, ...], aQuant); each out equals affine_f32(a, bQuant, bias)[0] bit for bit."""
+    import ctypes
+    a = a.contiguous()
+    be = _backend_of(a)
+    K = cols(a)
+    M = rows(a) if a.numel() else 0
+    n = len(weights)
+    _abort_if(n < 1 or n > 4, "between one and four weight matrices per call, got {}", n)
+    aQuant = QTensor.empty(a.shape, Type.intgemm8, a.device)
+    outs, keep = [], []
+    Bq_arr, bias_arr, out_arr, N_arr = ((ctypes.c_void_p * n)(), (ctypes.c_void_p * n)(), (ctypes.c_void_p * n)(),
+                                        (ctypes.c_int64 * n)())
+    for g, (bQuant, bias) in enumerate(weights):
+        _abort_if(not isinstance(bQuant, QTensor) or not isIntgemm(bQuant.type),
+                  "Intgemm expects type of B to be a variant of intgemm not {}", getattr(bQuant, "type", type(bQuant)))
+        _abort_if(isHardwareSpecific(bQuant.type) or sizeOf(bQuant.type) != 1,
+                  "Unsupported type {} for Intgemm type??", bQuant.type)
+        _abort_if(rows(bQuant) != K, "Matrix product requires inner dimensions to match: {} vs {}", K, rows(bQuant))
+        N = cols(bQuant)
+        if bias is not None:
+            _abort_if(bias.dtype != torch.float32 or bias.numel() != N, "bias must be float32 [1, {}]", N)
+            bias = bias.contiguous()
+            keep.append(bias)
+        out = torch.empty(tuple(a.shape[:-1]) + (N,), dtype=torch.float32, device=a.device)
+        outs.append(out)
+        Bq_arr[g], bias_arr[g], out_arr[g], N_arr[g] = (bQuant.data_ptr(), None if bias is None else bias.data_ptr(),
+                                                        out.data_ptr(), N)
+    st = be.lib.marian_hip_int8_affine_f32_grouped(
+        a.data_ptr(), aQuant.data_ptr(), n, Bq_arr, bias_arr, out_arr, N_arr, M, K, scale, int(relu),
+        None if absmax is None else absmax.data_ptr(), be.workspace.data_ptr(), be.workspace_bytes, be.stream())
+    _lib.check(st, "affineOrDot")
+    return outs, aQuant
+
+
 def multiply(aQuant, bQuant, bias=None, scale=1.0, relu=False, shortlist=None):
     """The multiply node of reference src/tensors/cpu/intgemm_interface.h:60-94."""
     be = _backend_of(aQuant)

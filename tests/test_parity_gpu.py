@@ -639,6 +639,75 @@ def test_model_file_weights_run_verbatim(integer, orc, synth, tmp_path):
     assert np.array_equal(got, want)
 
 
+GROUPED_CASES = [
+    # M, K, [N of every matrix], bias on?, ReLU, abs-max handed over
+    (128, 1024, [1024, 1024, 1024], True, False, True),     # self-attention projections of transformer-big
+    (128, 1024, [1024, 1024, 1024], True, False, False),
+    (128, 512, [512, 512, 512], True, False, False),        # transformer-base
+    (1, 512, [512, 512, 512], False, False, False),
+    (4, 512, [512], True, True, False),
+    (33, 192, [136, 8, 72, 1000], True, True, False),       # ragged widths, four matrices
+    (64, 1024, [2048, 1024], True, False, True),
+    (200, 1024, [504, 520], True, True, False),
+    (128, 4096, [1024, 1024], True, False, False),          # long rows: 16-row workgroups, K split eight ways
+    (256, 2048, [4096, 4096], True, False, False),          # too wide for one launch: one quantization, two multiplies
+    (300, 1024, [512, 512, 512], True, True, True),         # too many rows for the quantize-on-stage kernel
+    (16, 64, [8, 8], False, False, False),
+]
+
+
+@pytest.mark.parametrize("M,K,Ns,bias_on,relu,handed", GROUPED_CASES)
+def test_grouped_affine_equals_separate_calls_and_checker(integer, orc, synth, M, K, Ns, bias_on, relu, handed):
+    """One activation tensor through several weight matrices in one call: every output equals the
+    single-matrix call's and the CPU checker's bit for bit, and the quantized activations (written
+    once) are the checker's."""
+    from conftest import load
+    ops = load("ops")
+    say("grouped", M, K, Ns, bias_on, relu, handed)
+    A = synth.normal(900 + M + K, synth.STREAM_A, (M, K), 1.0)
+    Ws = [synth.normal(900 + g, synth.STREAM_W, (K, N), 0.02 * (g + 1)) for g, N in enumerate(Ns)]
+    biases = [synth.normal(900 + g, synth.STREAM_BIAS, (N,), 0.01) if bias_on and g != 1 else None
+              for g, N in enumerate(Ns)]          # (the second matrix never has a bias)
+    Aq_h = orc.prepare_a(A)
+    Bq_h = [orc.prepare_b(W) for W in Ws]
+    Bq = [upload_q(integer, b, (K, N)) for b, N in zip(Bq_h, Ns)]
+    dA = dev(A)
+    absmax = None
+    if handed:   # the abs-max as a producing kernel leaves it: a layer norm that reproduces A
+        import torch
+        ln, absmax = ops.layerNorm(dA, torch.ones(K, device="cuda"), None, 1e-9, want_absmax=True)
+        dA = ln
+        A = ln.cpu().numpy()
+        Aq_h = orc.prepare_a(A)
+    dbias = [None if b is None else dev(b) for b in biases]
+    outs, Aq = integer.affine_f32_grouped(dA, list(zip(Bq, dbias)), scale=0.5, relu=relu, absmax=absmax)
+    assert np.array_equal(Aq.numpy(), Aq_h), "quantized activations / quantMult"
+    for g, N in enumerate(Ns):
+        want, _ = orc.affine(Aq_h, Bq_h[g], biases[g], M, K, N, 0.5, relu)
+        single, _ = integer.affine_f32(dA, Bq[g], dbias[g], scale=0.5, relu=relu)
+        got = outs[g].cpu().numpy()
+        assert np.array_equal(got.view(np.uint32), single.cpu().numpy().view(np.uint32)), "matrix %d vs single call" % g
+        assert np.array_equal(got, want), "matrix %d vs checker" % g
+
+
+def test_grouped_affine_argument_checks(integer):
+    import ctypes
+    from conftest import load
+    L = load("_lib")
+    lib = L.lib()
+    buf = 0x1000
+    one = (ctypes.c_void_p * 1)(buf)
+    n8 = (ctypes.c_int64 * 1)(8)
+    call = lambda n, Bq, bias, out, N, M, K: lib.marian_hip_int8_affine_f32_grouped(
+        buf, buf, n, Bq, bias, out, N, M, K, 1.0, 0, None, buf, 4096, None)
+    assert call(0, one, None, one, n8, 1, 64) == L.ERR_SHAPE
+    assert call(5, one, None, one, n8, 1, 64) == L.ERR_SHAPE
+    assert call(1, None, None, one, n8, 1, 64) == L.ERR_NULL
+    assert call(1, one, None, one, (ctypes.c_int64 * 1)(12), 1, 64) == L.ERR_SHAPE
+    assert call(1, one, None, one, n8, 1, 100) == L.ERR_SHAPE
+    assert call(1, one, None, one, n8, 0, 64) == L.OK
+
+
 def write_host_check_fixture(path, orc, synth):
     """Inputs and the CPU checker's expected values for marian-dev_amd/host/host_check.cpp (layout in
     that file's header)."""
