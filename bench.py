@@ -31,13 +31,25 @@ PKG = "marian-dev_amd"
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 INT8_PEAK_TOPS = 5000.0      # MI355X dense int8 MFMA, published (5.0 POP/s)
 
-# HBM bytes per launch of the kernels named here, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# runs of `bench.py --pmc-probe` (KiB per dispatch, scaled by the same counters' reading for a
-# plain copy of known size); the runs are summarised under profiles/.  None = not measured.
-MEASURED_TRAFFIC = {
-    # (8677.6 KiB FETCH_SIZE x 1.9992 + 8033.8 KiB WRITE_SIZE) per dispatch
-    "stream32_fused_M64_K512_N32000": int((8677.6 * 1.9992 + 8033.8) * 1024),
-}
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic_pmc.txt")
+
+
+def measured_traffic():
+    """HBM bytes per launch of the kernels named in profiles/hbm_traffic_pmc.txt: the summary of two
+    rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE) of `bench.py --pmc-probe`, written by
+    `bench.py --pmc-summary`.  Lines `traffic_bytes_per_launch <key> = <bytes>`; `build_commit =`
+    names the commit of the sources the counters were taken from.  ({} when the file is absent.)"""
+    out = {"_commit": None}
+    if not os.path.exists(TRAFFIC_FILE):
+        return out
+    for line in open(TRAFFIC_FILE):
+        parts = line.split()
+        if len(parts) >= 4 and parts[0] == "traffic_bytes_per_launch" and parts[2] == "=":
+            out[parts[1]] = int(parts[3])
+        if len(parts) >= 3 and parts[0] == "build_commit" and parts[1] == "=":
+            out["_commit"] = parts[2]
+    return out
+
 
 DECODE_SHAPES = [(512, 1536), (512, 512), (512, 2048), (2048, 512), (512, 32000)]
 DECODE_M = [1, 4, 16, 64]
@@ -111,7 +123,7 @@ class BigDecoder:
     taken for the new position only.  Beam search itself (top-k, hypothesis bookkeeping) is not
     part of the step."""
 
-    def __init__(self, torch, integer, ops, sets, t_past=20, src_len=40, seed=300):
+    def __init__(self, torch, integer, ops, sets, t_past=20, src_len=60, seed=300):
         self.torch, self.integer, self.ops = torch, integer, ops
         self.d, self.ffn, self.V, self.H = 1024, 4096, 32000, 16
         self.beam, self.batch = 4, 32
@@ -154,6 +166,7 @@ class BigDecoder:
         self.Vself = [torch.randn(M * H, self.T, d // H, device="cuda", generator=g) for _ in range(6)]
         self.Kenc = [torch.randn(self.batch * H, self.L, d // H, device="cuda", generator=g) for _ in range(6)]
         self.Venc = [torch.randn(self.batch * H, self.L, d // H, device="cuda", generator=g) for _ in range(6)]
+        # source lengths uniform over 20 .. 60, padded to the longest (the mask covers the rest)
         lens = torch.randint(20, self.L + 1, (self.batch,), device="cuda", generator=g)
         self.mask = (torch.arange(self.L, device="cuda")[None, :] >= lens[:, None]).float() * -99999999.0
 
@@ -280,37 +293,116 @@ def per_launch_ms(torch, launches, repeat):
     return float(d.mean()), float(np.median(d))
 
 
-def cpu_baseline(seconds=12.0):
-    """The CPU restatement of the reference path (prepareA + VNNI multiply + unquantize/bias,
-    one thread, like one Marian CPU worker) on the same decode sweep, bounded in time."""
+def cpu_model():
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def cpu_sweep_work():
     from oracle import oracle as orc
     synth = importlib.import_module(PKG + ".synth")
     work = []
-    total_ops = 0
     for (K, N) in DECODE_SHAPES:
         W = synth.normal(1002, synth.STREAM_W, (K, N), 0.02)
         Bq = orc.prepare_b(W)
         bias = synth.normal(1002, synth.STREAM_BIAS, (N,), 0.01)
         for M in DECODE_M:
             A = synth.normal(1002, synth.STREAM_A, (M, K), 1.0)
-            work.append((orc.AffineF32(M, K, N), A, Bq, bias))
-            total_ops += 2 * M * K * N
-    for f, A, Bq, bias in work:
+            work.append((orc.AffineF32(M, K, N), A, Bq, bias, 2 * M * K * N))
+    for f, A, Bq, bias, _ in work:
         f(A, Bq, bias)
+    return work
+
+
+def cpu_sweep_passes(work, seconds):
     passes = 0
     t0 = time.perf_counter()
     while True:
-        for f, A, Bq, bias in work:
+        for f, A, Bq, bias, _ in work:
             f(A, Bq, bias)
         passes += 1
         dt = time.perf_counter() - t0
         if dt > seconds:
-            break
-    return {"value": round(total_ops * passes / dt / 1e12, 5), "unit": "TOPS", "cores": 1,
+            return passes, dt
+
+
+def cpu_worker(seconds):
+    """One of the independent instances of the aggregate CPU figure (no GPU, no torch)."""
+    work = cpu_sweep_work()
+    passes, dt = cpu_sweep_passes(work, seconds)
+    print(json.dumps({"passes": passes, "seconds": dt, "ops_per_pass": sum(w[4] for w in work)}))
+
+
+def cpu_baseline(seconds=10.0, aggregate_seconds=6.0, big_seconds=6.0):
+    """The CPU restatement of the reference path (prepareA + VNNI multiply + unquantize/bias, one
+    thread per GEMM like one Marian CPU worker, reference src/common/config.cpp:245-247) timed on
+    this host, bounded in time: the decode sweep on one core (whole and per shape), the same sweep
+    in one independent process per core of this job's share, and the 49 GEMMs of the
+    transformer-big decoding step at M = 128 on one core."""
+    import subprocess
+    from oracle import oracle as orc
+    work = cpu_sweep_work()
+    ops_per_pass = sum(w[4] for w in work)
+    passes, dt = cpu_sweep_passes(work, seconds)
+    per_shape = {}
+    for f, A, Bq, bias, ops in work:
+        n, t0 = 0, time.perf_counter()
+        while n < 3 or time.perf_counter() - t0 < 0.05:
+            f(A, Bq, bias)
+            n += 1
+        per_shape["M%d_%dx%d" % (f.M, f.K, f.N)] = round((time.perf_counter() - t0) / n * 1e6, 1)
+    # one instance per core of this job's share (at most 16: what a one-GPU job is given)
+    try:
+        share = len(os.sched_getaffinity(0))
+    except AttributeError:
+        share = os.cpu_count() or 1
+    instances = max(1, min(share, 16))
+    procs = [subprocess.Popen([sys.executable, os.path.abspath(__file__), "--cpu-worker", str(aggregate_seconds)],
+                              stdout=subprocess.PIPE, text=True) for _ in range(instances)]
+    agg_ops_per_s = 0.0
+    for pr in procs:
+        out, _ = pr.communicate()
+        r = json.loads(out.strip().splitlines()[-1])
+        agg_ops_per_s += r["passes"] * r["ops_per_pass"] / r["seconds"]
+    # transformer-big decoding step: 48 layer GEMMs + the vocabulary GEMM at M = 128, random int8
+    # weights (121 MB, every matrix its own memory), fp32 activations quantized per call
+    rng = np.random.default_rng(77)
+    d, ffn, V, M = 1024, 4096, 32000, 128
+    layer = [(d, d)] * 6 + [(d, ffn), (ffn, d)]
+    big = []
+    for (K, N) in layer * 6 + [(d, V)]:
+        Bq = rng.integers(-127, 128, size=K * N + 4, dtype=np.int8)
+        Bq[-4:] = np.frombuffer(np.float32(6000.0).tobytes(), np.int8)
+        big.append((orc.AffineF32(M, K, N), rng.standard_normal((M, K)).astype(np.float32), Bq,
+                    np.zeros(N, np.float32)))
+    for f, A, Bq, bias in big[:2]:
+        f(A, Bq, bias)
+    steps, t0 = 0, time.perf_counter()
+    while steps < 1 or time.perf_counter() - t0 < big_seconds:
+        for f, A, Bq, bias in big:
+            f(A, Bq, bias)
+        steps += 1
+    big_dt = (time.perf_counter() - t0) / steps
+    return {"value": round(ops_per_pass * passes / dt / 1e12, 5), "unit": "TOPS", "cores": 1,
             "kind": "port",
             "isa": "avx512-vnni" if orc.has_vnni() else "scalar",
-            "host_cpus": os.cpu_count(),
-            "sample": "%d passes of the same 20-shape decode sweep in %.1f s on one core" % (passes, dt)}
+            "cpu_model": cpu_model(), "host_cpus": os.cpu_count(), "cpus_in_share": share,
+            "sample": "%d passes of the same 20-shape decode sweep in %.1f s on one core" % (passes, dt),
+            "per_shape_single_core_us": per_shape,
+            "aggregate": {"value": round(agg_ops_per_s / 1e12, 4), "unit": "TOPS", "cores": instances,
+                          "sample": "%d independent single-threaded processes, %.0f s of the same sweep each"
+                                    % (instances, aggregate_seconds)},
+            "transformer_big_decode": {
+                "what": "GEMM-only decode step at M=128 (48 layer GEMMs + 32000-vocab GEMM, each with its "
+                        "prepareA) on one core",
+                "ms_per_step": round(big_dt * 1e3, 2), "hyp_tokens_per_s": round(M / big_dt, 1),
+                "output_tokens_per_s": round(32 / big_dt, 1), "cores": 1,
+                "sample": "%d steps in %.1f s" % (steps, big_dt * steps)}}
 
 
 def pmc_probe(torch, integer, lib, be):
@@ -335,6 +427,157 @@ def pmc_probe(torch, integer, lib, be):
         del e
 
 
+def probe_ceilings(torch):
+    """Machine ceilings behind the roofline discussion, measured with the probe kernels of the tuning
+    build (include/marian_hip_int8_tuning.h) and HIP events; prints a text table.  Nothing here
+    touches the shipped library's kernels."""
+    import ctypes
+    T = importlib.import_module(PKG + "._lib").tuning_lib()
+    st = torch.cuda.current_stream().cuda_stream
+    pool_bytes = 1 << 30
+    pool = torch.randint(-128, 128, (pool_bytes,), dtype=torch.int8, device="cuda")
+    dst = torch.empty(1 << 28, dtype=torch.int8, device="cuda")
+    print("machine ceilings on %s (%d compute units)" % (torch.cuda.get_device_name(0),
+                                                          torch.cuda.get_device_properties(0).multi_processor_count))
+
+    def stream(read_bytes, write_bytes, wgs, threads, u=8, nt=0, rotate=True):
+        n = max(1, pool_bytes // max(read_bytes, 16)) if rotate else 1
+        n = min(n, 64)
+        launches = [(lambda i=i: T.marian_hip_probe_stream(pool.data_ptr() + i * read_bytes, read_bytes, dst.data_ptr(),
+                                                            write_bytes, wgs, threads, u, nt, st)) for i in range(n)]
+        reps = max(3, 60 // n)
+        mean, med = per_launch_ms(torch, launches, reps)
+        return med * 1e3   # us
+
+    print("\n-- back-to-back launch floor (a kernel that moves 16 bytes, 100 launches per timed pass) --")
+    tiny = [(lambda: T.marian_hip_probe_stream(pool.data_ptr(), 16, dst.data_ptr(), 16, 1, 64, 1, 0, st))] * 100
+    print("  %.2f us per launch" % (per_launch_ms(torch, tiny, 5)[1] * 1e3))
+    print("\n-- read-only pass (1024 workgroups x 256 threads, 8 loads in flight), rotating over 1 GiB --")
+    for mb in (16, 32, 64, 256, 1024):
+        us = stream(mb << 20, 16, 1024, 256)
+        print("  %5d MiB  %8.2f us  %6.2f TB/s" % (mb, us, (mb << 20) / us / 1e6))
+    print("\n-- read-only pass over the same 64 MiB every launch (Infinity-Cache resident) --")
+    us = stream(64 << 20, 16, 1024, 256, rotate=False)
+    print("  %5d MiB  %8.2f us  %6.2f TB/s" % (64, us, (64 << 20) / us / 1e6))
+    print("\n-- write-only pass (1024 x 256), plain and non-temporal stores --")
+    for mb in (16, 64, 256):
+        for nt in (0, 1):
+            us = stream(16, mb << 20, 1024, 256, 8, nt)
+            print("  %5d MiB  %s  %8.2f us  %6.2f TB/s" % (mb, "nt   " if nt else "plain", us, (mb << 20) / us / 1e6))
+    print("\n-- copy of 64 MiB (read 64 MiB, then write 64 MiB) --")
+    us = stream(64 << 20, 64 << 20, 2048, 256)
+    print("  %8.2f us  %6.2f TB/s (read + written bytes)" % (us, 2 * (64 << 20) / us / 1e6))
+    print("\n-- data movement of the dominant decode call (M=64, K=512, N=32000: 16.4 MB of weights + 128 KB of"
+          " activations read, 8.2 MB written), the grid of its kernel (250 workgroups x 512 threads) --")
+    rb, wb = 512 * 32000 + 64 * 512 * 4, 64 * 32000 * 4
+    us_w = stream(rb, 16, 250, 512)
+    us_c = stream(rb, wb, 250, 512, 8, 1)
+    print("  weight stream alone     %8.2f us  %6.2f TB/s" % (us_w, rb / us_w / 1e6))
+    print("  reads + output stores   %8.2f us  %6.2f TB/s of the %d algorithmic bytes" % (us_c, (rb + wb) / us_c / 1e6, rb + wb))
+    print("  (HBM roofline of those bytes at 8 TB/s: %.2f us)" % ((rb + wb) / 8e6))
+    print("\n-- encoder-size operand and output sizes --")
+    for name, r_, w_ in (("read 4096x4096 fp32 (67 MB), as the abs-max pass", 4096 * 4096 * 4, 16),
+                         ("read 67 MB fp32 + write 16.8 MB int8, as the quantize pass", 4096 * 4096 * 4, 4096 * 4096),
+                         ("write 4096x4096 fp32 (67 MB), as the GEMM's output", 16, 4096 * 4096 * 4)):
+        us = stream(r_, w_, 2048, 256, 8, 0)
+        print("  %-62s %8.2f us  %6.2f TB/s" % (name, us, (max(r_, 16) + max(w_, 16)) / us / 1e6))
+    print("\n-- sustained v_mfma_i32_32x32x32_i8 rate on random operand bits --")
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    for per_cu in (1, 2):
+        wgs, iters = cus * per_cu, 4000
+        clocks = torch.zeros(2 * wgs, dtype=torch.int64, device="cuda")
+        sink = torch.zeros(4, dtype=torch.int32, device="cuda")
+        f = lambda: T.marian_hip_probe_mfma(pool.data_ptr(), iters, wgs, clocks.data_ptr(), sink.data_ptr(), st)
+        mean, med = per_launch_ms(torch, [f], 6)
+        c = clocks.cpu().numpy().reshape(-1, 2).astype(np.float64)
+        mhz = float(np.median(c[:, 0] / c[:, 1]) * 100.0)
+        ops = 2.0 * 32 ** 3 * 8 * iters * 4 * wgs
+        in_loop_s = float(np.median(c[:, 1])) / 100e6
+        print("  %d workgroup(s) of 4 waves per CU: %7.1f TOPS over the launch (%.1f us), %7.1f TOPS inside the loop, "
+              "shader clock %.0f MHz -> %d CUs x 8192 op/clk x clock = %.0f TOPS"
+              % (per_cu, ops / (med * 1e-3) / 1e12, med * 1e3, ops / in_loop_s / 1e12, mhz, cus, cus * 8192 * mhz * 1e6 / 1e12))
+
+
+def measured_int8_peak(torch):
+    """Sustained int8 matrix rate of this device from the tuning build's MFMA probe (HIP events around
+    the launches), with the shader clock it holds meanwhile and CUs x 8192 op/clk x that clock.  None
+    when the tuning build is absent."""
+    try:
+        T = importlib.import_module(PKG + "._lib").tuning_lib()
+    except Exception:
+        return None
+    st = torch.cuda.current_stream().cuda_stream
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    data = torch.randint(-128, 128, (4096,), dtype=torch.int8, device="cuda")
+    wgs, iters = cus, 4000
+    clocks = torch.zeros(2 * wgs, dtype=torch.int64, device="cuda")
+    sink = torch.zeros(4, dtype=torch.int32, device="cuda")
+    f = lambda: T.marian_hip_probe_mfma(data.data_ptr(), iters, wgs, clocks.data_ptr(), sink.data_ptr(), st)
+    mean, med = per_launch_ms(torch, [f, f, f], 4)
+    c = clocks.cpu().numpy().reshape(-1, 2).astype(np.float64)
+    mhz = float(np.median(c[:, 0] / c[:, 1]) * 100.0)
+    ops = 2.0 * 32 ** 3 * 8 * iters * 4 * wgs
+    return {"sustained_tops": round(ops / (med * 1e-3) / 1e12, 1),
+            "shader_clock_mhz": round(mhz, 0),
+            "cus_x_8192_x_clock_tops": round(cus * 8192 * mhz * 1e6 / 1e12, 1),
+            "how": "tuning build's MFMA probe: %d workgroups of 4 waves (one wave per SIMD), %d x 8 "
+                   "v_mfma_i32_32x32x32_i8 per wave on random operand bits, %.0f us per launch; clock = shader "
+                   "clocks / 100 MHz reference clocks inside the loop" % (wgs, iters, med * 1e3)}
+
+
+def pmc_summary(fetch_csv, write_csv):
+    """Summarises the two rocprofv3 --pmc runs of `bench.py --pmc-probe` (FETCH_SIZE, WRITE_SIZE; KiB
+    per dispatch) as the text of profiles/hbm_traffic_pmc.txt."""
+    import csv
+    import subprocess
+
+    def short(name):
+        for key, pat in (("copy64", "vectorized_elementwise_kernel<4, at::native::CUDAFunctorOnSelf_add<float>"),
+                         ("stream32_fused_M64_K512_N32000", "gemm_stream32_kernel<2, 4, 2, 8, 1, 4, 64"),
+                         ("gemm_pair", "gemm_pair_kernel"), ("gemm_mfma32", "gemm_mfma32_kernel"),
+                         ("absmax", "absmax_partial_kernel"), ("quantize_a", "quantize_a_kernel")):
+            if pat in name:
+                return key + ("|" + name.split("gemm_mfma32_kernel")[1].split("(")[0] if key == "gemm_mfma32" else "")
+        return None
+
+    def load(path, counter):
+        acc = {}
+        for row in csv.DictReader(open(path)):
+            if row["Counter_Name"] != counter:
+                continue
+            k = short(row["Kernel_Name"])
+            if k is None:
+                continue
+            k = (k, int(row["Grid_Size"]))
+            acc.setdefault(k, []).append(float(row["Counter_Value"]))
+        return {k: sum(v) / len(v) for k, v in acc.items()}
+
+    fetch, write = load(fetch_csv, "FETCH_SIZE"), load(write_csv, "WRITE_SIZE")
+    copy_key = [k for k in fetch if k[0] == "copy64"][0]
+    f_scale, w_scale = 65536.0 / fetch[copy_key], 65536.0 / write[copy_key]
+    try:
+        commit = subprocess.run(["git", "-C", ROOT, "rev-parse", "--short", "HEAD"], capture_output=True, text=True).stdout.strip()
+    except OSError:
+        commit = ""
+    print("yardstick: plain elementwise copy of 64 MiB fp32 (torch.add(src, 1.0, out=dst): reads 65536 KiB, writes 65536 KiB)")
+    print("  FETCH_SIZE %9.1f KiB -> scale factor %.4f" % (fetch[copy_key], f_scale))
+    print("  WRITE_SIZE %9.1f KiB -> scale factor %.4f" % (write[copy_key], w_scale))
+    print("")
+    print("%-58s %10s %12s %10s %12s" % ("kernel | grid size (threads)", "FETCH raw", "FETCH scaled", "WRITE", "total KiB"))
+    lines = []
+    for k in sorted(fetch):
+        if k[0] == "copy64":
+            continue
+        fs, w = fetch[k] * f_scale, write.get(k, 0.0) * w_scale
+        print("%-58s %10.1f %12.1f %10.1f %12.1f" % ("%s | %d" % k, fetch[k], fs, w, fs + w))
+        lines.append((k, int((fs + w) * 1024)))
+    print("")
+    for (name, grid), b in lines:
+        key = name if name.startswith("stream32") else "%s_grid%d" % (name.replace("|", "").replace(" ", "").replace(",", "_"), grid)
+        print("traffic_bytes_per_launch %s = %d" % (key, b))
+    print("build_commit = %s" % (commit or "unknown"))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -345,7 +588,22 @@ def main():
                     help="launch the dominant kernels and a plain copy a few times and exit "
                          "(for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)")
     ap.add_argument("--only", default="", help="comma list of extra workloads: encoder,shortlist,big")
+    ap.add_argument("--cpu-worker", type=float, default=0.0, metavar="SECONDS",
+                    help="(internal) one instance of the aggregate CPU baseline; no GPU")
+    ap.add_argument("--probe-ceilings", action="store_true",
+                    help="measure the machine ceilings (read / write / copy bandwidth by footprint, launch "
+                         "floor, data movement of the dominant call, sustained int8 MFMA rate and clock) "
+                         "with the tuning build's probe kernels, print a text table and exit")
+    ap.add_argument("--pmc-summary", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"),
+                    help="summarise two rocprofv3 --pmc counter_collection.csv files of --pmc-probe runs "
+                         "(the text of profiles/hbm_traffic_pmc.txt) and exit; no GPU")
     args = ap.parse_args()
+    if args.cpu_worker > 0:
+        cpu_worker(args.cpu_worker)
+        return
+    if args.pmc_summary:
+        pmc_summary(*args.pmc_summary)
+        return
     if args.gpus != 1:
         sys.exit("bench.py: this path runs on one GPU (no collectives are part of it); use --gpus 1")
 
@@ -360,6 +618,9 @@ def main():
 
     if args.pmc_probe:
         pmc_probe(torch, integer, lib, be)
+        return
+    if args.probe_ceilings:
+        probe_ceilings(torch)
         return
 
     # ---------------- headline: transformer-base decode sweep -------------------------------
@@ -394,10 +655,14 @@ def main():
     mean_ms, med_ms = per_launch_ms(
         torch, [(lambda c=c: dom.launch_fused(lib, be, c)) for c in range(sets)], 12)
     dom_bytes = algorithmic_bytes(dom.M, dom.K, dom.N)
+    traffic = measured_traffic()
     achieved = dom_bytes / (mean_ms * 1e-3) / 1e9
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                 "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                "traffic": MEASURED_TRAFFIC.get("stream32_fused_M64_K512_N32000"),
+                "traffic": traffic.get("stream32_fused_M64_K512_N32000"),
+                "traffic_source": "profiles/hbm_traffic_pmc.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a "
+                                  "64 MiB copy), sources at commit %s" % traffic["_commit"]
+                                  if traffic.get("stream32_fused_M64_K512_N32000") else None,
                 "kernel": "gemm_stream32_kernel<MT32=2,WN=4,KW=2,PW=8,fused> M=64 K=512 N=32000",
                 "bytes_per_launch": dom_bytes, "avg_launch_us": round(mean_ms * 1e3, 3),
                 "median_launch_us": round(med_ms * 1e3, 3),
@@ -446,10 +711,13 @@ def main():
             g_ms, g_med = per_launch_ms(
                 torch, [(lambda c=c: o.launch(lib, be, c, prepare=False)) for c in range(4)], 10)
             p_ms, _ = per_launch_ms(torch, [(lambda: o.launch(lib, be, 0, gemm=False))], 10)
-            t_all = (g_ms + p_ms) * 1e-3
+            # the call BASELINE defines (fp32 A in, fp32 out) through the single entry point, timed as one
+            f_ms, _ = per_launch_ms(torch, [(lambda c=c: o.launch_fused(lib, be, c)) for c in range(4)], 10)
+            t_all = f_ms * 1e-3
             enc["M%d_K%d_N%d" % (M, K, N)] = {
                 "gemm_us": round(g_ms * 1e3, 2), "gemm_median_us": round(g_med * 1e3, 2),
                 "prepare_a_us": round(p_ms * 1e3, 2),
+                "affine_f32_us": round(f_ms * 1e3, 2),
                 "gemm_tops": round(o.ops / (g_ms * 1e-3) / 1e12, 1),
                 "gemm_mfma_frac": round(o.ops / (g_ms * 1e-3) / 1e12 / INT8_PEAK_TOPS, 4),
                 "gemm_hbm_frac": round(gemm_kernel_bytes(M, K, N) / (g_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
@@ -458,6 +726,7 @@ def main():
             del o
         out["encoder"] = enc
         out["int8_peak_tops_used"] = INT8_PEAK_TOPS
+        out["int8_peak_measured"] = measured_int8_peak(torch)
 
     # ---------------- shortlisted output layer -------------------------------------------------
     if "shortlist" in extras:
@@ -524,7 +793,8 @@ def main():
         out["transformer_big_decode_full"] = {
             "what": "full decoder step through the host mirrors: 49 int8 affine calls + per layer "
                     "2 one-launch attentions (20 cached positions + the new one, appended by the call; "
-                    "40 source positions with mask), 3 skip-add+layer-norm; log-softmax over 32000, beam/batch transposition + n-best per "
+                    "source lengths uniform 20..60, padded to 60 positions with mask), 3 skip-add+layer-norm; the self-attention "
+                    "projections Wq, Wk, Wv through one grouped call; log-softmax over 32000, beam/batch transposition + n-best per "
                     "sentence; no hypothesis bookkeeping; the abs-max of every GEMM input is left by the kernel that "
                     "produced it",
             "ms_per_step": round(fdt / n * 1e3, 4),
@@ -537,7 +807,12 @@ def main():
         del full, gonly, dec
 
     if not args.no_cpu:
-        out["cpu_baseline"] = cpu_baseline()
+        cpu = cpu_baseline()
+        big_cpu = cpu.pop("transformer_big_decode")
+        out["cpu_baseline"] = cpu
+        if "transformer_big_decode" in out:   # the CPU figure beside the tokens/s it belongs to
+            out["transformer_big_decode"]["cpu_baseline"] = big_cpu
+            out["transformer_big_decode_full"]["cpu_baseline_gemm_only"] = big_cpu
     else:
         out["cpu_baseline"] = None
     print(json.dumps(out))

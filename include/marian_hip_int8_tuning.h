@@ -1,9 +1,9 @@
 /*
  * marian_hip_int8_tuning.h - measurement switches of the tuning build of the int8 backend.
  *
- * These two functions exist only in libmarian_hip_int8_tuning.so (built with
+ * These functions exist only in libmarian_hip_int8_tuning.so (built with
  * -DMARIAN_HIP_TUNING from the same sources as libmarian_hip_int8.so).  That build exports
- * everything include/marian_hip_int8.h and include/marian_hip_ops.h declare plus the two
+ * everything include/marian_hip_int8.h and include/marian_hip_ops.h declare plus the
  * functions below, carries kernel families that the automatic selection never picks, and reads
  * clocks inside its kernels.  The shipped library has none of this: no process-wide switch, no
  * retained pointer.  They have no counterpart in the reference; tests use them to run every
@@ -11,6 +11,8 @@
  */
 #ifndef MARIAN_HIP_INT8_TUNING_H
 #define MARIAN_HIP_INT8_TUNING_H
+
+#include <stddef.h>
 
 #ifdef __cplusplus
 extern "C" {
@@ -32,6 +34,24 @@ int marian_hip_int8_set_kernel(int which);
  * recording off before the buffer is freed.
  */
 void marian_hip_int8_debug_profile(long long* clocks);
+
+/*
+ * Machine-ceiling probes: the yardsticks the kernels' times are held against.
+ *
+ * marian_hip_probe_stream: `workgroups` x `threads` threads read read_bytes from src
+ * (16 bytes per load, loads_in_flight of them outstanding per thread: 1, 4 or 8) and then write
+ * write_bytes to dst (non-temporal stores if asked) - the data movement of a kernel without its
+ * arithmetic.  read_bytes and write_bytes are multiples of 16; dst holds write_bytes.
+ *
+ * marian_hip_probe_mfma: `workgroups` workgroups of four waves issue iters x 8 independent
+ * v_mfma_i32_32x32x32_i8 per wave on the 4 KB of operand bits at `data`; clocks[2 * w] and
+ * clocks[2 * w + 1] receive the shader clocks and the 100 MHz reference clocks workgroup w spent
+ * in the loop (sustained int8 rate = 2 * 32^3 * 8 * iters * 4 waves * workgroups / time; shader
+ * clock = 100 MHz * clocks ratio).  sink: one int of device memory.
+ */
+int marian_hip_probe_stream(const void* src, size_t read_bytes, void* dst, size_t write_bytes, int workgroups,
+                            int threads, int loads_in_flight, int nontemporal, void* stream);
+int marian_hip_probe_mfma(const void* data, int iters, int workgroups, long long* clocks, int* sink, void* stream);
 
 #ifdef __cplusplus
 }

@@ -5,6 +5,7 @@
 #include <hip/hip_runtime.h>
 
 #include <atomic>
+#include <random>
 
 #include "abi_common.h"
 #include "gemm_mfma32_kernel.h"
@@ -17,6 +18,7 @@
 #include "../../include/marian_hip_int8_tuning.h"
 #include "gemm_persistent_kernel.h"
 #include "gemm_tile_kernel.h"
+#include "probe_kernels.h"
 #endif
 
 using namespace marian_hip;
@@ -554,6 +556,17 @@ int run_gemm(const int8_t* Aq, const int8_t* Bq, const float* bias, const uint32
   return launch_gemm(a, reinterpret_cast<hipStream_t>(stream));
 }
 
+// One-pass prepareA: from this many values on (below, two launches are as fast or faster), how long a
+// workgroup polls before it helps itself (each poll is a memory round trip of about a microsecond),
+// and the nonce that starts its tags (random per process, so that words left in recycled device
+// memory by another process do not match).
+constexpr size_t kOnePassMinElems = 4u << 20;   // (measured: 8 MB of input - no gain; 16.8 MB: 10.3 -> 9.4 us; 67 MB: 30.4 -> 21.1 us)
+constexpr int kOnePassSpinLimit = 20000;
+unsigned next_nonce() {
+  static std::atomic<unsigned> nonce{(unsigned)std::random_device{}() | 1u};
+  return nonce.fetch_add(0x9E3779B1u, std::memory_order_relaxed);
+}
+
 int absmax_blocks(size_t n4) {
   size_t per_block = (size_t)kQuantThreads * 8;  // eight 16-byte loads per thread
   size_t g = (n4 + per_block - 1) / per_block;
@@ -591,6 +604,33 @@ size_t marian_hip_int8_workspace_bytes(void) { return kWorkspaceBytes; }
 int marian_hip_int8_set_kernel(int which) { return g_kernel_override.exchange(which); }
 
 void marian_hip_int8_debug_profile(long long* p) { g_prof.store(p); }
+
+int marian_hip_probe_stream(const void* src, size_t read_bytes, void* dst, size_t write_bytes, int workgroups,
+                            int threads, int loads_in_flight, int nontemporal, void* stream) {
+  if(!src || !dst) return MARIAN_HIP_ERR_NULL;
+  if(workgroups <= 0 || threads <= 0 || threads > 1024 || threads % 64 != 0) return MARIAN_HIP_ERR_SHAPE;
+  if(!aligned(src, 16) || !aligned(dst, 16)) return MARIAN_HIP_ERR_ALIGN;
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  const v4i* s = reinterpret_cast<const v4i*>(src);
+  v4i* d = reinterpret_cast<v4i*>(dst);
+  const size_t rv = read_bytes / 16, wv = write_bytes / 16;
+#define MH_PROBE(U, NT) hipLaunchKernelGGL((probe_stream_kernel<U, NT>), dim3(workgroups), dim3(threads), 0, st, s, rv, d, wv)
+  if(loads_in_flight >= 8) { if(nontemporal) MH_PROBE(8, true); else MH_PROBE(8, false); }
+  else if(loads_in_flight >= 4) { if(nontemporal) MH_PROBE(4, true); else MH_PROBE(4, false); }
+  else { if(nontemporal) MH_PROBE(1, true); else MH_PROBE(1, false); }
+#undef MH_PROBE
+  MH_HIP(hipGetLastError());
+  return MARIAN_HIP_OK;
+}
+
+int marian_hip_probe_mfma(const void* data, int iters, int workgroups, long long* clocks, int* sink, void* stream) {
+  if(!data || !clocks || !sink) return MARIAN_HIP_ERR_NULL;
+  if(iters <= 0 || workgroups <= 0) return MARIAN_HIP_ERR_SHAPE;
+  hipLaunchKernelGGL(probe_mfma_kernel, dim3(workgroups), dim3(256), 0, reinterpret_cast<hipStream_t>(stream),
+                     reinterpret_cast<const v4i*>(data), iters, clocks, sink);
+  MH_HIP(hipGetLastError());
+  return MARIAN_HIP_OK;
+}
 #endif
 
 int marian_hip_int8_prepare_a(const float* A, int8_t* Aq, int64_t M, int64_t K, void* workspace,
@@ -610,7 +650,36 @@ int marian_hip_int8_prepare_a(const float* A, int8_t* Aq, int64_t M, int64_t K, 
   }
   if(!workspace) return MARIAN_HIP_ERR_NULL;
   if(workspace_bytes < kWorkspaceBytes) return MARIAN_HIP_ERR_WORKSPACE;
-  if(!aligned(workspace, 4)) return MARIAN_HIP_ERR_ALIGN;
+  if(!aligned(workspace, 8)) return MARIAN_HIP_ERR_ALIGN;
+  // One pass over the input where it fits the register files of the chip's CUs (one workgroup per
+  // CU: 16.7 M values on 256 CUs) and is large enough for the second read to cost more than the
+  // exchange of the abs-max between the workgroups (measurement ids 700 / 701 force two passes /
+  // one pass; 702: one pass with no patience, every workgroup scans the whole input itself).
+  {
+    const int ov = kernel_override() % 1000;
+    const int cus = compute_units() < kOnePassMaxGroups ? compute_units() : kOnePassMaxGroups;
+    const size_t n16 = n / 16;
+    int sets = 1;
+    while(sets < 4 && (n16 + 1024 * (size_t)sets - 1) / (1024 * (size_t)sets) > (size_t)cus) sets *= 2;
+    const size_t groups = (n16 + 1024 * (size_t)sets - 1) / (1024 * (size_t)sets);
+    const bool fits = groups <= (size_t)cus;
+    if(fits && ov != 700 && (n >= kOnePassMinElems || ov == 701 || ov == 702)) {
+      unsigned char* ws = reinterpret_cast<unsigned char*>(workspace);
+      unsigned long long* slots = reinterpret_cast<unsigned long long*>(ws + kOnePassSlotsOffset);
+      unsigned long long* gen = reinterpret_cast<unsigned long long*>(ws + kOnePassGenOffset);
+      unsigned long long* mail = reinterpret_cast<unsigned long long*>(ws + kOnePassMailOffset);
+      const unsigned nonce = next_nonce();
+      const int spins = ov == 702 ? 0 : kOnePassSpinLimit;
+      if(sets == 1)
+        hipLaunchKernelGGL(prepare_a_onepass_kernel<1>, dim3((int)groups), dim3(1024), 0, st, A, (unsigned)n16, Aq, slots, gen, mail, nonce, spins);
+      else if(sets == 2)
+        hipLaunchKernelGGL(prepare_a_onepass_kernel<2>, dim3((int)groups), dim3(1024), 0, st, A, (unsigned)n16, Aq, slots, gen, mail, nonce, spins);
+      else
+        hipLaunchKernelGGL(prepare_a_onepass_kernel<4>, dim3((int)groups), dim3(1024), 0, st, A, (unsigned)n16, Aq, slots, gen, mail, nonce, spins);
+      MH_HIP(hipGetLastError());
+      return MARIAN_HIP_OK;
+    }
+  }
   float* partials = reinterpret_cast<float*>(workspace);
   const int g = absmax_blocks(n / 4);
   hipLaunchKernelGGL(absmax_partial_kernel, dim3(g), dim3(kQuantThreads), 0, st, A, n / 4,

@@ -6,8 +6,18 @@
 namespace marian_hip {
 
 constexpr int kQuantThreads = 256;
-constexpr int kMaxPartials = 1024;                  // floats of workspace used
-constexpr size_t kWorkspaceBytes = kMaxPartials * sizeof(float);
+constexpr int kMaxPartials = 1024;                  // floats of workspace used by the two-pass forms
+// Workspace layout: [0, 4 KB) abs-max partials of the two-pass forms; then the hand-over area of the
+// one-pass prepareA: 256 arrival slots of 8 bytes (a cache line each made no difference: 23.8 us
+// either way for 4096 x 4096), one generation word, and 16 mailboxes 256 bytes apart.
+constexpr int kOnePassMaxGroups = 256;              // workgroups of the one-pass form (one per CU)
+constexpr int kOnePassMailboxes = 16;
+constexpr int kOnePassStride = 1;                   // 8-byte words between two slots
+constexpr size_t kOnePassSlotsOffset = kMaxPartials * sizeof(float);
+constexpr size_t kOnePassGenOffset = kOnePassSlotsOffset + kOnePassMaxGroups * kOnePassStride * 8;
+constexpr size_t kOnePassMailOffset = 8192;
+constexpr size_t kWorkspaceBytes = kOnePassMailOffset + kOnePassMailboxes * 256;   // 12 KB
+static_assert(kOnePassGenOffset + 8 <= kOnePassMailOffset, "workspace layout");
 constexpr int kSingleBlockThreads = 1024;
 constexpr int kSingleBlockMaxElems = 32 * 1024;     // one workgroup does abs-max and quantize (beyond: 8.6 us against 6.4 us for two launches)
 
@@ -170,6 +180,139 @@ __global__ __launch_bounds__(kSingleBlockThreads) void prepare_a_single_block_ke
     o16[i] = q;
   }
   if(threadIdx.x == 0) *reinterpret_cast<float*>(out + (size_t)n16 * 16) = qm;
+}
+
+// ---- prepareA in one pass over the input ----------------------------------------------------
+// The two-pass form reads the fp32 input twice (abs-max, then quantize); at encoder sizes the
+// second read costs as much as the first (67 MB: 14 us each, the memory-side cache does not help).
+// Here the input stays in registers between the two steps: at most one workgroup of 1024 threads
+// per CU, each thread holding SETS x 16 values, so 256 CUs hold up to 16.7 M values (4096 x 4096).
+// In between, the workgroups exchange their abs-max through the workspace:
+//   * every workgroup stores (tag, abs-max bits) into its arrival slot - one 8-byte store at device
+//     scope, so tag and value arrive together;
+//   * workgroup 0 polls all slots (one slot per thread), takes the maximum and publishes (tag, max)
+//     to 16 mailboxes; the other workgroups poll one mailbox each (16 pollers per line);
+//   * nothing but these 8-byte words is handed over, so no fence is needed.
+// The tag is a host nonce plus a generation word that lives in the workspace and that workgroup 0
+// advances at the end of every launch: words left by an earlier launch - or by an earlier replay of
+// a recorded graph, which repeats the nonce - never match, whatever the workspace held before its
+// first use.  Every wait is bounded: a workgroup that runs out of patience (the device was shared
+// and not all workgroups were resident) takes the abs-max over the whole input itself - the
+// result is the same - clears its slot, and the launch still ends.
+template <int SETS>
+__global__ __launch_bounds__(1024) void prepare_a_onepass_kernel(const float* __restrict__ x, unsigned n16,
+                                                                 int8_t* __restrict__ out,
+                                                                 unsigned long long* slots,
+                                                                 unsigned long long* gen_word,
+                                                                 unsigned long long* mailboxes,
+                                                                 unsigned nonce, int spin_limit) {
+  __shared__ float red[1024 / kWave];
+  __shared__ float shared_max;
+  __shared__ unsigned shared_tag;
+  __shared__ __attribute__((aligned(16))) uint32_t turn[1024 * 4];   // 16 bytes per thread
+  const int tid = threadIdx.x, quad = tid / 4, qlane = tid % 4;
+  const int G = gridDim.x, g = blockIdx.x;
+  // (one thread per workgroup asks for the generation: every access to the word is served by the
+  // same memory channel, one after the other)
+  unsigned gen = 0;
+  if(tid == 0 && G > 1) gen = (unsigned)__hip_atomic_load(gen_word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  // set j of this workgroup: quads (g * SETS + j) * 256 .. + 255, a quad = four consecutive 16-value
+  // groups (256 contiguous bytes); load e brings lane i of the quad the i-th four values of group e
+  v4f vals[SETS][4];
+  bool live[SETS];
+  float m = 0.0f;
+#pragma unroll
+  for(int j = 0; j < SETS; ++j) {
+    const unsigned q = (unsigned)(g * SETS + j) * 256u + (unsigned)quad;
+    live[j] = 4u * q < n16;   // (n16 is a multiple of four: K % 64 == 0)
+    const unsigned qc = live[j] ? q : 0u;
+    const char* src = reinterpret_cast<const char*>(x) + (size_t)qc * 256 + qlane * 16;
+#pragma unroll
+    for(int e = 0; e < 4; ++e) vals[j][e] = *reinterpret_cast<const v4f*>(src + e * 64);
+  }
+#pragma unroll
+  for(int j = 0; j < SETS; ++j)
+    if(live[j]) {
+#pragma unroll
+      for(int e = 0; e < 4; ++e) m = abs4max(vals[j][e], m);
+    }
+  if(tid == 0) shared_tag = (nonce + gen) | 0x80000000u;   // never 0: a cleared word does not match
+  m = block_max(m, red);   // (its barriers also publish shared_tag)
+  const unsigned tag = shared_tag;
+
+  // abs-max over all of x by this workgroup alone (the way out of a wait that ran out)
+  auto scan_all = [&]() {
+    const v4f* x4 = reinterpret_cast<const v4f*>(x);
+    const size_t n4 = (size_t)n16 * 4;
+    float mm = 0.0f;
+    for(size_t i = tid; i < n4; i += 1024) mm = abs4max(x4[i], mm);
+    return block_max(mm, red);
+  };
+  auto pack = [](unsigned t, float v) { return ((unsigned long long)t << 32) | (unsigned long long)__float_as_uint(v); };
+  float amax = m;
+  if(G > 1) {
+    if(tid == 0) __hip_atomic_store(&slots[g * kOnePassStride], pack(tag, m), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    bool ok = true;
+    if(g == 0) {
+      float mine = 0.0f;
+      if(tid < G) {
+        ok = false;
+        for(int spin = 0; spin < spin_limit; ++spin) {
+          const unsigned long long w = __hip_atomic_load(&slots[tid * kOnePassStride], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          if((unsigned)(w >> 32) == tag) {
+            mine = __uint_as_float((unsigned)w);
+            ok = true;
+            break;
+          }
+          __builtin_amdgcn_s_sleep(4);
+        }
+      }
+      const bool all_ok = __syncthreads_and(ok ? 1 : 0) != 0;
+      amax = all_ok ? block_max(mine, red) : scan_all();
+      if(tid < kOnePassMailboxes)
+        __hip_atomic_store(&mailboxes[tid * 32], pack(tag, amax), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      // the next launch (or replay) expects another tag; every workgroup of this launch has read
+      // the generation by now, or will find its words unanswered and help itself
+      if(tid == 0) {
+        __hip_atomic_store(gen_word, (unsigned long long)(gen + 1u), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(&slots[0], 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    } else {
+      if(tid == 0) {
+        ok = false;
+        const unsigned long long* box = &mailboxes[(g % kOnePassMailboxes) * 32];
+        for(int spin = 0; spin < spin_limit; ++spin) {
+          const unsigned long long w = __hip_atomic_load(box, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          if((unsigned)(w >> 32) == tag) {
+            shared_max = __uint_as_float((unsigned)w);
+            ok = true;
+            break;
+          }
+          __builtin_amdgcn_s_sleep(8);
+        }
+        // answered or not, this launch is done with the slot
+        __hip_atomic_store(&slots[g * kOnePassStride], 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+      const bool answered = __syncthreads_and(ok ? 1 : 0) != 0;
+      amax = answered ? shared_max : scan_all();
+    }
+  }
+  const float qm = quant_mult_from_maxabs(amax);
+  const bool finite = qm < __builtin_inff();
+#pragma unroll
+  for(int j = 0; j < SETS; ++j) {
+    if(!live[j]) continue;
+    const unsigned q = (unsigned)(g * SETS + j) * 256u + (unsigned)quad;
+    // Lane i of the quad holds dword i of the quad's four 16-byte outputs; through LDS (the four
+    // lanes sit in one wave, whose LDS operations execute in order) it picks up the four dwords of
+    // output i, so that a wave stores 1 KB of contiguous bytes, 16 per lane.
+#pragma unroll
+    for(int e = 0; e < 4; ++e)
+      turn[(quad * 4 + e) * 4 + qlane] = finite ? quantize_pack4_finite(vals[j][e], qm) : quantize_pack4(vals[j][e], qm);
+    const uint4 w = *reinterpret_cast<const uint4*>(&turn[(quad * 4 + qlane) * 4]);
+    *reinterpret_cast<uint4*>(reinterpret_cast<char*>(out) + (size_t)q * 64 + qlane * 16) = w;
+  }
+  if(g == 0 && tid == 0) *reinterpret_cast<float*>(out + (size_t)n16 * 16) = qm;
 }
 
 // Pass 2 of prepareB: W fp32 [K x N] -> payload int8 [N x K] (quantized transpose) + tail.

@@ -86,6 +86,17 @@ def test_prepare_a_degenerate(integer, orc, kind, M, K):
     same_qtensor(integer.prepareA(dev(A)).numpy(), orc.prepare_a(A), "prepareA " + kind)
 
 
+@pytest.mark.parametrize("kernel", [700, 701])
+@pytest.mark.parametrize("kind", A_KINDS)
+def test_prepare_a_degenerate_both_forms(integer, orc, kind, kernel):
+    """the two-pass and the one-pass form of prepareA at a size both take"""
+    say("degenerate prepare_a forms", kind, kernel)
+    A = make_a(kind, 1024, 1024, 99)
+    with forced(kernel):
+        got = integer.prepareA(dev(A)).numpy()
+    same_qtensor(got, orc.prepare_a(A), "prepareA %s id %d" % (kind, kernel))
+
+
 @pytest.mark.parametrize("kind", A_KINDS)
 @pytest.mark.parametrize("K,N", [(64, 8), (512, 264), (1024, 1024)])
 def test_prepare_b_degenerate(integer, orc, kind, K, N):

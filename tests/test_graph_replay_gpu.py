@@ -62,3 +62,50 @@ def test_decoder_tail_replays(integer, synth):
         torch.cuda.synchronize()
         for got, w in zip(other, want):
             assert torch.equal(got, w)
+
+
+def test_one_pass_prepare_a_replays_with_new_inputs(integer, orc, synth):
+    """The one-pass prepareA hands the abs-max between its workgroups through tagged words in the
+    workspace.  A recorded graph repeats the host's part of the tag on every replay, so words left
+    by the previous replay must not be taken for this one's: the input changes between replays
+    (another abs-max, at another place) and every replay must give the checker's bytes.  The same
+    workspace also serves eager calls in between."""
+    import torch
+    from conftest import load
+    T = load("types")
+    M, K = 4096, 1024     # 4 M values: the one-pass form, all CUs
+    inputs = []
+    for r in range(4):
+        A = synth.normal(70 + r, synth.STREAM_A, (M, K), 1.0 + r)
+        A.flat[(r * 7919 + 13) % A.size] = np.float32(50.0 * (r + 1)) * (-1 if r % 2 else 1)
+        inputs.append(A)
+    want = [orc.prepare_a(A) for A in inputs]
+    dA = torch.from_numpy(inputs[0]).cuda()
+    out = integer.QTensor.empty((M, K), T.Type.intgemm8, "cuda")
+    be = integer.Backend.get(dA.device)
+
+    def call():
+        st = be.lib.marian_hip_int8_prepare_a(dA.data_ptr(), out.data_ptr(), M, K, be.workspace.data_ptr(),
+                                              be.workspace_bytes, be.stream())
+        assert st == 0
+
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        call()
+    torch.cuda.current_stream().wait_stream(s)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call()
+    for replay in range(8):
+        r = replay % 4
+        dA.copy_(torch.from_numpy(inputs[r]).cuda())
+        out.data.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert np.array_equal(out.numpy(), want[r]), "replay %d" % replay
+        if replay % 2:    # an eager call on another input, same workspace
+            other = integer.prepareA(torch.from_numpy(inputs[(r + 1) % 4]).cuda())
+            assert np.array_equal(other.numpy(), want[(r + 1) % 4])

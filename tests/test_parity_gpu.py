@@ -83,6 +83,26 @@ def test_prepare_a_keeps_leading_dims_and_saturates(integer, orc):
     assert got[30 * 64 - 1] == -127 and got[:-4].min() == -127
 
 
+@pytest.mark.parametrize("kernel", [0, 700, 701, 702])
+@pytest.mark.parametrize("M,K", [(2048, 1024), (4096, 1024), (4096, 4096), (3001, 1088), (128, 4096), (40, 1024),
+                                 (4100, 4096), (1500, 2048)])
+def test_prepare_a_one_pass_and_two_pass(integer, orc, synth, M, K, kernel):
+    """prepareA at encoder sizes: two passes over the input (id 700), one pass with the abs-max
+    exchanged between the workgroups (701; the automatic choice from 4 M values on), and one pass
+    in which no workgroup waits for the others and each scans the whole input itself (702, the way
+    out of a wait that ran out).  One, two and four 16-value sets per thread, ragged last
+    workgroups, inputs beyond what the one-pass form holds (4100 x 4096: two passes whatever the id)."""
+    if kernel == 702 and M * K > (4 << 20):
+        pytest.skip("every workgroup scanning 16 M values: correct, and slow on purpose")
+    say("prepare_a passes", M, K, kernel)
+    A = synth.normal(150 + M, synth.STREAM_A, (M, K), 1.0)
+    A.flat[(M * 31 + 7) % A.size] = np.float32(-9.5)      # the extreme sits in one workgroup's share
+    want = orc.prepare_a(A)
+    with forced(kernel):
+        got = integer.prepareA(dev(A)).numpy()
+    assert np.array_equal(got, want)
+
+
 @pytest.mark.parametrize("K,N", [(64, 8), (128, 24), (512, 2048), (2048, 512), (1024, 1000)])
 def test_prepare_b_bit_exact(integer, orc, synth, K, N):
     say("prepare_b", K, N)
