@@ -492,10 +492,9 @@ def probe_ceilings(torch):
         c = clocks.cpu().numpy().reshape(-1, 2).astype(np.float64)
         mhz = float(np.median(c[:, 0] / c[:, 1]) * 100.0)
         ops = 2.0 * 32 ** 3 * 8 * iters * 4 * wgs
-        in_loop_s = float(np.median(c[:, 1])) / 100e6
-        print("  %d workgroup(s) of 4 waves per CU: %7.1f TOPS over the launch (%.1f us), %7.1f TOPS inside the loop, "
+        print("  %d workgroup(s) of 4 waves per CU: %7.1f TOPS over the launch (%.1f us), "
               "shader clock %.0f MHz -> %d CUs x 8192 op/clk x clock = %.0f TOPS"
-              % (per_cu, ops / (med * 1e-3) / 1e12, med * 1e3, ops / in_loop_s / 1e12, mhz, cus, cus * 8192 * mhz * 1e6 / 1e12))
+              % (per_cu, ops / (med * 1e-3) / 1e12, med * 1e3, mhz, cus, cus * 8192 * mhz * 1e6 / 1e12))
 
 
 def measured_int8_peak(torch):
@@ -535,9 +534,12 @@ def pmc_summary(fetch_csv, write_csv):
         for key, pat in (("copy64", "vectorized_elementwise_kernel<4, at::native::CUDAFunctorOnSelf_add<float>"),
                          ("stream32_fused_M64_K512_N32000", "gemm_stream32_kernel<2, 4, 2, 8, 1, 4, 64"),
                          ("gemm_pair", "gemm_pair_kernel"), ("gemm_mfma32", "gemm_mfma32_kernel"),
-                         ("absmax", "absmax_partial_kernel"), ("quantize_a", "quantize_a_kernel")):
+                         ("absmax", "absmax_partial_kernel"), ("quantize_a", "quantize_a_kernel"),
+                         ("prepare_a_onepass", "prepare_a_onepass_kernel")):
             if pat in name:
-                return key + ("|" + name.split("gemm_mfma32_kernel")[1].split("(")[0] if key == "gemm_mfma32" else "")
+                if key in ("gemm_mfma32", "prepare_a_onepass"):   # keep the template arguments apart
+                    return key + "|" + name.split(pat)[1].split("(")[0]
+                return key
         return None
 
     def load(path, counter):
