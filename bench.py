@@ -114,134 +114,12 @@ class Op:
             assert r == 0, r
 
 
-class BigDecoder:
-    """Transformer-big decoder (6 layers, d = 1024, ffn = 4096, 16 heads, tied 32000-word output
-    layer) with random-init weights, driven through the host mirrors of the library: one full
-    decoding step at beam 4 x batch 32 (reference src/models/transformer.h:603-760 for the layer
-    structure, post-processing "dan", inference).  Self-attention keys/values of `t_past` earlier
-    positions and encoder keys/values of `src_len` positions are resident; K/V projections are
-    taken for the new position only.  Beam search itself (top-k, hypothesis bookkeeping) is not
-    part of the step."""
-
-    def __init__(self, torch, integer, ops, sets, t_past=20, src_len=60, seed=300):
-        self.torch, self.integer, self.ops = torch, integer, ops
-        self.d, self.ffn, self.V, self.H = 1024, 4096, 32000, 16
-        self.beam, self.batch = 4, 32
-        self.M = self.beam * self.batch
-        self.T, self.L = t_past + 1, src_len
-        g = torch.Generator(device="cuda")
-        g.manual_seed(seed)
-        d, ffn, V, H, M = self.d, self.ffn, self.V, self.H, self.M
-
-        def qw(K, N):
-            return integer.prepareB(torch.randn(K, N, device="cuda", generator=g) * 0.02)
-
-        def vec(n, scale=0.01, shift=0.0):
-            return torch.randn(n, device="cuda", generator=g) * scale + shift
-
-        first = {"layers": [], "out": (qw(d, V), vec(V))}
-        for _ in range(6):
-            ly = {}
-            for name, (K, N) in {"Wq": (d, d), "Wk": (d, d), "Wv": (d, d), "Wo": (d, d), "cWq": (d, d),
-                                 "cWo": (d, d), "W1": (d, ffn), "W2": (ffn, d)}.items():
-                ly[name] = (qw(K, N), vec(N))
-            for name in ("ln1", "ln2", "ln3"):
-                ly[name] = (vec(d, 0.1, 1.0), vec(d, 0.1))
-            first["layers"].append(ly)
-
-        def clone(x):
-            if isinstance(x, dict):
-                return {k: clone(v) for k, v in x.items()}
-            if isinstance(x, (list, tuple)):
-                return type(x)(clone(v) for v in x)
-            if isinstance(x, integer.QTensor):
-                return integer.QTensor(x.data.clone(), x.shape, x.type)
-            return x   # small fp32 vectors are shared
-        self.sets = [first] + [clone(first) for _ in range(sets - 1)]
-        self.weight_bytes = 6 * (6 * d * d + 2 * d * ffn) + d * V
-        self.gemm_ops = 2 * M * self.weight_bytes
-        # resident state
-        self.x = torch.randn(M, d, device="cuda", generator=g)
-        self.Kself = [torch.randn(M * H, self.T, d // H, device="cuda", generator=g) for _ in range(6)]
-        self.Vself = [torch.randn(M * H, self.T, d // H, device="cuda", generator=g) for _ in range(6)]
-        self.Kenc = [torch.randn(self.batch * H, self.L, d // H, device="cuda", generator=g) for _ in range(6)]
-        self.Venc = [torch.randn(self.batch * H, self.L, d // H, device="cuda", generator=g) for _ in range(6)]
-        # source lengths uniform over 20 .. 60, padded to the longest (the mask covers the rest)
-        lens = torch.randint(20, self.L + 1, (self.batch,), device="cuda", generator=g)
-        self.mask = (torch.arange(self.L, device="cuda")[None, :] >= lens[:, None]).float() * -99999999.0
-
-    def step(self, s, gemm_only=False, chained=True, grouped=True):
-        """chained: every tensor that feeds an affine call leaves its abs-max where it is
-        produced (layer norm, attention, the ReLU GEMM), so those calls skip their abs-max pass.
-        grouped: the self-attention projections Wq, Wk, Wv (one input, three weight matrices,
-        reference src/models/transformer.h:290-325) go through one call."""
-        integer, ops = self.integer, self.ops
-        W = self.sets[s % len(self.sets)]
-        H, M, d = self.H, self.M, self.d
-        dk = d // H
-        x, xmax = self.x, None
-        ch = chained and not gemm_only
-        for li, ly in enumerate(W["layers"]):
-            if grouped:   # one abs-max, one quantization, one launch for the three projections
-                (q, k, v), _ = integer.affine_f32_grouped(x, [ly["Wq"], ly["Wk"], ly["Wv"]], absmax=xmax)
-            else:
-                q, _ = integer.affine_f32(x, *ly["Wq"], absmax=xmax)
-                k, _ = integer.affine_f32(x, *ly["Wk"], absmax=xmax)
-                v, _ = integer.affine_f32(x, *ly["Wv"], absmax=xmax)
-            omax = x1max = comax = x2max = f1max = None
-            if gemm_only:
-                o = q
-            else:
-                # head split of a single position is a view; the attention call also appends the
-                # new key/value to the cache
-                o = ops.Attention(q.view(M * H, 1, dk), self.Kself[li], self.Vself[li], want_absmax=ch,
-                                  kNew=k.view(M * H, dk), vNew=v.view(M * H, dk))
-                if ch:
-                    o, omax = o
-                o = o.view(M, d)
-            a, _ = integer.affine_f32(o, *ly["Wo"], absmax=omax)
-            if gemm_only:
-                x1 = a
-            else:
-                x1 = ops.layerNorm(a, *ly["ln1"], eps=1e-6, add=x, want_absmax=ch)
-                if ch:
-                    x1, x1max = x1
-            cq, _ = integer.affine_f32(x1, *ly["cWq"], absmax=x1max)
-            if gemm_only:
-                co = cq
-            else:
-                co = ops.Attention(cq.view(M * H, 1, dk), self.Kenc[li], self.Venc[li], self.mask,
-                                   rowsPerMask=H, want_absmax=ch)
-                if ch:
-                    co, comax = co
-                co = co.view(M, d)
-            ca, _ = integer.affine_f32(co, *ly["cWo"], absmax=comax)
-            if gemm_only:
-                x2 = ca
-            else:
-                x2 = ops.layerNorm(ca, *ly["ln2"], eps=1e-6, add=x1, want_absmax=ch)
-                if ch:
-                    x2, x2max = x2
-            f1 = integer.affine_f32(x2, *ly["W1"], relu=True, absmax=x2max, want_absmax=ch)
-            if ch:
-                f1, _, f1max = f1
-            else:
-                f1 = f1[0]
-            f2, _ = integer.affine_f32(f1, *ly["W2"], absmax=f1max)
-            if gemm_only:
-                x = f2
-            else:
-                x = ops.layerNorm(f2, *ly["ln3"], eps=1e-6, add=x2, want_absmax=ch)
-                if ch:
-                    x, xmax = x
-        logits, _ = integer.affine_f32(x, *W["out"], absmax=xmax)
-        if gemm_only:
-            return logits
-        # log-probabilities, then the beam's n-best per sentence over beam x vocabulary
-        lp = ops.logsoftmax(logits)
-        # (the transposition to [batch, beam * V] of beam_search.cpp:472 happens inside the call)
-        ops.getNBestListOfBeams(lp.view(self.beam, 1, self.batch, self.V), self.beam)
-        return lp
+def BigDecoder(torch, integer, ops, sets):
+    """Transformer-big decoder step of the benchmark (configuration 3): 6 layers, d = 1024,
+    ffn = 4096, 16 heads, tied 32000-word output layer, beam 4 x batch 32, 20 cached target positions,
+    source lengths uniform 20..60."""
+    step_mod = importlib.import_module(PKG + ".decoder_step")
+    return step_mod.DecoderStep(sets=sets)
 
 
 def capture(torch, fn):
