@@ -39,6 +39,12 @@ SIGNATURES = {
     "marian_hip_int8_affine_shortlist": (_i, [_vp, _vp, _vp, _vp, _i64, _vp, _i64, _i64, _i64,
                                               _f, _i, _vp]),
     "marian_hip_int8_multiply_i32": (_i, [_vp, _vp, _vp, _i64, _vp, _i64, _i64, _i64, _vp]),
+    # include/marian_hip_int16.h
+    "marian_hip_int16_prepare_a": (_i, [_vp, _vp, _i64, _i64, _vp]),
+    "marian_hip_int16_prepare_b": (_i, [_vp, _vp, _i64, _i64, _vp]),
+    "marian_hip_int16_prepare_b_quantized_transposed": (_i, [_vp, _vp, _i64, _i64, _vp]),
+    "marian_hip_int16_affine": (_i, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _f, _i, _vp]),
+    "marian_hip_int16_multiply_i32": (_i, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),
     # include/marian_hip_ops.h
     "marian_hip_layer_norm": (_i, [_vp, _vp, _vp, _i64, _vp, _i64, _vp, _i64, _i64, _f, _vp, _vp]),
     "marian_hip_softmax": (_i, [_vp, _vp, _i64, _i64, _vp, _i64, _i64, _vp]),

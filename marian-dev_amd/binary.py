@@ -10,12 +10,10 @@ What differs from the reference loader (:88-114): a `Type::intgemm8` item is kep
 int8 W^T row-major [N, K] followed by the fp32 quantMult at byte K*N - because that is the layout the
 GPU kernels consume; the reference re-tiles it for the CPU it runs on (prepareAndTransposeB,
 src/tensors/cpu/integer_common.h:189-216).  Items whose type is one of the CPU-tiled variants
-(intgemm8ssse3/avx2/avx512/avx512vnni) cannot be used on a GPU and are refused.  So are the 16-bit
-intgemm types: their arithmetic (int16 operands, quantMult fixed at 1024,
-src/tensors/cpu/integer_common.h:174-175) exists for CPUs without 8-bit dot products and has no
-matrix-core form on gfx950; this backend implements the 8-bit path only and says so with the text
-of the reference's own dispatch (src/tensors/cpu/intgemm_interface.h:126).  A type id outside
-Marian's enum is reported with the item's name.
+(intgemm8ssse3/avx2/avx512/avx512vnni, intgemm16sse2/avx2/avx512) cannot be used on a GPU and are
+refused, and so are FBGEMM-packed items.  A hardware-agnostic `Type::intgemm16` item (int16 W^T
+[N, K] + quantMult 1024 at byte 2*K*N, src/tensors/cpu/expression_graph_packable.h:203-235) is kept
+verbatim like an intgemm8 one.  A type id outside Marian's enum is reported with the item's name.
 """
 import struct
 
@@ -37,13 +35,14 @@ class Item:
         self.bytes = np.ascontiguousarray(data).view(np.uint8).ravel()
 
     def quant_mult(self):
-        n = elements(self.shape)
+        n = elements(self.shape) * sizeOf(self.type)
         return self.bytes[n:n + 4].view(np.float32)[0]
 
     def payload(self):
-        """int8 W^T [N, K] for an intgemm8 item of logical shape [K, N]."""
+        """int8 (int16) W^T [N, K] for an intgemm8 (intgemm16) item of logical shape [K, N]."""
         K, N = self.shape
-        return self.bytes[: K * N].view(np.int8).reshape(N, K)
+        width = sizeOf(self.type)
+        return self.bytes[: K * N * width].view(np.int8 if width == 1 else np.int16).reshape(N, K)
 
 
 def _pad256(b):
@@ -57,6 +56,12 @@ def intgemm8_item(name, q_flat, shape):
     (reference src/tensors/cpu/expression_graph_packable.h:242-250)."""
     raw = np.ascontiguousarray(q_flat).view(np.uint8).tobytes()[: requiredBytes(shape, Type.intgemm8)]
     return Item(name, shape, Type.intgemm8, np.frombuffer(_pad256(raw), dtype=np.uint8))
+
+
+def intgemm16_item(name, q_flat, shape):
+    """Item for a 16-bit quantized weight: q_flat = int16 payload + quantMult tail (2*K*N + 4 bytes)."""
+    raw = np.ascontiguousarray(q_flat).view(np.uint8).tobytes()[: requiredBytes(shape, Type.intgemm16)]
+    return Item(name, shape, Type.intgemm16, np.frombuffer(_pad256(raw), dtype=np.uint8))
 
 
 def float_item(name, array):
@@ -120,17 +125,13 @@ def load_items(path):
         except ValueError:
             raise ValueError("Item {} has the unsupported item type 0x{:x} (this loader knows: {})".format(
                 name, h[1], ", ".join(t.name for t in Type))) from None
-        if isIntgemm(type_) and sizeOf(type_) != 1:
-            raise ValueError("Item {}: Unsupported type {} for Intgemm type?? (the HIP backend implements "
-                             "intgemm8 only; convert the model with marian-conv --gemm-type intgemm8)".format(
-                                 name, type_.name))
         if isPacked(type_):
             raise ValueError("Item {} has the FBGEMM-packed type {}: a CPU cache layout that a GPU backend "
                              "cannot consume (reference src/tensors/cpu/fbgemm/packed_gemm.h)".format(name, type_.name))
         if isHardwareSpecific(type_):
             raise ValueError(
                 "Item {} has the CPU-tiled type {}; a GPU backend needs the hardware-agnostic "
-                "intgemm8 payload (convert the model with marian-conv --gemm-type intgemm8)".format(
+                "intgemm8 / intgemm16 payload (convert the model with marian-conv --gemm-type intgemm8)".format(
                     name, type_.name))
         if isIntgemm(type_) and h[3] < requiredBytes(shape, type_):
             raise ValueError("Item {} is shorter than payload + quantMult".format(name))

@@ -21,6 +21,7 @@
 #include <string>
 #include <vector>
 
+#include "../../include/marian_hip_int16.h"
 #include "../../include/marian_hip_int8.h"
 #include "hip_device.h"
 
@@ -162,9 +163,15 @@ inline float getQuantMult(Backend& be, const Tensor& t) {
   return qm;
 }
 
-// Forward body of the prepareA node: out has shape of a, type intgemm8, requiredBytes(shape) bytes.
+// Forward body of the prepareA node: out has the shape of a and the type of the weights it will
+// meet - intgemm8 (abs-max quantMult) or intgemm16 (quantMult 1024) - and requiredBytes(shape) bytes.
 inline void prepareA(TensorAllocator& ta, const Tensor& a, Tensor& out) {
   if(!isFloat(a.type)) abortWith("Intgemm expects type of A to be float32");
+  if(out.type == Type::intgemm16) {
+    MARIAN_HIP_CHECK(marian_hip_int16_prepare_a(a.data<float>(), out.data<int16_t>(), rows(a), cols(a),
+                                                ta.backend().stream()));
+    return;
+  }
   void* ws = ta.workspace();   // (may allocate: before any pointer is read)
   MARIAN_HIP_CHECK(marian_hip_int8_prepare_a(a.data<float>(), out.data<int8_t>(), rows(a), cols(a), ws,
                                              ta.workspaceBytes(), ta.backend().stream()));
@@ -172,6 +179,11 @@ inline void prepareA(TensorAllocator& ta, const Tensor& a, Tensor& out) {
 
 // Offline quantizer body (marian-conv): w float32 [K, N] -> out intgemm8 [K, N] (payload W^T).
 inline void prepareB(TensorAllocator& ta, const Tensor& w, Tensor& out) {
+  if(out.type == Type::intgemm16) {
+    MARIAN_HIP_CHECK(marian_hip_int16_prepare_b(w.data<float>(), out.data<int16_t>(), w.shape[0], w.shape[1],
+                                                ta.backend().stream()));
+    return;
+  }
   void* ws = ta.workspace();
   MARIAN_HIP_CHECK(marian_hip_int8_prepare_b(w.data<float>(), out.data<int8_t>(), w.shape[0], w.shape[1],
                                              ws, ta.workspaceBytes(), ta.backend().stream()));
@@ -179,7 +191,8 @@ inline void prepareB(TensorAllocator& ta, const Tensor& w, Tensor& out) {
 
 inline void checkB(const Tensor& bQuant) {
   if(!isIntgemm(bQuant.type)) abortWith("Intgemm expects type of B to be a variant of intgemm");
-  if(isHardwareSpecific(bQuant.type) || sizeOf(bQuant.type) != 1) abortWith("Unsupported type for Intgemm type??");
+  if(isHardwareSpecific(bQuant.type) || (sizeOf(bQuant.type) != 1 && sizeOf(bQuant.type) != 2))
+    abortWith("Unsupported type for Intgemm type??");
 }
 
 // Forward body of the multiply node; bias may be null (dot).  relu fuses the in-place ReLU node.
@@ -187,6 +200,13 @@ inline void checkB(const Tensor& bQuant) {
 inline void multiply(Backend& be, const Tensor& aQuant, const Tensor& bQuant, const Tensor* bias, Tensor& out,
                      float scale, bool relu, const Tensor* shortlist = nullptr) {
   checkB(bQuant);
+  if(sizeOf(bQuant.type) == 2) {   // Type::intgemm16
+    if(shortlist) abortWith("the 16-bit path has no shortlist form");
+    MARIAN_HIP_CHECK(marian_hip_int16_affine(aQuant.data<int16_t>(), bQuant.data<int16_t>(),
+                                             bias ? bias->data<float>() : nullptr, out.data<float>(), rows(aQuant),
+                                             cols(aQuant), cols(bQuant), scale, relu ? 1 : 0, be.stream()));
+    return;
+  }
   if(shortlist)
     MARIAN_HIP_CHECK(marian_hip_int8_affine_shortlist(
         aQuant.data<int8_t>(), bQuant.data<int8_t>(), bias ? bias->data<float>() : nullptr,
@@ -220,6 +240,12 @@ inline void affineOrDot(TensorAllocator& ta, const Tensor& a, Tensor& aQuant, co
                         Tensor* absmaxOut = nullptr) {
   if(!isFloat(a.type)) abortWith("Intgemm expects type of A to be float32");
   checkB(bQuant);
+  if(sizeOf(bQuant.type) == 2) {   // Type::intgemm16: the two node bodies one after the other
+    if(aQuant.type != Type::intgemm16) abortWith("the prepareA node of a 16-bit weight must be typed intgemm16");
+    prepareA(ta, a, aQuant);
+    multiply(ta.backend(), aQuant, bQuant, bias, out, scale, relu, shortlist);
+    return;
+  }
   void* ws = ta.workspace();   // (may allocate and move the slab: before any pointer is read)
   const uint32_t* idx = shortlist ? shortlist->data<uint32_t>() : nullptr;
   const int64_t nIdx = shortlist ? (int64_t)shortlist->elements() : 0;

@@ -18,6 +18,7 @@
 //   float out2[M*N2]        affine(outRelu, W2), no bias
 //   float X[R*C], gamma[C], beta[C], ln[R*C] (eps 1e-6, skip input = X reversed), sm[R*C], lsm[R*C];
 //   float nbVal[R*nbestN]; uint32 nbKey[R*nbestN]     n-best of lsm
+//   int16 Aq16[M*K+2], Bq16[K*N+2]; float out16[M*N]  the 16-bit path: affine(A, W, bias), ReLU, scale 1
 #include <cmath>
 #include <cstring>
 #include <fstream>
@@ -117,6 +118,8 @@ int main(int argc, char** argv) {
          wantLsm = rd.take<float>((size_t)R * C);
     auto wantNbVal = rd.take<float>((size_t)R * nbestN);
     auto wantNbKey = rd.take<uint32_t>((size_t)R * nbestN);
+    auto wantAq16 = rd.take<int16_t>((size_t)M * K + 2), wantBq16 = rd.take<int16_t>((size_t)K * N + 2);
+    auto wantOut16 = rd.take<float>((size_t)M * N);
 
     Backend be(0);
     // a small step and a limit: growth happens often, and exhaustion can be provoked
@@ -259,17 +262,30 @@ int main(int argc, char** argv) {
     integer::affineOrDotStatic(be, a, bq, &b, oStatic, 1.0f, true);
     expect(sameBits(download<float>(be, oStatic, wantRelu.size()), wantRelu), "affineOrDotStatic (no Aq, no workspace)");
 
+    {   // the 16-bit path (Type::intgemm16) through the same wrappers, selected by the tensor types
+      Tensor aq16, bq16, o16;
+      ta.allocate(aq16, {M, K}, Type::intgemm16);
+      ta.allocate(bq16, {K, N}, Type::intgemm16);
+      ta.allocate(o16, {M, N}, Type::float32);
+      integer::prepareB(ta, w, bq16);
+      integer::affineOrDot(ta, a, aq16, bq16, &b, o16, 1.0f, /*relu=*/true);
+      expect(sameBits(download<int16_t>(be, bq16, wantBq16.size()), wantBq16) &&
+                 sameBits(download<int16_t>(be, aq16, wantAq16.size()), wantAq16),
+             "intgemm16: prepareB and prepareA, payload and quantMult 1024");
+      expect(sameBits(download<float>(be, o16, wantOut16.size()), wantOut16), "intgemm16: affineOrDot, bit for bit");
+    }
+
     // error paths: the reference's messages, as exceptions
     {
       bool tiled = false, sixteen = false, notq = false;
       Tensor t = bq;
       t.type = Type::intgemm8avx512;
       try { integer::affineOrDot(ta, a, aq, t, &b, o); } catch(const std::runtime_error& e) { tiled = std::strstr(e.what(), "Unsupported type") != nullptr; }
-      t.type = Type::intgemm16;
+      t.type = Type::intgemm16avx2;
       try { integer::affineOrDot(ta, a, aq, t, &b, o); } catch(const std::runtime_error& e) { sixteen = std::strstr(e.what(), "Unsupported type") != nullptr; }
       t.type = Type::float32;
       try { integer::affineOrDot(ta, a, aq, t, &b, o); } catch(const std::runtime_error& e) { notq = std::strstr(e.what(), "variant of intgemm") != nullptr; }
-      expect(tiled && sixteen && notq, "CPU-tiled, 16-bit and float weights are refused with the reference's texts");
+      expect(tiled && sixteen && notq, "CPU-tiled 8- and 16-bit and float weights are refused with the reference's texts");
     }
 
     // ---- float operators through their wrappers ----

@@ -66,8 +66,8 @@ class QTensor:
         return self.data[: self.elements()]
 
     def numpy(self):
-        """payload + tail as host bytes (elements + 4)."""
-        return self.data[: self.elements() + 4].cpu().numpy()
+        """payload + tail as host bytes (requiredBytes: elements * element size + 4)."""
+        return self.data[: requiredBytes(self.shape, self.type)].cpu().numpy()
 
     def data_ptr(self):
         return self.data.data_ptr()
@@ -86,7 +86,7 @@ def rows(t):
 def getQuantMult(q):
     """reference src/tensors/cpu/integer_common.h:101-111 (device read; for tests and tools)."""
     _abort_if(not isIntgemm(q.type), "getQuantMult does not work for type {}", q.type)
-    n = q.elements()
+    n = q.elements() * sizeOf(q.type)
     return float(q.data[n:n + 4].cpu().numpy().view(np.float32)[0])
 
 
@@ -162,14 +162,19 @@ def _backend_of(t):
     return Backend.get(dev)
 
 
-def prepareA(a):
-    """reference src/tensors/cpu/intgemm_interface.h:17-32 for vtype = intgemm8."""
+def prepareA(a, type_=Type.intgemm8):
+    """reference src/tensors/cpu/intgemm_interface.h:17-32 for vtype = intgemm8 (abs-max quantMult)
+    or intgemm16 (quantMult 1024, src/tensors/cpu/integer_common.h:174-175)."""
     _abort_if(a.dtype != torch.float32, "Intgemm expects type of A to be float32 not {}", a.dtype)
+    _abort_if(type_ not in (Type.intgemm8, Type.intgemm16), "Unsupported type {} for Intgemm type??", type_)
     a = a.contiguous()
     be = _backend_of(a)
-    out = QTensor.empty(a.shape, Type.intgemm8, a.device)
+    out = QTensor.empty(a.shape, type_, a.device)
     K = cols(a)
     M = rows(a) if a.numel() else 0
+    if type_ == Type.intgemm16:
+        _lib.check(be.lib.marian_hip_int16_prepare_a(a.data_ptr(), out.data_ptr(), M, K, be.stream()), "prepareA")
+        return out
     st = be.lib.marian_hip_int8_prepare_a(a.data_ptr(), out.data_ptr(), M, K,
                                           be.workspace.data_ptr(), be.workspace_bytes, be.stream())
     _lib.check(st, "prepareA")
@@ -180,12 +185,15 @@ def prepareB(w, type_=Type.intgemm8):
     """Offline weight quantizer, reference src/tensors/cpu/expression_graph_packable.h:153-253
     (intgemm8 branch): fp32 W [K, N] -> Type::intgemm8 tensor of shape [K, N] whose payload is
     the quantized transpose."""
-    _abort_if(type_ != Type.intgemm8, "Type {} is not supported", type_)
+    _abort_if(type_ not in (Type.intgemm8, Type.intgemm16), "Type {} is not supported", type_)
     _abort_if(w.dtype != torch.float32 or w.dim() != 2, "prepareB expects a float32 matrix, got {}", w.dtype)
     w = w.contiguous()
     be = _backend_of(w)
     K, N = w.shape
-    out = QTensor.empty((K, N), Type.intgemm8, w.device)
+    out = QTensor.empty((K, N), type_, w.device)
+    if type_ == Type.intgemm16:   # the 16-bit branch of the packer (:203-235): quantMult 1024
+        _lib.check(be.lib.marian_hip_int16_prepare_b(w.data_ptr(), out.data_ptr(), K, N, be.stream()), "prepareB")
+        return out
     st = be.lib.marian_hip_int8_prepare_b(w.data_ptr(), out.data_ptr(), K, N,
                                           be.workspace.data_ptr(), be.workspace_bytes, be.stream())
     _lib.check(st, "prepareB")
@@ -205,10 +213,13 @@ def affineOrDot(a, bQuant, bias=None, transA=False, transB=False, scale=1.0, rel
     _abort_if(not isinstance(bQuant, QTensor) or not isIntgemm(bQuant.type),
               "Intgemm expects type of B to be a variant of intgemm not {}",
               getattr(bQuant, "type", type(bQuant)))
-    _abort_if(isHardwareSpecific(bQuant.type) or sizeOf(bQuant.type) != 1,
+    _abort_if(isHardwareSpecific(bQuant.type) or sizeOf(bQuant.type) not in (1, 2),
               "Unsupported type {} for Intgemm type??", bQuant.type)
     if transA:
         a = a.transpose(-1, -2)
+    if sizeOf(bQuant.type) == 2:   # Type::intgemm16: the two nodes one after the other
+        _abort_if(shortlist is not None, "the 16-bit path has no shortlist form (type {})", bQuant.type)
+        return multiply(prepareA(a, Type.intgemm16), bQuant, bias, scale=scale, relu=relu)
     out, _ = affine_f32(a, bQuant, bias, scale=scale, relu=relu, shortlist=shortlist)
     return out
 
@@ -316,7 +327,13 @@ def multiply(aQuant, bQuant, bias=None, scale=1.0, relu=False, shortlist=None):
         _abort_if(bias.dtype != torch.float32 or bias.numel() != N, "bias must be float32 [1, {}]", N)
         bias = bias.contiguous()
         bias_ptr = bias.data_ptr()
-    if shortlist is None:
+    _abort_if(sizeOf(aQuant.type) != sizeOf(bQuant.type), "Intgemm operands of different widths: {} and {}",
+              aQuant.type, bQuant.type)
+    if sizeOf(bQuant.type) == 2:
+        _abort_if(shortlist is not None, "the 16-bit path has no shortlist form (type {})", bQuant.type)
+        st = be.lib.marian_hip_int16_affine(aQuant.data_ptr(), bQuant.data_ptr(), bias_ptr, out.data_ptr(), M, K, N,
+                                            scale, int(relu), be.stream())
+    elif shortlist is None:
         st = be.lib.marian_hip_int8_affine(aQuant.data_ptr(), bQuant.data_ptr(), bias_ptr,
                                            out.data_ptr(), M, K, N, scale, int(relu), be.stream())
     else:
@@ -335,6 +352,11 @@ def multiply_i32(aQuant, bQuant, shortlist=None):
     M = rows(aQuant) if aQuant.elements() else 0
     n_out = N if shortlist is None else int(shortlist.numel())
     acc = torch.empty(aQuant.shape[:-1] + (n_out,), dtype=torch.int32, device=aQuant.data.device)
+    if sizeOf(bQuant.type) == 2:
+        _abort_if(shortlist is not None, "the 16-bit path has no shortlist form (type {})", bQuant.type)
+        _lib.check(be.lib.marian_hip_int16_multiply_i32(aQuant.data_ptr(), bQuant.data_ptr(), acc.data_ptr(), M, K, N,
+                                                        be.stream()), "multiply_i32")
+        return acc
     st = be.lib.marian_hip_int8_multiply_i32(aQuant.data_ptr(), bQuant.data_ptr(),
                                              None if shortlist is None else shortlist.data_ptr(),
                                              n_out if shortlist is not None else 0, acc.data_ptr(),

@@ -9,7 +9,7 @@ import pytest
 
 from conftest import ROOT, load
 
-HEADERS = [os.path.join(ROOT, "include", h) for h in ("marian_hip_int8.h", "marian_hip_ops.h")]
+HEADERS = [os.path.join(ROOT, "include", h) for h in ("marian_hip_int8.h", "marian_hip_int16.h", "marian_hip_ops.h")]
 TUNING_HEADER = os.path.join(ROOT, "include", "marian_hip_int8_tuning.h")
 
 

@@ -64,11 +64,10 @@ def test_unaligned_item_is_refused_on_save(tmp_path):
                      [B.Item("a", (3,), T.Type.float32, np.zeros(12, np.uint8))])
 
 
-@pytest.mark.parametrize("name", ["intgemm16", "intgemm16sse2", "intgemm16avx2", "intgemm16avx512"])
-def test_sixteen_bit_intgemm_items_are_refused_with_the_reference_text(tmp_path, name):
-    """The HIP backend implements the 8-bit path; a 16-bit item (int16 payload, quantMult 1024,
-    reference src/tensors/cpu/integer_common.h:174-175) is refused at load with the text of the
-    reference's dispatch (src/tensors/cpu/intgemm_interface.h:126), naming the item."""
+@pytest.mark.parametrize("name", ["intgemm16sse2", "intgemm16avx2", "intgemm16avx512"])
+def test_cpu_tiled_sixteen_bit_items_are_refused(tmp_path, name):
+    """The CPU-tiled 16-bit variants (what the reference turns an intgemm16 item into at load,
+    src/common/binary.cpp:108-110) cannot be consumed by a GPU."""
     B = load("binary")
     T = load("types")
     raw = np.zeros(64 * 8 * 2 + 4, np.uint8)
@@ -76,8 +75,25 @@ def test_sixteen_bit_intgemm_items_are_refused_with_the_reference_text(tmp_path,
     it = B.Item("decoder_l1_ffn_W1", (64, 8), T.Type[name], np.frombuffer(B._pad256(raw.tobytes()), np.uint8))
     path = os.path.join(tmp_path, "w16.bin")
     B.save_items(path, [it])
-    with pytest.raises(ValueError, match=r"decoder_l1_ffn_W1: Unsupported type %s for Intgemm type\?\?" % name):
+    with pytest.raises(ValueError, match="decoder_l1_ffn_W1 has the CPU-tiled type %s" % name):
         B.load_items(path)
+
+
+def test_sixteen_bit_item_roundtrip_keeps_the_payload_verbatim(tmp_path, synth):
+    """A hardware-agnostic Type::intgemm16 item: int16 W^T [N, K] then quantMult 1024 at byte 2*K*N
+    (reference src/tensors/cpu/expression_graph_packable.h:203-235), kept as stored."""
+    from oracle import oracle16
+    B = load("binary")
+    T = load("types")
+    W = synth.normal(5, synth.STREAM_W, (64, 24), 0.02)
+    q = oracle16.prepare_b(W)
+    path = os.path.join(tmp_path, "m16.bin")
+    B.save_items(path, [B.intgemm16_item("decoder_l1_ffn_W1", q, (64, 24))])
+    (w,) = B.load_items(path)
+    assert w.type == T.Type.intgemm16 and w.shape == (64, 24) and w.quant_mult() == 1024.0
+    assert T.requiredBytes(w.shape, w.type) == 64 * 24 * 2 + 4
+    want = np.clip(np.rint((W.T * f32(1024.0)).astype(f32)), -32768, 32767).astype(np.int16)
+    assert np.array_equal(w.payload(), want)
 
 
 def test_unknown_item_type_is_reported_with_the_item_name(tmp_path):
@@ -97,14 +113,15 @@ def test_unknown_item_type_is_reported_with_the_item_name(tmp_path):
         B.load_items(path)
 
 
-def test_operator_refuses_sixteen_bit_weights_with_the_reference_text():
-    """affineOrDot's type switch (reference src/tensors/cpu/intgemm_interface.h:104-127): anything
-    but an 8-bit hardware-agnostic intgemm weight ends in its default branch."""
+def test_operator_refuses_cpu_tiled_weights_with_the_reference_text():
+    """affineOrDot's type switch (reference src/tensors/cpu/intgemm_interface.h:104-127): on a GPU
+    only the hardware-agnostic intgemm8 and intgemm16 weights can be multiplied; the CPU-tiled
+    variants end in the default branch."""
     import torch
     integer = load("integer")
     T = load("types")
     a = torch.zeros(2, 64)
-    for t in (T.Type.intgemm16, T.Type.intgemm16avx2, T.Type.intgemm8avx2):
+    for t in (T.Type.intgemm16avx2, T.Type.intgemm8avx2, T.Type.intgemm16sse2):
         w = integer.QTensor(torch.zeros(64 * 8 * 2 + 4, dtype=torch.int8), (64, 8), t)
         with pytest.raises(integer.MarianRuntimeError, match=r"Unsupported type .*%s.* for Intgemm type\?\?" % t.name):
             integer.affineOrDot(a, w)

@@ -749,13 +749,16 @@ def write_host_check_fixture(path, orc, synth):
     ln = decode_ops.layer_norm(X, gamma, beta, 1e-6, add=Xrev)
     sm, lsm = decode_ops.softmax(X), decode_ops.logsoftmax(X)
     nb_val, nb_key = decode_ops.nbest(lsm, nbestN)
+    from oracle import oracle16
+    Aq16, Bq16 = oracle16.prepare_a(A), oracle16.prepare_b(W)
+    out16, _ = oracle16.affine(Aq16, Bq16, bias, M, K, N, 1.0, True)
     with open(path, "wb") as f:
         f.write(b"MHC2")
         f.write(np.array([M, K, N, N2, idx.size, R, C, nbestN], np.int32).tobytes())
         for arr, ty in [(A, f32), (W, f32), (bias, f32), (W2, f32), (idx, np.uint32), (Aq, np.int8), (Bq, np.int8),
                         (Bq2, np.int8), (acc, np.int32), (out_relu, f32), (out_sl, f32), (out2, f32), (X, f32),
                         (gamma, f32), (beta, f32), (ln, f32), (sm, f32), (lsm, f32), (nb_val, f32),
-                        (nb_key, np.uint32)]:
+                        (nb_key, np.uint32), (Aq16, np.int16), (Bq16, np.int16), (out16, f32)]:
             f.write(np.ascontiguousarray(arr, dtype=ty).tobytes())
 
 
