@@ -77,7 +77,7 @@ class Op:
         self.Aq = integer.QTensor.empty((M, K), integer.Type.intgemm8, "cuda")
         W = torch.randn(K, N, device="cuda", generator=g) * 0.02
         first = integer.prepareB(W)
-        self.Bq = [first] + [integer.QTensor(first.data.clone(), first.shape, first.type)
+        self.Bq = [first] + [integer.QTensor(first.data.clone(), first.shape, first.type, first.prepared)
                              for _ in range(copies - 1)]
         self.idx = idx
         self.n_out = N if idx is None else int(idx.numel())

@@ -11,10 +11,21 @@
  * src/tensors/cpu/integer_common.h:101-106): `elements` int8 values followed by one fp32
  * quantMult at byte offset `elements`.
  *   activations  Aq : int8 row-major [M x K]            + quantMult tail  (M*K + 4 bytes)
- *   weights      Bq : int8 row-major [N x K] = W^T      + quantMult tail  (K*N + 4 bytes)
- *                     i.e. logical B[k, n] lives at byte n*K + k, exactly the payload of a
- *                     Type::intgemm8 item in a Marian .bin model file
- *                     (src/tensors/cpu/expression_graph_packable.h:160-201,242-250).
+ *   weights      Bq : the K*N int8 values of W^T        + quantMult tail  (K*N + 4 bytes), in one of
+ *                     two orders, like the reference's hardware-agnostic and hardware-specific types:
+ *     file order     : row-major [N x K], logical B[k, n] at byte n*K + k - the payload of a
+ *                      Type::intgemm8 item in a Marian .bin model file
+ *                      (src/tensors/cpu/expression_graph_packable.h:160-201,242-250).  No GEMM entry
+ *                      point takes it; marian_hip_int8_prepare_b_quantized_transposed converts it.
+ *     prepared order : what marian_hip_int8_prepare_b and _prepare_b_quantized_transposed write and
+ *                      every GEMM entry point reads ("K-blocked").  K is cut into sub-steps of 32
+ *                      values; within a sub-step the N columns follow each other in groups of eight;
+ *                      a group is 256 bytes: the lower 16 K values of its eight columns, 16 bytes per
+ *                      column, then the upper 16:
+ *                        byte of B[k, n] = (k/32)*32*N + (n/8)*256 + ((k/16)%2)*128 + (n%8)*16 + k%16
+ *                      (the counterpart of intgemm's own CPU tilings, which the reference produces
+ *                      with PrepareBQuantizedTransposed, src/tensors/cpu/integer_common.h:189-216:
+ *                      the operand of one gfx950 matrix instruction is 1 KB of consecutive memory).
  *
  * Shape rules (intgemm's own): K % 64 == 0, N % 8 == 0, shortlist length % 8 == 0.
  * Alignment: A, Aq, Bq, out and acc 16 bytes; bias and idx 4 bytes.
@@ -42,7 +53,8 @@ enum {
   MARIAN_HIP_ERR_WORKSPACE = 4, /* workspace too small */
   MARIAN_HIP_ERR_HIP = 5,       /* HIP runtime error, see marian_hip_last_hip_error() */
   MARIAN_HIP_ERR_RANGE = 6,     /* size exceeds what the kernels index (2^31 - 1 elements) */
-  MARIAN_HIP_ERR_STATIC_LIMIT = 7 /* M * K exceeds MARIAN_HIP_STATIC_MAX_ELEMS (static-scratch entry point) */
+  MARIAN_HIP_ERR_STATIC_LIMIT = 7, /* M * K exceeds MARIAN_HIP_STATIC_MAX_ELEMS (static-scratch entry point) */
+  MARIAN_HIP_ERR_ALIAS = 8      /* input and output overlap where the call cannot work in place */
 };
 
 /* Human-readable text for a status code (host pointer, static storage). */
@@ -71,7 +83,7 @@ int marian_hip_int8_prepare_a(const float* A, int8_t* Aq, int64_t M, int64_t K,
  * Replaces the intgemm8 branch of the offline packer, reference
  * src/tensors/cpu/expression_graph_packable.h:160-201: quantMult over the untransposed fp32
  * W [K x N], Transpose10, Int8::PrepareA on the transpose, quantMult stored at byte K*N.
- * Bq: K*N + 4 bytes, receives the [N x K] payload and the tail.
+ * Bq: K*N + 4 bytes, receives the payload in prepared order and the tail.
  */
 int marian_hip_int8_prepare_b(const float* W, int8_t* Bq, int64_t K, int64_t N,
                               void* workspace, size_t workspace_bytes, void* stream);
@@ -79,8 +91,9 @@ int marian_hip_int8_prepare_b(const float* W, int8_t* Bq, int64_t K, int64_t N,
 /*
  * Replaces prepareAndTransposeB<intgemm8>, reference
  * src/tensors/cpu/integer_common.h:189-216 (Kernels8::PrepareBQuantizedTransposed + tail
- * copy), which re-tiles the file payload for a CPU.  The GPU kernels consume the file
- * payload as it is, so this is a device-to-device copy of K*N + 4 bytes.
+ * copy), which re-tiles the file payload for the CPU it runs on; here: file order -> prepared
+ * order, and the tail.  in, out: K*N + 4 bytes each, 16-byte aligned, not overlapping
+ * (MARIAN_HIP_ERR_ALIAS).  K % 64 == 0, N % 8 == 0.
  */
 int marian_hip_int8_prepare_b_quantized_transposed(const int8_t* in, int8_t* out, int64_t K,
                                                    int64_t N, void* stream);

@@ -16,7 +16,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libmarian_hip_int8.so")
 TUNING_LIB_PATH = os.path.join(_HERE, "libmarian_hip_int8_tuning.so")
 
-OK, ERR_NULL, ERR_SHAPE, ERR_ALIGN, ERR_WORKSPACE, ERR_HIP, ERR_RANGE, ERR_STATIC_LIMIT = range(8)
+OK, ERR_NULL, ERR_SHAPE, ERR_ALIGN, ERR_WORKSPACE, ERR_HIP, ERR_RANGE, ERR_STATIC_LIMIT, ERR_ALIAS = range(9)
 
 # name -> (restype, argtypes); the single place the Python side states the ABI
 _c = ctypes

@@ -16,8 +16,6 @@
 #ifdef MARIAN_HIP_TUNING
 // kernel families that only measurements select, and the switches that select them
 #include "../../include/marian_hip_int8_tuning.h"
-#include "gemm_persistent_kernel.h"
-#include "gemm_tile_kernel.h"
 #include "probe_kernels.h"
 #endif
 
@@ -95,38 +93,15 @@ int launch_stream(const GemmArgs& a, hipStream_t st) {
   return MARIAN_HIP_OK;
 }
 
-#ifdef MARIAN_HIP_TUNING
-template <int WNT, int WMT>
-int launch_tile(const GemmArgs& a, hipStream_t st) {
-  using Cfg = TileCfg<WNT, WMT>;
-  auto kernel = gemm_tile_kernel<WNT, WMT>;
-  static std::atomic<uint64_t> lds_done{0};
-  const int lds_status = allow_lds(kernel, Cfg::kLdsBytes, lds_done);
-  if(lds_status != MARIAN_HIP_OK) return lds_status;
-  int tiles_n = (a.n_out + Cfg::BN - 1) / Cfg::BN;
-  int tiles_m = (a.M + Cfg::BM - 1) / Cfg::BM;
-  hipLaunchKernelGGL(kernel, dim3(tiles_n * tiles_m), dim3(Cfg::kThreads), Cfg::kLdsBytes, st, a,
-                     tiles_n, tiles_m);
-  MH_HIP(hipGetLastError());
-  return MARIAN_HIP_OK;
-}
-#endif
-
 template <int BM, int BN, int WM, int WN, int NSTAGE, bool PAIRED = true, bool NT = false>
 int launch_big(const GemmArgs& a, hipStream_t st) {
   using Cfg = BigCfg<BM, BN, WM, WN, NSTAGE>;
-  // whole 128-column K blocks, or (paired-fragment form) a last block of 64 columns; measurement id
-  // 350 keeps the 16x16x64 tile kernel for such K
+  // whole 128-column K blocks, or (paired-fragment form) a last block of 64 columns
   const int tiles_n = (a.n_out + BN - 1) / BN;
   const int tiles_m = (a.M + BM - 1) / BM;
   if(a.K % Cfg::BK != 0) {
-#ifdef MARIAN_HIP_TUNING
-    if(!PAIRED || a.K % 64 != 0 || kernel_override() % 1000 == 350)
-      return launch_tile<4, 4>(a, st);
-#else
-    static_assert(PAIRED, "the shipped dispatch uses the paired-fragment form only");
     if(a.K % 64 != 0) return MARIAN_HIP_ERR_SHAPE;   // (refused by the argument checks already)
-#endif
+    // (the plain-fragment forms, which only measurements select, have no half block)
     if constexpr(!Cfg::kHalfTailOk || !PAIRED) {
       return launch_big<128, 128, 2, 4, 2, true, NT>(a, st);
     } else {
@@ -391,31 +366,6 @@ int launch_stream32_auto(const GemmArgs& a, const FusedSrc& f, hipStream_t st, i
   }
 }
 
-#ifdef MARIAN_HIP_TUNING
-template <int BM, int BN, int WM, int WN, int NSTAGE, bool DIRECT = false>
-int launch_persistent(const GemmArgs& a, hipStream_t st, int per_cu = 1, int stagger = 0) {
-  using Cfg = PersistCfg<BM, BN, WM, WN, NSTAGE, DIRECT>;
-  // needs K % 128 == 0, at least NSTAGE K blocks per tile and a 16-byte aligned bias
-  if(a.K % Cfg::BK != 0 || a.K / Cfg::BK < NSTAGE || (a.bias && !aligned(a.bias, 16)))
-    return launch_big<BM, BN, WM, WN, 2>(a, st);
-  auto dense = gemm_persistent_kernel<BM, BN, WM, WN, NSTAGE, false, DIRECT>;
-  auto gather = gemm_persistent_kernel<BM, BN, WM, WN, NSTAGE, true, DIRECT>;
-  static std::atomic<uint64_t> dense_done{0}, gather_done{0};
-  const int lds_status = allow_lds(dense, Cfg::kLdsBytes, dense_done) | allow_lds(gather, Cfg::kLdsBytes, gather_done);
-  if(lds_status != MARIAN_HIP_OK) return lds_status;
-  int tiles_n = (a.n_out + BN - 1) / BN;
-  int tiles_m = (a.M + BM - 1) / BM;
-  int total = tiles_n * tiles_m;
-  int slots = compute_units() * per_cu;
-  int grid = total < slots ? total : slots;
-  if(grid < slots) stagger = 0;   // fewer workgroups than slots: no two share a CU by design
-  hipLaunchKernelGGL(a.idx ? gather : dense, dim3(grid), dim3(Cfg::kThreads), Cfg::kLdsBytes, st, a,
-                     tiles_n, tiles_m, stagger);
-  MH_HIP(hipGetLastError());
-  return MARIAN_HIP_OK;
-}
-#endif
-
 // wide: many weight rows, every wave streams its own rows over the whole K
 // narrow: few weight rows, the four waves split K and reduce
 template <int MT>
@@ -441,10 +391,6 @@ int launch_gemm(const GemmArgs& a, hipStream_t st) {
   switch(which) {
     case 101: if(a.M <= 128) return launch_stream_auto(a, st, 1); break;
     case 102: if(a.M <= 128) return launch_stream_auto(a, st, 2); break;
-    case 201: return launch_tile<4, 4>(a, st);
-    case 202: return launch_tile<8, 4>(a, st);
-    case 203: return launch_tile<4, 8>(a, st);
-    case 204: return launch_tile<2, 2>(a, st);
     case 301: return launch_big<256, 256, 2, 4, 2>(a, st);
     case 302: return launch_big<128, 128, 2, 2, 2>(a, st);
     case 303: return launch_big<256, 128, 2, 2, 2>(a, st);
@@ -472,16 +418,6 @@ int launch_gemm(const GemmArgs& a, hipStream_t st) {
     case 512: return launch_stream32_auto<kPrequant>(a, FusedSrc(), st, 2);
     case 514: return launch_stream32_auto<kPrequant>(a, FusedSrc(), st, 4);
     case 518: return launch_stream32_auto<kPrequant>(a, FusedSrc(), st, 8);
-    case 411: return launch_persistent<128, 128, 2, 2, 2, true>(a, st, 2, 0);
-    case 412: return launch_persistent<128, 128, 2, 2, 2, true>(a, st, 2, 1);
-    case 413: return launch_persistent<128, 128, 2, 2, 2, true>(a, st, 2, 2);
-    case 414: return launch_persistent<128, 128, 2, 2, 2, true>(a, st, 2, 3);
-    case 415: return launch_persistent<128, 128, 2, 2, 2, true>(a, st, 1, 0);
-    case 416: return launch_persistent<128, 128, 2, 2, 4, true>(a, st, 1, 0);
-    case 401: return launch_persistent<128, 128, 2, 2, 4>(a, st);
-    case 402: return launch_persistent<128, 128, 2, 2, 3>(a, st);
-    case 403: return launch_persistent<128, 128, 2, 2, 2>(a, st);
-    case 404: return launch_persistent<256, 128, 2, 2, 2>(a, st);
     default: break;
   }
 #endif
@@ -590,13 +526,14 @@ const char* marian_hip_status_string(int status) {
     case MARIAN_HIP_ERR_RANGE: return "tensor too large for 32-bit element indices";
     case MARIAN_HIP_ERR_STATIC_LIMIT:
       return "activations exceed MARIAN_HIP_STATIC_MAX_ELEMS, the capacity of the library's static scratch";
+    case MARIAN_HIP_ERR_ALIAS: return "input and output overlap";
     default: return "unknown status";
   }
 }
 
 int marian_hip_last_hip_error(void) { return g_last_hip_error; }
 
-int marian_hip_int8_abi_version(void) { return 2; }
+int marian_hip_int8_abi_version(void) { return 3; }
 
 size_t marian_hip_int8_workspace_bytes(void) { return kWorkspaceBytes; }
 
@@ -718,9 +655,16 @@ int marian_hip_int8_prepare_b_quantized_transposed(const int8_t* in, int8_t* out
                                                    int64_t N, void* stream) {
   if(!in || !out) return MARIAN_HIP_ERR_NULL;
   if(K <= 0 || N <= 0) return MARIAN_HIP_ERR_SHAPE;
-  if(in == out) return MARIAN_HIP_OK;
-  MH_HIP(hipMemcpyAsync(out, in, (size_t)K * (size_t)N + sizeof(float), hipMemcpyDeviceToDevice,
-                        reinterpret_cast<hipStream_t>(stream)));
+  if((K % 64) != 0 || (N % 8) != 0) return MARIAN_HIP_ERR_SHAPE;
+  if(K * N > kMaxElems) return MARIAN_HIP_ERR_RANGE;
+  if(!aligned(in, 16) || !aligned(out, 16)) return MARIAN_HIP_ERR_ALIGN;
+  // the two layouts are permutations of each other: not in place
+  const int8_t* in_end = in + K * N + sizeof(float);
+  if(in < out + K * N + (int64_t)sizeof(float) && out < in_end) return MARIAN_HIP_ERR_ALIAS;
+  const size_t chunks = (size_t)K * (size_t)N / 16;
+  hipLaunchKernelGGL(retile_b_kernel, dim3((unsigned)((chunks + 255) / 256)), dim3(256), 0,
+                     reinterpret_cast<hipStream_t>(stream), in, (int)K, (int)N, out);
+  MH_HIP(hipGetLastError());
   return MARIAN_HIP_OK;
 }
 

@@ -5,11 +5,13 @@
 // (32 cycles for 32x32x32 MACs; the 16x16x64 form issues at roughly half that rate).  Operand
 // traffic into a CU (about 64 bytes per clock through the vector L1) is the limit, so a
 // workgroup owns a large BM x BN output tile and each operand byte enters the CU once per tile:
-//   * K advances in 128-byte blocks.  A row of a block is one full 128-byte line in global
-//     memory (both operands are K-contiguous).  One global_load_lds_dwordx4 per wave moves 8
-//     rows (1 KB) straight into LDS; the lane that fills 16-byte slot p of row r fetches chunk
-//     p ^ ((r >> 1) & 7) of that row, so LDS holds each row with its chunks XOR-swizzled and the
-//     MFMA fragment reads (32 consecutive rows, one chunk each) are bank-conflict free.
+//   * K advances in 128-byte blocks.  A row of a block is one full 128-byte line of the
+//     activations in global memory.  One global_load_lds_dwordx4 per wave moves 8 rows (1 KB)
+//     straight into LDS; the lane that fills 16-byte slot p of row r fetches chunk p ^ ((r >> 1) & 7)
+//     of that row, so LDS holds each row with its chunks XOR-swizzled and the MFMA fragment reads
+//     (32 consecutive rows, one chunk each) are bank-conflict free.  The K-blocked weights need no
+//     swizzle: 32 columns x one sub-step are 1 KB of consecutive memory in operand order, one wave
+//     load copies them into LDS as they are, and a fragment read covers that 1 KB once.
 //   * NSTAGE LDS buffers; the loads of block k + NSTAGE are issued as soon as block k has been
 //     read, so they have NSTAGE - 1 blocks of MFMA time to land.
 //   * Fragments are double-buffered in registers: the ds_reads of sub-step s + 1 (also across
@@ -204,20 +206,28 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * kWave) void gemm_mfma32_kernel(
 
   // ---- global -> LDS: load j of this wave fills rows (j*kWaves + wave)*8 .. +7 of a stage.
   // Rows past the matrix edge re-read the last valid row; their products are never stored.
+  // Weights: load g = (j - kLoadsA) * kWaves + wave of a stage brings sub-step g / (BN/32) of the 32
+  // columns of tile g % (BN/32): 1 KB that is consecutive in the K-blocked weights (consecutive g:
+  // consecutive memory) and lands in LDS as it is, lane q holding half (q >> 3) & 1 of column
+  // (q >> 4) * 8 + (q & 7) of the tile - the layout the fragment reads below expect.  With a
+  // shortlist the lanes gather their columns.
+  constexpr int kTilesN = BN / 32;
   int goff[Cfg::kLoads];
 #pragma unroll
   for(int j = 0; j < Cfg::kLoads; ++j) {
-    const int row = (j * Cfg::kWaves + wave) * 8 + lane / 8;
-    const int chunk = (lane % 8) ^ ((row >> 1) & 7);
-    int src;
     if(j < Cfg::kLoadsA) {
-      src = min(m0 + row, M - 1);
+      const int row = (j * Cfg::kWaves + wave) * 8 + lane / 8;
+      const int chunk = (lane % 8) ^ ((row >> 1) & 7);
+      goff[j] = min(m0 + row, M - 1) * K + chunk * 16;
     } else {
-      const int n = min(n0 + row - BM, args.n_out - 1);
-      src = args.idx ? (int)args.idx[n] : n;
+      const int g = (j - Cfg::kLoadsA) * Cfg::kWaves + wave;
+      const int sub = g / kTilesN, tile = g % kTilesN;
+      const int n = min(n0 + tile * 32 + (lane >> 4) * 8 + (lane & 7), args.n_out - 1);
+      const int src = args.idx ? (int)args.idx[n] : n;
+      goff[j] = (int)b_chunk_offset(src, 2 * sub + ((lane >> 3) & 1), args.N);   // (K * N < 2^31)
     }
-    goff[j] = src * K + chunk * 16;
   }
+  const size_t b_block = (size_t)Cfg::BK * (size_t)args.N;   // bytes of all columns per K block
   // A half last block: the lanes of the upper four 16-byte chunks of a row would read past the
   // row (past the buffer, for the last row), so they re-read the lower half instead; what they
   // stage is never multiplied.  The chunk of a lane is the same for all its loads (the number of
@@ -225,10 +235,16 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * kWave) void gemm_mfma32_kernel(
   static_assert(Cfg::kWaves % 2 == 0, "the chunk of a lane must not depend on the load index");
   const int tail_adj = (((lane % 8) ^ ((((wave * 8 + lane / 8) >> 1)) & 7)) >= 4) ? 64 : 0;
   auto issue_one = [&](int kb, int stage, int j, auto check_tail) __attribute__((always_inline)) {
-    const int8_t* base = (j < Cfg::kLoadsA) ? args.Aq : args.Bq;
+    const bool is_a = j < Cfg::kLoadsA;
+    const int8_t* base = is_a ? args.Aq + (size_t)kb * Cfg::BK : args.Bq + (size_t)kb * b_block;
     int voff = goff[j];
-    if(decltype(check_tail)::value && half_tail && kb == KB - 1) voff -= tail_adj;
-    global_load_lds16(base + (size_t)kb * Cfg::BK, (unsigned)voff,
+    // (a half block has no chunks 4 .. 7 and no sub-steps 2, 3: such loads go two sub-steps back, 64
+    // bytes of an activation row or 64 * N bytes of the weights; what they stage is never multiplied)
+    if(decltype(check_tail)::value && half_tail && kb == KB - 1) {
+      if(is_a) voff -= tail_adj;
+      else if(((j - Cfg::kLoadsA) * Cfg::kWaves + wave) / kTilesN >= 2) voff -= 64 * args.N;
+    }
+    global_load_lds16(base, (unsigned)voff,
                       lds_base + stage * Cfg::kStageBytes + (j * Cfg::kWaves + wave) * 1024);
   };
   auto issue = [&](int kb) {
@@ -237,12 +253,14 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * kWave) void gemm_mfma32_kernel(
     for(int j = 0; j < Cfg::kLoads; ++j) issue_one(kb, stage, j, std::true_type());
   };
 
-  // ---- fragment addressing: lane (li, lg) reads row li of a 32-row tile, chunk kk*2 + lg ----
+  // ---- fragment addressing: lane (li, lg) reads row li of a 32-row activation tile, chunk kk*2 + lg;
+  //      of the weights, its 16 bytes of the 1 KB block (sub-step kk, column tile), see above ----
   int frag_off[4];
 #pragma unroll
   for(int kk = 0; kk < 4; ++kk) frag_off[kk] = li * 128 + (((kk * 2 + lg) ^ ((li >> 1) & 7)) * 16);
   const int a_row0 = wm * Cfg::WTM * 32;          // first activation row of this wave in a stage
-  const int b_row0 = BM + wn * Cfg::WTN * 32;     // first weight row
+  // this lane's 16 bytes of sub-step 0 of the wave's first column tile
+  const int b_frag0 = BM * 128 + wn * Cfg::WTN * 1024 + (li >> 3) * 256 + lg * 128 + (li & 7) * 16;
 
   v4i af[PAIRED ? 4 : 2][Cfg::WTM], bf[PAIRED ? 4 : 2][Cfg::WTN];
   auto read_frags = [&](int stage, int kk, int set) {
@@ -250,19 +268,19 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * kWave) void gemm_mfma32_kernel(
 #pragma unroll
     for(int a = 0; a < Cfg::WTM; ++a)
       af[set][a] = *reinterpret_cast<const v4i*>(buf + (a_row0 + a * 32) * 128);
+    const int8_t* bbuf = lds + stage * Cfg::kStageBytes + b_frag0 + kk * kTilesN * 1024;
 #pragma unroll
-    for(int b = 0; b < Cfg::WTN; ++b)
-      bf[set][b] = *reinterpret_cast<const v4i*>(buf + (b_row0 + b * 32) * 128);
+    for(int b = 0; b < Cfg::WTN; ++b) bf[set][b] = *reinterpret_cast<const v4i*>(bbuf + b * 1024);
   };
 
   // fragment `idx` of the pair of sub-steps (0, 1): idx = set * (WTM + WTN) + f
   auto read_one = [&](int stage, int idx) {
     const int set = idx / (Cfg::WTM + Cfg::WTN), f = idx % (Cfg::WTM + Cfg::WTN);
-    const int8_t* buf = lds + stage * Cfg::kStageBytes + frag_off[set];
+    const int8_t* buf = lds + stage * Cfg::kStageBytes;
     if(f < Cfg::WTM)
-      af[set][f] = *reinterpret_cast<const v4i*>(buf + (a_row0 + f * 32) * 128);
+      af[set][f] = *reinterpret_cast<const v4i*>(buf + frag_off[set] + (a_row0 + f * 32) * 128);
     else
-      bf[set][f - Cfg::WTM] = *reinterpret_cast<const v4i*>(buf + (b_row0 + (f - Cfg::WTM) * 32) * 128);
+      bf[set][f - Cfg::WTM] = *reinterpret_cast<const v4i*>(buf + b_frag0 + (set * kTilesN + f - Cfg::WTM) * 1024);
   };
 
   v16i acc[Cfg::WTM][Cfg::WTN];

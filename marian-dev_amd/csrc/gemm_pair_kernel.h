@@ -100,22 +100,32 @@ __global__ __launch_bounds__(PairCfg::kThreads) void gemm_pair_kernel(GemmArgs a
   }
   const int m0 = tm * BM, n0 = tn * 2 * BN;   // n0: first column of the first tile of the pair
 
-  // ---- global -> LDS: load j of this wave fills rows (j*4 + wave)*8 .. +7 of a stage ----
+  // ---- global -> LDS: activation load j of this wave fills rows (j*4 + wave)*8 .. +7 of a stage;
+  //      weight load g = (j - kLoadsA) * 4 + wave copies the 1 KB block (sub-step g / 4, column tile
+  //      g % 4) of the K-blocked weights as it is (see gemm_mfma32_kernel.h) ----
+  constexpr int kTilesN = BN / 32;
   unsigned goff[Cfg::kLoads];
 #pragma unroll
   for(int j = 0; j < Cfg::kLoads; ++j) {
-    const int row = (j * Cfg::kWaves + wave) * 8 + lane / 8;
-    const int chunk = (lane % 8) ^ ((row >> 1) & 7);
-    const int src = j < Cfg::kLoadsA ? m0 + row : n0 + row - BM;
-    goff[j] = (unsigned)src * (unsigned)K + chunk * 16;
+    if(j < Cfg::kLoadsA) {
+      const int row = (j * Cfg::kWaves + wave) * 8 + lane / 8;
+      const int chunk = (lane % 8) ^ ((row >> 1) & 7);
+      goff[j] = (unsigned)(m0 + row) * (unsigned)K + chunk * 16;
+    } else {
+      const int g = (j - Cfg::kLoadsA) * Cfg::kWaves + wave;
+      const int sub = g / kTilesN, tile = g % kTilesN;
+      goff[j] = (unsigned)b_chunk_offset(n0 + tile * 32 + (lane >> 4) * 8 + (lane & 7), 2 * sub + ((lane >> 3) & 1), args.N);
+    }
   }
-  const int8_t* const b_tile1 = args.Bq + (size_t)BN * (size_t)K;   // weight rows of the second tile
+  const int8_t* const b_tile1 = args.Bq + b_column_offset(BN);   // weight columns of the second tile
+  const size_t b_block = (size_t)Cfg::BK * (size_t)args.N;        // bytes of all columns per K block
   // K block g of the stream: tile g / KB, block g % KB of its K
   auto issue_one = [&](int g, int stage, int j) __attribute__((always_inline)) {
     const bool second = g >= KB;
     const int kb = second ? g - KB : g;
-    const int8_t* base = (j < Cfg::kLoadsA) ? args.Aq : (second ? b_tile1 : args.Bq);
-    global_load_lds16(base + (size_t)kb * Cfg::BK, goff[j],
+    const int8_t* base = (j < Cfg::kLoadsA) ? args.Aq + (size_t)kb * Cfg::BK
+                                            : (second ? b_tile1 : args.Bq) + (size_t)kb * b_block;
+    global_load_lds16(base, goff[j],
                       lds_base + stage * Cfg::kStageBytes + (j * Cfg::kWaves + wave) * 1024);
   };
 
@@ -124,13 +134,14 @@ __global__ __launch_bounds__(PairCfg::kThreads) void gemm_pair_kernel(GemmArgs a
 #pragma unroll
   for(int kk = 0; kk < 4; ++kk) frag_off[kk] = li * 128 + (((kk * 2 + lg) ^ ((li >> 1) & 7)) * 16);
   const int a_row0 = wm * Cfg::WTM * 32;
-  const int b_row0 = BM + wn * Cfg::WTN * 32;
+  // this lane's 16 bytes of sub-step 0 of the wave's first column tile
+  const int b_frag0 = BM * 128 + wn * Cfg::WTN * 1024 + (li >> 3) * 256 + lg * 128 + (li & 7) * 16;
   v4i af[4][Cfg::WTM], bf[4][Cfg::WTN];
   // fragment f (0..5: four activation, two weight) of sub-step / register set kk
   auto read_one = [&](int stage, int kk, int f) __attribute__((always_inline)) {
-    const int8_t* buf = lds + stage * Cfg::kStageBytes + frag_off[kk];
-    if(f < Cfg::WTM) af[kk][f] = *reinterpret_cast<const v4i*>(buf + (a_row0 + f * 32) * 128);
-    else bf[kk][f - Cfg::WTM] = *reinterpret_cast<const v4i*>(buf + (b_row0 + (f - Cfg::WTM) * 32) * 128);
+    const int8_t* buf = lds + stage * Cfg::kStageBytes;
+    if(f < Cfg::WTM) af[kk][f] = *reinterpret_cast<const v4i*>(buf + frag_off[kk] + (a_row0 + f * 32) * 128);
+    else bf[kk][f - Cfg::WTM] = *reinterpret_cast<const v4i*>(buf + b_frag0 + (kk * kTilesN + f - Cfg::WTM) * 1024);
   };
 
   // ---- dequantization constants and the write-out addresses of the first tile ----

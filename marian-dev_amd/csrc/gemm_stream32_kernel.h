@@ -170,7 +170,9 @@ __global__ __launch_bounds__(WN * KW * kWave) void gemm_stream32_kernel(GemmArgs
 #pragma unroll
     for(int i = 0; i < kAbsmaxSlots / kStream32Threads; ++i) amax = fmaxf(amax, pm[i]);
   }
-  const int8_t* wrow = args.Bq + (size_t)wsrc * (size_t)K + lg * 16;
+  // this lane's 16 bytes of K sub-step 0; a sub-step further is w_step bytes further for every column
+  const int8_t* wrow = args.Bq + b_column_offset(wsrc) + lg * 128;
+  const size_t w_step = 32u * (size_t)args.N;
   __builtin_amdgcn_sched_barrier(0);
 
   // FUSED: the fp32 activations are requested before anything else - they are needed first, and
@@ -285,18 +287,19 @@ __global__ __launch_bounds__(WN * KW * kWave) void gemm_stream32_kernel(GemmArgs
   v4i w[Cfg::PW];
   const int kw_s = __builtin_amdgcn_readfirstlane(kw);   // (a scalar for the compiler)
   const int step0 = kw * Cfg::PW;                        // this wave's first sub-step within a chunk
-  // weights of a chunk: 32 * PW consecutive bytes of the lane's weight row, one pointer and
-  // constant offsets when the wave's sub-steps all lie within K, clamped one by one otherwise
+  // weights of a chunk: PW sub-steps of the lane's column (a wave reads 1 KB of consecutive memory
+  // per sub-step), one pointer and uniform offsets when the wave's sub-steps all lie within K,
+  // clamped one by one otherwise
   auto load_weights = [&](int chunk, v4i (&dst)[Cfg::PW]) __attribute__((always_inline)) {
     if(chunk * Cfg::CS + (kw_s + 1) * Cfg::PW <= S) {
-      const int8_t* wp = wrow + (chunk * Cfg::CS + step0) * 32;
+      const int8_t* wp = wrow + (size_t)(chunk * Cfg::CS + step0) * w_step;
 #pragma unroll
-      for(int p = 0; p < Cfg::PW; ++p) dst[p] = load16(wp + p * 32);
+      for(int p = 0; p < Cfg::PW; ++p) dst[p] = load16(wp + (size_t)p * w_step);
     } else {
 #pragma unroll
       for(int p = 0; p < Cfg::PW; ++p) {
         const int s = chunk * Cfg::CS + step0 + p;
-        dst[p] = load16(wrow + min(s, S - 1) * 32);
+        dst[p] = load16(wrow + (size_t)min(s, S - 1) * w_step);
       }
     }
   };

@@ -47,12 +47,14 @@ __global__ __launch_bounds__(WN * KW * kWave) void gemm_stream_kernel(GemmArgs a
   // weight rows of this lane
   const int n_base = (blockIdx.x * WN + wn) * NT * 16;
   const int8_t* wrow[NT];
+  const size_t w_step = 64u * (size_t)args.N;   // bytes from one K step of 64 to the next, for every column
 #pragma unroll
   for(int nt = 0; nt < NT; ++nt) {
     int n = n_base + nt * 16 + li;
     int src = 0;
     if(n < args.n_out) src = args.idx ? (int)args.idx[n] : n;
-    wrow[nt] = args.Bq + (size_t)src * (size_t)K + lg * 16;
+    // 16-byte chunk lg of K step 0: sub-step lg / 2, half lg % 2
+    wrow[nt] = args.Bq + b_chunk_offset(src, lg, args.N);
   }
 
   // activation staging: 16-byte slot t of a stage is (step, m-tile, lane) in operand order
@@ -90,7 +92,7 @@ __global__ __launch_bounds__(WN * KW * kWave) void gemm_stream_kernel(GemmArgs a
 #pragma unroll
       for(int nt = 0; nt < NT; ++nt) {
         v4i v = {0, 0, 0, 0};
-        if(s < KS) v = load16(wrow[nt] + s * 64);
+        if(s < KS) v = load16(wrow[nt] + (size_t)s * w_step);
         w[p][nt] = v;
       }
     }

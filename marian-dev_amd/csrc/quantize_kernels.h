@@ -315,9 +315,9 @@ __global__ __launch_bounds__(1024) void prepare_a_onepass_kernel(const float* __
   if(g == 0 && tid == 0) *reinterpret_cast<float*>(out + (size_t)n16 * 16) = qm;
 }
 
-// Pass 2 of prepareB: W fp32 [K x N] -> payload int8 [N x K] (quantized transpose) + tail.
-// A workgroup transposes a 64(k) x 64(n) tile through LDS: reads are coalesced along n,
-// writes are 16-byte runs along k.
+// Pass 2 of prepareB: W fp32 [K x N] -> K-blocked int8 payload of the quantized transpose + tail.
+// A workgroup transposes a 64(k) x 64(n) tile through LDS: reads are coalesced along n, writes are
+// 16-byte chunks of K values, eight neighbouring columns side by side.
 __global__ __launch_bounds__(256) void quantize_b_transpose_kernel(
     const float* __restrict__ W, int K, int N, const float* __restrict__ partials,
     int n_partials, int8_t* __restrict__ out) {
@@ -344,16 +344,33 @@ __global__ __launch_bounds__(256) void quantize_b_transpose_kernel(
     tile[tn][kk / 4] = quantize_pack4(v, qm);
   }
   __syncthreads();
-  // 64 rows (n) x 64 bytes (k): 4 threads per row, 16 bytes each
-  const int rn = threadIdx.x / 4, ck = (threadIdx.x % 4) * 16;
+  // 64 columns (n) x four 16-byte chunks (k): a wave writes one chunk of all 64 columns, which in the
+  // K-blocked layout is eight runs of 128 bytes
+  const int rn = threadIdx.x % 64, ck = (threadIdx.x / 64) * 16;
   int n = n0 + rn, k = k0 + ck;
   if(n < N && k < K) {  // K % 64 == 0, so a 16-byte run is inside or outside as a whole
     uint4 v;
     v.x = tile[rn][ck / 4]; v.y = tile[rn][ck / 4 + 1]; v.z = tile[rn][ck / 4 + 2]; v.w = tile[rn][ck / 4 + 3];
-    *reinterpret_cast<uint4*>(out + (size_t)n * K + k) = v;
+    *reinterpret_cast<uint4*>(out + b_chunk_offset(n, k / 16, N)) = v;
   }
   if(blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0)
     *reinterpret_cast<float*>(out + (size_t)K * N) = qm;
+}
+
+// prepareBQuantizedTransposed: int8 W^T as plain rows [N x K] (the payload of a model file) -> the
+// K-blocked layout.  One 16-byte chunk per thread, in output order (writes are consecutive).
+__global__ __launch_bounds__(256) void retile_b_kernel(const int8_t* __restrict__ in, int K, int N,
+                                                       int8_t* __restrict__ out) {
+  const size_t chunks = (size_t)K * (size_t)N / 16;
+  const size_t o = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if(o < chunks) {
+    // chunk o of the output: sub-step o / (2 N), then group of eight columns, half, column
+    const int s = (int)(o / (2 * (size_t)N)), rem = (int)(o % (2 * (size_t)N));
+    const int n = (rem / 16) * 8 + rem % 8, half = (rem / 8) % 2;
+    const uint4 v = *reinterpret_cast<const uint4*>(in + (size_t)n * K + (size_t)(2 * s + half) * 16);
+    *reinterpret_cast<uint4*>(out + o * 16) = v;
+  }
+  if(o == 0) *reinterpret_cast<float*>(out + (size_t)K * N) = *reinterpret_cast<const float*>(in + (size_t)K * N);
 }
 
 }  // namespace marian_hip

@@ -53,7 +53,7 @@ class DecoderStep:
             if isinstance(x, (list, tuple)):
                 return type(x)(clone(v) for v in x)
             if isinstance(x, integer.QTensor):
-                return integer.QTensor(x.data.clone(), x.shape, x.type)
+                return integer.QTensor(x.data.clone(), x.shape, x.type, x.prepared)
             return x   # small fp32 vectors are shared
         self.sets = [first] + [clone(first) for _ in range(sets - 1)]
         self.weight_bytes = layers * (6 * d * d + 2 * d * ffn) + d * V

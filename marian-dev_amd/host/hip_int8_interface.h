@@ -177,7 +177,8 @@ inline void prepareA(TensorAllocator& ta, const Tensor& a, Tensor& out) {
                                              ta.workspaceBytes(), ta.backend().stream()));
 }
 
-// Offline quantizer body (marian-conv): w float32 [K, N] -> out intgemm8 [K, N] (payload W^T).
+// Offline quantizer body (marian-conv): w float32 [K, N] -> out intgemm8 [K, N] (payload: the quantized W^T
+// in the order the kernels read).
 inline void prepareB(TensorAllocator& ta, const Tensor& w, Tensor& out) {
   if(out.type == Type::intgemm16) {
     MARIAN_HIP_CHECK(marian_hip_int16_prepare_b(w.data<float>(), out.data<int16_t>(), w.shape[0], w.shape[1],
@@ -187,6 +188,21 @@ inline void prepareB(TensorAllocator& ta, const Tensor& w, Tensor& out) {
   void* ws = ta.workspace();
   MARIAN_HIP_CHECK(marian_hip_int8_prepare_b(w.data<float>(), out.data<int8_t>(), w.shape[0], w.shape[1],
                                              ws, ta.workspaceBytes(), ta.backend().stream()));
+}
+
+// A quantized weight item as a model file holds it (plain rows [N, K] + quantMult) -> the order the
+// kernels read; reference prepareAndTransposeB, src/tensors/cpu/integer_common.h:189-216 (there: the
+// tiling of the CPU the process runs on).  in and out are different tensors of the same shape and type.
+inline void prepareAndTransposeB(Backend& be, const Tensor& in, Tensor& out) {
+  if(!isIntgemm(in.type) || isHardwareSpecific(in.type) || in.type != out.type)
+    abortWith("prepareAndTransposeB expects a hardware-agnostic intgemm matrix");
+  if(in.type == Type::intgemm16) {
+    MARIAN_HIP_CHECK(marian_hip_int16_prepare_b_quantized_transposed(in.data<int16_t>(), out.data<int16_t>(),
+                                                                     in.shape[0], in.shape[1], be.stream()));
+    return;
+  }
+  MARIAN_HIP_CHECK(marian_hip_int8_prepare_b_quantized_transposed(in.data<int8_t>(), out.data<int8_t>(), in.shape[0],
+                                                                  in.shape[1], be.stream()));
 }
 
 inline void checkB(const Tensor& bQuant) {

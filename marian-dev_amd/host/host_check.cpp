@@ -10,9 +10,10 @@
 // affineOrDot calls and in the middle of a chained pair, so the "nothing is retained between
 // calls" contract of the library is exercised, not assumed.
 //
-// Fixture layout (little endian): "MHC2", int32 M, K, N, N2, nIdx, R, C, nbestN; then
+// Fixture layout (little endian): "MHC3", int32 M, K, N, N2, nIdx, R, C, nbestN; then
 //   float A[M*K], W[K*N], bias[N], W2[N*N2]; uint32 idx[nIdx];
-//   int8 Aq[M*K+4], Bq[K*N+4], Bq2[N*N2+4]; int32 acc[M*N];
+//   int8 Aq[M*K+4], Bq[K*N+4], Bq2[N*N2+4] (weights in the order the kernels read), fileBq[K*N+4] (the same
+//   values as a model file holds them, rows [N, K]); int32 acc[M*N];
 //   float outRelu[M*N]      affine(A, W, bias), ReLU, scale 1
 //   float outSl[M*nIdx]     affine over the shortlist idx, no ReLU, scale 0.5
 //   float out2[M*N2]        affine(outRelu, W2), no bias
@@ -101,7 +102,7 @@ int main(int argc, char** argv) {
   try {
     Reader rd(argv[1]);
     auto magic = rd.take<char>(4);
-    if(std::memcmp(magic.data(), "MHC2", 4) != 0) abortWith("not a host_check fixture");
+    if(std::memcmp(magic.data(), "MHC3", 4) != 0) abortWith("not a host_check fixture");
     auto dims = rd.take<int32_t>(8);
     const int M = dims[0], K = dims[1], N = dims[2], N2 = dims[3], nIdx = dims[4], R = dims[5], C = dims[6],
               nbestN = dims[7];
@@ -110,6 +111,7 @@ int main(int argc, char** argv) {
     auto idx = rd.take<uint32_t>(nIdx);
     auto wantAq = rd.take<int8_t>((size_t)M * K + 4), wantBq = rd.take<int8_t>((size_t)K * N + 4),
          wantBq2 = rd.take<int8_t>((size_t)N * N2 + 4);
+    auto fileBq = rd.take<int8_t>((size_t)K * N + 4);
     auto wantAcc = rd.take<int32_t>((size_t)M * N);
     auto wantRelu = rd.take<float>((size_t)M * N), wantSl = rd.take<float>((size_t)M * nIdx),
          want2 = rd.take<float>((size_t)M * N2);
@@ -220,7 +222,16 @@ int main(int argc, char** argv) {
     integer::prepareB(ta, w2, bq2);
     expect(sameBits(download<int8_t>(be, bq, wantBq.size()), wantBq) &&
                sameBits(download<int8_t>(be, bq2, wantBq2.size()), wantBq2),
-           "prepareB: payload and quantMult as the checker's");
+           "prepareB: the checker's values and quantMult, in the order the kernels read");
+    {
+      Tensor fromFile = upload(ta, fileBq, {K, N}, Type::intgemm8), retiled;
+      ta.allocate(retiled, {K, N}, Type::intgemm8);
+      integer::prepareAndTransposeB(be, fromFile, retiled);
+      expect(sameBits(download<int8_t>(be, retiled, wantBq.size()), wantBq),
+             "prepareAndTransposeB: a model file's rows [N, K] re-tiled to the same bytes as prepareB");
+      ta.free(retiled);
+      ta.free(fromFile);
+    }
     integer::prepareA(ta, a, aq);
     const void* aqBefore = aq.data<void>();
     expect(forceMove(ta, ballast) && aq.data<void>() != aqBefore, "slab moved between prepareA and multiply");

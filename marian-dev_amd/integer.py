@@ -16,7 +16,7 @@ import weakref
 import numpy as np
 import torch
 
-from . import _lib
+from . import _lib, layout
 from .types import Type, elements, isFloat, isHardwareSpecific, isIntgemm, requiredBytes, sizeOf
 
 MarianRuntimeError = _lib.MarianHipError
@@ -36,20 +36,26 @@ class QTensor:
     bytes (reference src/tensors/allocator.h:86,178-181); `shape` is the logical shape
     ([.., K] for activations, [K, N] for weights whose payload is the transposed [N, K])."""
 
-    def __init__(self, data, shape, type_):
+    def __init__(self, data, shape, type_, prepared=False):
         self.data = data
         self.shape = tuple(int(d) for d in shape)
         self.type = type_
+        # 8-bit weights only: the payload is in the order the GEMM kernels read (written by prepareB
+        # or prepareAndTransposeB), not in the file order [N, K].  The reference tells the two apart
+        # by type (intgemm8 against intgemm8avx2 ...: src/common/types.h); its enum has no GPU
+        # variant, so this mirror keeps a flag.
+        self.prepared = prepared
 
     @staticmethod
-    def empty(shape, type_, device):
+    def empty(shape, type_, device, prepared=False):
         nbytes = _align256(requiredBytes(shape, type_))
         # (the bytes past elements + 4 are allocation padding and are never read)
-        return QTensor(torch.empty(nbytes, dtype=torch.int8, device=device), shape, type_)
+        return QTensor(torch.empty(nbytes, dtype=torch.int8, device=device), shape, type_, prepared)
 
     @staticmethod
     def from_numpy(flat_int8, shape, type_, device):
-        """Upload payload+tail bytes (e.g. a Type::intgemm8 item of a .bin file) verbatim."""
+        """Upload payload+tail bytes (e.g. a Type::intgemm8 item of a .bin file) verbatim: for
+        8-bit weights that is the file order, which prepareAndTransposeB turns into a usable B."""
         q = QTensor.empty(shape, type_, device)
         src = torch.from_numpy(np.ascontiguousarray(flat_int8).view(np.int8))
         n = min(src.numel(), q.data.numel())
@@ -68,6 +74,15 @@ class QTensor:
     def numpy(self):
         """payload + tail as host bytes (requiredBytes: elements * element size + 4)."""
         return self.data[: requiredBytes(self.shape, self.type)].cpu().numpy()
+
+    def file_bytes(self):
+        """payload + tail as a model file holds them: prepared 8-bit weights are put back into
+        plain rows [N, K] (on the host); everything else is numpy()."""
+        raw = self.numpy()
+        if self.prepared and sizeOf(self.type) == 1:
+            K, N = self.shape
+            return layout.from_prepared(raw, K, N).view(np.int8)
+        return raw
 
     def data_ptr(self):
         return self.data.data_ptr()
@@ -190,7 +205,7 @@ def prepareB(w, type_=Type.intgemm8):
     w = w.contiguous()
     be = _backend_of(w)
     K, N = w.shape
-    out = QTensor.empty((K, N), type_, w.device)
+    out = QTensor.empty((K, N), type_, w.device, prepared=True)
     if type_ == Type.intgemm16:   # the 16-bit branch of the packer (:203-235): quantMult 1024
         _lib.check(be.lib.marian_hip_int16_prepare_b(w.data_ptr(), out.data_ptr(), K, N, be.stream()), "prepareB")
         return out
@@ -198,6 +213,31 @@ def prepareB(w, type_=Type.intgemm8):
                                           be.workspace.data_ptr(), be.workspace_bytes, be.stream())
     _lib.check(st, "prepareB")
     return out
+
+
+def prepareAndTransposeB(q):
+    """A quantized weight item as a model file holds it (plain rows [N, K] + quantMult) -> the
+    order the kernels read; reference prepareAndTransposeB, src/tensors/cpu/integer_common.h:189-216
+    (there: the tiling of the CPU the process runs on)."""
+    _abort_if(not isinstance(q, QTensor) or not isIntgemm(q.type) or isHardwareSpecific(q.type) or len(q.shape) != 2,
+              "prepareAndTransposeB expects a hardware-agnostic intgemm matrix, got {}", getattr(q, "type", type(q)))
+    _abort_if(q.prepared, "the weights are prepared already (type {})", q.type)
+    be = _backend_of(q)
+    K, N = q.shape
+    out = QTensor.empty((K, N), q.type, q.data.device, prepared=True)
+    fn = be.lib.marian_hip_int16_prepare_b_quantized_transposed if sizeOf(q.type) == 2 else \
+        be.lib.marian_hip_int8_prepare_b_quantized_transposed
+    _lib.check(fn(q.data_ptr(), out.data_ptr(), K, N, be.stream()), "prepareAndTransposeB")
+    return out
+
+
+def _check_weights(bQuant):
+    _abort_if(not isinstance(bQuant, QTensor) or not isIntgemm(bQuant.type),
+              "Intgemm expects type of B to be a variant of intgemm not {}", getattr(bQuant, "type", type(bQuant)))
+    _abort_if(isHardwareSpecific(bQuant.type) or sizeOf(bQuant.type) not in (1, 2),
+              "Unsupported type {} for Intgemm type??", bQuant.type)
+    _abort_if(sizeOf(bQuant.type) == 1 and not bQuant.prepared,
+              "B of type {} is in file order: it has to go through prepareAndTransposeB first", bQuant.type)
 
 
 def affineOrDot(a, bQuant, bias=None, transA=False, transB=False, scale=1.0, relu=False,
@@ -210,11 +250,7 @@ def affineOrDot(a, bQuant, bias=None, transA=False, transB=False, scale=1.0, rel
     uint32 device tensor of sorted unique output ids (multiple of 8 many)."""
     _abort_if(not isinstance(a, torch.Tensor) or not a.dtype.is_floating_point or a.dtype != torch.float32,
               "Intgemm expects type of A to be float32 not {}", getattr(a, "dtype", type(a)))
-    _abort_if(not isinstance(bQuant, QTensor) or not isIntgemm(bQuant.type),
-              "Intgemm expects type of B to be a variant of intgemm not {}",
-              getattr(bQuant, "type", type(bQuant)))
-    _abort_if(isHardwareSpecific(bQuant.type) or sizeOf(bQuant.type) not in (1, 2),
-              "Unsupported type {} for Intgemm type??", bQuant.type)
+    _check_weights(bQuant)
     if transA:
         a = a.transpose(-1, -2)
     if sizeOf(bQuant.type) == 2:   # Type::intgemm16: the two nodes one after the other
@@ -242,6 +278,7 @@ def affine_f32(a, bQuant, bias=None, scale=1.0, relu=False, shortlist=None, absm
     (one fused kernel for small activations).  Returns (out, aQuant): aQuant is what the
     prepareA node would have produced.  absmax: the AbsMax left by the call that produced `a`;
     want_absmax: also return an AbsMax of `out` as a third value."""
+    _check_weights(bQuant)
     a = a.contiguous()
     be = _backend_of(a)
     aQuant = QTensor.empty(a.shape, Type.intgemm8, a.device)
@@ -293,10 +330,8 @@ def affine_f32_grouped(a, weights, scale=1.0, relu=False, absmax=None):
     Bq_arr, bias_arr, out_arr, N_arr = ((ctypes.c_void_p * n)(), (ctypes.c_void_p * n)(), (ctypes.c_void_p * n)(),
                                         (ctypes.c_int64 * n)())
     for g, (bQuant, bias) in enumerate(weights):
-        _abort_if(not isinstance(bQuant, QTensor) or not isIntgemm(bQuant.type),
-                  "Intgemm expects type of B to be a variant of intgemm not {}", getattr(bQuant, "type", type(bQuant)))
-        _abort_if(isHardwareSpecific(bQuant.type) or sizeOf(bQuant.type) != 1,
-                  "Unsupported type {} for Intgemm type??", bQuant.type)
+        _check_weights(bQuant)
+        _abort_if(sizeOf(bQuant.type) != 1, "Unsupported type {} for Intgemm type??", bQuant.type)
         _abort_if(rows(bQuant) != K, "Matrix product requires inner dimensions to match: {} vs {}", K, rows(bQuant))
         N = cols(bQuant)
         if bias is not None:
@@ -316,6 +351,7 @@ def affine_f32_grouped(a, weights, scale=1.0, relu=False, absmax=None):
 
 def multiply(aQuant, bQuant, bias=None, scale=1.0, relu=False, shortlist=None):
     """The multiply node of reference src/tensors/cpu/intgemm_interface.h:60-94."""
+    _check_weights(bQuant)
     be = _backend_of(aQuant)
     K, N = cols(aQuant), cols(bQuant)
     _abort_if(rows(bQuant) != K, "Matrix product requires inner dimensions to match: {} vs {}", K, rows(bQuant))
@@ -347,6 +383,7 @@ def multiply(aQuant, bQuant, bias=None, scale=1.0, relu=False, shortlist=None):
 
 def multiply_i32(aQuant, bQuant, shortlist=None):
     """int32 accumulators of the multiply (what Kernels8::Multiply hands to its callback)."""
+    _check_weights(bQuant)
     be = _backend_of(aQuant)
     K, N = cols(aQuant), cols(bQuant)
     M = rows(aQuant) if aQuant.elements() else 0

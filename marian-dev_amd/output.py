@@ -88,9 +88,10 @@ class Output:
         V, D = self.Wt_.shape
         integer._abort_if(self.b_ is not None and self.b_.numel() != V, "bias must be [1 x {}]", V)
         # Quantized tied matrix: prepareA over Wt as a [V x D] tensor = per-tensor abs-max,
-        # row-major int8 + quantMult tail = the intgemm8 weight layout of the logical [D x V]
+        # row-major int8 + quantMult tail = the intgemm8 file order of the logical [D x V], which
+        # prepareAndTransposeB puts into the order the kernels read
         q = integer.prepareA(self.Wt_)
-        self.WtQuant_ = integer.QTensor(q.data, (D, V), Type.intgemm8)
+        self.WtQuant_ = integer.prepareAndTransposeB(integer.QTensor(q.data, (D, V), Type.intgemm8))
         self.shortlist_ = None
 
     def setShortlist(self, shortlist):

@@ -64,7 +64,7 @@ def test_shipped_library_exports_exactly_what_the_headers_declare():
 def test_status_strings_and_version():
     L = load("_lib")
     lib = L.lib()
-    assert lib.marian_hip_int8_abi_version() == 2
+    assert lib.marian_hip_int8_abi_version() == 3
     assert lib.marian_hip_int8_workspace_bytes() >= 4096
     seen = {lib.marian_hip_status_string(i) for i in range(8)}
     assert len(seen) == 8 and lib.marian_hip_status_string(0) == b"ok"

@@ -52,7 +52,7 @@ def check_trace(step, trace, orc, chk):
             A = h["a"].reshape(-1, h["a"].shape[-1])
             M, K = A.shape
             N = Bq.shape[1]
-            want, _ = orc.affine(orc.prepare_a(A), Bq.numpy(), bias.cpu().numpy(), M, K, N, 1.0, t["relu"])
+            want, _ = orc.affine(orc.prepare_a(A), Bq.file_bytes(), bias.cpu().numpy(), M, K, N, 1.0, t["relu"])
             assert np.array_equal(h["out"].reshape(M, N), want), "affine %dx%dx%d" % (M, K, N)
             n_affine += 1
         elif kind == "layer_norm":

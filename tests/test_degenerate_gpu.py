@@ -102,7 +102,7 @@ def test_prepare_a_degenerate_both_forms(integer, orc, kind, kernel):
 def test_prepare_b_degenerate(integer, orc, kind, K, N):
     say("degenerate prepare_b", kind, K, N)
     W = make_a(kind, K, N, 57 + N)
-    same_qtensor(integer.prepareB(dev(W)).numpy(), orc.prepare_b(W), "prepareB " + kind)
+    same_qtensor(integer.prepareB(dev(W)).file_bytes(), orc.prepare_b(W), "prepareB " + kind)
 
 
 # fused call: 0 = shipped library; 600 = separate launches; 611..618 one fused kernel with that K
@@ -121,7 +121,7 @@ def test_fused_affine_degenerate_activations(integer, orc, synth, kind, kernel):
         W = synth.normal(91, synth.STREAM_W, (K, N), 0.02)
         bias = synth.normal(91, synth.STREAM_BIAS, (N,), 0.01)
         Aq_h, Bq_h = orc.prepare_a(A), orc.prepare_b(W)
-        Bq = integer.QTensor.from_numpy(Bq_h, (K, N), T.Type.intgemm8, "cuda")
+        Bq = integer.prepareAndTransposeB(integer.QTensor.from_numpy(Bq_h, (K, N), T.Type.intgemm8, "cuda"))
         for relu in (False, True):
             want, _ = orc.affine(Aq_h, Bq_h, bias, M, K, N, 0.5, relu)
             with forced(kernel):
@@ -149,7 +149,7 @@ def test_multiply_degenerate_activations(integer, orc, synth, kind, kernel, M, K
     bias = synth.normal(92, synth.STREAM_BIAS, (N,), 0.01)
     Aq_h, Bq_h = orc.prepare_a(A), orc.prepare_b(W)
     Aq = integer.QTensor.from_numpy(Aq_h, (M, K), T.Type.intgemm8, "cuda")
-    Bq = integer.QTensor.from_numpy(Bq_h, (K, N), T.Type.intgemm8, "cuda")
+    Bq = integer.prepareAndTransposeB(integer.QTensor.from_numpy(Bq_h, (K, N), T.Type.intgemm8, "cuda"))
     for relu, use_bias in ((False, True), (True, True), (False, False), (True, False)):
         want, want_acc = orc.affine(Aq_h, Bq_h, bias if use_bias else None, M, K, N, 1.0, relu)
         with forced(kernel):
@@ -169,7 +169,7 @@ def test_degenerate_weights(integer, orc, synth, wkind, kernel, M, K, N):
     bias = synth.normal(93, synth.STREAM_BIAS, (N,), 0.01)
     Bq_h = orc.prepare_b(W)
     Bq = integer.prepareB(dev(W))
-    same_qtensor(Bq.numpy(), Bq_h, "prepareB " + wkind)
+    same_qtensor(Bq.file_bytes(), Bq_h, "prepareB " + wkind)
     for akind in ("normal", "zeros"):
         A = synth.normal(94, synth.STREAM_A, (M, K), 1.0) if akind == "normal" else np.zeros((M, K), f32)
         Aq_h = orc.prepare_a(A)

@@ -58,7 +58,7 @@ def test_tied_output_layer(integer, orc, synth):
 
     # the quantized tied matrix is byte for byte what the packer writes for W = Wt^T [D x V]
     Bq_h = orc.prepare_b(np.ascontiguousarray(Wt.T))
-    assert np.array_equal(layer.WtQuant_.numpy()[:V * D + 4], Bq_h[:V * D + 4])
+    assert np.array_equal(layer.WtQuant_.file_bytes()[:V * D + 4], Bq_h[:V * D + 4])
     assert layer.WtQuant_.shape == (D, V)
 
     # embedding lookup keeps the fp32 rows

@@ -56,7 +56,7 @@ def test_static_entry_point_matches_affine_f32(integer, orc, synth, first, secon
             idx = np.sort(np.random.default_rng(seed).choice(N, size=n_sl, replace=False)).astype(np.uint32)
         n_out = n_sl if n_sl else N
         Bq_h = orc.prepare_b(W)
-        Bq = integer.QTensor.from_numpy(Bq_h, (K, N), T.Type.intgemm8, "cuda")
+        Bq = integer.prepareAndTransposeB(integer.QTensor.from_numpy(Bq_h, (K, N), T.Type.intgemm8, "cuda"))
         dA = torch.from_numpy(A).cuda()
         dbias = None if bias is None else torch.from_numpy(bias).cuda()
         didx = None if idx is None else torch.from_numpy(idx.view(np.int32)).cuda()
