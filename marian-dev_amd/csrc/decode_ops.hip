@@ -393,12 +393,14 @@ __global__ __launch_bounds__(256) void attention_kernel(const float* __restrict_
                                                         const float* __restrict__ k_new,
                                                         const float* __restrict__ v_new,
                                                         const float* __restrict__ mask,
-                                                        long long n_masks, long long rows_per_mask,
-                                                        float* __restrict__ out, long long rows_total,
-                                                        long long batchKV, int m, int len, int dk,
+                                                        unsigned n_masks, unsigned rows_per_mask,
+                                                        float* __restrict__ out, unsigned rows_total,
+                                                        unsigned batchKV, int m, int len, int dk,
                                                         float scale, float* __restrict__ absmax_out) {
+  // (row counts are below 2^31, checked by the launcher: 32-bit divisions, a tenth of the
+  // instructions of 64-bit ones, and this kernel is a chain of short phases)
   extern __shared__ __attribute__((aligned(16))) float att_lds[];
-  const long long wr = (long long)blockIdx.x * 4 + threadIdx.x / 64;
+  const unsigned wr = blockIdx.x * 4 + threadIdx.x / 64;
   if(absmax_out && blockIdx.x == 0)   // slots past the last query row
     for(int sl = (int)rows_total + threadIdx.x; sl < kAbsmaxSlots; sl += 256) absmax_out[sl] = 0.0f;
   if(wr >= rows_total) return;   // whole waves leave; no workgroup barrier is used
@@ -408,13 +410,21 @@ __global__ __launch_bounds__(256) void attention_kernel(const float* __restrict_
   float* sc = att_lds + (threadIdx.x / 64) * (len4 + 256);
   float* part = sc + len4;
   const int lane = threadIdx.x % 64;
-  const long long i = wr / m;
+  const unsigned i = wr / (unsigned)m;
   const float* q = Q + (size_t)wr * dk;
   float* kb = Kt + (size_t)(i % batchKV) * len * dk;
   float* vb = V + (size_t)(i % batchKV) * len * dk;
-  if(k_new) {
-    // Newest position (m == 1, one wave per cache entry): its key and value rows go into the
-    // cache for the following steps; this step reads them from k_new / v_new directly.
+  // Newest position (m == 1, one wave per cache entry): its key and value rows go into the cache
+  // for the following steps; this step reads them from k_new / v_new directly.  Up to 64 values per
+  // row they are requested here and stored at the end of the kernel (nothing in this call waits
+  // for the copy, and a store right here would hold the wave for a memory round trip first).
+  float k_app = 0.0f, v_app = 0.0f;
+  const bool append_late = k_new && dk <= 64;
+  if(append_late && lane < dk) {
+    k_app = k_new[(size_t)wr * dk + lane];
+    v_app = v_new[(size_t)wr * dk + lane];
+  }
+  if(k_new && !append_late) {
     for(int d = lane; d < dk; d += 64) {
       kb[(size_t)(len - 1) * dk + d] = k_new[(size_t)wr * dk + d];
       vb[(size_t)(len - 1) * dk + d] = v_new[(size_t)wr * dk + d];
@@ -428,36 +438,60 @@ __global__ __launch_bounds__(256) void attention_kernel(const float* __restrict_
   float mx = -__builtin_inff();
   float omax = 0.0f;   // max |out| of this query row
   const bool fast = vec && dk == 64 && ((reinterpret_cast<uintptr_t>(vb) | reinterpret_cast<uintptr_t>(v_last)) % 16) == 0;
-  if(fast) {
-    // The usual head size.  Sixteen lanes cover the 64 values of a key or value row with 16 bytes
-    // each and the four groups of sixteen take four consecutive positions, so one load of the wave
-    // moves 1 KB of contiguous cache (every lane busy, whatever the number of positions).
-    const int g = lane / 16, c = lane % 16;
-    const v4f q4 = reinterpret_cast<const v4f*>(q)[c];
-    for(int base = 0; base < len; base += 32) {   // eight loads in flight
-      v4f kr[8];
+  // The usual head size.  Sixteen lanes cover the 64 values of a key or value row with 16 bytes each
+  // and the four groups of sixteen take four consecutive positions, so one load of the wave moves
+  // 1 KB of contiguous cache.  Up to sixteen loads, 64 positions, are in flight at a time, and the
+  // first 64 value rows are requested together with the first 64 key rows, so up to 64 positions
+  // the call is one memory round trip.  Loads and products stop at the last group of four that
+  // holds a position (the CU's address unit takes 16 clocks per load whether or not the row is a
+  // duplicate, and eight waves share it).  The mask joins the scores afterwards, a lane per
+  // position: one load for the first 64 positions, requested ahead of the key rows (inside the
+  // score loop it was a dependent load per group of four).
+  constexpr int kAttU = 16;
+  v4f vr[kAttU];
+  const int g = lane / 16, c = lane % 16;
+  auto load_rows = [&](const float* rows, const float* last, int base, v4f (&r)[kAttU]) __attribute__((always_inline)) {
 #pragma unroll
-      for(int u = 0; u < 8; ++u) {
+    for(int u = 0; u < kAttU; ++u) {
+      if(base + 4 * u < len) {   // (the same for the whole wave)
         const int pos = min(base + 4 * u + g, len - 1);
-        const float* krow = pos == len - 1 ? k_last : kb + (size_t)pos * dk;
-        kr[u] = reinterpret_cast<const v4f*>(krow)[c];
-      }
-#pragma unroll
-      for(int u = 0; u < 8; ++u) {
-        const int pos = base + 4 * u + g;
-        float s = q4.x * kr[u].x;
-        s = fmaf(q4.y, kr[u].y, s);
-        s = fmaf(q4.z, kr[u].z, s);
-        s = fmaf(q4.w, kr[u].w, s);
-        s = row16_sum(s);
-        if(c == 0 && pos < len) {
-          float z = scale * s;
-          if(mk) z = z + mk[pos];
-          sc[pos] = z;
-        }
+        const float* row = pos == len - 1 ? last : rows + (size_t)pos * dk;
+        r[u] = reinterpret_cast<const v4f*>(row)[c];
       }
     }
-    for(int pos = lane; pos < len; pos += 64) mx = fmaxf(mx, sc[pos]);
+  };
+  if(fast) {
+    float mk0 = 0.0f;
+    if(mk) mk0 = mk[min(lane, len - 1)];
+    const v4f q4 = reinterpret_cast<const v4f*>(q)[c];
+    v4f kr[kAttU];
+    load_rows(kb, k_last, 0, kr);
+    load_rows(vb, v_last, 0, vr);
+    for(int base = 0;;) {
+#pragma unroll
+      for(int u = 0; u < kAttU; ++u) {
+        if(base + 4 * u < len) {
+          const int pos = base + 4 * u + g;
+          float s = q4.x * kr[u].x;
+          s = fmaf(q4.y, kr[u].y, s);
+          s = fmaf(q4.z, kr[u].z, s);
+          s = fmaf(q4.w, kr[u].w, s);
+          s = row16_sum(s);
+          if(c == 0 && pos < len) sc[pos] = scale * s;
+        }
+      }
+      base += 4 * kAttU;
+      if(base >= len) break;
+      load_rows(kb, k_last, base, kr);
+    }
+    for(int pos = lane; pos < len; pos += 64) {
+      float z = sc[pos];
+      if(mk) {
+        z = z + (pos < 64 ? mk0 : mk[pos]);
+        sc[pos] = z;
+      }
+      mx = fmaxf(mx, z);
+    }
   }
   for(int pos = lane; pos < len && !fast; pos += 64) {
     float s = 0.0f;
@@ -501,24 +535,19 @@ __global__ __launch_bounds__(256) void attention_kernel(const float* __restrict_
   for(int pos = lane; pos < len; pos += 64) sc[pos] = expf(sc[pos] - mx) / sum;
   // (a wave's LDS writes are visible to its own later reads: same wave, program order)
   if(fast) {
-    const int g = lane / 16, c = lane % 16;
     v4f o4 = v4f{0.0f, 0.0f, 0.0f, 0.0f};
-    for(int base = 0; base < len; base += 32) {
-      v4f vr[8];
+    for(int base = 0; base < len; base += 4 * kAttU) {
+      if(base > 0) load_rows(vb, v_last, base, vr);
 #pragma unroll
-      for(int u = 0; u < 8; ++u) {
-        const int pos = min(base + 4 * u + g, len - 1);
-        const float* vrow = pos == len - 1 ? v_last : vb + (size_t)pos * dk;
-        vr[u] = reinterpret_cast<const v4f*>(vrow)[c];
-      }
-#pragma unroll
-      for(int u = 0; u < 8; ++u) {
-        const int pos = base + 4 * u + g;
-        const float w = pos < len ? sc[pos] : 0.0f;
-        o4.x = fmaf(w, vr[u].x, o4.x);
-        o4.y = fmaf(w, vr[u].y, o4.y);
-        o4.z = fmaf(w, vr[u].z, o4.z);
-        o4.w = fmaf(w, vr[u].w, o4.w);
+      for(int u = 0; u < kAttU; ++u) {
+        if(base + 4 * u < len) {
+          const int pos = base + 4 * u + g;
+          const float w = pos < len ? sc[pos] : 0.0f;
+          o4.x = fmaf(w, vr[u].x, o4.x);
+          o4.y = fmaf(w, vr[u].y, o4.y);
+          o4.z = fmaf(w, vr[u].z, o4.z);
+          o4.w = fmaf(w, vr[u].w, o4.w);
+        }
       }
     }
     reinterpret_cast<v4f*>(part)[g * 16 + c] = o4;   // partial sums of the positions g, g + 4, ...
@@ -543,6 +572,10 @@ __global__ __launch_bounds__(256) void attention_kernel(const float* __restrict_
   if(absmax_out) {   // slot = query row
     omax = wave_maxf(omax);
     if(lane == 0) absmax_out[wr] = omax;
+  }
+  if(append_late && lane < dk) {
+    kb[(size_t)(len - 1) * dk + lane] = k_app;
+    vb[(size_t)(len - 1) * dk + lane] = v_app;
   }
 }
 
@@ -1108,6 +1141,7 @@ int marian_hip_attention(const float* q, float* k, float* v, const float* mask, 
   if(absmax_out && !aligned4(absmax_out)) return MARIAN_HIP_ERR_ALIGN;
   if(batchQ < 0 || batchKV <= 0 || m <= 0 || len <= 0 || dk <= 0) return MARIAN_HIP_ERR_SHAPE;
   if(mask && (n_masks <= 0 || rows_per_mask <= 0)) return MARIAN_HIP_ERR_SHAPE;
+  if(mask && (n_masks > 2147483647LL || rows_per_mask > 2147483647LL)) return MARIAN_HIP_ERR_RANGE;
   if(len > 4096) return MARIAN_HIP_ERR_RANGE;
   if(batchQ == 0) return MARIAN_HIP_OK;
   if(!q || !k || !v || !out) return MARIAN_HIP_ERR_NULL;
@@ -1130,8 +1164,8 @@ int marian_hip_attention(const float* q, float* k, float* v, const float* mask, 
     }
   }
   hipLaunchKernelGGL(attention_kernel, dim3((unsigned)((rows_total + 3) / 4)), dim3(256), lds, st, q, k, v,
-                     k_new, v_new, mask, (long long)n_masks, (long long)rows_per_mask, out, rows_total,
-                     (long long)batchKV, (int)m, (int)len, (int)dk, scale, absmax_out);
+                     k_new, v_new, mask, (unsigned)n_masks, (unsigned)rows_per_mask, out, (unsigned)rows_total,
+                     (unsigned)batchKV, (int)m, (int)len, (int)dk, scale, absmax_out);
   MH_HIP(hipGetLastError());
   return MARIAN_HIP_OK;
 }
