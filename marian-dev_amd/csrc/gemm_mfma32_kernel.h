@@ -11,7 +11,8 @@
 //     of that row, so LDS holds each row with its chunks XOR-swizzled and the MFMA fragment reads
 //     (32 consecutive rows, one chunk each) are bank-conflict free.  The K-blocked weights need no
 //     swizzle: 32 columns x one sub-step are 1 KB of consecutive memory in operand order, one wave
-//     load copies them into LDS as they are, and a fragment read covers that 1 KB once.
+//     load brings them into LDS in the lane order of the operand, and a fragment read covers that
+//     1 KB once.
 //   * NSTAGE LDS buffers; the loads of block k + NSTAGE are issued as soon as block k has been
 //     read, so they have NSTAGE - 1 blocks of MFMA time to land.
 //   * Fragments are double-buffered in registers: the ds_reads of sub-step s + 1 (also across
@@ -208,9 +209,10 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * kWave) void gemm_mfma32_kernel(
   // Rows past the matrix edge re-read the last valid row; their products are never stored.
   // Weights: load g = (j - kLoadsA) * kWaves + wave of a stage brings sub-step g / (BN/32) of the 32
   // columns of tile g % (BN/32): 1 KB that is consecutive in the K-blocked weights (consecutive g:
-  // consecutive memory) and lands in LDS as it is, lane q holding half (q >> 3) & 1 of column
-  // (q >> 4) * 8 + (q & 7) of the tile - the layout the fragment reads below expect.  With a
-  // shortlist the lanes gather their columns.
+  // consecutive memory; eight lanes per 128-byte line).  Lane q fetches half q >> 5 of column q & 31
+  // of the tile, so the block sits in LDS in the lane order of the matrix operand and a fragment
+  // read is 1 KB of consecutive LDS (no bank conflicts).  With a shortlist the lanes gather their
+  // columns.
   constexpr int kTilesN = BN / 32;
   int goff[Cfg::kLoads];
 #pragma unroll
@@ -222,9 +224,9 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * kWave) void gemm_mfma32_kernel(
     } else {
       const int g = (j - Cfg::kLoadsA) * Cfg::kWaves + wave;
       const int sub = g / kTilesN, tile = g % kTilesN;
-      const int n = min(n0 + tile * 32 + (lane >> 4) * 8 + (lane & 7), args.n_out - 1);
+      const int n = min(n0 + tile * 32 + (lane & 31), args.n_out - 1);
       const int src = args.idx ? (int)args.idx[n] : n;
-      goff[j] = (int)b_chunk_offset(src, 2 * sub + ((lane >> 3) & 1), args.N);   // (K * N < 2^31)
+      goff[j] = (int)b_chunk_offset(src, 2 * sub + (lane >> 5), args.N);   // (K * N < 2^31)
     }
   }
   const size_t b_block = (size_t)Cfg::BK * (size_t)args.N;   // bytes of all columns per K block
@@ -260,7 +262,7 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * kWave) void gemm_mfma32_kernel(
   for(int kk = 0; kk < 4; ++kk) frag_off[kk] = li * 128 + (((kk * 2 + lg) ^ ((li >> 1) & 7)) * 16);
   const int a_row0 = wm * Cfg::WTM * 32;          // first activation row of this wave in a stage
   // this lane's 16 bytes of sub-step 0 of the wave's first column tile
-  const int b_frag0 = BM * 128 + wn * Cfg::WTN * 1024 + (li >> 3) * 256 + lg * 128 + (li & 7) * 16;
+  const int b_frag0 = BM * 128 + wn * Cfg::WTN * 1024 + lane * 16;
 
   v4i af[PAIRED ? 4 : 2][Cfg::WTM], bf[PAIRED ? 4 : 2][Cfg::WTN];
   auto read_frags = [&](int stage, int kk, int set) {

@@ -101,8 +101,8 @@ __global__ __launch_bounds__(PairCfg::kThreads) void gemm_pair_kernel(GemmArgs a
   const int m0 = tm * BM, n0 = tn * 2 * BN;   // n0: first column of the first tile of the pair
 
   // ---- global -> LDS: activation load j of this wave fills rows (j*4 + wave)*8 .. +7 of a stage;
-  //      weight load g = (j - kLoadsA) * 4 + wave copies the 1 KB block (sub-step g / 4, column tile
-  //      g % 4) of the K-blocked weights as it is (see gemm_mfma32_kernel.h) ----
+  //      weight load g = (j - kLoadsA) * 4 + wave brings the 1 KB block (sub-step g / 4, column tile
+  //      g % 4) of the K-blocked weights into LDS in operand lane order (see gemm_mfma32_kernel.h) ----
   constexpr int kTilesN = BN / 32;
   unsigned goff[Cfg::kLoads];
 #pragma unroll
@@ -114,7 +114,7 @@ __global__ __launch_bounds__(PairCfg::kThreads) void gemm_pair_kernel(GemmArgs a
     } else {
       const int g = (j - Cfg::kLoadsA) * Cfg::kWaves + wave;
       const int sub = g / kTilesN, tile = g % kTilesN;
-      goff[j] = (unsigned)b_chunk_offset(n0 + tile * 32 + (lane >> 4) * 8 + (lane & 7), 2 * sub + ((lane >> 3) & 1), args.N);
+      goff[j] = (unsigned)b_chunk_offset(n0 + tile * 32 + (lane & 31), 2 * sub + (lane >> 5), args.N);
     }
   }
   const int8_t* const b_tile1 = args.Bq + b_column_offset(BN);   // weight columns of the second tile
@@ -135,7 +135,7 @@ __global__ __launch_bounds__(PairCfg::kThreads) void gemm_pair_kernel(GemmArgs a
   for(int kk = 0; kk < 4; ++kk) frag_off[kk] = li * 128 + (((kk * 2 + lg) ^ ((li >> 1) & 7)) * 16);
   const int a_row0 = wm * Cfg::WTM * 32;
   // this lane's 16 bytes of sub-step 0 of the wave's first column tile
-  const int b_frag0 = BM * 128 + wn * Cfg::WTN * 1024 + (li >> 3) * 256 + lg * 128 + (li & 7) * 16;
+  const int b_frag0 = BM * 128 + wn * Cfg::WTN * 1024 + lane * 16;
   v4i af[4][Cfg::WTM], bf[4][Cfg::WTN];
   // fragment f (0..5: four activation, two weight) of sub-step / register set kk
   auto read_one = [&](int stage, int kk, int f) __attribute__((always_inline)) {
