@@ -19,13 +19,12 @@
  *                      point takes it; marian_hip_int8_prepare_b_quantized_transposed converts it.
  *     prepared order : what marian_hip_int8_prepare_b and _prepare_b_quantized_transposed write and
  *                      every GEMM entry point reads ("K-blocked").  K is cut into sub-steps of 32
- *                      values; within a sub-step the N columns follow each other in groups of eight;
- *                      a group is 256 bytes: the lower 16 K values of its eight columns, 16 bytes per
- *                      column, then the upper 16:
- *                        byte of B[k, n] = (k/32)*32*N + (n/8)*256 + ((k/16)%2)*128 + (n%8)*16 + k%16
+ *                      values; within a sub-step the N columns follow each other, 32 bytes each:
+ *                        byte of B[k, n] = (k/32)*32*N + n*32 + k%32
  *                      (the counterpart of intgemm's own CPU tilings, which the reference produces
  *                      with PrepareBQuantizedTransposed, src/tensors/cpu/integer_common.h:189-216:
- *                      the operand of one gfx950 matrix instruction is 1 KB of consecutive memory).
+ *                      the operand of one gfx950 matrix instruction, 32 columns x 32 values of K,
+ *                      is 1 KB of consecutive memory).
  *
  * Shape rules (intgemm's own): K % 64 == 0, N % 8 == 0, shortlist length % 8 == 0.
  * Alignment: A, Aq, Bq, out and acc 16 bytes; bias and idx 4 bytes.

@@ -209,9 +209,9 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * kWave) void gemm_mfma32_kernel(
   // Rows past the matrix edge re-read the last valid row; their products are never stored.
   // Weights: load g = (j - kLoadsA) * kWaves + wave of a stage brings sub-step g / (BN/32) of the 32
   // columns of tile g % (BN/32): 1 KB that is consecutive in the K-blocked weights (consecutive g:
-  // consecutive memory; eight lanes per 128-byte line).  Lane q fetches half q >> 5 of column q & 31
-  // of the tile, so the block sits in LDS in the lane order of the matrix operand and a fragment
-  // read is 1 KB of consecutive LDS (no bank conflicts).  With a shortlist the lanes gather their
+  // consecutive memory).  Lane q fetches half q >> 5 of column q & 31 of the tile, so the block sits
+  // in LDS in the lane order of the matrix operand and a fragment read is 1 KB of consecutive LDS
+  // (no bank conflicts).  With a shortlist the lanes gather their
   // columns.
   constexpr int kTilesN = BN / 32;
   int goff[Cfg::kLoads];

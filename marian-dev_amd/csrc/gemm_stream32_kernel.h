@@ -171,7 +171,7 @@ __global__ __launch_bounds__(WN * KW * kWave) void gemm_stream32_kernel(GemmArgs
     for(int i = 0; i < kAbsmaxSlots / kStream32Threads; ++i) amax = fmaxf(amax, pm[i]);
   }
   // this lane's 16 bytes of K sub-step 0; a sub-step further is w_step bytes further for every column
-  const int8_t* wrow = args.Bq + b_column_offset(wsrc) + lg * 128;
+  const int8_t* wrow = args.Bq + b_column_offset(wsrc) + lg * 16;
   const size_t w_step = 32u * (size_t)args.N;
   __builtin_amdgcn_sched_barrier(0);
 

@@ -317,7 +317,7 @@ __global__ __launch_bounds__(1024) void prepare_a_onepass_kernel(const float* __
 
 // Pass 2 of prepareB: W fp32 [K x N] -> K-blocked int8 payload of the quantized transpose + tail.
 // A workgroup transposes a 64(k) x 64(n) tile through LDS: reads are coalesced along n, writes are
-// 16-byte chunks of K values, eight neighbouring columns side by side.
+// 16-byte chunks of K values, the columns of a K sub-step side by side.
 __global__ __launch_bounds__(256) void quantize_b_transpose_kernel(
     const float* __restrict__ W, int K, int N, const float* __restrict__ partials,
     int n_partials, int8_t* __restrict__ out) {
@@ -344,9 +344,9 @@ __global__ __launch_bounds__(256) void quantize_b_transpose_kernel(
     tile[tn][kk / 4] = quantize_pack4(v, qm);
   }
   __syncthreads();
-  // 64 columns (n) x four 16-byte chunks (k): a wave writes one chunk of all 64 columns, which in the
-  // K-blocked layout is eight runs of 128 bytes
-  const int rn = threadIdx.x % 64, ck = (threadIdx.x / 64) * 16;
+  // 64 columns (n) x four 16-byte chunks (k): two neighbouring threads write the two halves of a
+  // column's sub-step, a wave 32 columns of one sub-step (1 KB of consecutive memory)
+  const int rn = (threadIdx.x / 2) % 64, ck = (threadIdx.x / 128) * 32 + (threadIdx.x % 2) * 16;
   int n = n0 + rn, k = k0 + ck;
   if(n < N && k < K) {  // K % 64 == 0, so a 16-byte run is inside or outside as a whole
     uint4 v;
@@ -364,9 +364,9 @@ __global__ __launch_bounds__(256) void retile_b_kernel(const int8_t* __restrict_
   const size_t chunks = (size_t)K * (size_t)N / 16;
   const size_t o = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   if(o < chunks) {
-    // chunk o of the output: sub-step o / (2 N), then group of eight columns, half, column
+    // chunk o of the output: sub-step o / (2 N), then column, half
     const int s = (int)(o / (2 * (size_t)N)), rem = (int)(o % (2 * (size_t)N));
-    const int n = (rem / 16) * 8 + rem % 8, half = (rem / 8) % 2;
+    const int n = rem / 2, half = rem % 2;
     const uint4 v = *reinterpret_cast<const uint4*>(in + (size_t)n * K + (size_t)(2 * s + half) * 16);
     *reinterpret_cast<uint4*>(out + o * 16) = v;
   }

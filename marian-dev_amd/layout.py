@@ -3,7 +3,7 @@
 The kernels read the K*N int8 values of W^T in the order marian_hip_int8_prepare_b and
 marian_hip_int8_prepare_b_quantized_transposed write (include/marian_hip_int8.h):
 
-    byte of B[k, n] = (k // 32) * 32 * N + (n // 8) * 256 + ((k // 16) % 2) * 128 + (n % 8) * 16 + k % 16
+    byte of B[k, n] = (k // 32) * 32 * N + n * 32 + k % 32
 
 A Marian `.bin` file holds the same values as plain rows [N, K] (reference
 src/tensors/cpu/expression_graph_packable.h:160-201).  The functions here convert between the two on
@@ -17,7 +17,7 @@ def prepared_offsets(K, N):
     assert K % 64 == 0 and N % 8 == 0, (K, N)
     n = np.arange(N, dtype=np.int64)[:, None]
     k = np.arange(K, dtype=np.int64)[None, :]
-    return (k // 32) * (32 * N) + (n // 8) * 256 + ((k // 16) % 2) * 128 + (n % 8) * 16 + k % 16
+    return (k // 32) * (32 * N) + n * 32 + k % 32
 
 
 def to_prepared(flat, K, N):

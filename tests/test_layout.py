@@ -7,17 +7,14 @@ from conftest import load
 
 
 def offsets_by_description(K, N):
-    """K in sub-steps of 32; per sub-step the columns in groups of eight; a group = the lower 16 K
-    values of its eight columns (16 bytes each), then the upper 16."""
+    """K in sub-steps of 32; per sub-step the columns one after the other, 32 bytes each."""
     off = np.empty((N, K), dtype=np.int64)
     pos = 0
     for s in range(K // 32):
-        for g in range(N // 8):
-            for half in range(2):
-                for c in range(8):
-                    for b in range(16):
-                        off[g * 8 + c, s * 32 + half * 16 + b] = pos
-                        pos += 1
+        for n in range(N):
+            for b in range(32):
+                off[n, s * 32 + b] = pos
+                pos += 1
     assert pos == K * N
     return off
 
@@ -33,8 +30,8 @@ def test_offsets_follow_the_description(K, N):
 @pytest.mark.parametrize("K,N", [(64, 32), (128, 96), (256, 1000)])
 def test_operand_blocks_are_contiguous(K, N):
     """32 consecutive columns x one sub-step = 1 KB of consecutive bytes (what one wave loads for one
-    32x32x32 matrix instruction); 16 columns x 64 K values = two runs of 512 bytes (the 16x16x64 form);
-    a step along K is 32 * N bytes for every column."""
+    32x32x32 matrix instruction); 16 columns x one sub-step = 512 bytes; a step along K is 32 * N
+    bytes for every column; a column's 32 values of a sub-step stay together (shortlist gathers)."""
     L = load("layout")
     off = L.prepared_offsets(K, N)
     for n0 in range(0, N - 31, 32):
@@ -45,8 +42,7 @@ def test_operand_blocks_are_contiguous(K, N):
         blk = off[n0:n0 + 16, 0:32].ravel()
         assert blk.max() - blk.min() == 511
     assert np.array_equal(off[:, 32:] - off[:, :-32], np.full((N, K - 32), 32 * N))
-    # a 16-byte chunk of K values stays 16 consecutive bytes
-    assert np.array_equal(off[:, 1::16] - off[:, 0::16], np.ones((N, K // 16), dtype=np.int64))
+    assert np.array_equal(off[:, 31::32] - off[:, 0::32], np.full((N, K // 32), 31))
 
 
 def test_conversions_are_inverse_and_keep_the_tail():
