@@ -6,10 +6,10 @@ Restates the reader and writer of reference src/common/binary.cpp:
           zero bytes so that the payload starts on a 256-byte boundary  (:217-254, :158-215)
   payload items back to back, each padded to a multiple of 256 bytes                  (:242-250)
 
-What differs from the reference loader (:88-114): a `Type::intgemm8` item is kept exactly as stored -
-int8 W^T row-major [N, K] followed by the fp32 quantMult at byte K*N - because that is the layout the
-GPU kernels consume; the reference re-tiles it for the CPU it runs on (prepareAndTransposeB,
-src/tensors/cpu/integer_common.h:189-216).  Items whose type is one of the CPU-tiled variants
+What differs from the reference loader (:88-114): a `Type::intgemm8` item is returned exactly as
+stored - int8 W^T row-major [N, K] followed by the fp32 quantMult at byte K*N; the reference re-tiles
+it on the spot for the CPU it runs on (prepareAndTransposeB, src/tensors/cpu/integer_common.h:189-216),
+here that step happens on the device once the bytes are uploaded (integer.prepareAndTransposeB).  Items whose type is one of the CPU-tiled variants
 (intgemm8ssse3/avx2/avx512/avx512vnni, intgemm16sse2/avx2/avx512) cannot be used on a GPU and are
 refused, and so are FBGEMM-packed items.  A hardware-agnostic `Type::intgemm16` item (int16 W^T
 [N, K] + quantMult 1024 at byte 2*K*N, src/tensors/cpu/expression_graph_packable.h:203-235) is kept

@@ -11,10 +11,11 @@ Mirrors the parts of the reference that sit either side of the output-layer GEMM
   reference src/layers/embedding.cpp:160-170   Embedding::applyIndices = rows(E, ids)
 
 The reference runs the shortlisted product in fp32 (index_select of rows of Wt, then dot with
-transB).  Here the matrix Wt [V x D] row-major *is* the Type::intgemm8 payload of the logical
+transB).  Here the matrix Wt [V x D] row-major *is* the Type::intgemm8 file payload of the logical
 B = Wt^T (K = D, N = V): quantizing Wt row by row with one per-tensor quantMult gives exactly
-the bytes the weight packer would write for B, so the tied matrix is quantized once, its fp32
-rows stay available for the embedding lookup, and the shortlist is a row gather inside the GEMM.
+the bytes the weight packer would write for B; prepareAndTransposeB puts them into the order the
+kernels read.  The tied matrix is quantized once, its fp32 rows stay available for the embedding
+lookup, and the shortlist is a column gather inside the GEMM.
 """
 import bisect
 
