@@ -319,6 +319,8 @@ def affine_f32_grouped(a, weights, scale=1.0, relu=False, absmax=None):
     src/models/transformer.h:290-325 read the same input.  weights: list of (bQuant, bias or None).
     Returns ([out, ...], aQuant); each out equals affine_f32(a, bQuant, bias)[0] bit for bit."""
     import ctypes
+    for bQuant, _ in weights:
+        _check_weights(bQuant)
     a = a.contiguous()
     be = _backend_of(a)
     K = cols(a)

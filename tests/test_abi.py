@@ -107,6 +107,12 @@ def test_argument_validation_returns_codes_not_aborts():
     assert lib.marian_hip_int8_prepare_a(buf, buf, 4096, 1024, buf, 16, None) == L.ERR_WORKSPACE
     assert lib.marian_hip_int8_prepare_a(buf, buf, 0, 64, None, 0, None) == L.OK
     assert lib.marian_hip_int8_prepare_b(buf, buf, 64, 8, None, 4096, None) == L.ERR_NULL
+    # the re-tiling of a model file's weights is a permutation: not in place, not on overlapping buffers
+    assert lib.marian_hip_int8_prepare_b_quantized_transposed(buf, buf, 64, 8, None) == L.ERR_ALIAS
+    assert lib.marian_hip_int8_prepare_b_quantized_transposed(buf, buf + 256, 64, 8, None) == L.ERR_ALIAS
+    assert lib.marian_hip_int8_prepare_b_quantized_transposed(buf, buf + 1024, 100, 8, None) == L.ERR_SHAPE
+    assert lib.marian_hip_int8_prepare_b_quantized_transposed(buf, None, 64, 8, None) == L.ERR_NULL
+    assert lib.marian_hip_status_string(L.ERR_ALIAS).decode() == "input and output overlap"
     with pytest.raises(L.MarianHipError):
         L.check(L.ERR_SHAPE, "test")
 

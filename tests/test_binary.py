@@ -127,3 +127,11 @@ def test_operator_refuses_cpu_tiled_weights_with_the_reference_text():
             integer.affineOrDot(a, w)
     with pytest.raises(integer.MarianRuntimeError, match="Intgemm expects type of B to be a variant of intgemm"):
         integer.affineOrDot(a, integer.QTensor(torch.zeros(64 * 8 * 4, dtype=torch.int8), (64, 8), T.Type.float32))
+    # 8-bit weights as a model file holds them (plain rows) are refused until they have been re-tiled
+    from_file = integer.QTensor(torch.zeros(64 * 8 + 4, dtype=torch.int8), (64, 8), T.Type.intgemm8)
+    assert not from_file.prepared
+    for call in (lambda: integer.affineOrDot(a, from_file), lambda: integer.affine_f32(a, from_file),
+                 lambda: integer.affine_f32_grouped(a, [(from_file, None)]),
+                 lambda: integer.multiply(integer.QTensor(torch.zeros(2 * 64 + 4, dtype=torch.int8), (2, 64), T.Type.intgemm8), from_file)):
+        with pytest.raises(integer.MarianRuntimeError, match="file order.*prepareAndTransposeB"):
+            call()
