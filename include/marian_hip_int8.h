@@ -185,8 +185,8 @@ int marian_hip_int8_affine_f32_static(const float* A, const int8_t* Bq, const fl
 /*
  * Shortlisted output layer.  Reference (fp32): index_select(Wt, 0, idx), index_select(b, -1,
  * idx), then dot/affine with transB (src/data/shortlist.cpp:62-79,
- * src/layers/output.cpp:335-350).  Here rows idx[j] of the [N x K] payload and bias[idx[j]]
- * are gathered inside the GEMM; bqm is the quantMult of the full matrix.
+ * src/layers/output.cpp:335-350).  Here columns idx[j] of the prepared weights (rows of W^T) and
+ * bias[idx[j]] are gathered inside the GEMM; bqm is the quantMult of the full matrix.
  * idx: n_idx sorted unique uint32 ids < N.  out: fp32 [M x n_idx].
  */
 int marian_hip_int8_affine_shortlist(const int8_t* Aq, const int8_t* Bq, const float* bias,

@@ -4,8 +4,8 @@
  * These functions exist only in libmarian_hip_int8_tuning.so (built with
  * -DMARIAN_HIP_TUNING from the same sources as libmarian_hip_int8.so).  That build exports
  * everything include/marian_hip_int8.h and include/marian_hip_ops.h declare plus the
- * functions below, carries kernel families that the automatic selection never picks, and reads
- * clocks inside its kernels.  The shipped library has none of this: no process-wide switch, no
+ * functions below, can pin every kernel family and tile shape the sources hold, whatever the
+ * automatic selection would pick, and reads clocks inside its kernels.  The shipped library has none of this: no process-wide switch, no
  * retained pointer.  They have no counterpart in the reference; tests use them to run every
  * kernel family on every shape, measurements to compare kernels and to time their phases.
  */

@@ -201,7 +201,7 @@ def test_multiply_mid_size_dispatch(integer, orc, synth, M, K, N):
                                    (1300, 2112, 776)])
 def test_multiply_half_last_k_block(integer, orc, synth, M, K, N, kernel):
     """K a multiple of 64 but not of 128 at encoder sizes: the large-M kernels take a last block of
-    64 columns (one, two and many blocks; 350 keeps the 16x16x64 tile kernel for comparison)."""
+    64 columns (one, two and many blocks)."""
     say("multiply half last block", M, K, N, "kernel", kernel)
     run_case(integer, orc, synth, 480 + M + N, M, K, N, kernel, bias_on=True, relu=(K % 256 == 64), scale=0.75)
 
