@@ -75,6 +75,11 @@ struct Tensor {
   MemoryPiece::PtrType memory;
   Shape shape;
   Type type = Type::float32;
+  // 8-bit weights only: the payload is in the order the GEMM kernels read (written by prepareB or
+  // prepareAndTransposeB), not in the file order [N, K].  The reference tells such tensors apart by
+  // type (intgemm8avx2 ... next to the hardware-agnostic intgemm8, src/common/types.h); a Marian
+  // build with this backend would add an enum value of that kind, this stand-in keeps a flag.
+  bool prepared = false;
   size_t elements() const { return ::marian::hip::elements(shape); }
   template <typename T>
   T* data() const { return memory ? memory->data<T>() : nullptr; }
@@ -188,6 +193,7 @@ inline void prepareB(TensorAllocator& ta, const Tensor& w, Tensor& out) {
   void* ws = ta.workspace();
   MARIAN_HIP_CHECK(marian_hip_int8_prepare_b(w.data<float>(), out.data<int8_t>(), w.shape[0], w.shape[1],
                                              ws, ta.workspaceBytes(), ta.backend().stream()));
+  out.prepared = true;
 }
 
 // A quantized weight item as a model file holds it (plain rows [N, K] + quantMult) -> the order the
@@ -201,14 +207,18 @@ inline void prepareAndTransposeB(Backend& be, const Tensor& in, Tensor& out) {
                                                                      in.shape[0], in.shape[1], be.stream()));
     return;
   }
+  if(in.prepared) abortWith("the weights are prepared already");
   MARIAN_HIP_CHECK(marian_hip_int8_prepare_b_quantized_transposed(in.data<int8_t>(), out.data<int8_t>(), in.shape[0],
                                                                   in.shape[1], be.stream()));
+  out.prepared = true;
 }
 
 inline void checkB(const Tensor& bQuant) {
   if(!isIntgemm(bQuant.type)) abortWith("Intgemm expects type of B to be a variant of intgemm");
   if(isHardwareSpecific(bQuant.type) || (sizeOf(bQuant.type) != 1 && sizeOf(bQuant.type) != 2))
     abortWith("Unsupported type for Intgemm type??");
+  if(sizeOf(bQuant.type) == 1 && !bQuant.prepared)
+    abortWith("B is in file order: it has to go through prepareAndTransposeB first");
 }
 
 // Forward body of the multiply node; bias may be null (dot).  relu fuses the in-place ReLU node.

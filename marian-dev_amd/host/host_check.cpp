@@ -297,6 +297,11 @@ int main(int argc, char** argv) {
       t.type = Type::float32;
       try { integer::affineOrDot(ta, a, aq, t, &b, o); } catch(const std::runtime_error& e) { notq = std::strstr(e.what(), "variant of intgemm") != nullptr; }
       expect(tiled && sixteen && notq, "CPU-tiled 8- and 16-bit and float weights are refused with the reference's texts");
+      bool fileOrder = false;
+      t = bq;
+      t.prepared = false;   // as uploaded from a model file
+      try { integer::affineOrDot(ta, a, aq, t, &b, o); } catch(const std::runtime_error& e) { fileOrder = std::strstr(e.what(), "prepareAndTransposeB") != nullptr; }
+      expect(fileOrder, "8-bit weights in file order are refused until they have been re-tiled");
     }
 
     // ---- float operators through their wrappers ----
