@@ -85,6 +85,9 @@ __global__ __launch_bounds__(256) void layer_norm_kernel(const float* in,
   if(CACHE > 0) {
     const int cols4 = cols / 4;
     v4f v[CACHE > 0 ? CACHE : 1];
+    // scale and shift are requested together with the row: read where they are used, behind the two
+    // reductions, they would cost the kernel another memory round trip
+    float gm[CACHE > 0 ? CACHE : 1][4], bt[CACHE > 0 ? CACHE : 1][4];
     float sum = 0.0f;
 #pragma unroll
     for(int j = 0; j < CACHE; ++j) {
@@ -92,8 +95,14 @@ __global__ __launch_bounds__(256) void layer_norm_kernel(const float* in,
       v[j] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
       if(i < cols4) {
         v[j] = reinterpret_cast<const v4f*>(x)[i];
+        v4f t = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+        if(a) t = reinterpret_cast<const v4f*>(a)[i];
+#pragma unroll
+        for(int e = 0; e < 4; ++e) {
+          gm[j][e] = gamma[gamma_stride * (4 * i + e)];
+          bt[j][e] = beta ? beta[beta_stride * (4 * i + e)] : 0.0f;
+        }
         if(a) {
-          const v4f t = reinterpret_cast<const v4f*>(a)[i];
           v[j].x = v[j].x + t.x; v[j].y = v[j].y + t.y; v[j].z = v[j].z + t.z; v[j].w = v[j].w + t.w;
         }
         sum += (v[j].x + v[j].y) + (v[j].z + v[j].w);
@@ -116,8 +125,8 @@ __global__ __launch_bounds__(256) void layer_norm_kernel(const float* in,
         float r[4] = {v[j].x, v[j].y, v[j].z, v[j].w};
 #pragma unroll
         for(int e = 0; e < 4; ++e) {
-          float t = gamma[gamma_stride * (4 * i + e)] * ((r[e] - mean) / sigma);
-          if(beta) t = t + beta[beta_stride * (4 * i + e)];
+          float t = gm[j][e] * ((r[e] - mean) / sigma);
+          if(beta) t = t + bt[j][e];
           r[e] = t;
           omax = fmaxf(omax, fabsf(t));
         }
