@@ -539,9 +539,14 @@ __global__ __launch_bounds__(256) void attention_kernel(const float* __restrict_
   }
   mx = wave_maxf(mx);
   float sum = 0.0f;
-  for(int pos = lane; pos < len; pos += 64) sum += expf(sc[pos] - mx);
+  float e_first = 0.0f;   // exp of this lane's first position, kept for the division below
+  for(int pos = lane; pos < len; pos += 64) {
+    const float e = expf(sc[pos] - mx);
+    if(pos == lane) e_first = e;
+    sum += e;
+  }
   sum = wave_sum(sum);
-  for(int pos = lane; pos < len; pos += 64) sc[pos] = expf(sc[pos] - mx) / sum;
+  for(int pos = lane; pos < len; pos += 64) sc[pos] = (pos == lane ? e_first : expf(sc[pos] - mx)) / sum;
   // (a wave's LDS writes are visible to its own later reads: same wave, program order)
   if(fast) {
     v4f o4 = v4f{0.0f, 0.0f, 0.0f, 0.0f};
