@@ -419,10 +419,12 @@ __global__ __launch_bounds__(256) void attention_kernel(const float* __restrict_
   float* sc = att_lds + (threadIdx.x / 64) * (len4 + 256);
   float* part = sc + len4;
   const int lane = threadIdx.x % 64;
-  const unsigned i = wr / (unsigned)m;
+  // (no division in the usual cases: one position per entry, as many cache entries as entries)
+  const unsigned i = m == 1 ? wr : wr / (unsigned)m;
+  const unsigned entry = i < batchKV ? i : i % batchKV;
   const float* q = Q + (size_t)wr * dk;
-  float* kb = Kt + (size_t)(i % batchKV) * len * dk;
-  float* vb = V + (size_t)(i % batchKV) * len * dk;
+  float* kb = Kt + (size_t)entry * len * dk;
+  float* vb = V + (size_t)entry * len * dk;
   // Newest position (m == 1, one wave per cache entry): its key and value rows go into the cache
   // for the following steps; this step reads them from k_new / v_new directly.  Up to 64 values per
   // row they are requested here and stored at the end of the kernel (nothing in this call waits
@@ -441,7 +443,12 @@ __global__ __launch_bounds__(256) void attention_kernel(const float* __restrict_
   }
   const float* k_last = k_new ? k_new + (size_t)wr * dk : kb + (size_t)(len - 1) * dk;
   const float* v_last = v_new ? v_new + (size_t)wr * dk : vb + (size_t)(len - 1) * dk;
-  const float* mk = mask ? mask + (size_t)((wr / rows_per_mask) % n_masks) * len : nullptr;
+  unsigned mask_row = 0;
+  if(mask) {
+    mask_row = rows_per_mask == 1 ? wr : wr / rows_per_mask;
+    if(mask_row >= n_masks) mask_row %= n_masks;
+  }
+  const float* mk = mask ? mask + (size_t)mask_row * len : nullptr;
   const bool vec = (dk % 4) == 0 && ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(kb) |
                                      reinterpret_cast<uintptr_t>(k_last)) % 16) == 0;
   float mx = -__builtin_inff();
@@ -459,13 +466,19 @@ __global__ __launch_bounds__(256) void attention_kernel(const float* __restrict_
   constexpr int kAttU = 16;
   v4f vr[kAttU];
   const int g = lane / 16, c = lane % 16;
+  // Group of four positions U = (base + 4 u) / 4: this lane's position is 4 U + g, its row 4 U dk
+  // floats behind the lane's first row; from group u_last on the lane's position is the last one
+  // or past it, and it reads the last row (given separately: it may not be in the cache yet).
+  const int u_last = (len + 2 - g) / 4;   // = ceil((len - 1 - g) / 4)
   auto load_rows = [&](const float* rows, const float* last, int base, v4f (&r)[kAttU]) __attribute__((always_inline)) {
+    const float* first = rows + (size_t)g * dk + 4 * c;
+    const float* last_c = last + 4 * c;
 #pragma unroll
     for(int u = 0; u < kAttU; ++u) {
       if(base + 4 * u < len) {   // (the same for the whole wave)
-        const int pos = min(base + 4 * u + g, len - 1);
-        const float* row = pos == len - 1 ? last : rows + (size_t)pos * dk;
-        r[u] = reinterpret_cast<const v4f*>(row)[c];
+        const int U = base / 4 + u;
+        const float* p = U >= u_last ? last_c : first + (size_t)U * 4 * dk;
+        r[u] = *reinterpret_cast<const v4f*>(p);
       }
     }
   };
