@@ -195,17 +195,12 @@ __global__ __launch_bounds__(THREADS < 256 ? 256 : THREADS) void softmax_kernel(
 // once: 256 threads with four float4 each for rows up to 4096 values, 1024 threads with eight or
 // sixteen for vocabulary-size rows (up to 32768 / 65536).  Same
 // operations per element as softmax_kernel.
+// softmax_wide_row leaves in v (vector j of thread t = elements 4 * (j * THREADS + t) .. + 3 of the
+// row, where they exist): LOG: x - max, and returns log(sum of exp(x - max)); otherwise exp(x - max),
+// and returns their sum.
 template <bool LOG, int THREADS, int VPT>
-__global__ __launch_bounds__(THREADS) void softmax_wide_kernel(const float* in, const float* __restrict__ mask,
-                                                                long long n_masks, long long rows_per_mask,
-                                                                float* out, int cols) {
-  __shared__ float red[THREADS / 64];
-  const size_t row = blockIdx.x;
-  const v4f* x = reinterpret_cast<const v4f*>(in + row * cols);
-  const v4f* mk = mask ? reinterpret_cast<const v4f*>(mask + (size_t)((row / rows_per_mask) % n_masks) * cols) : nullptr;
-  v4f* y = reinterpret_cast<v4f*>(out + row * cols);
-  const int cols4 = cols / 4, t = threadIdx.x;
-  v4f v[VPT];
+__device__ __forceinline__ float softmax_wide_row(const v4f* x, const v4f* mk, int cols4, v4f (&v)[VPT], float* red) {
+  const int t = threadIdx.x;
   float mx = -__builtin_inff();
   // (all loads at once, positions past the row clamped and dropped afterwards: a load behind a
   // range check is waited for inside its branch, one memory latency per load)
@@ -248,13 +243,27 @@ __global__ __launch_bounds__(THREADS) void softmax_wide_kernel(const float* in, 
     }
   }
   sum = row_reduce<THREADS, false>(sum, red);
-  const float log_sum = logf(sum);
+  return LOG ? logf(sum) : sum;
+}
+
+template <bool LOG, int THREADS, int VPT>
+__global__ __launch_bounds__(THREADS) void softmax_wide_kernel(const float* in, const float* __restrict__ mask,
+                                                                long long n_masks, long long rows_per_mask,
+                                                                float* out, int cols) {
+  __shared__ float red[THREADS / 64];
+  const size_t row = blockIdx.x;
+  const v4f* x = reinterpret_cast<const v4f*>(in + row * cols);
+  const v4f* mk = mask ? reinterpret_cast<const v4f*>(mask + (size_t)((row / rows_per_mask) % n_masks) * cols) : nullptr;
+  v4f* y = reinterpret_cast<v4f*>(out + row * cols);
+  const int cols4 = cols / 4, t = threadIdx.x;
+  v4f v[VPT];
+  const float s = softmax_wide_row<LOG, THREADS, VPT>(x, mk, cols4, v, red);   // log(sum) or sum
 #pragma unroll
   for(int j = 0; j < VPT; ++j) {
     const int i = j * THREADS + t;
     if(i < cols4) {
-      if(LOG) y[i] = v4f{v[j].x - log_sum, v[j].y - log_sum, v[j].z - log_sum, v[j].w - log_sum};
-      else y[i] = v4f{v[j].x / sum, v[j].y / sum, v[j].z / sum, v[j].w / sum};
+      if(LOG) y[i] = v4f{v[j].x - s, v[j].y - s, v[j].z - s, v[j].w - s};
+      else y[i] = v4f{v[j].x / s, v[j].y / s, v[j].z / s, v[j].w / s};
     }
   }
 }
@@ -739,44 +748,19 @@ __device__ __forceinline__ void nbest_wave_draw(const float* lv, const unsigned*
 
 // The N best of x[0 .. rowLen), by the whole workgroup (1024 threads).  emit(r, value, index) is
 // called once for r = 0 .. N-1 (best first) by one thread each; index is the position within x.
-template <int KEEP, typename Emit>
-__device__ __forceinline__ void nbest_of_row(const float* __restrict__ x, long long rowLen, int N,
-                                             NbestShared& sh, Emit emit) {
+// scan(f) calls f(value, index) for every element this thread owns (each element of the row is
+// owned by exactly one thread of the workgroup; the order does not matter).
+template <int KEEP, typename Scan, typename Emit>
+__device__ __forceinline__ void nbest_core(Scan scan, int N, NbestShared& sh, Emit emit) {
   const int tid = threadIdx.x;
   const float ninf = -__builtin_inff();
   const unsigned none = 0xFFFFFFFFu;
 
   // 1. largest score of this thread, of its wave, and the N-th largest of the 16 wave maxima: the
   //    bound T.  The maxima belong to 16 distinct elements and N <= 16, so at least N elements of the
-  //    row are >= T; for N = 16 and scores without structure some 50 are.  (Values only: one
-  //    instruction per element.  Both scans keep eight 16-byte loads in flight per thread; the last
-  //    round reads clamped positions unconditionally and drops them afterwards, because loads
-  //    behind a range check would be waited for one by one.)
+  //    row are >= T; for N = 16 and scores without structure some 50 are.
   float mv = ninf;
-  const bool vec = (rowLen % 4) == 0 && (reinterpret_cast<uintptr_t>(x) % 16) == 0;
-  const long long n4 = rowLen / 4;
-  if(vec) {   // elements 4 * (t + 1024 * j) .. + 3
-    const v4f* x4 = reinterpret_cast<const v4f*>(x);
-    for(long long i = tid; i < n4; i += 8 * 1024) {
-      v4f v[8];
-#pragma unroll
-      for(int u = 0; u < 8; ++u) v[u] = x4[min(i + u * 1024, n4 - 1)];
-#pragma unroll
-      for(int u = 0; u < 8; ++u) {
-        if(i + u * 1024 >= n4) break;
-        mv = fmaxf(fmaxf(mv, fmaxf(v[u].x, v[u].y)), fmaxf(v[u].z, v[u].w));
-      }
-    }
-  } else {
-    for(long long i = tid; i < rowLen; i += 16 * 1024) {
-      float v[16];
-#pragma unroll
-      for(int u = 0; u < 16; ++u) v[u] = x[min(i + u * 1024, rowLen - 1)];
-#pragma unroll
-      for(int u = 0; u < 16; ++u)
-        if(i + u * 1024 < rowLen) mv = fmaxf(mv, v[u]);
-    }
-  }
+  scan([&](float v, unsigned) { mv = fmaxf(mv, v); });
   float tv = ninf;   // (a wave without elements contributes -inf; with fewer than N waves that hold
                      // elements the bound is -inf and everything passes)
   {
@@ -799,37 +783,14 @@ __device__ __forceinline__ void nbest_of_row(const float* __restrict__ x, long l
   // 2. collect what is >= the bound
   if(tid == 0) sh.count = 0;
   __syncthreads();
-  auto collect = [&](float v, unsigned i) {
+  scan([&](float v, unsigned i) {
     if(v >= tv) {
       const int slot = atomicAdd(&sh.count, 1);
       if(slot < 1024) {
         sh.cand_val[slot] = v; sh.cand_idx[slot] = i;
       }
     }
-  };
-  if(vec) {
-    const v4f* x4 = reinterpret_cast<const v4f*>(x);
-    for(long long i = tid; i < n4; i += 8 * 1024) {
-      v4f v[8];
-#pragma unroll
-      for(int u = 0; u < 8; ++u) v[u] = x4[min(i + u * 1024, n4 - 1)];
-#pragma unroll
-      for(int u = 0; u < 8; ++u) {
-        if(i + u * 1024 >= n4) break;
-        const unsigned b = (unsigned)(4 * (i + u * 1024));
-        collect(v[u].x, b); collect(v[u].y, b + 1); collect(v[u].z, b + 2); collect(v[u].w, b + 3);
-      }
-    }
-  } else {
-    for(long long i = tid; i < rowLen; i += 16 * 1024) {
-      float v[16];
-#pragma unroll
-      for(int u = 0; u < 16; ++u) v[u] = x[min(i + u * 1024, rowLen - 1)];
-#pragma unroll
-      for(int u = 0; u < 16; ++u)
-        if(i + u * 1024 < rowLen) collect(v[u], (unsigned)(i + u * 1024));
-    }
-  }
+  });
   __syncthreads();
   const int count = sh.count;
 
@@ -861,11 +822,10 @@ __device__ __forceinline__ void nbest_of_row(const float* __restrict__ x, long l
     val[j] = ninf;
     idx[j] = none;
   }
-  for(long long i = tid; i < rowLen; i += 1024) {
-    const float v = x[i];
-    if(nbest_before(v, (unsigned)i, val[KEEP - 1], idx[KEEP - 1])) {
+  scan([&](float v, unsigned i) {
+    if(nbest_before(v, i, val[KEEP - 1], idx[KEEP - 1])) {
       val[KEEP - 1] = v;
-      idx[KEEP - 1] = (unsigned)i;
+      idx[KEEP - 1] = i;
 #pragma unroll
       for(int j = KEEP - 1; j > 0; --j) {
         if(nbest_before(val[j], idx[j], val[j - 1], idx[j - 1])) {
@@ -874,7 +834,7 @@ __device__ __forceinline__ void nbest_of_row(const float* __restrict__ x, long l
         }
       }
     }
-  }
+  });
   for(int n = 0; n < N; ++n) {
     float gv; unsigned gi; int who;
     nbest_arg_best(val[0], idx[0], sh, gv, gi, who);
@@ -889,6 +849,43 @@ __device__ __forceinline__ void nbest_of_row(const float* __restrict__ x, long l
       idx[KEEP - 1] = none;
     }
   }
+}
+
+// The row in memory.  (Every scan keeps eight 16-byte loads in flight per thread; the last round
+// reads clamped positions unconditionally and drops them afterwards, because loads behind a range
+// check would be waited for one by one.)
+template <int KEEP, typename Emit>
+__device__ __forceinline__ void nbest_of_row(const float* __restrict__ x, long long rowLen, int N,
+                                             NbestShared& sh, Emit emit) {
+  const int tid = threadIdx.x;
+  const bool vec = (rowLen % 4) == 0 && (reinterpret_cast<uintptr_t>(x) % 16) == 0;
+  const long long n4 = rowLen / 4;
+  auto scan = [&](auto f) __attribute__((always_inline)) {
+    if(vec) {   // elements 4 * (t + 1024 * j) .. + 3
+      const v4f* x4 = reinterpret_cast<const v4f*>(x);
+      for(long long i = tid; i < n4; i += 8 * 1024) {
+        v4f v[8];
+#pragma unroll
+        for(int u = 0; u < 8; ++u) v[u] = x4[min(i + u * 1024, n4 - 1)];
+#pragma unroll
+        for(int u = 0; u < 8; ++u) {
+          if(i + u * 1024 >= n4) break;
+          const unsigned b = (unsigned)(4 * (i + u * 1024));
+          f(v[u].x, b); f(v[u].y, b + 1); f(v[u].z, b + 2); f(v[u].w, b + 3);
+        }
+      }
+    } else {
+      for(long long i = tid; i < rowLen; i += 16 * 1024) {
+        float v[16];
+#pragma unroll
+        for(int u = 0; u < 16; ++u) v[u] = x[min(i + u * 1024, rowLen - 1)];
+#pragma unroll
+        for(int u = 0; u < 16; ++u)
+          if(i + u * 1024 < rowLen) f(v[u], (unsigned)(i + u * 1024));
+      }
+    }
+  };
+  nbest_core<KEEP>(scan, N, sh, emit);
 }
 
 template <int KEEP>
