@@ -131,6 +131,26 @@ int marian_hip_nbest_beams(const float* scores, int64_t beam, int64_t dimBatch, 
                            void* stream);
 
 /*
+ * The end of a beam-search step in one call: the log-softmax of the decoder's logits (LogSoftmax,
+ * src/tensors/cpu/tensor_operators.cpp:474-526, as marian_hip_logsoftmax computes it), the addition of
+ * the hypotheses' path scores (expandedPathScores = prevPathScores + logProbs,
+ * src/translator/beam_search.cpp:433-436) and the transposition + n-best selection of
+ * marian_hip_nbest_beams (:472, :492), without writing the log-probabilities and reading them back.
+ *   logits: [beam, dimBatch, vocab]; vocab % 4 == 0, 4096 < vocab <= 32768 (a row is held in the
+ *   registers of one 1024-thread workgroup, as marian_hip_logsoftmax does for these sizes; other
+ *   sizes: MARIAN_HIP_ERR_SHAPE - use the separate calls), 16-byte aligned.
+ *   rowAdd: NULL, or one value per row [beam * dimBatch] that is added to every log-probability of
+ *   the row before the selection (the path score; what is written to logProbs is without it).
+ *   logProbs: NULL, or [beam, dimBatch, vocab] that receives the log-probabilities as well.
+ * outScores, outKeys, N, workspace: as for marian_hip_nbest_beams (a workspace sized and initialised
+ * for it with the same beam, dimBatch, vocab and N serves this call too); the results are those of
+ * marian_hip_logsoftmax (+ rowAdd) followed by marian_hip_nbest_beams, bit for bit.
+ */
+int marian_hip_logsoftmax_nbest_beams(const float* logits, const float* rowAdd, float* logProbs, int64_t beam,
+                                      int64_t dimBatch, int64_t vocab, int64_t N, float* outScores,
+                                      uint32_t* outKeys, void* workspace, size_t workspace_bytes, void* stream);
+
+/*
  * Replaces gpu::fill, reference src/tensors/gpu/algorithm.cu:37-60 (gFill): `count` elements of
  * elem_bytes (1, 2, 4 or 8) bytes each, starting at `begin` (aligned to elem_bytes), receive the
  * low elem_bytes bytes of `pattern` - the bit pattern of the value, so one entry point serves

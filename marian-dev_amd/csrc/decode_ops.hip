@@ -900,6 +900,52 @@ __global__ __launch_bounds__(1024) void nbest_kernel(const float* __restrict__ s
   });
 }
 
+// Hand-over of per-part candidates to the workgroup that finishes an entry last, without fences.
+// What it relies on (gfx942/gfx950 memory model as the AMDGPU backend documents it): an agent-scope
+// store or atomic bypasses the XCD-local L2 and is performed at the memory side, where all XCDs see
+// it; a wave's vmcnt reaches zero only once each of its stores has been acknowledged from there; an
+// agent-scope load reads from there too.  So: candidates stored (agent scope) -> vmcnt(0) in every
+// wave -> workgroup barrier -> counter incremented; the workgroup that reads parts - 1 from the
+// counter then loads (agent scope) candidates that are all in memory already.  Building with
+// -DMARIAN_HIP_NBEST_FENCED makes the counter update an acquire-release operation instead (the
+// compiler then adds the cache write-back / invalidate the language-level memory model asks for;
+// ~8 us slower): if results ever differ between the two builds, the hand-over is at fault and not
+// the selection.  rowLen: length of an entry's whole row (keys are b * rowLen + position).
+__device__ __forceinline__ void nbest_hand_over(NbestShared& sh, int* is_last, long long b, int parts, int N,
+                                                long long rowLen, float* candVal, unsigned* candIdx,
+                                                unsigned* counters, float* __restrict__ outScores,
+                                                unsigned* __restrict__ outKeys) {
+#ifdef MARIAN_HIP_NBEST_FENCED
+  constexpr int kCounterOrder = __ATOMIC_ACQ_REL;
+#else
+  constexpr int kCounterOrder = __ATOMIC_RELAXED;
+#endif
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // every wave's stores have reached memory ...
+  __syncthreads();
+  if(threadIdx.x == 0)                               // ... before the count goes up
+    *is_last = __hip_atomic_fetch_add(&counters[b * kNbestCounterStride], 1u, kCounterOrder,
+                                      __HIP_MEMORY_SCOPE_AGENT) == (unsigned)(parts - 1);
+  __syncthreads();
+  if(!*is_last) return;
+  // the entry's candidates (at most 1024 pairs), read past this XCD's caches, into LDS
+  const int total = parts * N;
+  for(int e = threadIdx.x; e < total; e += 1024) {
+    sh.cand_val[e] = __hip_atomic_load(candVal + (size_t)b * total + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    sh.cand_idx[e] = __hip_atomic_load(candIdx + (size_t)b * total + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  __syncthreads();
+  if(threadIdx.x < 64) {
+    auto result = [&](int r, float v, unsigned i) {
+      outScores[b * N + r] = v;
+      outKeys[b * N + r] = (unsigned)(b * rowLen) + i;
+    };
+    if(total <= 64) nbest_small_draw(sh.cand_val, sh.cand_idx, total, N, result);
+    else nbest_wave_draw(sh.cand_val, sh.cand_idx, total, N, result);
+    if(threadIdx.x == 0)   // for the next call (every part of this entry has arrived: nobody else touches it)
+      __hip_atomic_store(&counters[b * kNbestCounterStride], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+}
+
 // Beam-major scores [beam, dimBatch, vocab]; the row of batch entry b is the beam's `beam` segments
 // of `vocab` scores, element (k, v) at logical position k * vocab + v.  Workgroup (part, b) takes
 // slice part % perSeg of segment part / perSeg and leaves the N best of it, with their logical
@@ -952,46 +998,60 @@ __global__ __launch_bounds__(1024) void nbest_part_kernel(const float* __restric
     nbest_of_row<KEEP>(scores + ((size_t)k * dimBatch + b) * vocab + v0, len, N, sh,
                        [&](int r, float v, unsigned i) { publish(r, v, base + i); });
   }
-  // Hand-over without fences.  What it relies on (gfx942/gfx950 memory model as the AMDGPU backend
-  // documents it): an agent-scope store or atomic bypasses the XCD-local L2 and is performed at the
-  // memory side, where all XCDs see it; a wave's vmcnt reaches zero only once each of its stores
-  // has been acknowledged from there; an agent-scope load reads from there too.  So: candidates
-  // stored (agent scope) -> vmcnt(0) in every wave -> workgroup barrier -> counter incremented; the
-  // workgroup that reads parts - 1 from the counter then loads (agent scope) candidates that are all
-  // in memory already.  Building with -DMARIAN_HIP_NBEST_FENCED makes the counter update an
-  // acquire-release operation instead (the compiler then adds the cache write-back / invalidate
-  // the language-level memory model asks for; ~8 us slower): if results ever differ between the
-  // two builds, the hand-over is at fault and not the selection.
-#ifdef MARIAN_HIP_NBEST_FENCED
-  constexpr int kCounterOrder = __ATOMIC_ACQ_REL;
-#else
-  constexpr int kCounterOrder = __ATOMIC_RELAXED;
-#endif
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // every wave's stores have reached memory ...
-  __syncthreads();
-  if(threadIdx.x == 0)                               // ... before the count goes up
-    is_last = __hip_atomic_fetch_add(&counters[b * kNbestCounterStride], 1u, kCounterOrder,
-                                     __HIP_MEMORY_SCOPE_AGENT) == (unsigned)(parts - 1);
-  __syncthreads();
-  if(!is_last) return;
-  // the entry's candidates (at most 1024 pairs), read past this XCD's caches, into LDS
-  const int total = parts * N;
-  for(int e = threadIdx.x; e < total; e += 1024) {
-    sh.cand_val[e] = __hip_atomic_load(candVal + (size_t)b * total + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    sh.cand_idx[e] = __hip_atomic_load(candIdx + (size_t)b * total + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  nbest_hand_over(sh, &is_last, b, parts, N, (long long)(parts / perSeg) * vocab, candVal, candIdx, counters,
+                  outScores, outKeys);
+}
+
+// Log-softmax of the rows of beam-major logits [beam, dimBatch, vocab] and the N best of every
+// batch entry's beam * vocab log-probabilities in one launch: workgroup (k, b) keeps row (k, b) in
+// registers (read once), computes the log-probabilities exactly as softmax_wide_kernel<true> does
+// (optionally adds the row's path score and optionally writes them out), selects the N best of the
+// row from the registers and leaves them as part k of entry b; the workgroup that finishes an
+// entry last draws the N best of its beam * N candidates.
+template <int VPT, int KEEP>
+__global__ __launch_bounds__(1024) void logsoftmax_nbest_kernel(const float* __restrict__ in,
+                                                                const float* __restrict__ rowAdd,
+                                                                float* __restrict__ lpOut, long long dimBatch,
+                                                                int vocab, int N, float* candVal,
+                                                                unsigned* candIdx, unsigned* counters,
+                                                                float* __restrict__ outScores,
+                                                                unsigned* __restrict__ outKeys) {
+  __shared__ NbestShared sh;
+  __shared__ int is_last;
+  __shared__ float red[16];
+  const int k = blockIdx.x, parts = gridDim.x, t = threadIdx.x;
+  const long long b = blockIdx.y;
+  const size_t row = (size_t)k * dimBatch + b;
+  const int cols4 = vocab / 4;
+  v4f v[VPT];
+  const float log_sum = softmax_wide_row<true, 1024, VPT>(reinterpret_cast<const v4f*>(in + row * vocab), nullptr,
+                                                          cols4, v, red);
+  const float add = rowAdd ? rowAdd[row] : 0.0f;
+#pragma unroll
+  for(int j = 0; j < VPT; ++j) {
+    v[j] = v4f{v[j].x - log_sum, v[j].y - log_sum, v[j].z - log_sum, v[j].w - log_sum};
+    if(lpOut && j * 1024 + t < cols4) reinterpret_cast<v4f*>(lpOut + row * vocab)[j * 1024 + t] = v[j];
+    if(rowAdd) v[j] = v4f{v[j].x + add, v[j].y + add, v[j].z + add, v[j].w + add};
   }
-  __syncthreads();
-  if(threadIdx.x < 64) {
-    const long long rowLen = (long long)(parts / perSeg) * vocab;
-    auto result = [&](int r, float v, unsigned i) {
-      outScores[b * N + r] = v;
-      outKeys[b * N + r] = (unsigned)(b * rowLen) + i;
-    };
-    if(total <= 64) nbest_small_draw(sh.cand_val, sh.cand_idx, total, N, result);
-    else nbest_wave_draw(sh.cand_val, sh.cand_idx, total, N, result);
-    if(threadIdx.x == 0)   // for the next call (every part of this entry has arrived: nobody else touches it)
-      __hip_atomic_store(&counters[b * kNbestCounterStride], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  }
+  auto scan = [&](auto f) __attribute__((always_inline)) {
+#pragma unroll
+    for(int j = 0; j < VPT; ++j) {
+      const int i4 = j * 1024 + t;
+      if(i4 < cols4) {
+        const unsigned e = 4u * (unsigned)i4;
+        f(v[j].x, e); f(v[j].y, e + 1); f(v[j].z, e + 2); f(v[j].w, e + 3);
+      }
+    }
+  };
+  float* cv = candVal + ((size_t)b * parts + k) * N;
+  unsigned* ci = candIdx + ((size_t)b * parts + k) * N;
+  const unsigned base = (unsigned)k * (unsigned)vocab;
+  __syncthreads();   // (red is done with; the selection has its own LDS)
+  nbest_core<KEEP>(scan, N, sh, [&](int r, float val, unsigned i) {
+    __hip_atomic_store(cv + r, val, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(ci + r, base + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  });
+  nbest_hand_over(sh, &is_last, b, parts, N, (long long)parts * vocab, candVal, candIdx, counters, outScores, outKeys);
 }
 
 // Fill: the 16-byte aligned middle of the range with 16-byte stores of the repeated pattern, the
@@ -1280,6 +1340,38 @@ int marian_hip_nbest_beams(const float* scores, int64_t beam, int64_t dimBatch, 
     hipLaunchKernelGGL(nbest_part_kernel<8>, grid, dim3(1024), 0, st, scores, (long long)dimBatch, (long long)vocab, plan.perSeg, plan.sliceLen, (int)N, candVal, candIdx, counters, outScores, outKeys);
   else
     hipLaunchKernelGGL(nbest_part_kernel<16>, grid, dim3(1024), 0, st, scores, (long long)dimBatch, (long long)vocab, plan.perSeg, plan.sliceLen, (int)N, candVal, candIdx, counters, outScores, outKeys);
+  MH_HIP(hipGetLastError());
+  return MARIAN_HIP_OK;
+}
+
+int marian_hip_logsoftmax_nbest_beams(const float* logits, const float* rowAdd, float* logProbs, int64_t beam,
+                                      int64_t dimBatch, int64_t vocab, int64_t N, float* outScores,
+                                      uint32_t* outKeys, void* workspace, size_t workspace_bytes, void* stream) {
+  if(beam <= 0 || dimBatch < 0 || vocab <= 0 || N <= 0 || N > kNbestMax || N > vocab) return MARIAN_HIP_ERR_SHAPE;
+  // (a row in the registers of one workgroup, and the sizes for which marian_hip_logsoftmax takes the
+  // same row computation, softmax_wide_kernel<true, 1024, 8>: the results are to be the same bits)
+  if(beam * N > 1024 || (vocab % 4) != 0 || vocab <= 4096 || vocab > 32768) return MARIAN_HIP_ERR_SHAPE;
+  if(dimBatch == 0) return MARIAN_HIP_OK;
+  if(!logits || !outScores || !outKeys || !workspace) return MARIAN_HIP_ERR_NULL;
+  if(dimBatch * beam * vocab > 4294967295LL || dimBatch > kNbestMaxBatch) return MARIAN_HIP_ERR_RANGE;   // keys are uint32
+  if(!aligned16(logits) || (logProbs && !aligned16(logProbs)) || (rowAdd && !aligned4(rowAdd)) ||
+     !aligned4(outScores) || !aligned4(outKeys) || !aligned4(workspace))
+    return MARIAN_HIP_ERR_ALIGN;
+  const size_t entries = (size_t)dimBatch * beam * N;
+  if(workspace_bytes < kNbestCounterBytes + entries * 8) return MARIAN_HIP_ERR_WORKSPACE;
+  // (the layout of marian_hip_nbest_beams with one part per beam entry)
+  unsigned* counters = reinterpret_cast<unsigned*>(workspace);
+  float* candVal = reinterpret_cast<float*>(counters + kNbestMaxBatch * kNbestCounterStride);
+  unsigned* candIdx = reinterpret_cast<unsigned*>(candVal + entries);
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  const dim3 grid((unsigned)beam, (unsigned)dimBatch);
+#define MH_LSNB(VPT, KEEP)                                                                                   \
+  hipLaunchKernelGGL((logsoftmax_nbest_kernel<VPT, KEEP>), grid, dim3(1024), 0, st, logits, rowAdd, logProbs, \
+                     (long long)dimBatch, (int)vocab, (int)N, candVal, candIdx, counters, outScores, outKeys)
+  if(N <= 4) MH_LSNB(8, 4);
+  else if(N <= 8) MH_LSNB(8, 8);
+  else MH_LSNB(8, 16);
+#undef MH_LSNB
   MH_HIP(hipGetLastError());
   return MARIAN_HIP_OK;
 }

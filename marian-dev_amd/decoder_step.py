@@ -69,11 +69,13 @@ class DecoderStep:
         self.src_lens = lens
         self.mask = (torch.arange(self.L, device="cuda")[None, :] >= lens[:, None]).float() * -99999999.0
 
-    def step(self, s, gemm_only=False, chained=True, grouped=True):
+    def step(self, s, gemm_only=False, chained=True, grouped=True, fused_tail=False):
         """chained: every tensor that feeds an affine call leaves its abs-max where it is
         produced (layer norm, attention, the ReLU GEMM), so those calls skip their abs-max pass.
         grouped: the self-attention projections Wq, Wk, Wv (one input, three weight matrices,
-        reference src/models/transformer.h:290-325) go through one call."""
+        reference src/models/transformer.h:290-325) go through one call.
+        fused_tail: log-softmax and n-best in one launch (the log-probabilities are not written);
+        the step then returns (scores, keys) of the n-best instead of the log-probabilities."""
         integer, ops = self.integer, self.ops
         W = self.sets[s % len(self.sets)]
         tr = self.trace
@@ -159,6 +161,10 @@ class DecoderStep:
         rec("affine", a=x, w=W["out"], out=logits, relu=False)
         if gemm_only:
             return logits
+        if fused_tail:
+            vals, keys = ops.logsoftmaxNBestOfBeams(logits.view(self.beam, 1, self.batch, self.V), self.beam)
+            rec("logsoftmax_nbest", logits=logits, vals=vals, keys=keys)
+            return vals, keys
         # log-probabilities, then the beam's n-best per sentence over beam x vocabulary
         lp = ops.logsoftmax(logits)
         # (the transposition to [batch, beam * V] of beam_search.cpp:472 happens inside the call)

@@ -103,7 +103,45 @@ public:
                                             ta_.backend().stream()));
   }
 
+  // The end of a beam-search step in one call: LogSoftmax of the logits [beam, dimBatch, vocab], + the
+  // path score of each hypothesis (pathScores: null or [beam, dimBatch]), transposition + n-best;
+  // logProbs: null, or a tensor that also receives the log-probabilities.
+  void logSoftmaxNBestOfBeams(const Tensor& logits, const Tensor* pathScores, int64_t N, Tensor& outScores,
+                              Tensor& outKeys, Tensor* logProbs = nullptr) {
+    if(logits.shape.size() != 3) abortWith("logSoftmaxNBestOfBeams expects [beam, batch, vocab]");
+    const int64_t beam = logits.shape[0], dimBatch = logits.shape[1], vocab = logits.shape[2];
+    if(vocab % 4 != 0 || vocab <= 4096 || vocab > 32768) {   // sizes the one-launch form does not take
+      if(pathScores) abortWith("logSoftmaxNBestOfBeams: path scores need the one-launch form (4096 < vocab <= 32768)");
+      Tensor lp;
+      Tensor& target = logProbs ? *logProbs : lp;
+      ta_.allocate(target, logits.shape, Type::float32);
+      Tensor rows = logits, out = target;
+      rows.shape = {(int)(beam * dimBatch), (int)vocab};
+      out.shape = rows.shape;
+      LogSoftmax(ta_.backend(), out, rows);
+      getNBestListOfBeams(target, N, outScores, outKeys);
+      if(!logProbs) ta_.free(lp);
+      return;
+    }
+    ta_.allocate(outScores, {(int)(dimBatch * N)}, Type::float32);
+    ta_.allocate(outKeys, {(int)(dimBatch * N)}, Type::uint32);
+    if(logProbs) ta_.allocate(*logProbs, logits.shape, Type::float32);
+    reserveWorkspace(beam, dimBatch, vocab, N);
+    MARIAN_HIP_CHECK(marian_hip_logsoftmax_nbest_beams(
+        logits.data<float>(), pathScores ? pathScores->data<float>() : nullptr, logProbs ? logProbs->data<float>() : nullptr,
+        beam, dimBatch, vocab, N, outScores.data<float>(), outKeys.data<uint32_t>(), workspace_.data<void>(),
+        workspace_.elements(), ta_.backend().stream()));
+  }
+
 private:
+  void reserveWorkspace(int64_t beam, int64_t dimBatch, int64_t vocab, int64_t N) {
+    const size_t need = marian_hip_nbest_beams_workspace_bytes(beam, dimBatch, vocab, N);
+    if(!workspace_ || workspace_.elements() < need) {
+      if(workspace_) ta_.free(workspace_);
+      ta_.allocate(workspace_, {(int)need}, Type::int8);
+      MARIAN_HIP_CHECK(marian_hip_nbest_beams_workspace_init(workspace_.data<void>(), need, ta_.backend().stream()));
+    }
+  }
   TensorAllocator& ta_;
   Tensor workspace_;
 };

@@ -332,6 +332,39 @@ int main(int argc, char** argv) {
       expect(sameBits(download<float>(be, nbV2, wantNbVal.size()), wantNbVal) &&
                  sameBits(download<uint32_t>(be, nbK2, wantNbKey.size()), wantNbKey),
              "NthElement::getNBestListOfBeams: the same list");
+      // the fused end of a step against the separate calls on the same logits
+      Tensor xb = x, lsmGpu = lsm, fusedV, fusedK, sepV, sepK, fusedLp;
+      xb.shape = {1, R, C};
+      lsmGpu.shape = {1, R, C};
+      nth.getNBestListOfBeams(lsmGpu, nbestN, sepV, sepK);
+      nth.logSoftmaxNBestOfBeams(xb, nullptr, nbestN, fusedV, fusedK, &fusedLp);
+      expect(sameBits(download<float>(be, fusedV, (size_t)R * nbestN), download<float>(be, sepV, (size_t)R * nbestN)) &&
+                 sameBits(download<uint32_t>(be, fusedK, (size_t)R * nbestN), download<uint32_t>(be, sepK, (size_t)R * nbestN)) &&
+                 sameBits(download<float>(be, fusedLp, (size_t)R * C), download<float>(be, lsm, (size_t)R * C)),
+             "NthElement::logSoftmaxNBestOfBeams (short rows: the separate calls inside), bit for bit");
+      // rows long enough for the one-launch form: 2 beam entries x 3 sentences x 4100 words
+      const int kBeam = 2, kBatch = 3, kVocab = 4100;
+      std::vector<float> logits((size_t)kBeam * kBatch * kVocab), path((size_t)kBeam * kBatch);
+      uint32_t rng = 12345u;
+      for(auto& v : logits) { rng = rng * 1664525u + 1013904223u; v = (float)(rng >> 8) * (1.0f / 1048576.0f) - 8.0f; }
+      for(size_t i = 0; i < path.size(); ++i) path[i] = -0.75f * (float)i;
+      logits[5] = logits[kVocab + 77] = logits[3 * kVocab + 9] = 9.5f;   // equal scores across rows
+      Tensor lg = upload(ta, logits, {kBeam, kBatch, kVocab}, Type::float32), ps = upload(ta, path, {kBeam, kBatch}, Type::float32);
+      Tensor oneV, oneK, oneLp, twoLp, twoV, twoK;
+      nth.logSoftmaxNBestOfBeams(lg, &ps, nbestN, oneV, oneK, &oneLp);
+      ta.allocate(twoLp, {kBeam * kBatch, kVocab}, Type::float32);
+      Tensor rowsIn = lg;
+      rowsIn.shape = {kBeam * kBatch, kVocab};
+      LogSoftmax(be, twoLp, rowsIn);
+      std::vector<float> lpHost = download<float>(be, twoLp, logits.size());
+      expect(sameBits(download<float>(be, oneLp, logits.size()), lpHost), "one-launch form: the log-probabilities of LogSoftmax");
+      for(size_t r = 0; r < path.size(); ++r)
+        for(int c = 0; c < kVocab; ++c) lpHost[r * kVocab + c] = lpHost[r * kVocab + c] + path[r];
+      Tensor scored = upload(ta, lpHost, {kBeam, kBatch, kVocab}, Type::float32);
+      nth.getNBestListOfBeams(scored, nbestN, twoV, twoK);
+      expect(sameBits(download<float>(be, oneV, (size_t)kBatch * nbestN), download<float>(be, twoV, (size_t)kBatch * nbestN)) &&
+                 sameBits(download<uint32_t>(be, oneK, (size_t)kBatch * nbestN), download<uint32_t>(be, twoK, (size_t)kBatch * nbestN)),
+             "one-launch form with path scores: the n-best of LogSoftmax + path score, bit for bit");
     }
     be.synchronize();
     std::printf("host_check: %d failure(s), slab moved %zu times -> %s\n", failures,

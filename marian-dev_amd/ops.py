@@ -216,3 +216,43 @@ def getNBestListOfBeams(scores, N):
                                        keys.data_ptr(), ws.data_ptr(), ws.numel(), be.stream())
     _lib.check(st, "getNBestListOfBeams")
     return vals, keys
+
+
+def logsoftmaxNBestOfBeams(logits, N, pathScores=None, want_logprobs=False):
+    """The end of a beam-search step in one call: logsoftmax over the vocabulary (reference
+    src/tensors/cpu/tensor_operators.cpp:474-526), + the hypotheses' path scores
+    (src/translator/beam_search.cpp:433-436), then what getNBestListOfBeams does (:472, :492).
+    logits [beam, 1, dimBatch, vocab] (or [beam, dimBatch, vocab]); pathScores: None or one value
+    per row [beam, dimBatch]; returns (vals, keys), and the log-probabilities as a third value when
+    asked for.  Bit for bit what the separate calls give."""
+    logits = _f32c(logits, "logsoftmaxNBestOfBeams")
+    be = _backend_of(logits)
+    beam, vocab = logits.shape[0], logits.shape[-1]
+    dimBatch = logits.numel() // (beam * vocab) if beam * vocab else 0
+    if not (vocab % 4 == 0 and 4096 < vocab <= 32768 and logits.data_ptr() % 16 == 0):
+        # sizes the one-launch form does not take: the separate calls
+        lp = logsoftmax(logits)
+        scored = lp if pathScores is None else lp + _f32c(pathScores, "logsoftmaxNBestOfBeams").reshape(
+            (beam,) + (1,) * (logits.dim() - 3) + (dimBatch, 1))
+        vals, keys = getNBestListOfBeams(scored, N)
+        return (vals, keys, lp) if want_logprobs else (vals, keys)
+    add = None
+    if pathScores is not None:
+        add = _f32c(pathScores, "logsoftmaxNBestOfBeams").reshape(-1)
+        _abort_if(add.numel() != beam * dimBatch, "one path score per hypothesis, got {}", add.numel())
+    vals = torch.empty(dimBatch * N, dtype=torch.float32, device=logits.device)
+    keys = torch.empty(dimBatch * N, dtype=torch.int32, device=logits.device)
+    lp = torch.empty_like(logits) if want_logprobs else None
+    need = be.lib.marian_hip_nbest_beams_workspace_bytes(beam, dimBatch, vocab, N)
+    held = _nbest_workspaces.setdefault((logits.device, be.stream()), [])
+    if not held or held[-1].numel() < need:
+        ws = torch.empty(max(int(need), 4), dtype=torch.uint8, device=logits.device)
+        _lib.check(be.lib.marian_hip_nbest_beams_workspace_init(ws.data_ptr(), ws.numel(), be.stream()),
+                   "logsoftmaxNBestOfBeams")
+        held.append(ws)
+    ws = held[-1]
+    st = be.lib.marian_hip_logsoftmax_nbest_beams(
+        logits.data_ptr(), None if add is None else add.data_ptr(), None if lp is None else lp.data_ptr(), beam,
+        dimBatch, vocab, N, vals.data_ptr(), keys.data_ptr(), ws.data_ptr(), ws.numel(), be.stream())
+    _lib.check(st, "logsoftmaxNBestOfBeams")
+    return (vals, keys, lp) if want_logprobs else (vals, keys)

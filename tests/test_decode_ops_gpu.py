@@ -416,6 +416,66 @@ def test_nbest_of_beams(ops, chk, synth, batch, beam, V, N):
         assert np.array_equal(vals.cpu().numpy(), cv) and np.array_equal(keys.cpu().numpy().view(np.uint32), ck)
 
 
+@pytest.mark.parametrize("batch,beam,V,N,with_scores", [(32, 4, 32000, 4, False), (32, 4, 32000, 4, True), (1, 1, 32000, 12, True),
+                                                        (7, 6, 5000, 6, True), (9, 3, 8196, 5, True), (40, 2, 4100, 2, False),
+                                                        (2, 12, 32768, 16, True), (3, 64, 4104, 16, False), (1, 2, 6000, 8, True),
+                                                        # sizes the one-launch form does not take: the mirror falls back
+                                                        (3, 1, 20, 16, False), (2, 2, 8, 8, True), (5, 4, 3000, 1, False),
+                                                        (2, 2, 4098, 3, True), (1, 2, 40000, 4, False)])
+def test_logsoftmax_nbest_of_beams_is_the_separate_calls(ops, chk, synth, batch, beam, V, N, with_scores):
+    """The end of a beam-search step in one launch: bit for bit the log-softmax entry point, the
+    addition of the path scores and the n-best over beams one after the other; the log-probabilities
+    it writes on request are those of the separate call; and for sizes the CPU checker finishes
+    quickly, its n-best of its own log-softmax (values within the float bar of that operator, keys
+    equal wherever the checker's values are not tied within that bar)."""
+    import torch
+    x = synth.normal(77 + V + beam, 0, (beam, 1, batch, V), 3.0)
+    if V >= 1000:
+        x[:, 0, 0, ::499] = np.float32(6.25)      # equal logits inside a row and across the beam
+        x[0, 0, -1, :] = np.float32(0.5)          # a constant row
+    path = synth.normal(5 + beam, 1, (beam, batch), 1.5) if with_scores else None
+    dx = dev(x)
+    lp_sep = ops.logsoftmax(dx)
+    scored = lp_sep if path is None else lp_sep + dev(path).view(beam, 1, batch, 1)
+    want_v, want_k = ops.getNBestListOfBeams(scored, N)
+    vals, keys, lp = ops.logsoftmaxNBestOfBeams(dx, N, None if path is None else dev(path), want_logprobs=True)
+    assert torch.equal(lp, lp_sep)
+    assert torch.equal(vals, want_v) and torch.equal(keys, want_k)
+    vals2, keys2 = ops.logsoftmaxNBestOfBeams(dx, N, None if path is None else dev(path))      # without the copy
+    assert torch.equal(vals2, want_v) and torch.equal(keys2, want_k)
+    if batch * beam * V <= 60000:
+        ref = chk.logsoftmax(x.reshape(beam * batch, V)).reshape(beam, 1, batch, V)
+        if path is not None:
+            ref = ref + path.reshape(beam, 1, batch, 1)
+        flat = np.ascontiguousarray(np.swapaxes(ref, 0, 2)).reshape(batch, -1)
+        got_v = vals.cpu().numpy().reshape(batch, N)
+        got_k = keys.cpu().numpy().view(np.uint32).reshape(batch, N).astype(np.int64) - np.arange(batch)[:, None] * flat.shape[1]
+        assert np.allclose(got_v, np.take_along_axis(flat, got_k, 1), rtol=2e-5, atol=4e-6)
+        order = np.argsort(-flat, axis=1, kind="stable")[:, :N]
+        assert np.allclose(got_v, np.take_along_axis(flat, order, 1), rtol=2e-5, atol=4e-6)
+
+
+def test_logsoftmax_nbest_of_beams_argument_checks(ops):
+    import torch
+    from conftest import load
+    L = load("_lib")
+    lib = L.lib()
+    x = torch.zeros(1, 1, 40000, device="cuda")
+    need = lib.marian_hip_nbest_beams_workspace_bytes(1, 1, 5000, 4)
+    ws = torch.zeros(need, dtype=torch.uint8, device="cuda")
+    out = torch.zeros(64, device="cuda")
+    call = lambda beam, batch, V, N, wb: lib.marian_hip_logsoftmax_nbest_beams(
+        x.data_ptr(), None, None, beam, batch, V, N, out.data_ptr(), out.data_ptr(), ws.data_ptr(), wb, None)
+    assert call(1, 1, 5000, 4, need) == L.OK
+    assert call(1, 1, 5000, 4, 16) == L.ERR_WORKSPACE
+    assert call(4, 2, 100, 4, need) == L.ERR_SHAPE            # short rows: the separate calls
+    assert call(1, 1, 5002, 4, need) == L.ERR_SHAPE           # rows of whole 16-byte units only
+    assert call(1, 1, 40000, 4, need) == L.ERR_SHAPE          # longer than a workgroup's registers hold
+    assert call(1, 1, 5000, 17, need) == L.ERR_SHAPE
+    assert call(4, 0, 5000, 4, 0) == L.OK
+    torch.cuda.synchronize()
+
+
 def _random_nbest_cases(n):
     rng = np.random.default_rng(20261127)
     cases = []

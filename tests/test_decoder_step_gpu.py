@@ -135,3 +135,9 @@ def test_decoder_step_every_call_against_the_checker(integer, orc, size):
     for t, c in zip(step.Kself + step.Vself, caches):
         t.copy_(c)
     assert torch.equal(step.step(0, chained=False, grouped=False), lp)
+    # log-softmax and n-best as one launch (the form bench.py times): the n-best of the step above
+    for t, c in zip(step.Kself + step.Vself, caches):
+        t.copy_(c)
+    nbest = [e for kind, e in trace if kind == "nbest"][0]
+    vals, keys = step.step(0, fused_tail=True)
+    assert torch.equal(vals, nbest["vals"]) and torch.equal(keys, nbest["keys"])

@@ -15,7 +15,7 @@ pytestmark = pytest.mark.gpu
 def test_decoder_tail_replays(integer, synth):
     import torch
     ops = load("ops")
-    M, K, V, beam, batch = 32, 512, 4096, 4, 8
+    M, K, V, beam, batch = 32, 512, 4104, 4, 8
     g = torch.Generator(device="cuda")
     g.manual_seed(5)
     x = torch.randn(M, K, device="cuda", generator=g)
@@ -35,9 +35,12 @@ def test_decoder_tail_replays(integer, synth):
         logits, _ = integer.affine_f32(h1, Wv, bv, absmax=h1max)
         lp = ops.logsoftmax(logits)
         vals, keys = ops.getNBestListOfBeams(lp.view(beam, 1, batch, V), beam)
-        return lp, vals, keys
+        # ... and log-softmax + n-best once more as one launch (the same workspace, the same counters)
+        vals1, keys1 = ops.logsoftmaxNBestOfBeams(logits.view(beam, 1, batch, V), beam)
+        return lp, vals, keys, vals1, keys1
 
     want = [t.clone() for t in step()]
+    assert torch.equal(want[1], want[3]) and torch.equal(want[2], want[4])
     torch.cuda.synchronize()
 
     s = torch.cuda.Stream()
