@@ -659,8 +659,9 @@ int marian_hip_int8_prepare_b_quantized_transposed(const int8_t* in, int8_t* out
   if(K * N > kMaxElems) return MARIAN_HIP_ERR_RANGE;
   if(!aligned(in, 16) || !aligned(out, 16)) return MARIAN_HIP_ERR_ALIGN;
   // the two layouts are permutations of each other: not in place
-  const int8_t* in_end = in + K * N + sizeof(float);
-  if(in < out + K * N + (int64_t)sizeof(float) && out < in_end) return MARIAN_HIP_ERR_ALIAS;
+  const uintptr_t a0 = reinterpret_cast<uintptr_t>(in), b0 = reinterpret_cast<uintptr_t>(out);
+  const uintptr_t bytes = (uintptr_t)K * (uintptr_t)N + sizeof(float);
+  if(a0 < b0 + bytes && b0 < a0 + bytes) return MARIAN_HIP_ERR_ALIAS;
   const size_t chunks = (size_t)K * (size_t)N / 16;
   hipLaunchKernelGGL(retile_b_kernel, dim3((unsigned)((chunks + 255) / 256)), dim3(256), 0,
                      reinterpret_cast<hipStream_t>(stream), in, (int)K, (int)N, out);
