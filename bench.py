@@ -680,7 +680,8 @@ def main():
         gonly = [capture(torch, (lambda c=c: dec.step(c, gemm_only=True))) for c in range(bsets)]
         gdt = time_graphs(torch, gonly, n, max(4, args.warmup // 2))
         out["transformer_big_decode_full"] = {
-            "what": "full decoder step through the host mirrors: 49 int8 affine calls + per layer "
+            "what": "full decoder step through the host mirrors, from the previous step's word indices: embedding rows x "
+                    "sqrt(d) + position signal (one launch), 49 int8 affine calls + per layer "
                     "2 one-launch attentions (20 cached positions + the new one, appended by the call; "
                     "source lengths uniform 20..60, padded to 60 positions with mask), 3 skip-add+layer-norm; the self-attention "
                     "projections Wq, Wk, Wv through one grouped call; log-softmax over 32000, beam/batch transposition + n-best per "

@@ -97,6 +97,38 @@ int marian_hip_attention(const float* q, float* k, float* v, const float* mask, 
                          const float* k_new, const float* v_new, void* stream);
 
 /*
+ * The embedding step in front of the first layer, reference src/layers/embedding.cpp:161-168
+ * (rows(E, ids): CopyRows, src/tensors/cpu/tensor_operators.cpp:577-603), followed by
+ * src/models/transformer.h:93 (sqrt(dimEmb) * embeddings) and :117 (embeddings + signal, the
+ * sinusoidal position signal of src/tensors/cpu/tensor_operators.cpp:1733-1746) as one launch:
+ *   out[r, :] = scale * E[ids[r], :] + signal[(r / rows_per_signal) % n_signals, :]
+ * with the product and the sum rounded one after the other like the reference's two nodes, so
+ * the result equals theirs bit for bit.
+ *   E: [vocab, dimEmb] float32; ids: rows word indices (uint32, the reference's IndexType), on the
+ *   device.  The reference reads past the table for an id >= vocab; this call reads the table's
+ *   last row instead.
+ *   signal: NULL (no sum: a pure gather when scale == 1), or [n_signals, dimEmb].  A decoding step
+ *   passes the one row of its position (n_signals == 1); a whole sentence batch [dimWords,
+ *   dimBatch] passes rows_per_signal = dimBatch, n_signals = dimWords.
+ *   absmax_out: as for marian_hip_layer_norm (needs rows <= 2048): the int8 products of the first
+ *   layer then need no abs-max launch of their own.
+ */
+int marian_hip_embed(const float* E, const uint32_t* ids, int64_t rows, int64_t vocab, int64_t dimEmb,
+                     float scale, const float* signal, int64_t rows_per_signal, int64_t n_signals,
+                     float* out, float* absmax_out, void* stream);
+
+/*
+ * Replaces SinusoidalPositionEmbeddings, reference src/tensors/cpu/tensor_operators.cpp:1733-1746,
+ * the initializer of the constant that src/models/transformer.h:110-111 adds to the embeddings:
+ *   host_out[j, i] = sin or cos of (j + start) * exp((i % (dimEmb / 2)) * -log(10000) / (dimEmb / 2 - 1)),
+ * sine for the first half of a row, cosine for the rest, in float arithmetic with the C library's
+ * functions like the reference's loop.  host_out: dimWords * dimEmb floats in HOST memory (the
+ * constant is made once per position on the host and copied to the device by the caller);
+ * dimEmb >= 4 (with fewer the reference's increment divides by zero).  No HIP call is made.
+ */
+int marian_hip_sinusoidal_position_embeddings(float* host_out, int64_t dimWords, int64_t dimEmb, int64_t start);
+
+/*
  * Replaces NthElement::getNBestList, reference src/translator/nth_element.cpp:26-67 (CPU) and
  * src/translator/nth_element.cu (GPU): for each of dimBatch rows of rowLen = beam * vocabulary
  * scores, the N best scores in descending order and their keys = absolute positions

@@ -11,6 +11,7 @@
 #include <hip/hip_runtime.h>
 
 #include <atomic>
+#include <cmath>
 
 #include "../../include/marian_hip_int8.h"
 #include "abi_common.h"
@@ -1074,6 +1075,51 @@ __global__ __launch_bounds__(256) void fill_kernel(unsigned char* __restrict__ p
   }
 }
 
+// ---------------------------------------------------------------- embedding step
+// One workgroup per output row: out[r, :] = scale * E[ids[r], :] (+ signal[(r / rows_per_signal) %
+// n_signals, :]).  The product and the sum round separately.  An id at or past the table's end reads
+// the table's last row.
+template <bool VEC>
+__global__ __launch_bounds__(256) void embed_kernel(const float* __restrict__ E, const uint32_t* __restrict__ ids,
+                                                    unsigned vocab, int dimEmb, float scale,
+                                                    const float* __restrict__ signal, unsigned rows_per_signal,
+                                                    unsigned n_signals, float* __restrict__ out,
+                                                    float* __restrict__ absmax_out) {
+  __shared__ float red[4];
+  const unsigned row = blockIdx.x;
+  const int tid = threadIdx.x;
+  unsigned id = ids[row];
+  id = id < vocab ? id : vocab - 1u;
+  const float* src = E + (size_t)id * dimEmb;
+  const float* sg = signal ? signal + (size_t)((row / rows_per_signal) % n_signals) * dimEmb : nullptr;
+  float* y = out + (size_t)row * dimEmb;
+  float omax = 0.0f;
+  if(VEC) {
+    for(int i = tid; i < dimEmb / 4; i += 256) {
+      const v4f e = reinterpret_cast<const v4f*>(src)[i];
+      v4f s = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+      if(sg) s = reinterpret_cast<const v4f*>(sg)[i];
+      v4f r = v4f{scale * e.x, scale * e.y, scale * e.z, scale * e.w};
+      if(sg) r = v4f{r.x + s.x, r.y + s.y, r.z + s.z, r.w + s.w};
+      omax = fmaxf(fmaxf(omax, fmaxf(fabsf(r.x), fabsf(r.y))), fmaxf(fabsf(r.z), fabsf(r.w)));
+      reinterpret_cast<v4f*>(y)[i] = r;
+    }
+  } else {
+    for(int i = tid; i < dimEmb; i += 256) {
+      float r = scale * src[i];
+      if(sg) r = r + sg[i];
+      omax = fmaxf(omax, fabsf(r));
+      y[i] = r;
+    }
+  }
+  if(absmax_out) {   // slot `row`; workgroup 0 zeroes the slots past the last row
+    omax = row_reduce<256, true>(omax, red);
+    if(tid == 0) absmax_out[row] = omax;
+    if(row == 0)
+      for(int sl = gridDim.x + tid; sl < kAbsmaxSlots; sl += 256) absmax_out[sl] = 0.0f;
+  }
+}
+
 __global__ __launch_bounds__(256) void zero_words_kernel(unsigned* __restrict__ p, long long n) {
   for(long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long long)gridDim.x * blockDim.x)
     p[i] = 0u;
@@ -1117,6 +1163,51 @@ int marian_hip_layer_norm(const float* in, const float* add, const float* gamma,
   else
     hipLaunchKernelGGL(layer_norm_kernel<0>, dim3((unsigned)rows), dim3(256), 0, st, in, add, gamma, gs, beta, bs, out, (int)cols, eps, absmax_out);
   MH_HIP(hipGetLastError());
+  return MARIAN_HIP_OK;
+}
+
+int marian_hip_embed(const float* E, const uint32_t* ids, int64_t rows, int64_t vocab, int64_t dimEmb,
+                     float scale, const float* signal, int64_t rows_per_signal, int64_t n_signals,
+                     float* out, float* absmax_out, void* stream) {
+  if(absmax_out && rows > kAbsmaxSlots) return MARIAN_HIP_ERR_RANGE;
+  if(absmax_out && !aligned4(absmax_out)) return MARIAN_HIP_ERR_ALIGN;
+  if(rows < 0 || vocab <= 0 || dimEmb <= 0) return MARIAN_HIP_ERR_SHAPE;
+  if(signal && (rows_per_signal <= 0 || n_signals <= 0)) return MARIAN_HIP_ERR_SHAPE;
+  if(rows == 0) return MARIAN_HIP_OK;
+  if(!E || !ids || !out) return MARIAN_HIP_ERR_NULL;
+  if(rows * dimEmb > kMaxElemsOps || vocab > 0xFFFFFFFFLL || rows_per_signal > 0x7FFFFFFFLL ||
+     n_signals > 0x7FFFFFFFLL || (signal && n_signals * dimEmb > kMaxElemsOps))
+    return MARIAN_HIP_ERR_RANGE;
+  if(!aligned4(E) || !aligned4(ids) || !aligned4(out) || (signal && !aligned4(signal))) return MARIAN_HIP_ERR_ALIGN;
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  const bool vec = dimEmb % 4 == 0 && aligned16(E) && aligned16(out) && (!signal || aligned16(signal));
+  const unsigned rps = signal ? (unsigned)rows_per_signal : 1u, ns = signal ? (unsigned)n_signals : 1u;
+  if(vec)
+    hipLaunchKernelGGL(embed_kernel<true>, dim3((unsigned)rows), dim3(256), 0, st, E, ids, (unsigned)vocab, (int)dimEmb,
+                       scale, signal, rps, ns, out, absmax_out);
+  else
+    hipLaunchKernelGGL(embed_kernel<false>, dim3((unsigned)rows), dim3(256), 0, st, E, ids, (unsigned)vocab, (int)dimEmb,
+                       scale, signal, rps, ns, out, absmax_out);
+  MH_HIP(hipGetLastError());
+  return MARIAN_HIP_OK;
+}
+
+int marian_hip_sinusoidal_position_embeddings(float* host_out, int64_t dimWords, int64_t dimEmb, int64_t start) {
+  if(dimWords < 0 || dimEmb < 4) return MARIAN_HIP_ERR_SHAPE;   // (one timescale: the increment divides by zero)
+  if(dimWords == 0) return MARIAN_HIP_OK;
+  if(!host_out) return MARIAN_HIP_ERR_NULL;
+  if(dimWords * dimEmb > kMaxElemsOps || start < 0 || start + dimWords > 0x7FFFFFFFLL) return MARIAN_HIP_ERR_RANGE;
+  const float numTimescales = (float)dimEmb / 2;
+  const int half = (int)numTimescales;
+  const float logTimescaleIncrement = std::log(10000.f) / (numTimescales - 1.f);
+  for(int64_t j = 0; j < dimWords; ++j) {
+    const int position = (int)(j + start);
+    float* row = host_out + j * dimEmb;
+    for(int i = 0; i < (int)dimEmb; ++i) {
+      const float v = (float)position * std::exp((float)(i % half) * -logTimescaleIncrement);
+      row[i] = i < half ? std::sin(v) : std::cos(v);
+    }
+  }
   return MARIAN_HIP_OK;
 }
 

@@ -1,6 +1,8 @@
 """One decoding step of a Marian transformer decoder on the HIP library, through the host mirrors
-(integer.py, ops.py): the call sequence of reference src/models/transformer.h:603-760 for one new
-target position at inference (post-processing "dan": skip connection, then layer norm), followed by
+(integer.py, ops.py): the embedding of the previous step's words (reference
+src/models/transformer.h:92-117: rows of the table times sqrt(d), plus the position signal), the
+call sequence of reference src/models/transformer.h:603-760 for one new target position at
+inference (post-processing "dan": skip connection, then layer norm), followed by
 the log-softmax and the beam search's n-best selection (src/translator/beam_search.cpp:472-492).
 Weights are random; the key/value caches of earlier target positions and of the encoder are
 resident.  bench.py times it at transformer-big size; tests check every call of it against the CPU
@@ -16,8 +18,10 @@ class DecoderStep:
     decoding step at beam 4 x batch 32 (reference src/models/transformer.h:603-760 for the layer
     structure, post-processing "dan", inference).  Self-attention keys/values of `t_past` earlier
     positions and encoder keys/values of `src_len` positions are resident; K/V projections are
-    taken for the new position only.  Beam search itself (top-k, hypothesis bookkeeping) is not
-    part of the step."""
+    taken for the new position only.  The step starts from the word indices the previous step
+    chose (the float32 embedding table is the transposed output matrix: tied embeddings, which
+    intgemm models keep in float32, reference src/tensors/cpu/expression_graph_packable.h:154).
+    Beam search's hypothesis bookkeeping is not part of the step."""
 
     def __init__(self, sets=1, d=1024, ffn=4096, heads=16, vocab=32000, layers=6, beam=4, batch=32,
                  t_past=20, src_len=60, min_src_len=20, seed=300):
@@ -37,7 +41,9 @@ class DecoderStep:
         def vec(n, scale=0.01, shift=0.0):
             return torch.randn(n, device="cuda", generator=g) * scale + shift
 
-        first = {"layers": [], "out": (qw(d, V), vec(V))}
+        # tied embeddings: one float32 table [V, d] for the lookup, its transpose quantized for the output layer
+        self.E = torch.randn(V, d, device="cuda", generator=g) * 0.02
+        first = {"layers": [], "out": (integer.prepareB(self.E.t().contiguous()), vec(V))}
         for _ in range(layers):
             ly = {}
             for name, (K, N) in {"Wq": (d, d), "Wk": (d, d), "Wv": (d, d), "Wo": (d, d), "cWq": (d, d),
@@ -59,7 +65,10 @@ class DecoderStep:
         self.weight_bytes = layers * (6 * d * d + 2 * d * ffn) + d * V
         self.gemm_ops = 2 * M * self.weight_bytes
         # resident state
-        self.x = torch.randn(M, d, device="cuda", generator=g)
+        self.words = torch.randint(0, V, (M,), device="cuda", generator=g).to(torch.int32)
+        self.signal = ops.sinusoidalPositionEmbeddings(1, d, t_past, device="cuda")
+        self.emb_scale = float(torch.sqrt(torch.tensor(float(d))))
+        self.x = torch.randn(M, d, device="cuda", generator=g)   # (input of the GEMM-only chain)
         self.Kself = [torch.randn(M * H, self.T, d // H, device="cuda", generator=g) for _ in range(layers)]
         self.Vself = [torch.randn(M * H, self.T, d // H, device="cuda", generator=g) for _ in range(layers)]
         self.Kenc = [torch.randn(self.batch * H, self.L, d // H, device="cuda", generator=g) for _ in range(layers)]
@@ -87,6 +96,11 @@ class DecoderStep:
         dk = d // H
         x, xmax = self.x, None
         ch = chained and not gemm_only
+        if not gemm_only:
+            x = ops.scaledEmbeddings(self.E, self.words, self.emb_scale, self.signal, M, want_absmax=ch)
+            if ch:
+                x, xmax = x
+            rec("embed", E=self.E, ids=self.words, scale=self.emb_scale, signal=self.signal, out=x)
         for li, ly in enumerate(W["layers"]):
             if grouped:   # one abs-max, one quantization, one launch for the three projections
                 (q, k, v), _ = integer.affine_f32_grouped(x, [ly["Wq"], ly["Wk"], ly["Wv"]], absmax=xmax)

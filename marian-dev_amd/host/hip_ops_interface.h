@@ -7,6 +7,9 @@
 //   src/tensors/gpu/prod.cpp:471-574                                   ProdBatchedLegacy
 //   src/models/transformer.h:241-280                                   Attention()
 //   src/translator/nth_element.cpp:26-67, nth_element.cu               NthElement::getNBestList
+//   src/tensors/cpu/tensor_operators.cpp:577-603                       CopyRows
+//   src/tensors/cpu/tensor_operators.cpp:1733-1746                     SinusoidalPositionEmbeddings
+//   src/models/transformer.h:92-117                                    ScaledEmbeddings (rows * sqrt(d) + signal)
 #pragma once
 
 #include "../../include/marian_hip_ops.h"
@@ -24,6 +27,33 @@ inline void LayerNormalization(Backend& be, Tensor& out, const Tensor& in, const
       in.data<float>(), add ? add->data<float>() : nullptr, gamma.data<float>(), (int64_t)gamma.elements(),
       beta ? beta->data<float>() : nullptr, beta ? (int64_t)beta->elements() : 0, out.data<float>(), rows(in),
       cols(in), eps, absmaxOut ? absmaxOut->data<float>() : nullptr, be.stream()));
+}
+
+// out[r, :] = scale * in[indices[r], :] (+ signal[(r / rowsPerSignal) % rows(signal), :]): the embedding
+// step in front of the first layer as one launch.  indices: uint32 tensor on the device.
+inline void ScaledEmbeddings(Backend& be, Tensor& out, const Tensor& in, const Tensor& indices, float scale,
+                             const Tensor* signal = nullptr, int64_t rowsPerSignal = 1, Tensor* absmaxOut = nullptr) {
+  if(indices.type != Type::uint32) abortWith("ScaledEmbeddings expects indices of type uint32");
+  if(in.shape.size() != 2) abortWith("ScaledEmbeddings expects a [rows, cols] table");
+  if(cols(out) != cols(in) || out.elements() != indices.elements() * (size_t)cols(in))
+    abortWith("ScaledEmbeddings: the output has to hold one row of the table per index");
+  if(signal && cols(*signal) != cols(in)) abortWith("ScaledEmbeddings: signal rows and table rows differ in length");
+  MARIAN_HIP_CHECK(marian_hip_embed(in.data<float>(), indices.data<uint32_t>(), (int64_t)indices.elements(),
+                                    rows(in), cols(in), scale, signal ? signal->data<float>() : nullptr,
+                                    rowsPerSignal, signal ? (int64_t)rows(*signal) : 0, out.data<float>(),
+                                    absmaxOut ? absmaxOut->data<float>() : nullptr, be.stream()));
+}
+
+// out[j, :] = in[indices[j], :]
+inline void CopyRows(Backend& be, Tensor& out, const Tensor& in, const Tensor& indices) {
+  ScaledEmbeddings(be, out, in, indices, 1.0f);
+}
+
+// The constant [dimWords, 1, dimEmb] of the position signal, made on the host: `host` receives
+// dimWords * dimEmb floats for positions start, start + 1, ...
+inline void SinusoidalPositionEmbeddings(std::vector<float>& host, int64_t dimWords, int64_t dimEmb, int start) {
+  host.resize((size_t)(dimWords * dimEmb));
+  MARIAN_HIP_CHECK(marian_hip_sinusoidal_position_embeddings(host.data(), dimWords, dimEmb, start));
 }
 
 // mask: optional [nMasks, cols] log-mask; row r of `in` uses mask row (r / rowsPerMask) % nMasks.

@@ -366,6 +366,47 @@ int main(int argc, char** argv) {
                  sameBits(download<uint32_t>(be, oneK, (size_t)kBatch * nbestN), download<uint32_t>(be, twoK, (size_t)kBatch * nbestN)),
              "one-launch form with path scores: the n-best of LogSoftmax + path score, bit for bit");
     }
+    // ---- the embedding step: rows of a table (the reference's own vectors for rows(),
+    // src/tests/units/operator_tests.cpp:773-826), then scale and position signal ----
+    {
+      const std::vector<float> table{1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12};
+      const std::vector<uint32_t> picks{2, 1, 1, 0, 3};
+      const std::vector<float> wantRows{7, 8, 9, 4, 5, 6, 4, 5, 6, 1, 2, 3, 10, 11, 12};
+      Tensor tb = upload(ta, table, {4, 3}, Type::float32), ix = upload(ta, picks, {(int)picks.size()}, Type::uint32);
+      Tensor got;
+      ta.allocate(got, {(int)picks.size(), 3}, Type::float32);
+      CopyRows(be, got, tb, ix);
+      expect(sameBits(download<float>(be, got, wantRows.size()), wantRows), "CopyRows: the reference's rows() vectors");
+      const int dE = 8, nWords = 6, perSignal = 3;
+      std::vector<float> emb((size_t)5 * dE), signal;
+      for(size_t i = 0; i < emb.size(); ++i) emb[i] = 0.013f * (float)((int)(i * 7 % 23) - 11);
+      SinusoidalPositionEmbeddings(signal, 2, dE, 4);
+      expect(signal.size() == (size_t)2 * dE && std::fabs(signal[0] - std::sin(4.0f)) < 1e-6f &&
+                 std::fabs(signal[dE / 2] - std::cos(4.0f)) < 1e-6f && std::fabs(signal[dE + dE / 2 - 1] - std::sin(5.0e-4f)) < 1e-9f,
+             "SinusoidalPositionEmbeddings: sine half, cosine half, slowest timescale");
+      const std::vector<uint32_t> words{4, 0, 3, 3, 1, 2};
+      const float scale = std::sqrt((float)dE);
+      std::vector<float> wantEmb((size_t)nWords * dE);
+      for(int r = 0; r < nWords; ++r)
+        for(int i = 0; i < dE; ++i) {
+          volatile float scaled = scale * emb[(size_t)words[r] * dE + i];   // two roundings, like two graph nodes
+          wantEmb[(size_t)r * dE + i] = scaled + signal[(size_t)(r / perSignal) * dE + i];
+        }
+      Tensor et = upload(ta, emb, {5, dE}, Type::float32), wt = upload(ta, words, {nWords}, Type::uint32);
+      Tensor sg = upload(ta, signal, {2, dE}, Type::float32), eo, emax;
+      ta.allocate(eo, {nWords, dE}, Type::float32);
+      ta.allocate(emax, {MARIAN_HIP_ABSMAX_SLOTS}, Type::float32);
+      ScaledEmbeddings(be, eo, et, wt, scale, &sg, perSignal, &emax);
+      expect(sameBits(download<float>(be, eo, wantEmb.size()), wantEmb), "ScaledEmbeddings: sqrt(d) * rows + position signal, bit for bit");
+      std::vector<float> slots = download<float>(be, emax, MARIAN_HIP_ABSMAX_SLOTS);
+      bool slotsOk = true;
+      for(int r = 0; r < MARIAN_HIP_ABSMAX_SLOTS; ++r) {
+        float m = 0.0f;
+        for(int i = 0; r < nWords && i < dE; ++i) m = std::max(m, std::fabs(wantEmb[(size_t)r * dE + i]));
+        slotsOk = slotsOk && slots[r] == m;
+      }
+      expect(slotsOk, "ScaledEmbeddings: abs-max slot per row, zero past the last row");
+    }
     be.synchronize();
     std::printf("host_check: %d failure(s), slab moved %zu times -> %s\n", failures,
                 ta.allocator()->device()->moves(), failures == 0 ? "OK" : "FAILED");

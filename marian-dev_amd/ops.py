@@ -7,6 +7,9 @@ Mirrors, name for name:
                                                          transpose(a, {0, 2, 1, 3}),
                                                          bdot_legacy(a, b, transA, transB, scalar)
   reference src/models/transformer.h:145-170             SplitHeads, JoinHeads
+  reference src/graph/expression_operators.cpp           rows(a, indices)
+  reference src/graph/node_initializers.cpp:224-226      sinusoidalPositionEmbeddings(start)
+  reference src/models/transformer.h:93,110-117          scaledEmbeddings: sqrt(dimEmb) * rows(E, ids) + signal
 
 Tensors are torch float32 tensors on the GPU (device memory and streams only); every arithmetic
 step is a call into the C ABI.  There is no CPU fallback.
@@ -46,6 +49,48 @@ def layerNorm(x, gamma, beta=None, eps=1e-9, add=None, want_absmax=False):
         out.data_ptr(), rows, cols, eps, None if omax is None else omax.data_ptr(), be.stream())
     _lib.check(st, "layerNorm")
     return (out, omax) if want_absmax else out
+
+
+def scaledEmbeddings(E, ids, scale=1.0, signal=None, rowsPerSignal=1, want_absmax=False):
+    """scale * E[ids] (+ signal): the embedding step in front of the first layer (reference
+    src/layers/embedding.cpp:161-168 and src/models/transformer.h:93,117) as one launch.  E
+    [vocab, dimEmb]; ids: integer tensor on the device, any shape; signal: None or [n, dimEmb],
+    output row r taking signal row (r / rowsPerSignal) % n.  Returns [*ids.shape, dimEmb]."""
+    E = _f32c(E, "scaledEmbeddings")
+    be = _backend_of(E)
+    _abort_if(E.dim() != 2, "scaledEmbeddings: the table has to be a matrix, got shape {}", tuple(E.shape))
+    _abort_if(ids.dtype not in (torch.int32, torch.int64, torch.uint32) or ids.device != E.device,
+              "scaledEmbeddings: indices have to be an integer tensor on the table's device")
+    vocab, dimEmb = E.shape
+    words = ids.contiguous()
+    if words.dtype == torch.int64:   # the reference's IndexType has 32 bits
+        words = words.to(torch.int32)
+    n_signals = 0
+    if signal is not None:
+        signal = _f32c(signal, "scaledEmbeddings").reshape(-1, dimEmb)
+        n_signals = signal.shape[0]
+    out = torch.empty(tuple(ids.shape) + (dimEmb,), dtype=torch.float32, device=E.device)
+    omax = AbsMax(E.device) if want_absmax else None
+    st = be.lib.marian_hip_embed(E.data_ptr(), words.data_ptr(), words.numel(), vocab, dimEmb, float(scale),
+                                 None if signal is None else signal.data_ptr(), rowsPerSignal, n_signals,
+                                 out.data_ptr(), None if omax is None else omax.data_ptr(), be.stream())
+    _lib.check(st, "scaledEmbeddings")
+    return (out, omax) if want_absmax else out
+
+
+def rows(a, indices):
+    """reference rows(a, indices) (CopyRows, src/tensors/cpu/tensor_operators.cpp:577-603)"""
+    return scaledEmbeddings(a, indices.reshape(-1))
+
+
+def sinusoidalPositionEmbeddings(dimWords, dimEmb, start=0, device=None):
+    """The constant [dimWords, 1, dimEmb] of reference src/models/transformer.h:110-111, made on the
+    host by the library (reference src/tensors/cpu/tensor_operators.cpp:1733-1746) and copied to
+    `device` when one is given."""
+    out = torch.empty((dimWords, 1, dimEmb), dtype=torch.float32)
+    _lib.check(_lib.lib().marian_hip_sinusoidal_position_embeddings(out.data_ptr(), dimWords, dimEmb, start),
+               "sinusoidalPositionEmbeddings")
+    return out if device is None else out.to(device)
 
 
 def softmax(a, mask=None, rowsPerMask=1):

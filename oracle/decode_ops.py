@@ -40,6 +40,10 @@ def lib():
                                          c.c_float]
         L.oracle_nbest.restype = None
         L.oracle_nbest.argtypes = [fp, i64, i64, i64, fp, c.POINTER(c.c_uint32)]
+        L.oracle_embed.restype = None
+        L.oracle_embed.argtypes = [fp, fp, c.POINTER(c.c_uint32), i64, i64, c.c_float, fp, i64, i64]
+        L.oracle_sinusoidal_position_embeddings.restype = None
+        L.oracle_sinusoidal_position_embeddings.argtypes = [fp, i64, i64, c.c_int]
         _lib = L
     return _lib
 
@@ -123,3 +127,24 @@ def nbest(scores, N):
     lib().oracle_nbest(_p(scores), dimBatch, rowLen, N, _p(vals),
                        keys.ctypes.data_as(ctypes.POINTER(ctypes.c_uint32)))
     return vals, keys
+
+
+def embed(E, ids, scale=1.0, signal=None, rows_per_signal=1):
+    """scale * E[ids] (+ the position signal: row (r // rows_per_signal) % n_signals for output row r)"""
+    E = _f32(E)
+    ids = np.ascontiguousarray(ids, dtype=np.uint32).ravel()
+    d = E.shape[-1]
+    n_signals = 1
+    if signal is not None:
+        signal = _f32(signal).reshape(-1, d)
+        n_signals = signal.shape[0]
+    out = np.empty((ids.size, d), dtype=np.float32)
+    lib().oracle_embed(_p(out), _p(E), ids.ctypes.data_as(ctypes.POINTER(ctypes.c_uint32)), ids.size, d,
+                       np.float32(scale), _p(signal), rows_per_signal, n_signals)
+    return out
+
+
+def sinusoidal_position_embeddings(dimWords, dimEmb, start=0):
+    out = np.empty((dimWords, dimEmb), dtype=np.float32)
+    lib().oracle_sinusoidal_position_embeddings(_p(out), dimWords, dimEmb, int(start))
+    return out

@@ -15,13 +15,21 @@
  *   oracle_transpose0213   reference src/tensors/cpu/tensor_operators.cpp:220-246
  *   oracle_bdot_legacy     reference src/tensors/cpu/prod.cpp:233-330 (ProdBatchedLegacy, beta = 0)
  *   oracle_nbest           reference src/translator/nth_element.cpp:26-67 (getNBestList)
+ *   oracle_embed           reference src/layers/embedding.cpp:161-168 (rows(E, ids), i.e. CopyRows,
+ *                          src/tensors/cpu/tensor_operators.cpp:577-603) followed by the two nodes of
+ *                          src/models/transformer.h:93 (sqrt(dimEmb) * embeddings) and :117
+ *                          (embeddings + signal, the signal row shared by the words of a position)
+ *   oracle_sinusoidal_position_embeddings
+ *                          reference src/tensors/cpu/tensor_operators.cpp:1733-1746
  *
  * Pinning status (tests/test_decode_ops.py): every function is checked against float64 closed
  * forms in numpy and against invariants that a dropped term or a wrong index would break
  * (softmax rows sum to one and are shift invariant; layer-norm output has mean beta and
  * variance gamma^2 for constant gamma/beta; transposing twice is the identity; the batched
  * product against numpy matmul including the batch broadcast i % batchA, i % batchB; the n-best
- * list against a full numpy sort): pinned.
+ * list against a full numpy sort; the embedding step against numpy indexing with scale 1 and no
+ * signal - a pure row copy - and against float64 with both; the position signal against float64
+ * sin/cos of position / 10000^(i / (d/2 - 1)) and its values at position 0: zeros and ones): pinned.
  */
 #include <math.h>
 #include <stddef.h>
@@ -158,4 +166,31 @@ void oracle_nbest(const float* scores, int64_t dimBatch, int64_t rowLen, int64_t
       outKeys[b * N + n] = (uint32_t)(b * rowLen + best);
     }
   }
+}
+
+/* out[r, :] = scale * E[ids[r], :] (+ signal[(r / rows_per_signal) % n_signals, :]); the product and
+ * the sum round separately (two graph nodes in the reference). */
+void oracle_embed(float* out, const float* E, const uint32_t* ids, int64_t rows, int64_t dimEmb,
+                  float scale, const float* signal, int64_t rows_per_signal, int64_t n_signals) {
+  for(int64_t r = 0; r < rows; ++r) {
+    const float* src = E + (size_t)ids[r] * dimEmb;
+    const float* sg = signal ? signal + ((r / rows_per_signal) % n_signals) * dimEmb : NULL;
+    for(int64_t i = 0; i < dimEmb; ++i) {
+      volatile float scaled = scale * src[i];   /* (kept apart from the addition: no fused multiply-add) */
+      out[r * dimEmb + i] = sg ? scaled + sg[i] : scaled;
+    }
+  }
+}
+
+/* t[j, i] = sin or cos of (j + start) * exp((i % (d/2)) * -log(10000) / (d/2 - 1)), sine for the
+ * first half of the row, cosine for the second; float arithmetic and the C library's expf / sinf /
+ * cosf, as the reference's loop has them. */
+void oracle_sinusoidal_position_embeddings(float* t, int64_t dimWords, int64_t dimEmb, int start) {
+  const float numTimescales = (float)dimEmb / 2;
+  const float logTimescaleIncrement = logf(10000.f) / (numTimescales - 1.f);
+  for(int64_t j = 0; j < dimWords; ++j)
+    for(int64_t i = 0; i < dimEmb; ++i) {
+      const float v = (float)(j + start) * expf((float)(i % (int)numTimescales) * -logTimescaleIncrement);
+      t[j * dimEmb + i] = i < (int)numTimescales ? sinf(v) : cosf(v);
+    }
 }

@@ -103,6 +103,15 @@ def test_argument_validation_returns_codes_not_aborts():
     assert lib.marian_hip_attention(buf, buf, None, None, 0, 0, buf, 2, 2, 1, 40, 64, 0.125, None, None, None, None) == L.ERR_NULL
     assert lib.marian_hip_attention(buf, buf, buf, None, 0, 0, buf, 4, 2, 1, 40, 64, 0.125, None, buf, buf, None) == L.ERR_SHAPE
     assert lib.marian_hip_int8_affine_shortlist(buf, buf, None, buf, 12, buf, 1, 64, 8, 1.0, 0, None) == L.ERR_SHAPE
+    assert lib.marian_hip_embed(buf, buf, 4, 0, 8, 1.0, None, 0, 0, buf, None, None) == L.ERR_SHAPE
+    assert lib.marian_hip_embed(buf, buf, 4, 10, 8, 1.0, buf, 0, 1, buf, None, None) == L.ERR_SHAPE
+    assert lib.marian_hip_embed(buf, None, 4, 10, 8, 1.0, None, 0, 0, buf, None, None) == L.ERR_NULL
+    assert lib.marian_hip_embed(buf, buf, 4096, 10, 8, 1.0, None, 0, 0, buf, buf, None) == L.ERR_RANGE
+    assert lib.marian_hip_embed(buf, buf + 2, 4, 10, 8, 1.0, None, 0, 0, buf, None, None) == L.ERR_ALIGN
+    assert lib.marian_hip_embed(buf, buf, 0, 10, 8, 1.0, None, 0, 0, buf, None, None) == L.OK
+    assert lib.marian_hip_sinusoidal_position_embeddings(None, 4, 8, 0) == L.ERR_NULL
+    assert lib.marian_hip_sinusoidal_position_embeddings(None, 4, 3, 0) == L.ERR_SHAPE
+    assert lib.marian_hip_sinusoidal_position_embeddings(None, 0, 8, 0) == L.OK
     assert lib.marian_hip_int8_prepare_a(buf, buf, 4, 100, buf, 4096, None) == L.ERR_SHAPE
     assert lib.marian_hip_int8_prepare_a(buf, buf, 4096, 1024, buf, 16, None) == L.ERR_WORKSPACE
     assert lib.marian_hip_int8_prepare_a(buf, buf, 0, 64, None, 0, None) == L.OK
@@ -115,6 +124,19 @@ def test_argument_validation_returns_codes_not_aborts():
     assert lib.marian_hip_status_string(L.ERR_ALIAS).decode() == "input and output overlap"
     with pytest.raises(L.MarianHipError):
         L.check(L.ERR_SHAPE, "test")
+
+
+def test_position_signal_made_on_the_host_equals_the_checker():
+    """marian_hip_sinusoidal_position_embeddings makes no HIP call: it runs here, and its rows are
+    the checker's bit for bit (the same float expressions through the same C library)."""
+    import numpy as np
+    from oracle import decode_ops as chk
+    chk.lib()
+    ops = load("ops")
+    for words, d, start in ((1, 1024, 0), (1, 1024, 37), (50, 512, 0), (7, 6, 3), (3, 7, 1), (2, 4, 5)):
+        got = ops.sinusoidalPositionEmbeddings(words, d, start)
+        assert tuple(got.shape) == (words, 1, d)
+        assert np.array_equal(got.numpy().reshape(words, d), chk.sinusoidal_position_embeddings(words, d, start)), (words, d, start)
 
 
 def test_types_match_marian_enum():

@@ -613,3 +613,73 @@ def test_reference_topk_vectors(ops):
     vals2, keys2 = ops.getNBestListOfBeams(dev(x.reshape(1, 1, 4, 3)), v["k"])
     assert np.array_equal(vals2.cpu().numpy(), vals.cpu().numpy())
     assert np.array_equal(keys2.cpu().numpy(), keys.cpu().numpy())
+
+
+def test_reference_rows_vectors(ops):
+    import torch
+    v = reference_vectors()["rows"]
+    A = np.array(v["A"], np.float32).reshape(v["A_shape"])
+    for case in v["cases"]:
+        ids = torch.tensor(case["indices"], dtype=torch.int32, device="cuda")
+        got = ops.rows(dev(A), ids).cpu().numpy()
+        assert got.shape == (len(case["indices"]), 3)
+        assert np.array_equal(got.ravel(), np.array(case["out"], np.float32))
+
+
+@pytest.mark.parametrize("vocab,d,shape,n_sig,rps", [(32000, 1024, (128,), 1, 1), (32000, 1024, (21, 32), 21, 32),
+                                                     (500, 1023, (7, 3), 7, 3), (77, 6, (40,), 3, 8),
+                                                     (1000, 512, (2048,), 4, 1), (64, 8196, (5,), 0, 1),
+                                                     (9, 64, (3000,), 2, 1500)])
+def test_scaled_embeddings_bit_for_bit(ops, chk, integer, synth, vocab, d, shape, n_sig, rps):
+    """the embedding step through the library equals the checker's two float operations per value
+    bit for bit, for decoding-step and whole-sentence shapes, rows that are not a multiple of four
+    wide (the scalar kernel), int32 and int64 indices, ids past the table clamped to its last row;
+    the abs-max slots it leaves are those of a scan of its output"""
+    import torch
+    E = synth.normal(vocab + d, 0, (vocab, d), 0.05)
+    n = int(np.prod(shape))
+    ids = (synth.normal(n, 1, (n,), 1e4).astype(np.int64) % vocab).astype(np.int64)
+    ids[::5] = vocab - 1
+    sig = chk.sinusoidal_position_embeddings(n_sig, d, 3) if n_sig else None
+    scale = np.float32(np.sqrt(np.float32(d)))
+    want = chk.embed(E, ids, scale, sig, rps)
+    dE, dsig = dev(E), (None if sig is None else dev(sig))
+    for dtype in (torch.int32, torch.int64):
+        got = ops.scaledEmbeddings(dE, torch.from_numpy(ids).to(dtype).cuda().reshape(shape), scale, dsig, rps)
+        assert tuple(got.shape) == tuple(shape) + (d,)
+        assert np.array_equal(got.cpu().numpy().reshape(n, d), want)
+    if n <= 2048:
+        got, gmax = ops.scaledEmbeddings(dE, torch.from_numpy(ids).cuda(), scale, dsig, rps, want_absmax=True)
+        assert np.array_equal(got.cpu().numpy(), want)
+        slots = gmax.data.cpu().numpy()
+        assert np.array_equal(slots[:n], np.abs(want).max(-1)) and not slots[n:].any()
+    far = torch.tensor([vocab, 2 ** 31 - 1, 0], dtype=torch.int64, device="cuda")
+    got = ops.scaledEmbeddings(dE, far, 1.0).cpu().numpy()
+    assert np.array_equal(got, E[[vocab - 1, vocab - 1, 0]])
+
+
+def test_scaled_embeddings_feed_the_first_affine_call(ops, integer, synth):
+    """an affine call that takes the abs-max the embedding step leaves gives the bits of the call
+    that scans the embeddings itself"""
+    import torch
+    E = dev(synth.normal(61, 0, (4000, 1024), 0.05))
+    ids = torch.arange(0, 128 * 31, 31, dtype=torch.int32, device="cuda")
+    sig = ops.sinusoidalPositionEmbeddings(1, 1024, 9, device="cuda")
+    x, xmax = ops.scaledEmbeddings(E, ids, 32.0, sig, 128, want_absmax=True)
+    Bq = integer.prepareB(torch.randn(1024, 1024, device="cuda") * 0.02)
+    got, aq = integer.affine_f32(x, Bq, None, absmax=xmax)
+    want, aq_ref = integer.affine_f32(x, Bq, None)
+    assert np.array_equal(aq.numpy(), aq_ref.numpy()) and np.array_equal(got.cpu().numpy(), want.cpu().numpy())
+
+
+def test_scaled_embeddings_argument_checks(ops):
+    import torch
+    mh = load("_lib").MarianHipError
+    E = torch.zeros(10, 8, device="cuda")
+    with pytest.raises(mh):
+        ops.scaledEmbeddings(E, torch.zeros(3, device="cuda"))             # float indices
+    with pytest.raises(mh):
+        ops.scaledEmbeddings(E.view(2, 5, 8), torch.zeros(3, dtype=torch.int32, device="cuda"))
+    with pytest.raises(mh):
+        ops.scaledEmbeddings(E, torch.zeros(3, dtype=torch.int32))           # indices on the host
+    assert tuple(ops.scaledEmbeddings(E, torch.zeros(0, dtype=torch.int32, device="cuda")).shape) == (0, 8)

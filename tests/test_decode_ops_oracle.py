@@ -180,3 +180,49 @@ def test_reference_topk_vectors(ops):
     assert np.array_equal(vals, np.array(v["values"], np.float32))
     rows = np.repeat(np.arange(x.shape[0]), v["k"])
     assert np.array_equal(keys - rows * x.shape[1], np.array(v["indices"], np.uint32))
+
+
+def test_reference_rows_vectors(ops):
+    v = reference_vectors()["rows"]
+    A = np.array(v["A"], np.float32).reshape(v["A_shape"])
+    for case in v["cases"]:
+        got = ops.embed(A, case["indices"])
+        assert got.shape == (len(case["indices"]), 3)
+        assert np.array_equal(got.ravel(), np.array(case["out"], np.float32))
+
+
+def test_embed_scale_and_signal(ops):
+    """scale * E[ids] + signal[(r // rows_per_signal) % n]: against numpy indexing in float64, where
+    the product of two floats is exact and the sum rounds once, so float32(float32(s * e) + g) is what
+    two separate float operations give; a fused multiply-add, a signal row picked by r % n instead
+    of r // rows_per_signal, or a missing scale fail it."""
+    rng = np.random.default_rng(5)
+    E = rng.standard_normal((50, 24)).astype(np.float32)
+    ids = rng.integers(0, 50, 12)
+    sig = rng.standard_normal((4, 24)).astype(np.float32)
+    scale = np.float32(np.sqrt(24.0))
+    prod = (E[ids].astype(f64) * f64(scale)).astype(np.float32)
+    assert np.array_equal(ops.embed(E, ids, scale), prod)
+    want = (prod.astype(f64) + sig[(np.arange(12) // 3) % 4].astype(f64)).astype(np.float32)
+    got = ops.embed(E, ids, scale, sig, rows_per_signal=3)
+    assert np.array_equal(got, want)
+    fused = (E[ids].astype(f64) * f64(scale) + sig[(np.arange(12) // 3) % 4].astype(f64)).astype(np.float32)
+    assert not np.array_equal(fused, want)     # the case does tell one rounding from two
+    wrapped = ops.embed(E, ids, scale, sig[:2], rows_per_signal=3)     # 4 groups of rows, 2 signal rows
+    assert np.array_equal(wrapped[6:], (prod[6:].astype(f64) + sig[(np.arange(6) // 3) % 2].astype(f64)).astype(np.float32))
+
+
+def test_sinusoidal_position_embeddings(ops):
+    """sin / cos of position * 10000^(-i / (d/2 - 1)): float64 closed form within float rounding of
+    the argument (position * 1e-7 relative), zeros and ones at position 0, the two halves of a row
+    a quarter turn apart, `start` a shift of the rows."""
+    d, n = 64, 40
+    t = ops.sinusoidal_position_embeddings(n, d)
+    assert np.array_equal(t[0, :d // 2], np.zeros(d // 2, np.float32)) and np.array_equal(t[0, d // 2:], np.ones(d // 2, np.float32))
+    pos = np.arange(n, dtype=f64)[:, None]
+    freq = 10000.0 ** (-(np.arange(d // 2, dtype=f64)) / (d // 2 - 1))
+    want = np.concatenate([np.sin(pos * freq), np.cos(pos * freq)], axis=1)
+    assert np.all(np.abs(t - want) <= 4e-7 * np.tile(1 + pos * freq, (1, 2)))
+    assert close(t[:, :d // 2] ** 2 + t[:, d // 2:] ** 2, np.ones((n, d // 2)), 1e-6, 0)
+    assert np.array_equal(ops.sinusoidal_position_embeddings(5, d, start=7), t[7:12])
+    assert abs(t[1, 0] - np.sin(1.0)) < 6e-8 and abs(t[1, d // 2 - 1] - 1e-4) < 1e-9

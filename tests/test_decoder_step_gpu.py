@@ -47,7 +47,11 @@ def check_trace(step, trace, orc, chk):
     n_affine = 0
     for kind, t in trace:
         h = {k: (v.cpu().numpy() if hasattr(v, "cpu") else v) for k, v in t.items()}
-        if kind == "affine":
+        if kind == "embed":
+            want = chk.embed(h["E"], h["ids"], np.float32(h["scale"]), h["signal"].reshape(1, -1), step.M)
+            assert np.array_equal(h["out"], want), "embedding step"
+            assert np.array_equal(h["signal"].reshape(-1), chk.sinusoidal_position_embeddings(1, step.d, step.T - 1)[0])
+        elif kind == "affine":
             Bq, bias = t["w"]
             A = h["a"].reshape(-1, h["a"].shape[-1])
             M, K = A.shape
@@ -91,9 +95,11 @@ def check_chain(trace):
     kinds = [k for k, _ in trace]
     per_layer = ["affine"] * 3 + ["self_attention", "affine", "layer_norm", "affine", "context_attention", "affine",
                                   "layer_norm", "affine", "affine", "layer_norm"]
-    layers = (len(kinds) - 3) // len(per_layer)
-    assert kinds == per_layer * layers + ["affine", "logsoftmax", "nbest"]
+    layers = (len(kinds) - 4) // len(per_layer)
+    assert kinds == ["embed"] + per_layer * layers + ["affine", "logsoftmax", "nbest"]
     import torch
+    assert torch.equal(trace[1][1]["a"], trace[0][1]["out"])
+    trace = trace[1:]
     for l in range(layers):
         c = [t for _, t in trace[l * len(per_layer):(l + 1) * len(per_layer)]]
         q, k, v, att, wo, ln1, cq, catt, cwo, ln2, w1, w2, ln3 = c
