@@ -159,6 +159,87 @@ __global__ __launch_bounds__(256) void layer_norm_kernel(const float* in,
   }
 }
 
+// Rows of up to 1024 values: one wave per row and one row per workgroup, four float4 per lane.  The three reductions stay inside the wave, so the kernel has
+// no workgroup barrier and no LDS traffic between its load and its store; scale and shift come as
+// 16-byte loads (gamma_stride / beta_stride 1, 16-byte aligned) or as one broadcast value (0).
+__device__ __forceinline__ float wave_sum16(float v) {   // DPP within rows of 16 lanes, then across the four rows
+  v = row16_sum(v);
+  v += __shfl_xor(v, 16, 64);
+  v += __shfl_xor(v, 32, 64);
+  return v;
+}
+__global__ __launch_bounds__(64) void layer_norm_wave_kernel(const float* in, const float* __restrict__ add,
+                                                             const float* __restrict__ gamma, int gamma_stride,
+                                                             const float* __restrict__ beta, int beta_stride,
+                                                             float* out, int cols, float eps,
+                                                             float* __restrict__ absmax_out) {
+  constexpr int VPL = 4;
+  const size_t row = blockIdx.x;
+  const int lane = threadIdx.x, cols4 = cols / 4;
+  const v4f* x = reinterpret_cast<const v4f*>(in + row * cols);
+  const v4f* a = add ? reinterpret_cast<const v4f*>(add + row * cols) : nullptr;
+  v4f* y = reinterpret_cast<v4f*>(out + row * cols);
+  const v4f zero = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+  v4f v[VPL], t[VPL], gm[VPL], bt[VPL];
+  // all loads at once, positions past the row clamped and dropped afterwards
+#pragma unroll
+  for(int j = 0; j < VPL; ++j) {
+    const int i = min(j * 64 + lane, cols4 - 1);
+    v[j] = x[i];
+    t[j] = a ? a[i] : zero;
+    if(gamma_stride) gm[j] = reinterpret_cast<const v4f*>(gamma)[i];
+    if(beta && beta_stride) bt[j] = reinterpret_cast<const v4f*>(beta)[i];
+  }
+  if(!gamma_stride) {
+    const float g0 = gamma[0];
+#pragma unroll
+    for(int j = 0; j < VPL; ++j) gm[j] = v4f{g0, g0, g0, g0};
+  }
+  if(!(beta && beta_stride)) {
+    const float b0 = beta ? beta[0] : 0.0f;
+#pragma unroll
+    for(int j = 0; j < VPL; ++j) bt[j] = v4f{b0, b0, b0, b0};
+  }
+  float sum = 0.0f;
+#pragma unroll
+  for(int j = 0; j < VPL; ++j) {
+    if(a) v[j] = v4f{v[j].x + t[j].x, v[j].y + t[j].y, v[j].z + t[j].z, v[j].w + t[j].w};
+    if(j * 64 + lane < cols4) sum += (v[j].x + v[j].y) + (v[j].z + v[j].w);
+  }
+  const float mean = wave_sum16(sum) / (float)cols;
+  float sq = 0.0f;
+#pragma unroll
+  for(int j = 0; j < VPL; ++j) {
+    if(j * 64 + lane < cols4) {
+      const float d0 = v[j].x - mean, d1 = v[j].y - mean, d2 = v[j].z - mean, d3 = v[j].w - mean;
+      sq += (d0 * d0 + d1 * d1) + (d2 * d2 + d3 * d3);
+    }
+  }
+  const float sigma = sqrtf(wave_sum16(sq) / (float)cols + eps);
+  float omax = 0.0f;
+#pragma unroll
+  for(int j = 0; j < VPL; ++j) {
+    const int i = j * 64 + lane;
+    if(i < cols4) {
+      float r[4] = {v[j].x, v[j].y, v[j].z, v[j].w};
+      const float g[4] = {gm[j].x, gm[j].y, gm[j].z, gm[j].w}, b[4] = {bt[j].x, bt[j].y, bt[j].z, bt[j].w};
+#pragma unroll
+      for(int e = 0; e < 4; ++e) {
+        float o = g[e] * ((r[e] - mean) / sigma);
+        if(beta) o = o + b[e];
+        r[e] = o;
+        omax = fmaxf(omax, fabsf(o));
+      }
+      y[i] = v4f{r[0], r[1], r[2], r[3]};
+    }
+  }
+  if(absmax_out) {   // slot `row`; the slots past the last row are zeroed by all workgroups together
+    omax = wave_maxf(omax);
+    if(lane == 0) absmax_out[row] = omax;
+    for(int sl = (int)gridDim.x + (int)row * 64 + lane; sl < kAbsmaxSlots; sl += (int)gridDim.x * 64) absmax_out[sl] = 0.0f;
+  }
+}
+
 // ---------------------------------------------------------------- softmax / log-softmax
 // THREADS threads per row, 256 / THREADS... rows per workgroup: 64 (a wave per row, four rows
 // per workgroup: attention scores) or 1024 (vocabulary-size rows).  Three passes over the row:
@@ -1154,7 +1235,11 @@ int marian_hip_layer_norm(const float* in, const float* add, const float* gamma,
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   const int gs = gamma_cols > 1 ? 1 : 0, bs = (beta && beta_cols > 1) ? 1 : 0;
   const bool vec = cols % 4 == 0 && aligned16(in) && aligned16(out) && (!add || aligned16(add));
-  if(vec && cols <= 1024)
+  const bool wave_form = vec && cols <= 1024 && (gs == 0 || aligned16(gamma)) &&
+                         (!beta || bs == 0 || aligned16(beta));
+  if(wave_form)
+    hipLaunchKernelGGL(layer_norm_wave_kernel, dim3((unsigned)rows), dim3(64), 0, st, in, add, gamma, gs, beta, bs, out, (int)cols, eps, absmax_out);
+  else if(vec && cols <= 1024)
     hipLaunchKernelGGL(layer_norm_kernel<1>, dim3((unsigned)rows), dim3(256), 0, st, in, add, gamma, gs, beta, bs, out, (int)cols, eps, absmax_out);
   else if(vec && cols <= 4096)
     hipLaunchKernelGGL(layer_norm_kernel<4>, dim3((unsigned)rows), dim3(256), 0, st, in, add, gamma, gs, beta, bs, out, (int)cols, eps, absmax_out);

@@ -683,3 +683,42 @@ def test_scaled_embeddings_argument_checks(ops):
     with pytest.raises(mh):
         ops.scaledEmbeddings(E, torch.zeros(3, dtype=torch.int32))           # indices on the host
     assert tuple(ops.scaledEmbeddings(E, torch.zeros(0, dtype=torch.int32, device="cuda")).shape) == (0, 8)
+
+
+@pytest.mark.parametrize("rows,cols", [(3000, 512), (300, 768), (70, 1024), (2048, 256), (9, 4)])
+def test_layer_norm_one_wave_per_row(ops, chk, synth, rows, cols):
+    """rows of up to 1024 values take the kernel that gives a row to one wave: scale and shift as
+    vectors, as single values and from addresses that are not 16-byte aligned (the workgroup-per-row
+    kernel behind the same entry point), with and without the skip input; the abs-max slots are
+    those of a scan of the output, zero past the last row"""
+    import torch
+    x = synth.normal(rows + cols, 0, (rows, cols), 1.5) - np.float32(0.2)
+    add = synth.normal(rows + cols, 1, (rows, cols), 0.7)
+    g = synth.normal(cols, 2, (cols + 1,), 0.2) + np.float32(1.0)
+    b = synth.normal(cols, 3, (cols + 1,), 0.5)
+
+    def want(g_, b_, add_):
+        xs = (x if add_ is None else x + add_).astype(f64)
+        mean = xs.mean(-1, keepdims=True)
+        var = ((xs - mean) ** 2).mean(-1, keepdims=True)
+        return g_.astype(f64) * (xs - mean) / np.sqrt(var + 1e-6) + (0 if b_ is None else b_.astype(f64))
+    dg, db = dev(g), dev(b)
+    for g_, b_, add_, dg_, db_ in ((g[:cols], b[:cols], add, dg[:cols], db[:cols]),
+                                   (g[1:], b[1:], None, dg[1:], db[1:]),            # 4 bytes off a 16-byte boundary
+                                   (g[:1], None, add, dg[:1], None),
+                                   (g[:cols], b[:1], None, dg[:cols], db[:1])):
+        got = ops.layerNorm(dev(x), dg_, db_, 1e-6, None if add_ is None else dev(add_))
+        close(got.cpu().numpy(), want(g_, b_, add_), REL, 2e-6)
+        close(got.cpu().numpy(), chk.layer_norm(x, g_, b_, 1e-6, add=add_), 2 * REL, 4e-6)
+    if rows <= 2048:
+        y, ymax = ops.layerNorm(dev(x), dg[:cols], db[:cols], 1e-6, dev(add), want_absmax=True)
+        slots = ymax.data.cpu().numpy()
+        assert np.array_equal(slots[:rows], np.abs(y.cpu().numpy()).max(-1)) and not slots[rows:].any()
+    # in place: the output may be the input
+    xin = dev(x)
+    ref = ops.layerNorm(xin, dg[:cols], db[:cols], 1e-6).cpu().numpy()
+    L = load("_lib")
+    st = L.lib().marian_hip_layer_norm(xin.data_ptr(), None, dg.data_ptr(), cols, db.data_ptr(), cols, xin.data_ptr(),
+                                       rows, cols, 1e-6, None, None)
+    torch.cuda.synchronize()
+    assert st == 0 and np.array_equal(xin.cpu().numpy(), ref)
