@@ -679,6 +679,9 @@ def main():
         fdt = time_graphs(torch, full, n, max(4, args.warmup // 2))
         gonly = [capture(torch, (lambda c=c: dec.step(c, gemm_only=True))) for c in range(bsets)]
         gdt = time_graphs(torch, gonly, n, max(4, args.warmup // 2))
+        sel = [capture(torch, (lambda c=c: dec.step(c, fused_tail=True, select=True))) for c in range(bsets)]
+        seldt = time_graphs(torch, sel, n, max(4, args.warmup // 2))
+        del sel
         out["transformer_big_decode_full"] = {
             "what": "full decoder step through the host mirrors, from the previous step's word indices: embedding rows x "
                     "sqrt(d) + position signal (one launch), 49 int8 affine calls + per layer "
@@ -688,6 +691,10 @@ def main():
                     "sentence in one launch (the log-probabilities are not written out); no hypothesis bookkeeping; the "
                     "abs-max of every GEMM input is left by the kernel that produced it",
             "ms_per_step": round(fdt / n * 1e3, 4),
+            "ms_per_step_with_state_selection": round(seldt / n * 1e3, 4),
+            "state_selection": "the step preceded by the beam search's selection of the surviving hypotheses' cached keys "
+                               "and values (rows(state, hypIndices) over all layers as one gather, %d MB read and written); "
+                               "hypothesis indices resident on the device" % round(dec.state.numel() * 4 / 1e6),
             "ms_per_step_logsoftmax_and_nbest_as_two_launches": round(sdt / n * 1e3, 4),
             "one_launch_tail_equals_two_launches": same_tail,
             "ms_per_step_unchained": round(udt / n * 1e3, 4),

@@ -110,8 +110,12 @@ int marian_hip_attention(const float* q, float* k, float* v, const float* mask, 
  *   signal: NULL (no sum: a pure gather when scale == 1), or [n_signals, dimEmb].  A decoding step
  *   passes the one row of its position (n_signals == 1); a whole sentence batch [dimWords,
  *   dimBatch] passes rows_per_signal = dimBatch, n_signals = dimWords.
- *   absmax_out: as for marian_hip_layer_norm (needs rows <= 2048): the int8 products of the first
- *   layer then need no abs-max launch of their own.
+ *   absmax_out: as for marian_hip_layer_norm (needs rows * ceil(dimEmb / 4096) <= 2048): the int8
+ *   products of the first layer then need no abs-max launch of their own.
+ * With scale 1 and no signal the call is rows(E, ids) itself, which is also the selection of the
+ * surviving hypotheses' decoder states between two steps of the beam search (reference
+ * src/rnn/types.h:22-42: rows(reshape(state, [beam * batch, positions * depth]), selIdx)); rows
+ * longer than 4096 values are split over several workgroups.
  */
 int marian_hip_embed(const float* E, const uint32_t* ids, int64_t rows, int64_t vocab, int64_t dimEmb,
                      float scale, const float* signal, int64_t rows_per_signal, int64_t n_signals,

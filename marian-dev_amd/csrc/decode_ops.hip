@@ -1157,9 +1157,12 @@ __global__ __launch_bounds__(256) void fill_kernel(unsigned char* __restrict__ p
 }
 
 // ---------------------------------------------------------------- embedding step
-// One workgroup per output row: out[r, :] = scale * E[ids[r], :] (+ signal[(r / rows_per_signal) %
-// n_signals, :]).  The product and the sum round separately.  An id at or past the table's end reads
-// the table's last row.
+// Workgroup (r, chunk) takes kEmbedChunk values of output row r: out[r, :] = scale * E[ids[r], :]
+// (+ signal[(r / rows_per_signal) % n_signals, :]); rows of an embedding table are one chunk, the
+// long rows of a decoder state (all cached positions of a hypothesis) many, so that such a gather
+// fills the chip.  The product and the sum round separately.  An id at or past the table's end
+// reads the table's last row.
+constexpr int kEmbedChunk = 4096;
 template <bool VEC>
 __global__ __launch_bounds__(256) void embed_kernel(const float* __restrict__ E, const uint32_t* __restrict__ ids,
                                                     unsigned vocab, int dimEmb, float scale,
@@ -1167,37 +1170,49 @@ __global__ __launch_bounds__(256) void embed_kernel(const float* __restrict__ E,
                                                     unsigned n_signals, float* __restrict__ out,
                                                     float* __restrict__ absmax_out) {
   __shared__ float red[4];
-  const unsigned row = blockIdx.x;
+  const unsigned row = blockIdx.x, chunk = blockIdx.y;
   const int tid = threadIdx.x;
   unsigned id = ids[row];
   id = id < vocab ? id : vocab - 1u;
+  const int c0 = (int)chunk * kEmbedChunk, c1 = min(c0 + kEmbedChunk, dimEmb);
   const float* src = E + (size_t)id * dimEmb;
   const float* sg = signal ? signal + (size_t)((row / rows_per_signal) % n_signals) * dimEmb : nullptr;
   float* y = out + (size_t)row * dimEmb;
   float omax = 0.0f;
-  if(VEC) {
-    for(int i = tid; i < dimEmb / 4; i += 256) {
-      const v4f e = reinterpret_cast<const v4f*>(src)[i];
-      v4f s = v4f{0.0f, 0.0f, 0.0f, 0.0f};
-      if(sg) s = reinterpret_cast<const v4f*>(sg)[i];
-      v4f r = v4f{scale * e.x, scale * e.y, scale * e.z, scale * e.w};
-      if(sg) r = v4f{r.x + s.x, r.y + s.y, r.z + s.z, r.w + s.w};
-      omax = fmaxf(fmaxf(omax, fmaxf(fabsf(r.x), fabsf(r.y))), fmaxf(fabsf(r.z), fabsf(r.w)));
-      reinterpret_cast<v4f*>(y)[i] = r;
+  if(VEC) {   // (four 16-byte loads per thread and operand, all requested before the first is used)
+    constexpr int kV = kEmbedChunk / 4 / 256;
+    const int last = c1 / 4 - 1;
+    v4f e[kV], s[kV];
+#pragma unroll
+    for(int j = 0; j < kV; ++j) {
+      const int i = min(c0 / 4 + j * 256 + tid, last);
+      e[j] = reinterpret_cast<const v4f*>(src)[i];
+      s[j] = sg ? reinterpret_cast<const v4f*>(sg)[i] : v4f{0.0f, 0.0f, 0.0f, 0.0f};
+    }
+#pragma unroll
+    for(int j = 0; j < kV; ++j) {
+      const int i = c0 / 4 + j * 256 + tid;
+      if(i <= last) {
+        v4f r = v4f{scale * e[j].x, scale * e[j].y, scale * e[j].z, scale * e[j].w};
+        if(sg) r = v4f{r.x + s[j].x, r.y + s[j].y, r.z + s[j].z, r.w + s[j].w};
+        omax = fmaxf(fmaxf(omax, fmaxf(fabsf(r.x), fabsf(r.y))), fmaxf(fabsf(r.z), fabsf(r.w)));
+        reinterpret_cast<v4f*>(y)[i] = r;
+      }
     }
   } else {
-    for(int i = tid; i < dimEmb; i += 256) {
+    for(int i = c0 + tid; i < c1; i += 256) {
       float r = scale * src[i];
       if(sg) r = r + sg[i];
       omax = fmaxf(omax, fabsf(r));
       y[i] = r;
     }
   }
-  if(absmax_out) {   // slot `row`; workgroup 0 zeroes the slots past the last row
+  if(absmax_out) {   // a slot per workgroup; the first workgroup zeroes the slots past the last one
+    const unsigned slot = row * gridDim.y + chunk, slots = gridDim.x * gridDim.y;
     omax = row_reduce<256, true>(omax, red);
-    if(tid == 0) absmax_out[row] = omax;
-    if(row == 0)
-      for(int sl = gridDim.x + tid; sl < kAbsmaxSlots; sl += 256) absmax_out[sl] = 0.0f;
+    if(tid == 0) absmax_out[slot] = omax;
+    if(slot == 0)
+      for(int sl = (int)slots + tid; sl < kAbsmaxSlots; sl += 256) absmax_out[sl] = 0.0f;
   }
 }
 
@@ -1254,13 +1269,14 @@ int marian_hip_layer_norm(const float* in, const float* add, const float* gamma,
 int marian_hip_embed(const float* E, const uint32_t* ids, int64_t rows, int64_t vocab, int64_t dimEmb,
                      float scale, const float* signal, int64_t rows_per_signal, int64_t n_signals,
                      float* out, float* absmax_out, void* stream) {
-  if(absmax_out && rows > kAbsmaxSlots) return MARIAN_HIP_ERR_RANGE;
-  if(absmax_out && !aligned4(absmax_out)) return MARIAN_HIP_ERR_ALIGN;
   if(rows < 0 || vocab <= 0 || dimEmb <= 0) return MARIAN_HIP_ERR_SHAPE;
+  const int64_t chunks = (dimEmb + kEmbedChunk - 1) / kEmbedChunk;
+  if(absmax_out && rows * chunks > kAbsmaxSlots) return MARIAN_HIP_ERR_RANGE;
+  if(absmax_out && !aligned4(absmax_out)) return MARIAN_HIP_ERR_ALIGN;
   if(signal && (rows_per_signal <= 0 || n_signals <= 0)) return MARIAN_HIP_ERR_SHAPE;
   if(rows == 0) return MARIAN_HIP_OK;
   if(!E || !ids || !out) return MARIAN_HIP_ERR_NULL;
-  if(rows * dimEmb > kMaxElemsOps || vocab > 0xFFFFFFFFLL || rows_per_signal > 0x7FFFFFFFLL ||
+  if(chunks > 65535 || rows * dimEmb > kMaxElemsOps || vocab > 0xFFFFFFFFLL || rows_per_signal > 0x7FFFFFFFLL ||
      n_signals > 0x7FFFFFFFLL || (signal && n_signals * dimEmb > kMaxElemsOps))
     return MARIAN_HIP_ERR_RANGE;
   if(!aligned4(E) || !aligned4(ids) || !aligned4(out) || (signal && !aligned4(signal))) return MARIAN_HIP_ERR_ALIGN;
@@ -1268,11 +1284,11 @@ int marian_hip_embed(const float* E, const uint32_t* ids, int64_t rows, int64_t 
   const bool vec = dimEmb % 4 == 0 && aligned16(E) && aligned16(out) && (!signal || aligned16(signal));
   const unsigned rps = signal ? (unsigned)rows_per_signal : 1u, ns = signal ? (unsigned)n_signals : 1u;
   if(vec)
-    hipLaunchKernelGGL(embed_kernel<true>, dim3((unsigned)rows), dim3(256), 0, st, E, ids, (unsigned)vocab, (int)dimEmb,
-                       scale, signal, rps, ns, out, absmax_out);
+    hipLaunchKernelGGL(embed_kernel<true>, dim3((unsigned)rows, (unsigned)chunks), dim3(256), 0, st, E, ids,
+                       (unsigned)vocab, (int)dimEmb, scale, signal, rps, ns, out, absmax_out);
   else
-    hipLaunchKernelGGL(embed_kernel<false>, dim3((unsigned)rows), dim3(256), 0, st, E, ids, (unsigned)vocab, (int)dimEmb,
-                       scale, signal, rps, ns, out, absmax_out);
+    hipLaunchKernelGGL(embed_kernel<false>, dim3((unsigned)rows, (unsigned)chunks), dim3(256), 0, st, E, ids,
+                       (unsigned)vocab, (int)dimEmb, scale, signal, rps, ns, out, absmax_out);
   MH_HIP(hipGetLastError());
   return MARIAN_HIP_OK;
 }

@@ -69,8 +69,18 @@ class DecoderStep:
         self.signal = ops.sinusoidalPositionEmbeddings(1, d, t_past, device="cuda")
         self.emb_scale = float(torch.sqrt(torch.tensor(float(d))))
         self.x = torch.randn(M, d, device="cuda", generator=g)   # (input of the GEMM-only chain)
-        self.Kself = [torch.randn(M * H, self.T, d // H, device="cuda", generator=g) for _ in range(layers)]
-        self.Vself = [torch.randn(M * H, self.T, d // H, device="cuda", generator=g) for _ in range(layers)]
+        # the self-attention caches of all layers are rows of one tensor [2 * layers * M, H * T * dk] (a
+        # hypothesis's cached positions of one layer are one row), so that the beam search's selection
+        # of the surviving hypotheses is one gather; a second tensor of that size receives it
+        self.state = torch.randn(2 * layers * M, H * self.T * (d // H), device="cuda", generator=g)
+        self.state_next = torch.empty_like(self.state)
+        self._cache_views()
+        # back-pointers of a beam-search step: hypothesis (k, b) continues hypothesis (k', b) of the
+        # same sentence; flat index k * batch + b, one copy per cache tensor
+        parent = torch.randint(0, beam, (beam, batch), device="cuda", generator=g) * batch + torch.arange(batch, device="cuda")
+        self.hyp_indices = parent.reshape(-1).to(torch.int32)
+        self.state_rows = (torch.arange(2 * layers, device="cuda", dtype=torch.int32)[:, None] * M +
+                           self.hyp_indices[None, :]).reshape(-1).contiguous()
         self.Kenc = [torch.randn(self.batch * H, self.L, d // H, device="cuda", generator=g) for _ in range(layers)]
         self.Venc = [torch.randn(self.batch * H, self.L, d // H, device="cuda", generator=g) for _ in range(layers)]
         # source lengths uniform over min_src_len .. src_len, padded to the longest (the mask covers the rest)
@@ -78,13 +88,28 @@ class DecoderStep:
         self.src_lens = lens
         self.mask = (torch.arange(self.L, device="cuda")[None, :] >= lens[:, None]).float() * -99999999.0
 
-    def step(self, s, gemm_only=False, chained=True, grouped=True, fused_tail=False):
+    def _cache_views(self):
+        M, H, T, dk, layers = self.M, self.H, self.T, self.d // self.H, self.layers
+        self.Kself = [self.state[l * M:(l + 1) * M].view(M * H, T, dk) for l in range(layers)]
+        self.Vself = [self.state[(layers + l) * M:(layers + l + 1) * M].view(M * H, T, dk) for l in range(layers)]
+
+    def select_states(self):
+        """The decoder state of the surviving hypotheses (reference src/models/states.h:87-107,
+        src/rnn/types.h:22-42: rows(state, hypIndices) per cached tensor) for all layers in one
+        gather; the two state tensors swap roles."""
+        self.ops.rows(self.state, self.state_rows, out=self.state_next)
+        self.state, self.state_next = self.state_next, self.state
+        self._cache_views()
+
+    def step(self, s, gemm_only=False, chained=True, grouped=True, fused_tail=False, select=False):
         """chained: every tensor that feeds an affine call leaves its abs-max where it is
         produced (layer norm, attention, the ReLU GEMM), so those calls skip their abs-max pass.
         grouped: the self-attention projections Wq, Wk, Wv (one input, three weight matrices,
         reference src/models/transformer.h:290-325) go through one call.
         fused_tail: log-softmax and n-best in one launch (the log-probabilities are not written);
-        the step then returns (scores, keys) of the n-best instead of the log-probabilities."""
+        the step then returns (scores, keys) of the n-best instead of the log-probabilities.
+        select: the step starts with the selection of the surviving hypotheses' cached keys and
+        values by the back-pointers self.hyp_indices, as a beam-search step does."""
         integer, ops = self.integer, self.ops
         W = self.sets[s % len(self.sets)]
         tr = self.trace
@@ -96,6 +121,10 @@ class DecoderStep:
         dk = d // H
         x, xmax = self.x, None
         ch = chained and not gemm_only
+        if select and not gemm_only:
+            before = self.state
+            self.select_states()
+            rec("select", state=before, rows=self.state_rows, out=self.state)
         if not gemm_only:
             x = ops.scaledEmbeddings(self.E, self.words, self.emb_scale, self.signal, M, want_absmax=ch)
             if ch:

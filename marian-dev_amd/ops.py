@@ -51,11 +51,12 @@ def layerNorm(x, gamma, beta=None, eps=1e-9, add=None, want_absmax=False):
     return (out, omax) if want_absmax else out
 
 
-def scaledEmbeddings(E, ids, scale=1.0, signal=None, rowsPerSignal=1, want_absmax=False):
+def scaledEmbeddings(E, ids, scale=1.0, signal=None, rowsPerSignal=1, want_absmax=False, out=None):
     """scale * E[ids] (+ signal): the embedding step in front of the first layer (reference
     src/layers/embedding.cpp:161-168 and src/models/transformer.h:93,117) as one launch.  E
     [vocab, dimEmb]; ids: integer tensor on the device, any shape; signal: None or [n, dimEmb],
-    output row r taking signal row (r / rowsPerSignal) % n.  Returns [*ids.shape, dimEmb]."""
+    output row r taking signal row (r / rowsPerSignal) % n.  Returns [*ids.shape, dimEmb] (`out`
+    when given: a contiguous float32 tensor of that many values that does not overlap E)."""
     E = _f32c(E, "scaledEmbeddings")
     be = _backend_of(E)
     _abort_if(E.dim() != 2, "scaledEmbeddings: the table has to be a matrix, got shape {}", tuple(E.shape))
@@ -69,7 +70,14 @@ def scaledEmbeddings(E, ids, scale=1.0, signal=None, rowsPerSignal=1, want_absma
     if signal is not None:
         signal = _f32c(signal, "scaledEmbeddings").reshape(-1, dimEmb)
         n_signals = signal.shape[0]
-    out = torch.empty(tuple(ids.shape) + (dimEmb,), dtype=torch.float32, device=E.device)
+    if out is None:
+        out = torch.empty(tuple(ids.shape) + (dimEmb,), dtype=torch.float32, device=E.device)
+    else:
+        _abort_if(out.dtype != torch.float32 or not out.is_contiguous() or out.device != E.device or
+                  out.numel() != ids.numel() * dimEmb, "scaledEmbeddings: out has to be a contiguous float32 "
+                  "tensor of {} x {} values on the table's device", ids.numel(), dimEmb)
+        lo, hi = out.data_ptr(), out.data_ptr() + 4 * out.numel()
+        _abort_if(lo < E.data_ptr() + 4 * E.numel() and E.data_ptr() < hi, "scaledEmbeddings: out overlaps the table")
     omax = AbsMax(E.device) if want_absmax else None
     st = be.lib.marian_hip_embed(E.data_ptr(), words.data_ptr(), words.numel(), vocab, dimEmb, float(scale),
                                  None if signal is None else signal.data_ptr(), rowsPerSignal, n_signals,
@@ -78,9 +86,11 @@ def scaledEmbeddings(E, ids, scale=1.0, signal=None, rowsPerSignal=1, want_absma
     return (out, omax) if want_absmax else out
 
 
-def rows(a, indices):
-    """reference rows(a, indices) (CopyRows, src/tensors/cpu/tensor_operators.cpp:577-603)"""
-    return scaledEmbeddings(a, indices.reshape(-1))
+def rows(a, indices, out=None):
+    """reference rows(a, indices) (CopyRows, src/tensors/cpu/tensor_operators.cpp:577-603); also
+    the selection of the surviving hypotheses' decoder states between two steps of the beam search
+    (reference src/rnn/types.h:22-42)"""
+    return scaledEmbeddings(a, indices.reshape(-1), out=out)
 
 
 def sinusoidalPositionEmbeddings(dimWords, dimEmb, start=0, device=None):

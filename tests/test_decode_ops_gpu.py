@@ -648,14 +648,30 @@ def test_scaled_embeddings_bit_for_bit(ops, chk, integer, synth, vocab, d, shape
         got = ops.scaledEmbeddings(dE, torch.from_numpy(ids).to(dtype).cuda().reshape(shape), scale, dsig, rps)
         assert tuple(got.shape) == tuple(shape) + (d,)
         assert np.array_equal(got.cpu().numpy().reshape(n, d), want)
-    if n <= 2048:
+    chunks = (d + 4095) // 4096     # a slot per 4096 values of a row
+    if n * chunks <= 2048:
         got, gmax = ops.scaledEmbeddings(dE, torch.from_numpy(ids).cuda(), scale, dsig, rps, want_absmax=True)
         assert np.array_equal(got.cpu().numpy(), want)
         slots = gmax.data.cpu().numpy()
-        assert np.array_equal(slots[:n], np.abs(want).max(-1)) and not slots[n:].any()
+        padded = np.zeros((n, chunks * 4096), np.float32)
+        padded[:, :d] = np.abs(want)
+        assert np.array_equal(slots[:n * chunks], padded.reshape(n * chunks, 4096).max(-1)) and not slots[n * chunks:].any()
     far = torch.tensor([vocab, 2 ** 31 - 1, 0], dtype=torch.int64, device="cuda")
     got = ops.scaledEmbeddings(dE, far, 1.0).cpu().numpy()
     assert np.array_equal(got, E[[vocab - 1, vocab - 1, 0]])
+
+
+@pytest.mark.parametrize("hyps,row", [(128, 16 * 21 * 64), (12, 4096 * 3 + 4), (40, 8193), (5, 4096), (3, 70001)])
+def test_rows_of_a_decoder_state(ops, synth, hyps, row):
+    """rows() as the beam search uses it between two steps: the cached positions of the surviving
+    hypotheses, one long row each (split over several workgroups), picked by their back-pointers -
+    a pure copy, so the result is the numpy gather bit for bit"""
+    import torch
+    state = synth.normal(hyps + row, 0, (hyps, row), 1.0)
+    back = (synth.normal(hyps, 1, (hyps,), 1e3).astype(np.int64) % hyps)
+    got = ops.rows(dev(state), torch.from_numpy(back).cuda())
+    assert tuple(got.shape) == (hyps, row)
+    assert np.array_equal(got.cpu().numpy(), state[back])
 
 
 def test_scaled_embeddings_feed_the_first_affine_call(ops, integer, synth):

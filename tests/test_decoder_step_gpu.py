@@ -147,3 +147,14 @@ def test_decoder_step_every_call_against_the_checker(integer, orc, size):
     nbest = [e for kind, e in trace if kind == "nbest"][0]
     vals, keys = step.step(0, fused_tail=True)
     assert torch.equal(vals, nbest["vals"]) and torch.equal(keys, nbest["keys"])
+    # a beam-search step starts with the selection of the surviving hypotheses' cached keys and values
+    # (one gather over all layers): the step on the gathered caches
+    for t, c in zip(step.Kself + step.Vself, caches):
+        t.copy_(c)
+    gathered = step.state[step.state_rows.long()].clone()
+    vals_s, keys_s = step.step(0, fused_tail=True, select=True)
+    torch.cuda.synchronize()
+    step.state.copy_(gathered)
+    vals_r, keys_r = step.step(0, fused_tail=True)
+    assert torch.equal(vals_s, vals_r) and torch.equal(keys_s, keys_r)
+    assert not torch.equal(vals_s, vals)
