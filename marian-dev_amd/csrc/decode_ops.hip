@@ -65,6 +65,23 @@ __device__ __forceinline__ float row_reduce(float v, float* red) {
   return v;
 }
 
+// The same for a `red` that nothing has read or written since the last workgroup barrier (a
+// fresh array per reduction): no barrier in front.
+template <int THREADS, bool MAX>
+__device__ __forceinline__ float row_reduce_fresh(float v, float* red) {
+  v = MAX ? wave_maxf(v) : wave_sum(v);
+  if(THREADS > 64) {
+    const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+    if(lane == 0) red[wave] = v;
+    __syncthreads();
+    float r = red[0];
+#pragma unroll
+    for(int w = 1; w < THREADS / 64; ++w) r = MAX ? (red[w] > r ? red[w] : r) : r + red[w];
+    v = r;
+  }
+  return v;
+}
+
 // ---------------------------------------------------------------- layer normalization
 // One workgroup of 256 threads per row.  CACHE float4 vectors per thread hold the row in
 // registers (cols <= 1024 * CACHE, cols % 4 == 0, 16-byte aligned rows); CACHE == 0 is the
@@ -279,9 +296,16 @@ __global__ __launch_bounds__(THREADS < 256 ? 256 : THREADS) void softmax_kernel(
 // operations per element as softmax_kernel.
 // softmax_wide_row leaves in v (vector j of thread t = elements 4 * (j * THREADS + t) .. + 3 of the
 // row, where they exist): LOG: x - max, and returns log(sum of exp(x - max)); otherwise exp(x - max),
-// and returns their sum.
-template <bool LOG, int THREADS, int VPT>
-__device__ __forceinline__ float softmax_wide_row(const v4f* x, const v4f* mk, int cols4, v4f (&v)[VPT], float* red) {
+// and returns their sum.  red: 2 * THREADS / 64 floats that nothing else uses meanwhile (the wave
+// maxima, then the wave sums: no barrier in front of either reduction).  after_max(max, wave maxima)
+// runs between the two reductions, when the THREADS / 64 wave maxima are in red[0 ...]; they stay
+// there.
+struct NoAfterMax {
+  __device__ void operator()(float, const float*) const {}
+};
+template <bool LOG, int THREADS, int VPT, typename AfterMax = NoAfterMax>
+__device__ __forceinline__ float softmax_wide_row(const v4f* x, const v4f* mk, int cols4, v4f (&v)[VPT], float* red,
+                                                  AfterMax after_max = AfterMax()) {
   const int t = threadIdx.x;
   float mx = -__builtin_inff();
   // (all loads at once, positions past the row clamped and dropped afterwards: a load behind a
@@ -306,7 +330,8 @@ __device__ __forceinline__ float softmax_wide_row(const v4f* x, const v4f* mk, i
       mx = c > mx ? c : mx;
     }
   }
-  mx = row_reduce<THREADS, true>(mx, red);
+  mx = row_reduce_fresh<THREADS, true>(mx, red);
+  after_max(mx, red);
   float sum = 0.0f;
 #pragma unroll
   for(int j = 0; j < VPT; ++j) {
@@ -324,7 +349,7 @@ __device__ __forceinline__ float softmax_wide_row(const v4f* x, const v4f* mk, i
       }
     }
   }
-  sum = row_reduce<THREADS, false>(sum, red);
+  sum = row_reduce_fresh<THREADS, false>(sum, red + THREADS / 64);
   return LOG ? logf(sum) : sum;
 }
 
@@ -332,7 +357,7 @@ template <bool LOG, int THREADS, int VPT>
 __global__ __launch_bounds__(THREADS) void softmax_wide_kernel(const float* in, const float* __restrict__ mask,
                                                                 long long n_masks, long long rows_per_mask,
                                                                 float* out, int cols) {
-  __shared__ float red[THREADS / 64];
+  __shared__ float red[2 * THREADS / 64];
   const size_t row = blockIdx.x;
   const v4f* x = reinterpret_cast<const v4f*>(in + row * cols);
   const v4f* mk = mask ? reinterpret_cast<const v4f*>(mask + (size_t)((row / rows_per_mask) % n_masks) * cols) : nullptr;
@@ -832,39 +857,32 @@ __device__ __forceinline__ void nbest_wave_draw(const float* lv, const unsigned*
 // called once for r = 0 .. N-1 (best first) by one thread each; index is the position within x.
 // scan(f) calls f(value, index) for every element this thread owns (each element of the row is
 // owned by exactly one thread of the workgroup; the order does not matter).
+// The N-th largest of 16 values in LDS (equal values in index order), the same in every thread:
+// lane l % 16 ranks value l % 16, the one of rank N - 1 is it (the cost does not grow with N).
+__device__ __forceinline__ float nth_largest_of_16(const float* w16, int N) {
+  const int c = threadIdx.x % 16;
+  const float cvv = w16[c];
+  int rank = 0;
+#pragma unroll
+  for(int w = 0; w < 16; ++w) rank += (w16[w] > cvv || (w16[w] == cvv && w < c)) ? 1 : 0;
+  const unsigned long long holders = __ballot(rank == N - 1) & 0xFFFFull;
+  return __shfl(cvv, __ffsll((long long)holders) - 1, 64);   // (ranks 0..15 are all taken: one holder)
+}
+
+// Steps 2 and 3: tv is a bound that at least N elements of the row reach (or -inf).
+// count_is_zero: sh.count has been zero since a workgroup barrier that every thread has passed.
 template <int KEEP, typename Scan, typename Emit>
-__device__ __forceinline__ void nbest_core(Scan scan, int N, NbestShared& sh, Emit emit) {
+__device__ __forceinline__ void nbest_from_bound(Scan scan, int N, NbestShared& sh, Emit emit, float tv,
+                                                 bool count_is_zero) {
   const int tid = threadIdx.x;
   const float ninf = -__builtin_inff();
   const unsigned none = 0xFFFFFFFFu;
 
-  // 1. largest score of this thread, of its wave, and the N-th largest of the 16 wave maxima: the
-  //    bound T.  The maxima belong to 16 distinct elements and N <= 16, so at least N elements of the
-  //    row are >= T; for N = 16 and scores without structure some 50 are.
-  float mv = ninf;
-  scan([&](float v, unsigned) { mv = fmaxf(mv, v); });
-  float tv = ninf;   // (a wave without elements contributes -inf; with fewer than N waves that hold
-                     // elements the bound is -inf and everything passes)
-  {
-    float wv = mv;
-#pragma unroll
-    for(int o = 32; o > 0; o >>= 1) wv = fmaxf(wv, __shfl_xor(wv, o, 64));
-    if(tid % 64 == 0) sh.val[tid / 64] = wv;
-    __syncthreads();
-    // lane l % 16 ranks wave maximum l % 16 (equal values in wave order); the one of rank N - 1
-    // is the bound (the cost does not grow with N)
-    const int c = tid % 16;
-    const float cvv = sh.val[c];
-    int rank = 0;
-#pragma unroll
-    for(int w = 0; w < 16; ++w) rank += (sh.val[w] > cvv || (sh.val[w] == cvv && w < c)) ? 1 : 0;
-    const unsigned long long holders = __ballot(rank == N - 1) & 0xFFFFull;
-    tv = __shfl(cvv, __ffsll((long long)holders) - 1, 64);   // (ranks 0..15 are all taken: one holder)
-  }
-
   // 2. collect what is >= the bound
-  if(tid == 0) sh.count = 0;
-  __syncthreads();
+  if(!count_is_zero) {
+    if(tid == 0) sh.count = 0;
+    __syncthreads();
+  }
   scan([&](float v, unsigned i) {
     if(v >= tv) {
       const int slot = atomicAdd(&sh.count, 1);
@@ -931,6 +949,25 @@ __device__ __forceinline__ void nbest_core(Scan scan, int N, NbestShared& sh, Em
       idx[KEEP - 1] = none;
     }
   }
+}
+
+template <int KEEP, typename Scan, typename Emit>
+__device__ __forceinline__ void nbest_core(Scan scan, int N, NbestShared& sh, Emit emit) {
+  const int tid = threadIdx.x;
+  // 1. largest score of this thread, of its wave, and the N-th largest of the 16 wave maxima: the
+  //    bound T.  The maxima belong to 16 distinct elements and N <= 16, so at least N elements of the
+  //    row are >= T; for N = 16 and scores without structure some 50 are.  (A wave without elements
+  //    contributes -inf; with fewer than N waves that hold elements the bound is -inf and
+  //    everything passes.)
+  float mv = -__builtin_inff();
+  scan([&](float v, unsigned) { mv = fmaxf(mv, v); });
+  float wv = mv;
+#pragma unroll
+  for(int o = 32; o > 0; o >>= 1) wv = fmaxf(wv, __shfl_xor(wv, o, 64));
+  if(tid % 64 == 0) sh.val[tid / 64] = wv;
+  __syncthreads();
+  const float tv = nth_largest_of_16(sh.val, N);
+  nbest_from_bound<KEEP>(scan, N, sh, emit, tv, false);
 }
 
 // The row in memory.  (Every scan keeps eight 16-byte loads in flight per thread; the last round
@@ -1100,15 +1137,25 @@ __global__ __launch_bounds__(1024) void logsoftmax_nbest_kernel(const float* __r
                                                                 unsigned* __restrict__ outKeys) {
   __shared__ NbestShared sh;
   __shared__ int is_last;
-  __shared__ float red[16];
+  __shared__ float red[32];
   const int k = blockIdx.x, parts = gridDim.x, t = threadIdx.x;
   const long long b = blockIdx.y;
   const size_t row = (size_t)k * dimBatch + b;
   const int cols4 = vocab / 4;
   v4f v[VPT];
-  const float log_sum = softmax_wide_row<true, 1024, VPT>(reinterpret_cast<const v4f*>(in + row * vocab), nullptr,
-                                                          cols4, v, red);
+  if(t == 0) sh.count = 0;   // (the selection starts behind the barriers of the two reductions)
+  // The selection's bound comes out of the softmax's own maximum: the N-th largest of the 16 wave
+  // maxima of the logits (at least N logits reach it), taken through the same operations as every
+  // element below, which are monotonic, so at least N scores reach the result.
+  float bound_logit = -__builtin_inff(), row_max = 0.0f;
+  const float log_sum = softmax_wide_row<true, 1024, VPT>(
+      reinterpret_cast<const v4f*>(in + row * vocab), nullptr, cols4, v, red, [&](float mx, const float* wave_max) {
+        row_max = mx;
+        bound_logit = nth_largest_of_16(wave_max, N);
+      });
   const float add = rowAdd ? rowAdd[row] : 0.0f;
+  float tv = (bound_logit - row_max) - log_sum;
+  if(rowAdd) tv = tv + add;
 #pragma unroll
   for(int j = 0; j < VPT; ++j) {
     v[j] = v4f{v[j].x - log_sum, v[j].y - log_sum, v[j].z - log_sum, v[j].w - log_sum};
@@ -1128,11 +1175,10 @@ __global__ __launch_bounds__(1024) void logsoftmax_nbest_kernel(const float* __r
   float* cv = candVal + ((size_t)b * parts + k) * N;
   unsigned* ci = candIdx + ((size_t)b * parts + k) * N;
   const unsigned base = (unsigned)k * (unsigned)vocab;
-  __syncthreads();   // (red is done with; the selection has its own LDS)
-  nbest_core<KEEP>(scan, N, sh, [&](int r, float val, unsigned i) {
+  nbest_from_bound<KEEP>(scan, N, sh, [&](int r, float val, unsigned i) {
     __hip_atomic_store(cv + r, val, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __hip_atomic_store(ci + r, base + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  });
+  }, tv, true);
   nbest_hand_over(sh, &is_last, b, parts, N, (long long)parts * vocab, candVal, candIdx, counters, outScores, outKeys);
 }
 
