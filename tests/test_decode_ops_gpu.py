@@ -298,6 +298,34 @@ def test_absmax_outputs_of_layer_norm_and_attention(ops, integer, synth):
         assert np.array_equal(aq.numpy(), aq_ref.numpy()) and np.array_equal(got.cpu().numpy(), want.cpu().numpy())
 
 
+@pytest.mark.parametrize("beam,entries,L,masked,rows_per_mask", [(4, 512, 60, True, 16), (4, 512, 21, False, 1),
+                                                               (2, 48, 130, True, 16), (3, 16, 7, True, 1),
+                                                               (6, 32, 64, True, 16), (12, 8, 1, False, 1),
+                                                               (8, 5, 1024, True, 1)])
+def test_attention_rows_that_share_keys_and_values(ops, synth, beam, entries, L, masked, rows_per_mask):
+    """hypotheses of a sentence over the encoder's keys and values: the call that names the shared
+    cache once (batchKV = batchQ / beam, query row i reads entry i % batchKV) gives the bits of the
+    call on a cache that holds a copy per query row; the abs-max slots agree too"""
+    import torch
+    dk = 64
+    BQ = beam * entries
+    q = dev(synth.normal(BQ + L, 0, (BQ, 1, dk), 1.0))
+    k = dev(synth.normal(BQ + L, 1, (entries, L, dk), 1.0))
+    v = dev(synth.normal(BQ + L, 2, (entries, L, dk), 1.0))
+    mask = None
+    if masked:
+        n_masks = max(1, entries // rows_per_mask)
+        lens = 1 + (np.arange(n_masks) * 7) % L
+        mask = dev(((np.arange(L)[None, :] >= lens[:, None]) * -99999999.0).astype(np.float32))
+    got, gmax = ops.Attention(q, k, v, mask, rowsPerMask=rows_per_mask, want_absmax=BQ <= 2048) if BQ <= 2048 else \
+        (ops.Attention(q, k, v, mask, rowsPerMask=rows_per_mask), None)
+    want = ops.Attention(q, k.repeat(beam, 1, 1), v.repeat(beam, 1, 1), mask, rowsPerMask=rows_per_mask, want_absmax=BQ <= 2048)
+    if BQ <= 2048:
+        want, wmax = want
+        assert torch.equal(gmax.data, wmax.data)
+    assert torch.equal(got, want)
+
+
 @pytest.mark.parametrize("BQ,BKV,m,L,dk,masked", [(24, 24, 40, 40, 64, True), (16, 8, 9, 33, 32, False)])
 def test_attention_with_many_query_positions(ops, synth, BQ, BKV, m, L, dk, masked):
     """Encoder-size use (many query positions per head; the host mirror runs the three operators):
