@@ -595,6 +595,8 @@ __global__ __launch_bounds__(256) void attention_kernel(const float* __restrict_
         const int U = base / 4 + u;
         const float* p = U >= u_last ? last_c : first + (size_t)U * 4 * dk;
         r[u] = *reinterpret_cast<const v4f*>(p);
+      } else if(base + 4 * (u & ~3) < len) {   // (read with its group of sixteen positions below)
+        r[u] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
       }
     }
   };
@@ -605,17 +607,29 @@ __global__ __launch_bounds__(256) void attention_kernel(const float* __restrict_
     v4f kr[kAttU];
     load_rows(kb, k_last, 0, kr);
     load_rows(vb, v_last, 0, vr);
+    // (sixteen positions at a time without a branch between them: the four products and the four
+    // exchange steps of a group of four positions depend on one another, and only independent
+    // groups side by side keep the wave issuing; rows that were not loaded are zeros here and their
+    // results are dropped)
     for(int base = 0;;) {
 #pragma unroll
-      for(int u = 0; u < kAttU; ++u) {
-        if(base + 4 * u < len) {
-          const int pos = base + 4 * u + g;
-          float s = q4.x * kr[u].x;
-          s = fmaf(q4.y, kr[u].y, s);
-          s = fmaf(q4.z, kr[u].z, s);
-          s = fmaf(q4.w, kr[u].w, s);
-          s = row16_sum(s);
-          if(c == 0 && pos < len) sc[pos] = scale * s;
+      for(int u0 = 0; u0 < kAttU; u0 += 4) {
+        if(base + 4 * u0 < len) {
+          float s[4];
+#pragma unroll
+          for(int u = u0; u < u0 + 4; ++u) {
+            float t = q4.x * kr[u].x;
+            t = fmaf(q4.y, kr[u].y, t);
+            t = fmaf(q4.z, kr[u].z, t);
+            s[u - u0] = fmaf(q4.w, kr[u].w, t);
+          }
+#pragma unroll
+          for(int u = 0; u < 4; ++u) s[u] = row16_sum(s[u]);
+#pragma unroll
+          for(int u = u0; u < u0 + 4; ++u) {
+            const int pos = base + 4 * u + g;
+            if(c == 0 && pos < len) sc[pos] = scale * s[u - u0];
+          }
         }
       }
       base += 4 * kAttU;
@@ -682,14 +696,21 @@ __global__ __launch_bounds__(256) void attention_kernel(const float* __restrict_
     for(int base = 0; base < len; base += 4 * kAttU) {
       if(base > 0) load_rows(vb, v_last, base, vr);
 #pragma unroll
-      for(int u = 0; u < kAttU; ++u) {
-        if(base + 4 * u < len) {
-          const int pos = base + 4 * u + g;
-          const float w = pos < len ? sc[pos] : 0.0f;
-          o4.x = fmaf(w, vr[u].x, o4.x);
-          o4.y = fmaf(w, vr[u].y, o4.y);
-          o4.z = fmaf(w, vr[u].z, o4.z);
-          o4.w = fmaf(w, vr[u].w, o4.w);
+      for(int u0 = 0; u0 < kAttU; u0 += 4) {
+        if(base + 4 * u0 < len) {
+          // the four weights first (reads inside this wave's score area: a position past the row
+          // reads a stale value there, which is replaced by zero)
+          float w[4];
+#pragma unroll
+          for(int u = u0; u < u0 + 4; ++u) w[u - u0] = sc[min(base + 4 * u + g, len4 + 255)];
+#pragma unroll
+          for(int u = u0; u < u0 + 4; ++u) {
+            const float wu = base + 4 * u + g < len ? w[u - u0] : 0.0f;
+            o4.x = fmaf(wu, vr[u].x, o4.x);
+            o4.y = fmaf(wu, vr[u].y, o4.y);
+            o4.z = fmaf(wu, vr[u].z, o4.z);
+            o4.w = fmaf(wu, vr[u].w, o4.w);
+          }
         }
       }
     }
