@@ -38,12 +38,16 @@ __device__ __forceinline__ float row16_sum(float v) {
   v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xF, 0xF, false));  // row_mirror
   return v;
 }
+// Maximum over the wave, left in all lanes (NaN operands are passed over, as by `t > v ? t : v`):
+// the same four DPP steps within rows of 16 lanes, then the two exchanges across the four rows.
 __device__ __forceinline__ float wave_maxf(float v) {
-#pragma unroll
-  for(int o = 32; o > 0; o >>= 1) {
-    const float t = __shfl_xor(v, o, 64);
-    v = t > v ? t : v;
-  }
+  auto pick = [](float t, float v) { return t > v ? t : v; };
+  v = pick(__builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, false)), v);
+  v = pick(__builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, false)), v);
+  v = pick(__builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xF, 0xF, false)), v);
+  v = pick(__builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xF, 0xF, false)), v);
+  v = pick(__shfl_xor(v, 16, 64), v);
+  v = pick(__shfl_xor(v, 32, 64), v);
   return v;
 }
 
@@ -688,7 +692,10 @@ __global__ __launch_bounds__(256) void attention_kernel(const float* __restrict_
     if(pos == lane) e_first = e;
     sum += e;
   }
-  sum = wave_sum(sum);
+  // (the usual head size adds the lanes up within rows of 16 first, four DPP steps and two lane
+  // exchanges instead of six exchanges; the other sizes keep softmax_kernel's order, whose bits
+  // they reproduce)
+  sum = fast ? wave_sum16(sum) : wave_sum(sum);
   for(int pos = lane; pos < len; pos += 64) sc[pos] = (pos == lane ? e_first : expf(sc[pos] - mx)) / sum;
   // (a wave's LDS writes are visible to its own later reads: same wave, program order)
   if(fast) {

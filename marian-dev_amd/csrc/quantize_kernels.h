@@ -80,13 +80,28 @@ __device__ __forceinline__ float abs4max(v4f x, float m) {
   return m;
 }
 
+// Max over each row of 16 lanes, left in all 16 of them: four DPP steps (the two lane swaps within
+// a quad, the mirror within half a row and within the row).  All lanes of the wave must be active.
+// (fmaxf passes over NaN operands whatever the order, so the result does not depend on the order.)
+__device__ __forceinline__ float row16_max(float m) {
+  m = fmaxf(m, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, m), 0xB1, 0xF, 0xF, false)));   // quad_perm [1,0,3,2]
+  m = fmaxf(m, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, m), 0x4E, 0xF, 0xF, false)));   // quad_perm [2,3,0,1]
+  m = fmaxf(m, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, m), 0x141, 0xF, 0xF, false)));  // row_half_mirror
+  m = fmaxf(m, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, m), 0x140, 0xF, 0xF, false)));  // row_mirror
+  return m;
+}
+// Max over the wave, in all lanes: within the rows, then two lane exchanges across the four rows
+// (an exchange goes through the LDS crossbar and costs ten times a DPP step; these reductions sit
+// between the arrival of the activations and their quantization in every fused call).
 __device__ __forceinline__ float wave_max(float m) {
-#pragma unroll
-  for(int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+  m = row16_max(m);
+  m = fmaxf(m, __shfl_xor(m, 16, 64));
+  m = fmaxf(m, __shfl_xor(m, 32, 64));
   return m;
 }
 
-// Max over the workgroup; every thread returns the result.  red: >= blockDim/64 floats of LDS.
+// Max over the workgroup (whole waves, at most 16 of them); every thread returns the result.
+// red: >= blockDim/64 floats of LDS.
 __device__ __forceinline__ float block_max(float m, float* red) {
   m = wave_max(m);
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
@@ -94,8 +109,9 @@ __device__ __forceinline__ float block_max(float m, float* red) {
   __syncthreads();
   if(lane == 0) red[wave] = m;
   __syncthreads();
-  float r = (lane < nw) ? red[lane] : 0.0f;
-  return wave_max(r);
+  // every row of 16 lanes reads all the wave maxima, so the rows need no exchange afterwards
+  const float r = (lane % 16 < nw) ? red[lane % 16] : 0.0f;
+  return row16_max(r);
 }
 
 // quantMult = 127.0f / maxabs as one correctly rounded fp32 division (via double).
