@@ -216,8 +216,24 @@ __global__ __launch_bounds__(WN * KW * kWave) void gemm_stream32_kernel(GemmArgs
     }
   }
 
+  // Where the quad's first group lies (two integer divisions: worked out here, while the loads
+  // are in flight, not behind the abs-max where the quantization waits for them).
+  const unsigned k16n = K / 16;   // 16-byte chunks per activation row (a multiple of four)
+  unsigned row = 0, c16 = 0, drow = 0, dc16 = 0;
+  if(FUSED) {
+    row = 4 * quad / k16n;
+    c16 = 4 * quad % k16n;
+    drow = kStream32Threads / k16n;
+    dc16 = kStream32Threads % k16n;
+    asm volatile("" : "+v"(row), "+v"(c16));
+  }
+
   float aqm = 0.0f;        // quantMult of the activations (fused modes)
   bool finite_t = false;   // kFusedTiled: the quantMult is finite
+  // The multiplier of the epilogue (a division through double precision) is worked out as soon as
+  // the quantMult of the activations is known, under the matrix instructions.
+  float unquant = 0.0f;
+  if(MODE == kPrequant) unquant = unquant_mult(aqm_pre, bqm, args.scale);
   // Otherwise a chunk of activations is fetched into registers (all loads in flight at once) and
   // then dropped into LDS, so the fetch of chunk c+1 overlaps the multiplication of chunk c.
   // Pre-quantized: thread slot (sub-step, m-tile, lane) in operand order.  kFusedTiled: fp32
@@ -325,6 +341,7 @@ __global__ __launch_bounds__(WN * KW * kWave) void gemm_stream32_kernel(GemmArgs
   if(TILED) {
     amax = block_max(amax, red);
     aqm = quant_mult_from_maxabs(amax);
+    unquant = unquant_mult(aqm, bqm, args.scale);
     finite_t = aqm < __builtin_inff();   // (see the fused form below)
     if(MH_PROF(args)) tp[1] = MH_CLOCK();
     if(aq_out && blockIdx.x == 0 && blockIdx.y == 0 && tid == 0)
@@ -345,14 +362,12 @@ __global__ __launch_bounds__(WN * KW * kWave) void gemm_stream32_kernel(GemmArgs
     amax = block_max(amax, red);
     if(MH_PROF(args)) tp[1] = MH_CLOCK();
     aqm = quant_mult_from_maxabs(amax);
+    unquant = unquant_mult(aqm, bqm, args.scale);
     // With a finite quantMult no product can leave [-127.0001, 127.0001]: finite values are at
     // most the abs-max in magnitude, and an infinite value makes the quantMult 0 and its product
     // NaN.  (An abs-max of zero, or one below 127 / FLT_MAX, gives an infinite quantMult, and then
     // infinite products, which the conversion of the CPU path turns into -127, not +127.)
     const bool finite = aqm < __builtin_inff();
-    const unsigned k16n = K / 16;   // 16-byte chunks per activation row (a multiple of four)
-    unsigned row = 4 * quad / k16n, c16 = 4 * quad % k16n;   // of the quad's first group
-    const unsigned drow = kStream32Threads / k16n, dc16 = kStream32Threads % k16n;
     uint32_t q[kFusedGroups][4];
 #pragma unroll
     for(int j = 0; j < kFusedGroups; ++j) {
@@ -482,7 +497,6 @@ __global__ __launch_bounds__(WN * KW * kWave) void gemm_stream32_kernel(GemmArgs
   float omax = 0.0f;   // max |y| over what this wave stores
   {
     constexpr int kPieces = R * 8 / KW;        // 16-byte pieces this wave finishes (32 .. 1024)
-    const float unquant = unquant_mult(MODE == kPrequant ? aqm_pre : aqm, bqm, args.scale);
     const bool has_bias = args.bias != nullptr;
     const int n = n0 + 4 * (lane % 8);
     const int8_t* tiles = lds + (size_t)(wn * KW) * kTileBytes;
