@@ -24,11 +24,6 @@ namespace {
 
 constexpr int64_t kMaxElemsOps = 2147483647LL;
 
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for(int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
-  return v;
-}
 // Sum over each group of 16 consecutive lanes, left in all 16 of them (four DPP steps: the two
 // lane swaps within a quad, then the mirror within half a row and within the row).
 __device__ __forceinline__ float row16_sum(float v) {
@@ -36,6 +31,14 @@ __device__ __forceinline__ float row16_sum(float v) {
   v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, false));   // quad_perm [2,3,0,1]
   v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xF, 0xF, false));  // row_half_mirror
   v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xF, 0xF, false));  // row_mirror
+  return v;
+}
+// Sum over the wave, left in all lanes: within the rows of 16 lanes by DPP, then two lane exchanges
+// across the four rows (an exchange goes through the LDS crossbar and costs ten times a DPP step).
+__device__ __forceinline__ float wave_sum(float v) {
+  v = row16_sum(v);
+  v += __shfl_xor(v, 16, 64);
+  v += __shfl_xor(v, 32, 64);
   return v;
 }
 // Maximum over the wave, left in all lanes (NaN operands are passed over, as by `t > v ? t : v`):
@@ -183,12 +186,6 @@ __global__ __launch_bounds__(256) void layer_norm_kernel(const float* in,
 // Rows of up to 1024 values: one wave per row and one row per workgroup, four float4 per lane.  The three reductions stay inside the wave, so the kernel has
 // no workgroup barrier and no LDS traffic between its load and its store; scale and shift come as
 // 16-byte loads (gamma_stride / beta_stride 1, 16-byte aligned) or as one broadcast value (0).
-__device__ __forceinline__ float wave_sum16(float v) {   // DPP within rows of 16 lanes, then across the four rows
-  v = row16_sum(v);
-  v += __shfl_xor(v, 16, 64);
-  v += __shfl_xor(v, 32, 64);
-  return v;
-}
 __global__ __launch_bounds__(64) void layer_norm_wave_kernel(const float* in, const float* __restrict__ add,
                                                              const float* __restrict__ gamma, int gamma_stride,
                                                              const float* __restrict__ beta, int beta_stride,
@@ -227,7 +224,7 @@ __global__ __launch_bounds__(64) void layer_norm_wave_kernel(const float* in, co
     if(a) v[j] = v4f{v[j].x + t[j].x, v[j].y + t[j].y, v[j].z + t[j].z, v[j].w + t[j].w};
     if(j * 64 + lane < cols4) sum += (v[j].x + v[j].y) + (v[j].z + v[j].w);
   }
-  const float mean = wave_sum16(sum) / (float)cols;
+  const float mean = wave_sum(sum) / (float)cols;
   float sq = 0.0f;
 #pragma unroll
   for(int j = 0; j < VPL; ++j) {
@@ -236,7 +233,7 @@ __global__ __launch_bounds__(64) void layer_norm_wave_kernel(const float* in, co
       sq += (d0 * d0 + d1 * d1) + (d2 * d2 + d3 * d3);
     }
   }
-  const float sigma = sqrtf(wave_sum16(sq) / (float)cols + eps);
+  const float sigma = sqrtf(wave_sum(sq) / (float)cols + eps);
   float omax = 0.0f;
 #pragma unroll
   for(int j = 0; j < VPL; ++j) {
@@ -692,10 +689,7 @@ __global__ __launch_bounds__(256) void attention_kernel(const float* __restrict_
     if(pos == lane) e_first = e;
     sum += e;
   }
-  // (the usual head size adds the lanes up within rows of 16 first, four DPP steps and two lane
-  // exchanges instead of six exchanges; the other sizes keep softmax_kernel's order, whose bits
-  // they reproduce)
-  sum = fast ? wave_sum16(sum) : wave_sum(sum);
+  sum = wave_sum(sum);
   for(int pos = lane; pos < len; pos += 64) sc[pos] = (pos == lane ? e_first : expf(sc[pos] - mx)) / sum;
   // (a wave's LDS writes are visible to its own later reads: same wave, program order)
   if(fast) {
@@ -989,9 +983,7 @@ __device__ __forceinline__ void nbest_core(Scan scan, int N, NbestShared& sh, Em
   //    everything passes.)
   float mv = -__builtin_inff();
   scan([&](float v, unsigned) { mv = fmaxf(mv, v); });
-  float wv = mv;
-#pragma unroll
-  for(int o = 32; o > 0; o >>= 1) wv = fmaxf(wv, __shfl_xor(wv, o, 64));
+  const float wv = wave_maxf(mv);
   if(tid % 64 == 0) sh.val[tid / 64] = wv;
   __syncthreads();
   const float tv = nth_largest_of_16(sh.val, N);
