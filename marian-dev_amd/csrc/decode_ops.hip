@@ -33,25 +33,28 @@ __device__ __forceinline__ float row16_sum(float v) {
   v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xF, 0xF, false));  // row_mirror
   return v;
 }
-// Sum over the wave, left in all lanes: within the rows of 16 lanes by DPP, then two lane exchanges
-// across the four rows (an exchange goes through the LDS crossbar and costs ten times a DPP step).
+// Sum over the wave, the same value in all lanes: within the rows of 16 lanes, then across them
+// with the two row-broadcast DPP steps (rows 1 and 3 take in the last lane of the row before them,
+// then rows 2 and 3 the last lane of row 1), which leaves the total in lane 63, read from there as
+// a scalar.  No step goes through the LDS crossbar (a lane exchange there costs ten times a DPP
+// step).  All lanes of the wave must be active.
 __device__ __forceinline__ float wave_sum(float v) {
   v = row16_sum(v);
-  v += __shfl_xor(v, 16, 64);
-  v += __shfl_xor(v, 32, 64);
-  return v;
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x142, 0xA, 0xF, false));   // row_bcast:15
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x143, 0xC, 0xF, false));   // row_bcast:31
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
 }
-// Maximum over the wave, left in all lanes (NaN operands are passed over, as by `t > v ? t : v`):
-// the same four DPP steps within rows of 16 lanes, then the two exchanges across the four rows.
+// Maximum over the wave, the same value in all lanes (`t > v ? t : v` at every step): the same
+// steps.
 __device__ __forceinline__ float wave_maxf(float v) {
   auto pick = [](float t, float v) { return t > v ? t : v; };
   v = pick(__builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, false)), v);
   v = pick(__builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, false)), v);
   v = pick(__builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xF, 0xF, false)), v);
   v = pick(__builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xF, 0xF, false)), v);
-  v = pick(__shfl_xor(v, 16, 64), v);
-  v = pick(__shfl_xor(v, 32, 64), v);
-  return v;
+  v = pick(__builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, v), __builtin_bit_cast(int, v), 0x142, 0xA, 0xF, false)), v);   // row_bcast:15
+  v = pick(__builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, v), __builtin_bit_cast(int, v), 0x143, 0xC, 0xF, false)), v);   // row_bcast:31
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
 }
 
 // Reduction over the THREADS threads that share a row (64: one wave, no LDS; more: through LDS).

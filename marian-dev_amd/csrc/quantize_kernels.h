@@ -90,14 +90,17 @@ __device__ __forceinline__ float row16_max(float m) {
   m = fmaxf(m, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, m), 0x140, 0xF, 0xF, false)));  // row_mirror
   return m;
 }
-// Max over the wave, in all lanes: within the rows, then two lane exchanges across the four rows
-// (an exchange goes through the LDS crossbar and costs ten times a DPP step; these reductions sit
-// between the arrival of the activations and their quantization in every fused call).
+// Max over the wave, in all lanes: within the rows, then across them with the two row-broadcast
+// DPP steps (rows 1 and 3 take in the last lane of the row before them, then rows 2 and 3 the last
+// lane of row 1), which leaves the result in lane 63, read from there as a scalar.  No step goes
+// through the LDS crossbar (a lane exchange there costs ten times a DPP step, and these reductions
+// sit between the arrival of the activations and their quantization in every fused call).  All
+// lanes of the wave must be active.
 __device__ __forceinline__ float wave_max(float m) {
   m = row16_max(m);
-  m = fmaxf(m, __shfl_xor(m, 16, 64));
-  m = fmaxf(m, __shfl_xor(m, 32, 64));
-  return m;
+  m = fmaxf(m, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, m), __builtin_bit_cast(int, m), 0x142, 0xA, 0xF, false)));   // row_bcast:15
+  m = fmaxf(m, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, m), __builtin_bit_cast(int, m), 0x143, 0xC, 0xF, false)));   // row_bcast:31
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, m), 63));
 }
 
 // Max over the workgroup (whole waves, at most 16 of them); every thread returns the result.
