@@ -97,6 +97,21 @@ int marian_hip_attention(const float* q, float* k, float* v, const float* mask, 
                          const float* k_new, const float* v_new, void* stream);
 
 /*
+ * marian_hip_attention on caches that have room to grow: k and v are [batchKV, kv_capacity, dk]
+ * with the first len positions of every entry in use (kv_capacity >= len; the mask still has len
+ * values per row).  The decoder state of a translation then stays where it is from step to step:
+ * the reference concatenates the new position onto the cached ones into a fresh tensor every
+ * step (src/models/transformer.h:409-416), here a step passes len = positions so far + 1 with k_new,
+ * v_new, which the call stores at position len - 1, and the selection of the surviving
+ * hypotheses between two steps (src/rnn/types.h:22-42) is rows() over entries of kv_capacity * dk
+ * values.  marian_hip_attention is this call with kv_capacity = len.
+ */
+int marian_hip_attention_cached(const float* q, float* k, float* v, const float* mask, int64_t n_masks,
+                                int64_t rows_per_mask, float* out, int64_t batchQ, int64_t batchKV,
+                                int64_t m, int64_t len, int64_t kv_capacity, int64_t dk, float scale,
+                                float* absmax_out, const float* k_new, const float* v_new, void* stream);
+
+/*
  * The embedding step in front of the first layer, reference src/layers/embedding.cpp:161-168
  * (rows(E, ids): CopyRows, src/tensors/cpu/tensor_operators.cpp:577-603), followed by
  * src/models/transformer.h:93 (sqrt(dimEmb) * embeddings) and :117 (embeddings + signal, the

@@ -61,6 +61,8 @@ SIGNATURES = {
     "marian_hip_fill": (_i, [_vp, _i64, _i, _c.c_uint64, _vp]),
     "marian_hip_attention": (_i, [_vp, _vp, _vp, _vp, _i64, _i64, _vp, _i64, _i64, _i64, _i64, _i64,
                                   _f, _vp, _vp, _vp, _vp]),
+    "marian_hip_attention_cached": (_i, [_vp, _vp, _vp, _vp, _i64, _i64, _vp, _i64, _i64, _i64, _i64, _i64, _i64,
+                                         _f, _vp, _vp, _vp, _vp]),
 }
 
 # include/marian_hip_int8_tuning.h (tuning build only)

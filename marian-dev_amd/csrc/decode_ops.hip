@@ -524,8 +524,9 @@ __global__ __launch_bounds__(256) void attention_kernel(const float* __restrict_
                                                         const float* __restrict__ mask,
                                                         unsigned n_masks, unsigned rows_per_mask,
                                                         float* __restrict__ out, unsigned rows_total,
-                                                        unsigned batchKV, int m, int len, int dk,
+                                                        unsigned batchKV, int m, int len, int kv_cap, int dk,
                                                         float scale, float* __restrict__ absmax_out) {
+  // kv_cap: positions a cache entry has room for (its stride, in rows of dk values); len of them are in use
   // (row counts are below 2^31, checked by the launcher: 32-bit divisions, a tenth of the
   // instructions of 64-bit ones, and this kernel is a chain of short phases)
   extern __shared__ __attribute__((aligned(16))) float att_lds[];
@@ -543,8 +544,8 @@ __global__ __launch_bounds__(256) void attention_kernel(const float* __restrict_
   const unsigned i = m == 1 ? wr : wr / (unsigned)m;
   const unsigned entry = i < batchKV ? i : i % batchKV;
   const float* q = Q + (size_t)wr * dk;
-  float* kb = Kt + (size_t)entry * len * dk;
-  float* vb = V + (size_t)entry * len * dk;
+  float* kb = Kt + (size_t)entry * kv_cap * dk;
+  float* vb = V + (size_t)entry * kv_cap * dk;
   // Newest position (m == 1, one wave per cache entry): its key and value rows go into the cache
   // for the following steps; this step reads them from k_new / v_new directly.  Up to 64 values per
   // row they are requested here and stored at the end of the kernel (nothing in this call waits
@@ -1479,7 +1480,16 @@ int marian_hip_attention(const float* q, float* k, float* v, const float* mask, 
                          int64_t rows_per_mask, float* out, int64_t batchQ, int64_t batchKV,
                          int64_t m, int64_t len, int64_t dk, float scale, float* absmax_out,
                          const float* k_new, const float* v_new, void* stream) {
+  return marian_hip_attention_cached(q, k, v, mask, n_masks, rows_per_mask, out, batchQ, batchKV, m, len, len, dk,
+                                     scale, absmax_out, k_new, v_new, stream);
+}
+
+int marian_hip_attention_cached(const float* q, float* k, float* v, const float* mask, int64_t n_masks,
+                                int64_t rows_per_mask, float* out, int64_t batchQ, int64_t batchKV,
+                                int64_t m, int64_t len, int64_t kv_capacity, int64_t dk, float scale,
+                                float* absmax_out, const float* k_new, const float* v_new, void* stream) {
   if((k_new != nullptr) != (v_new != nullptr)) return MARIAN_HIP_ERR_NULL;
+  if(kv_capacity < len) return MARIAN_HIP_ERR_SHAPE;
   if(k_new && (m != 1 || batchKV != batchQ)) return MARIAN_HIP_ERR_SHAPE;
   if(k_new && (!aligned4(k_new) || !aligned4(v_new))) return MARIAN_HIP_ERR_ALIGN;
   if(absmax_out && batchQ * m > kAbsmaxSlots) return MARIAN_HIP_ERR_RANGE;
@@ -1490,7 +1500,8 @@ int marian_hip_attention(const float* q, float* k, float* v, const float* mask, 
   if(len > 4096) return MARIAN_HIP_ERR_RANGE;
   if(batchQ == 0) return MARIAN_HIP_OK;
   if(!q || !k || !v || !out) return MARIAN_HIP_ERR_NULL;
-  if(batchQ * m * dk > kMaxElemsOps || batchKV * len * dk > kMaxElemsOps) return MARIAN_HIP_ERR_RANGE;
+  if(kv_capacity > kMaxElemsOps || batchQ * m * dk > kMaxElemsOps || batchKV * kv_capacity * dk > kMaxElemsOps)
+    return MARIAN_HIP_ERR_RANGE;
   if(!aligned4(q) || !aligned4(k) || !aligned4(v) || !aligned4(out) || (mask && !aligned4(mask)))
     return MARIAN_HIP_ERR_ALIGN;
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
@@ -1510,7 +1521,7 @@ int marian_hip_attention(const float* q, float* k, float* v, const float* mask, 
   }
   hipLaunchKernelGGL(attention_kernel, dim3((unsigned)((rows_total + 3) / 4)), dim3(256), lds, st, q, k, v,
                      k_new, v_new, mask, (unsigned)n_masks, (unsigned)rows_per_mask, out, (unsigned)rows_total,
-                     (unsigned)batchKV, (int)m, (int)len, (int)dk, scale, absmax_out);
+                     (unsigned)batchKV, (int)m, (int)len, (int)kv_capacity, (int)dk, scale, absmax_out);
   MH_HIP(hipGetLastError());
   return MARIAN_HIP_OK;
 }

@@ -24,12 +24,14 @@ class DecoderStep:
     Beam search's hypothesis bookkeeping is not part of the step."""
 
     def __init__(self, sets=1, d=1024, ffn=4096, heads=16, vocab=32000, layers=6, beam=4, batch=32,
-                 t_past=20, src_len=60, min_src_len=20, seed=300):
+                 t_past=20, src_len=60, min_src_len=20, seed=300, t_capacity=None):
         self.torch, self.integer, self.ops = torch, integer, ops
         self.d, self.ffn, self.V, self.H = d, ffn, vocab, heads
         self.beam, self.batch, self.layers = beam, batch, layers
         self.M = self.beam * self.batch
-        self.T, self.L = t_past + 1, src_len
+        self.T, self.L = t_past + 1, src_len   # T: cached positions in use, the step's new one included
+        self.cap = self.T if t_capacity is None else int(t_capacity)   # positions the caches have room for
+        assert self.cap >= self.T
         self.trace = None   # a list: every operator call of step() is recorded into it (tests)
         g = torch.Generator(device="cuda")
         g.manual_seed(seed)
@@ -69,18 +71,16 @@ class DecoderStep:
         self.signal = ops.sinusoidalPositionEmbeddings(1, d, t_past, device="cuda")
         self.emb_scale = float(torch.sqrt(torch.tensor(float(d))))
         self.x = torch.randn(M, d, device="cuda", generator=g)   # (input of the GEMM-only chain)
-        # the self-attention caches of all layers are rows of one tensor [2 * layers * M, H * T * dk] (a
+        # the self-attention caches of all layers are rows of one tensor [2 * layers * M, H * cap * dk] (a
         # hypothesis's cached positions of one layer are one row), so that the beam search's selection
         # of the surviving hypotheses is one gather; a second tensor of that size receives it
-        self.state = torch.randn(2 * layers * M, H * self.T * (d // H), device="cuda", generator=g)
+        self.state = torch.randn(2 * layers * M, H * self.cap * (d // H), device="cuda", generator=g)
         self.state_next = torch.empty_like(self.state)
         self._cache_views()
         # back-pointers of a beam-search step: hypothesis (k, b) continues hypothesis (k', b) of the
         # same sentence; flat index k * batch + b, one copy per cache tensor
         parent = torch.randint(0, beam, (beam, batch), device="cuda", generator=g) * batch + torch.arange(batch, device="cuda")
-        self.hyp_indices = parent.reshape(-1).to(torch.int32)
-        self.state_rows = (torch.arange(2 * layers, device="cuda", dtype=torch.int32)[:, None] * M +
-                           self.hyp_indices[None, :]).reshape(-1).contiguous()
+        self.set_hypotheses(parent.reshape(-1))
         self.Kenc = [torch.randn(self.batch * H, self.L, d // H, device="cuda", generator=g) for _ in range(layers)]
         self.Venc = [torch.randn(self.batch * H, self.L, d // H, device="cuda", generator=g) for _ in range(layers)]
         # source lengths uniform over min_src_len .. src_len, padded to the longest (the mask covers the rest)
@@ -89,9 +89,25 @@ class DecoderStep:
         self.mask = (torch.arange(self.L, device="cuda")[None, :] >= lens[:, None]).float() * -99999999.0
 
     def _cache_views(self):
-        M, H, T, dk, layers = self.M, self.H, self.T, self.d // self.H, self.layers
-        self.Kself = [self.state[l * M:(l + 1) * M].view(M * H, T, dk) for l in range(layers)]
-        self.Vself = [self.state[(layers + l) * M:(layers + l + 1) * M].view(M * H, T, dk) for l in range(layers)]
+        M, H, cap, dk, layers = self.M, self.H, self.cap, self.d // self.H, self.layers
+        self.Kself = [self.state[l * M:(l + 1) * M].view(M * H, cap, dk) for l in range(layers)]
+        self.Vself = [self.state[(layers + l) * M:(layers + l + 1) * M].view(M * H, cap, dk) for l in range(layers)]
+
+    def set_hypotheses(self, hyp_indices):
+        """back-pointers of the next step: hypothesis i continues hypothesis hyp_indices[i] (flat
+        index beam entry * batch + sentence), one copy per cache tensor for the gather"""
+        self.hyp_indices = hyp_indices.to(device="cuda", dtype=torch.int32).contiguous()
+        self.state_rows = (torch.arange(2 * self.layers, device="cuda", dtype=torch.int32)[:, None] * self.M +
+                           self.hyp_indices[None, :]).reshape(-1).contiguous()
+
+    def advance(self, words, hyp_indices):
+        """The next target position: the words the beam search chose, the hypotheses they continue
+        (step(select=True) then gathers their caches), one more cached position in use."""
+        assert self.T < self.cap, "the caches are full"
+        self.words = words.to(device="cuda", dtype=torch.int32).contiguous()
+        self.set_hypotheses(hyp_indices)
+        self.T += 1
+        self.signal = self.ops.sinusoidalPositionEmbeddings(1, self.d, self.T - 1, device="cuda")
 
     def select_states(self):
         """The decoder state of the surviving hypotheses (reference src/models/states.h:87-107,
@@ -129,7 +145,7 @@ class DecoderStep:
             x = ops.scaledEmbeddings(self.E, self.words, self.emb_scale, self.signal, M, want_absmax=ch)
             if ch:
                 x, xmax = x
-            rec("embed", E=self.E, ids=self.words, scale=self.emb_scale, signal=self.signal, out=x)
+            rec("embed", E=self.E, ids=self.words, scale=self.emb_scale, signal=self.signal, out=x, position=self.T - 1)
         for li, ly in enumerate(W["layers"]):
             if grouped:   # one abs-max, one quantization, one launch for the three projections
                 (q, k, v), _ = integer.affine_f32_grouped(x, [ly["Wq"], ly["Wk"], ly["Wv"]], absmax=xmax)
@@ -148,12 +164,12 @@ class DecoderStep:
                 if tr is not None:
                     k_before, v_before = self.Kself[li].clone(), self.Vself[li].clone()
                 o = ops.Attention(q.view(M * H, 1, dk), self.Kself[li], self.Vself[li], want_absmax=ch,
-                                  kNew=k.view(M * H, dk), vNew=v.view(M * H, dk))
+                                  kNew=k.view(M * H, dk), vNew=v.view(M * H, dk), kvLen=self.T)
                 if ch:
                     o, omax = o
                 if tr is not None:
                     rec("self_attention", q=q, k_new=k, v_new=v, k_cache=k_before, v_cache=v_before,
-                        k_after=self.Kself[li], v_after=self.Vself[li], out=o)
+                        k_after=self.Kself[li], v_after=self.Vself[li], out=o, len=self.T)
                 o = o.view(M, d)
             a, _ = integer.affine_f32(o, *ly["Wo"], absmax=omax)
             rec("affine", a=o, w=ly["Wo"], out=a, relu=False)

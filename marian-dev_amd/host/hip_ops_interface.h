@@ -88,16 +88,17 @@ inline void ProdBatchedLegacy(Backend& be, Tensor& C, const Tensor& A, const Ten
                                           transB ? 1 : 0, scalar, be.stream()));
 }
 
-// q [batchQ, m, dk]; k, v [batchKV, len, dk]; out [batchQ, m, dk].  kNew / vNew [batchQ, dk]: the
-// newest position of a decoding step, appended to k and v by the call.
+// q [batchQ, m, dk]; k, v [batchKV, positions, dk]; out [batchQ, m, dk].  kNew / vNew [batchQ, dk]:
+// the newest position of a decoding step, appended to k and v by the call.  kvLen: the first kvLen
+// of the cache's positions are in use (caches that stay in place from step to step); 0: all.
 inline void Attention(Backend& be, Tensor& out, const Tensor& q, Tensor& k, Tensor& v, float scale,
                       const Tensor* mask = nullptr, int64_t rowsPerMask = 1, Tensor* absmaxOut = nullptr,
-                      const Tensor* kNew = nullptr, const Tensor* vNew = nullptr) {
+                      const Tensor* kNew = nullptr, const Tensor* vNew = nullptr, int64_t kvLen = 0) {
   if(q.shape.size() != 3 || k.shape.size() != 3) abortWith("Attention expects [batch, positions, dk] tensors");
-  MARIAN_HIP_CHECK(marian_hip_attention(
+  MARIAN_HIP_CHECK(marian_hip_attention_cached(
       q.data<float>(), k.data<float>(), v.data<float>(), mask ? mask->data<float>() : nullptr,
       mask ? (int64_t)rows(*mask) : 0, rowsPerMask, out.data<float>(), q.shape[0], k.shape[0], q.shape[1],
-      k.shape[1], q.shape[2], scale, absmaxOut ? absmaxOut->data<float>() : nullptr,
+      kvLen ? kvLen : k.shape[1], k.shape[1], q.shape[2], scale, absmaxOut ? absmaxOut->data<float>() : nullptr,
       kNew ? kNew->data<float>() : nullptr, vNew ? vNew->data<float>() : nullptr, be.stream()));
 }
 

@@ -183,13 +183,15 @@ def bdot_legacy(a, b, transA=False, transB=False, scalar=1.0):
     return out
 
 
-def Attention(q, k, v, mask=None, rowsPerMask=1, want_absmax=False, kNew=None, vNew=None):
+def Attention(q, k, v, mask=None, rowsPerMask=1, want_absmax=False, kNew=None, vNew=None, kvLen=None):
     """reference src/models/transformer.h:241-280 (inference: no dropout, weights not kept):
     softmax(bdot_legacy(q, k, false, true, 1/sqrt(dk)) + mask) then bdot_legacy(weights, v), in
     one launch.  q: [batch*beam, heads, tgt, dk]; k, v: [batch(*beam), heads, len, dk].
     kNew, vNew [batch*beam*heads, dk]: key and value of the newest position of a decoding step;
     they stand for position len - 1 and are also stored there in k and v (the concatenation onto
-    the cached positions, src/models/transformer.h:683-700)."""
+    the cached positions, src/models/transformer.h:683-700).
+    kvLen: k and v have room for k.shape[-2] positions per entry, of which the first kvLen are in
+    use (caches that stay in place from step to step); None: all of them."""
     q = _f32c(q, "Attention")
     _abort_if(k.dtype != torch.float32 or v.dtype != torch.float32, "Attention expects float32, got {}", k.dtype)
     if kNew is None:
@@ -198,12 +200,14 @@ def Attention(q, k, v, mask=None, rowsPerMask=1, want_absmax=False, kNew=None, v
         _abort_if(not (k.is_contiguous() and v.is_contiguous()), "Attention: the key/value cache must be contiguous{}", "")
         kNew, vNew = _f32c(kNew, "Attention"), _f32c(vNew, "Attention")
     be = _backend_of(q)
-    dk, m, L = q.shape[-1], q.shape[-2], k.shape[-2]
+    dk, m, cap = q.shape[-1], q.shape[-2], k.shape[-2]
+    L = cap if kvLen is None else int(kvLen)
+    _abort_if(not 0 < L <= cap, "Attention: {} positions in use of {} the cache has room for", L, cap)
     _abort_if(k.shape[-1] != dk or tuple(v.shape) != tuple(k.shape), "Attention: key/value shapes {} {} vs dk {}",
               tuple(k.shape), tuple(v.shape), dk)
     batchQ = q.numel() // (m * dk)
-    batchKV = k.numel() // (L * dk)
-    if m >= 8 and kNew is None and not want_absmax:
+    batchKV = k.numel() // (cap * dk)
+    if m >= 8 and kNew is None and not want_absmax and L == cap:
         # Many query positions per head (encoder layers, whole target sentences): the one-launch
         # form gives every query row a wave that walks the head's keys and values on its own; the
         # three operators share them through LDS tiles (1024 heads of 64 x 64 x 64: 57 us against 105).
@@ -216,12 +220,12 @@ def Attention(q, k, v, mask=None, rowsPerMask=1, want_absmax=False, kNew=None, v
         n_masks = mask.shape[0]
     out = torch.empty_like(q)
     omax = AbsMax(q.device) if want_absmax else None
-    st = be.lib.marian_hip_attention(q.data_ptr(), k.data_ptr(), v.data_ptr(),
-                                     None if mask is None else mask.data_ptr(), n_masks, rowsPerMask,
-                                     out.data_ptr(), batchQ, batchKV, m, L, dk, 1.0 / float(dk) ** 0.5,
-                                     None if omax is None else omax.data_ptr(),
-                                     None if kNew is None else kNew.data_ptr(),
-                                     None if vNew is None else vNew.data_ptr(), be.stream())
+    st = be.lib.marian_hip_attention_cached(q.data_ptr(), k.data_ptr(), v.data_ptr(),
+                                            None if mask is None else mask.data_ptr(), n_masks, rowsPerMask,
+                                            out.data_ptr(), batchQ, batchKV, m, L, cap, dk, 1.0 / float(dk) ** 0.5,
+                                            None if omax is None else omax.data_ptr(),
+                                            None if kNew is None else kNew.data_ptr(),
+                                            None if vNew is None else vNew.data_ptr(), be.stream())
     _lib.check(st, "Attention")
     return (out, omax) if want_absmax else out
 

@@ -102,6 +102,10 @@ def test_argument_validation_returns_codes_not_aborts():
     assert lib.marian_hip_nbest(buf, 2, 100, 4, None, buf, None) == L.ERR_NULL
     assert lib.marian_hip_attention(buf, buf, None, None, 0, 0, buf, 2, 2, 1, 40, 64, 0.125, None, None, None, None) == L.ERR_NULL
     assert lib.marian_hip_attention(buf, buf, buf, None, 0, 0, buf, 4, 2, 1, 40, 64, 0.125, None, buf, buf, None) == L.ERR_SHAPE
+    assert lib.marian_hip_attention_cached(buf, buf, buf, None, 0, 0, buf, 2, 2, 1, 40, 39, 64, 0.125, None, None, None, None) == L.ERR_SHAPE
+    assert lib.marian_hip_attention_cached(buf, buf, buf, None, 0, 0, buf, 2, 2, 1, 5000, 6000, 64, 0.125, None, None, None, None) == L.ERR_RANGE
+    assert lib.marian_hip_attention_cached(buf, None, buf, None, 0, 0, buf, 2, 2, 1, 40, 64, 64, 0.125, None, None, None, None) == L.ERR_NULL
+    assert lib.marian_hip_attention_cached(buf, buf, buf, None, 0, 0, buf, 0, 2, 1, 40, 64, 64, 0.125, None, None, None, None) == L.OK
     assert lib.marian_hip_int8_affine_shortlist(buf, buf, None, buf, 12, buf, 1, 64, 8, 1.0, 0, None) == L.ERR_SHAPE
     assert lib.marian_hip_embed(buf, buf, 4, 0, 8, 1.0, None, 0, 0, buf, None, None) == L.ERR_SHAPE
     assert lib.marian_hip_embed(buf, buf, 4, 10, 8, 1.0, buf, 0, 1, buf, None, None) == L.ERR_SHAPE

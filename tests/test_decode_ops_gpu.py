@@ -766,3 +766,34 @@ def test_layer_norm_one_wave_per_row(ops, chk, synth, rows, cols):
                                        rows, cols, 1e-6, None, None)
     torch.cuda.synchronize()
     assert st == 0 and np.array_equal(xin.cpu().numpy(), ref)
+
+
+@pytest.mark.parametrize("BQ,BKV,L,cap,dk,masked,append", [(2048, 2048, 21, 32, 64, False, True), (96, 24, 40, 64, 64, True, False),
+                                                           (30, 30, 7, 7, 64, False, True), (16, 16, 5, 9, 32, False, True),
+                                                           (12, 4, 70, 100, 20, True, False), (8, 8, 1, 4, 64, False, True)])
+def test_attention_on_caches_with_room_to_grow(ops, synth, BQ, BKV, L, cap, dk, masked, append):
+    """keys and values in [entries, capacity, dk] tensors of which the first L positions are in use
+    give the bits of the call on [entries, L, dk] tensors, whatever the rest of the cache holds;
+    the appended position lands at L - 1 of the roomy cache and nothing else in it changes"""
+    import torch
+    q = dev(synth.normal(BQ + L, 0, (BQ, 1, dk), 1.0))
+    k = synth.normal(BQ + L, 1, (BKV, L, dk), 1.0)
+    v = synth.normal(BQ + L, 2, (BKV, L, dk), 1.0)
+    roomy_k = synth.normal(BQ + L, 3, (BKV, cap, dk), 50.0)
+    roomy_v = synth.normal(BQ + L, 4, (BKV, cap, dk), 50.0)
+    roomy_k[:, :L], roomy_v[:, :L] = k, v
+    mask = None
+    if masked:
+        lens = 1 + (np.arange(BKV) * 5) % L
+        mask = dev(((np.arange(L)[None, :] >= lens[:, None]) * -99999999.0).astype(np.float32))
+    kn = dev(synth.normal(BQ + L, 5, (BQ, dk), 1.0)) if append else None
+    vn = dev(synth.normal(BQ + L, 6, (BQ, dk), 1.0)) if append else None
+    dk_, dv_ = dev(k), dev(v)
+    want = ops.Attention(q, dk_, dv_, mask, kNew=kn, vNew=vn)
+    rk, rv = dev(roomy_k), dev(roomy_v)
+    got = ops.Attention(q, rk, rv, mask, kNew=kn, vNew=vn, kvLen=L)
+    assert torch.equal(got, want)
+    if append:
+        roomy_k[:, L - 1], roomy_v[:, L - 1] = kn.cpu().numpy(), vn.cpu().numpy()
+        assert np.array_equal(rk.cpu().numpy(), roomy_k) and np.array_equal(rv.cpu().numpy(), roomy_v)
+        assert torch.equal(dk_[:, L - 1], kn) and torch.equal(dv_[:, L - 1], vn)

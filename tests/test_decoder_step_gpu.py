@@ -47,10 +47,12 @@ def check_trace(step, trace, orc, chk):
     n_affine = 0
     for kind, t in trace:
         h = {k: (v.cpu().numpy() if hasattr(v, "cpu") else v) for k, v in t.items()}
-        if kind == "embed":
+        if kind == "select":
+            assert np.array_equal(h["out"], h["state"][h["rows"].astype(np.int64)]), "state selection"
+        elif kind == "embed":
             want = chk.embed(h["E"], h["ids"], np.float32(h["scale"]), h["signal"].reshape(1, -1), step.M)
             assert np.array_equal(h["out"], want), "embedding step"
-            assert np.array_equal(h["signal"].reshape(-1), chk.sinusoidal_position_embeddings(1, step.d, step.T - 1)[0])
+            assert np.array_equal(h["signal"].reshape(-1), chk.sinusoidal_position_embeddings(1, step.d, t["position"])[0])
         elif kind == "affine":
             Bq, bias = t["w"]
             A = h["a"].reshape(-1, h["a"].shape[-1])
@@ -66,10 +68,11 @@ def check_trace(step, trace, orc, chk):
             MH = step.M * step.H
             dk = step.d // step.H
             k_full, v_full = h["k_cache"].copy(), h["v_cache"].copy()
-            k_full[:, -1, :] = h["k_new"].reshape(MH, dk)      # the new position takes the last slot
-            v_full[:, -1, :] = h["v_new"].reshape(MH, dk)
+            T = h["len"]                                         # positions in use; the cache may have room for more
+            k_full[:, T - 1, :] = h["k_new"].reshape(MH, dk)     # the new position takes the last slot in use
+            v_full[:, T - 1, :] = h["v_new"].reshape(MH, dk)
             assert np.array_equal(h["k_after"], k_full) and np.array_equal(h["v_after"], v_full), "cache append"
-            want = attention_reference(h["q"].reshape(MH, dk), k_full, v_full, None, step.H, MH)
+            want = attention_reference(h["q"].reshape(MH, dk), k_full[:, :T], v_full[:, :T], None, step.H, MH)
             close(h["out"].reshape(MH, dk), want, 2e-5, 1e-5)
         elif kind == "context_attention":
             MH = step.M * step.H
@@ -92,6 +95,8 @@ def check_trace(step, trace, orc, chk):
 
 def check_chain(trace):
     """the data flow of the layer: what a call reads is what the call before it wrote"""
+    if trace[0][0] == "select":
+        trace = trace[1:]
     kinds = [k for k, _ in trace]
     per_layer = ["affine"] * 3 + ["self_attention", "affine", "layer_norm", "affine", "context_attention", "affine",
                                   "layer_norm", "affine", "affine", "layer_norm"]
@@ -158,3 +163,38 @@ def test_decoder_step_every_call_against_the_checker(integer, orc, size):
     vals_r, keys_r = step.step(0, fused_tail=True)
     assert torch.equal(vals_s, vals_r) and torch.equal(keys_s, keys_r)
     assert not torch.equal(vals_s, vals)
+
+
+def test_beam_search_steps_in_place(integer, orc):
+    """Three consecutive decoding steps of a small decoder whose caches have room to grow: each
+    step's n-best gives the next step its words and back-pointers (src/translator/beam_search.cpp:
+    the key of a candidate is sentence * beam * vocab + beam entry * vocab + word), the next step
+    gathers the caches of the hypotheses that go on, embeds their words at the next position and
+    appends one more cached position in place - and every operator call of every step is checked
+    against the CPU checker on the inputs it received."""
+    import torch
+    from oracle import decode_ops as chk
+    chk.lib()
+    D = load("decoder_step")
+    step = D.DecoderStep(sets=1, d=256, ffn=1024, heads=4, vocab=4000, layers=2, beam=3, batch=5,
+                         t_past=2, src_len=9, min_src_len=3, seed=23, t_capacity=8)
+    beam, batch, V = step.beam, step.batch, step.V
+    for s in range(3):
+        say("step", s, "positions in use", step.T)
+        step.trace = []
+        step.step(0, select=s > 0)
+        torch.cuda.synchronize()
+        trace, step.trace = step.trace, None
+        assert trace[0][0] == ("select" if s > 0 else "embed")
+        check_chain(trace)
+        assert check_trace(step, trace, orc, chk) == 8 * step.layers + 1
+        keys = [e for kind, e in trace if kind == "nbest"][0]["keys"].cpu().numpy().astype(np.int64).reshape(batch, beam)
+        sentence = keys // (beam * V)
+        assert np.array_equal(sentence, np.arange(batch)[:, None].repeat(beam, 1))
+        came_from = (keys % (beam * V)) // V           # beam entry the candidate continues
+        word = keys % V
+        # the k-th best candidate of sentence b becomes hypothesis (k, b)
+        hyp = (came_from * batch + np.arange(batch)[:, None]).T.reshape(-1)
+        if s < 2:
+            step.advance(torch.from_numpy(word.T.reshape(-1).copy()), torch.from_numpy(hyp.copy()))
+    assert step.T == 5
