@@ -693,8 +693,8 @@ def main():
             "ms_per_step": round(fdt / n * 1e3, 4),
             "ms_per_step_with_state_selection": round(seldt / n * 1e3, 4),
             "state_selection": "the step preceded by the beam search's selection of the surviving hypotheses' cached keys "
-                               "and values (rows(state, hypIndices) over all layers as one gather, %d MB read and written); "
-                               "hypothesis indices resident on the device" % round(dec.state.numel() * 4 / 1e6),
+                               "and values (rows(state, hypIndices) over all layers as one gather of the positions in use, %d MB read and written); "
+                               "hypothesis indices resident on the device" % round(dec.state.numel() * 4 / 1e6 * (dec.T - 1) / dec.cap),
             "ms_per_step_logsoftmax_and_nbest_as_two_launches": round(sdt / n * 1e3, 4),
             "one_launch_tail_equals_two_launches": same_tail,
             "ms_per_step_unchained": round(udt / n * 1e3, 4),

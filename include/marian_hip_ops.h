@@ -137,6 +137,20 @@ int marian_hip_embed(const float* E, const uint32_t* ids, int64_t rows, int64_t 
                      float* out, float* absmax_out, void* stream);
 
 /*
+ * The selection of the surviving hypotheses' decoder states between two steps of the beam search
+ * (reference src/models/states.h:87-107, src/rnn/types.h:22-42: rows(reshape(state, [beam * batch,
+ * positions * depth]), selIdx)) for states that stay in place and have room to grow:
+ *   state: [entries, segments, seg_capacity] float32 (the caches of marian_hip_attention_cached:
+ *   segments = heads, seg_capacity = kv_capacity * dk), out: [rows, segments, seg_capacity];
+ *   out[r, s, 0 .. seg_len) = state[ids[r], s, 0 .. seg_len), seg_len = positions in use * dk.
+ * What lies behind seg_len is neither read nor written.  state and out must not overlap
+ * (MARIAN_HIP_ERR_ALIAS); an id at or past `entries` reads the last entry.
+ * With seg_len == seg_capacity and one segment this is marian_hip_embed with scale 1.
+ */
+int marian_hip_select_state(const float* state, const uint32_t* ids, int64_t rows, int64_t entries,
+                            int64_t segments, int64_t seg_capacity, int64_t seg_len, float* out, void* stream);
+
+/*
  * Replaces SinusoidalPositionEmbeddings, reference src/tensors/cpu/tensor_operators.cpp:1733-1746,
  * the initializer of the constant that src/models/transformer.h:110-111 adds to the embeddings:
  *   host_out[j, i] = sin or cos of (j + start) * exp((i % (dimEmb / 2)) * -log(10000) / (dimEmb / 2 - 1)),

@@ -1286,6 +1286,37 @@ __global__ __launch_bounds__(256) void embed_kernel(const float* __restrict__ E,
   }
 }
 
+// The selection of decoder states whose entries are `segs` segments of seg_cap values of which the
+// first seg_len are in use (cached positions of the heads of a hypothesis): workgroup (r * segs + s,
+// chunk) copies kEmbedChunk values of segment s of entry ids[r]; what lies behind seg_len is neither
+// read nor written.
+template <bool VEC>
+__global__ __launch_bounds__(256) void select_state_kernel(const float* __restrict__ in, const uint32_t* __restrict__ ids,
+                                                           unsigned entries, unsigned segs, long long seg_cap,
+                                                           int seg_len, float* __restrict__ out) {
+  const unsigned row = blockIdx.x / segs, seg = blockIdx.x % segs, chunk = blockIdx.y;
+  const int tid = threadIdx.x;
+  unsigned id = ids[row];
+  id = id < entries ? id : entries - 1u;
+  const int c0 = (int)chunk * kEmbedChunk, c1 = min(c0 + kEmbedChunk, seg_len);
+  const float* src = in + ((size_t)id * segs + seg) * (size_t)seg_cap;
+  float* dst = out + ((size_t)row * segs + seg) * (size_t)seg_cap;
+  if(VEC) {
+    constexpr int kV = kEmbedChunk / 4 / 256;
+    const int last = c1 / 4 - 1;
+    v4f e[kV];
+#pragma unroll
+    for(int j = 0; j < kV; ++j) e[j] = reinterpret_cast<const v4f*>(src)[min(c0 / 4 + j * 256 + tid, last)];
+#pragma unroll
+    for(int j = 0; j < kV; ++j) {
+      const int i = c0 / 4 + j * 256 + tid;
+      if(i <= last) reinterpret_cast<v4f*>(dst)[i] = e[j];
+    }
+  } else {
+    for(int i = c0 + tid; i < c1; i += 256) dst[i] = src[i];
+  }
+}
+
 __global__ __launch_bounds__(256) void zero_words_kernel(unsigned* __restrict__ p, long long n) {
   for(long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long long)gridDim.x * blockDim.x)
     p[i] = 0u;
@@ -1359,6 +1390,35 @@ int marian_hip_embed(const float* E, const uint32_t* ids, int64_t rows, int64_t 
   else
     hipLaunchKernelGGL(embed_kernel<false>, dim3((unsigned)rows, (unsigned)chunks), dim3(256), 0, st, E, ids,
                        (unsigned)vocab, (int)dimEmb, scale, signal, rps, ns, out, absmax_out);
+  MH_HIP(hipGetLastError());
+  return MARIAN_HIP_OK;
+}
+
+int marian_hip_select_state(const float* state, const uint32_t* ids, int64_t rows, int64_t entries,
+                            int64_t segments, int64_t seg_capacity, int64_t seg_len, float* out, void* stream) {
+  if(rows < 0 || entries <= 0 || segments <= 0 || seg_capacity <= 0 || seg_len < 0 || seg_len > seg_capacity)
+    return MARIAN_HIP_ERR_SHAPE;
+  if(rows == 0 || seg_len == 0) return MARIAN_HIP_OK;
+  if(!state || !ids || !out) return MARIAN_HIP_ERR_NULL;
+  const int64_t chunks = (seg_len + kEmbedChunk - 1) / kEmbedChunk;
+  if(entries > 0xFFFFFFFFLL || segments > 65535 || rows > kMaxElemsOps / segments || chunks > 65535 ||
+     seg_len > kMaxElemsOps ||
+     entries * segments > kMaxElemsOps / seg_capacity || rows * segments > kMaxElemsOps / seg_capacity)
+    return MARIAN_HIP_ERR_RANGE;
+  if(!aligned4(state) || !aligned4(ids) || !aligned4(out)) return MARIAN_HIP_ERR_ALIGN;
+  // not in place: an entry may be read after the row of the same number has been written
+  const uintptr_t a0 = reinterpret_cast<uintptr_t>(state), a1 = a0 + (uintptr_t)(entries * segments * seg_capacity) * 4;
+  const uintptr_t b0 = reinterpret_cast<uintptr_t>(out), b1 = b0 + (uintptr_t)(rows * segments * seg_capacity) * 4;
+  if(a0 < b1 && b0 < a1) return MARIAN_HIP_ERR_ALIAS;
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  const bool vec = seg_len % 4 == 0 && seg_capacity % 4 == 0 && aligned16(state) && aligned16(out);
+  const dim3 grid((unsigned)(rows * segments), (unsigned)chunks);
+  if(vec)
+    hipLaunchKernelGGL(select_state_kernel<true>, grid, dim3(256), 0, st, state, ids, (unsigned)entries, (unsigned)segments,
+                       (long long)seg_capacity, (int)seg_len, out);
+  else
+    hipLaunchKernelGGL(select_state_kernel<false>, grid, dim3(256), 0, st, state, ids, (unsigned)entries, (unsigned)segments,
+                       (long long)seg_capacity, (int)seg_len, out);
   MH_HIP(hipGetLastError());
   return MARIAN_HIP_OK;
 }

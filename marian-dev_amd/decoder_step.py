@@ -113,7 +113,10 @@ class DecoderStep:
         """The decoder state of the surviving hypotheses (reference src/models/states.h:87-107,
         src/rnn/types.h:22-42: rows(state, hypIndices) per cached tensor) for all layers in one
         gather; the two state tensors swap roles."""
-        self.ops.rows(self.state, self.state_rows, out=self.state_next)
+        H, span = self.H, self.cap * (self.d // self.H)
+        # (the positions cached so far: the step's own position is appended behind them afterwards)
+        self.ops.selectState(self.state.view(-1, H, span), self.state_rows, self.state_next.view(-1, H, span),
+                             used=(self.T - 1) * (self.d // self.H))
         self.state, self.state_next = self.state_next, self.state
         self._cache_views()
 
@@ -140,7 +143,7 @@ class DecoderStep:
         if select and not gemm_only:
             before = self.state
             self.select_states()
-            rec("select", state=before, rows=self.state_rows, out=self.state)
+            rec("select", state=before, rows=self.state_rows, out=self.state, heads=H, used=(self.T - 1) * dk)
         if not gemm_only:
             x = ops.scaledEmbeddings(self.E, self.words, self.emb_scale, self.signal, M, want_absmax=ch)
             if ch:

@@ -93,6 +93,29 @@ def rows(a, indices, out=None):
     return scaledEmbeddings(a, indices.reshape(-1), out=out)
 
 
+def selectState(state, indices, out, used=None):
+    """The decoder state of the surviving hypotheses (reference src/models/states.h:87-107,
+    src/rnn/types.h:22-42): out[r, s, :used] = state[indices[r], s, :used] for a state [entries,
+    segments, capacity] whose segments (the cached positions of a head) are in use up to `used`
+    values (None: entirely); out [len(indices), segments, capacity] is a tensor of its own."""
+    _abort_if(state.dtype != torch.float32 or out.dtype != torch.float32 or state.dim() != 3 or out.dim() != 3 or
+              not state.is_contiguous() or not out.is_contiguous(), "selectState expects contiguous float32 "
+              "tensors [entries, segments, capacity], got {} and {}", tuple(state.shape), tuple(out.shape))
+    be = _backend_of(state)
+    entries, segments, cap = state.shape
+    _abort_if(tuple(out.shape) != (indices.numel(), segments, cap), "selectState: out has shape {}, not {}",
+              tuple(out.shape), (indices.numel(), segments, cap))
+    _abort_if(indices.dtype not in (torch.int32, torch.int64, torch.uint32) or indices.device != state.device,
+              "selectState: indices have to be an integer tensor on the state's device")
+    ids = indices.contiguous()
+    if ids.dtype == torch.int64:
+        ids = ids.to(torch.int32)
+    st = be.lib.marian_hip_select_state(state.data_ptr(), ids.data_ptr(), ids.numel(), entries, segments, cap,
+                                        cap if used is None else int(used), out.data_ptr(), be.stream())
+    _lib.check(st, "selectState")
+    return out
+
+
 def sinusoidalPositionEmbeddings(dimWords, dimEmb, start=0, device=None):
     """The constant [dimWords, 1, dimEmb] of reference src/models/transformer.h:110-111, made on the
     host by the library (reference src/tensors/cpu/tensor_operators.cpp:1733-1746) and copied to

@@ -797,3 +797,24 @@ def test_attention_on_caches_with_room_to_grow(ops, synth, BQ, BKV, L, cap, dk, 
         roomy_k[:, L - 1], roomy_v[:, L - 1] = kn.cpu().numpy(), vn.cpu().numpy()
         assert np.array_equal(rk.cpu().numpy(), roomy_k) and np.array_equal(rv.cpu().numpy(), roomy_v)
         assert torch.equal(dk_[:, L - 1], kn) and torch.equal(dv_[:, L - 1], vn)
+
+
+@pytest.mark.parametrize("entries,rows,segs,cap,used", [(1536, 1536, 16, 21 * 64, 20 * 64), (30, 45, 4, 8 * 64, 3 * 64),
+                                                        (7, 7, 3, 10, 7), (12, 5, 2, 5000 * 4, 4097 * 4), (9, 9, 16, 64, 0),
+                                                        (4, 6, 1, 4096, 4096)])
+def test_select_state_copies_the_positions_in_use(ops, synth, entries, rows, segs, cap, used):
+    """the state selection between two beam-search steps on states with room to grow: the values in
+    use of every segment of the chosen entries, bit for bit; what lies behind them in the output is
+    left as it was"""
+    import torch
+    state = synth.normal(entries + cap, 0, (entries, segs, cap), 1.0)
+    back = synth.normal(rows, 1, (rows,), 1e3).astype(np.int64) % entries
+    old = synth.normal(entries + cap, 2, (rows, segs, cap), 1.0)
+    out = dev(old)
+    ops.selectState(dev(state), torch.from_numpy(back).cuda(), out, used=used)
+    want = old.copy()
+    want[:, :, :used] = state[back][:, :, :used]
+    assert np.array_equal(out.cpu().numpy(), want)
+    L = load("_lib")
+    s = dev(state)
+    assert L.lib().marian_hip_select_state(s.data_ptr(), s.data_ptr(), 1, entries, segs, cap, used, s.data_ptr(), None) == (L.ERR_ALIAS if used else L.OK)

@@ -48,7 +48,9 @@ def check_trace(step, trace, orc, chk):
     for kind, t in trace:
         h = {k: (v.cpu().numpy() if hasattr(v, "cpu") else v) for k, v in t.items()}
         if kind == "select":
-            assert np.array_equal(h["out"], h["state"][h["rows"].astype(np.int64)]), "state selection"
+            before = h["state"].reshape(h["state"].shape[0], h["heads"], -1)      # [entries, heads, capacity * dk]
+            after = h["out"].reshape(before.shape)
+            assert np.array_equal(after[:, :, :h["used"]], before[h["rows"].astype(np.int64)][:, :, :h["used"]]), "state selection"
         elif kind == "embed":
             want = chk.embed(h["E"], h["ids"], np.float32(h["scale"]), h["signal"].reshape(1, -1), step.M)
             assert np.array_equal(h["out"], want), "embedding step"
