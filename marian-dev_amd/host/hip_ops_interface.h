@@ -10,6 +10,7 @@
 //   src/tensors/cpu/tensor_operators.cpp:577-603                       CopyRows
 //   src/tensors/cpu/tensor_operators.cpp:1733-1746                     SinusoidalPositionEmbeddings
 //   src/models/transformer.h:92-117                                    ScaledEmbeddings (rows * sqrt(d) + signal)
+//   src/rnn/types.h:22-42                                              SelectState (State::select)
 #pragma once
 
 #include "../../include/marian_hip_ops.h"
@@ -47,6 +48,18 @@ inline void ScaledEmbeddings(Backend& be, Tensor& out, const Tensor& in, const T
 // out[j, :] = in[indices[j], :]
 inline void CopyRows(Backend& be, Tensor& out, const Tensor& in, const Tensor& indices) {
   ScaledEmbeddings(be, out, in, indices, 1.0f);
+}
+
+// The decoder state of the surviving hypotheses (State::select, src/rnn/types.h:22-42) for states
+// [entries, segments, capacity] that stay in place: out[r, s, 0 .. used) = state[indices[r], s, 0 .. used).
+inline void SelectState(Backend& be, Tensor& out, const Tensor& state, const Tensor& indices, int64_t used) {
+  if(indices.type != Type::uint32) abortWith("SelectState expects indices of type uint32");
+  if(state.shape.size() != 3 || out.shape.size() != 3 || out.shape[1] != state.shape[1] || out.shape[2] != state.shape[2] ||
+     (size_t)out.shape[0] != indices.elements())
+    abortWith("SelectState expects [entries, segments, capacity] tensors and one index per output entry");
+  MARIAN_HIP_CHECK(marian_hip_select_state(state.data<float>(), indices.data<uint32_t>(), (int64_t)indices.elements(),
+                                           state.shape[0], state.shape[1], state.shape[2], used, out.data<float>(),
+                                           be.stream()));
 }
 
 // The constant [dimWords, 1, dimEmb] of the position signal, made on the host: `host` receives

@@ -406,6 +406,18 @@ int main(int argc, char** argv) {
         slotsOk = slotsOk && slots[r] == m;
       }
       expect(slotsOk, "ScaledEmbeddings: abs-max slot per row, zero past the last row");
+      // state selection: 3 entries x 2 segments x capacity 6, four values of every segment in use
+      std::vector<float> stateHost(3 * 2 * 6), before(4 * 2 * 6, -1.0f);
+      for(size_t i = 0; i < stateHost.size(); ++i) stateHost[i] = (float)i;
+      const std::vector<uint32_t> back{2, 0, 2, 1};
+      Tensor stT = upload(ta, stateHost, {3, 2, 6}, Type::float32), bk = upload(ta, back, {4}, Type::uint32);
+      Tensor sel = upload(ta, before, {4, 2, 6}, Type::float32);
+      SelectState(be, sel, stT, bk, 4);
+      std::vector<float> wantSel = before;
+      for(int r = 0; r < 4; ++r)
+        for(int sg = 0; sg < 2; ++sg)
+          for(int i = 0; i < 4; ++i) wantSel[(size_t)(r * 2 + sg) * 6 + i] = stateHost[(size_t)(back[r] * 2 + sg) * 6 + i];
+      expect(sameBits(download<float>(be, sel, wantSel.size()), wantSel), "SelectState: the values in use of the chosen entries, the rest untouched");
     }
     be.synchronize();
     std::printf("host_check: %d failure(s), slab moved %zu times -> %s\n", failures,
