@@ -682,6 +682,14 @@ def main():
         sel = [capture(torch, (lambda c=c: dec.step(c, fused_tail=True, select=True))) for c in range(bsets)]
         seldt = time_graphs(torch, sel, n, max(4, args.warmup // 2))
         del sel
+        dec.by_ancestors = True    # the same step on caches that are never moved
+        dec.anc = torch.randint(0, dec.M, (dec.M, dec.cap), device="cuda", dtype=torch.int32)
+        dec.anc = (dec.anc // dec.batch * dec.batch + torch.arange(dec.M, device="cuda", dtype=torch.int32)[:, None] % dec.batch).contiguous()
+        dec.anc_next = torch.empty_like(dec.anc)
+        sel = [capture(torch, (lambda c=c: dec.step(c, fused_tail=True, select=True))) for c in range(bsets)]
+        ancdt = time_graphs(torch, sel, n, max(4, args.warmup // 2))
+        del sel
+        dec.by_ancestors = False
         out["transformer_big_decode_full"] = {
             "what": "full decoder step through the host mirrors, from the previous step's word indices: embedding rows x "
                     "sqrt(d) + position signal (one launch), 49 int8 affine calls + per layer "
@@ -692,6 +700,11 @@ def main():
                     "abs-max of every GEMM input is left by the kernel that produced it",
             "ms_per_step": round(fdt / n * 1e3, 4),
             "ms_per_step_with_state_selection": round(seldt / n * 1e3, 4),
+            "ms_per_step_with_state_selection_by_ancestors": round(ancdt / n * 1e3, 4),
+            "state_selection_by_ancestors": "the caches stay where they were written; a table [hypotheses, positions] says in "
+                                            "whose cache entry a position of a hypothesis's history lies (here: a random "
+                                            "hypothesis of the same sentence per position), the selection rewrites the table "
+                                            "and the self-attention follows it",
             "state_selection": "the step preceded by the beam search's selection of the surviving hypotheses' cached keys "
                                "and values (rows(state, hypIndices) over all layers as one gather of the positions in use, %d MB read and written); "
                                "hypothesis indices resident on the device" % round(dec.state.numel() * 4 / 1e6 * (dec.T - 1) / dec.cap),

@@ -137,6 +137,28 @@ int marian_hip_embed(const float* E, const uint32_t* ids, int64_t rows, int64_t 
                      float* out, float* absmax_out, void* stream);
 
 /*
+ * Self-attention of a decoding step on caches that are never moved: where the reference selects
+ * the surviving hypotheses' states between two steps by copying them (src/rnn/types.h:22-42), a
+ * table of ancestors says in whose cache entry a position of a hypothesis's history lies, and the
+ * call follows it.  No counterpart in the reference; the result is that of
+ * marian_hip_attention_cached on caches gathered position by position, bit for bit.
+ *   q, k_new, v_new, out: [n_hyp * heads, dk]; k, v: [n_hyp * heads, kv_capacity, dk], entry =
+ *   hypothesis * heads + head; ancestors: uint32 [n_hyp, kv_capacity] on the device: cached position
+ *   p < len - 1 of hypothesis h is read from the entry of hypothesis ancestors[h * kv_capacity + p]
+ *   (values at or past n_hyp read the last hypothesis); position len - 1 is k_new / v_new, which the
+ *   call stores into hypothesis h's own entry.  dk == 64, all tensors 16-byte aligned.
+ * marian_hip_ancestors_advance makes the table of the next step: next[h, p] = prev[parents[h], p]
+ * for the len_prev positions cached so far and next[h, len_prev] = h (prev and next must not
+ * overlap); parents: uint32 [n_hyp], the back-pointers of the beam search.
+ */
+int marian_hip_attention_ancestors(const float* q, float* k, float* v, float* out, int64_t n_hyp, int64_t heads,
+                                   int64_t len, int64_t kv_capacity, int64_t dk, float scale, float* absmax_out,
+                                   const float* k_new, const float* v_new, const uint32_t* ancestors,
+                                   void* stream);
+int marian_hip_ancestors_advance(const uint32_t* prev, const uint32_t* parents, int64_t n_hyp, int64_t kv_capacity,
+                                 int64_t len_prev, uint32_t* next, void* stream);
+
+/*
  * The selection of the surviving hypotheses' decoder states between two steps of the beam search
  * (reference src/models/states.h:87-107, src/rnn/types.h:22-42: rows(reshape(state, [beam * batch,
  * positions * depth]), selIdx)) for states that stay in place and have room to grow:

@@ -58,6 +58,8 @@ SIGNATURES = {
     "marian_hip_logsoftmax_nbest_beams": (_i, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp, _vp, _vp, _sz, _vp]),
     "marian_hip_embed": (_i, [_vp, _vp, _i64, _i64, _i64, _f, _vp, _i64, _i64, _vp, _vp, _vp]),
     "marian_hip_sinusoidal_position_embeddings": (_i, [_vp, _i64, _i64, _i64]),
+    "marian_hip_attention_ancestors": (_i, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _f, _vp, _vp, _vp, _vp, _vp]),
+    "marian_hip_ancestors_advance": (_i, [_vp, _vp, _i64, _i64, _i64, _vp, _vp]),
     "marian_hip_select_state": (_i, [_vp, _vp, _i64, _i64, _i64, _i64, _i64, _vp, _vp]),
     "marian_hip_fill": (_i, [_vp, _i64, _i, _c.c_uint64, _vp]),
     "marian_hip_attention": (_i, [_vp, _vp, _vp, _vp, _i64, _i64, _vp, _i64, _i64, _i64, _i64, _i64,

@@ -518,6 +518,12 @@ __global__ __launch_bounds__(256) void bdot_tile_kernel(const float* __restrict_
 // as bdot_kernel walks them), softmax over them exactly as softmax_kernel<64> computes it, then
 // the weighted sum of the value rows (a lane per output column, positions in ascending order,
 // as bdot_kernel does).  The scores of a row live in LDS: `len` floats per wave.
+// ANC (m == 1, dk == 64, one cache entry per query row, entry = hypothesis * heads + head): cached
+// position p of hypothesis h is read from the entry of hypothesis anc[h * kv_cap + p] - the caches
+// of a beam search stay where they were written and the table of ancestors says whose row a
+// position of a hypothesis's history is; the newest position comes from k_new / v_new and goes into
+// the hypothesis's own entry.
+template <bool ANC>
 __global__ __launch_bounds__(256) void attention_kernel(const float* __restrict__ Q, float* Kt, float* V,
                                                         const float* __restrict__ k_new,
                                                         const float* __restrict__ v_new,
@@ -525,7 +531,8 @@ __global__ __launch_bounds__(256) void attention_kernel(const float* __restrict_
                                                         unsigned n_masks, unsigned rows_per_mask,
                                                         float* __restrict__ out, unsigned rows_total,
                                                         unsigned batchKV, int m, int len, int kv_cap, int dk,
-                                                        float scale, float* __restrict__ absmax_out) {
+                                                        float scale, float* __restrict__ absmax_out,
+                                                        const uint32_t* __restrict__ anc, unsigned heads) {
   // kv_cap: positions a cache entry has room for (its stride, in rows of dk values); len of them are in use
   // (row counts are below 2^31, checked by the launcher: 32-bit divisions, a tenth of the
   // instructions of 64-bit ones, and this kernel is a chain of short phases)
@@ -605,13 +612,50 @@ __global__ __launch_bounds__(256) void attention_kernel(const float* __restrict_
       }
     }
   };
+  // ANC: the entry a cached position is read from differs from position to position.  The lane's
+  // (up to sixteen) ancestors of a batch of 64 positions are requested together, one round trip
+  // ahead of the key and value rows.
+  unsigned au[ANC ? kAttU : 1];
+  const unsigned hyp = ANC ? wr / heads : 0u, head = ANC ? wr % heads : 0u;
+  auto load_ancestors = [&](int base) __attribute__((always_inline)) {
+    if(ANC) {
+      const uint32_t* row = anc + (size_t)hyp * kv_cap;
+      const unsigned n_hyp = rows_total / heads;
+#pragma unroll
+      for(int u = 0; u < kAttU; ++u)
+        if(base + 4 * u < len) au[u] = min(row[min(base + 4 * u + g, len - 1)], n_hyp - 1u);
+    }
+  };
+  auto load_rows_anc = [&](const float* tensor, const float* last, int base, v4f (&r)[kAttU]) __attribute__((always_inline)) {
+    const float* last_c = last + 4 * c;
+#pragma unroll
+    for(int u = 0; u < kAttU; ++u) {
+      if(base + 4 * u < len) {   // (the same for the whole wave)
+        const int U = base / 4 + u;
+        const float* p = U >= u_last ? last_c
+                                     : tensor + ((size_t)(au[ANC ? u : 0] * heads + head) * kv_cap + (size_t)(4 * U + g)) * dk + 4 * c;
+        r[u] = *reinterpret_cast<const v4f*>(p);
+      } else if(base + 4 * (u & ~3) < len) {
+        r[u] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+      }
+    }
+  };
+  auto load_k = [&](int base, v4f (&r)[kAttU]) __attribute__((always_inline)) {
+    if(ANC) load_rows_anc(Kt, k_last, base, r);
+    else load_rows(kb, k_last, base, r);
+  };
+  auto load_v = [&](int base, v4f (&r)[kAttU]) __attribute__((always_inline)) {
+    if(ANC) load_rows_anc(V, v_last, base, r);
+    else load_rows(vb, v_last, base, r);
+  };
   if(fast) {
     float mk0 = 0.0f;
     if(mk) mk0 = mk[min(lane, len - 1)];
     const v4f q4 = reinterpret_cast<const v4f*>(q)[c];
     v4f kr[kAttU];
-    load_rows(kb, k_last, 0, kr);
-    load_rows(vb, v_last, 0, vr);
+    load_ancestors(0);
+    load_k(0, kr);
+    load_v(0, vr);
     // (sixteen positions at a time without a branch between them: the four products and the four
     // exchange steps of a group of four positions depend on one another, and only independent
     // groups side by side keep the wave issuing; rows that were not loaded are zeros here and their
@@ -639,7 +683,8 @@ __global__ __launch_bounds__(256) void attention_kernel(const float* __restrict_
       }
       base += 4 * kAttU;
       if(base >= len) break;
-      load_rows(kb, k_last, base, kr);
+      load_ancestors(base);
+      load_k(base, kr);
     }
     for(int pos = lane; pos < len; pos += 64) {
       float z = sc[pos];
@@ -699,7 +744,10 @@ __global__ __launch_bounds__(256) void attention_kernel(const float* __restrict_
   if(fast) {
     v4f o4 = v4f{0.0f, 0.0f, 0.0f, 0.0f};
     for(int base = 0; base < len; base += 4 * kAttU) {
-      if(base > 0) load_rows(vb, v_last, base, vr);
+      if(base > 0) {
+        load_ancestors(base);
+        load_v(base, vr);
+      }
 #pragma unroll
       for(int u0 = 0; u0 < kAttU; u0 += 4) {
         if(base + 4 * u0 < len) {
@@ -1544,10 +1592,71 @@ int marian_hip_attention(const float* q, float* k, float* v, const float* mask, 
                                      scale, absmax_out, k_new, v_new, stream);
 }
 
+static int attention_impl(const float* q, float* k, float* v, const float* mask, int64_t n_masks,
+                          int64_t rows_per_mask, float* out, int64_t batchQ, int64_t batchKV, int64_t m,
+                          int64_t len, int64_t kv_capacity, int64_t dk, float scale, float* absmax_out,
+                          const float* k_new, const float* v_new, const uint32_t* ancestors, int64_t heads,
+                          void* stream);
+
 int marian_hip_attention_cached(const float* q, float* k, float* v, const float* mask, int64_t n_masks,
                                 int64_t rows_per_mask, float* out, int64_t batchQ, int64_t batchKV,
                                 int64_t m, int64_t len, int64_t kv_capacity, int64_t dk, float scale,
                                 float* absmax_out, const float* k_new, const float* v_new, void* stream) {
+  return attention_impl(q, k, v, mask, n_masks, rows_per_mask, out, batchQ, batchKV, m, len, kv_capacity, dk, scale,
+                        absmax_out, k_new, v_new, nullptr, 1, stream);
+}
+
+int marian_hip_attention_ancestors(const float* q, float* k, float* v, float* out, int64_t n_hyp, int64_t heads,
+                                   int64_t len, int64_t kv_capacity, int64_t dk, float scale, float* absmax_out,
+                                   const float* k_new, const float* v_new, const uint32_t* ancestors,
+                                   void* stream) {
+  if(n_hyp < 0 || heads <= 0 || dk != 64) return MARIAN_HIP_ERR_SHAPE;
+  if(n_hyp == 0) return MARIAN_HIP_OK;
+  if(!ancestors || !k_new || !v_new) return MARIAN_HIP_ERR_NULL;
+  if(n_hyp > kMaxElemsOps / heads) return MARIAN_HIP_ERR_RANGE;
+  if(!aligned4(ancestors)) return MARIAN_HIP_ERR_ALIGN;
+  if(q && k && v && (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(k_new) || !aligned16(v_new)))
+    return MARIAN_HIP_ERR_ALIGN;
+  return attention_impl(q, k, v, nullptr, 0, 0, out, n_hyp * heads, n_hyp * heads, 1, len, kv_capacity, dk, scale,
+                        absmax_out, k_new, v_new, ancestors, heads, stream);
+}
+
+// next[h, p] = prev[parents[h], p] for the len_prev positions cached so far, next[h, len_prev] = h:
+// the position the coming step appends lies in the hypothesis's own entry.
+__global__ __launch_bounds__(256) void ancestors_advance_kernel(const uint32_t* __restrict__ prev,
+                                                                const uint32_t* __restrict__ parents, unsigned n_hyp,
+                                                                unsigned kv_cap, unsigned len_prev,
+                                                                uint32_t* __restrict__ next) {
+  const unsigned i = blockIdx.x * 256 + threadIdx.x;
+  if(i >= n_hyp * (len_prev + 1)) return;
+  const unsigned h = i / (len_prev + 1), p = i % (len_prev + 1);
+  const unsigned from = min(parents[h], n_hyp - 1u);
+  next[(size_t)h * kv_cap + p] = p < len_prev ? prev[(size_t)from * kv_cap + p] : h;
+}
+
+int marian_hip_ancestors_advance(const uint32_t* prev, const uint32_t* parents, int64_t n_hyp, int64_t kv_capacity,
+                                 int64_t len_prev, uint32_t* next, void* stream) {
+  if(n_hyp < 0 || kv_capacity <= 0 || len_prev < 0 || len_prev >= kv_capacity) return MARIAN_HIP_ERR_SHAPE;
+  if(n_hyp == 0) return MARIAN_HIP_OK;
+  if(!prev || !parents || !next) return MARIAN_HIP_ERR_NULL;
+  if(n_hyp > kMaxElemsOps / kv_capacity) return MARIAN_HIP_ERR_RANGE;
+  if(!aligned4(prev) || !aligned4(parents) || !aligned4(next)) return MARIAN_HIP_ERR_ALIGN;
+  const uintptr_t a0 = reinterpret_cast<uintptr_t>(prev), b0 = reinterpret_cast<uintptr_t>(next);
+  const uintptr_t bytes = (uintptr_t)(n_hyp * kv_capacity) * 4;
+  if(a0 < b0 + bytes && b0 < a0 + bytes) return MARIAN_HIP_ERR_ALIAS;   // (a row may be read after the row of the same number has been written)
+  const int64_t n = n_hyp * (len_prev + 1);
+  hipLaunchKernelGGL(ancestors_advance_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,
+                     reinterpret_cast<hipStream_t>(stream), prev, parents, (unsigned)n_hyp, (unsigned)kv_capacity,
+                     (unsigned)len_prev, next);
+  MH_HIP(hipGetLastError());
+  return MARIAN_HIP_OK;
+}
+
+static int attention_impl(const float* q, float* k, float* v, const float* mask, int64_t n_masks,
+                          int64_t rows_per_mask, float* out, int64_t batchQ, int64_t batchKV, int64_t m,
+                          int64_t len, int64_t kv_capacity, int64_t dk, float scale, float* absmax_out,
+                          const float* k_new, const float* v_new, const uint32_t* ancestors, int64_t heads,
+                          void* stream) {
   if((k_new != nullptr) != (v_new != nullptr)) return MARIAN_HIP_ERR_NULL;
   if(kv_capacity < len) return MARIAN_HIP_ERR_SHAPE;
   if(k_new && (m != 1 || batchKV != batchQ)) return MARIAN_HIP_ERR_SHAPE;
@@ -1574,14 +1683,23 @@ int marian_hip_attention_cached(const float* q, float* k, float* v, const float*
     MH_HIP(hipGetDevice(&dev));
     if(dev < 0 || dev >= 64) return MARIAN_HIP_ERR_RANGE;
     if(!(lds_done.load(std::memory_order_acquire) & (1ull << dev))) {
-      MH_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(attention_kernel),
+      MH_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(attention_kernel<false>),
+                                 hipFuncAttributeMaxDynamicSharedMemorySize, 72 * 1024));
+      MH_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(attention_kernel<true>),
                                  hipFuncAttributeMaxDynamicSharedMemorySize, 72 * 1024));
       lds_done.fetch_or(1ull << dev, std::memory_order_release);
     }
   }
-  hipLaunchKernelGGL(attention_kernel, dim3((unsigned)((rows_total + 3) / 4)), dim3(256), lds, st, q, k, v,
-                     k_new, v_new, mask, (unsigned)n_masks, (unsigned)rows_per_mask, out, (unsigned)rows_total,
-                     (unsigned)batchKV, (int)m, (int)len, (int)kv_capacity, (int)dk, scale, absmax_out);
+  if(ancestors)
+    hipLaunchKernelGGL(attention_kernel<true>, dim3((unsigned)((rows_total + 3) / 4)), dim3(256), lds, st, q, k, v,
+                       k_new, v_new, mask, (unsigned)n_masks, (unsigned)rows_per_mask, out, (unsigned)rows_total,
+                       (unsigned)batchKV, (int)m, (int)len, (int)kv_capacity, (int)dk, scale, absmax_out, ancestors,
+                       (unsigned)heads);
+  else
+    hipLaunchKernelGGL(attention_kernel<false>, dim3((unsigned)((rows_total + 3) / 4)), dim3(256), lds, st, q, k, v,
+                       k_new, v_new, mask, (unsigned)n_masks, (unsigned)rows_per_mask, out, (unsigned)rows_total,
+                       (unsigned)batchKV, (int)m, (int)len, (int)kv_capacity, (int)dk, scale, absmax_out, ancestors,
+                       1u);
   MH_HIP(hipGetLastError());
   return MARIAN_HIP_OK;
 }

@@ -24,7 +24,7 @@ class DecoderStep:
     Beam search's hypothesis bookkeeping is not part of the step."""
 
     def __init__(self, sets=1, d=1024, ffn=4096, heads=16, vocab=32000, layers=6, beam=4, batch=32,
-                 t_past=20, src_len=60, min_src_len=20, seed=300, t_capacity=None):
+                 t_past=20, src_len=60, min_src_len=20, seed=300, t_capacity=None, ancestors=False):
         self.torch, self.integer, self.ops = torch, integer, ops
         self.d, self.ffn, self.V, self.H = d, ffn, vocab, heads
         self.beam, self.batch, self.layers = beam, batch, layers
@@ -81,6 +81,12 @@ class DecoderStep:
         # same sentence; flat index k * batch + b, one copy per cache tensor
         parent = torch.randint(0, beam, (beam, batch), device="cuda", generator=g) * batch + torch.arange(batch, device="cuda")
         self.set_hypotheses(parent.reshape(-1))
+        # ancestors: the caches are never moved; a table says in whose entry a position of a
+        # hypothesis's history lies (at the start: in its own), and the state selection rewrites the table
+        self.by_ancestors = bool(ancestors)
+        if self.by_ancestors:
+            self.anc = torch.arange(M, device="cuda", dtype=torch.int32)[:, None].repeat(1, self.cap).contiguous()
+            self.anc_next = torch.empty_like(self.anc)
         self.Kenc = [torch.randn(self.batch * H, self.L, d // H, device="cuda", generator=g) for _ in range(layers)]
         self.Venc = [torch.randn(self.batch * H, self.L, d // H, device="cuda", generator=g) for _ in range(layers)]
         # source lengths uniform over min_src_len .. src_len, padded to the longest (the mask covers the rest)
@@ -113,6 +119,10 @@ class DecoderStep:
         """The decoder state of the surviving hypotheses (reference src/models/states.h:87-107,
         src/rnn/types.h:22-42: rows(state, hypIndices) per cached tensor) for all layers in one
         gather; the two state tensors swap roles."""
+        if self.by_ancestors:
+            self.ops.advanceAncestors(self.anc, self.hyp_indices, self.T - 1, self.anc_next)
+            self.anc, self.anc_next = self.anc_next, self.anc
+            return
         H, span = self.H, self.cap * (self.d // self.H)
         # (the positions cached so far: the step's own position is appended behind them afterwards)
         self.ops.selectState(self.state.view(-1, H, span), self.state_rows, self.state_next.view(-1, H, span),
@@ -143,7 +153,8 @@ class DecoderStep:
         if select and not gemm_only:
             before = self.state
             self.select_states()
-            rec("select", state=before, rows=self.state_rows, out=self.state, heads=H, used=(self.T - 1) * dk)
+            if not self.by_ancestors:
+                rec("select", state=before, rows=self.state_rows, out=self.state, heads=H, used=(self.T - 1) * dk)
         if not gemm_only:
             x = ops.scaledEmbeddings(self.E, self.words, self.emb_scale, self.signal, M, want_absmax=ch)
             if ch:
@@ -166,8 +177,12 @@ class DecoderStep:
                 # new key/value to the cache
                 if tr is not None:
                     k_before, v_before = self.Kself[li].clone(), self.Vself[li].clone()
-                o = ops.Attention(q.view(M * H, 1, dk), self.Kself[li], self.Vself[li], want_absmax=ch,
-                                  kNew=k.view(M * H, dk), vNew=v.view(M * H, dk), kvLen=self.T)
+                if self.by_ancestors:
+                    o = ops.AttentionByAncestors(q.view(M * H, 1, dk), self.Kself[li], self.Vself[li], self.anc, self.T,
+                                                 k.view(M * H, dk), v.view(M * H, dk), want_absmax=ch)
+                else:
+                    o = ops.Attention(q.view(M * H, 1, dk), self.Kself[li], self.Vself[li], want_absmax=ch,
+                                      kNew=k.view(M * H, dk), vNew=v.view(M * H, dk), kvLen=self.T)
                 if ch:
                     o, omax = o
                 if tr is not None:

@@ -10,7 +10,8 @@
 //   src/tensors/cpu/tensor_operators.cpp:577-603                       CopyRows
 //   src/tensors/cpu/tensor_operators.cpp:1733-1746                     SinusoidalPositionEmbeddings
 //   src/models/transformer.h:92-117                                    ScaledEmbeddings (rows * sqrt(d) + signal)
-//   src/rnn/types.h:22-42                                              SelectState (State::select)
+//   src/rnn/types.h:22-42                                              SelectState (State::select); AdvanceAncestors +
+//                                                                      AttentionByAncestors do without the copy
 #pragma once
 
 #include "../../include/marian_hip_ops.h"
@@ -113,6 +114,31 @@ inline void Attention(Backend& be, Tensor& out, const Tensor& q, Tensor& k, Tens
       mask ? (int64_t)rows(*mask) : 0, rowsPerMask, out.data<float>(), q.shape[0], k.shape[0], q.shape[1],
       kvLen ? kvLen : k.shape[1], k.shape[1], q.shape[2], scale, absmaxOut ? absmaxOut->data<float>() : nullptr,
       kNew ? kNew->data<float>() : nullptr, vNew ? vNew->data<float>() : nullptr, be.stream()));
+}
+
+// Self-attention of a decoding step on caches that are never moved: cached position p of hypothesis
+// h is read from the entry of hypothesis ancestors[h, p] (uint32 [hypotheses, capacity]); kNew / vNew
+// become position kvLen - 1 of the hypotheses' own entries.  q, kNew, vNew, out [hyps * heads, 1 or -, 64].
+inline void AttentionByAncestors(Backend& be, Tensor& out, const Tensor& q, Tensor& k, Tensor& v, float scale,
+                                 const Tensor& ancestors, int64_t kvLen, const Tensor& kNew, const Tensor& vNew,
+                                 Tensor* absmaxOut = nullptr) {
+  if(k.shape.size() != 3 || ancestors.shape.size() != 2 || ancestors.type != Type::uint32 ||
+     ancestors.shape[1] != k.shape[1] || k.shape[0] % ancestors.shape[0] != 0)
+    abortWith("AttentionByAncestors expects caches [entries, capacity, dk] and uint32 ancestors [hypotheses, capacity]");
+  MARIAN_HIP_CHECK(marian_hip_attention_ancestors(
+      q.data<float>(), k.data<float>(), v.data<float>(), out.data<float>(), ancestors.shape[0],
+      k.shape[0] / ancestors.shape[0], kvLen, k.shape[1], k.shape[2], scale,
+      absmaxOut ? absmaxOut->data<float>() : nullptr, kNew.data<float>(), vNew.data<float>(),
+      ancestors.data<uint32_t>(), be.stream()));
+}
+
+// The table of the next step: next[h, p] = prev[parents[h], p] for p < lenPrev, next[h, lenPrev] = h.
+inline void AdvanceAncestors(Backend& be, Tensor& next, const Tensor& prev, const Tensor& parents, int64_t lenPrev) {
+  if(prev.shape.size() != 2 || next.shape != prev.shape || prev.type != Type::uint32 || next.type != Type::uint32 ||
+     parents.type != Type::uint32 || parents.elements() != (size_t)prev.shape[0])
+    abortWith("AdvanceAncestors expects uint32 tables [hypotheses, capacity] and one back-pointer per hypothesis");
+  MARIAN_HIP_CHECK(marian_hip_ancestors_advance(prev.data<uint32_t>(), parents.data<uint32_t>(), prev.shape[0],
+                                                prev.shape[1], lenPrev, next.data<uint32_t>(), be.stream()));
 }
 
 // The beam search's n-best selection; it owns its device buffers like the reference's NthElement.

@@ -418,6 +418,42 @@ int main(int argc, char** argv) {
         for(int sg = 0; sg < 2; ++sg)
           for(int i = 0; i < 4; ++i) wantSel[(size_t)(r * 2 + sg) * 6 + i] = stateHost[(size_t)(back[r] * 2 + sg) * 6 + i];
       expect(sameBits(download<float>(be, sel, wantSel.size()), wantSel), "SelectState: the values in use of the chosen entries, the rest untouched");
+      // the same beam-search step without the copy: 3 hypotheses x 2 heads, two cached positions + the new one
+      const int nh = 3, hd = 2, cp = 4, ln = 3, dkk = 64;
+      std::vector<float> kc((size_t)nh * hd * cp * dkk), vc(kc.size()), qv((size_t)nh * hd * dkk), knv(qv.size()), vnv(qv.size());
+      uint32_t r2 = 777u;
+      auto nextf = [&]() { r2 = r2 * 1664525u + 1013904223u; return (float)(r2 >> 8) * (1.0f / 8388608.0f) - 1.0f; };
+      for(auto& x : kc) x = nextf();
+      for(auto& x : vc) x = nextf();
+      for(auto& x : qv) x = nextf();
+      for(auto& x : knv) x = nextf();
+      for(auto& x : vnv) x = nextf();
+      const std::vector<uint32_t> prevAnc{0, 0, 0, 0, 1, 1, 1, 1, 2, 2, 2, 2}, parents{2, 2, 0};
+      Tensor pa = upload(ta, prevAnc, {nh, cp}, Type::uint32), pr = upload(ta, parents, {nh}, Type::uint32), na;
+      ta.allocate(na, {nh, cp}, Type::uint32);
+      AdvanceAncestors(be, na, pa, pr, ln - 1);
+      const std::vector<uint32_t> gotAnc = download<uint32_t>(be, na, (size_t)nh * cp);
+      expect(gotAnc[0] == 2 && gotAnc[1] == 2 && gotAnc[2] == 0 && gotAnc[4] == 2 && gotAnc[6] == 1 && gotAnc[8] == 0 &&
+                 gotAnc[9] == 0 && gotAnc[10] == 2,
+             "AdvanceAncestors: the parents' rows, then the hypothesis itself");
+      // reference: the caches of the parents copied (SelectState), then the attention on them
+      std::vector<uint32_t> rowsOfParents;
+      for(int h = 0; h < nh; ++h) rowsOfParents.push_back(parents[h]);
+      Tensor kT = upload(ta, kc, {nh, hd, cp * dkk}, Type::float32), vT = upload(ta, vc, {nh, hd, cp * dkk}, Type::float32);
+      Tensor kG = upload(ta, kc, {nh, hd, cp * dkk}, Type::float32), vG = upload(ta, vc, {nh, hd, cp * dkk}, Type::float32);
+      Tensor rp = upload(ta, rowsOfParents, {nh}, Type::uint32);
+      SelectState(be, kG, kT, rp, (ln - 1) * dkk);
+      SelectState(be, vG, vT, rp, (ln - 1) * dkk);
+      Tensor qT = upload(ta, qv, {nh * hd, 1, dkk}, Type::float32), knT = upload(ta, knv, {nh * hd, dkk}, Type::float32);
+      Tensor vnT = upload(ta, vnv, {nh * hd, dkk}, Type::float32), o1, o2;
+      ta.allocate(o1, {nh * hd, 1, dkk}, Type::float32);
+      ta.allocate(o2, {nh * hd, 1, dkk}, Type::float32);
+      kG.shape = {nh * hd, cp, dkk}; vG.shape = kG.shape;
+      Attention(be, o1, qT, kG, vG, 0.125f, nullptr, 1, nullptr, &knT, &vnT, ln);
+      kT.shape = {nh * hd, cp, dkk}; vT.shape = kT.shape;
+      AttentionByAncestors(be, o2, qT, kT, vT, 0.125f, na, ln, knT, vnT);
+      expect(sameBits(download<float>(be, o2, qv.size()), download<float>(be, o1, qv.size())),
+             "AttentionByAncestors: the attention on the copied caches, bit for bit");
     }
     be.synchronize();
     std::printf("host_check: %d failure(s), slab moved %zu times -> %s\n", failures,

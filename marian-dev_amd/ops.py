@@ -253,6 +253,52 @@ def Attention(q, k, v, mask=None, rowsPerMask=1, want_absmax=False, kNew=None, v
     return (out, omax) if want_absmax else out
 
 
+def AttentionByAncestors(q, k, v, ancestors, kvLen, kNew, vNew, want_absmax=False):
+    """Self-attention of a decoding step on caches that are never moved (no counterpart in the
+    reference, which copies the surviving hypotheses' states, src/rnn/types.h:22-42): cached
+    position p of hypothesis h is read from the cache entry of hypothesis ancestors[h, p].
+    q [hyps * heads, 1, dk]; k, v [hyps * heads, capacity, dk]; ancestors int32 [hyps, capacity];
+    kNew, vNew [hyps * heads, dk] become position kvLen - 1 of the hypotheses' own entries."""
+    q, kNew, vNew = _f32c(q, "AttentionByAncestors"), _f32c(kNew, "AttentionByAncestors"), _f32c(vNew, "AttentionByAncestors")
+    be = _backend_of(q)
+    _abort_if(k.dtype != torch.float32 or v.dtype != torch.float32 or not (k.is_contiguous() and v.is_contiguous()) or
+              k.dim() != 3 or tuple(k.shape) != tuple(v.shape), "AttentionByAncestors: the caches have to be contiguous "
+              "float32 tensors [entries, capacity, dk], got {} and {}", tuple(k.shape), tuple(v.shape))
+    entries, cap, dk = k.shape
+    _abort_if(ancestors.dtype not in (torch.int32, torch.uint32) or ancestors.dim() != 2 or ancestors.shape[1] != cap or
+              not ancestors.is_contiguous() or entries % ancestors.shape[0] != 0,
+              "AttentionByAncestors: ancestors have to be a contiguous int32 tensor [hypotheses, {}]", cap)
+    hyps = ancestors.shape[0]
+    _abort_if(q.numel() != entries * dk or kNew.numel() != entries * dk or vNew.numel() != entries * dk,
+              "AttentionByAncestors: one query, key and value row of {} values per cache entry", dk)
+    out = torch.empty_like(q)
+    omax = AbsMax(q.device) if want_absmax else None
+    st = be.lib.marian_hip_attention_ancestors(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), hyps,
+                                               entries // hyps, int(kvLen), cap, dk, 1.0 / float(dk) ** 0.5,
+                                               None if omax is None else omax.data_ptr(), kNew.data_ptr(),
+                                               vNew.data_ptr(), ancestors.data_ptr(), be.stream())
+    _lib.check(st, "AttentionByAncestors")
+    return (out, omax) if want_absmax else out
+
+
+def advanceAncestors(prev, parents, lenPrev, out):
+    """the table of ancestors of the next step: out[h, p] = prev[parents[h], p] for p < lenPrev,
+    out[h, lenPrev] = h (prev, out: int32 [hypotheses, capacity], two tensors)"""
+    _abort_if(prev.dtype != torch.int32 or out.dtype != torch.int32 or tuple(prev.shape) != tuple(out.shape) or
+              prev.dim() != 2 or not (prev.is_contiguous() and out.is_contiguous()),
+              "advanceAncestors expects two contiguous int32 tensors [hypotheses, capacity]{}", "")
+    be = _backend_of(prev)
+    par = parents.contiguous()
+    if par.dtype == torch.int64:
+        par = par.to(torch.int32)
+    _abort_if(par.dtype not in (torch.int32, torch.uint32) or par.numel() != prev.shape[0],
+              "advanceAncestors: one int32 back-pointer per hypothesis{}", "")
+    st = be.lib.marian_hip_ancestors_advance(prev.data_ptr(), par.data_ptr(), prev.shape[0], prev.shape[1], int(lenPrev),
+                                             out.data_ptr(), be.stream())
+    _lib.check(st, "advanceAncestors")
+    return out
+
+
 def getNBestList(scores, N):
     """reference src/translator/nth_element.cpp:26-67: scores [dimBatch, 1, beam, vocab]; returns
     (pathScores, keys) of dimBatch * N entries, keys = position in the flattened tensor."""

@@ -113,6 +113,13 @@ def test_argument_validation_returns_codes_not_aborts():
     assert lib.marian_hip_embed(buf, buf, 4096, 10, 8, 1.0, None, 0, 0, buf, buf, None) == L.ERR_RANGE
     assert lib.marian_hip_embed(buf, buf + 2, 4, 10, 8, 1.0, None, 0, 0, buf, None, None) == L.ERR_ALIGN
     assert lib.marian_hip_embed(buf, buf, 0, 10, 8, 1.0, None, 0, 0, buf, None, None) == L.OK
+    assert lib.marian_hip_attention_ancestors(buf, buf, buf, buf, 4, 2, 5, 8, 32, 0.125, None, buf, buf, buf, None) == L.ERR_SHAPE
+    assert lib.marian_hip_attention_ancestors(buf, buf, buf, buf, 4, 2, 5, 8, 64, 0.125, None, buf, buf, None, None) == L.ERR_NULL
+    assert lib.marian_hip_attention_ancestors(buf, buf, buf, buf, 4, 2, 5, 8, 64, 0.125, None, buf + 4, buf, buf, None) == L.ERR_ALIGN
+    assert lib.marian_hip_attention_ancestors(buf, buf, buf, buf, 4, 2, 9, 8, 64, 0.125, None, buf, buf, buf, None) == L.ERR_SHAPE
+    assert lib.marian_hip_attention_ancestors(buf, buf, buf, buf, 0, 2, 5, 8, 64, 0.125, None, buf, buf, buf, None) == L.OK
+    assert lib.marian_hip_ancestors_advance(buf, buf, 4, 8, 8, buf + 4096, None) == L.ERR_SHAPE
+    assert lib.marian_hip_ancestors_advance(buf, None, 4, 8, 3, buf + 4096, None) == L.ERR_NULL
     assert lib.marian_hip_select_state(buf, buf, 4, 8, 2, 64, 65, buf + 65536, None) == L.ERR_SHAPE
     assert lib.marian_hip_select_state(buf, None, 4, 8, 2, 64, 64, buf + 65536, None) == L.ERR_NULL
     assert lib.marian_hip_select_state(buf, buf, 4, 8, 2, 64, 64, buf + 1024, None) == L.ERR_ALIAS

@@ -818,3 +818,51 @@ def test_select_state_copies_the_positions_in_use(ops, synth, entries, rows, seg
     L = load("_lib")
     s = dev(state)
     assert L.lib().marian_hip_select_state(s.data_ptr(), s.data_ptr(), 1, entries, segs, cap, used, s.data_ptr(), None) == (L.ERR_ALIAS if used else L.OK)
+
+
+@pytest.mark.parametrize("hyps,heads,L,cap", [(128, 16, 21, 21), (128, 16, 21, 40), (12, 4, 70, 100), (6, 2, 1, 3),
+                                              (9, 3, 64, 64), (5, 8, 65, 66), (20, 1, 130, 140)])
+def test_attention_by_ancestors_is_attention_on_gathered_caches(ops, synth, hyps, heads, L, cap):
+    """caches that are never moved: cached position p of hypothesis h read from the entry of
+    hypothesis ancestors[h, p] gives the bits of the call on caches into which those rows were
+    copied first; the new position lands in the hypothesis's own entry and nothing else changes"""
+    import torch
+    dk, E = 64, hyps * heads
+    q = dev(synth.normal(E + L, 0, (E, 1, dk), 1.0))
+    k = synth.normal(E + L, 1, (E, cap, dk), 1.0)
+    v = synth.normal(E + L, 2, (E, cap, dk), 1.0)
+    kn, vn = synth.normal(E + L, 3, (E, dk), 1.0), synth.normal(E + L, 4, (E, dk), 1.0)
+    anc = (synth.normal(E + L, 5, (hyps, cap), 1e3).astype(np.int64) % hyps).astype(np.int32)
+    anc[:, L - 1] = np.arange(hyps)
+    # gathered caches: entry (h, head), position p <- entry (anc[h, p], head), position p
+    kg, vg = k.copy().reshape(hyps, heads, cap, dk), v.copy().reshape(hyps, heads, cap, dk)
+    k4, v4 = k.reshape(hyps, heads, cap, dk), v.reshape(hyps, heads, cap, dk)
+    for p in range(L - 1):
+        kg[:, :, p] = k4[anc[:, p], :, p]
+        vg[:, :, p] = v4[anc[:, p], :, p]
+    want, wmax = ops.Attention(q, dev(kg.reshape(E, cap, dk)), dev(vg.reshape(E, cap, dk)), kNew=dev(kn), vNew=dev(vn),
+                               kvLen=L, want_absmax=E <= 2048) if E <= 2048 else (None, None)
+    dk_, dv_ = dev(k), dev(v)
+    got, gmax = ops.AttentionByAncestors(q, dk_, dv_, dev(anc), L, dev(kn), dev(vn), want_absmax=True)
+    assert torch.equal(got, want) and torch.equal(gmax.data, wmax.data)
+    k[:, L - 1], v[:, L - 1] = kn, vn
+    assert np.array_equal(dk_.cpu().numpy(), k) and np.array_equal(dv_.cpu().numpy(), v)
+
+
+def test_advance_ancestors(ops, synth):
+    import torch
+    hyps, cap = 37, 19
+    L = load("_lib")
+    for len_prev in (0, 1, 7, 18):
+        prev = (synth.normal(len_prev, 0, (hyps, cap), 1e3).astype(np.int64) % hyps).astype(np.int32)
+        parents = (synth.normal(len_prev, 1, (hyps,), 1e3).astype(np.int64) % hyps).astype(np.int32)
+        old = np.full((hyps, cap), -5, np.int32)
+        out = dev(old)
+        ops.advanceAncestors(dev(prev), dev(parents), len_prev, out)
+        want = old.copy()
+        want[:, :len_prev] = prev[parents][:, :len_prev]
+        want[:, len_prev] = np.arange(hyps)
+        assert np.array_equal(out.cpu().numpy(), want)
+    t = dev(prev)
+    assert L.lib().marian_hip_ancestors_advance(t.data_ptr(), t.data_ptr(), hyps, cap, 3, t.data_ptr(), None) == L.ERR_ALIAS
+    assert L.lib().marian_hip_ancestors_advance(t.data_ptr(), t.data_ptr(), hyps, cap, cap, out.data_ptr(), None) == L.ERR_SHAPE

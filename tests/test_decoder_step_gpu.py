@@ -180,13 +180,17 @@ def test_beam_search_steps_in_place(integer, orc):
     D = load("decoder_step")
     step = D.DecoderStep(sets=1, d=256, ffn=1024, heads=4, vocab=4000, layers=2, beam=3, batch=5,
                          t_past=2, src_len=9, min_src_len=3, seed=23, t_capacity=8)
+    # the same decoder on caches that are never moved (a table of ancestors instead of the copy)
+    lazy = D.DecoderStep(sets=1, d=256, ffn=1024, heads=4, vocab=4000, layers=2, beam=3, batch=5,
+                         t_past=2, src_len=9, min_src_len=3, seed=23, t_capacity=8, ancestors=True)
     beam, batch, V = step.beam, step.batch, step.V
     for s in range(3):
         say("step", s, "positions in use", step.T)
         step.trace = []
-        step.step(0, select=s > 0)
+        lp = step.step(0, select=s > 0)
         torch.cuda.synchronize()
         trace, step.trace = step.trace, None
+        assert torch.equal(lazy.step(0, select=s > 0), lp), "ancestor table against copied caches"
         assert trace[0][0] == ("select" if s > 0 else "embed")
         check_chain(trace)
         assert check_trace(step, trace, orc, chk) == 8 * step.layers + 1
@@ -199,4 +203,5 @@ def test_beam_search_steps_in_place(integer, orc):
         hyp = (came_from * batch + np.arange(batch)[:, None]).T.reshape(-1)
         if s < 2:
             step.advance(torch.from_numpy(word.T.reshape(-1).copy()), torch.from_numpy(hyp.copy()))
+            lazy.advance(torch.from_numpy(word.T.reshape(-1).copy()), torch.from_numpy(hyp.copy()))
     assert step.T == 5
