@@ -205,3 +205,28 @@ def test_beam_search_steps_in_place(integer, orc):
             step.advance(torch.from_numpy(word.T.reshape(-1).copy()), torch.from_numpy(hyp.copy()))
             lazy.advance(torch.from_numpy(word.T.reshape(-1).copy()), torch.from_numpy(hyp.copy()))
     assert step.T == 5
+
+
+def test_ancestor_table_at_benchmark_size():
+    """transformer-big, beam 4 x batch 32, caches with room for 24 positions: two beam-search steps
+    with random back-pointers; the decoder whose caches are never moved (table of ancestors) gives
+    the log-probabilities of the one that copies the surviving hypotheses' caches, bit for bit"""
+    import torch
+    D = load("decoder_step")
+    kw = dict(sets=1, t_past=20, t_capacity=24, seed=41)
+    copied, lazy = D.DecoderStep(**kw), D.DecoderStep(ancestors=True, **kw)
+    assert torch.equal(copied.state, lazy.state) and torch.equal(copied.words, lazy.words)
+    g = torch.Generator(device="cuda")
+    g.manual_seed(5)
+    for s in range(3):
+        say("step", s, "positions in use", copied.T)
+        a = copied.step(0, select=s > 0)
+        b = lazy.step(0, select=s > 0)
+        torch.cuda.synchronize()
+        assert torch.equal(a, b), "step %d" % s
+        if s < 2:
+            parents = torch.randint(0, copied.beam, (copied.beam, copied.batch), device="cuda", generator=g) * copied.batch + \
+                torch.arange(copied.batch, device="cuda")
+            words = torch.randint(0, copied.V, (copied.M,), device="cuda", generator=g)
+            copied.advance(words, parents.reshape(-1))
+            lazy.advance(words, parents.reshape(-1))
