@@ -112,3 +112,61 @@ def test_one_pass_prepare_a_replays_with_new_inputs(integer, orc, synth):
         if replay % 2:    # an eager call on another input, same workspace
             other = integer.prepareA(torch.from_numpy(inputs[(r + 1) % 4]).cuda())
             assert np.array_equal(other.numpy(), want[(r + 1) % 4])
+
+
+def test_beam_step_on_unmoved_caches_replays(integer, synth):
+    """embedding -> table of ancestors advanced -> self-attention that follows it (appending the
+    new position) -> the copy form of the same selection, recorded once: every replay gives the
+    eager results, with eager calls of the same kind in between.  (The replays start from the same
+    caches: the appended position is rewritten with the same values.)"""
+    import torch
+    ops = load("ops")
+    hyps, heads, cap, L, dk, vocab = 12, 4, 9, 6, 64, 300
+    g = torch.Generator(device="cuda")
+    g.manual_seed(9)
+    E = torch.randn(vocab, heads * dk, device="cuda", generator=g)
+    words = torch.randint(0, vocab, (hyps,), device="cuda", generator=g).to(torch.int32)
+    signal = ops.sinusoidalPositionEmbeddings(1, heads * dk, L - 1, device="cuda")
+    k = torch.randn(hyps * heads, cap, dk, device="cuda", generator=g)
+    v = torch.randn(hyps * heads, cap, dk, device="cuda", generator=g)
+    prev = torch.randint(0, hyps, (hyps, cap), device="cuda", generator=g).to(torch.int32)
+    parents = torch.randint(0, hyps, (hyps,), device="cuda", generator=g).to(torch.int32)
+    nxt = torch.empty_like(prev)
+    k2, v2 = torch.empty_like(k), torch.empty_like(v)
+
+    def step():
+        x, xmax = ops.scaledEmbeddings(E, words, 16.0, signal, hyps, want_absmax=True)
+        q = x.view(hyps * heads, 1, dk)
+        ops.advanceAncestors(prev, parents, L - 1, nxt)
+        o = ops.AttentionByAncestors(q, k, v, nxt, L, x.view(hyps * heads, dk), x.view(hyps * heads, dk))
+        ops.selectState(k.view(hyps, heads, cap * dk), parents, k2.view(hyps, heads, cap * dk), used=(L - 1) * dk)
+        ops.selectState(v.view(hyps, heads, cap * dk), parents, v2.view(hyps, heads, cap * dk), used=(L - 1) * dk)
+        return x, xmax.data, o, nxt, k2, v2
+
+    k2.zero_(); v2.zero_()
+    want = [t.clone() for t in step()]
+    torch.cuda.synchronize()
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        step()
+    torch.cuda.current_stream().wait_stream(s)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        outs = step()
+    for replay in range(4):
+        for t in outs[:3]:
+            t.fill_(float("nan"))
+        nxt.fill_(-1)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for i, (got, w) in enumerate(zip(outs, want)):
+            if i == 3:   # (the table's columns past the positions in use are not written)
+                assert torch.equal(got[:, :L], w[:, :L])
+            else:
+                assert torch.equal(got, w), "replay %d, output %d differs from the eager result" % (replay, i)
+        other = step()
+        torch.cuda.synchronize()
+        assert torch.equal(other[2], want[2])
