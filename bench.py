@@ -359,8 +359,73 @@ def probe_ceilings(torch):
                          ("write 4096x4096 fp32 (67 MB), as the GEMM's output", 16, 4096 * 4096 * 4)):
         us = stream(r_, w_, 2048, 256, 8, 0)
         print("  %-62s %8.2f us  %6.2f TB/s" % (name, us, (max(r_, 16) + max(w_, 16)) / us / 1e6))
-    print("\n-- sustained v_mfma_i32_32x32x32_i8 rate on random operand bits --")
     cus = torch.cuda.get_device_properties(0).multi_processor_count
+    print("\n-- one compute unit's LDS, vector L1 and matrix cores under instruction mixes (marian_hip_probe_mix: every "
+          "wave repeats a body of 16 slots with R ds_read_b128, M v_mfma_i32_32x32x32_i8, D global_load_lds_dwordx4 and "
+          "G global_load_dwordx4, 1 KB per wave and memory instruction; one workgroup per CU on all CUs; bytes per shader "
+          "clock and CU, median over the workgroups) --")
+    print("  %-5s %-3s %-3s %-3s %-3s %-8s | %9s %9s %9s %9s | %6s %8s" %
+          ("waves", "R", "M", "D", "G", "span", "LDS rd", "DMA", "to regs", "LDS total", "MFMA", "clock"))
+    print("  %-5s %-3s %-3s %-3s %-3s %-8s | %9s %9s %9s %9s | %6s %8s" %
+          ("", "", "", "", "", "", "B/clk/CU", "B/clk/CU", "B/clk/CU", "B/clk/CU", "issue", "MHz"))
+
+    def mix(waves, R, M, D, G, span, iters=400, split=0):
+        clocks = torch.zeros(2 * cus, dtype=torch.int64, device="cuda")
+        sink = torch.zeros(4, dtype=torch.int32, device="cuda")
+        for _ in range(2):
+            r = T.marian_hip_probe_mix(pool.data_ptr(), span, waves, R, M, D, G, split, iters, cus, clocks.data_ptr(),
+                                       sink.data_ptr(), st)
+            assert r == 0, r
+        torch.cuda.synchronize()
+        c = clocks.cpu().numpy().reshape(-1, 2).astype(np.float64)
+        clk = float(np.median(c[:, 0]))
+        mhz = float(np.median(c[:, 0] / c[:, 1]) * 100.0)
+        per = waves * 1024.0 * iters / clk
+        cw = lw = waves
+        if split:
+            cw = lw = 4
+        name = "%d KB" % (span >> 10) if span < (1 << 20) else "%d MB" % (span >> 20)
+        rd, dma, gl = R * per * cw / waves, D * per * lw / waves, G * per * lw / waves
+        print("  %-5s %-3d %-3d %-3d %-3d %-8s | %9.1f %9.1f %9.1f %9.1f | %5.0f%% %8.0f" %
+              ("4+4" if split else str(waves), R, M, D, G, name, rd, dma, gl, rd + dma,
+               100.0 * (cw / 4.0) * M * 32.0 * iters / clk, mhz))
+
+    KB, MB = 1 << 10, 1 << 20
+    for waves in (4, 8, 16):
+        mix(waves, 16, 0, 0, 0, 64 * KB)                 # LDS reads alone
+    for waves in (4, 8):
+        mix(waves, 16, 0, 8, 0, 2 * MB)                  # with operand blocks arriving, 2 : 1
+        mix(waves, 16, 0, 4, 0, 2 * MB)
+    for span in (64 * KB, 2 * MB, 32 * MB, 1024 * MB):    # global -> LDS alone: L1 hits, L2 hits, Infinity Cache, HBM
+        for waves in (4, 8, 16):
+            mix(waves, 0, 0, 16, 0, span)
+    for span in (64 * KB, 2 * MB, 32 * MB):               # global -> registers alone
+        for waves in (4, 8, 16):
+            mix(waves, 0, 0, 0, 16, span)
+    mix(4, 0, 0, 8, 8, 2 * MB)
+    mix(8, 0, 0, 8, 8, 2 * MB)
+    for waves in (4, 8):                                  # matrix instructions with 0 / 0.5 / 0.75 / 1 / 1.5 / 2 KB of fragments each
+        for R in (0, 4, 6, 8, 12, 16):
+            mix(waves, R, 8, 0, 0, 64 * KB)
+    for waves in (4, 8):                                  # matrix instructions with operand blocks arriving only
+        mix(waves, 0, 8, 4, 0, 2 * MB)
+        mix(waves, 0, 8, 0, 4, 2 * MB)
+    mix(4, 8, 8, 4, 0, 2 * MB)     # the 128x128 tile, four waves of 64x64
+    mix(8, 12, 8, 4, 0, 2 * MB)    # the same tile by eight waves of 64x32 (two per SIMD)
+    mix(8, 8, 8, 4, 0, 2 * MB)
+    mix(8, 8, 8, 4, 0, 2 * MB, split=1)   # four waves multiply, four waves load
+    mix(8, 8, 8, 3, 0, 2 * MB, split=1)   # the same at 48 bytes per clock of operand blocks
+    mix(8, 8, 8, 2, 0, 2 * MB, split=1)   # and at 32
+    mix(8, 0, 8, 4, 0, 2 * MB, split=1)
+    mix(4, 8, 8, 3, 0, 2 * MB)
+    mix(4, 8, 8, 2, 0, 2 * MB)
+    mix(8, 6, 8, 3, 0, 2 * MB, split=1)
+    mix(4, 6, 8, 3, 0, 2 * MB)     # two 256x128 tiles, four waves of 128x64
+    mix(8, 6, 8, 2, 0, 2 * MB)     # the 256x256 tile, eight waves of 128x64
+    mix(8, 4, 8, 1, 2, 2 * MB)     # the same with the weights from global memory straight into registers
+    mix(8, 4, 8, 2, 2, 2 * MB)
+    mix(4, 4, 8, 2, 4, 2 * MB)     # 128x128, four waves, weights straight into registers
+    print("\n-- sustained v_mfma_i32_32x32x32_i8 rate on random operand bits --")
     for per_cu in (1, 2):
         wgs, iters = cus * per_cu, 4000
         clocks = torch.zeros(2 * wgs, dtype=torch.int64, device="cuda")
@@ -585,6 +650,7 @@ def main():
     # ---------------- encoder-size GEMMs (MFMA-bound case) ------------------------------------
     if "encoder" in extras:
         enc = {}
+        sustained = measured_int8_peak(torch)
         for (M, K, N) in [(4096, 1024, 4096), (4096, 4096, 1024)]:
             o = Op(torch, integer, M, K, N, relu=True, copies=4, seed=77)
             o.launch(lib, be, 0, prepare=True, gemm=False)
@@ -593,20 +659,53 @@ def main():
             p_ms, _ = per_launch_ms(torch, [(lambda: o.launch(lib, be, 0, gemm=False))], 10)
             # the call BASELINE defines (fp32 A in, fp32 out) through the single entry point, timed as one
             f_ms, _ = per_launch_ms(torch, [(lambda c=c: o.launch_fused(lib, be, c)) for c in range(4)], 10)
+            # the same call when the producer of A left its abs-max (no abs-max pass) and this call leaves
+            # the abs-max of its own output for the next one
+            amax_in = torch.zeros(2048, device="cuda")
+            amax_in[0] = o.A.abs().max()
+            amax_out = torch.empty(2048, device="cuda")
+
+            def chained(c, o=o, amax_in=amax_in, amax_out=amax_out):
+                b = o.Bq[c % len(o.Bq)]
+                r = lib.marian_hip_int8_affine_f32_chained(
+                    o.A.data_ptr(), o.Aq.data_ptr(), b.data_ptr(), o.bias.data_ptr(), None, 0, o.out.data_ptr(),
+                    o.M, o.K, o.N, 1.0, o.relu, amax_in.data_ptr(), amax_out.data_ptr(),
+                    be.workspace.data_ptr(), be.workspace_bytes, be.stream())
+                assert r == 0, r
+            c_ms, _ = per_launch_ms(torch, [(lambda c=c: chained(c)) for c in range(4)], 10)
+            chained(0)
+            torch.cuda.synchronize()
+            slots_ok = bool(float(amax_out.max()) == float(o.out.abs().max()))
             t_all = f_ms * 1e-3
             enc["M%d_K%d_N%d" % (M, K, N)] = {
                 "gemm_us": round(g_ms * 1e3, 2), "gemm_median_us": round(g_med * 1e3, 2),
                 "prepare_a_us": round(p_ms * 1e3, 2),
                 "affine_f32_us": round(f_ms * 1e3, 2),
+                "affine_f32_chained_us": round(c_ms * 1e3, 2),
+                "chained_leaves_exact_absmax": slots_ok,
                 "gemm_tops": round(o.ops / (g_ms * 1e-3) / 1e12, 1),
                 "gemm_mfma_frac": round(o.ops / (g_ms * 1e-3) / 1e12 / INT8_PEAK_TOPS, 4),
+                "gemm_frac_of_sustained": None if not sustained else
+                    round(o.ops / (g_ms * 1e-3) / 1e12 / sustained["sustained_tops"], 4),
                 "gemm_hbm_frac": round(gemm_kernel_bytes(M, K, N) / (g_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
                 "affine_tops": round(o.ops / t_all / 1e12, 1),
-                "affine_hbm_frac": round(algorithmic_bytes(M, K, N) / t_all / 1e9 / HBM_PEAK_GBS, 4)}
+                "affine_hbm_frac": round(algorithmic_bytes(M, K, N) / t_all / 1e9 / HBM_PEAK_GBS, 4),
+                "affine_chained_hbm_frac": round(algorithmic_bytes(M, K, N) / (c_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+            del o
+        # a few rows or columns past a whole number of tiles (encoder M is a sum of sentence lengths)
+        for (M, K, N) in [(4100, 1024, 4096), (2050, 1024, 2056), (4100, 4096, 1024)]:
+            o = Op(torch, integer, M, K, N, relu=True, copies=4, seed=78)
+            o.launch(lib, be, 0, prepare=True, gemm=False)
+            g_ms, g_med = per_launch_ms(
+                torch, [(lambda c=c: o.launch(lib, be, c, prepare=False)) for c in range(4)], 10)
+            enc["M%d_K%d_N%d" % (M, K, N)] = {
+                "gemm_us": round(g_ms * 1e3, 2), "gemm_median_us": round(g_med * 1e3, 2),
+                "gemm_tops": round(o.ops / (g_ms * 1e-3) / 1e12, 1),
+                "gemm_mfma_frac": round(o.ops / (g_ms * 1e-3) / 1e12 / INT8_PEAK_TOPS, 4)}
             del o
         out["encoder"] = enc
         out["int8_peak_tops_used"] = INT8_PEAK_TOPS
-        out["int8_peak_measured"] = measured_int8_peak(torch)
+        out["int8_peak_measured"] = sustained
 
     # ---------------- shortlisted output layer -------------------------------------------------
     if "shortlist" in extras:

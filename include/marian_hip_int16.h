@@ -46,7 +46,8 @@ int marian_hip_int16_prepare_b(const float* W, int16_t* Bq, int64_t K, int64_t N
 /*
  * Replaces prepareAndTransposeB<intgemm16>, reference src/tensors/cpu/integer_common.h:189-216 and
  * src/common/binary.cpp:108-110: the file payload is the GPU layout, so this is a copy of
- * 2*K*N + 4 bytes.
+ * 2*K*N + 4 bytes.  K % 32 == 0, N % 8 == 0; in == out is a no-op, buffers that overlap in part
+ * return MARIAN_HIP_ERR_ALIAS.
  */
 int marian_hip_int16_prepare_b_quantized_transposed(const int16_t* in, int16_t* out, int64_t K, int64_t N,
                                                     void* stream);

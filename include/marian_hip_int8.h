@@ -169,8 +169,10 @@ int marian_hip_int8_affine_f32_grouped(const float* A, int8_t* Aq, int64_t n_gro
  * graph's allocator).  The caller passes inputs and the output only; the quantized activations
  * (M*K + 4 bytes) and the abs-max partials live in an array of
  * MARIAN_HIP_STATIC_MAX_ELEMS + 256 + marian_hip_int8_workspace_bytes() bytes that the library
- * holds on every GPU it runs on until the process ends.  The call makes no hipMalloc / hipFree
- * and no allocating library call.  `out` is what marian_hip_int8_affine_f32 writes, bit for bit.
+ * holds on every GPU it runs on until the process ends (16 MiB + 256 B + the 12 KB workspace).
+ * The words workgroups exchange through the workspace (one-pass prepareA, M * K >= 4 Mi) persist
+ * between calls and are told apart by tags; nothing in the array is ever cleared.  The call makes
+ * no hipMalloc / hipFree and no allocating library call.  `out` is what marian_hip_int8_affine_f32 writes, bit for bit.
  *   M * K > MARIAN_HIP_STATIC_MAX_ELEMS returns MARIAN_HIP_ERR_STATIC_LIMIT (checked first).
  *   The device must be current and `stream` must belong to it.  The first call on a device looks
  *   up the array's address (make that call outside a graph capture).

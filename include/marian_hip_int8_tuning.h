@@ -53,6 +53,21 @@ int marian_hip_probe_stream(const void* src, size_t read_bytes, void* dst, size_
                             int threads, int loads_in_flight, int nontemporal, void* stream);
 int marian_hip_probe_mfma(const void* data, int iters, int workgroups, long long* clocks, int* sink, void* stream);
 
+/*
+ * marian_hip_probe_mix: what one compute unit's LDS, vector L1 and matrix cores deliver under a
+ * chosen instruction mix.  `workgroups` workgroups of `waves` waves (4, 8 or 16: one, two or four per SIMD)
+ * repeat `iters` times a body of 16 slots over which `reads` conflict-free ds_read_b128 (1 KB per
+ * wave each), `mfmas` v_mfma_i32_32x32x32_i8, `dmas` global_load_lds_dwordx4 (1 KB per wave from
+ * global memory straight into LDS) and `gloads` global_load_dwordx4 (1 KB per wave into registers)
+ * are spread evenly.  The global addresses walk over span_bytes (a power of two, at least 64 KB)
+ * behind src, so the span decides which cache serves them.  Only the mixes the measurements use are
+ * instantiated; another one returns MARIAN_HIP_ERR_SHAPE.  split (eight waves only): the first four
+ * waves issue the LDS reads and matrix instructions, the other four the global loads.  The time is
+ * that of the slowest wave.  clocks as for marian_hip_probe_mfma.
+ */
+int marian_hip_probe_mix(const void* src, size_t span_bytes, int waves, int reads, int mfmas, int dmas, int gloads,
+                         int split, int iters, int workgroups, long long* clocks, int* sink, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -27,7 +27,9 @@ extern "C" {
  * the transformer's post-processing (`output + prevInput`, src/models/transformer.h:192-193,207):
  * x = in + add, else x = in.
  * absmax_out: NULL, or MARIAN_HIP_ABSMAX_SLOTS (2048) floats that receive values whose maximum is
- * max|out|, for marian_hip_int8_affine_f32_chained (needs rows <= 2048).
+ * max|out|, for marian_hip_int8_affine_f32_chained.  Up to 2048 rows own a slot each; more rows
+ * (an encoder's sentence batch) share the slots, which a second small kernel of the same call
+ * clears first.
  */
 int marian_hip_layer_norm(const float* in, const float* add, const float* gamma,
                           int64_t gamma_cols, const float* beta, int64_t beta_cols, float* out,

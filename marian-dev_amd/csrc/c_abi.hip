@@ -93,6 +93,25 @@ int launch_stream(const GemmArgs& a, hipStream_t st) {
   return MARIAN_HIP_OK;
 }
 
+// Compute units of the current device (looked up once per device; 256 if the query fails).
+int compute_units() {
+  static std::atomic<int> cus[kMaxDevices];
+  int dev = 0;
+  if(hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 256;
+  int n = cus[dev].load(std::memory_order_relaxed);
+  if(n > 0) return n;
+  if(hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+    n = 256;
+  cus[dev].store(n, std::memory_order_relaxed);
+  return n;
+}
+
+// Whether a large-M launch of `workgroups` workgroups leaves the abs-max of its output itself: one
+// slot per workgroup (not for accumulator dumps).
+inline bool big_leaves_absmax(const GemmArgs& a, long long workgroups) {
+  return a.absmax_out && !a.dump && workgroups <= kAbsmaxSlots;
+}
+
 template <int BM, int BN, int WM, int WN, int NSTAGE, bool PAIRED = true, bool NT = false>
 int launch_big(const GemmArgs& a, hipStream_t st) {
   using Cfg = BigCfg<BM, BN, WM, WN, NSTAGE>;
@@ -115,6 +134,20 @@ int launch_big(const GemmArgs& a, hipStream_t st) {
       return MARIAN_HIP_OK;
     }
   }
+  if constexpr(PAIRED) {
+    if(big_leaves_absmax(a, (long long)tiles_n * tiles_m)) {
+      auto kernel = gemm_mfma32_kernel<BM, BN, WM, WN, NSTAGE, true, NT, false, true>;
+      static std::atomic<uint64_t> amax_lds_done{0};
+      const int lds_status = allow_lds(kernel, Cfg::kLdsBytes, amax_lds_done);
+      if(lds_status != MARIAN_HIP_OK) return lds_status;
+      GemmArgs a2 = a;
+      a2.absmax_used = tiles_n * tiles_m;
+      hipLaunchKernelGGL(kernel, dim3(tiles_n * tiles_m), dim3(Cfg::kThreads), Cfg::kLdsBytes, st, a2, tiles_n, tiles_m);
+      MH_HIP(hipGetLastError());
+      t_absmax_written = true;
+      return MARIAN_HIP_OK;
+    }
+  }
   auto kernel = gemm_mfma32_kernel<BM, BN, WM, WN, NSTAGE, PAIRED, NT>;
   static std::atomic<uint64_t> lds_done{0};
   const int lds_status = allow_lds(kernel, Cfg::kLdsBytes, lds_done);
@@ -125,25 +158,134 @@ int launch_big(const GemmArgs& a, hipStream_t st) {
   return MARIAN_HIP_OK;
 }
 
-// Two side-by-side 256x128 tiles per workgroup, the first written out while the second is multiplied.
-inline bool pair_kernel_fits(const GemmArgs& a) {
-  return !a.dump && !a.idx && a.M % PairCfg::BM == 0 && a.n_out % (2 * PairCfg::BN) == 0 &&
-         a.K % PairCfg::BK == 0 && a.K / PairCfg::BK >= PairCfg::kSideBlocks &&
-         (!a.bias || aligned(a.bias, 16));
+// ---- outputs that are not a whole number of main tiles ----
+// With whole and partial tiles alike (the launchers above) a few rows or columns past a whole number
+// of tiles add a row or column of full-price tiles, and where the whole tiles just fill the chip
+// that is a second round of workgroups: 4100 instead of 4096 rows cost +55 %.  The ragged launch
+// gives the whole main tiles to the first workgroups and covers the rest with small tiles, which
+// run in the slots the main tiles leave or as a short tail.  It is taken when it saves a round.
+struct Ragged {
+  bool use = false;
+  RaggedPlan plan;
+  int workgroups = 0;
+};
+// BM x BN: main tile; EBM x EBN: tiles of the strip below; RBM x RBN: tiles of the strip to the right;
+// per_cu: main workgroups that share a CU; plain_cost: what a tile of the launch that would run
+// otherwise costs relative to a main tile of this one.
+// The choice compares rounds of workgroups: the plain launch needs ceil(all tiles / slots) rounds of
+// main-tile time; the ragged one ceil(whole tiles / slots), its small tiles (a fifth of a main
+// tile's time, measured at K = 1024) running in the slots the whole tiles leave idle and, what
+// does not fit there, as a tail.
+inline Ragged plan_ragged(const GemmArgs& a, int BM, int BN, int EBM, int EBN, int RBM, int RBN, int per_cu,
+                          double plain_cost = 1.0) {
+  Ragged r;
+  const int ov = kernel_override() % 1000;
+  if(a.K % 128 != 0 || ov == 350) return r;   // (measurement id 350: never)
+  const long long cm = (a.M + BM - 1) / BM, cn = (a.n_out + BN - 1) / BN;
+  const long long fm = a.M / BM, fn = a.n_out / BN;
+  const long long slots = (long long)compute_units() * per_cu;
+  if(fm * fn == 0 || fm * fn == cm * cn) return r;
+  const int rows_left = a.M - (int)fm * BM, cols_left = a.n_out - (int)fn * BN;
+  r.plan.main_tiles_n = (int)fn;
+  r.plan.main_tiles_m = (int)fm;
+  r.plan.bottom_tiles_m = (rows_left + EBM - 1) / EBM;
+  r.plan.bottom_tiles_n = rows_left ? (a.n_out + EBN - 1) / EBN : 0;
+  r.plan.right_tiles_n = (cols_left + RBN - 1) / RBN;
+  r.plan.right_tiles_m = cols_left ? ((int)fm * BM + RBM - 1) / RBM : 0;
+  const long long edge = (long long)r.plan.bottom_tiles_m * r.plan.bottom_tiles_n + (long long)r.plan.right_tiles_m * r.plan.right_tiles_n;
+  r.workgroups = (int)(fm * fn + edge);
+  constexpr double kEdgeCost = 0.2;
+  const long long rounds_f = (fm * fn + slots - 1) / slots, rounds_c = (cm * cn + slots - 1) / slots;
+  const long long idle = rounds_f * slots - fm * fn;           // slots the whole tiles leave, a main tile's time each
+  const long long tail = edge - idle * (long long)(1.0 / kEdgeCost);
+  const double ragged_time = (double)rounds_f + (tail > 0 ? (double)((tail + slots - 1) / slots) * kEdgeCost : 0.0);
+  const double plain_time = (double)rounds_c * plain_cost;
+  // (measurement ids 351 and 361 .. 368: whenever there is a whole main tile)
+  r.use = ragged_time + 0.02 < plain_time || ov == 351 || (ov >= 361 && ov <= 368);
+  return r;
 }
 
-template <bool NT>
-int launch_pair(const GemmArgs& a, hipStream_t st) {
-  if(!pair_kernel_fits(a)) return launch_big<256, 256, 2, 4, 2>(a, st);
-  auto kernel = gemm_pair_kernel<NT>;
+// Main tile BM x BN with WM x WN waves; the edge tiles are 64 x 128 below and 128 x 64 to the right,
+// with the same number of waves.
+template <int BM, int BN, int WM, int WN, int NSTAGE, bool NT, bool AMAX>
+int launch_big_ragged_as(const GemmArgs& a, const Ragged& r, hipStream_t st) {
+  constexpr bool eight = WM * WN == 8;
+  constexpr int EWM = 2, EWN = eight ? 4 : 2, ES = 3;              // 64 x 128 (three stages: a small tile's K loop waits for its loads, not for its products)
+  constexpr int RWM = eight ? 4 : 2, RWN = 2, RS = 3;              // 128 x 64
+  using Cfg = BigCfg<BM, BN, WM, WN, NSTAGE>;
+  using ECfg = BigCfg<64, 128, EWM, EWN, ES>;
+  using RCfg = BigCfg<128, 64, RWM, RWN, RS>;
+  constexpr int lds = Cfg::kLdsBytes > ECfg::kLdsBytes ? (Cfg::kLdsBytes > RCfg::kLdsBytes ? Cfg::kLdsBytes : RCfg::kLdsBytes)
+                                                       : (ECfg::kLdsBytes > RCfg::kLdsBytes ? ECfg::kLdsBytes : RCfg::kLdsBytes);
+  auto kernel = gemm_mfma32_ragged_kernel<BM, BN, WM, WN, NSTAGE, 64, 128, EWM, EWN, ES, 128, 64, RWM, RWN, RS, NT, AMAX>;
+  static std::atomic<uint64_t> lds_done{0};
+  const int lds_status = allow_lds(kernel, lds, lds_done);
+  if(lds_status != MARIAN_HIP_OK) return lds_status;
+  GemmArgs a2 = a;
+  a2.absmax_used = r.workgroups;
+  hipLaunchKernelGGL(kernel, dim3(r.workgroups), dim3(Cfg::kThreads), lds, st, a2, r.plan);
+  MH_HIP(hipGetLastError());
+  if(AMAX) t_absmax_written = true;
+  return MARIAN_HIP_OK;
+}
+
+// The launch for a main tile shape: ragged where that saves a round, else whole and partial tiles alike.
+template <int BM, int BN, int WM, int WN, int NSTAGE, bool NT>
+int launch_big_auto(const GemmArgs& a, hipStream_t st, int per_cu) {
+  const Ragged r = plan_ragged(a, BM, BN, 64, 128, 128, 64, per_cu);
+  if(!r.use) return launch_big<BM, BN, WM, WN, NSTAGE, true, NT>(a, st);
+  if(big_leaves_absmax(a, r.workgroups)) return launch_big_ragged_as<BM, BN, WM, WN, NSTAGE, NT, true>(a, r, st);
+  return launch_big_ragged_as<BM, BN, WM, WN, NSTAGE, NT, false>(a, r, st);
+}
+
+// Two side-by-side 256x128 tiles per workgroup, the first written out while the second is multiplied.
+inline bool pair_kernel_ok(const GemmArgs& a) {   // everything but the shape
+  return !a.dump && !a.idx && a.K % PairCfg::BK == 0 && a.K / PairCfg::BK >= PairCfg::kSideBlocks &&
+         (!a.bias || aligned(a.bias, 16));
+}
+inline bool pair_kernel_fits(const GemmArgs& a) {
+  return pair_kernel_ok(a) && a.M % PairCfg::BM == 0 && a.n_out % (2 * PairCfg::BN) == 0;
+}
+
+template <bool NT, bool AMAX>
+int launch_pair_as(const GemmArgs& a, hipStream_t st) {
+  auto kernel = gemm_pair_kernel<NT, AMAX>;
   static std::atomic<uint64_t> lds_done{0};
   const int lds_status = allow_lds(kernel, PairCfg::kLdsBytes, lds_done);
   if(lds_status != MARIAN_HIP_OK) return lds_status;
   int pairs_n = a.n_out / (2 * PairCfg::BN);
   int tiles_m = a.M / PairCfg::BM;
-  hipLaunchKernelGGL(kernel, dim3(pairs_n * tiles_m), dim3(PairCfg::kThreads), PairCfg::kLdsBytes, st, a,
+  GemmArgs a2 = a;
+  a2.absmax_used = pairs_n * tiles_m;
+  hipLaunchKernelGGL(kernel, dim3(pairs_n * tiles_m), dim3(PairCfg::kThreads), PairCfg::kLdsBytes, st, a2,
                      pairs_n, tiles_m);
   MH_HIP(hipGetLastError());
+  if(AMAX) t_absmax_written = true;
+  return MARIAN_HIP_OK;
+}
+
+template <bool NT>
+int launch_pair(const GemmArgs& a, hipStream_t st) {
+  if(!pair_kernel_fits(a)) return launch_big<256, 256, 2, 4, 2>(a, st);
+  if(big_leaves_absmax(a, (long long)(a.n_out / (2 * PairCfg::BN)) * (a.M / PairCfg::BM))) return launch_pair_as<NT, true>(a, st);
+  return launch_pair_as<NT, false>(a, st);
+}
+
+template <bool NT, bool AMAX>
+int launch_pair_ragged_as(const GemmArgs& a, const Ragged& r, hipStream_t st) {
+  using ECfg = BigCfg<64, 128, 2, 2, 3>;
+  using RCfg = BigCfg<128, 64, 2, 2, 3>;
+  constexpr int lds = PairCfg::kLdsBytes > ECfg::kLdsBytes ? (PairCfg::kLdsBytes > RCfg::kLdsBytes ? PairCfg::kLdsBytes : RCfg::kLdsBytes)
+                                                           : (ECfg::kLdsBytes > RCfg::kLdsBytes ? ECfg::kLdsBytes : RCfg::kLdsBytes);
+  auto kernel = gemm_pair_ragged_kernel<NT, AMAX>;
+  static std::atomic<uint64_t> lds_done{0};
+  const int lds_status = allow_lds(kernel, lds, lds_done);
+  if(lds_status != MARIAN_HIP_OK) return lds_status;
+  GemmArgs a2 = a;
+  a2.absmax_used = r.workgroups;
+  hipLaunchKernelGGL(kernel, dim3(r.workgroups), dim3(PairCfg::kThreads), lds, st, a2, r.plan);
+  MH_HIP(hipGetLastError());
+  if(AMAX) t_absmax_written = true;
   return MARIAN_HIP_OK;
 }
 
@@ -155,19 +297,6 @@ inline int stream32_fused_lds_bytes(int mt32, int K) { return mt32 * 32 * K; }
 inline bool stream32_can_fuse(int64_t M, int64_t K) {
   const int mt32 = M <= 32 ? 1 : (M <= 64 ? 2 : 4);
   return M <= 128 && M * K <= kFusedMaxElems && stream32_fused_lds_bytes(mt32, (int)K) <= 64 * 1024;
-}
-
-// Compute units of the current device (looked up once per device; 256 if the query fails).
-int compute_units() {
-  static std::atomic<int> cus[kMaxDevices];
-  int dev = 0;
-  if(hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 256;
-  int n = cus[dev].load(std::memory_order_relaxed);
-  if(n > 0) return n;
-  if(hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
-    n = 256;
-  cus[dev].store(n, std::memory_order_relaxed);
-  return n;
 }
 
 struct FusedSrc {   // what the fused modes read and write besides GemmArgs
@@ -410,6 +539,23 @@ int launch_gemm(const GemmArgs& a, hipStream_t st) {
     case 312: return launch_big<128, 128, 2, 4, 2>(a, st);
     case 313: return launch_big<128, 64, 2, 2, 3>(a, st);
     case 314: return launch_big<128, 64, 4, 2, 2>(a, st);
+    // 361 .. 368: a main tile shape with small tiles for the rest wherever a whole main tile exists
+    // (plain and non-temporal stores); shapes or calls the form does not take fall through
+    case 361: case 365:
+      if(pair_kernel_ok(a)) {
+        const Ragged r = plan_ragged(a, PairCfg::BM, 2 * PairCfg::BN, 64, 128, 128, 64, 1);
+        if(r.use) {
+          if(big_leaves_absmax(a, r.workgroups)) return launch_pair_ragged_as<true, true>(a, r, st);
+          return launch_pair_ragged_as<true, false>(a, r, st);
+        }
+      }
+      break;
+    case 362: return launch_big_auto<256, 256, 2, 4, 2, false>(a, st, 1);
+    case 366: return launch_big_auto<256, 256, 2, 4, 2, true>(a, st, 1);
+    case 363: return launch_big_auto<128, 128, 2, 4, 2, false>(a, st, 2);
+    case 367: return launch_big_auto<128, 128, 2, 4, 2, true>(a, st, 2);
+    case 364: return launch_big_auto<128, 128, 2, 2, 3, false>(a, st, 1);
+    case 368: return launch_big_auto<128, 128, 2, 2, 3, true>(a, st, 1);
     case 501: return launch_stream32_auto<kPrequant>(a, FusedSrc(), st, 0);
     case 521: return launch_stream32_auto<kPrequant>(a, FusedSrc(), st, 0, 1);
     case 522: return launch_stream32_auto<kPrequant>(a, FusedSrc(), st, 0, 2);
@@ -438,23 +584,46 @@ int launch_gemm(const GemmArgs& a, hipStream_t st) {
   const bool stream_out = (long long)a.M * a.n_out * 4 <= (32ll << 20) && !a.dump;
   if(tiles256 >= 192) {
     // short K: the fp32 output is most of the bytes; write one tile out while the next is multiplied
-    if(pair_kernel_fits(a) && a.K <= 1536 && kernel_override() % 1000 != 332)
-      return launch_pair<true>(a, st);
-    if(stream_out) return launch_big<256, 256, 2, 4, 2, true, true>(a, st);
-    return launch_big<256, 256, 2, 4, 2>(a, st);
+    if(a.K <= 1536 && kernel_override() % 1000 != 332) {
+      if(pair_kernel_fits(a)) return launch_pair<true>(a, st);
+      if(pair_kernel_ok(a)) {   // whole tile pairs + small tiles for the rest (the 256x256-tile kernel,
+                                // which would take the output otherwise, is about a tenth slower per tile)
+        const Ragged r = plan_ragged(a, PairCfg::BM, 2 * PairCfg::BN, 64, 128, 128, 64, 1, 1.1);
+        if(r.use) {
+          if(big_leaves_absmax(a, r.workgroups)) return launch_pair_ragged_as<true, true>(a, r, st);
+          return launch_pair_ragged_as<true, false>(a, r, st);
+        }
+      }
+    }
+    if(stream_out) return launch_big_auto<256, 256, 2, 4, 2, true>(a, st, 1);
+    return launch_big_auto<256, 256, 2, 4, 2, false>(a, st, 1);
   }
   // two or more 128x128 tiles per CU: eight waves and two LDS stages, so that two workgroups share
   // a CU and one multiplies while the other writes its tile out; otherwise four waves, three stages
   const long long tiles128 = ((a.M + 127) / 128) * (long long)((a.n_out + 127) / 128);
   if(tiles128 >= 2 * compute_units()) {
-    if(stream_out) return launch_big<128, 128, 2, 4, 2, true, true>(a, st);
-    return launch_big<128, 128, 2, 4, 2>(a, st);
+    if(stream_out) return launch_big_auto<128, 128, 2, 4, 2, true>(a, st, 2);
+    return launch_big_auto<128, 128, 2, 4, 2, false>(a, st, 2);
   }
   // so few 128x128 tiles that half the CUs would idle: 128x64 tiles (measured -20 % to -25 % for
   // M = 512 .. 1024, K = 4096, N = 1024; measurement id 340 keeps the square tiles)
   if(2 * tiles128 <= compute_units() && kernel_override() % 1000 != 340) {
     if(stream_out) return launch_big<128, 64, 2, 2, 3, true, true>(a, st);
     return launch_big<128, 64, 2, 2, 3>(a, st);
+  }
+  // A few rows or columns more than one 128x128 tile per CU: whole tiles plus small ones, by the
+  // eight-wave form, two of whose workgroups share a CU - the small tiles then run beside the whole
+  // ones from the start (measured: 2050 x 1024 x 2056 11.7 instead of 15.4 us with the four-wave form,
+  // whose 96 KB of LDS leave no room for a second workgroup, and 17.3 us with 289 tiles alike).
+  {
+    const Ragged r = plan_ragged(a, 128, 128, 64, 128, 128, 64, 1);
+    if(r.use) {
+      const bool amax = big_leaves_absmax(a, r.workgroups);
+      if(stream_out) return amax ? launch_big_ragged_as<128, 128, 2, 4, 2, true, true>(a, r, st)
+                                 : launch_big_ragged_as<128, 128, 2, 4, 2, true, false>(a, r, st);
+      return amax ? launch_big_ragged_as<128, 128, 2, 4, 2, false, true>(a, r, st)
+                  : launch_big_ragged_as<128, 128, 2, 4, 2, false, false>(a, r, st);
+    }
   }
   if(stream_out) return launch_big<128, 128, 2, 2, 3, true, true>(a, st);
   return launch_big<128, 128, 2, 2, 3>(a, st);
@@ -509,6 +678,27 @@ int absmax_blocks(size_t n4) {
   if(g < 1) g = 1;
   if(g > (size_t)kMaxPartials) g = kMaxPartials;
   return (int)g;
+}
+
+// Quantization of n values whose abs-max the producer left in kAbsmaxSlots slots (measurement id
+// 710 keeps the narrow kernel for large inputs).
+int quantize_with_known_absmax(const float* A, size_t n, const float* absmax_in, int8_t* Aq, hipStream_t st) {
+  if(n >= (1u << 20) && n / 16 <= 0xFFFFFFFFull && kernel_override() % 1000 != 710) {
+    // a 64 KB set per workgroup and step; up to four workgroups' worth of sets per CU at a time
+    const size_t sets = (n / 64 + 255) / 256;
+    size_t blocks = sets;
+    if(blocks > 4 * (size_t)compute_units()) blocks = 4 * (size_t)compute_units();
+    hipLaunchKernelGGL(quantize_a_wide_kernel, dim3((int)blocks), dim3(1024), 0, st, A, (unsigned)(n / 16), absmax_in,
+                       (int)kAbsmaxSlots, Aq);
+    MH_HIP(hipGetLastError());
+    return MARIAN_HIP_OK;
+  }
+  size_t qblocks = (n / 16 + kQuantThreads - 1) / kQuantThreads;
+  if(qblocks > 4096) qblocks = 4096;
+  hipLaunchKernelGGL(quantize_a_kernel, dim3((int)qblocks), dim3(kQuantThreads), 0, st, A, n / 16, absmax_in,
+                     (int)kAbsmaxSlots, Aq);
+  MH_HIP(hipGetLastError());
+  return MARIAN_HIP_OK;
 }
 
 }  // namespace
@@ -567,6 +757,39 @@ int marian_hip_probe_mfma(const void* data, int iters, int workgroups, long long
                      reinterpret_cast<const v4i*>(data), iters, clocks, sink);
   MH_HIP(hipGetLastError());
   return MARIAN_HIP_OK;
+}
+
+int marian_hip_probe_mix(const void* src, size_t span_bytes, int waves, int reads, int mfmas, int dmas, int gloads,
+                         int split, int iters, int workgroups, long long* clocks, int* sink, void* stream) {
+  if(!src || !clocks || !sink) return MARIAN_HIP_ERR_NULL;
+  if(iters <= 0 || workgroups <= 0 || (waves != 4 && waves != 8 && waves != 16)) return MARIAN_HIP_ERR_SHAPE;
+  if((mfmas > 0 && waves > 8) || (split && waves != 8)) return MARIAN_HIP_ERR_SHAPE;
+  if(span_bytes < 65536 || (span_bytes & (span_bytes - 1)) != 0 || span_bytes > (1ull << 31)) return MARIAN_HIP_ERR_SHAPE;
+  if(!aligned(src, 16)) return MARIAN_HIP_ERR_ALIGN;
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  constexpr int kLds = 128 * 1024;
+#define MH_MIX(R, M, D, G) MH_MIX2(R, M, D, G, false)
+#define MH_MIX2(R, M, D, G, S)                                                                                  \
+  if(reads == R && mfmas == M && dmas == D && gloads == G && (split != 0) == S) {                              \
+    auto kernel = probe_mix_kernel<R, M, D, G, S>;                                                             \
+    static std::atomic<uint64_t> lds_done{0};                                                                  \
+    const int lds_status = allow_lds(kernel, kLds, lds_done);                                                  \
+    if(lds_status != MARIAN_HIP_OK) return lds_status;                                                         \
+    hipLaunchKernelGGL(kernel, dim3(workgroups), dim3(waves * 64), kLds, st, reinterpret_cast<const int8_t*>(src), \
+                       (unsigned)span_bytes, iters, clocks, sink);                                             \
+    MH_HIP(hipGetLastError());                                                                                 \
+    return MARIAN_HIP_OK;                                                                                      \
+  }
+  MH_MIX(16, 0, 0, 0) MH_MIX(16, 0, 8, 0) MH_MIX(16, 0, 4, 0)
+  MH_MIX(0, 0, 16, 0) MH_MIX(0, 0, 0, 16) MH_MIX(0, 0, 8, 8)
+  MH_MIX(0, 8, 0, 0) MH_MIX(4, 8, 0, 0) MH_MIX(6, 8, 0, 0) MH_MIX(8, 8, 0, 0) MH_MIX(12, 8, 0, 0) MH_MIX(16, 8, 0, 0)
+  MH_MIX(0, 8, 4, 0) MH_MIX(0, 8, 8, 0) MH_MIX(0, 8, 0, 4) MH_MIX(0, 8, 0, 8)
+  MH_MIX(8, 8, 4, 0) MH_MIX(6, 8, 3, 0) MH_MIX(6, 8, 2, 0) MH_MIX(4, 8, 1, 2) MH_MIX(4, 8, 2, 2) MH_MIX(4, 8, 2, 4)
+  MH_MIX2(8, 8, 4, 0, true) MH_MIX2(6, 8, 3, 0, true) MH_MIX2(0, 8, 4, 0, true) MH_MIX2(8, 8, 3, 0, true)
+  MH_MIX(8, 8, 3, 0) MH_MIX(8, 8, 2, 0) MH_MIX2(8, 8, 2, 0, true) MH_MIX(12, 8, 4, 0)
+#undef MH_MIX
+#undef MH_MIX2
+  return MARIAN_HIP_ERR_SHAPE;   // (a mix that is not instantiated)
 }
 #endif
 
@@ -735,12 +958,8 @@ static int affine_f32_impl(const float* A, int8_t* Aq, const int8_t* Bq, const f
     return launch_stream32_auto<kFusedTiled>(a, f, hst, want_tiled ? which - 620 : 0);
   }
   if(absmax_in) {   // quantize with the abs-max the producer left, then the GEMM
-    const size_t n = (size_t)M * (size_t)K;
-    size_t qblocks = (n / 16 + kQuantThreads - 1) / kQuantThreads;
-    if(qblocks > 4096) qblocks = 4096;
-    hipLaunchKernelGGL(quantize_a_kernel, dim3((int)qblocks), dim3(kQuantThreads), 0, hst, A, n / 16,
-                       absmax_in, (int)kAbsmaxSlots, Aq);
-    MH_HIP(hipGetLastError());
+    st = quantize_with_known_absmax(A, (size_t)M * (size_t)K, absmax_in, Aq, hst);
+    if(st != MARIAN_HIP_OK) return st;
   } else {
     st = marian_hip_int8_prepare_a(A, Aq, M, K, workspace, workspace_bytes, stream);
     if(st != MARIAN_HIP_OK) return st;
@@ -853,12 +1072,8 @@ int marian_hip_int8_affine_f32_grouped(const float* A, int8_t* Aq, int64_t n_gro
   }
   // Otherwise the activations are quantized once and every matrix gets its own multiplication.
   if(absmax_in) {
-    const size_t n = (size_t)M * (size_t)K;
-    size_t qblocks = (n / 16 + kQuantThreads - 1) / kQuantThreads;
-    if(qblocks > 4096) qblocks = 4096;
-    hipLaunchKernelGGL(quantize_a_kernel, dim3((int)qblocks), dim3(kQuantThreads), 0, hst, A, n / 16, absmax_in,
-                       (int)kAbsmaxSlots, Aq);
-    MH_HIP(hipGetLastError());
+    int st = quantize_with_known_absmax(A, (size_t)M * (size_t)K, absmax_in, Aq, hst);
+    if(st != MARIAN_HIP_OK) return st;
   } else {
     int st = marian_hip_int8_prepare_a(A, Aq, M, K, workspace, workspace_bytes, stream);
     if(st != MARIAN_HIP_OK) return st;
@@ -914,8 +1129,12 @@ int marian_hip_int8_affine_f32_static(const float* A, const int8_t* Bq, const fl
   if(st != MARIAN_HIP_OK) return st;
   int8_t* Aq = reinterpret_cast<int8_t*>(base);
   void* workspace = base + kStaticAqBytes;
-  // every byte the kernels read from the array was written earlier in the same call (the
-  // activations by the quantizer, the partials by the abs-max pass): nothing has to start at zero
+  // The quantized activations and the abs-max partials are written earlier in the same call than
+  // they are read.  The hand-over area of the one-pass prepareA (M * K >= 4 Mi: arrival slots,
+  // generation word, mailboxes) is different: its words persist from call to call and are matched
+  // by tag (a per-process nonce plus the generation word, top bit always set), so a word left by
+  // an earlier call - or the zeros the array starts with - never passes for a fresh one.  Nothing
+  // has to be cleared between calls.
   return affine_f32_impl(A, Aq, Bq, bias, idx, n_idx, out, M, K, N, scale, relu, nullptr, nullptr,
                          workspace, kWorkspaceBytes, stream);
 }

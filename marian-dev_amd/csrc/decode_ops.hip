@@ -102,7 +102,7 @@ __global__ __launch_bounds__(256) void layer_norm_kernel(const float* in,
                                                          const float* __restrict__ gamma, int gamma_stride,
                                                          const float* __restrict__ beta, int beta_stride,
                                                          float* out, int cols, float eps,
-                                                         float* __restrict__ absmax_out) {
+                                                         float* __restrict__ absmax_out, int absmax_wrap) {
   __shared__ float red[4];
   float omax = 0.0f;   // max |y| over what this thread writes
   const size_t row = blockIdx.x;
@@ -180,9 +180,15 @@ __global__ __launch_bounds__(256) void layer_norm_kernel(const float* in,
   }
   if(absmax_out) {   // slot `row`; workgroup 0 zeroes the slots past the last row
     omax = row_reduce<256, true>(omax, red);
-    if(tid == 0) absmax_out[row] = omax;
-    if(row == 0)
-      for(int sl = gridDim.x + tid; sl < kAbsmaxSlots; sl += 256) absmax_out[sl] = 0.0f;
+    if(absmax_wrap) {
+      // more rows than slots: the rows share the slots (cleared by the launcher) through an integer
+      // maximum on the bits, which orders non-negative floats as the floats themselves
+      if(tid == 0) atomicMax(reinterpret_cast<int*>(absmax_out) + (int)(row % kAbsmaxSlots), __float_as_int(omax));
+    } else {
+      if(tid == 0) absmax_out[row] = omax;
+      if(row == 0)
+        for(int sl = gridDim.x + tid; sl < kAbsmaxSlots; sl += 256) absmax_out[sl] = 0.0f;
+    }
   }
 }
 
@@ -193,7 +199,7 @@ __global__ __launch_bounds__(64) void layer_norm_wave_kernel(const float* in, co
                                                              const float* __restrict__ gamma, int gamma_stride,
                                                              const float* __restrict__ beta, int beta_stride,
                                                              float* out, int cols, float eps,
-                                                             float* __restrict__ absmax_out) {
+                                                             float* __restrict__ absmax_out, int absmax_wrap) {
   constexpr int VPL = 4;
   const size_t row = blockIdx.x;
   const int lane = threadIdx.x, cols4 = cols / 4;
@@ -256,8 +262,12 @@ __global__ __launch_bounds__(64) void layer_norm_wave_kernel(const float* in, co
   }
   if(absmax_out) {   // slot `row`; the slots past the last row are zeroed by all workgroups together
     omax = wave_maxf(omax);
-    if(lane == 0) absmax_out[row] = omax;
-    for(int sl = (int)gridDim.x + (int)row * 64 + lane; sl < kAbsmaxSlots; sl += (int)gridDim.x * 64) absmax_out[sl] = 0.0f;
+    if(absmax_wrap) {   // more rows than slots, see layer_norm_kernel
+      if(lane == 0) atomicMax(reinterpret_cast<int*>(absmax_out) + (int)(row % kAbsmaxSlots), __float_as_int(omax));
+    } else {
+      if(lane == 0) absmax_out[row] = omax;
+      for(int sl = (int)gridDim.x + (int)row * 64 + lane; sl < kAbsmaxSlots; sl += (int)gridDim.x * 64) absmax_out[sl] = 0.0f;
+    }
   }
 }
 
@@ -1386,7 +1396,6 @@ extern "C" {
 int marian_hip_layer_norm(const float* in, const float* add, const float* gamma, int64_t gamma_cols,
                           const float* beta, int64_t beta_cols, float* out, int64_t rows,
                           int64_t cols, float eps, float* absmax_out, void* stream) {
-  if(absmax_out && rows > kAbsmaxSlots) return MARIAN_HIP_ERR_RANGE;
   if(absmax_out && !aligned4(absmax_out)) return MARIAN_HIP_ERR_ALIGN;
   if(rows < 0 || cols <= 0) return MARIAN_HIP_ERR_SHAPE;
   if((gamma_cols != cols && gamma_cols != 1) || (beta && beta_cols != cols && beta_cols != 1))
@@ -1401,16 +1410,24 @@ int marian_hip_layer_norm(const float* in, const float* add, const float* gamma,
   const bool vec = cols % 4 == 0 && aligned16(in) && aligned16(out) && (!add || aligned16(add));
   const bool wave_form = vec && cols <= 1024 && (gs == 0 || aligned16(gamma)) &&
                          (!beta || bs == 0 || aligned16(beta));
+  // more rows than abs-max slots (an encoder's sentence batch): the rows share the slots, which are
+  // cleared first (a kernel, so that the call may sit in a recorded graph)
+  const int wrap = absmax_out && rows > kAbsmaxSlots ? 1 : 0;
+  if(wrap) {
+    hipLaunchKernelGGL(zero_words_kernel, dim3(kAbsmaxSlots / 256), dim3(256), 0, st, reinterpret_cast<unsigned*>(absmax_out),
+                       (long long)kAbsmaxSlots);
+    MH_HIP(hipGetLastError());
+  }
   if(wave_form)
-    hipLaunchKernelGGL(layer_norm_wave_kernel, dim3((unsigned)rows), dim3(64), 0, st, in, add, gamma, gs, beta, bs, out, (int)cols, eps, absmax_out);
+    hipLaunchKernelGGL(layer_norm_wave_kernel, dim3((unsigned)rows), dim3(64), 0, st, in, add, gamma, gs, beta, bs, out, (int)cols, eps, absmax_out, wrap);
   else if(vec && cols <= 1024)
-    hipLaunchKernelGGL(layer_norm_kernel<1>, dim3((unsigned)rows), dim3(256), 0, st, in, add, gamma, gs, beta, bs, out, (int)cols, eps, absmax_out);
+    hipLaunchKernelGGL(layer_norm_kernel<1>, dim3((unsigned)rows), dim3(256), 0, st, in, add, gamma, gs, beta, bs, out, (int)cols, eps, absmax_out, wrap);
   else if(vec && cols <= 4096)
-    hipLaunchKernelGGL(layer_norm_kernel<4>, dim3((unsigned)rows), dim3(256), 0, st, in, add, gamma, gs, beta, bs, out, (int)cols, eps, absmax_out);
+    hipLaunchKernelGGL(layer_norm_kernel<4>, dim3((unsigned)rows), dim3(256), 0, st, in, add, gamma, gs, beta, bs, out, (int)cols, eps, absmax_out, wrap);
   else if(vec && cols <= 8192)
-    hipLaunchKernelGGL(layer_norm_kernel<8>, dim3((unsigned)rows), dim3(256), 0, st, in, add, gamma, gs, beta, bs, out, (int)cols, eps, absmax_out);
+    hipLaunchKernelGGL(layer_norm_kernel<8>, dim3((unsigned)rows), dim3(256), 0, st, in, add, gamma, gs, beta, bs, out, (int)cols, eps, absmax_out, wrap);
   else
-    hipLaunchKernelGGL(layer_norm_kernel<0>, dim3((unsigned)rows), dim3(256), 0, st, in, add, gamma, gs, beta, bs, out, (int)cols, eps, absmax_out);
+    hipLaunchKernelGGL(layer_norm_kernel<0>, dim3((unsigned)rows), dim3(256), 0, st, in, add, gamma, gs, beta, bs, out, (int)cols, eps, absmax_out, wrap);
   MH_HIP(hipGetLastError());
   return MARIAN_HIP_OK;
 }

@@ -25,6 +25,7 @@
 #include <type_traits>
 
 #include "int8_common.h"
+#include "quantize_kernels.h"
 
 namespace marian_hip {
 
@@ -107,10 +108,12 @@ __device__ __forceinline__ void store_tile32(const v16i& acc, char* out, size_t 
 // wave cover WTN * 128 contiguous bytes of an output row (measured on the store burst alone: tile
 // after tile is 50 % slower).  `out` points at this lane's element of row 4*(lane/32) of the first
 // tile; tile b starts 128 bytes further per b.
-template <int WTN, bool DUMP, bool BIAS, bool RELU, bool GUARD, bool NT>
+// AMAX: also keeps the maximum of |y| over what this lane stores in `omax` (one more vector
+// operation per value; only calls that hand their abs-max to the next call ask for it).
+template <int WTN, bool DUMP, bool BIAS, bool RELU, bool GUARD, bool NT, bool AMAX>
 __device__ __forceinline__ void store_tiles32_rowwise(const v16i (&acc)[WTN], char* out, size_t row_bytes,
                                                       float unquant, const float (&bias_v)[WTN],
-                                                      int rows_left, const bool (&col_valid)[WTN]) {
+                                                      int rows_left, const bool (&col_valid)[WTN], float& omax) {
 #pragma unroll
   for(int v = 0; v < 16; ++v) {
     const int r = 8 * (v / 4) + (v % 4);
@@ -126,6 +129,7 @@ __device__ __forceinline__ void store_tiles32_rowwise(const v16i (&acc)[WTN], ch
         float y = (float)acc[b][v] * unquant;
         if(BIAS) y = y + bias_v[b];
         if(RELU) y = y > 0.0f ? y : 0.0f;
+        if(AMAX) omax = fmaxf(omax, fabsf(y));
         if(NT) __builtin_nontemporal_store(y, reinterpret_cast<float*>(p));
         else *reinterpret_cast<float*>(p) = y;
       }
@@ -133,16 +137,16 @@ __device__ __forceinline__ void store_tiles32_rowwise(const v16i (&acc)[WTN], ch
   }
 }
 
-template <int WTN, bool GUARD, bool NT>
+template <int WTN, bool GUARD, bool NT, bool AMAX>
 __device__ __forceinline__ void store_tiles32_rowwise_any(const v16i (&acc)[WTN], char* out, size_t row_bytes,
                                                           float unquant, const float (&bias_v)[WTN],
                                                           int rows_left, const bool (&col_valid)[WTN],
-                                                          int dump, bool bias, int relu) {
-  if(dump) store_tiles32_rowwise<WTN, true, false, false, GUARD, NT>(acc, out, row_bytes, unquant, bias_v, rows_left, col_valid);
-  else if(bias && relu) store_tiles32_rowwise<WTN, false, true, true, GUARD, NT>(acc, out, row_bytes, unquant, bias_v, rows_left, col_valid);
-  else if(bias) store_tiles32_rowwise<WTN, false, true, false, GUARD, NT>(acc, out, row_bytes, unquant, bias_v, rows_left, col_valid);
-  else if(relu) store_tiles32_rowwise<WTN, false, false, true, GUARD, NT>(acc, out, row_bytes, unquant, bias_v, rows_left, col_valid);
-  else store_tiles32_rowwise<WTN, false, false, false, GUARD, NT>(acc, out, row_bytes, unquant, bias_v, rows_left, col_valid);
+                                                          int dump, bool bias, int relu, float& omax) {
+  if(dump) store_tiles32_rowwise<WTN, true, false, false, GUARD, NT, false>(acc, out, row_bytes, unquant, bias_v, rows_left, col_valid, omax);
+  else if(bias && relu) store_tiles32_rowwise<WTN, false, true, true, GUARD, NT, AMAX>(acc, out, row_bytes, unquant, bias_v, rows_left, col_valid, omax);
+  else if(bias) store_tiles32_rowwise<WTN, false, true, false, GUARD, NT, AMAX>(acc, out, row_bytes, unquant, bias_v, rows_left, col_valid, omax);
+  else if(relu) store_tiles32_rowwise<WTN, false, false, true, GUARD, NT, AMAX>(acc, out, row_bytes, unquant, bias_v, rows_left, col_valid, omax);
+  else store_tiles32_rowwise<WTN, false, false, false, GUARD, NT, AMAX>(acc, out, row_bytes, unquant, bias_v, rows_left, col_valid, omax);
 }
 
 template <bool GUARD>
@@ -166,12 +170,48 @@ __device__ __forceinline__ void store_tile32_any(const v16i& acc, char* out, siz
 // does not fit anyway and is 2 % slower with them).
 // HALF: K is a multiple of 64 but not of 128, the last block holds 64 columns (an instantiation of
 // its own, so that whole-block calls run code without the checks).
+// XCD-aware tile order: workgroups of one XCD (ids congruent mod 8 under round-robin dispatch)
+// take a compact block of tiles - 4 tiles along n by a run along m - so that the XCD's L2 holds
+// few weight panels and few activation panels at a time.
+__device__ __forceinline__ void xcd_tile(int tiles_n, int tiles_m, int block, int& tn, int& tm) {
+  const int total = tiles_n * tiles_m;
+  int t = block;
+  if(total % 8 == 0) t = (block % 8) * (total / 8) + block / 8;
+  const int band = 4;
+  const int b = t / (band * tiles_m);
+  const int r = t % (band * tiles_m);
+  const int bw = (tiles_n - b * band) < band ? (tiles_n - b * band) : band;
+  tn = b * band + r % bw;
+  tm = r / bw;
+}
+
+// Abs-max hand-over of a large-M launch: slot `slot` receives the maximum of |y| over the tile this
+// workgroup stored (omax: this lane's share), the workgroup of slot 0 zeroes the slots past the
+// `used` ones the launch fills.  red: the LDS ring, free once every wave is past its last fragment
+// read (the first barrier).  All threads of the workgroup call it.
+__device__ __forceinline__ void publish_tile_absmax(float omax, float* absmax_out, int slot, int used, float* red) {
+  const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave, nw = blockDim.x / kWave;
+  omax = wave_max(omax);
+  __syncthreads();
+  if(lane == 0) red[wave] = omax;
+  __syncthreads();
+  if(tid == 0) {
+    float m = red[0];
+    for(int w = 1; w < nw; ++w) m = fmaxf(m, red[w]);
+    absmax_out[slot] = m;
+  }
+  if(slot == 0)
+    for(int sl = used + tid; sl < kAbsmaxSlots; sl += (int)blockDim.x) absmax_out[sl] = 0.0f;
+}
+
+// One BM x BN output tile at rows m0 .., columns n0 .. (any multiples of 32; the tile may hang over
+// the edge of the output).  slot: the workgroup's number among the tiles of the launch (abs-max
+// slot, clock record).
 template <int BM, int BN, int WAVES_M, int WAVES_N, int NSTAGE, bool PAIRED = true, bool NT = false,
-          bool HALF = false>
-__global__ __launch_bounds__(WAVES_M * WAVES_N * kWave) void gemm_mfma32_kernel(
-    GemmArgs args, int tiles_n, int tiles_m) {
+          bool HALF = false, bool AMAX = false>
+__device__ __forceinline__ void gemm_mfma32_tile(const GemmArgs& args, const int m0, const int n0, int8_t* lds,
+                                                 const int slot) {
   using Cfg = BigCfg<BM, BN, WAVES_M, WAVES_N, NSTAGE>;
-  extern __shared__ __attribute__((aligned(16))) int8_t lds[];
   const unsigned lds_base = (unsigned)(size_t)lds;  // LDS byte address of the ring
 
   const long long t_start = MH_CLOCK();
@@ -187,23 +227,6 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * kWave) void gemm_mfma32_kernel(
   static_assert(!HALF || (PAIRED && Cfg::kHalfTailOk), "no half last block in this form");
   const int KB = HALF ? (K + Cfg::BK - 1) / Cfg::BK : K / Cfg::BK;
   constexpr bool half_tail = HALF;
-
-  int tn, tm;
-  {
-    // Workgroups of one XCD (ids congruent mod 8 under round-robin dispatch) take a compact
-    // block of tiles - 4 tiles along n by a run along m - so that the XCD's L2 holds few weight
-    // panels and few activation panels at a time.
-    const int total = tiles_n * tiles_m;
-    int t = blockIdx.x;
-    if(total % 8 == 0) t = (blockIdx.x % 8) * (total / 8) + blockIdx.x / 8;
-    const int band = 4;
-    const int b = t / (band * tiles_m);
-    const int r = t % (band * tiles_m);
-    const int bw = (tiles_n - b * band) < band ? (tiles_n - b * band) : band;
-    tn = b * band + r % bw;
-    tm = r / bw;
-  }
-  const int m0 = tm * BM, n0 = tn * BN;
 
   // ---- global -> LDS: load j of this wave fills rows (j*kWaves + wave)*8 .. +7 of a stage.
   // Rows past the matrix edge re-read the last valid row; their products are never stored.
@@ -460,19 +483,68 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * kWave) void gemm_mfma32_kernel(
 #pragma unroll
     for(int b = 0; b < Cfg::WTN; ++b) asm volatile("" ::"v"(bias_v[b]));
     asm volatile("" ::"v"(unquant));
+    float omax = 0.0f;
 #pragma unroll
     for(int a = 0; a < Cfg::WTM; ++a) {
       const int mbase = m0 + (wm * Cfg::WTM + a) * 32 + 4 * lg;
       char* outp = reinterpret_cast<char*>(args.out) + ((size_t)mbase * (size_t)args.n_out + (size_t)nw) * 4;
       if(interior)
-        store_tiles32_rowwise_any<Cfg::WTN, false, NT>(acc[a], outp, row_bytes, unquant, bias_v, 32, nvalid, args.dump, has_bias, args.relu);
+        store_tiles32_rowwise_any<Cfg::WTN, false, NT, AMAX>(acc[a], outp, row_bytes, unquant, bias_v, 32, nvalid, args.dump, has_bias, args.relu, omax);
       else
-        store_tiles32_rowwise_any<Cfg::WTN, true, NT>(acc[a], outp, row_bytes, unquant, bias_v, M - mbase, nvalid, args.dump, has_bias, args.relu);
+        store_tiles32_rowwise_any<Cfg::WTN, true, NT, AMAX>(acc[a], outp, row_bytes, unquant, bias_v, M - mbase, nvalid, args.dump, has_bias, args.relu, omax);
     }
+    if(AMAX && args.absmax_out && !args.dump)
+      publish_tile_absmax(omax, args.absmax_out, slot, args.absmax_used, reinterpret_cast<float*>(lds));
   }
   if(MH_PROF(args) && tid == 0) {
-    long long* p = MH_PROF(args) + (size_t)blockIdx.x * 8;
+    long long* p = MH_PROF(args) + (size_t)slot * 8;
     p[0] = t_start; p[1] = t_prologue; p[2] = t_main; p[3] = MH_CLOCK(); p[6] = w_start; p[7] = MH_WALL();
+  }
+}
+
+template <int BM, int BN, int WAVES_M, int WAVES_N, int NSTAGE, bool PAIRED = true, bool NT = false,
+          bool HALF = false, bool AMAX = false>
+__global__ __launch_bounds__(WAVES_M * WAVES_N * kWave) void gemm_mfma32_kernel(
+    GemmArgs args, int tiles_n, int tiles_m) {
+  extern __shared__ __attribute__((aligned(16))) int8_t lds[];
+  int tn, tm;
+  xcd_tile(tiles_n, tiles_m, blockIdx.x, tn, tm);
+  gemm_mfma32_tile<BM, BN, WAVES_M, WAVES_N, NSTAGE, PAIRED, NT, HALF, AMAX>(args, tm * BM, tn * BN, lds, blockIdx.x);
+}
+
+// A launch whose output is not a whole number of main tiles: `main_tiles` whole BM x BN tiles
+// (the first workgroups, in the XCD-aware order), then small tiles over the rows below them (EBM x
+// EBN tiles: a strip `bottom_tiles_n` tiles wide over all columns, starting at row main_tiles_m * BM)
+// and over the columns to their right (RBM x RBN tiles, `right_tiles_m` tiles high, starting at
+// column main_tiles_n * BN, over the rows of the main tiles).  The few rows or columns past a whole
+// number of main tiles then cost a short tail of small tiles instead of a second round of large
+// ones.  All three tile shapes run with the same number of waves.
+struct RaggedPlan {
+  int main_tiles_n, main_tiles_m;
+  int bottom_tiles_n, bottom_tiles_m;   // EBM x EBN tiles below the main tiles (all columns)
+  int right_tiles_n, right_tiles_m;     // RBM x RBN tiles to the right of the main tiles (main rows only)
+};
+
+template <int BM, int BN, int WAVES_M, int WAVES_N, int NSTAGE, int EBM, int EBN, int EWM, int EWN, int ESTAGE,
+          int RBM, int RBN, int RWM, int RWN, int RSTAGE, bool NT = false, bool AMAX = false>
+__global__ __launch_bounds__(WAVES_M * WAVES_N * kWave) void gemm_mfma32_ragged_kernel(GemmArgs args, RaggedPlan plan) {
+  static_assert(WAVES_M * WAVES_N == EWM * EWN && WAVES_M * WAVES_N == RWM * RWN, "one workgroup size");
+  extern __shared__ __attribute__((aligned(16))) int8_t lds[];
+  const int block = blockIdx.x;
+  const int n_main = plan.main_tiles_n * plan.main_tiles_m;
+  const int n_bottom = plan.bottom_tiles_n * plan.bottom_tiles_m;
+  if(block < n_main) {
+    int tn, tm;
+    xcd_tile(plan.main_tiles_n, plan.main_tiles_m, block, tn, tm);
+    gemm_mfma32_tile<BM, BN, WAVES_M, WAVES_N, NSTAGE, true, NT, false, AMAX>(args, tm * BM, tn * BN, lds, block);
+  } else if(block < n_main + n_bottom) {
+    const int t = block - n_main;
+    const int tn = t % plan.bottom_tiles_n, tm = t / plan.bottom_tiles_n;
+    gemm_mfma32_tile<EBM, EBN, EWM, EWN, ESTAGE, true, NT, false, AMAX>(args, plan.main_tiles_m * BM + tm * EBM, tn * EBN, lds, block);
+  } else {
+    const int t = block - n_main - n_bottom;
+    const int tm = t % plan.right_tiles_m, tn = t / plan.right_tiles_m;
+    gemm_mfma32_tile<RBM, RBN, RWM, RWN, RSTAGE, true, NT, false, AMAX>(args, tm * RBM, plan.main_tiles_n * BN + tn * RBN, lds, block);
   }
 }
 

@@ -65,12 +65,14 @@ constexpr int pair_younger_ops(int kbi) {
   return n;
 }
 
-template <bool NT>
-__global__ __launch_bounds__(PairCfg::kThreads) void gemm_pair_kernel(GemmArgs args, int pairs_n,
-                                                                      int tiles_m) {
+// The two tiles at rows m0 .., columns n0 .. and n0 + 128 .. (whole tiles inside the output).
+// slot: the workgroup's number among the workgroups of the launch (abs-max slot, clock record).
+// AMAX: the workgroup leaves the maximum of |y| over its two tiles in args.absmax_out[slot].
+template <bool NT, bool AMAX>
+__device__ __forceinline__ void gemm_pair_tiles(const GemmArgs& args, const int m0, const int n0, int8_t* lds,
+                                                const int slot) {
   using Cfg = PairCfg;
   constexpr int BM = Cfg::BM, BN = Cfg::BN, NSTAGE = Cfg::NSTAGE;
-  extern __shared__ __attribute__((aligned(16))) int8_t lds[];
   const unsigned lds_base = (unsigned)(size_t)lds;
 
   const long long t_start = MH_CLOCK();
@@ -83,22 +85,6 @@ __global__ __launch_bounds__(PairCfg::kThreads) void gemm_pair_kernel(GemmArgs a
   const int K = args.K;
   const int KB = K / Cfg::BK;
   const int total_blocks = 2 * KB;
-
-
-  int tn, tm;
-  {
-    // Workgroups of one XCD (ids congruent mod 8) take a compact block of tile pairs.
-    const int total = pairs_n * tiles_m;
-    int t = blockIdx.x;
-    if(total % 8 == 0) t = (blockIdx.x % 8) * (total / 8) + blockIdx.x / 8;
-    const int band = 4;
-    const int b = t / (band * tiles_m);
-    const int r = t % (band * tiles_m);
-    const int bw = (pairs_n - b * band) < band ? (pairs_n - b * band) : band;
-    tn = b * band + r % bw;
-    tm = r / bw;
-  }
-  const int m0 = tm * BM, n0 = tn * 2 * BN;   // n0: first column of the first tile of the pair
 
   // ---- global -> LDS: activation load j of this wave fills rows (j*4 + wave)*8 .. +7 of a stage;
   //      weight load g = (j - kLoadsA) * 4 + wave brings the 1 KB block (sub-step g / 4, column tile
@@ -157,6 +143,7 @@ __global__ __launch_bounds__(PairCfg::kThreads) void gemm_pair_kernel(GemmArgs a
   v16i acc[2][Cfg::WTM][Cfg::WTN];
   float bias0[Cfg::WTN], bias1[Cfg::WTN];   // this lane's columns of the first and of the second tile
   float unquant;
+  float omax = 0.0f;                        // AMAX: max |y| over what this lane has stored
 
   // value v (0..127) of the first tile, row by row across the two side-by-side accumulator tiles
   auto side_store = [&](int v) __attribute__((always_inline)) {
@@ -165,6 +152,7 @@ __global__ __launch_bounds__(PairCfg::kThreads) void gemm_pair_kernel(GemmArgs a
     float y = (float)acc[0][a][b][e] * unquant;
     y = y + bias0[b];
     y = fmaxf(y, relu_floor);
+    if(AMAX) omax = fmaxf(omax, fabsf(y));
     global_store_f32<NT>(out_base0 + (size_t)r * row_bytes + b * 128, out_voff, y);
   };
 
@@ -281,12 +269,47 @@ __global__ __launch_bounds__(PairCfg::kThreads) void gemm_pair_kernel(GemmArgs a
       float y = (float)acc[1][a][b][e] * unquant;
       y = y + bias1[b];
       y = fmaxf(y, relu_floor);
+      if(AMAX) omax = fmaxf(omax, fabsf(y));
       global_store_f32<NT>(out_base1 + (size_t)r * row_bytes + b * 128, out_voff, y);
     }
   }
+  if(AMAX && args.absmax_out)
+    publish_tile_absmax(omax, args.absmax_out, slot, args.absmax_used, reinterpret_cast<float*>(lds));
   if(MH_PROF(args) && tid == 0) {
-    long long* p = MH_PROF(args) + (size_t)blockIdx.x * 8;
+    long long* p = MH_PROF(args) + (size_t)slot * 8;
     p[0] = t_start; p[1] = t_prologue; p[2] = t_main; p[3] = MH_CLOCK(); p[4] = t_main; p[5] = t_side; p[6] = w_start; p[7] = MH_WALL();
+  }
+}
+
+template <bool NT, bool AMAX = false>
+__global__ __launch_bounds__(PairCfg::kThreads) void gemm_pair_kernel(GemmArgs args, int pairs_n, int tiles_m) {
+  extern __shared__ __attribute__((aligned(16))) int8_t lds[];
+  int tn, tm;
+  xcd_tile(pairs_n, tiles_m, blockIdx.x, tn, tm);   // a compact block of tile pairs per XCD
+  gemm_pair_tiles<NT, AMAX>(args, tm * PairCfg::BM, tn * 2 * PairCfg::BN, lds, blockIdx.x);
+}
+
+// The same for an output that is not a whole number of tile pairs: pairs over the whole 256 x 256
+// blocks, then 64 x 128 tiles over the rows below them and 128 x 64 tiles over the columns to their
+// right (see RaggedPlan; main_tiles_n counts pairs).
+template <bool NT, bool AMAX = false>
+__global__ __launch_bounds__(PairCfg::kThreads) void gemm_pair_ragged_kernel(GemmArgs args, RaggedPlan plan) {
+  extern __shared__ __attribute__((aligned(16))) int8_t lds[];
+  const int block = blockIdx.x;
+  const int n_main = plan.main_tiles_n * plan.main_tiles_m;
+  const int n_bottom = plan.bottom_tiles_n * plan.bottom_tiles_m;
+  if(block < n_main) {
+    int tn, tm;
+    xcd_tile(plan.main_tiles_n, plan.main_tiles_m, block, tn, tm);
+    gemm_pair_tiles<NT, AMAX>(args, tm * PairCfg::BM, tn * 2 * PairCfg::BN, lds, block);
+  } else if(block < n_main + n_bottom) {
+    const int t = block - n_main;
+    const int tn = t % plan.bottom_tiles_n, tm = t / plan.bottom_tiles_n;
+    gemm_mfma32_tile<64, 128, 2, 2, 3, true, NT, false, AMAX>(args, plan.main_tiles_m * PairCfg::BM + tm * 64, tn * 128, lds, block);
+  } else {
+    const int t = block - n_main - n_bottom;
+    const int tm = t % plan.right_tiles_m, tn = t / plan.right_tiles_m;
+    gemm_mfma32_tile<128, 64, 2, 2, 3, true, NT, false, AMAX>(args, tm * 128, plan.main_tiles_n * 2 * PairCfg::BN + tn * 64, lds, block);
   }
 }
 

@@ -221,8 +221,13 @@ int marian_hip_int16_prepare_b(const float* W, int16_t* Bq, int64_t K, int64_t N
 
 int marian_hip_int16_prepare_b_quantized_transposed(const int16_t* in, int16_t* out, int64_t K, int64_t N, void* stream) {
   if(!in || !out) return MARIAN_HIP_ERR_NULL;
-  if(K <= 0 || N <= 0) return MARIAN_HIP_ERR_SHAPE;
-  if(in == out) return MARIAN_HIP_OK;
+  if(K <= 0 || N <= 0 || (K % 32) != 0 || (N % 8) != 0) return MARIAN_HIP_ERR_SHAPE;
+  if(K * N > 2147483647LL) return MARIAN_HIP_ERR_RANGE;
+  if(in == out) return MARIAN_HIP_OK;   // the two orders are the same for 16-bit tensors: nothing to do in place
+  // a copy between buffers that overlap only in part has no defined result
+  const uintptr_t a0 = reinterpret_cast<uintptr_t>(in), b0 = reinterpret_cast<uintptr_t>(out);
+  const uintptr_t bytes = 2 * (uintptr_t)K * (uintptr_t)N + sizeof(float);
+  if(a0 < b0 + bytes && b0 < a0 + bytes) return MARIAN_HIP_ERR_ALIAS;
   MH_HIP(hipMemcpyAsync(out, in, 2 * (size_t)K * (size_t)N + sizeof(float), hipMemcpyDeviceToDevice,
                         reinterpret_cast<hipStream_t>(stream)));
   return MARIAN_HIP_OK;

@@ -120,6 +120,7 @@ struct GemmArgs {
   // kAbsmaxSlots floats that receive values whose maximum is max|out| (the next call's abs-max,
   // taken where the tensor is produced), or null
   float* absmax_out = nullptr;
+  int absmax_used = 0;   // large-M launches: how many slots the launch fills (one per workgroup)
   // write the output with non-temporal stores (set by the launchers for outputs of several MB,
   // which would otherwise sit dirty in L2 until the kernel ends and be written back then)
   int stream_out = 0;

@@ -334,6 +334,52 @@ __global__ __launch_bounds__(1024) void prepare_a_onepass_kernel(const float* __
   if(g == 0 && tid == 0) *reinterpret_cast<float*>(out + (size_t)n16 * 16) = qm;
 }
 
+// Quantization alone for large inputs whose abs-max is known (left in `partials` by the kernel that
+// produced x): the memory access pattern of the one-pass kernel above - a quad of lanes reads 64
+// contiguous bytes per load, four loads in flight per thread (eight while the next set is on its
+// way), the packed bytes take a turn through LDS so that a wave stores 1 KB of contiguous output -
+// without its exchange.  A set = 256 quads = 64 KB of input per workgroup and step.
+__global__ __launch_bounds__(1024) void quantize_a_wide_kernel(const float* __restrict__ x, unsigned n16,
+                                                               const float* __restrict__ partials, int n_partials,
+                                                               int8_t* __restrict__ out) {
+  __shared__ float red[1024 / kWave];
+  __shared__ __attribute__((aligned(16))) uint32_t turn[1024 * 4];   // 16 bytes per thread
+  const int tid = threadIdx.x, quad = tid / 4, qlane = tid % 4;
+  const unsigned n_sets = (n16 / 4 + 255) / 256;
+  auto load_set = [&](unsigned set, v4f (&v)[4]) {
+    const unsigned q = set * 256u + (unsigned)quad;
+    const unsigned qc = 4u * q < n16 ? q : 0u;   // (n16 is a multiple of four: whole quads)
+    const char* src = reinterpret_cast<const char*>(x) + (size_t)qc * 256 + qlane * 16;
+#pragma unroll
+    for(int e = 0; e < 4; ++e) v[e] = *reinterpret_cast<const v4f*>(src + e * 64);
+  };
+  // the first loads are on their way while the partials are reduced
+  unsigned set = blockIdx.x;
+  v4f vals[4];
+  if(set < n_sets) load_set(set, vals);
+  float m = 0.0f;
+  for(int p = tid; p < n_partials; p += 1024) m = fmaxf(m, partials[p]);
+  m = block_max(m, red);
+  const float qm = quant_mult_from_maxabs(m);
+  const bool finite = qm < __builtin_inff();
+  for(; set < n_sets; set += gridDim.x) {
+    v4f cur[4];
+#pragma unroll
+    for(int e = 0; e < 4; ++e) cur[e] = vals[e];
+    if(set + gridDim.x < n_sets) load_set(set + gridDim.x, vals);
+    const unsigned q = set * 256u + (unsigned)quad;
+    if(4u * q < n16) {
+      // (the four lanes of a quad sit in one wave, whose LDS operations execute in order)
+#pragma unroll
+      for(int e = 0; e < 4; ++e)
+        turn[(quad * 4 + e) * 4 + qlane] = finite ? quantize_pack4_finite(cur[e], qm) : quantize_pack4(cur[e], qm);
+      const uint4 w = *reinterpret_cast<const uint4*>(&turn[(quad * 4 + qlane) * 4]);
+      *reinterpret_cast<uint4*>(reinterpret_cast<char*>(out) + (size_t)q * 64 + qlane * 16) = w;
+    }
+  }
+  if(blockIdx.x == 0 && tid == 0) *reinterpret_cast<float*>(out + (size_t)n16 * 16) = qm;
+}
+
 // Pass 2 of prepareB: W fp32 [K x N] -> K-blocked int8 payload of the quantized transpose + tail.
 // A workgroup transposes a 64(k) x 64(n) tile through LDS: reads are coalesced along n, writes are
 // 16-byte chunks of K values, the columns of a K sub-step side by side.

@@ -9,6 +9,7 @@
 //   src/tensors/gpu/backend.h:23-110           Backend (stream, synchronize), reduced to this path
 //   src/tensors/tensor_allocator.h:12-93       TensorAllocator (tensors carved from hip_device.h's Allocator)
 //   src/tensors/gpu/cuda_helpers.h:15-19       CUDA_CHECK -> MARIAN_HIP_CHECK (status code -> abort)
+//   src/graph/expression_graph.cpp:120-185     forward tape (inference mode clears a node's children)  -> graph::
 //
 // Tensors hold a MemoryPiece handle, not a pointer: the allocator may move its slab whenever
 // something is allocated, and every wrapper below reads the pointers at the moment of the call.
@@ -18,6 +19,8 @@
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
+#include <functional>
+#include <list>
 #include <string>
 #include <vector>
 
@@ -163,8 +166,9 @@ namespace integer {
 inline float getQuantMult(Backend& be, const Tensor& t) {
   if(!isIntgemm(t.type)) abortWith("getQuantMult does not work for this type");
   float qm = 0.f;
-  copy(be.stream(), reinterpret_cast<const float*>(t.data<int8_t>() + t.elements()),
-       reinterpret_cast<const float*>(t.data<int8_t>() + t.elements()) + 1, &qm);
+  // the tail sits behind the payload: elements * 1 byte for intgemm8, * 2 bytes for intgemm16
+  const float* tail = reinterpret_cast<const float*>(t.data<int8_t>() + t.elements() * sizeOf(t.type));
+  copy(be.stream(), tail, tail + 1, &qm);
   return qm;
 }
 
@@ -331,5 +335,125 @@ inline void affineOrDotStatic(Backend& be, const Tensor& a, const Tensor& bQuant
 }
 
 }  // namespace integer
+
+// ---- the graph side: lambda nodes on a forward tape, reduced to what this path needs -------
+// Mirrors (reference file:line):
+//   src/graph/node_operators_binary.h:16-80, src/graph/expression_operators.h:29-34   LambdaNodeOp, lambda()
+//   src/graph/expression_graph.cpp:120-185   ExpressionGraph::forward: for every node of the tape in
+//       order - allocate its value, run its forward functor, and in inference mode clear its
+//       children (:168-169) so that a tensor is given back as soon as no later node holds it
+//   src/graph/node.cpp (Node::free)          a node that nobody holds any more gives its value back
+// The affine binding below is what a src/tensors/hip/int8_interface.h of a Marian build would hold;
+// here it runs on these minimal types so that it is compiled and exercised (host_check.cpp).
+namespace graph {
+
+struct Node;
+typedef std::shared_ptr<Node> Expr;
+typedef std::function<void(Expr out, const std::vector<Expr>& in)> LambdaNodeFunctor;
+
+struct Node {
+  TensorAllocator& ta;
+  std::vector<Expr> children;
+  Shape shape;
+  Type type;
+  LambdaNodeFunctor forward;
+  Tensor val;
+  bool parameter = false;   // parameters own their memory elsewhere; the tape never frees it
+  Node(TensorAllocator& ta_, std::vector<Expr> children_, Shape shape_, Type type_, LambdaNodeFunctor forward_)
+      : ta(ta_), children(std::move(children_)), shape(std::move(shape_)), type(type_), forward(std::move(forward_)) {}
+  Node(const Node&) = delete;
+  Node& operator=(const Node&) = delete;
+  ~Node() {
+    if(!parameter && val.memory && val.memory->data()) ta.free(val);
+  }
+  Type value_type() const { return type; }
+};
+
+class ExpressionGraph {
+public:
+  ExpressionGraph(TensorAllocator& ta, bool inferenceOnly) : ta_(ta), inferenceOnly_(inferenceOnly) {}
+  TensorAllocator& allocator() const { return ta_; }
+
+  // A parameter or constant input: wraps a tensor that lives outside the tape.
+  Expr param(const Tensor& t) {
+    auto n = std::make_shared<Node>(ta_, std::vector<Expr>(), t.shape, t.type, LambdaNodeFunctor());
+    n->val = t;
+    n->parameter = true;
+    return n;
+  }
+  // lambda(nodes, shape, type, forward): a node whose forward step is the given functor.
+  Expr lambda(std::vector<Expr> nodes, Shape shape, Type type, LambdaNodeFunctor forward) {
+    auto n = std::make_shared<Node>(ta_, std::move(nodes), std::move(shape), type, std::move(forward));
+    tape_.push_back(n);
+    return n;
+  }
+  // Runs the tape front to back.  afterNode (optional) is called after every node with the tape's
+  // own reference already dropped, i.e. at the point where the node's inputs may have been freed.
+  void forward(const std::function<void(const Node&)>& afterNode = nullptr) {
+    while(!tape_.empty()) {
+      Expr v = tape_.front();
+      tape_.pop_front();
+      ta_.allocate(v->val, v->shape, v->type);
+      if(v->forward) v->forward(v, v->children);
+      if(inferenceOnly_) v->children.clear();
+      if(afterNode) afterNode(*v);
+    }
+  }
+
+private:
+  TensorAllocator& ta_;
+  bool inferenceOnly_;
+  std::list<Expr> tape_;
+};
+
+// affineOrDot of the HIP backend: the reference's node structure (src/tensors/cpu/intgemm_interface.h:
+// 46-99) - node 1 holds the quantized activations (typed like the weights, M * K + 4 bytes), node 2
+// the float32 product - with BOTH node bodies run by node 2 in one library call
+// (marian_hip_int8_affine_f32: one kernel at decode sizes).  Node 2 therefore reads the float32
+// input itself and must hold it as a DIRECT child: in inference mode the tape clears node 1's
+// children as soon as node 1 has run (src/graph/expression_graph.cpp:168-169), and an input held only
+// through node 1 would be freed - and its memory handed to node 2's own output - before node 2 runs.
+// Children of node 2: {aQuant, bQuant, [bias,] a}; `a` is last, so a bias is present iff there are four.
+inline Expr affineOrDot(ExpressionGraph& g, Expr a, Expr bQuant, Expr bias, bool transA, bool /*transB*/,
+                        float scale, bool relu = false) {
+  if(!isFloat(a->value_type())) abortWith("Intgemm expects type of A to be float32");
+  integer::checkB(bQuant->val);
+  if(transA) abortWith("transA: put a transpose node in front (the reference does, intgemm_interface.h:52)");
+  // node 1: the output tensor of prepareA.  Its functor is empty - node 2's call fills it, exactly
+  // as prepareA would - but it is a real node: the tape allocates its value and frees it after use.
+  Expr aQuant = g.lambda({a}, a->shape, bQuant->value_type(), [](Expr, const std::vector<Expr>&) {});
+  Shape outShape = a->shape;
+  outShape.back() = bQuant->shape.back();
+  auto fwd = [scale, relu](Expr out, const std::vector<Expr>& in) {
+    Expr aQ = in[0], bQ = in[1], a_ = in.back();
+    Expr bias_ = in.size() > 3 ? in[2] : nullptr;
+    integer::affineOrDot(out->ta, a_->val, aQ->val, bQ->val, bias_ ? &bias_->val : nullptr, out->val, scale, relu);
+  };
+  std::vector<Expr> children = {aQuant, bQuant};
+  if(bias) children.push_back(bias);
+  children.push_back(a);
+  return g.lambda(children, outShape, Type::float32, fwd);   // inference-only node
+}
+
+// The same as two real nodes, the reference's structure one to one: node 1 runs prepareA, node 2
+// reads nothing but the values of its children {aQuant, bQuant, [bias]}.
+inline Expr affineOrDotTwoNodes(ExpressionGraph& g, Expr a, Expr bQuant, Expr bias, float scale, bool relu = false) {
+  if(!isFloat(a->value_type())) abortWith("Intgemm expects type of A to be float32");
+  integer::checkB(bQuant->val);
+  Expr aQuant = g.lambda({a}, a->shape, bQuant->value_type(), [](Expr out, const std::vector<Expr>& in) {
+    integer::prepareA(out->ta, in[0]->val, out->val);
+  });
+  Shape outShape = a->shape;
+  outShape.back() = bQuant->shape.back();
+  auto fwd = [scale, relu](Expr out, const std::vector<Expr>& in) {
+    Expr bias_ = in.size() > 2 ? in[2] : nullptr;
+    integer::multiply(out->ta.backend(), in[0]->val, in[1]->val, bias_ ? &bias_->val : nullptr, out->val, scale, relu);
+  };
+  std::vector<Expr> children = {aQuant, bQuant};
+  if(bias) children.push_back(bias);
+  return g.lambda(children, outShape, Type::float32, fwd);
+}
+
+}  // namespace graph
 }  // namespace hip
 }  // namespace marian

@@ -268,6 +268,50 @@ int main(int argc, char** argv) {
                  sameBits(download<float>(be, g2, wantRelu.size()), download<float>(be, o, wantRelu.size())),
              "affineOrDotGrouped: both outputs as the separate calls'");
     }
+
+    // ---- the binding on a forward tape in inference mode (graph::affineOrDot) ----
+    {
+      const size_t nA = (size_t)M * K;
+      auto copyFwd = [&be, nA](graph::Expr out, const std::vector<graph::Expr>& in) {
+        copy(be.stream(), in[0]->val.data<float>(), in[0]->val.data<float>() + nA, out->val.data<float>());
+      };
+      // after every node, whatever the tape has given back is overwritten (0xFF bytes: NaN as floats)
+      auto spoil = [&](const graph::Node&) {
+        be.synchronize();
+        uint8_t* base = ta.allocator()->device()->data();
+        ta.allocator()->forEachGap([&](size_t offset, size_t size) {
+          fill(be.stream(), base + offset, base + offset + size, (uint8_t)0xFF);
+        });
+      };
+      for(int form = 0; form < 2; ++form) {
+        graph::ExpressionGraph g(ta, /*inferenceOnly=*/true);
+        graph::Expr x = g.param(a), wq = g.param(bq), bb = g.param(b);
+        // the activations are a node of the tape (a copy of the input): the tape owns and frees them
+        graph::Expr act = g.lambda({x}, a.shape, Type::float32, copyFwd);
+        std::weak_ptr<graph::Node> actAlive = act;
+        graph::Expr y = form == 0 ? graph::affineOrDot(g, act, wq, bb, false, false, 1.0f, /*relu=*/true)
+                                  : graph::affineOrDotTwoNodes(g, act, wq, bb, 1.0f, /*relu=*/true);
+        act.reset();   // from here on only nodes hold the input, as in a model's forward pass
+        g.forward(spoil);
+        expect(sameBits(download<float>(be, y->val, wantRelu.size()), wantRelu),
+               form == 0 ? "tape, inference mode: one-call binding (input a direct child of node 2), freed memory overwritten"
+                         : "tape, inference mode: two real nodes as in the reference, freed memory overwritten");
+        expect(actAlive.expired(), "the input is given back once the last node that reads it has run");
+      }
+      {   // why the one-call form needs the input as a direct child of node 2
+        graph::ExpressionGraph g(ta, true);
+        graph::Expr x = g.param(a), wq = g.param(bq), bb = g.param(b);
+        graph::Expr act = g.lambda({x}, a.shape, Type::float32, copyFwd);
+        std::weak_ptr<graph::Node> actAlive = act;
+        graph::Expr n1 = g.lambda({act}, a.shape, Type::intgemm8, [](graph::Expr, const std::vector<graph::Expr>&) {});
+        bool goneBeforeNode2 = false;
+        graph::Expr n2 = g.lambda({n1, wq, bb}, Shape{M, N}, Type::float32,
+                                  [&](graph::Expr, const std::vector<graph::Expr>&) { goneBeforeNode2 = actAlive.expired(); });
+        act.reset();
+        g.forward();
+        expect(goneBeforeNode2, "an input held only through node 1 is freed before node 2 runs");
+      }
+    }
     Tensor oStatic;
     ta.allocate(oStatic, {M, N}, Type::float32);
     integer::affineOrDotStatic(be, a, bq, &b, oStatic, 1.0f, true);
@@ -284,6 +328,8 @@ int main(int argc, char** argv) {
                  sameBits(download<int16_t>(be, aq16, wantAq16.size()), wantAq16),
              "intgemm16: prepareB and prepareA, payload and quantMult 1024");
       expect(sameBits(download<float>(be, o16, wantOut16.size()), wantOut16), "intgemm16: affineOrDot, bit for bit");
+      expect(integer::getQuantMult(be, aq16) == 1024.0f && integer::getQuantMult(be, bq16) == 1024.0f,
+             "intgemm16: getQuantMult reads the tail behind 2 * elements bytes");
     }
 
     // error paths: the reference's messages, as exceptions

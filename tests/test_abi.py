@@ -56,7 +56,7 @@ def test_shipped_library_exports_exactly_what_the_headers_declare():
     assert os.path.exists(L.TUNING_LIB_PATH), "build the library first (__graft_entry__.build())"
     tuning = declared_functions([TUNING_HEADER])
     assert tuning == ["marian_hip_int8_debug_profile", "marian_hip_int8_set_kernel", "marian_hip_probe_mfma",
-                      "marian_hip_probe_stream"]
+                      "marian_hip_probe_mix", "marian_hip_probe_stream"]
     assert exported_symbols(L.TUNING_LIB_PATH) == sorted(declared_functions() + tuning)
     assert sorted(L.TUNING_SIGNATURES) == tuning
 
@@ -89,7 +89,6 @@ def test_argument_validation_returns_codes_not_aborts():
     assert lib.marian_hip_layer_norm(buf, None, buf, 7, None, 0, buf, 2, 8, 1e-9, None, None) == L.ERR_SHAPE
     assert lib.marian_hip_layer_norm(None, None, buf, 8, None, 0, buf, 2, 8, 1e-9, None, None) == L.ERR_NULL
     assert lib.marian_hip_layer_norm(buf, None, buf, 8, None, 0, buf, 0, 8, 1e-9, None, None) == L.OK
-    assert lib.marian_hip_layer_norm(buf, None, buf, 8, None, 0, buf, 4096, 8, 1e-9, buf, None) == L.ERR_RANGE
     assert lib.marian_hip_softmax(buf, buf, 0, 1, buf, 2, 8, None) == L.ERR_SHAPE
     assert lib.marian_hip_softmax(buf + 2, None, 0, 0, buf, 2, 8, None) == L.ERR_ALIGN
     assert lib.marian_hip_logsoftmax(buf, None, 2, 8, None) == L.ERR_NULL
@@ -137,6 +136,13 @@ def test_argument_validation_returns_codes_not_aborts():
     assert lib.marian_hip_int8_prepare_b_quantized_transposed(buf, buf + 1024, 100, 8, None) == L.ERR_SHAPE
     assert lib.marian_hip_int8_prepare_b_quantized_transposed(buf, None, 64, 8, None) == L.ERR_NULL
     assert lib.marian_hip_status_string(L.ERR_ALIAS).decode() == "input and output overlap"
+    # the 16-bit counterpart (a copy): shapes as for the other 16-bit calls, in place is a no-op,
+    # a partial overlap is refused
+    assert lib.marian_hip_int16_prepare_b_quantized_transposed(buf, buf + 256, 64, 8, None) == L.ERR_ALIAS
+    assert lib.marian_hip_int16_prepare_b_quantized_transposed(buf, buf, 64, 8, None) == L.OK
+    assert lib.marian_hip_int16_prepare_b_quantized_transposed(buf, buf + 4096, 48, 8, None) == L.ERR_SHAPE
+    assert lib.marian_hip_int16_prepare_b_quantized_transposed(buf, buf + 4096, 64, 12, None) == L.ERR_SHAPE
+    assert lib.marian_hip_int16_prepare_b_quantized_transposed(None, buf, 64, 8, None) == L.ERR_NULL
     with pytest.raises(L.MarianHipError):
         L.check(L.ERR_SHAPE, "test")
 

@@ -417,6 +417,56 @@ def test_config5_shortlist(integer, orc, synth, M):
     assert np.array_equal(dense_acc[rows], want_acc) and np.array_equal(dense[rows], want)
 
 
+def _ragged_cases():
+    """M and N a whole number of main tiles plus or minus 1 / 8 / about 100, for every large-M
+    family that has a ragged form (forced: the automatic choice takes it only where it saves a
+    round of workgroups on the whole chip)."""
+    cases = []
+    for kernel, T in ((361, 256), (362, 256), (366, 256), (363, 128), (367, 128), (364, 128), (368, 128)):
+        K = 1024 if kernel in (361, 362, 366) else 256
+        for dm, dn in ((1, 8), (-1, -8), (100, 104), (8, 0), (0, 8), (-100, 96), (1, -104)):
+            cases.append((kernel, 2 * T + dm, K, 2 * T + dn))
+    return cases
+
+
+@pytest.mark.parametrize("kernel,M,K,N", _ragged_cases())
+def test_multiply_ragged_main_and_edge_tiles(integer, orc, synth, kernel, M, K, N):
+    """Whole main tiles for the first workgroups, 64 x 128 tiles below and 128 x 64 tiles to the
+    right of them: accumulators and outputs as the checker's, with and without bias and ReLU."""
+    say("multiply main + edge tiles", M, K, N, "kernel", kernel)
+    run_case(integer, orc, synth, 490 + M + N, M, K, N, kernel, bias_on=(M % 2 == 1), relu=(N % 16 == 8), scale=0.5)
+
+
+@pytest.mark.parametrize("M,K,N", [(4100, 1024, 4096), (4100, 1024, 4104), (2050, 1024, 2056), (4100, 4096, 1024),
+                                   (4352, 1024, 4096), (4097, 512, 4096)])
+def test_multiply_ragged_at_full_size(integer, orc, synth, M, K, N):
+    """The shapes where a few rows or columns past a whole number of main tiles used to cost a
+    second round of workgroups: the automatic choice, against sampled rows of the checker and an
+    int64 column-sum identity over everything."""
+    import torch
+    say("ragged at full size", M, K, N)
+    A, W, bias = inputs(synth, 495 + M + N, M, K, N)
+    Aq_h, Bq_h = orc.prepare_a(A), orc.prepare_b(W)
+    Aq, Bq = upload_q(integer, Aq_h, (M, K)), upload_b(integer, Bq_h, (K, N))
+    acc = integer.multiply_i32(Aq, Bq).cpu().numpy()
+    out = integer.multiply(Aq, Bq, dev(bias), relu=True).cpu().numpy()
+    # every column sum of the accumulators = (column sums of Aq) . Bq, in int64
+    a8 = Aq_h[:M * K].view(np.int8).reshape(M, K).astype(np.int64)
+    b8 = Bq_h[:K * N].view(np.int8).reshape(N, K).astype(np.int64)
+    assert np.array_equal(acc.astype(np.int64).sum(axis=0), b8 @ a8.sum(axis=0))
+    assert np.array_equal(acc.astype(np.int64).sum(axis=1), a8 @ b8.sum(axis=0))
+    # sampled rows (the last rows and columns are where the small tiles sit) against the checker
+    rows = sorted(set([0, 1, 255, 256, M // 2, M - 130, M - 65, M - 5, M - 4, M - 3, M - 2, M - 1]))
+    sub = np.ascontiguousarray(np.concatenate([Aq_h[:M * K].reshape(M, K)[rows].reshape(-1), Aq_h[M * K:]]))
+    want, want_acc = orc.affine(sub, Bq_h, bias, len(rows), K, N, 1.0, True)
+    assert np.array_equal(acc[rows], want_acc)
+    assert np.array_equal(out[rows], np.asarray(want, dtype=f32).reshape(len(rows), N))
+    # the whole fp32 image follows from the accumulators
+    unquant = orc.unquant_mult(orc.tail(Aq_h, M * K), orc.tail(Bq_h, K * N), 1.0)
+    img = np.maximum((acc.astype(f32) * f32(unquant)) + bias[None, :].astype(f32), f32(0))
+    assert np.array_equal(out, img)
+
+
 # ---------------------------------------------------------------- abs-max handed between calls
 
 @pytest.mark.parametrize("M,K,N,N2", [(128, 1024, 1024, 1024), (128, 1024, 4096, 1024), (128, 4096, 1024, 512),
@@ -442,6 +492,54 @@ def test_absmax_chaining_equals_recomputation(integer, orc, synth, M, K, N, N2):
     got, Aq2 = integer.affine_f32(out, Bq2, None, absmax=omax)
     want, Aq2_ref = integer.affine_f32(ref, Bq2, None)
     assert np.array_equal(Aq2.numpy(), Aq2_ref.numpy()) and np.array_equal(got.cpu().numpy(), want.cpu().numpy())
+
+
+@pytest.mark.parametrize("M", [4096, 4100, 2304])
+def test_encoder_layer_chain_hands_absmax_through_large_m_kernels(integer, orc, synth, M):
+    """Layer norm -> W1 + ReLU -> W2 at encoder size (d = 1024, ffn = 4096): every kernel leaves
+    the abs-max of what it wrote (the layer norm with more rows than slots, the large-M GEMM
+    epilogues one slot per workgroup), so the chained calls never scan a tensor for it.  The
+    slots' maximum is max|tensor| exactly, quantized activations and outputs equal the unchained
+    calls' and the checker's, bit for bit."""
+    import torch
+    ops = load("ops")
+    d, ffn = 1024, 4096
+    say("encoder chain", M)
+    X = synth.normal(9100 + M, synth.STREAM_A, (M, d), 1.0)
+    gamma = (1.0 + 0.1 * synth.normal(9101, synth.STREAM_BIAS, (d,), 1.0)).astype(f32)
+    beta = synth.normal(9102, synth.STREAM_BIAS, (d,), 0.1)
+    W1 = synth.normal(9103, synth.STREAM_W, (d, ffn), 0.02)
+    W2 = synth.normal(9104, synth.STREAM_W, (ffn, d), 0.02)
+    b1 = synth.normal(9105, synth.STREAM_BIAS, (ffn,), 0.01)
+    b2 = synth.normal(9106, synth.STREAM_BIAS, (d,), 0.01)
+    B1h, B2h = orc.prepare_b(W1), orc.prepare_b(W2)
+    B1, B2 = upload_b(integer, B1h, (d, ffn)), upload_b(integer, B2h, (ffn, d))
+    x, xmax = ops.layerNorm(dev(X), dev(gamma), dev(beta), eps=1e-6, want_absmax=True)
+    x_plain = ops.layerNorm(dev(X), dev(gamma), dev(beta), eps=1e-6)
+    xh = x.cpu().numpy()
+    assert np.array_equal(xh, x_plain.cpu().numpy())
+    assert float(xmax.data.max()) == float(np.abs(xh).max())
+    h, Aq1, hmax = integer.affine_f32(x, B1, dev(b1), relu=True, absmax=xmax, want_absmax=True)
+    h_ref, Aq1_ref = integer.affine_f32(x, B1, dev(b1), relu=True)
+    hh = h.cpu().numpy()
+    assert np.array_equal(Aq1.numpy(), Aq1_ref.numpy()) and np.array_equal(hh, h_ref.cpu().numpy())
+    assert float(hmax.data.max()) == float(np.abs(hh).max())
+    Aq1_h = orc.prepare_a(xh)
+    assert np.array_equal(Aq1.numpy(), Aq1_h)
+    rows = sorted(set([0, 1, 255, 256, 2047, 2048, M // 2, M - 129, M - 5, M - 4, M - 1]))
+    sub = np.ascontiguousarray(np.concatenate([Aq1_h[:M * d].reshape(M, d)[rows].reshape(-1), Aq1_h[M * d:]]))
+    want1, _ = orc.affine(sub, B1h, b1, len(rows), d, ffn, 1.0, True)
+    assert np.array_equal(hh[rows], np.asarray(want1, dtype=f32).reshape(len(rows), ffn))
+    y, Aq2, ymax = integer.affine_f32(h, B2, dev(b2), absmax=hmax, want_absmax=True)
+    y_ref, Aq2_ref = integer.affine_f32(h, B2, dev(b2))
+    yh = y.cpu().numpy()
+    assert np.array_equal(Aq2.numpy(), Aq2_ref.numpy()) and np.array_equal(yh, y_ref.cpu().numpy())
+    assert float(ymax.data.max()) == float(np.abs(yh).max())
+    Aq2_h = orc.prepare_a(hh)
+    assert np.array_equal(Aq2.numpy(), Aq2_h)
+    sub2 = np.ascontiguousarray(np.concatenate([Aq2_h[:M * ffn].reshape(M, ffn)[rows].reshape(-1), Aq2_h[M * ffn:]]))
+    want2, _ = orc.affine(sub2, B2h, b2, len(rows), ffn, d, 1.0, False)
+    assert np.array_equal(yh[rows], np.asarray(want2, dtype=f32).reshape(len(rows), d))
 
 
 # ---------------------------------------------------------------- random shapes

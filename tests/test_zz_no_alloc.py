@@ -34,20 +34,25 @@ CASES = [
     ((300, 1024, 512, True, True, 0), (16, 256, 64, True, False, 0)),       # two launches, then one fused kernel
     ((128, 1024, 1024, True, False, 0), (64, 512, 2048, False, True, 0)),   # abs-max launch + quantize-on-stage, then fused
     ((1024, 2048, 1024, True, True, 0), (256, 1024, 32000, True, False, 1000)),   # large-M kernel, then shortlisted output layer
+    # 4 Mi values and more: the one-pass prepareA, whose workgroups exchange their abs-max through
+    # words of the static workspace that persist from call to call (arrival slots, generation word,
+    # mailboxes) - twice in a row on different inputs, a two-set input, then a small call
+    ((4096, 1024, 256, True, True, 0), (4096, 1024, 264, True, False, 0), (2048, 4096, 128, False, True, 0),
+     (64, 512, 512, True, False, 0)),
 ]
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("first,second", CASES)
-def test_static_entry_point_matches_affine_f32(integer, orc, synth, first, second):
+@pytest.mark.parametrize("calls", CASES)
+def test_static_entry_point_matches_affine_f32(integer, orc, synth, calls):
     import torch
     L = load("_lib")
     T = load("types")
     lib = L.lib()
     be = integer.Backend.get(torch.device("cuda", torch.cuda.current_device()))
-    for call, (M, K, N, bias_on, relu, n_sl) in enumerate((first, second)):
+    for call, (M, K, N, bias_on, relu, n_sl) in enumerate(calls):
         say("static affine call", call, M, K, N, bias_on, relu, n_sl)
-        seed = 4100 + M + N
+        seed = 4100 + M + N + 7 * call
         A = synth.normal(seed, synth.STREAM_A, (M, K), 1.0)
         W = synth.normal(seed, synth.STREAM_W, (K, N), 0.02)
         bias = synth.normal(seed, synth.STREAM_BIAS, (N,), 0.01) if bias_on else None
