@@ -30,6 +30,27 @@
  * Alignment: A, Aq, Bq, out and acc 16 bytes; bias and idx 4 bytes.
  * M may be any value >= 0 (M == 0 or N == 0 is a no-op).
  *
+ * Threads and streams (reference src/translator/translator.h:158-164: one graph and backend per
+ * worker thread, several workers may share a device).  Every entry point may be called from any
+ * number of host threads at once; the stream is passed per call and calls on different streams
+ * may overlap on the device.  What may be shared between overlapping calls and what may not:
+ *   - weights, bias, shortlist ids, any input: read only, share freely;
+ *   - the workspace (marian_hip_int8_workspace_bytes()): ONE PER STREAM.  It holds the abs-max
+ *     partials of the call in flight and the words the workgroups of a one-pass prepareA exchange;
+ *     calls on one stream run one after the other and share it, calls on different streams must
+ *     each bring their own (a backend object per worker, as in the reference, does that);
+ *   - the n-best workspace of marian_hip_nbest_beams / marian_hip_logsoftmax_nbest_beams
+ *     (include/marian_hip_ops.h): one per stream, for the same reason (arrival counters);
+ *   - the static scratch behind marian_hip_int8_affine_f32_static: one per device, so those calls
+ *     must not overlap on a device at all;
+ *   - outputs and Aq: whatever the caller's graph guarantees, the library keeps no pointer.
+ * The library's own process-wide state is limited to caches that are written once per device
+ * (kernel attributes, the number of compute units, the address of the static scratch) and a
+ * counter for tags, all atomics; the last HIP error is kept per thread.  A one-pass prepareA
+ * puts a workgroup on every compute unit; while another stream keeps compute units busy its
+ * workgroups may not all be resident, their waits for one another are bounded, and the call then
+ * finishes by the slower route with the same result.
+ *
  * Return value: MARIAN_HIP_OK or an error code; a HIP runtime failure returns
  * MARIAN_HIP_ERR_HIP and the hipError_t is available from marian_hip_last_hip_error().
  * Nothing aborts or throws across this boundary; the C++ wrappers turn codes into ABORT.

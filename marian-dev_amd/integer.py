@@ -107,14 +107,17 @@ def getQuantMult(q):
 
 class Backend:
     """Per-device state the path needs: a stream and the abs-max workspace, the counterpart of
-    gpu::Backend (reference src/tensors/gpu/backend.h:23-110) reduced to this path."""
+    gpu::Backend (reference src/tensors/gpu/backend.h:23-110) reduced to this path.  The stream is
+    torch's current stream of the calling thread, and every stream has a workspace of its own:
+    worker threads that share a device (reference src/translator/translator.h:158-164) each run on
+    their own stream and never meet in a workspace."""
 
     _instances = {}
 
     def __init__(self, device):
         self.device = torch.device(device)
         self.workspace_bytes = int(self.lib.marian_hip_int8_workspace_bytes())
-        self.workspace = torch.empty(self.workspace_bytes, dtype=torch.uint8, device=self.device)
+        self._workspaces = {}   # stream handle -> workspace (kept for good: a graph may have recorded it)
         # float32 weights are quantized on first use and remembered when this is Type.intgemm8:
         # the counterpart of getGemmType() (reference src/tensors/backend.h:36-40) with the
         # memoized packing of src/graph/expression_operators.cpp:564-598 (its FBGEMM branch
@@ -125,6 +128,16 @@ class Backend:
     @property
     def lib(self):
         return _lib.lib()
+
+    @property
+    def workspace(self):
+        """The workspace of the current stream (calls on one stream run one after the other and
+        share it; calls on different streams may overlap and must not)."""
+        key = self.stream()
+        ws = self._workspaces.get(key)
+        if ws is None:
+            ws = self._workspaces.setdefault(key, torch.empty(self.workspace_bytes, dtype=torch.uint8, device=self.device))
+        return ws
 
     def setGemmType(self, type_):
         _abort_if(type_ not in (None, Type.intgemm8), "Unsupported type {} for Intgemm type??", type_)
