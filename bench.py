@@ -240,13 +240,27 @@ def cpu_baseline(seconds=10.0, aggregate_seconds=6.0, big_seconds=6.0):
     except AttributeError:
         share = os.cpu_count() or 1
     instances = max(1, min(share, 16))
-    procs = [subprocess.Popen([sys.executable, os.path.abspath(__file__), "--cpu-worker", str(aggregate_seconds)],
-                              stdout=subprocess.PIPE, text=True) for _ in range(instances)]
+    procs = []
     agg_ops_per_s = 0.0
-    for pr in procs:
-        out, _ = pr.communicate()
-        r = json.loads(out.strip().splitlines()[-1])
-        agg_ops_per_s += r["passes"] * r["ops_per_pass"] / r["seconds"]
+    try:
+        for _ in range(instances):
+            procs.append(subprocess.Popen([sys.executable, os.path.abspath(__file__), "--cpu-worker", str(aggregate_seconds)],
+                                          stdout=subprocess.PIPE, stdin=subprocess.DEVNULL, text=True))
+        for pr in procs:
+            out, _ = pr.communicate(timeout=aggregate_seconds * 10 + 120)
+            r = json.loads(out.strip().splitlines()[-1])
+            agg_ops_per_s += r["passes"] * r["ops_per_pass"] / r["seconds"]
+    finally:
+        # every child is reaped on every path (an exception above, a worker that hangs)
+        for pr in procs:
+            if pr.poll() is None:
+                pr.kill()
+            try:
+                pr.wait(timeout=10)
+            except subprocess.TimeoutExpired:
+                pass
+            if pr.stdout:
+                pr.stdout.close()
     # transformer-big decoding step: 48 layer GEMMs + the vocabulary GEMM at M = 128, random int8
     # weights (121 MB, every matrix its own memory), fp32 activations quantized per call
     rng = np.random.default_rng(77)
@@ -369,11 +383,12 @@ def probe_ceilings(torch):
     print("  %-5s %-3s %-3s %-3s %-3s %-8s | %9s %9s %9s %9s | %6s %8s" %
           ("", "", "", "", "", "", "B/clk/CU", "B/clk/CU", "B/clk/CU", "B/clk/CU", "issue", "MHz"))
 
-    def mix(waves, R, M, D, G, span, iters=400, split=0):
-        clocks = torch.zeros(2 * cus, dtype=torch.int64, device="cuda")
+    def mix(waves, R, M, D, G, span, iters=400, split=0, stagger=65536, wgs=None):
+        wgs = wgs or cus
+        clocks = torch.zeros(2 * wgs, dtype=torch.int64, device="cuda")
         sink = torch.zeros(4, dtype=torch.int32, device="cuda")
         for _ in range(2):
-            r = T.marian_hip_probe_mix(pool.data_ptr(), span, waves, R, M, D, G, split, iters, cus, clocks.data_ptr(),
+            r = T.marian_hip_probe_mix(pool.data_ptr(), span, stagger, waves, R, M, D, G, split, iters, wgs, clocks.data_ptr(),
                                        sink.data_ptr(), st)
             assert r == 0, r
         torch.cuda.synchronize()
@@ -394,15 +409,14 @@ def probe_ceilings(torch):
     for waves in (4, 8, 16):
         mix(waves, 16, 0, 0, 0, 64 * KB)                 # LDS reads alone
     for waves in (4, 8):
-        mix(waves, 16, 0, 8, 0, 2 * MB)                  # with operand blocks arriving, 2 : 1
+        mix(waves, 16, 0, 8, 0, 2 * MB)                  # with operand blocks arriving, 2 : 1 and 4 : 1
         mix(waves, 16, 0, 4, 0, 2 * MB)
-    for span in (64 * KB, 2 * MB, 32 * MB, 1024 * MB):    # global -> LDS alone: L1 hits, L2 hits, Infinity Cache, HBM
+    for span in (64 * KB, 2 * MB):                        # global -> LDS alone: vector L1 hits, L2 hits
         for waves in (4, 8, 16):
             mix(waves, 0, 0, 16, 0, span)
-    for span in (64 * KB, 2 * MB, 32 * MB):               # global -> registers alone
+    for span in (64 * KB, 2 * MB):                        # global -> registers alone
         for waves in (4, 8, 16):
             mix(waves, 0, 0, 0, 16, span)
-    mix(4, 0, 0, 8, 8, 2 * MB)
     mix(8, 0, 0, 8, 8, 2 * MB)
     for waves in (4, 8):                                  # matrix instructions with 0 / 0.5 / 0.75 / 1 / 1.5 / 2 KB of fragments each
         for R in (0, 4, 6, 8, 12, 16):
@@ -410,21 +424,58 @@ def probe_ceilings(torch):
     for waves in (4, 8):                                  # matrix instructions with operand blocks arriving only
         mix(waves, 0, 8, 4, 0, 2 * MB)
         mix(waves, 0, 8, 0, 4, 2 * MB)
+    print("  -- the large-M kernels' own mixes --")
     mix(4, 8, 8, 4, 0, 2 * MB)     # the 128x128 tile, four waves of 64x64
     mix(8, 12, 8, 4, 0, 2 * MB)    # the same tile by eight waves of 64x32 (two per SIMD)
-    mix(8, 8, 8, 4, 0, 2 * MB)
     mix(8, 8, 8, 4, 0, 2 * MB, split=1)   # four waves multiply, four waves load
     mix(8, 8, 8, 3, 0, 2 * MB, split=1)   # the same at 48 bytes per clock of operand blocks
     mix(8, 8, 8, 2, 0, 2 * MB, split=1)   # and at 32
-    mix(8, 0, 8, 4, 0, 2 * MB, split=1)
     mix(4, 8, 8, 3, 0, 2 * MB)
     mix(4, 8, 8, 2, 0, 2 * MB)
-    mix(8, 6, 8, 3, 0, 2 * MB, split=1)
     mix(4, 6, 8, 3, 0, 2 * MB)     # two 256x128 tiles, four waves of 128x64
+    mix(8, 6, 8, 3, 0, 2 * MB, split=1)
     mix(8, 6, 8, 2, 0, 2 * MB)     # the 256x256 tile, eight waves of 128x64
     mix(8, 4, 8, 1, 2, 2 * MB)     # the same with the weights from global memory straight into registers
     mix(8, 4, 8, 2, 2, 2 * MB)
     mix(4, 4, 8, 2, 4, 2 * MB)     # 128x128, four waves, weights straight into registers
+
+    print("\n-- read-only streaming from HBM by instruction form and bytes in flight (marian_hip_probe_mix over 1 GiB, every "
+          "workgroup its own 4 MiB-apart region; 16 KB per wave and round; chip-wide rate from the 100 MHz clock) --")
+
+    def hbm(waves, D, G, wgs, iters=48):
+        clocks = torch.zeros(2 * wgs, dtype=torch.int64, device="cuda")
+        sink = torch.zeros(4, dtype=torch.int32, device="cuda")
+        span = 1024 * MB
+        for _ in range(2):
+            r = T.marian_hip_probe_mix(pool.data_ptr(), span, span // wgs, waves, 0, 0, D, G, 0, iters, wgs,
+                                       clocks.data_ptr(), sink.data_ptr(), st)
+            assert r == 0, r
+        torch.cuda.synchronize()
+        c = clocks.cpu().numpy().reshape(-1, 2).astype(np.float64)
+        secs = float(np.median(c[:, 1])) * 1e-8
+        total = wgs * waves * 1024.0 * (D + G) * iters
+        print("  %3d workgroups x %2d waves, %-34s %7.1f MB in %7.1f us  %5.2f TB/s" %
+              (wgs, waves, "global_load_lds_dwordx4 (no VGPRs)" if D else "global_load_dwordx4 into registers", total / 1e6,
+               secs * 1e6, total / secs / 1e12))
+
+    for waves in (4, 8, 16):
+        hbm(waves, 16, 0, cus)
+        hbm(waves, 0, 16, cus)
+
+    print("\n-- the same access pattern as whole launches (HIP events, back-to-back launches, each over fresh bytes): one "
+          "workgroup of 16 waves per CU reads its own contiguous share of the buffer, 16 KB per workgroup and step --")
+    for mb in (64, 256, 1024):
+        span = mb * MB
+        iters = span // (cus * 16 * 16 * KB)
+        n = max(1, min(16, pool_bytes // span))
+        clocks = torch.zeros(2 * cus, dtype=torch.int64, device="cuda")
+        sink = torch.zeros(4, dtype=torch.int32, device="cuda")
+        for form, (D, G) in (("global_load_lds_dwordx4", (16, 0)), ("global_load_dwordx4", (0, 16))):
+            launches = [(lambda i=i, D=D, G=G: T.marian_hip_probe_mix(pool.data_ptr() + i * span, span, span // cus, 16, 0, 0, D, G, 0,
+                                                                  iters, cus, clocks.data_ptr(), sink.data_ptr(), st))
+                        for i in range(n)]
+            mean, med = per_launch_ms(torch, launches, max(3, 48 // n))
+            print("  %5d MiB  %-24s %8.2f us  %6.2f TB/s" % (mb, form, med * 1e3, span / (med * 1e-3) / 1e12))
     print("\n-- sustained v_mfma_i32_32x32x32_i8 rate on random operand bits --")
     for per_cu in (1, 2):
         wgs, iters = cus * per_cu, 4000
@@ -465,6 +516,27 @@ def measured_int8_peak(torch):
             "how": "tuning build's MFMA probe: %d workgroups of 4 waves (one wave per SIMD), %d x 8 "
                    "v_mfma_i32_32x32x32_i8 per wave on random operand bits, %.0f us per launch; clock = shader "
                    "clocks / 100 MHz reference clocks inside the loop" % (wgs, iters, med * 1e3)}
+
+
+def measured_read_bw(torch):
+    """What a read-only pass over 256 MiB (rotating over 1 GiB, so from HBM) reaches on this device,
+    with the tuning build's streaming probe (1024 workgroups x 256 threads, 8 loads of 16 bytes in
+    flight per thread; HIP events around the launches).  None when the tuning build is absent."""
+    try:
+        T = importlib.import_module(PKG + "._lib").tuning_lib()
+    except Exception:
+        return None
+    st = torch.cuda.current_stream().cuda_stream
+    pool = torch.empty(1 << 30, dtype=torch.int8, device="cuda").random_(-128, 127)
+    dst = torch.empty(4096, dtype=torch.int8, device="cuda")
+    rb = 256 << 20
+    launches = [(lambda i=i: T.marian_hip_probe_stream(pool.data_ptr() + i * rb, rb, dst.data_ptr(), 16, 1024, 256, 8, 0, st))
+                for i in range(4)]
+    mean, med = per_launch_ms(torch, launches, 6)
+    del pool
+    return {"gbs": round(rb / (med * 1e-3) / 1e9, 1),
+            "how": "tuning build's streaming probe: read-only pass over 256 MiB, four regions of a 1 GiB pool in turn, "
+                   "1024 workgroups x 256 threads, 8 x 16 bytes in flight per thread, %.1f us per launch" % (med * 1e3)}
 
 
 def pmc_summary(fetch_csv, write_csv):
@@ -602,8 +674,11 @@ def main():
     dom_bytes = algorithmic_bytes(dom.M, dom.K, dom.N)
     traffic = measured_traffic()
     achieved = dom_bytes / (mean_ms * 1e-3) / 1e9
+    read_bw = measured_read_bw(torch)
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                 "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+                "frac_of_measured_read_bw": None if not read_bw else round(achieved / read_bw["gbs"], 4),
+                "measured_read_bw": read_bw,
                 "traffic": traffic.get("stream32_fused_M64_K512_N32000"),
                 "traffic_source": "profiles/hbm_traffic_pmc.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a "
                                   "64 MiB copy), sources at commit %s" % traffic["_commit"]
@@ -778,6 +853,20 @@ def main():
         fdt = time_graphs(torch, full, n, max(4, args.warmup // 2))
         gonly = [capture(torch, (lambda c=c: dec.step(c, gemm_only=True))) for c in range(bsets)]
         gdt = time_graphs(torch, gonly, n, max(4, args.warmup // 2))
+        # the same step launched eagerly, call by call, from this Python host (Marian launches its
+        # forward tape eagerly too, from C++): the host's own time per call - ctypes, torch's
+        # allocator for every output - is part of this figure
+        for c in range(3):
+            dec.step(c, fused_tail=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for c in range(10):
+            dec.step(c, fused_tail=True)
+        torch.cuda.synchronize()
+        eager_full_ms = (time.perf_counter() - t0) / 10 * 1e3
+        dk = dec.d // dec.H
+        cache_bytes = 2 * dec.layers * 4 * dk * dec.H * (dec.M * dec.T + dec.batch * dec.L)
+        step_bytes_big = dec.weight_bytes + cache_bytes + 4 * dec.M * dec.V
         sel = [capture(torch, (lambda c=c: dec.step(c, fused_tail=True, select=True))) for c in range(bsets)]
         seldt = time_graphs(torch, sel, n, max(4, args.warmup // 2))
         del sel
@@ -811,6 +900,11 @@ def main():
             "one_launch_tail_equals_two_launches": same_tail,
             "ms_per_step_unchained": round(udt / n * 1e3, 4),
             "chained_equals_unchained": same,
+            "eager_ms_per_step_python_host": round(eager_full_ms, 4),
+            "step_hbm_frac": round(step_bytes_big * n / fdt / 1e9 / HBM_PEAK_GBS, 4),
+            "weight_hbm_frac": round(dec.weight_bytes * n / fdt / 1e9 / HBM_PEAK_GBS, 4),
+            "step_algorithmic_bytes": {"int8_weights": dec.weight_bytes, "cached_keys_and_values_read": cache_bytes,
+                                       "logits_written": 4 * dec.M * dec.V},
             "hyp_tokens_per_s": round(dec.M * n / fdt, 1),
             "output_tokens_per_s": round(dec.batch * n / fdt, 1),
             "gemm_only_ms_per_step_same_harness": round(gdt / n * 1e3, 4),

@@ -60,12 +60,14 @@ int marian_hip_probe_mfma(const void* data, int iters, int workgroups, long long
  * wave each), `mfmas` v_mfma_i32_32x32x32_i8, `dmas` global_load_lds_dwordx4 (1 KB per wave from
  * global memory straight into LDS) and `gloads` global_load_dwordx4 (1 KB per wave into registers)
  * are spread evenly.  The global addresses walk over span_bytes (a power of two, at least 64 KB)
- * behind src, so the span decides which cache serves them.  Only the mixes the measurements use are
+ * behind src, workgroup b starting b * stagger_bytes in (a multiple of 1 KB): span and stagger decide
+ * which cache serves them - 64 KB apart over a few MB: the XCD's L2; span / workgroups apart over
+ * a GiB: HBM.  Only the mixes the measurements use are
  * instantiated; another one returns MARIAN_HIP_ERR_SHAPE.  split (eight waves only): the first four
  * waves issue the LDS reads and matrix instructions, the other four the global loads.  The time is
  * that of the slowest wave.  clocks as for marian_hip_probe_mfma.
  */
-int marian_hip_probe_mix(const void* src, size_t span_bytes, int waves, int reads, int mfmas, int dmas, int gloads,
+int marian_hip_probe_mix(const void* src, size_t span_bytes, size_t stagger_bytes, int waves, int reads, int mfmas, int dmas, int gloads,
                          int split, int iters, int workgroups, long long* clocks, int* sink, void* stream);
 
 #ifdef __cplusplus

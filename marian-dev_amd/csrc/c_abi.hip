@@ -759,12 +759,13 @@ int marian_hip_probe_mfma(const void* data, int iters, int workgroups, long long
   return MARIAN_HIP_OK;
 }
 
-int marian_hip_probe_mix(const void* src, size_t span_bytes, int waves, int reads, int mfmas, int dmas, int gloads,
+int marian_hip_probe_mix(const void* src, size_t span_bytes, size_t stagger_bytes, int waves, int reads, int mfmas, int dmas, int gloads,
                          int split, int iters, int workgroups, long long* clocks, int* sink, void* stream) {
   if(!src || !clocks || !sink) return MARIAN_HIP_ERR_NULL;
   if(iters <= 0 || workgroups <= 0 || (waves != 4 && waves != 8 && waves != 16)) return MARIAN_HIP_ERR_SHAPE;
   if((mfmas > 0 && waves > 8) || (split && waves != 8)) return MARIAN_HIP_ERR_SHAPE;
   if(span_bytes < 65536 || (span_bytes & (span_bytes - 1)) != 0 || span_bytes > (1ull << 31)) return MARIAN_HIP_ERR_SHAPE;
+  if(stagger_bytes % 1024 != 0 || stagger_bytes > span_bytes) return MARIAN_HIP_ERR_SHAPE;
   if(!aligned(src, 16)) return MARIAN_HIP_ERR_ALIGN;
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   constexpr int kLds = 128 * 1024;
@@ -776,7 +777,7 @@ int marian_hip_probe_mix(const void* src, size_t span_bytes, int waves, int read
     const int lds_status = allow_lds(kernel, kLds, lds_done);                                                  \
     if(lds_status != MARIAN_HIP_OK) return lds_status;                                                         \
     hipLaunchKernelGGL(kernel, dim3(workgroups), dim3(waves * 64), kLds, st, reinterpret_cast<const int8_t*>(src), \
-                       (unsigned)span_bytes, iters, clocks, sink);                                             \
+                       (unsigned)span_bytes, (unsigned)stagger_bytes, iters, clocks, sink);                                             \
     MH_HIP(hipGetLastError());                                                                                 \
     return MARIAN_HIP_OK;                                                                                      \
   }

@@ -70,15 +70,17 @@ __global__ __launch_bounds__(256) void probe_mfma_kernel(const v4i* __restrict__
 // ds_read_b128 (1 KB per wave each), M v_mfma_i32_32x32x32_i8, D global_load_lds_dwordx4 (1 KB per
 // wave from global memory straight into LDS) and G global_load_dwordx4 (1 KB per wave into
 // registers) are spread evenly, in that fixed order (inline assembly and scheduling barriers).
-// Global addresses walk over `span` bytes (a power of two) behind src, 1 KB per wave load, so the
-// span decides whether the loads hit the vector L1, the XCD's L2 or neither.  Up to 12 LDS reads and
+// Global addresses walk over `span` bytes (a power of two) behind src, 1 KB per wave load, workgroup
+// b starting b * stagger bytes in: a small span and stagger make the loads hit the vector L1 or the
+// XCD's L2 (the workgroups follow each other over the same lines), a large span cut into one
+// region per workgroup (stagger = span / workgroups) makes them stream from HBM.  Up to 12 LDS reads and
 // 24 vector-memory loads of a wave are in flight.  clocks[2 * workgroup] = shader clocks,
 // [2 * workgroup + 1] = 100 MHz reference clocks from the common start until the last wave has finished.
 // SPLIT (eight waves): the first four waves, one per SIMD, issue only the LDS reads and the matrix
 // instructions, the other four only the global loads - a wave that cannot issue a load because the
 // vector memory path is full then does not hold up matrix instructions behind it.
 template <int R, int M, int D, int G, bool SPLIT = false>
-__global__ __launch_bounds__(M > 0 ? 512 : 1024) void probe_mix_kernel(const int8_t* __restrict__ src, unsigned span, int iters,
+__global__ __launch_bounds__(M > 0 ? 512 : 1024) void probe_mix_kernel(const int8_t* __restrict__ src, unsigned span, unsigned stagger, int iters,
                                                          long long* __restrict__ clocks, int* __restrict__ sink) {
   extern __shared__ __attribute__((aligned(16))) int8_t lds[];   // 64 KB that are read + 64 KB that the DMA fills
   const unsigned lds_base = (unsigned)(size_t)lds;
@@ -97,7 +99,7 @@ __global__ __launch_bounds__(M > 0 ? 512 : 1024) void probe_mix_kernel(const int
   const unsigned rd_addr = lds_base + (unsigned)((wave % 8) * 8192 + lane * 16);
   const unsigned voff = (unsigned)lane * 16u;
   const unsigned step = (unsigned)(SPLIT ? 4 : waves) * 1024u;
-  unsigned goff = __builtin_amdgcn_readfirstlane(((unsigned)blockIdx.x * 65536u + (unsigned)wave * 1024u) & (span - 1));
+  unsigned goff = __builtin_amdgcn_readfirstlane(((unsigned)blockIdx.x * stagger + (unsigned)wave * 1024u) & (span - 1));
   unsigned dma_slot = (unsigned)wave;
   v4i rd = {0, 0, 0, 0}, gl = {0, 0, 0, 0};
   // (SPLIT: two loops behind one wave-uniform branch, so that neither has a branch per slot)
