@@ -851,6 +851,13 @@ def main():
         del sep
         full = [capture(torch, (lambda c=c: dec.step(c, fused_tail=True))) for c in range(bsets)]
         fdt = time_graphs(torch, full, n, max(4, args.warmup // 2))
+        # the same bits whether projections and attention are one launch or two
+        o_f = dec.step(0, fused_tail=True)
+        o_s = dec.step(0, fused_tail=True, fused_attention=False)
+        same_att = bool(torch.equal(o_f[0], o_s[0]) and torch.equal(o_f[1], o_s[1]))
+        sepatt = [capture(torch, (lambda c=c: dec.step(c, fused_tail=True, fused_attention=False))) for c in range(bsets)]
+        sadt = time_graphs(torch, sepatt, n, max(4, args.warmup // 2))
+        del sepatt
         gonly = [capture(torch, (lambda c=c: dec.step(c, gemm_only=True))) for c in range(bsets)]
         gdt = time_graphs(torch, gonly, n, max(4, args.warmup // 2))
         # the same step launched eagerly, call by call, from this Python host (Marian launches its
@@ -880,10 +887,11 @@ def main():
         dec.by_ancestors = False
         out["transformer_big_decode_full"] = {
             "what": "full decoder step through the host mirrors, from the previous step's word indices: embedding rows x "
-                    "sqrt(d) + position signal (one launch), 49 int8 affine calls + per layer "
-                    "2 one-launch attentions (20 cached positions + the new one, appended by the call; "
+                    "sqrt(d) + position signal (one launch), 49 int8 affine products + per layer "
+                    "2 attentions (20 cached positions + the new one, appended by the call; "
                     "source lengths uniform 20..60, padded to 60 positions with mask), 3 skip-add+layer-norm; the self-attention "
-                    "projections Wq, Wk, Wv through one grouped call; log-softmax over 32000, beam/batch transposition + n-best per "
+                    "projections Wq, Wk, Wv and the self-attention are one launch, the context attention's Wq and the context "
+                    "attention another (58 launches per step); log-softmax over 32000, beam/batch transposition + n-best per "
                     "sentence in one launch (the log-probabilities are not written out); no hypothesis bookkeeping; the "
                     "abs-max of every GEMM input is left by the kernel that produced it",
             "ms_per_step": round(fdt / n * 1e3, 4),
@@ -896,6 +904,8 @@ def main():
             "state_selection": "the step preceded by the beam search's selection of the surviving hypotheses' cached keys "
                                "and values (rows(state, hypIndices) over all layers as one gather of the positions in use, %d MB read and written); "
                                "hypothesis indices resident on the device" % round(dec.state.numel() * 4 / 1e6 * (dec.T - 1) / dec.cap),
+            "ms_per_step_projections_and_attention_as_separate_launches": round(sadt / n * 1e3, 4),
+            "one_launch_attention_equals_separate_launches": same_att,
             "ms_per_step_logsoftmax_and_nbest_as_two_launches": round(sdt / n * 1e3, 4),
             "one_launch_tail_equals_two_launches": same_tail,
             "ms_per_step_unchained": round(udt / n * 1e3, 4),

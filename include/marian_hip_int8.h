@@ -184,6 +184,38 @@ int marian_hip_int8_affine_f32_grouped(const float* A, int8_t* Aq, int64_t n_gro
                                        size_t workspace_bytes, void* stream);
 
 /*
+ * The projections in front of an attention and the attention itself, for ONE new target position
+ * per query row, in one launch (reference src/models/transformer.h:279-348, MultiHead: q =
+ * affine(input, Wq, bq) and, for self-attention, k / v = affine(input, Wk / Wv, ..), the head
+ * split, then Attention(), :240-277).  A workgroup owns the 64 columns of one head in every
+ * projection for a few rows of the input and runs that head's attention for them before it exits,
+ * so q (k, v) never travel through memory.  Head size 64; N = heads * 64 columns per matrix.
+ *   n_proj = 3: Bq / bias / proj_out hold {Wq, Wk, Wv}; the new key and value rows are appended to
+ *     the caches at position len - 1 (as marian_hip_attention_cached does with k_new / v_new) and
+ *     the attention runs over positions 0 .. len - 1; batchKV = M * heads.
+ *   n_proj = 1: Bq / bias / proj_out hold {Wq}; the caches are complete (the encoder's keys and
+ *     values), query row r uses cache entry r % batchKV.
+ *   A: fp32 [M x K]; Aq receives what marian_hip_int8_prepare_a would write.  K % 128 == 0,
+ *     K <= 1024, len <= 512.  Bq, bias, proj_out: HOST arrays of n_proj device pointers, read
+ *     during the call; bias and proj_out (and their entries) may be NULL.  proj_out[g], where
+ *     given, receives the projection itself, fp32 [M x N] - bit for bit what
+ *     marian_hip_int8_affine_f32 writes.
+ *   k_cache, v_cache: [batchKV, kv_capacity, 64] fp32, `len` positions in use; mask: NULL or
+ *     [n_masks, len], row (r / heads) % n_masks for query row r of the [M * heads] rows;
+ *     out: [M * heads, 64] = [M x N]; att_scale: the 1 / sqrt(64) of transformer.h:261.
+ *   absmax_in / absmax_out / workspace: as for marian_hip_int8_affine_f32_chained (absmax_out
+ *     needs M * heads <= 2048; the workspace is only used when absmax_in is NULL).
+ * The result has the bits of the separate calls (marian_hip_int8_affine_f32_grouped, then
+ * marian_hip_attention_cached).
+ */
+int marian_hip_int8_proj_attention(const float* A, int8_t* Aq, int64_t n_proj, const int8_t* const* Bq,
+                                   const float* const* bias, float* const* proj_out, int64_t M, int64_t K,
+                                   int64_t heads, float* k_cache, float* v_cache, int64_t batchKV, int64_t len,
+                                   int64_t kv_capacity, const float* mask, int64_t n_masks, float att_scale,
+                                   float* out, const float* absmax_in, float* absmax_out, void* workspace,
+                                   size_t workspace_bytes, void* stream);
+
+/*
  * marian_hip_int8_affine_f32 for callers that cannot allocate and have no workspace to pass: code
  * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no
  * counterpart in the reference (there the prepareA node's output and every temporary come from the

@@ -35,6 +35,8 @@ SIGNATURES = {
     "marian_hip_int8_affine_f32_chained": (_i, [_vp, _vp, _vp, _vp, _vp, _i64, _vp, _i64, _i64, _i64, _f,
                                                 _i, _vp, _vp, _vp, _sz, _vp]),
     "marian_hip_int8_affine_f32_grouped": (_i, [_vp, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _f, _i, _vp, _vp, _sz, _vp]),
+    "marian_hip_int8_proj_attention": (_i, [_vp, _vp, _i64, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _vp, _i64, _i64, _i64, _vp,
+                                            _i64, _f, _vp, _vp, _vp, _vp, _sz, _vp]),
     "marian_hip_int8_affine_f32_static": (_i, [_vp, _vp, _vp, _vp, _i64, _vp, _i64, _i64, _i64, _f, _i, _vp]),
     "marian_hip_int8_affine_shortlist": (_i, [_vp, _vp, _vp, _vp, _i64, _vp, _i64, _i64, _i64,
                                               _f, _i, _vp]),

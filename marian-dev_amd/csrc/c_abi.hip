@@ -32,6 +32,19 @@ int marian_hip::record_hip_error(int e) {
   return MARIAN_HIP_ERR_HIP;
 }
 
+int marian_hip::launch_absmax_partials(const float* A, unsigned long n, float* partials, int* n_partials, void* stream) {
+  const size_t n4 = (size_t)n / 4, per_block = (size_t)kQuantThreads * 8;   // eight 16-byte loads per thread
+  size_t g = (n4 + per_block - 1) / per_block;
+  if(g < 1) g = 1;
+  if(g > (size_t)kMaxPartials) g = kMaxPartials;
+  hipLaunchKernelGGL(absmax_partial_kernel, dim3((unsigned)g), dim3(kQuantThreads), 0, reinterpret_cast<hipStream_t>(stream),
+                     A, n4, partials);
+  const hipError_t e = hipGetLastError();
+  if(e != hipSuccess) return marian_hip::record_hip_error((int)e);
+  *n_partials = (int)g;
+  return MARIAN_HIP_OK;
+}
+
 namespace {
 
 // The shipped library has no switches: kernel_override() is the constant 0 there and the

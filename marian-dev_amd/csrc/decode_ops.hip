@@ -17,6 +17,7 @@
 #include "abi_common.h"
 #include "int8_common.h"
 #include "nbest_plan.h"
+#include "quantize_common.h"
 
 using namespace marian_hip;
 
@@ -803,6 +804,338 @@ __global__ __launch_bounds__(256) void attention_kernel(const float* __restrict_
   if(append_late && lane < dk) {
     kb[(size_t)(len - 1) * dk + lane] = k_app;
     vb[(size_t)(len - 1) * dk + lane] = v_app;
+  }
+}
+
+// ---------------------------------------------------------------- projection + attention in one launch
+// The projections in front of an attention and the attention itself for one new target position
+// (reference src/models/transformer.h:279-348: q = affine(input, Wq, bq), for self-attention also
+// k, v = affine(input, Wk / Wv, ..), split into heads, then Attention()): a workgroup owns the 64
+// columns of ONE head in every projection for R rows of the input, so it has everything that
+// head's attention needs for its rows and runs it before it exits - one launch instead of two, and
+// q (k, v) never travel through memory.
+//   1. the abs-max of the input comes from the slots its producer left (or an abs-max launch);
+//   2. the workgroup quantizes its R rows of the float32 input into LDS in matrix-operand order
+//      (exactly the quantize-on-stage form of the decode GEMM: same quantizer, same layout); the
+//      workgroups of head 0 also write them out, so the prepareA node's tensor still exists;
+//   3. eight waves = 2 column tiles x 4 ranges of K; every wave requests its weights of all
+//      projections at kernel start (up to 24 loads of 1 KB in flight), multiplies, and drops its
+//      partial tiles into LDS;
+//   4. the partial tiles are added (exact), dequantized with bias exactly like the GEMM epilogues
+//      (two roundings) and kept in LDS as q[R][64] (k_new, v_new); k_new and v_new also go into
+//      the caches at position len - 1, and all three into proj_out where a caller asks for them;
+//   5. wave w runs the attention of row w: the code of attention_kernel's 64-wide path, operation
+//      for operation, with q and the newest key/value row read from LDS.
+// Requirements (checked by the launcher): head size 64, K % 128 == 0, K <= 1024, len <= 512.
+// Measured (transformer-big step, 128 rows, 16 heads): 13.5 us against 8.2 + 8.4 us for q, k, v and
+// the self-attention over 21 positions, 13.9 against 5.3 + 8.4 us for Wq and the context attention over
+// 60 positions - the attention is bound by the bytes of keys and values it reads (22 MB per layer),
+// so the launch saved is most of the gain.  Tried and dropped: asking for a row's keys and values
+// at kernel start so that they reach L2 under the projections (loads into a scratch word of LDS):
+// +16 us per step - they queue ahead of the weights and the input, which everything waits for.
+constexpr int kProjThreads = 512, kProjMaxK = 1024, kProjMaxLen = 512;
+
+struct ProjAttentionArgs {
+  const float* A;           // [M, K] float32
+  int8_t* aq_out;           // [M, K] int8 + quantMult tail
+  const float* partials;    // abs-max slots of A
+  int n_partials;
+  const int8_t* Bq[3];      // prepared weights [K, heads * 64]
+  const float* bias[3];     // or null
+  float* proj_out[3];       // [M, heads * 64] or null: the projections themselves, for callers that want them
+  int M, K, heads;
+  float* k_cache;           // [batchKV, kv_cap, 64]
+  float* v_cache;
+  unsigned batchKV;
+  int len, kv_cap;
+  const float* mask;        // [n_masks, len] or null, one row per (query row / heads) % n_masks
+  unsigned n_masks;
+  float att_scale;
+  float* out;               // [M * heads, 64]
+  float* absmax_out;        // slots or null
+};
+
+// the row permutation of the staged activations (gemm_stream32_kernel.h: stream32_row_key)
+__device__ __forceinline__ int proj_row_key(int c16) { return (c16 ^ (c16 >> 2)) & 7; }
+
+// One query row of 64 values by one wave: attention_kernel's path for that head size (sixteen lanes
+// cover a key or value row, four consecutive positions per load, up to 64 positions in flight), the
+// same operations in the same order, so the result has the same bits.  q, k_last, v_last may lie
+// in LDS.  sc: len4 floats of this wave, part: 256 floats behind them.  Returns |out| of this lane.
+__device__ __forceinline__ float attention_row64(const float* q, const float* kb, const float* vb, const float* k_last,
+                                                 const float* v_last, const float* mk, int len, float scale, float* sc,
+                                                 float* part, float* out_row, int lane) {
+  constexpr int kAttU = 16, dk = 64;
+  const int len4 = (len + 3) & ~3;
+  const int g = lane / 16, c = lane % 16;
+  const int u_last = (len + 2 - g) / 4;
+  auto load_rows = [&](const float* rows, const float* last, int base, v4f (&r)[kAttU]) __attribute__((always_inline)) {
+    const float* first = rows + (size_t)g * dk + 4 * c;
+    const float* last_c = last + 4 * c;
+#pragma unroll
+    for(int u = 0; u < kAttU; ++u) {
+      if(base + 4 * u < len) {
+        const int U = base / 4 + u;
+        if(U >= u_last) r[u] = *reinterpret_cast<const v4f*>(last_c);
+        else r[u] = *reinterpret_cast<const v4f*>(first + (size_t)U * 4 * dk);
+      } else if(base + 4 * (u & ~3) < len) {
+        r[u] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+      }
+    }
+  };
+  float mk0 = 0.0f;
+  if(mk) mk0 = mk[min(lane, len - 1)];
+  const v4f q4 = reinterpret_cast<const v4f*>(q)[c];
+  v4f kr[kAttU], vr[kAttU];
+  load_rows(kb, k_last, 0, kr);
+  load_rows(vb, v_last, 0, vr);
+  for(int base = 0;;) {
+#pragma unroll
+    for(int u0 = 0; u0 < kAttU; u0 += 4) {
+      if(base + 4 * u0 < len) {
+        float s[4];
+#pragma unroll
+        for(int u = u0; u < u0 + 4; ++u) {
+          float t = q4.x * kr[u].x;
+          t = fmaf(q4.y, kr[u].y, t);
+          t = fmaf(q4.z, kr[u].z, t);
+          s[u - u0] = fmaf(q4.w, kr[u].w, t);
+        }
+#pragma unroll
+        for(int u = 0; u < 4; ++u) s[u] = row16_sum(s[u]);
+#pragma unroll
+        for(int u = u0; u < u0 + 4; ++u) {
+          const int pos = base + 4 * u + g;
+          if(c == 0 && pos < len) sc[pos] = scale * s[u - u0];
+        }
+      }
+    }
+    base += 4 * kAttU;
+    if(base >= len) break;
+    load_rows(kb, k_last, base, kr);
+  }
+  float mx = -__builtin_inff();
+  for(int pos = lane; pos < len; pos += 64) {
+    float z = sc[pos];
+    if(mk) {
+      z = z + (pos < 64 ? mk0 : mk[pos]);
+      sc[pos] = z;
+    }
+    mx = fmaxf(mx, z);
+  }
+  mx = wave_maxf(mx);
+  float sum = 0.0f;
+  float e_first = 0.0f;
+  for(int pos = lane; pos < len; pos += 64) {
+    const float e = expf(sc[pos] - mx);
+    if(pos == lane) e_first = e;
+    sum += e;
+  }
+  sum = wave_sum(sum);
+  for(int pos = lane; pos < len; pos += 64) sc[pos] = (pos == lane ? e_first : expf(sc[pos] - mx)) / sum;
+  v4f o4 = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+  for(int base = 0; base < len; base += 4 * kAttU) {
+    if(base > 0) load_rows(vb, v_last, base, vr);
+#pragma unroll
+    for(int u0 = 0; u0 < kAttU; u0 += 4) {
+      if(base + 4 * u0 < len) {
+        float w[4];
+#pragma unroll
+        for(int u = u0; u < u0 + 4; ++u) w[u - u0] = sc[min(base + 4 * u + g, len4 + 255)];
+#pragma unroll
+        for(int u = u0; u < u0 + 4; ++u) {
+          const float wu = base + 4 * u + g < len ? w[u - u0] : 0.0f;
+          o4.x = fmaf(wu, vr[u].x, o4.x);
+          o4.y = fmaf(wu, vr[u].y, o4.y);
+          o4.z = fmaf(wu, vr[u].z, o4.z);
+          o4.w = fmaf(wu, vr[u].w, o4.w);
+        }
+      }
+    }
+  }
+  reinterpret_cast<v4f*>(part)[g * 16 + c] = o4;
+  const float o = ((part[lane] + part[64 + lane]) + part[128 + lane]) + part[192 + lane];
+  out_row[lane] = o;
+  return fabsf(o);
+}
+
+// NPROJ: 3 (q, k_new, v_new: self-attention, the new key/value row is appended to the caches) or
+// 1 (q only: attention over caches that are complete, e.g. the encoder's).  R: input rows per
+// workgroup, 8 (a wave per row in the attention).
+template <int NPROJ, int R>
+__global__ __launch_bounds__(kProjThreads) void proj_attention_kernel(ProjAttentionArgs p) {
+  static_assert(R == 8, "one wave per row in the attention");
+  typedef int v16i_p __attribute__((ext_vector_type(16)));
+  extern __shared__ __attribute__((aligned(16))) int8_t plds[];
+  __shared__ float red[kProjThreads / 64];
+  const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
+  const int wn = wave % 2, kw = wave / 2, li = lane % 32, lg = lane / 32;
+  const int h = blockIdx.x, m_base = blockIdx.y * R;
+  const int K = p.K, M = p.M, S = K / 32, PW = S / 4, N = p.heads * 64;
+  int8_t* a_lds = plds;                                   // 32 rows x K bytes, operand order
+  int8_t* part_lds = a_lds + 32 * K;                      // NPROJ x 2 x 4 partial tiles of R rows x 128 bytes
+  float* proj_lds = reinterpret_cast<float*>(part_lds + NPROJ * 8 * R * 128);   // [NPROJ][R][64]
+  float* att_lds = proj_lds + NPROJ * R * 64;             // per wave: scores + 256 partial outputs
+
+  // ---- everything this workgroup will need is requested now: abs-max slots, weights, the input
+  //      rows, the quantization multipliers of the weights, bias ----
+  float pm[kAbsmaxSlots / kProjThreads];
+#pragma unroll
+  for(int i = 0; i < kAbsmaxSlots / kProjThreads; ++i) pm[i] = p.partials[min(tid + i * kProjThreads, p.n_partials - 1)];
+  v4i w[NPROJ][8];
+  const int ncol = h * 64 + wn * 32 + li;
+#pragma unroll
+  for(int g = 0; g < NPROJ; ++g) {
+    const int8_t* wrow = p.Bq[g] + b_column_offset(ncol) + lg * 16;
+#pragma unroll
+    for(int pp = 0; pp < 8; ++pp) w[g][pp] = load16(wrow + (size_t)min(kw * PW + pp, S - 1) * 32u * (size_t)N);
+  }
+  // a quad of lanes takes four consecutive 16-value groups of one row: 64 contiguous bytes per load
+  const int grp = (tid / 4) * 4, qlane = tid % 4;
+  const int r_in = grp / (2 * S), c16 = grp % (2 * S);
+  const bool has_in = r_in < R;
+  v4f in[4];
+  {
+    const int m = min(m_base + min(r_in, R - 1), M - 1);
+    const float* src = p.A + (size_t)m * (size_t)K + (size_t)c16 * 16 + qlane * 4;
+#pragma unroll
+    for(int e = 0; e < 4; ++e) in[e] = *reinterpret_cast<const v4f*>(src + e * 16);
+  }
+  float bqm[NPROJ];
+#pragma unroll
+  for(int g = 0; g < NPROJ; ++g) bqm[g] = tail_quant_mult(p.Bq[g], (size_t)K * (size_t)N);
+  // the (up to two) pieces of four outputs this thread finishes in step 4, and their bias
+  constexpr int kItems = NPROJ * 2 * R * 8;
+  v4f bias4[2];
+#pragma unroll
+  for(int it = 0; it < 2; ++it) {
+    const int item = min(it * kProjThreads + tid, kItems - 1);
+    const int tg = item / (R * 8), pc = item % 8;
+    const float* b = p.bias[tg / 2];
+    bias4[it] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+    if(b) bias4[it] = *reinterpret_cast<const v4f*>(b + h * 64 + (tg % 2) * 32 + pc * 4);
+  }
+
+  // ---- 1, 2: abs-max, quantize into LDS ----
+  float amax = 0.0f;
+#pragma unroll
+  for(int i = 0; i < kAbsmaxSlots / kProjThreads; ++i) amax = fmaxf(amax, pm[i]);
+  amax = block_max(amax, red);
+  const float aqm = quant_mult_from_maxabs(amax);
+  const bool finite = aqm < __builtin_inff();
+  float unquant[NPROJ];
+#pragma unroll
+  for(int g = 0; g < NPROJ; ++g) unquant[g] = unquant_mult(aqm, bqm[g], 1.0f);
+  if(has_in) {
+    uint32_t q[4];
+#pragma unroll
+    for(int e = 0; e < 4; ++e) q[e] = finite ? quantize_pack4_finite(in[e], aqm) : quantize_pack4(in[e], aqm);
+    const int slot0 = (c16 / 2) * 64, x = r_in ^ proj_row_key(c16);
+    const int m = m_base + r_in;
+#pragma unroll
+    for(int e = 0; e < 4; ++e) {
+      const int sw = slot0 + (e / 2) * 64 + (e % 2) * 32 + (x ^ e);
+      *reinterpret_cast<uint32_t*>(a_lds + sw * 16 + qlane * 4) = q[e];
+      if(p.aq_out && h == 0 && m < M)
+        *reinterpret_cast<uint32_t*>(p.aq_out + (size_t)m * (size_t)K + (size_t)(c16 + e) * 16 + qlane * 4) = q[e];
+    }
+  }
+  if(p.aq_out && h == 0 && blockIdx.y == 0 && tid == 0) *reinterpret_cast<float*>(p.aq_out + (size_t)M * K) = aqm;
+  __syncthreads();
+
+  // ---- 3: multiply (rows R .. 31 of the operand are whatever LDS held: they only feed output rows
+  //      that are never looked at) ----
+  v16i_p acc[NPROJ];
+#pragma unroll
+  for(int g = 0; g < NPROJ; ++g)
+#pragma unroll
+    for(int v = 0; v < 16; ++v) acc[g][v] = 0;
+#pragma unroll
+  for(int pp = 0; pp < 8; ++pp) {
+    if(pp < PW) {   // (the same for the whole workgroup)
+      const int s = kw * PW + pp;
+      const v4i a = *reinterpret_cast<const v4i*>(a_lds + s * 1024 + (lg * 32 + (li ^ proj_row_key(2 * s + lg))) * 16);
+#pragma unroll
+      for(int g = 0; g < NPROJ; ++g) acc[g] = __builtin_amdgcn_mfma_i32_32x32x32_i8(w[g][pp], a, acc[g], 0, 0, 0);
+    }
+  }
+  // accumulator value v of lane (li, lg): input row li, column 8 * (v / 4) + 4 * lg + v % 4 of the
+  // wave's 32; a tile row is 128 bytes, its eight 16-byte pieces XOR-permuted by the row number
+  if(li < R) {
+#pragma unroll
+    for(int g = 0; g < NPROJ; ++g) {
+      int8_t* mine = part_lds + ((g * 2 + wn) * 4 + kw) * (R * 128);
+#pragma unroll
+      for(int q = 0; q < 4; ++q)
+        *reinterpret_cast<v4i*>(mine + li * 128 + (((2 * q + lg) ^ (li & 7)) * 16)) =
+            v4i{acc[g][4 * q], acc[g][4 * q + 1], acc[g][4 * q + 2], acc[g][4 * q + 3]};
+    }
+  }
+  __syncthreads();
+
+  // ---- 4: add the four K ranges, dequantize, keep in LDS, append k_new / v_new to the caches ----
+#pragma unroll
+  for(int it = 0; it < 2; ++it) {
+    const int item = it * kProjThreads + tid;
+    if(item < kItems) {
+      const int tg = item / (R * 8), r = (item / 8) % R, pc = item % 8;
+      const int g = tg / 2, col = (tg % 2) * 32 + pc * 4;
+      const int8_t* src = part_lds + (tg * 4) * (R * 128) + r * 128 + ((pc ^ (r & 7)) * 16);
+      v4i sum = *reinterpret_cast<const v4i*>(src);
+#pragma unroll
+      for(int t = 1; t < 4; ++t) sum += *reinterpret_cast<const v4i*>(src + t * (R * 128));
+      float uq = unquant[0];
+      if constexpr(NPROJ == 3) uq = g == 0 ? unquant[0] : (g == 1 ? unquant[1] : unquant[2]);
+      const bool has_bias = p.bias[g] != nullptr;
+      const float b[4] = {bias4[it].x, bias4[it].y, bias4[it].z, bias4[it].w};
+      float y[4];
+#pragma unroll
+      for(int e = 0; e < 4; ++e) {
+        y[e] = (float)sum[e] * uq;
+        if(has_bias) y[e] = y[e] + b[e];
+      }
+      const v4f yv = v4f{y[0], y[1], y[2], y[3]};
+      *reinterpret_cast<v4f*>(proj_lds + (g * R + r) * 64 + col) = yv;
+      const int m = m_base + r;
+      if(m < M) {
+        if(p.proj_out[g]) *reinterpret_cast<v4f*>(p.proj_out[g] + (size_t)m * (size_t)N + h * 64 + col) = yv;
+        if(NPROJ == 3 && g > 0) {
+          float* cache = g == 1 ? p.k_cache : p.v_cache;
+          const size_t entry = (size_t)m * (size_t)p.heads + (size_t)h;
+          *reinterpret_cast<v4f*>(cache + (entry * (size_t)p.kv_cap + (size_t)(p.len - 1)) * 64 + col) = yv;
+        }
+      }
+    }
+  }
+  __syncthreads();
+
+  // ---- 5: the attention of row `wave` ----
+  const int rows_total = M * p.heads;
+  if(p.absmax_out && blockIdx.x == 0 && blockIdx.y == 0)   // slots past the last query row
+    for(int sl = rows_total + tid; sl < kAbsmaxSlots; sl += kProjThreads) p.absmax_out[sl] = 0.0f;
+  const int m = m_base + wave;
+  if(wave < R && m < M) {   // (whole waves)
+    const unsigned wr = (unsigned)m * (unsigned)p.heads + (unsigned)h;
+    const unsigned entry = wr < p.batchKV ? wr : wr % p.batchKV;
+    const float* kb = p.k_cache + (size_t)entry * p.kv_cap * 64;
+    const float* vb = p.v_cache + (size_t)entry * p.kv_cap * 64;
+    const float* q = proj_lds + wave * 64;
+    const float* k_last = NPROJ == 3 ? proj_lds + (R + wave) * 64 : kb + (size_t)(p.len - 1) * 64;
+    const float* v_last = NPROJ == 3 ? proj_lds + (2 * R + wave) * 64 : vb + (size_t)(p.len - 1) * 64;
+    const float* mk = nullptr;
+    if(p.mask) {
+      unsigned mask_row = (unsigned)m;
+      if(mask_row >= p.n_masks) mask_row %= p.n_masks;
+      mk = p.mask + (size_t)mask_row * p.len;
+    }
+    const int len4 = (p.len + 3) & ~3;
+    float* sc = att_lds + wave * (len4 + 256);
+    float omax = attention_row64(q, kb, vb, k_last, v_last, mk, p.len, p.att_scale, sc, sc + len4,
+                                 p.out + (size_t)wr * 64, lane);
+    if(p.absmax_out) {
+      omax = wave_maxf(omax);
+      if(lane == 0) p.absmax_out[wr] = omax;
+    }
   }
 }
 
@@ -1717,6 +2050,85 @@ static int attention_impl(const float* q, float* k, float* v, const float* mask,
                        k_new, v_new, mask, (unsigned)n_masks, (unsigned)rows_per_mask, out, (unsigned)rows_total,
                        (unsigned)batchKV, (int)m, (int)len, (int)kv_capacity, (int)dk, scale, absmax_out, ancestors,
                        1u);
+  MH_HIP(hipGetLastError());
+  return MARIAN_HIP_OK;
+}
+
+int marian_hip_int8_proj_attention(const float* A, int8_t* Aq, int64_t n_proj, const int8_t* const* Bq,
+                                   const float* const* bias, float* const* proj_out, int64_t M, int64_t K,
+                                   int64_t heads, float* k_cache, float* v_cache, int64_t batchKV, int64_t len,
+                                   int64_t kv_capacity, const float* mask, int64_t n_masks, float att_scale,
+                                   float* out, const float* absmax_in, float* absmax_out, void* workspace,
+                                   size_t workspace_bytes, void* stream) {
+  if(n_proj != 1 && n_proj != 3) return MARIAN_HIP_ERR_SHAPE;
+  if(M < 0 || K <= 0 || heads <= 0 || (K % 128) != 0 || K > kProjMaxK) return MARIAN_HIP_ERR_SHAPE;
+  if(len <= 0 || len > kProjMaxLen || kv_capacity < len || batchKV <= 0) return MARIAN_HIP_ERR_SHAPE;
+  if(mask && n_masks <= 0) return MARIAN_HIP_ERR_SHAPE;
+  if(M == 0) return MARIAN_HIP_OK;
+  if(!A || !Aq || !Bq || !k_cache || !v_cache || !out) return MARIAN_HIP_ERR_NULL;
+  if(M * heads > kMaxElemsOps / 64 || batchKV * kv_capacity > kMaxElemsOps / 64 || M * K > kMaxElemsOps ||
+     K * heads * 64 > kMaxElemsOps || n_masks > 2147483647LL)
+    return MARIAN_HIP_ERR_RANGE;
+  // the self-attention form appends to the caches: every query row needs an entry of its own
+  if(n_proj == 3 && batchKV != M * heads) return MARIAN_HIP_ERR_SHAPE;
+  if(absmax_out && M * heads > kAbsmaxSlots) return MARIAN_HIP_ERR_RANGE;
+  if(!aligned16(A) || !aligned16(Aq) || !aligned16(k_cache) || !aligned16(v_cache) || !aligned16(out))
+    return MARIAN_HIP_ERR_ALIGN;
+  if((mask && !aligned4(mask)) || (absmax_in && !aligned4(absmax_in)) || (absmax_out && !aligned4(absmax_out)))
+    return MARIAN_HIP_ERR_ALIGN;
+  ProjAttentionArgs p;
+  for(int g = 0; g < 3; ++g) {
+    p.Bq[g] = nullptr; p.bias[g] = nullptr; p.proj_out[g] = nullptr;
+  }
+  for(int64_t g = 0; g < n_proj; ++g) {
+    if(!Bq[g]) return MARIAN_HIP_ERR_NULL;
+    p.Bq[g] = Bq[g];
+    p.bias[g] = bias ? bias[g] : nullptr;
+    p.proj_out[g] = proj_out ? proj_out[g] : nullptr;
+    if(!aligned16(p.Bq[g]) || (p.bias[g] && !aligned16(p.bias[g])) || (p.proj_out[g] && !aligned16(p.proj_out[g])))
+      return MARIAN_HIP_ERR_ALIGN;
+  }
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  p.A = A; p.aq_out = Aq;
+  if(absmax_in) {
+    p.partials = absmax_in;
+    p.n_partials = kAbsmaxSlots;
+  } else {   // nobody left the abs-max of the input: a launch for it
+    if(!workspace) return MARIAN_HIP_ERR_NULL;
+    if(workspace_bytes < kWorkspaceBytes) return MARIAN_HIP_ERR_WORKSPACE;
+    if(!aligned4(workspace)) return MARIAN_HIP_ERR_ALIGN;
+    float* partials = reinterpret_cast<float*>(workspace);
+    int n_partials = 0;
+    const int pst = launch_absmax_partials(A, (size_t)M * (size_t)K, partials, &n_partials, stream);
+    if(pst != MARIAN_HIP_OK) return pst;
+    p.partials = partials;
+    p.n_partials = n_partials;
+  }
+  p.M = (int)M; p.K = (int)K; p.heads = (int)heads;
+  p.k_cache = k_cache; p.v_cache = v_cache; p.batchKV = (unsigned)batchKV;
+  p.len = (int)len; p.kv_cap = (int)kv_capacity;
+  p.mask = mask; p.n_masks = mask ? (unsigned)n_masks : 1u;
+  p.att_scale = att_scale; p.out = out; p.absmax_out = absmax_out;
+  constexpr int R = 8;
+  const int len4 = ((int)len + 3) & ~3;
+  const size_t lds = (size_t)32 * (size_t)K + (size_t)n_proj * 8 * R * 128 + (size_t)n_proj * R * 64 * 4 +
+                     (size_t)R * (size_t)(len4 + 256) * 4;
+  {   // the kernels' dynamic LDS limit, raised once per device (one bit per device)
+    static std::atomic<uint64_t> lds_done{0};
+    int dev = 0;
+    MH_HIP(hipGetDevice(&dev));
+    if(dev < 0 || dev >= 64) return MARIAN_HIP_ERR_RANGE;
+    if(!(lds_done.load(std::memory_order_acquire) & (1ull << dev))) {
+      MH_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(proj_attention_kernel<1, R>),
+                                 hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024));
+      MH_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(proj_attention_kernel<3, R>),
+                                 hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024));
+      lds_done.fetch_or(1ull << dev, std::memory_order_release);
+    }
+  }
+  const dim3 grid((unsigned)heads, (unsigned)((M + R - 1) / R));
+  if(n_proj == 3) hipLaunchKernelGGL((proj_attention_kernel<3, R>), grid, dim3(kProjThreads), lds, st, p);
+  else hipLaunchKernelGGL((proj_attention_kernel<1, R>), grid, dim3(kProjThreads), lds, st, p);
   MH_HIP(hipGetLastError());
   return MARIAN_HIP_OK;
 }

@@ -130,7 +130,7 @@ class DecoderStep:
         self.state, self.state_next = self.state_next, self.state
         self._cache_views()
 
-    def step(self, s, gemm_only=False, chained=True, grouped=True, fused_tail=False, select=False):
+    def step(self, s, gemm_only=False, chained=True, grouped=True, fused_tail=False, select=False, fused_attention=True):
         """chained: every tensor that feeds an affine call leaves its abs-max where it is
         produced (layer norm, attention, the ReLU GEMM), so those calls skip their abs-max pass.
         grouped: the self-attention projections Wq, Wk, Wv (one input, three weight matrices,
@@ -138,7 +138,9 @@ class DecoderStep:
         fused_tail: log-softmax and n-best in one launch (the log-probabilities are not written);
         the step then returns (scores, keys) of the n-best instead of the log-probabilities.
         select: the step starts with the selection of the surviving hypotheses' cached keys and
-        values by the back-pointers self.hyp_indices, as a beam-search step does."""
+        values by the back-pointers self.hyp_indices, as a beam-search step does.
+        fused_attention: the projections in front of an attention (Wq, Wk, Wv; the context
+        attention's Wq) and the attention itself are one launch each (ops.ProjectedAttention)."""
         integer, ops = self.integer, self.ops
         W = self.sets[s % len(self.sets)]
         tr = self.trace
@@ -161,34 +163,49 @@ class DecoderStep:
                 x, xmax = x
             rec("embed", E=self.E, ids=self.words, scale=self.emb_scale, signal=self.signal, out=x, position=self.T - 1)
         for li, ly in enumerate(W["layers"]):
-            if grouped:   # one abs-max, one quantization, one launch for the three projections
-                (q, k, v), _ = integer.affine_f32_grouped(x, [ly["Wq"], ly["Wk"], ly["Wv"]], absmax=xmax)
-            else:
-                q, _ = integer.affine_f32(x, *ly["Wq"], absmax=xmax)
-                k, _ = integer.affine_f32(x, *ly["Wk"], absmax=xmax)
-                v, _ = integer.affine_f32(x, *ly["Wv"], absmax=xmax)
-            for name, t in (("Wq", q), ("Wk", k), ("Wv", v)):
-                rec("affine", a=x, w=ly[name], out=t, relu=False)
             omax = x1max = comax = x2max = f1max = None
-            if gemm_only:
-                o = q
-            else:
-                # head split of a single position is a view; the attention call also appends the
-                # new key/value to the cache
+            fuse = fused_attention and not gemm_only and not self.by_ancestors and ch
+            if fuse:   # q, k, v and the self-attention over the cache (the new position appended) in one launch
                 if tr is not None:
                     k_before, v_before = self.Kself[li].clone(), self.Vself[li].clone()
-                if self.by_ancestors:
-                    o = ops.AttentionByAncestors(q.view(M * H, 1, dk), self.Kself[li], self.Vself[li], self.anc, self.T,
-                                                 k.view(M * H, dk), v.view(M * H, dk), want_absmax=ch)
-                else:
-                    o = ops.Attention(q.view(M * H, 1, dk), self.Kself[li], self.Vself[li], want_absmax=ch,
-                                      kNew=k.view(M * H, dk), vNew=v.view(M * H, dk), kvLen=self.T)
-                if ch:
-                    o, omax = o
+                res = ops.ProjectedAttention(x, [ly["Wq"], ly["Wk"], ly["Wv"]], self.Kself[li], self.Vself[li], H,
+                                             kvLen=self.T, absmax=xmax, want_absmax=True, want_projections=tr is not None)
+                o, omax = res[0], res[2]
                 if tr is not None:
+                    q, k, v = res[3]
+                    for name, t in (("Wq", q), ("Wk", k), ("Wv", v)):
+                        rec("affine", a=x, w=ly[name], out=t, relu=False)
                     rec("self_attention", q=q, k_new=k, v_new=v, k_cache=k_before, v_cache=v_before,
                         k_after=self.Kself[li], v_after=self.Vself[li], out=o, len=self.T)
                 o = o.view(M, d)
+            else:
+                if grouped:   # one abs-max, one quantization, one launch for the three projections
+                    (q, k, v), _ = integer.affine_f32_grouped(x, [ly["Wq"], ly["Wk"], ly["Wv"]], absmax=xmax)
+                else:
+                    q, _ = integer.affine_f32(x, *ly["Wq"], absmax=xmax)
+                    k, _ = integer.affine_f32(x, *ly["Wk"], absmax=xmax)
+                    v, _ = integer.affine_f32(x, *ly["Wv"], absmax=xmax)
+                for name, t in (("Wq", q), ("Wk", k), ("Wv", v)):
+                    rec("affine", a=x, w=ly[name], out=t, relu=False)
+                if gemm_only:
+                    o = q
+                else:
+                    # head split of a single position is a view; the attention call also appends the
+                    # new key/value to the cache
+                    if tr is not None:
+                        k_before, v_before = self.Kself[li].clone(), self.Vself[li].clone()
+                    if self.by_ancestors:
+                        o = ops.AttentionByAncestors(q.view(M * H, 1, dk), self.Kself[li], self.Vself[li], self.anc, self.T,
+                                                     k.view(M * H, dk), v.view(M * H, dk), want_absmax=ch)
+                    else:
+                        o = ops.Attention(q.view(M * H, 1, dk), self.Kself[li], self.Vself[li], want_absmax=ch,
+                                          kNew=k.view(M * H, dk), vNew=v.view(M * H, dk), kvLen=self.T)
+                    if ch:
+                        o, omax = o
+                    if tr is not None:
+                        rec("self_attention", q=q, k_new=k, v_new=v, k_cache=k_before, v_cache=v_before,
+                            k_after=self.Kself[li], v_after=self.Vself[li], out=o, len=self.T)
+                    o = o.view(M, d)
             a, _ = integer.affine_f32(o, *ly["Wo"], absmax=omax)
             rec("affine", a=o, w=ly["Wo"], out=a, relu=False)
             if gemm_only:
@@ -198,17 +215,27 @@ class DecoderStep:
                 if ch:
                     x1, x1max = x1
                 rec("layer_norm", x=a, add=x, gamma=ly["ln1"][0], beta=ly["ln1"][1], out=x1)
-            cq, _ = integer.affine_f32(x1, *ly["cWq"], absmax=x1max)
-            rec("affine", a=x1, w=ly["cWq"], out=cq, relu=False)
-            if gemm_only:
-                co = cq
-            else:
-                co = ops.Attention(cq.view(M * H, 1, dk), self.Kenc[li], self.Venc[li], self.mask,
-                                   rowsPerMask=H, want_absmax=ch)
-                if ch:
-                    co, comax = co
-                rec("context_attention", q=cq, k=self.Kenc[li], v=self.Venc[li], mask=self.mask, out=co)
+            if fused_attention and not gemm_only and ch:   # the context attention's Wq and the attention in one launch
+                res = ops.ProjectedAttention(x1, [ly["cWq"]], self.Kenc[li], self.Venc[li], H, mask=self.mask,
+                                             absmax=x1max, want_absmax=True, want_projections=tr is not None)
+                co, comax = res[0], res[2]
+                if tr is not None:
+                    cq = res[3][0]
+                    rec("affine", a=x1, w=ly["cWq"], out=cq, relu=False)
+                    rec("context_attention", q=cq, k=self.Kenc[li], v=self.Venc[li], mask=self.mask, out=co)
                 co = co.view(M, d)
+            else:
+                cq, _ = integer.affine_f32(x1, *ly["cWq"], absmax=x1max)
+                rec("affine", a=x1, w=ly["cWq"], out=cq, relu=False)
+                if gemm_only:
+                    co = cq
+                else:
+                    co = ops.Attention(cq.view(M * H, 1, dk), self.Kenc[li], self.Venc[li], self.mask,
+                                       rowsPerMask=H, want_absmax=ch)
+                    if ch:
+                        co, comax = co
+                    rec("context_attention", q=cq, k=self.Kenc[li], v=self.Venc[li], mask=self.mask, out=co)
+                    co = co.view(M, d)
             ca, _ = integer.affine_f32(co, *ly["cWo"], absmax=comax)
             rec("affine", a=co, w=ly["cWo"], out=ca, relu=False)
             if gemm_only:

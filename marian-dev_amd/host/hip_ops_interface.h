@@ -116,6 +116,34 @@ inline void Attention(Backend& be, Tensor& out, const Tensor& q, Tensor& k, Tens
       kNew ? kNew->data<float>() : nullptr, vNew ? vNew->data<float>() : nullptr, be.stream()));
 }
 
+// The projections in front of an attention and the attention itself for one new target position
+// per row of a, in one launch (reference src/models/transformer.h:279-348).  weights: {Wq} - caches
+// complete, e.g. the encoder's - or {Wq, Wk, Wv} - self-attention, the new key and value go into
+// the caches at position kvLen - 1; biases: one entry per matrix (null entries allowed) or empty.
+// a [M, K] float32; aQuant: the prepareA node's tensor; k, v [entries, capacity, 64]; out [M, heads * 64].
+inline void ProjectedAttention(TensorAllocator& ta, Tensor& out, const Tensor& a, Tensor& aQuant,
+                               const std::vector<const Tensor*>& weights, const std::vector<const Tensor*>& biases,
+                               Tensor& k, Tensor& v, int64_t heads, int64_t kvLen = 0, const Tensor* mask = nullptr,
+                               const Tensor* absmaxIn = nullptr, Tensor* absmaxOut = nullptr) {
+  if((weights.size() != 1 && weights.size() != 3) || (!biases.empty() && biases.size() != weights.size()))
+    abortWith("ProjectedAttention: one projection (q) or three (q, k, v), one bias entry each");
+  if(k.shape.size() != 3 || k.shape[2] != 64 || v.shape != k.shape) abortWith("ProjectedAttention expects caches [entries, capacity, 64]");
+  void* ws = ta.workspace();   // (may allocate and move the slab: before any pointer is read)
+  const int8_t* bq[3] = {nullptr, nullptr, nullptr};
+  const float* bi[3] = {nullptr, nullptr, nullptr};
+  for(size_t g = 0; g < weights.size(); ++g) {
+    integer::checkB(*weights[g]);
+    bq[g] = weights[g]->data<int8_t>();
+    if(!biases.empty() && biases[g]) bi[g] = biases[g]->data<float>();
+  }
+  MARIAN_HIP_CHECK(marian_hip_int8_proj_attention(
+      a.data<float>(), aQuant.data<int8_t>(), (int64_t)weights.size(), bq, bi, nullptr, rows(a), cols(a), heads,
+      k.data<float>(), v.data<float>(), k.shape[0], kvLen ? kvLen : k.shape[1], k.shape[1],
+      mask ? mask->data<float>() : nullptr, mask ? (int64_t)rows(*mask) : 0, 0.125f, out.data<float>(),
+      absmaxIn ? absmaxIn->data<float>() : nullptr, absmaxOut ? absmaxOut->data<float>() : nullptr, ws,
+      ta.workspaceBytes(), ta.backend().stream()));
+}
+
 // Self-attention of a decoding step on caches that are never moved: cached position p of hypothesis
 // h is read from the entry of hypothesis ancestors[h, p] (uint32 [hypotheses, capacity]); kNew / vNew
 // become position kvLen - 1 of the hypotheses' own entries.  q, kNew, vNew, out [hyps * heads, 1 or -, 64].

@@ -501,6 +501,43 @@ int main(int argc, char** argv) {
       expect(sameBits(download<float>(be, o2, qv.size()), download<float>(be, o1, qv.size())),
              "AttentionByAncestors: the attention on the copied caches, bit for bit");
     }
+
+    {   // projections + attention in one launch against the separate wrappers: 5 rows of 128 values, 2 heads (N = 128)
+      const int hd = 2, NN = hd * 64, Mr = 5, cap = 6, len = 4, K5 = 128;
+      if((size_t)Mr * K5 <= A.size()) {
+        std::vector<float> wq((size_t)K5 * NN), wk(wq.size()), wv(wq.size()), kc((size_t)Mr * hd * cap * 64), vc(kc.size());
+        uint32_t r3 = 4242u;
+        auto nx = [&]() { r3 = r3 * 1664525u + 1013904223u; return (float)(r3 >> 8) * (1.0f / 8388608.0f) - 1.0f; };
+        for(auto& x : wq) x = 0.02f * nx();
+        for(auto& x : wk) x = 0.02f * nx();
+        for(auto& x : wv) x = 0.02f * nx();
+        for(auto& x : kc) x = nx();
+        for(auto& x : vc) x = nx();
+        std::vector<float> a5(A.begin(), A.begin() + (size_t)Mr * K5);
+        Tensor a5t = upload(ta, a5, {Mr, K5}, Type::float32);
+        Tensor wqf = upload(ta, wq, {K5, NN}, Type::float32), wkf = upload(ta, wk, {K5, NN}, Type::float32),
+               wvf = upload(ta, wv, {K5, NN}, Type::float32);
+        Tensor wqq, wkq, wvq, aqa, aqb, q5, k5, v5, o1, o2;
+        for(Tensor* t : {&wqq, &wkq, &wvq}) ta.allocate(*t, {K5, NN}, Type::intgemm8);
+        integer::prepareB(ta, wqf, wqq);
+        integer::prepareB(ta, wkf, wkq);
+        integer::prepareB(ta, wvf, wvq);
+        ta.allocate(aqa, {Mr, K5}, Type::intgemm8);
+        ta.allocate(aqb, {Mr, K5}, Type::intgemm8);
+        for(Tensor* t : {&q5, &k5, &v5, &o1, &o2}) ta.allocate(*t, {Mr, NN}, Type::float32);
+        Tensor kA = upload(ta, kc, {Mr * hd, cap, 64}, Type::float32), vA = upload(ta, vc, {Mr * hd, cap, 64}, Type::float32);
+        Tensor kB = upload(ta, kc, {Mr * hd, cap, 64}, Type::float32), vB = upload(ta, vc, {Mr * hd, cap, 64}, Type::float32);
+        integer::affineOrDotGrouped(ta, a5t, aqa, {&wqq, &wkq, &wvq}, {}, {&q5, &k5, &v5});
+        Tensor q3 = q5, kn = k5, vn = v5, o13 = o1;
+        q3.shape = {Mr * hd, 1, 64}; o13.shape = q3.shape; kn.shape = {Mr * hd, 64}; vn.shape = kn.shape;
+        Attention(be, o13, q3, kA, vA, 0.125f, nullptr, 1, nullptr, &kn, &vn, len);
+        ProjectedAttention(ta, o2, a5t, aqb, {&wqq, &wkq, &wvq}, {}, kB, vB, hd, len);
+        expect(sameBits(download<float>(be, o2, (size_t)Mr * NN), download<float>(be, o1, (size_t)Mr * NN)) &&
+                   sameBits(download<float>(be, kB, kc.size()), download<float>(be, kA, kc.size())) &&
+                   sameBits(download<int8_t>(be, aqb, (size_t)Mr * K5 + 4), download<int8_t>(be, aqa, (size_t)Mr * K5 + 4)),
+               "ProjectedAttention: the grouped affine + Attention, output, caches and quantized input bit for bit");
+      }
+    }
     be.synchronize();
     std::printf("host_check: %d failure(s), slab moved %zu times -> %s\n", failures,
                 ta.allocator()->device()->moves(), failures == 0 ? "OK" : "FAILED");

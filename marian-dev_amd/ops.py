@@ -253,6 +253,70 @@ def Attention(q, k, v, mask=None, rowsPerMask=1, want_absmax=False, kNew=None, v
     return (out, omax) if want_absmax else out
 
 
+def ProjectedAttention(x, weights, k, v, heads, kvLen=None, mask=None, absmax=None, want_absmax=False,
+                       want_projections=False):
+    """The projections in front of an attention and the attention itself for one new target
+    position, in one launch (reference src/models/transformer.h:279-348: MultiHead's affine nodes
+    for q - and, in self-attention, k and v - then the head split and Attention()).
+    x [M, K] float32; weights: [(Wq, bq)] - attention over caches that are complete (the encoder's
+    keys and values) - or [(Wq, bq), (Wk, bk), (Wv, bv)] - self-attention: the new key and value
+    are appended to the caches k, v at position kvLen - 1 (quantized weights, bias or None each).
+    k, v [entries, capacity, 64] with kvLen positions in use; mask [n, len] or None, one row per
+    sentence (query row r of [M * heads] uses row (r // heads) % n).  absmax: the AbsMax the producer
+    of x left.  Returns (out [M, heads * 64], aQuant) and, when asked for, the AbsMax of out and
+    the projections themselves - bit for bit what affine_f32_grouped / affine_f32 followed by
+    Attention give."""
+    import ctypes
+    from . import integer
+    x = _f32c(x, "ProjectedAttention")
+    be = _backend_of(x)
+    n = len(weights)
+    _abort_if(n not in (1, 3), "ProjectedAttention: one projection (q) or three (q, k, v), got {}", n)
+    K = x.shape[-1]
+    M = x.numel() // K if x.numel() else 0
+    N = heads * 64
+    _abort_if(not (k.is_contiguous() and v.is_contiguous()) or k.dtype != torch.float32 or v.dtype != torch.float32,
+              "ProjectedAttention: the key/value caches must be contiguous float32{}", "")
+    _abort_if(k.shape[-1] != 64 or tuple(k.shape) != tuple(v.shape), "ProjectedAttention: head size 64, got caches {} {}",
+              tuple(k.shape), tuple(v.shape))
+    cap = k.shape[-2]
+    L = cap if kvLen is None else int(kvLen)
+    batchKV = k.numel() // (cap * 64)
+    aQuant = integer.QTensor.empty(x.shape, integer.Type.intgemm8, x.device)
+    Bq_arr, bias_arr, proj_arr = (ctypes.c_void_p * n)(), (ctypes.c_void_p * n)(), (ctypes.c_void_p * n)()
+    keep, projections = [], []
+    for g, (bQuant, bias) in enumerate(weights):
+        integer._check_weights(bQuant)
+        _abort_if(integer.rows(bQuant) != K or integer.cols(bQuant) != N, "ProjectedAttention: weights {} vs [{}, {}]",
+                  tuple(bQuant.shape), K, N)
+        Bq_arr[g] = bQuant.data_ptr()
+        if bias is not None:
+            bias = _f32c(bias, "ProjectedAttention")
+            keep.append(bias)
+        bias_arr[g] = None if bias is None else bias.data_ptr()
+        if want_projections:
+            projections.append(torch.empty(tuple(x.shape[:-1]) + (N,), dtype=torch.float32, device=x.device))
+        proj_arr[g] = projections[g].data_ptr() if want_projections else None
+    n_masks = 0
+    if mask is not None:
+        mask = _f32c(mask, "ProjectedAttention").reshape(-1, L)
+        n_masks = mask.shape[0]
+    out = torch.empty(tuple(x.shape[:-1]) + (N,), dtype=torch.float32, device=x.device)
+    omax = AbsMax(x.device) if want_absmax else None
+    st = be.lib.marian_hip_int8_proj_attention(
+        x.data_ptr(), aQuant.data_ptr(), n, Bq_arr, bias_arr, proj_arr, M, K, heads, k.data_ptr(), v.data_ptr(), batchKV,
+        L, cap, None if mask is None else mask.data_ptr(), n_masks, 1.0 / 8.0, out.data_ptr(),
+        None if absmax is None else absmax.data_ptr(), None if omax is None else omax.data_ptr(),
+        be.workspace.data_ptr(), be.workspace_bytes, be.stream())
+    _lib.check(st, "ProjectedAttention")
+    res = (out, aQuant)
+    if want_absmax:
+        res += (omax,)
+    if want_projections:
+        res += (projections,)
+    return res
+
+
 def AttentionByAncestors(q, k, v, ancestors, kvLen, kNew, vNew, want_absmax=False):
     """Self-attention of a decoding step on caches that are never moved (no counterpart in the
     reference, which copies the surviving hypotheses' states, src/rnn/types.h:22-42): cached
