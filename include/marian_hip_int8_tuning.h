@@ -70,6 +70,16 @@ int marian_hip_probe_mfma(const void* data, int iters, int workgroups, long long
 int marian_hip_probe_mix(const void* src, size_t span_bytes, size_t stagger_bytes, int waves, int reads, int mfmas, int dmas, int gloads,
                          int split, int iters, int workgroups, long long* clocks, int* sink, void* stream);
 
+/*
+ * The hand-over of candidates between the workgroups of marian_hip_nbest_beams and
+ * marian_hip_logsoftmax_nbest_beams, PROCESS-WIDE: 0 (default) = what the shipped library does -
+ * device-scope stores, a wait for their acknowledgement, a relaxed counter; 1 = the counter update
+ * as an acquire-release operation at device scope, i.e. with the cache write-back and invalidation
+ * the language's memory model asks for (about 8 us slower per call).  The two forms must give the
+ * same bits; tests compare them.  Returns the previous value.
+ */
+int marian_hip_nbest_set_fenced(int on);
+
 #ifdef __cplusplus
 }
 #endif

@@ -77,6 +77,7 @@ TUNING_SIGNATURES = {
     "marian_hip_probe_stream": (_i, [_vp, _sz, _vp, _sz, _i, _i, _i, _i, _vp]),
     "marian_hip_probe_mfma": (_i, [_vp, _i, _i, _vp, _vp, _vp]),
     "marian_hip_probe_mix": (_i, [_vp, _sz, _sz, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp]),
+    "marian_hip_nbest_set_fenced": (_i, [_i]),
 }
 
 ABSMAX_SLOTS = 2048   # MARIAN_HIP_ABSMAX_SLOTS

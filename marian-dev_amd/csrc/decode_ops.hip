@@ -986,9 +986,9 @@ __global__ __launch_bounds__(kProjThreads) void proj_attention_kernel(ProjAttent
   const int ncol = h * 64 + wn * 32 + li;
 #pragma unroll
   for(int g = 0; g < NPROJ; ++g) {
-    const int8_t* wrow = p.Bq[g] + b_column_offset(ncol) + lg * 16;
+    const int8_t* wrow = p.Bq[g] + stream32_lane_offset(ncol, lg);
 #pragma unroll
-    for(int pp = 0; pp < 8; ++pp) w[g][pp] = load16(wrow + (size_t)min(kw * PW + pp, S - 1) * 32u * (size_t)N);
+    for(int pp = 0; pp < 8; ++pp) w[g][pp] = load16(wrow + (size_t)stream32_clamped_substep(kw * PW + pp, S) * 32u * (size_t)N);
   }
   // a quad of lanes takes four consecutive 16-value groups of one row: 64 contiguous bytes per load
   const int grp = (tid / 4) * 4, qlane = tid % 4;
@@ -1440,20 +1440,18 @@ __global__ __launch_bounds__(1024) void nbest_kernel(const float* __restrict__ s
 // it; a wave's vmcnt reaches zero only once each of its stores has been acknowledged from there; an
 // agent-scope load reads from there too.  So: candidates stored (agent scope) -> vmcnt(0) in every
 // wave -> workgroup barrier -> counter incremented; the workgroup that reads parts - 1 from the
-// counter then loads (agent scope) candidates that are all in memory already.  Building with
-// -DMARIAN_HIP_NBEST_FENCED makes the counter update an acquire-release operation instead (the
-// compiler then adds the cache write-back / invalidate the language-level memory model asks for;
-// ~8 us slower): if results ever differ between the two builds, the hand-over is at fault and not
-// the selection.  rowLen: length of an entry's whole row (keys are b * rowLen + position).
+// counter then loads (agent scope) candidates that are all in memory already.  FENCED makes the
+// counter update an acquire-release operation instead (the compiler then adds the cache write-back /
+// invalidate the language-level memory model asks for; ~8 us slower).  The tuning build holds both
+// forms (marian_hip_nbest_set_fenced) and a GPU test compares them: if results ever differ, the
+// hand-over is at fault and not the selection.  rowLen: length of an entry's whole row (keys are
+// b * rowLen + position).
+template <bool FENCED>
 __device__ __forceinline__ void nbest_hand_over(NbestShared& sh, int* is_last, long long b, int parts, int N,
                                                 long long rowLen, float* candVal, unsigned* candIdx,
                                                 unsigned* counters, float* __restrict__ outScores,
                                                 unsigned* __restrict__ outKeys) {
-#ifdef MARIAN_HIP_NBEST_FENCED
-  constexpr int kCounterOrder = __ATOMIC_ACQ_REL;
-#else
-  constexpr int kCounterOrder = __ATOMIC_RELAXED;
-#endif
+  constexpr int kCounterOrder = FENCED ? __ATOMIC_ACQ_REL : __ATOMIC_RELAXED;
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // every wave's stores have reached memory ...
   __syncthreads();
   if(threadIdx.x == 0)                               // ... before the count goes up
@@ -1487,7 +1485,7 @@ __device__ __forceinline__ void nbest_hand_over(NbestShared& sh, int* is_last, l
 // (-inf, none), which sorts last.  The workgroup that finishes last for a batch entry (a counter per
 // entry, zero between calls) draws the N best of all the entry's candidates.  No workgroup waits
 // for another.
-template <int KEEP>
+template <int KEEP, bool FENCED = false>
 __global__ __launch_bounds__(1024) void nbest_part_kernel(const float* __restrict__ scores, long long dimBatch,
                                                           long long vocab, int perSeg, long long sliceLen,
                                                           int N, float* candVal, unsigned* candIdx,
@@ -1532,7 +1530,7 @@ __global__ __launch_bounds__(1024) void nbest_part_kernel(const float* __restric
     nbest_of_row<KEEP>(scores + ((size_t)k * dimBatch + b) * vocab + v0, len, N, sh,
                        [&](int r, float v, unsigned i) { publish(r, v, base + i); });
   }
-  nbest_hand_over(sh, &is_last, b, parts, N, (long long)(parts / perSeg) * vocab, candVal, candIdx, counters,
+  nbest_hand_over<FENCED>(sh, &is_last, b, parts, N, (long long)(parts / perSeg) * vocab, candVal, candIdx, counters,
                   outScores, outKeys);
 }
 
@@ -1542,7 +1540,7 @@ __global__ __launch_bounds__(1024) void nbest_part_kernel(const float* __restric
 // (optionally adds the row's path score and optionally writes them out), selects the N best of the
 // row from the registers and leaves them as part k of entry b; the workgroup that finishes an
 // entry last draws the N best of its beam * N candidates.
-template <int VPT, int KEEP>
+template <int VPT, int KEEP, bool FENCED = false>
 __global__ __launch_bounds__(1024) void logsoftmax_nbest_kernel(const float* __restrict__ in,
                                                                 const float* __restrict__ rowAdd,
                                                                 float* __restrict__ lpOut, long long dimBatch,
@@ -1594,7 +1592,7 @@ __global__ __launch_bounds__(1024) void logsoftmax_nbest_kernel(const float* __r
     __hip_atomic_store(cv + r, val, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __hip_atomic_store(ci + r, base + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }, tv, true);
-  nbest_hand_over(sh, &is_last, b, parts, N, (long long)parts * vocab, candVal, candIdx, counters, outScores, outKeys);
+  nbest_hand_over<FENCED>(sh, &is_last, b, parts, N, (long long)parts * vocab, candVal, candIdx, counters, outScores, outKeys);
 }
 
 // Fill: the 16-byte aligned middle of the range with 16-byte stores of the repeated pattern, the
@@ -1722,9 +1720,22 @@ inline bool aligned4(const void* p) { return (reinterpret_cast<uintptr_t>(p) % 4
     if(e_ != hipSuccess) return record_hip_error((int)e_); \
   } while(0)
 
+// Which form of the n-best hand-over the launchers take: the shipped library has the unfenced one
+// only; the tuning build holds both behind a process-wide switch.
+#ifdef MARIAN_HIP_TUNING
+std::atomic<int> g_nbest_fenced{0};
+inline bool nbest_fenced() { return g_nbest_fenced.load(std::memory_order_relaxed) != 0; }
+#else
+constexpr bool nbest_fenced() { return false; }
+#endif
+
 }  // namespace
 
 extern "C" {
+
+#ifdef MARIAN_HIP_TUNING
+int marian_hip_nbest_set_fenced(int on) { return g_nbest_fenced.exchange(on ? 1 : 0); }
+#endif
 
 int marian_hip_layer_norm(const float* in, const float* add, const float* gamma, int64_t gamma_cols,
                           const float* beta, int64_t beta_cols, float* out, int64_t rows,
@@ -2213,12 +2224,22 @@ int marian_hip_nbest_beams(const float* scores, int64_t beam, int64_t dimBatch, 
   unsigned* candIdx = reinterpret_cast<unsigned*>(candVal + entries);
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   const dim3 grid((unsigned)plan.parts, (unsigned)dimBatch);
-  if(N <= 4)
-    hipLaunchKernelGGL(nbest_part_kernel<4>, grid, dim3(1024), 0, st, scores, (long long)dimBatch, (long long)vocab, plan.perSeg, plan.sliceLen, (int)N, candVal, candIdx, counters, outScores, outKeys);
-  else if(N <= 8)
-    hipLaunchKernelGGL(nbest_part_kernel<8>, grid, dim3(1024), 0, st, scores, (long long)dimBatch, (long long)vocab, plan.perSeg, plan.sliceLen, (int)N, candVal, candIdx, counters, outScores, outKeys);
-  else
-    hipLaunchKernelGGL(nbest_part_kernel<16>, grid, dim3(1024), 0, st, scores, (long long)dimBatch, (long long)vocab, plan.perSeg, plan.sliceLen, (int)N, candVal, candIdx, counters, outScores, outKeys);
+#define MH_NBP(KEEP, FENCED)                                                                                   \
+  hipLaunchKernelGGL((nbest_part_kernel<KEEP, FENCED>), grid, dim3(1024), 0, st, scores, (long long)dimBatch, \
+                     (long long)vocab, plan.perSeg, plan.sliceLen, (int)N, candVal, candIdx, counters,         \
+                     outScores, outKeys)
+  if(nbest_fenced()) {
+#ifdef MARIAN_HIP_TUNING
+    if(N <= 4) MH_NBP(4, true);
+    else if(N <= 8) MH_NBP(8, true);
+    else MH_NBP(16, true);
+#endif
+  } else {
+    if(N <= 4) MH_NBP(4, false);
+    else if(N <= 8) MH_NBP(8, false);
+    else MH_NBP(16, false);
+  }
+#undef MH_NBP
   MH_HIP(hipGetLastError());
   return MARIAN_HIP_OK;
 }
@@ -2244,12 +2265,20 @@ int marian_hip_logsoftmax_nbest_beams(const float* logits, const float* rowAdd, 
   unsigned* candIdx = reinterpret_cast<unsigned*>(candVal + entries);
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   const dim3 grid((unsigned)beam, (unsigned)dimBatch);
-#define MH_LSNB(VPT, KEEP)                                                                                   \
-  hipLaunchKernelGGL((logsoftmax_nbest_kernel<VPT, KEEP>), grid, dim3(1024), 0, st, logits, rowAdd, logProbs, \
+#define MH_LSNB(VPT, KEEP, FENCED)                                                                                   \
+  hipLaunchKernelGGL((logsoftmax_nbest_kernel<VPT, KEEP, FENCED>), grid, dim3(1024), 0, st, logits, rowAdd, logProbs, \
                      (long long)dimBatch, (int)vocab, (int)N, candVal, candIdx, counters, outScores, outKeys)
-  if(N <= 4) MH_LSNB(8, 4);
-  else if(N <= 8) MH_LSNB(8, 8);
-  else MH_LSNB(8, 16);
+  if(nbest_fenced()) {
+#ifdef MARIAN_HIP_TUNING
+    if(N <= 4) MH_LSNB(8, 4, true);
+    else if(N <= 8) MH_LSNB(8, 8, true);
+    else MH_LSNB(8, 16, true);
+#endif
+  } else {
+    if(N <= 4) MH_LSNB(8, 4, false);
+    else if(N <= 8) MH_LSNB(8, 8, false);
+    else MH_LSNB(8, 16, false);
+  }
 #undef MH_LSNB
   MH_HIP(hipGetLastError());
   return MARIAN_HIP_OK;

@@ -241,15 +241,12 @@ __device__ __forceinline__ void gemm_mfma32_tile(const GemmArgs& args, const int
 #pragma unroll
   for(int j = 0; j < Cfg::kLoads; ++j) {
     if(j < Cfg::kLoadsA) {
-      const int row = (j * Cfg::kWaves + wave) * 8 + lane / 8;
-      const int chunk = (lane % 8) ^ ((row >> 1) & 7);
-      goff[j] = min(m0 + row, M - 1) * K + chunk * 16;
+      goff[j] = stage_a_offset(j, Cfg::kWaves, wave, lane, m0, M, K);
     } else {
       const int g = (j - Cfg::kLoadsA) * Cfg::kWaves + wave;
-      const int sub = g / kTilesN, tile = g % kTilesN;
-      const int n = min(n0 + tile * 32 + (lane & 31), args.n_out - 1);
+      const int n = stage_b_column(g, kTilesN, lane, n0, args.n_out);
       const int src = args.idx ? (int)args.idx[n] : n;
-      goff[j] = (int)b_chunk_offset(src, 2 * sub + (lane >> 5), args.N);   // (K * N < 2^31)
+      goff[j] = (int)stage_b_offset(g, kTilesN, lane, src, args.N);   // (K * N < 2^31)
     }
   }
   const size_t b_block = (size_t)Cfg::BK * (size_t)args.N;   // bytes of all columns per K block
@@ -258,7 +255,7 @@ __device__ __forceinline__ void gemm_mfma32_tile(const GemmArgs& args, const int
   // stage is never multiplied.  The chunk of a lane is the same for all its loads (the number of
   // waves is even, so (row >> 1) & 7 does not depend on j).
   static_assert(Cfg::kWaves % 2 == 0, "the chunk of a lane must not depend on the load index");
-  const int tail_adj = (((lane % 8) ^ ((((wave * 8 + lane / 8) >> 1)) & 7)) >= 4) ? 64 : 0;
+  const int tail_adj = stage_a_tail_adjust(wave, lane);
   auto issue_one = [&](int kb, int stage, int j, auto check_tail) __attribute__((always_inline)) {
     const bool is_a = j < Cfg::kLoadsA;
     const int8_t* base = is_a ? args.Aq + (size_t)kb * Cfg::BK : args.Bq + (size_t)kb * b_block;
@@ -267,7 +264,7 @@ __device__ __forceinline__ void gemm_mfma32_tile(const GemmArgs& args, const int
     // bytes of an activation row or 64 * N bytes of the weights; what they stage is never multiplied)
     if(decltype(check_tail)::value && half_tail && kb == KB - 1) {
       if(is_a) voff -= tail_adj;
-      else if(((j - Cfg::kLoadsA) * Cfg::kWaves + wave) / kTilesN >= 2) voff -= 64 * args.N;
+      else if(stage_b_goes_back((j - Cfg::kLoadsA) * Cfg::kWaves + wave, kTilesN)) voff -= 64 * args.N;
     }
     global_load_lds16(base, (unsigned)voff,
                       lds_base + stage * Cfg::kStageBytes + (j * Cfg::kWaves + wave) * 1024);

@@ -94,13 +94,12 @@ __device__ __forceinline__ void gemm_pair_tiles(const GemmArgs& args, const int 
 #pragma unroll
   for(int j = 0; j < Cfg::kLoads; ++j) {
     if(j < Cfg::kLoadsA) {
-      const int row = (j * Cfg::kWaves + wave) * 8 + lane / 8;
-      const int chunk = (lane % 8) ^ ((row >> 1) & 7);
-      goff[j] = (unsigned)(m0 + row) * (unsigned)K + chunk * 16;
+      // (whole tiles only: no row or column of a tile lies past the matrix)
+      const int row = stage_a_row(j, Cfg::kWaves, wave, lane);
+      goff[j] = (unsigned)(m0 + row) * (unsigned)K + stage_a_chunk(row, lane) * 16;
     } else {
       const int g = (j - Cfg::kLoadsA) * Cfg::kWaves + wave;
-      const int sub = g / kTilesN, tile = g % kTilesN;
-      goff[j] = (unsigned)b_chunk_offset(n0 + tile * 32 + (lane & 31), 2 * sub + (lane >> 5), args.N);
+      goff[j] = (unsigned)stage_b_offset(g, kTilesN, lane, n0 + (g % kTilesN) * 32 + (lane & 31), args.N);
     }
   }
   const int8_t* const b_tile1 = args.Bq + b_column_offset(BN);   // weight columns of the second tile

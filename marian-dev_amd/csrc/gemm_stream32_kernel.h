@@ -143,7 +143,7 @@ __global__ __launch_bounds__(WN * KW * kWave) void gemm_stream32_kernel(GemmArgs
   // ---- weight row of this lane and where the bias of the four columns this lane will write
   //      sits (see the epilogue), both through the shortlist ids when there are any ----
   const int n0 = (bx * WN + wn) * 32;
-  int wsrc = min(n0 + li, args.n_out - 1);
+  int wsrc = stream32_lane_column(n0, li, args.n_out);
   const int bias_n = min(n0 + 4 * (lane % 8), args.n_out - 4);   // n_out % 8 == 0: four valid columns
   uint32_t bias_at[4];
 #pragma unroll
@@ -171,7 +171,7 @@ __global__ __launch_bounds__(WN * KW * kWave) void gemm_stream32_kernel(GemmArgs
     for(int i = 0; i < kAbsmaxSlots / kStream32Threads; ++i) amax = fmaxf(amax, pm[i]);
   }
   // this lane's 16 bytes of K sub-step 0; a sub-step further is w_step bytes further for every column
-  const int8_t* wrow = args.Bq + b_column_offset(wsrc) + lg * 16;
+  const int8_t* wrow = args.Bq + stream32_lane_offset(wsrc, lg);
   const size_t w_step = 32u * (size_t)args.N;
   __builtin_amdgcn_sched_barrier(0);
 
@@ -307,7 +307,7 @@ __global__ __launch_bounds__(WN * KW * kWave) void gemm_stream32_kernel(GemmArgs
   // per sub-step), one pointer and uniform offsets when the wave's sub-steps all lie within K,
   // clamped one by one otherwise
   auto load_weights = [&](int chunk, v4i (&dst)[Cfg::PW]) __attribute__((always_inline)) {
-    if(chunk * Cfg::CS + (kw_s + 1) * Cfg::PW <= S) {
+    if(stream32_chunk_is_whole(chunk, Cfg::CS, kw_s, Cfg::PW, S)) {
       const int8_t* wp = wrow + (size_t)(chunk * Cfg::CS + step0) * w_step;
 #pragma unroll
       for(int p = 0; p < Cfg::PW; ++p) dst[p] = load16(wp + (size_t)p * w_step);
@@ -315,7 +315,7 @@ __global__ __launch_bounds__(WN * KW * kWave) void gemm_stream32_kernel(GemmArgs
 #pragma unroll
       for(int p = 0; p < Cfg::PW; ++p) {
         const int s = chunk * Cfg::CS + step0 + p;
-        dst[p] = load16(wrow + (size_t)min(s, S - 1) * w_step);
+        dst[p] = load16(wrow + (size_t)stream32_clamped_substep(s, S) * w_step);
       }
     }
   };

@@ -54,7 +54,7 @@ __global__ __launch_bounds__(WN * KW * kWave) void gemm_stream_kernel(GemmArgs a
     int src = 0;
     if(n < args.n_out) src = args.idx ? (int)args.idx[n] : n;
     // 16-byte chunk lg of K step 0: sub-step lg / 2, half lg % 2
-    wrow[nt] = args.Bq + b_chunk_offset(src, lg, args.N);
+    wrow[nt] = args.Bq + stream16_lane_offset(src, lg, args.N);
   }
 
   // activation staging: 16-byte slot t of a stage is (step, m-tile, lane) in operand order

@@ -4,6 +4,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "operand_addressing.h"
+
 namespace marian_hip {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
@@ -24,20 +26,7 @@ __device__ __forceinline__ v4i load16(const int8_t* p) {
   return *reinterpret_cast<const v4i*>(p);
 }
 
-// Prepared weights ("K-blocked"): the K*N int8 values of W^T are stored by K sub-step of 32 values;
-// within a sub-step the N columns follow each other, 32 bytes (the sub-step's 32 K values) each:
-//   byte of (column n, k) = (k / 32) * 32 * N + n * 32 + k % 32
-// The operand of one matrix instruction for 32 (or 16) consecutive columns is then 1 KB (512 bytes)
-// of consecutive memory, which a wave fetches with one fully coalesced load; advancing along K adds
-// 32 * N bytes for every column alike.  (With the plain [N x K] rows every lane of such a load reads
-// a different 128-byte line: the address unit then takes four times as long per load, measured as
-// 2 k of 16 k clocks of the dominant decode call.  A gathered column - shortlist - still finds the
-// two 16-byte halves of a sub-step side by side.)
-__host__ __device__ __forceinline__ unsigned b_column_offset(int n) { return (unsigned)n * 32u; }
-// 16-byte chunk k16 (K values 16 * k16 .. + 15) of column n
-__host__ __device__ __forceinline__ size_t b_chunk_offset(int n, int k16, int N) {
-  return (size_t)(k16 >> 1) * 32u * (size_t)N + b_column_offset(n) + (unsigned)(k16 & 1) * 16u;
-}
+// (the prepared weight order and every operand offset of the kernels: operand_addressing.h)
 
 // quantMult stored behind `elements` int8 values (reference
 // src/tensors/cpu/integer_common.h:101-106).

@@ -483,6 +483,38 @@ def test_logsoftmax_nbest_of_beams_is_the_separate_calls(ops, chk, synth, batch,
         assert np.allclose(got_v, np.take_along_axis(flat, order, 1), rtol=2e-5, atol=4e-6)
 
 
+@pytest.mark.parametrize("batch,beam,V,N", [(32, 4, 32000, 4), (32, 4, 32000, 8), (64, 6, 8196, 6), (300, 2, 4100, 2)])
+def test_nbest_hand_over_with_and_without_fences(ops, synth, batch, beam, V, N):
+    """The hand-over of candidates between workgroups relies on device-scope stores and a wait for
+    their acknowledgement instead of the fences the language's memory model asks for.  The tuning
+    build holds both forms: same values and keys from both, for both entry points that use the
+    hand-over, at the size of a beam-search step and with many sentences, twenty calls each (a stale
+    candidate would show as a different n-best)."""
+    import torch
+    L = load("_lib")
+    x = dev(synth.normal(313 + V + N, 0, (beam, 1, batch, V), 3.0))
+    path = dev(synth.normal(314 + V, 1, (beam, batch), 1.0))
+    with L.forced_kernel(0) as T:
+        results = {}
+        for fenced in (0, 1):
+            prev = T.marian_hip_nbest_set_fenced(fenced)
+            try:
+                runs = []
+                for _ in range(20):
+                    v, k = ops.getNBestListOfBeams(x, N)
+                    v2, k2 = ops.logsoftmaxNBestOfBeams(x, N, pathScores=path)
+                    runs.append((v, k, v2, k2))
+                torch.cuda.synchronize()
+                results[fenced] = [[t.cpu().numpy() for t in r] for r in runs]
+            finally:
+                assert T.marian_hip_nbest_set_fenced(prev) == fenced
+    first = results[0][0]
+    for fenced in (0, 1):
+        for r in results[fenced]:
+            for got, want in zip(r, first):
+                assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
 def test_logsoftmax_nbest_of_beams_argument_checks(ops):
     import torch
     from conftest import load
