@@ -549,10 +549,11 @@ def pmc_summary(fetch_csv, write_csv):
         for key, pat in (("copy64", "vectorized_elementwise_kernel<4, at::native::CUDAFunctorOnSelf_add<float>"),
                          ("stream32_fused_M64_K512_N32000", "gemm_stream32_kernel<2, 4, 2, 8, 1, 4, 64"),
                          ("gemm_pair", "gemm_pair_kernel"), ("gemm_mfma32", "gemm_mfma32_kernel"),
+                         ("gemm_mfma32_split", "gemm_mfma32_split_kernel"),
                          ("absmax", "absmax_partial_kernel"), ("quantize_a", "quantize_a_kernel"),
                          ("prepare_a_onepass", "prepare_a_onepass_kernel")):
             if pat in name:
-                if key in ("gemm_mfma32", "prepare_a_onepass"):   # keep the template arguments apart
+                if key in ("gemm_mfma32", "gemm_mfma32_split", "prepare_a_onepass"):   # keep the template arguments apart
                     return key + "|" + name.split(pat)[1].split("(")[0]
                 return key
         return None

@@ -125,6 +125,33 @@ inline bool big_leaves_absmax(const GemmArgs& a, long long workgroups) {
   return a.absmax_out && !a.dump && workgroups <= kAbsmaxSlots;
 }
 
+// The split form (loading waves beside the multiplying ones): whole K blocks only; any M and N.
+template <int BM, int BN, int WM, int WN, int NSTAGE, bool NT>
+int launch_big_split(const GemmArgs& a, hipStream_t st) {
+  using Cfg = BigCfg<BM, BN, WM, WN, NSTAGE>;
+  if(a.K % Cfg::BK != 0) return MARIAN_HIP_ERR_SHAPE;
+  const int tiles_n = (a.n_out + BN - 1) / BN;
+  const int tiles_m = (a.M + BM - 1) / BM;
+  static std::atomic<uint64_t> lds_done[2];
+  GemmArgs a2 = a;
+  if(big_leaves_absmax(a, (long long)tiles_n * tiles_m)) {
+    auto kernel = gemm_mfma32_split_kernel<BM, BN, WM, WN, NSTAGE, NT, true>;
+    const int lds_status = allow_lds(kernel, Cfg::kLdsBytes, lds_done[1]);
+    if(lds_status != MARIAN_HIP_OK) return lds_status;
+    a2.absmax_used = tiles_n * tiles_m;
+    hipLaunchKernelGGL(kernel, dim3(tiles_n * tiles_m), dim3(2 * Cfg::kThreads), Cfg::kLdsBytes, st, a2, tiles_n, tiles_m);
+    MH_HIP(hipGetLastError());
+    t_absmax_written = true;
+    return MARIAN_HIP_OK;
+  }
+  auto kernel = gemm_mfma32_split_kernel<BM, BN, WM, WN, NSTAGE, NT, false>;
+  const int lds_status = allow_lds(kernel, Cfg::kLdsBytes, lds_done[0]);
+  if(lds_status != MARIAN_HIP_OK) return lds_status;
+  hipLaunchKernelGGL(kernel, dim3(tiles_n * tiles_m), dim3(2 * Cfg::kThreads), Cfg::kLdsBytes, st, a2, tiles_n, tiles_m);
+  MH_HIP(hipGetLastError());
+  return MARIAN_HIP_OK;
+}
+
 template <int BM, int BN, int WM, int WN, int NSTAGE, bool PAIRED = true, bool NT = false>
 int launch_big(const GemmArgs& a, hipStream_t st) {
   using Cfg = BigCfg<BM, BN, WM, WN, NSTAGE>;
@@ -567,6 +594,14 @@ int launch_gemm(const GemmArgs& a, hipStream_t st) {
     case 366: return launch_big_auto<256, 256, 2, 4, 2, true>(a, st, 1);
     case 363: return launch_big_auto<128, 128, 2, 4, 2, false>(a, st, 2);
     case 367: return launch_big_auto<128, 128, 2, 4, 2, true>(a, st, 2);
+    // 371 .. 377: the split form (whole K blocks; other calls fall through)
+    case 371: if(a.K % 128 == 0) return launch_big_split<128, 128, 2, 2, 3, false>(a, st); break;
+    case 372: if(a.K % 128 == 0) return launch_big_split<128, 128, 2, 2, 3, true>(a, st); break;
+    case 373: if(a.K % 128 == 0) return launch_big_split<128, 128, 2, 2, 4, true>(a, st); break;
+    case 375: if(a.K % 128 == 0) return launch_big_split<128, 64, 2, 2, 3, true>(a, st); break;
+    case 376: if(a.K % 128 == 0) return launch_big_split<128, 64, 2, 2, 4, true>(a, st); break;
+    case 377: if(a.K % 128 == 0) return launch_big_split<128, 64, 2, 2, 4, false>(a, st); break;
+    case 374: if(a.K % 128 == 0) return launch_big_split<128, 128, 2, 2, 4, false>(a, st); break;
     case 364: return launch_big_auto<128, 128, 2, 2, 3, false>(a, st, 1);
     case 368: return launch_big_auto<128, 128, 2, 2, 3, true>(a, st, 1);
     case 501: return launch_stream32_auto<kPrequant>(a, FusedSrc(), st, 0);
@@ -620,7 +655,12 @@ int launch_gemm(const GemmArgs& a, hipStream_t st) {
   }
   // so few 128x128 tiles that half the CUs would idle: 128x64 tiles (measured -20 % to -25 % for
   // M = 512 .. 1024, K = 4096, N = 1024; measurement id 340 keeps the square tiles)
+  // Tiles of which a CU gets one: whole K blocks go to the split form - four more waves per workgroup
+  // issue the loads, the multiplying waves spend no issue slots on them (measured -2 % to -9 %;
+  // measurement id 369 keeps the four-wave form)
+  const bool split = a.K % 128 == 0 && kernel_override() % 1000 != 369;
   if(2 * tiles128 <= compute_units() && kernel_override() % 1000 != 340) {
+    if(split) return stream_out ? launch_big_split<128, 64, 2, 2, 4, true>(a, st) : launch_big_split<128, 64, 2, 2, 4, false>(a, st);
     if(stream_out) return launch_big<128, 64, 2, 2, 3, true, true>(a, st);
     return launch_big<128, 64, 2, 2, 3>(a, st);
   }
@@ -638,6 +678,7 @@ int launch_gemm(const GemmArgs& a, hipStream_t st) {
                   : launch_big_ragged_as<128, 128, 2, 4, 2, false, false>(a, r, st);
     }
   }
+  if(split) return stream_out ? launch_big_split<128, 128, 2, 2, 3, true>(a, st) : launch_big_split<128, 128, 2, 2, 3, false>(a, st);
   if(stream_out) return launch_big<128, 128, 2, 2, 3, true, true>(a, st);
   return launch_big<128, 128, 2, 2, 3>(a, st);
 }

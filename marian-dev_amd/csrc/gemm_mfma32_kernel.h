@@ -49,7 +49,7 @@ struct BigCfg {
   static constexpr bool kHalfTailOk = !(BM == 256 && BN == 256 && kWaves == 8);
   static_assert((BM / 8) % kWaves == 0 && (BN / 8) % kWaves == 0, "tile rows vs waves");
   static_assert(BM % (WAVES_M * 32) == 0 && BN % (WAVES_N * 32) == 0, "tile vs wave grid");
-  static_assert(NSTAGE == 2 || NSTAGE == 3, "two or three LDS stages");
+  static_assert(NSTAGE >= 2 && NSTAGE <= 4, "two to four LDS stages (four: the split form only)");
 };
 
 // s_waitcnt with only vmcnt (up to 63) or only lgkmcnt constrained (gfx9 encoding).
@@ -207,8 +207,15 @@ __device__ __forceinline__ void publish_tile_absmax(float omax, float* absmax_ou
 // One BM x BN output tile at rows m0 .., columns n0 .. (any multiples of 32; the tile may hang over
 // the edge of the output).  slot: the workgroup's number among the tiles of the launch (abs-max
 // slot, clock record).
+// SPLIT: the workgroup has twice the waves of the tile's wave grid.  The first WAVES_M * WAVES_N waves
+// multiply and never touch global memory before the write-out; the others ("loaders", one more wave
+// per SIMD) issue every global -> LDS load of the tile and wait for them.  Both kinds meet at the one
+// workgroup barrier per K block, which says "block kb + 1 has landed" and "stage kb is free" at once.
+// The multiplying waves then spend no issue slots on loads and their waits (measured with the
+// instruction mixes alone: 90 % instead of 63 % matrix-instruction issue for the 128 x 128 tile).
+// Whole blocks only (no HALF).
 template <int BM, int BN, int WAVES_M, int WAVES_N, int NSTAGE, bool PAIRED = true, bool NT = false,
-          bool HALF = false, bool AMAX = false>
+          bool HALF = false, bool AMAX = false, bool SPLIT = false>
 __device__ __forceinline__ void gemm_mfma32_tile(const GemmArgs& args, const int m0, const int n0, int8_t* lds,
                                                  const int slot) {
   using Cfg = BigCfg<BM, BN, WAVES_M, WAVES_N, NSTAGE>;
@@ -217,7 +224,10 @@ __device__ __forceinline__ void gemm_mfma32_tile(const GemmArgs& args, const int
   const long long t_start = MH_CLOCK();
   const long long w_start = MH_WALL();
   const int tid = threadIdx.x;
-  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+  static_assert(!SPLIT || (PAIRED && !HALF), "the split form exists for whole blocks of the paired-fragment form");
+  const int wave_of_group = __builtin_amdgcn_readfirstlane(tid / kWave);
+  const bool loader = SPLIT && wave_of_group >= Cfg::kWaves;
+  const int wave = loader ? wave_of_group - Cfg::kWaves : wave_of_group;   // its number among its kind
   const int lane = tid % kWave;
   const int wm = wave / WAVES_N, wn = wave % WAVES_N;
   const int li = lane % 32, lg = lane / 32;
@@ -318,7 +328,7 @@ __device__ __forceinline__ void gemm_mfma32_tile(const GemmArgs& args, const int
   // (The loads are inline assembly, so the order is pinned slot by slot.)
   auto second_half = [&](auto steady_c, bool may_issue, int kb) __attribute__((always_inline)) {
     // steady: block kb + NSTAGE exists, its loads are issued without a branch between the MFMAs
-    const bool do_issue = decltype(steady_c)::value || may_issue;
+    const bool do_issue = !SPLIT && (decltype(steady_c)::value || may_issue);
     constexpr int nM = Cfg::WTM * Cfg::WTN;
     constexpr int LPS = (Cfg::kLoads + 2 * nM - 1) / (2 * nM);
     constexpr int nR = 2 * (Cfg::WTM + Cfg::WTN);
@@ -364,15 +374,42 @@ __device__ __forceinline__ void gemm_mfma32_tile(const GemmArgs& args, const int
   };
   auto mfma_only = [&]() { __builtin_amdgcn_sched_group_barrier(0x008, Cfg::WTM * Cfg::WTN, 0); };
 
-  // ---- prologue: fill all stages, wait for block 0 only ----
+  // (SPLIT) what a loader wave does instead of everything up to the write-out: all loads of the tile,
+  // each K block waited for before the barrier that hands it to the multiplying waves.  `ahead`
+  // blocks issued after the one waited for may still be in flight (loads retire in issue order).
+  auto wait_for_block = [&](int ahead) {
+    if(ahead >= 3) wait_vmcnt<3 * Cfg::kLoads>();
+    else if(ahead == 2) wait_vmcnt<2 * Cfg::kLoads>();
+    else if(ahead == 1) wait_vmcnt<Cfg::kLoads>();
+    else wait_vmcnt<0>();
+  };
+  static_assert(!SPLIT || 3 * Cfg::kLoads <= 63, "vmcnt holds 63 at most");
+  long long t_prologue = 0;
+  if(SPLIT && loader) {
 #pragma unroll
-  for(int s = 0; s < NSTAGE; ++s)
-    if(s < KB) issue(s);
-  if(NSTAGE == 3 && KB >= 3) wait_vmcnt<2 * Cfg::kLoads>();
-  else if(KB >= 2) wait_vmcnt<Cfg::kLoads>();
-  else wait_vmcnt<0>();
+    for(int s = 0; s < NSTAGE; ++s)
+      if(s < KB) issue(s);
+    wait_for_block(min(NSTAGE, KB) - 1);
+    __builtin_amdgcn_s_barrier();
+    t_prologue = MH_CLOCK();
+    for(int kb = 0; kb + 1 < KB; ++kb) {
+      const int last_issued = min(kb + NSTAGE - 1, KB - 1);
+      wait_for_block(last_issued - (kb + 1));   // block kb + 1 has landed ...
+      __builtin_amdgcn_s_barrier();              // ... and nobody reads stage kb any more
+      if(kb + NSTAGE < KB) issue(kb + NSTAGE);
+    }
+  } else {
+  // ---- prologue: fill all stages, wait for block 0 only ----
+  if constexpr(!SPLIT) {
+#pragma unroll
+    for(int s = 0; s < NSTAGE; ++s)
+      if(s < KB) issue(s);
+    if(NSTAGE == 3 && KB >= 3) wait_vmcnt<2 * Cfg::kLoads>();
+    else if(KB >= 2) wait_vmcnt<Cfg::kLoads>();
+    else wait_vmcnt<0>();
+  }
   __builtin_amdgcn_s_barrier();
-  const long long t_prologue = MH_CLOCK();
+  t_prologue = MH_CLOCK();
   if constexpr(!PAIRED) {
     auto spread = [&]() {   // one LDS read after each MFMA
 #pragma unroll
@@ -400,7 +437,7 @@ __device__ __forceinline__ void gemm_mfma32_tile(const GemmArgs& args, const int
         else wait_vmcnt<0>();
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
-        if(kb + NSTAGE < KB && !(MH_DBG(args, 1))) issue(kb + NSTAGE);
+        if(!SPLIT && kb + NSTAGE < KB && !(MH_DBG(args, 1))) issue(kb + NSTAGE);
         read_frags((kb + 1) % NSTAGE, 0, 0);
       }
       multiply(1);
@@ -422,8 +459,10 @@ __device__ __forceinline__ void gemm_mfma32_tile(const GemmArgs& args, const int
       // is free.  Block kb+1 must have landed (this wave's share); later blocks may be in flight.
       __builtin_amdgcn_sched_barrier(0);  // keep the MFMAs above on this side of the wait
       wait_lgkmcnt0();
-      if(NSTAGE == 3 && (decltype(steady_c)::value || kb + 2 < KB)) wait_vmcnt<Cfg::kLoads>();
-      else wait_vmcnt<0>();
+      if constexpr(!SPLIT) {
+        if(NSTAGE == 3 && (decltype(steady_c)::value || kb + 2 < KB)) wait_vmcnt<Cfg::kLoads>();
+        else wait_vmcnt<0>();
+      }
       __builtin_amdgcn_s_barrier();
       __builtin_amdgcn_sched_barrier(0);
       second_half(steady_c, kb + NSTAGE < KB && !(MH_DBG(args, 1)), kb);
@@ -450,6 +489,7 @@ __device__ __forceinline__ void gemm_mfma32_tile(const GemmArgs& args, const int
       mfma_only();
     }
   }
+  }   // (not a loader wave)
 
   const long long t_main = MH_CLOCK();
   // ---- epilogue: element v of a 32x32 tile is row 8*(v/4) + 4*lg + v%4, column li ----
@@ -462,7 +502,8 @@ __device__ __forceinline__ void gemm_mfma32_tile(const GemmArgs& args, const int
   const bool interior = (m0 + BM <= M) && (n0 + BN <= args.n_out);
   const size_t row_bytes = (size_t)args.n_out * 4;
   const bool has_bias = args.bias != nullptr;
-  if(!(MH_DBG(args, 2))) {
+  float omax = 0.0f;
+  if(!(MH_DBG(args, 2)) && !loader) {
     const int nw = n0 + wn * Cfg::WTN * 32 + li;   // this lane's column in the first of the wave's tiles
     float bias_v[Cfg::WTN];
     bool nvalid[Cfg::WTN];
@@ -480,7 +521,6 @@ __device__ __forceinline__ void gemm_mfma32_tile(const GemmArgs& args, const int
 #pragma unroll
     for(int b = 0; b < Cfg::WTN; ++b) asm volatile("" ::"v"(bias_v[b]));
     asm volatile("" ::"v"(unquant));
-    float omax = 0.0f;
 #pragma unroll
     for(int a = 0; a < Cfg::WTM; ++a) {
       const int mbase = m0 + (wm * Cfg::WTM + a) * 32 + 4 * lg;
@@ -490,9 +530,9 @@ __device__ __forceinline__ void gemm_mfma32_tile(const GemmArgs& args, const int
       else
         store_tiles32_rowwise_any<Cfg::WTN, true, NT, AMAX>(acc[a], outp, row_bytes, unquant, bias_v, M - mbase, nvalid, args.dump, has_bias, args.relu, omax);
     }
-    if(AMAX && args.absmax_out && !args.dump)
-      publish_tile_absmax(omax, args.absmax_out, slot, args.absmax_used, reinterpret_cast<float*>(lds));
   }
+  if(!(MH_DBG(args, 2)) && AMAX && args.absmax_out && !args.dump)   // (all waves: it has barriers)
+    publish_tile_absmax(omax, args.absmax_out, slot, args.absmax_used, reinterpret_cast<float*>(lds));
   if(MH_PROF(args) && tid == 0) {
     long long* p = MH_PROF(args) + (size_t)slot * 8;
     p[0] = t_start; p[1] = t_prologue; p[2] = t_main; p[3] = MH_CLOCK(); p[6] = w_start; p[7] = MH_WALL();
@@ -507,6 +547,15 @@ __global__ __launch_bounds__(WAVES_M * WAVES_N * kWave) void gemm_mfma32_kernel(
   int tn, tm;
   xcd_tile(tiles_n, tiles_m, blockIdx.x, tn, tm);
   gemm_mfma32_tile<BM, BN, WAVES_M, WAVES_N, NSTAGE, PAIRED, NT, HALF, AMAX>(args, tm * BM, tn * BN, lds, blockIdx.x);
+}
+
+template <int BM, int BN, int WAVES_M, int WAVES_N, int NSTAGE, bool NT = false, bool AMAX = false>
+__global__ __launch_bounds__(2 * WAVES_M * WAVES_N * kWave) void gemm_mfma32_split_kernel(
+    GemmArgs args, int tiles_n, int tiles_m) {
+  extern __shared__ __attribute__((aligned(16))) int8_t lds[];
+  int tn, tm;
+  xcd_tile(tiles_n, tiles_m, blockIdx.x, tn, tm);
+  gemm_mfma32_tile<BM, BN, WAVES_M, WAVES_N, NSTAGE, true, NT, false, AMAX, true>(args, tm * BM, tn * BN, lds, blockIdx.x);
 }
 
 // A launch whose output is not a whole number of main tiles: `main_tiles` whole BM x BN tiles

@@ -134,7 +134,8 @@ def test_fused_affine_degenerate_activations(integer, orc, synth, kind, kernel):
 # pre-quantized operands: small-M families, the large-M tiles, the tile-pair kernel
 MULT_CASES = [(0, 8, 256, 64), (101, 8, 256, 64), (102, 16, 512, 512), (501, 64, 512, 2048),
               (0, 300, 1024, 512), (301, 512, 1024, 512), (307, 300, 320, 264), (312, 512, 2048, 1024),
-              (313, 640, 1024, 1024), (330, 512, 1024, 512), (331, 256, 1280, 512), (0, 4096, 1024, 1024)]
+              (313, 640, 1024, 1024), (330, 512, 1024, 512), (331, 256, 1280, 512), (0, 4096, 1024, 1024),
+              (372, 512, 1024, 512), (376, 300, 1024, 264)]
 
 
 @pytest.mark.parametrize("kernel,M,K,N", MULT_CASES)

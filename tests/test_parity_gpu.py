@@ -179,7 +179,8 @@ def test_multiply_all_kernels_small_m(integer, orc, synth, M, K, N, kernel):
     run_case(integer, orc, synth, 300 + M + N, M, K, N, kernel, bias_on=True, relu=(M % 2 == 0))
 
 
-@pytest.mark.parametrize("kernel", [0, 501, 512, 521, 522, 524, 301, 302, 303, 304, 305, 306, 307, 308, 311, 312, 313, 330, 340])
+@pytest.mark.parametrize("kernel", [0, 501, 512, 521, 522, 524, 301, 302, 303, 304, 305, 306, 307, 308, 311, 312, 313, 330, 340,
+                                    369, 371, 372, 373, 374, 375, 376, 377])
 @pytest.mark.parametrize("M,K,N", [(129, 64, 8), (256, 1024, 504), (300, 320, 1000), (513, 128, 264)])
 def test_multiply_tile_kernels_ragged(integer, orc, synth, M, K, N, kernel):
     say("multiply ragged", M, K, N, "kernel", kernel)
@@ -196,7 +197,7 @@ def test_multiply_mid_size_dispatch(integer, orc, synth, M, K, N):
     run_case(integer, orc, synth, 470 + M + N, M, K, N, 0, bias_on=True, relu=(M % 128 == 0), scale=1.5)
 
 
-@pytest.mark.parametrize("kernel", [0, 301, 302, 303, 307, 308, 309, 311, 312, 313, 330])
+@pytest.mark.parametrize("kernel", [0, 301, 302, 303, 307, 308, 309, 311, 312, 313, 330, 369])
 @pytest.mark.parametrize("M,K,N", [(512, 192, 512), (1024, 1088, 1024), (640, 448, 264), (2048, 64, 2048),
                                    (1300, 2112, 776)])
 def test_multiply_half_last_k_block(integer, orc, synth, M, K, N, kernel):
@@ -204,6 +205,19 @@ def test_multiply_half_last_k_block(integer, orc, synth, M, K, N, kernel):
     64 columns (one, two and many blocks)."""
     say("multiply half last block", M, K, N, "kernel", kernel)
     run_case(integer, orc, synth, 480 + M + N, M, K, N, kernel, bias_on=True, relu=(K % 256 == 64), scale=0.75)
+
+
+@pytest.mark.parametrize("kernel", [0, 369, 371, 372, 373, 374, 375, 376, 377])
+@pytest.mark.parametrize("M,K,N,bias_on,relu", [(128, 128, 128, True, False), (256, 256, 64, False, True), (640, 384, 1024, True, True),
+                                                (1000, 512, 1032, True, False), (2048, 1024, 1024, False, False),
+                                                (130, 2048, 136, True, True), (4096, 128, 1024, True, False)])
+def test_multiply_split_form(integer, orc, synth, M, K, N, bias_on, relu, kernel):
+    """The large-M form whose loads are issued by four waves of their own beside the four that
+    multiply (three and four LDS stages, 128 x 128 and 128 x 64 tiles, plain and non-temporal
+    stores): one K block (nothing to pipeline), fewer blocks than stages, many; tiles that hang over
+    the edge of the output; 369 is the four-wave form the automatic choice took before."""
+    say("multiply split form", M, K, N, "kernel", kernel)
+    run_case(integer, orc, synth, 520 + M + N, M, K, N, kernel, bias_on=bias_on, relu=relu, scale=1.25)
 
 
 @pytest.mark.parametrize("kernel", [330, 331])
@@ -255,7 +269,7 @@ def test_fused_shortlist(integer, orc, synth):
     assert np.array_equal(Aq.numpy(), Aq_h) and np.array_equal(out.cpu().numpy(), want)
 
 
-@pytest.mark.parametrize("kernel", [0, 101, 102, 301, 307, 312, 501, 511, 512, 514, 518, 521, 522, 524, 600, 611, 612, 614, 618, 620, 621, 624, 628, 641, 651, 661, 670, 690])
+@pytest.mark.parametrize("kernel", [0, 101, 102, 301, 307, 312, 372, 376, 501, 511, 512, 514, 518, 521, 522, 524, 600, 611, 612, 614, 618, 620, 621, 624, 628, 641, 651, 661, 670, 690])
 @pytest.mark.parametrize("M", [8, 100])
 def test_shortlist_every_kernel_family(integer, orc, synth, M, kernel):
     """The row gather of W^T and of the bias inside each kernel family (ids >= 600: fused call)."""
