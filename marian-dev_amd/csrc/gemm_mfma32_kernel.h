@@ -569,6 +569,12 @@ struct RaggedPlan {
   int main_tiles_n, main_tiles_m;
   int bottom_tiles_n, bottom_tiles_m;   // EBM x EBN tiles below the main tiles (all columns)
   int right_tiles_n, right_tiles_m;     // RBM x RBN tiles to the right of the main tiles (main rows only)
+  // 0: the small tiles take the workgroup numbers behind the main tiles.  Otherwise (a multiple of
+  // eight, at least the number of small tiles): they take the first `lead` numbers - where a main
+  // workgroup fills a CU's LDS, the small tiles then run ahead of the main tiles of a few CUs instead
+  // of after the main tiles of all (numbers in between are idle; a multiple of eight keeps every main
+  // tile on the XCD its number modulo eight names)
+  int lead = 0;
 };
 
 template <int BM, int BN, int WAVES_M, int WAVES_N, int NSTAGE, int EBM, int EBN, int EWM, int EWN, int ESTAGE,

@@ -294,21 +294,34 @@ __global__ __launch_bounds__(PairCfg::kThreads) void gemm_pair_kernel(GemmArgs a
 template <bool NT, bool AMAX = false>
 __global__ __launch_bounds__(PairCfg::kThreads) void gemm_pair_ragged_kernel(GemmArgs args, RaggedPlan plan) {
   extern __shared__ __attribute__((aligned(16))) int8_t lds[];
-  const int block = blockIdx.x;
+  const int slot = blockIdx.x;
   const int n_main = plan.main_tiles_n * plan.main_tiles_m;
   const int n_bottom = plan.bottom_tiles_n * plan.bottom_tiles_m;
+  const int n_small = n_bottom + plan.right_tiles_n * plan.right_tiles_m;
+  // number among the main tiles (0 .. n_main - 1) or n_main + number among the small tiles
+  int block = slot;
+  if(plan.lead) {
+    if(slot >= plan.lead) {
+      block = slot - plan.lead;
+    } else if(slot < n_small) {
+      block = n_main + slot;
+    } else {   // an idle number between the small and the main tiles
+      if(AMAX && args.absmax_out && threadIdx.x == 0) args.absmax_out[slot] = 0.0f;
+      return;
+    }
+  }
   if(block < n_main) {
     int tn, tm;
     xcd_tile(plan.main_tiles_n, plan.main_tiles_m, block, tn, tm);
-    gemm_pair_tiles<NT, AMAX>(args, tm * PairCfg::BM, tn * 2 * PairCfg::BN, lds, block);
+    gemm_pair_tiles<NT, AMAX>(args, tm * PairCfg::BM, tn * 2 * PairCfg::BN, lds, slot);
   } else if(block < n_main + n_bottom) {
     const int t = block - n_main;
     const int tn = t % plan.bottom_tiles_n, tm = t / plan.bottom_tiles_n;
-    gemm_mfma32_tile<64, 128, 2, 2, 3, true, NT, false, AMAX>(args, plan.main_tiles_m * PairCfg::BM + tm * 64, tn * 128, lds, block);
+    gemm_mfma32_tile<64, 128, 2, 2, 3, true, NT, false, AMAX>(args, plan.main_tiles_m * PairCfg::BM + tm * 64, tn * 128, lds, slot);
   } else {
     const int t = block - n_main - n_bottom;
     const int tm = t % plan.right_tiles_m, tn = t / plan.right_tiles_m;
-    gemm_mfma32_tile<128, 64, 2, 2, 3, true, NT, false, AMAX>(args, tm * 128, plan.main_tiles_n * 2 * PairCfg::BN + tn * 64, lds, block);
+    gemm_mfma32_tile<128, 64, 2, 2, 3, true, NT, false, AMAX>(args, tm * 128, plan.main_tiles_n * 2 * PairCfg::BN + tn * 64, lds, slot);
   }
 }
 
