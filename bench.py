@@ -216,6 +216,22 @@ def cpu_worker(seconds):
     print(json.dumps({"passes": passes, "seconds": dt, "ops_per_pass": sum(w[4] for w in work)}))
 
 
+def eager_sweep_cpp_host():
+    """The same twenty calls per pass launched one after the other from a C++ host thread through the
+    C++ wrappers (marian-dev_amd/host/eager_sweep, built by build()): ms per pass, or None when the
+    program is not there.  It runs as a child process while this one is idle."""
+    import subprocess
+    exe = os.path.join(ROOT, PKG, "host", "eager_sweep")
+    if not os.path.exists(exe):
+        return None
+    try:
+        out = subprocess.run([exe, "300", "30"], capture_output=True, text=True, timeout=120)
+        return round(json.loads(out.stdout.strip().splitlines()[-1])["eager_ms_per_pass_cpp_host"], 4)
+    except Exception as e:   # noqa: BLE001 - a measurement that is reported as absent, not a failure of the run
+        print("eager_sweep failed: %r" % (e,), file=sys.stderr)
+        return None
+
+
 def cpu_baseline(seconds=10.0, aggregate_seconds=6.0, big_seconds=6.0):
     """The CPU restatement of the reference path (prepareA + VNNI multiply + unquantize/bias, one
     thread per GEMM like one Marian CPU worker, reference src/common/config.cpp:245-247) timed on
@@ -665,6 +681,7 @@ def main():
         step(i)
     torch.cuda.synchronize()
     eager_ms = (time.perf_counter() - t0) / 20 * 1e3
+    eager_cpp = eager_sweep_cpp_host()
 
     # ---------------- roofline of the dominant kernel ----------------------------------------
     # vocabulary projection of the sweep at M = 64 (16.4 MB of int8 weights, 8.2 MB of output):
@@ -717,6 +734,7 @@ def main():
         "step_hbm_frac": round(step_bytes / (dt / args.steps) / 1e9 / HBM_PEAK_GBS, 4),
         "value_cache_resident_tops": round(step_ops / (dt_res / args.steps) / 1e12, 4),
         "eager_ms_per_step": round(eager_ms, 4),
+        "eager_ms_per_step_cpp_host": eager_cpp,
         "roofline": roofline,
         "per_shape": per_shape,
     }
