@@ -216,20 +216,26 @@ def cpu_worker(seconds):
     print(json.dumps({"passes": passes, "seconds": dt, "ops_per_pass": sum(w[4] for w in work)}))
 
 
-def eager_sweep_cpp_host():
-    """The same twenty calls per pass launched one after the other from a C++ host thread through the
-    C++ wrappers (marian-dev_amd/host/eager_sweep, built by build()): ms per pass, or None when the
-    program is not there.  It runs as a child process while this one is idle."""
+def cpp_host_figure(program, key, args=("300", "30")):
+    """A figure measured by one of the C++ host programs of marian-dev_amd/host (built by build()),
+    which launch call after call from a C++ thread through the C++ wrappers, no recorded graph: the
+    value of `key` in the line of JSON the program prints, or None when the program is not there.
+    It runs as a child process while this one is idle."""
     import subprocess
-    exe = os.path.join(ROOT, PKG, "host", "eager_sweep")
+    exe = os.path.join(ROOT, PKG, "host", program)
     if not os.path.exists(exe):
         return None
     try:
-        out = subprocess.run([exe, "300", "30"], capture_output=True, text=True, timeout=120)
-        return round(json.loads(out.stdout.strip().splitlines()[-1])["eager_ms_per_pass_cpp_host"], 4)
+        out = subprocess.run([exe] + list(args), capture_output=True, text=True, timeout=180)
+        return round(json.loads(out.stdout.strip().splitlines()[-1])[key], 4)
     except Exception as e:   # noqa: BLE001 - a measurement that is reported as absent, not a failure of the run
-        print("eager_sweep failed: %r" % (e,), file=sys.stderr)
+        print("%s failed: %r" % (program, e), file=sys.stderr)
         return None
+
+
+def eager_sweep_cpp_host():
+    """The twenty calls of the decode sweep, ms per pass (host/eager_sweep.cpp)."""
+    return cpp_host_figure("eager_sweep", "eager_ms_per_pass_cpp_host")
 
 
 def cpu_baseline(seconds=10.0, aggregate_seconds=6.0, big_seconds=6.0):
@@ -930,6 +936,7 @@ def main():
             "ms_per_step_unchained": round(udt / n * 1e3, 4),
             "chained_equals_unchained": same,
             "eager_ms_per_step_python_host": round(eager_full_ms, 4),
+            "eager_ms_per_step_cpp_host": cpp_host_figure("eager_step", "eager_ms_per_step_cpp_host", ("200", "20")),
             "step_hbm_frac": round(step_bytes_big * n / fdt / 1e9 / HBM_PEAK_GBS, 4),
             "weight_hbm_frac": round(dec.weight_bytes * n / fdt / 1e9 / HBM_PEAK_GBS, 4),
             "step_algorithmic_bytes": {"int8_weights": dec.weight_bytes, "cached_keys_and_values_read": cache_bytes,

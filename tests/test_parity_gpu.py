@@ -904,3 +904,22 @@ def test_cpp_host_side(integer, orc, synth, tmp_path):
     r = subprocess.run([exe, fixture], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=120)
     print(r.stdout)
     assert r.returncode == 0 and "-> OK" in r.stdout and "FAILED" not in r.stdout, r.stdout
+
+
+@pytest.mark.parametrize("program,key", [("eager_sweep", "eager_ms_per_pass_cpp_host"), ("eager_step", "eager_ms_per_step_cpp_host")])
+def test_cpp_host_programs_that_launch_call_by_call(program, key):
+    """The two C++ programs bench.py takes its eager figures from (the decode sweep and the full
+    transformer-big decoding step through the C++ wrappers, no recorded graph) run and report; the
+    step's own check - finite log-probabilities, every n-best key inside its sentence - holds."""
+    import json
+    import subprocess
+    from conftest import ROOT
+    exe = os.path.join(ROOT, "marian-dev_amd", "host", program)
+    assert os.path.exists(exe), program + " not built"
+    say(program)
+    r = subprocess.run([exe, "3", "1"], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=150)
+    assert r.returncode == 0, r.stderr[-1000:]
+    line = json.loads(r.stdout.strip().splitlines()[-1])
+    assert line[key] > 0
+    if program == "eager_step":
+        assert line["nbest_sane"] is True and line["launches_per_step"] == 58
