@@ -944,6 +944,7 @@ def main():
         ancdt = time_graphs(torch, sel, n, max(4, args.warmup // 2))
         del sel
         dec.by_ancestors = False
+        eager_step_ms = cpp_host_figure("eager_step", "eager_ms_per_step_cpp_host", ("200", "20"))
         out["transformer_big_decode_full"] = {
             "what": "full decoder step through the host mirrors, from the previous step's word indices: embedding rows x "
                     "sqrt(d) + position signal (one launch), 49 int8 affine products + per layer "
@@ -970,7 +971,8 @@ def main():
             "ms_per_step_unchained": round(udt / n * 1e3, 4),
             "chained_equals_unchained": same,
             "eager_ms_per_step_python_host": round(eager_full_ms, 4),
-            "eager_ms_per_step_cpp_host": cpp_host_figure("eager_step", "eager_ms_per_step_cpp_host", ("200", "20")),
+            "eager_ms_per_step_cpp_host": eager_step_ms,
+            "eager_hyp_tokens_per_s_cpp_host": round(dec.M / (eager_step_ms * 1e-3), 1) if eager_step_ms else None,
             "step_hbm_frac": round(step_bytes_big * n / fdt / 1e9 / HBM_PEAK_GBS, 4),
             "weight_hbm_frac": round(dec.weight_bytes * n / fdt / 1e9 / HBM_PEAK_GBS, 4),
             "step_algorithmic_bytes": {"int8_weights": dec.weight_bytes, "cached_keys_and_values_read": cache_bytes,
