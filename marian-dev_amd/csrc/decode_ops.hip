@@ -826,14 +826,29 @@ __global__ __launch_bounds__(256) void attention_kernel(const float* __restrict_
 //      the caches at position len - 1, and all three into proj_out where a caller asks for them;
 //   5. wave w runs the attention of row w: the code of attention_kernel's 64-wide path, operation
 //      for operation, with q and the newest key/value row read from LDS.
+// Where the caches are complete and shared - the encoder's keys and values, which every hypothesis
+// of a sentence attends to (row m reads sentence m % sentences) - a workgroup takes hypotheses of
+// the same one or two sentences instead of eight consecutive rows, reads these sentences' keys and
+// values once (asked for as soon as the abs-max is known, stored to LDS in step 4) and its waves
+// take them from LDS: a quarter of the bytes through the CU's memory path with four hypotheses a
+// sentence (60 positions: 60 KB instead of 240 KB per workgroup).
 // Requirements (checked by the launcher): head size 64, K % 128 == 0, K <= 1024, len <= 512.
 // Measured (transformer-big step, 128 rows, 16 heads): 13.5 us against 8.2 + 8.4 us for q, k, v and
 // the self-attention over 21 positions, 13.9 against 5.3 + 8.4 us for Wq and the context attention over
-// 60 positions - the attention is bound by the bytes of keys and values it reads (22 MB per layer),
-// so the launch saved is most of the gain.  Tried and dropped: asking for a row's keys and values
-// at kernel start so that they reach L2 under the projections (loads into a scratch word of LDS):
-// +16 us per step - they queue ahead of the weights and the input, which everything waits for.
+// 60 positions with every wave reading its own keys and values; staging the shared ones takes the
+// whole step from 0.437 to 0.425 ms.  Clocks read inside the kernel (weights and caches of 24
+// layers in rotation, so that they come from HBM): the launch is bound by what a CU can fetch,
+// about 15 bytes per clock when most of it misses L2 - the self-attention form's 310 KB per
+// workgroup (192 KB of weights, 32 KB of input, 86 KB of keys and values) in 26 000 clocks, the
+// context form's 156 KB (staged) in 17 700.  Tried and dropped, each without a gain in the step:
+// asking for a row's keys and values at kernel start (loads into a scratch word of LDS, by the
+// multiplying waves or by two more waves), or into registers once the abs-max is known in the
+// self-attention form - the attention then waits less and the quantization more, for the same
+// bytes; barriers that put every wave's small requests in front of any wave's large ones.
 constexpr int kProjThreads = 512, kProjMaxK = 1024, kProjMaxLen = 512;
+// keys and values shared by the rows of a workgroup are staged in LDS up to this many positions
+constexpr int kProjStageLen = 96;
+constexpr int kProjMaxLds = 160 * 1024 - 256;   // dynamic LDS of a workgroup (a few bytes are static)
 
 struct ProjAttentionArgs {
   const float* A;           // [M, K] float32
@@ -853,6 +868,14 @@ struct ProjAttentionArgs {
   float att_scale;
   float* out;               // [M * heads, 64]
   float* absmax_out;        // slots or null
+  // Which input rows a workgroup takes.  share_shift < 0: eight consecutive ones.  Otherwise the
+  // caches hold `share_nb` sentences that several hypotheses each attend to (row m reads sentence
+  // m % share_nb), and a workgroup takes 8 >> share_shift hypotheses of 1 << share_shift
+  // neighbouring sentences, so that the waves that read the same keys and values sit on one CU.
+  int share_shift, share_nb;
+  // With it (and sentences two or one to a workgroup, len <= kProjStageLen): the keys and values of
+  // the workgroup's sentences are read once, into LDS, and every hypothesis' wave takes them from there.
+  int stage_kv;
 };
 
 // the row permutation of the staged activations (gemm_stream32_kernel.h: stream32_row_key)
@@ -862,8 +885,10 @@ __device__ __forceinline__ int proj_row_key(int c16) { return (c16 ^ (c16 >> 2))
 // cover a key or value row, four consecutive positions per load, up to 64 positions in flight), the
 // same operations in the same order, so the result has the same bits.  q, k_last, v_last may lie
 // in LDS.  sc: len4 floats of this wave, part: 256 floats behind them.  Returns |out| of this lane.
+// LAST_IN_ROWS: k_last and v_last are row len - 1 of kb and vb (one address computation for all rows).
+template <bool LAST_IN_ROWS = false>
 __device__ __forceinline__ float attention_row64(const float* q, const float* kb, const float* vb, const float* k_last,
-                                                 const float* v_last, const float* mk, int len, float scale, float* sc,
+                                                 const float* v_last, const float* mk, float mk0, int len, float scale, float* sc,
                                                  float* part, float* out_row, int lane) {
   constexpr int kAttU = 16, dk = 64;
   const int len4 = (len + 3) & ~3;
@@ -876,15 +901,14 @@ __device__ __forceinline__ float attention_row64(const float* q, const float* kb
     for(int u = 0; u < kAttU; ++u) {
       if(base + 4 * u < len) {
         const int U = base / 4 + u;
-        if(U >= u_last) r[u] = *reinterpret_cast<const v4f*>(last_c);
+        if constexpr(LAST_IN_ROWS) r[u] = *reinterpret_cast<const v4f*>(rows + (size_t)min(4 * U + g, len - 1) * dk + 4 * c);
+        else if(U >= u_last) r[u] = *reinterpret_cast<const v4f*>(last_c);
         else r[u] = *reinterpret_cast<const v4f*>(first + (size_t)U * 4 * dk);
       } else if(base + 4 * (u & ~3) < len) {
         r[u] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
       }
     }
   };
-  float mk0 = 0.0f;
-  if(mk) mk0 = mk[min(lane, len - 1)];
   const v4f q4 = reinterpret_cast<const v4f*>(q)[c];
   v4f kr[kAttU], vr[kAttU];
   load_rows(kb, k_last, 0, kr);
@@ -962,26 +986,51 @@ __device__ __forceinline__ float attention_row64(const float* q, const float* kb
 // NPROJ: 3 (q, k_new, v_new: self-attention, the new key/value row is appended to the caches) or
 // 1 (q only: attention over caches that are complete, e.g. the encoder's).  R: input rows per
 // workgroup, 8 (a wave per row in the attention).
-template <int NPROJ, int R>
+template <int NPROJ, int R, int SEGS, int PASSES>
 __global__ __launch_bounds__(kProjThreads) void proj_attention_kernel(ProjAttentionArgs p) {
   static_assert(R == 8, "one wave per row in the attention");
+  constexpr bool STAGED = SEGS > 0;
+  static_assert(!STAGED || NPROJ == 1, "keys and values are shared only where the caches are complete");
+  static_assert(SEGS == 0 || SEGS == 2 || SEGS == 4, "keys and values of one or two sentences");
+  static_assert(PASSES * 32 <= kProjStageLen, "32 positions per pass");
   typedef int v16i_p __attribute__((ext_vector_type(16)));
   extern __shared__ __attribute__((aligned(16))) int8_t plds[];
   __shared__ float red[kProjThreads / 64];
   const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
   const int wn = wave % 2, kw = wave / 2, li = lane % 32, lg = lane / 32;
-  const int h = blockIdx.x, m_base = blockIdx.y * R;
+  const int h = blockIdx.x;
+  // input row r of this workgroup (rows past the end: M or more)
+  const int sent_groups = p.share_shift < 0 ? 1 : p.share_nb >> p.share_shift;
+  const int hyp_base = p.share_shift < 0 ? 0 : ((int)blockIdx.y / sent_groups) * (R >> p.share_shift);
+  const int sent_base = p.share_shift < 0 ? 0 : ((int)blockIdx.y % sent_groups) << p.share_shift;
+  auto row_of = [&](int r) -> int {
+    if(p.share_shift < 0) return (int)blockIdx.y * R + r;
+    return (hyp_base + (r >> p.share_shift)) * p.share_nb + sent_base + (r & ((1 << p.share_shift) - 1));
+  };
   const int K = p.K, M = p.M, S = K / 32, PW = S / 4, N = p.heads * 64;
   int8_t* a_lds = plds;                                   // 32 rows x K bytes, operand order
   int8_t* part_lds = a_lds + 32 * K;                      // NPROJ x 2 x 4 partial tiles of R rows x 128 bytes
   float* proj_lds = reinterpret_cast<float*>(part_lds + NPROJ * 8 * R * 128);   // [NPROJ][R][64]
   float* att_lds = proj_lds + NPROJ * R * 64;             // per wave: scores + 256 partial outputs
+  const int len4s = (p.len + 3) & ~3;
+  float* kv_lds = att_lds + R * (len4s + 256);            // staged keys and values: [sentence][k, v][len][64]
 
   // ---- everything this workgroup will need is requested now: abs-max slots, weights, the input
   //      rows, the quantization multipliers of the weights, bias ----
   float pm[kAbsmaxSlots / kProjThreads];
 #pragma unroll
   for(int i = 0; i < kAbsmaxSlots / kProjThreads; ++i) pm[i] = p.partials[min(tid + i * kProjThreads, p.n_partials - 1)];
+  // a quad of lanes takes four consecutive 16-value groups of one row: 64 contiguous bytes per load
+  const int grp = (tid / 4) * 4, qlane = tid % 4;
+  const int r_in = grp / (2 * S), c16 = grp % (2 * S);
+  const bool has_in = r_in < R;
+  v4f in[4];
+  {
+    const int m = min(row_of(min(r_in, R - 1)), M - 1);
+    const float* src = p.A + (size_t)m * (size_t)K + (size_t)c16 * 16 + qlane * 4;
+#pragma unroll
+    for(int e = 0; e < 4; ++e) in[e] = *reinterpret_cast<const v4f*>(src + e * 16);
+  }
   v4i w[NPROJ][8];
   const int ncol = h * 64 + wn * 32 + li;
 #pragma unroll
@@ -990,17 +1039,18 @@ __global__ __launch_bounds__(kProjThreads) void proj_attention_kernel(ProjAttent
 #pragma unroll
     for(int pp = 0; pp < 8; ++pp) w[g][pp] = load16(wrow + (size_t)stream32_clamped_substep(kw * PW + pp, S) * 32u * (size_t)N);
   }
-  // a quad of lanes takes four consecutive 16-value groups of one row: 64 contiguous bytes per load
-  const int grp = (tid / 4) * 4, qlane = tid % 4;
-  const int r_in = grp / (2 * S), c16 = grp % (2 * S);
-  const bool has_in = r_in < R;
-  v4f in[4];
-  {
-    const int m = min(m_base + min(r_in, R - 1), M - 1);
-    const float* src = p.A + (size_t)m * (size_t)K + (size_t)c16 * 16 + qlane * 4;
-#pragma unroll
-    for(int e = 0; e < 4; ++e) in[e] = *reinterpret_cast<const v4f*>(src + e * 16);
+  // keys and values of the workgroup's sentences: sixteen threads per position, 32 positions per pass
+  constexpr int kStageSegs = STAGED ? SEGS : 1, kStagePasses = STAGED ? PASSES : 1;
+  v4f stage[kStageSegs][kStagePasses];
+  // the mask value of this wave's row for position `lane`
+  const int m_wave = row_of(min(wave, R - 1));
+  const float* mk = nullptr;
+  if(p.mask && m_wave < M) {
+    unsigned mask_row = (unsigned)m_wave;
+    if(mask_row >= p.n_masks) mask_row %= p.n_masks;
+    mk = p.mask + (size_t)mask_row * p.len;
   }
+  const float mk0 = *(mk ? mk + min(lane, p.len - 1) : p.partials);   // (the latter not looked at)
   float bqm[NPROJ];
 #pragma unroll
   for(int g = 0; g < NPROJ; ++g) bqm[g] = tail_quant_mult(p.Bq[g], (size_t)K * (size_t)N);
@@ -1012,8 +1062,8 @@ __global__ __launch_bounds__(kProjThreads) void proj_attention_kernel(ProjAttent
     const int item = min(it * kProjThreads + tid, kItems - 1);
     const int tg = item / (R * 8), pc = item % 8;
     const float* b = p.bias[tg / 2];
-    bias4[it] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
-    if(b) bias4[it] = *reinterpret_cast<const v4f*>(b + h * 64 + (tg % 2) * 32 + pc * 4);
+    // (no bias: sixteen bytes of the weights instead, not looked at)
+    bias4[it] = *reinterpret_cast<const v4f*>(b ? b + h * 64 + (tg % 2) * 32 + pc * 4 : reinterpret_cast<const float*>(p.Bq[0]));
   }
 
   // ---- 1, 2: abs-max, quantize into LDS ----
@@ -1021,6 +1071,20 @@ __global__ __launch_bounds__(kProjThreads) void proj_attention_kernel(ProjAttent
 #pragma unroll
   for(int i = 0; i < kAbsmaxSlots / kProjThreads; ++i) amax = fmaxf(amax, pm[i]);
   amax = block_max(amax, red);
+  // The keys and values are asked for last - a wave's loads complete in the order of their issue,
+  // and they are needed last - and only now: in front of the abs-max values they would delay them.
+  // No branches around them (positions past the end repeat the last one; the number of loads is
+  // the kernel's), so that the waits in front of the earlier loads' uses count exactly.
+  if constexpr(STAGED) {
+#pragma unroll
+    for(int seg = 0; seg < SEGS; ++seg) {
+      const unsigned entry = (unsigned)(sent_base + (seg >> 1)) * (unsigned)p.heads + (unsigned)h;
+      const float* src = ((seg & 1) ? p.v_cache : p.k_cache) + (size_t)entry * p.kv_cap * 64 + (tid % 16) * 4;
+#pragma unroll
+      for(int j = 0; j < PASSES; ++j)
+        stage[seg][j] = *reinterpret_cast<const v4f*>(src + (size_t)min(tid / 16 + 32 * j, p.len - 1) * 64);
+    }
+  }
   const float aqm = quant_mult_from_maxabs(amax);
   const bool finite = aqm < __builtin_inff();
   float unquant[NPROJ];
@@ -1031,7 +1095,7 @@ __global__ __launch_bounds__(kProjThreads) void proj_attention_kernel(ProjAttent
 #pragma unroll
     for(int e = 0; e < 4; ++e) q[e] = finite ? quantize_pack4_finite(in[e], aqm) : quantize_pack4(in[e], aqm);
     const int slot0 = (c16 / 2) * 64, x = r_in ^ proj_row_key(c16);
-    const int m = m_base + r_in;
+    const int m = row_of(min(r_in, R - 1));
 #pragma unroll
     for(int e = 0; e < 4; ++e) {
       const int sw = slot0 + (e / 2) * 64 + (e % 2) * 32 + (x ^ e);
@@ -1096,7 +1160,7 @@ __global__ __launch_bounds__(kProjThreads) void proj_attention_kernel(ProjAttent
       }
       const v4f yv = v4f{y[0], y[1], y[2], y[3]};
       *reinterpret_cast<v4f*>(proj_lds + (g * R + r) * 64 + col) = yv;
-      const int m = m_base + r;
+      const int m = row_of(r);
       if(m < M) {
         if(p.proj_out[g]) *reinterpret_cast<v4f*>(p.proj_out[g] + (size_t)m * (size_t)N + h * 64 + col) = yv;
         if(NPROJ == 3 && g > 0) {
@@ -1107,13 +1171,23 @@ __global__ __launch_bounds__(kProjThreads) void proj_attention_kernel(ProjAttent
       }
     }
   }
+  if constexpr(STAGED) {
+#pragma unroll
+    for(int seg = 0; seg < SEGS; ++seg) {
+#pragma unroll
+      for(int j = 0; j < PASSES; ++j) {
+        const int pos = tid / 16 + 32 * j;
+        if(pos < p.len) *reinterpret_cast<v4f*>(kv_lds + ((size_t)(seg * p.len + pos) * 64 + (tid % 16) * 4)) = stage[seg][j];
+      }
+    }
+  }
   __syncthreads();
 
   // ---- 5: the attention of row `wave` ----
   const int rows_total = M * p.heads;
   if(p.absmax_out && blockIdx.x == 0 && blockIdx.y == 0)   // slots past the last query row
     for(int sl = rows_total + tid; sl < kAbsmaxSlots; sl += kProjThreads) p.absmax_out[sl] = 0.0f;
-  const int m = m_base + wave;
+  const int m = m_wave;
   if(wave < R && m < M) {   // (whole waves)
     const unsigned wr = (unsigned)m * (unsigned)p.heads + (unsigned)h;
     const unsigned entry = wr < p.batchKV ? wr : wr % p.batchKV;
@@ -1122,16 +1196,18 @@ __global__ __launch_bounds__(kProjThreads) void proj_attention_kernel(ProjAttent
     const float* q = proj_lds + wave * 64;
     const float* k_last = NPROJ == 3 ? proj_lds + (R + wave) * 64 : kb + (size_t)(p.len - 1) * 64;
     const float* v_last = NPROJ == 3 ? proj_lds + (2 * R + wave) * 64 : vb + (size_t)(p.len - 1) * 64;
-    const float* mk = nullptr;
-    if(p.mask) {
-      unsigned mask_row = (unsigned)m;
-      if(mask_row >= p.n_masks) mask_row %= p.n_masks;
-      mk = p.mask + (size_t)mask_row * p.len;
-    }
     const int len4 = (p.len + 3) & ~3;
     float* sc = att_lds + wave * (len4 + 256);
-    float omax = attention_row64(q, kb, vb, k_last, v_last, mk, p.len, p.att_scale, sc, sc + len4,
-                                 p.out + (size_t)wr * 64, lane);
+    float omax;
+    if constexpr(STAGED) {
+      const float* ks = kv_lds + (size_t)(2 * (wave & ((1 << p.share_shift) - 1))) * p.len * 64;
+      const float* vs = ks + (size_t)p.len * 64;
+      omax = attention_row64<true>(q, ks, vs, ks + (size_t)(p.len - 1) * 64, vs + (size_t)(p.len - 1) * 64, mk, mk0, p.len,
+                             p.att_scale, sc, sc + len4, p.out + (size_t)wr * 64, lane);
+    } else {
+      omax = attention_row64(q, kb, vb, k_last, v_last, mk, mk0, p.len, p.att_scale, sc, sc + len4,
+                             p.out + (size_t)wr * 64, lane);
+    }
     if(p.absmax_out) {
       omax = wave_maxf(omax);
       if(lane == 0) p.absmax_out[wr] = omax;
@@ -2122,24 +2198,64 @@ int marian_hip_int8_proj_attention(const float* A, int8_t* Aq, int64_t n_proj, c
   p.att_scale = att_scale; p.out = out; p.absmax_out = absmax_out;
   constexpr int R = 8;
   const int len4 = ((int)len + 3) & ~3;
-  const size_t lds = (size_t)32 * (size_t)K + (size_t)n_proj * 8 * R * 128 + (size_t)n_proj * R * 64 * 4 +
-                     (size_t)R * (size_t)(len4 + 256) * 4;
+  size_t lds = (size_t)32 * (size_t)K + (size_t)n_proj * 8 * R * 128 + (size_t)n_proj * R * 64 * 4 +
+               (size_t)R * (size_t)(len4 + 256) * 4;
   {   // the kernels' dynamic LDS limit, raised once per device (one bit per device)
     static std::atomic<uint64_t> lds_done{0};
     int dev = 0;
     MH_HIP(hipGetDevice(&dev));
     if(dev < 0 || dev >= 64) return MARIAN_HIP_ERR_RANGE;
     if(!(lds_done.load(std::memory_order_acquire) & (1ull << dev))) {
-      MH_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(proj_attention_kernel<1, R>),
+      const void* staged[] = {
+          reinterpret_cast<const void*>(proj_attention_kernel<1, R, 2, 1>), reinterpret_cast<const void*>(proj_attention_kernel<1, R, 2, 2>),
+          reinterpret_cast<const void*>(proj_attention_kernel<1, R, 2, 3>), reinterpret_cast<const void*>(proj_attention_kernel<1, R, 4, 1>),
+          reinterpret_cast<const void*>(proj_attention_kernel<1, R, 4, 2>), reinterpret_cast<const void*>(proj_attention_kernel<1, R, 4, 3>)};
+      for(const void* f : staged) MH_HIP(hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, kProjMaxLds));
+      MH_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(proj_attention_kernel<1, R, 0, 0>),
                                  hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024));
-      MH_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(proj_attention_kernel<3, R>),
+      MH_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(proj_attention_kernel<3, R, 0, 0>),
                                  hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024));
       lds_done.fetch_or(1ull << dev, std::memory_order_release);
     }
   }
+  p.share_shift = -1;
+  p.share_nb = 0;
+  p.stage_kv = 0;
+  if(n_proj == 1 && batchKV % heads == 0) {
+    const int64_t nb = batchKV / heads;   // sentences; row m attends to sentence m % nb
+    if(nb < M && M % nb == 0) {
+      const int64_t hyps = M / nb;
+      const int per_wg = hyps % 8 == 0 ? 8 : (hyps % 4 == 0 ? 4 : (hyps % 2 == 0 ? 2 : 1));
+      const int shift = per_wg == 8 ? 0 : (per_wg == 4 ? 1 : 2);
+      if(per_wg > 1 && nb % (1 << shift) == 0) {
+        p.share_shift = shift;
+        p.share_nb = (int)nb;
+        const size_t kv_bytes = (size_t)(2 << shift) * (size_t)len * 256;
+        if(shift <= 1 && len <= kProjStageLen && lds + kv_bytes <= (size_t)kProjMaxLds) {
+          p.stage_kv = 1;
+          lds += kv_bytes;
+        }
+      }
+    }
+  }
   const dim3 grid((unsigned)heads, (unsigned)((M + R - 1) / R));
-  if(n_proj == 3) hipLaunchKernelGGL((proj_attention_kernel<3, R>), grid, dim3(kProjThreads), lds, st, p);
-  else hipLaunchKernelGGL((proj_attention_kernel<1, R>), grid, dim3(kProjThreads), lds, st, p);
+#define MH_PA(NP, SEGS, PASSES) \
+  hipLaunchKernelGGL((proj_attention_kernel<NP, R, SEGS, PASSES>), grid, dim3(kProjThreads), lds, st, p)
+  if(n_proj == 3) MH_PA(3, 0, 0);
+  else if(!p.stage_kv) MH_PA(1, 0, 0);
+  else {
+    const int passes = ((int)len + 31) / 32;   // 1 .. 3
+    if(p.share_shift == 0) {   // one sentence per workgroup
+      if(passes == 1) MH_PA(1, 2, 1);
+      else if(passes == 2) MH_PA(1, 2, 2);
+      else MH_PA(1, 2, 3);
+    } else {
+      if(passes == 1) MH_PA(1, 4, 1);
+      else if(passes == 2) MH_PA(1, 4, 2);
+      else MH_PA(1, 4, 3);
+    }
+  }
+#undef MH_PA
   MH_HIP(hipGetLastError());
   return MARIAN_HIP_OK;
 }

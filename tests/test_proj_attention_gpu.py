@@ -76,7 +76,13 @@ def test_self_attention_form_equals_the_separate_calls(integer, orc, synth, M, K
 
 
 @pytest.mark.parametrize("M,K,heads,batch,L,masked,chained", [(128, 1024, 16, 32, 60, True, True), (128, 1024, 16, 32, 21, False, False),
-                                                              (30, 512, 8, 10, 7, True, True), (12, 256, 4, 12, 200, True, False)])
+                                                              (30, 512, 8, 10, 7, True, True), (12, 256, 4, 12, 200, True, False),
+                                                              # hypotheses of a sentence in one workgroup: 8, 4, 2 of them; lengths
+                                                              # at and past what is staged in LDS; an odd number of sentences
+                                                              (64, 256, 4, 8, 96, True, True), (64, 256, 4, 8, 97, True, False),
+                                                              (32, 256, 4, 16, 33, True, True), (48, 128, 2, 12, 50, False, True),
+                                                              (40, 128, 2, 10, 64, True, False), (20, 128, 2, 5, 30, True, True),
+                                                              (128, 1024, 16, 16, 1, True, True)])
 def test_context_attention_form_equals_the_separate_calls(integer, orc, synth, M, K, heads, batch, L, masked, chained):
     import torch
     ops = load("ops")
