@@ -844,7 +844,9 @@ __global__ __launch_bounds__(256) void attention_kernel(const float* __restrict_
 // asking for a row's keys and values at kernel start (loads into a scratch word of LDS, by the
 // multiplying waves or by two more waves), or into registers once the abs-max is known in the
 // self-attention form - the attention then waits less and the quantization more, for the same
-// bytes; barriers that put every wave's small requests in front of any wave's large ones.
+// bytes; barriers that put every wave's small requests in front of any wave's large ones; the
+// workgroups of a head starting at different sub-steps of K, so that they would not all miss L2 on
+// the same lines of the weights at the same time (+5 us per step).
 constexpr int kProjThreads = 512, kProjMaxK = 1024, kProjMaxLen = 512;
 // keys and values shared by the rows of a workgroup are staged in LDS up to this many positions
 constexpr int kProjStageLen = 96;
