@@ -82,7 +82,9 @@ def test_self_attention_form_equals_the_separate_calls(integer, orc, synth, M, K
                                                               (64, 256, 4, 8, 96, True, True), (64, 256, 4, 8, 97, True, False),
                                                               (32, 256, 4, 16, 33, True, True), (48, 128, 2, 12, 50, False, True),
                                                               (40, 128, 2, 10, 64, True, False), (20, 128, 2, 5, 30, True, True),
-                                                              (128, 1024, 16, 16, 1, True, True)])
+                                                              (128, 1024, 16, 16, 1, True, True),
+                                                              # the most LDS the staged form asks for
+                                                              (128, 1024, 16, 32, 96, True, False)])
 def test_context_attention_form_equals_the_separate_calls(integer, orc, synth, M, K, heads, batch, L, masked, chained):
     import torch
     ops = load("ops")
