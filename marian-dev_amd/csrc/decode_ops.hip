@@ -880,6 +880,16 @@ struct ProjAttentionArgs {
   int stage_kv;
 };
 
+// Entry g of one of the argument arrays, g differing between the threads: selected from the three
+// values in scalar registers.  (Indexed by a thread-dependent g the compiler reads the entry from
+// the kernel-argument memory with a vector load, and the wait for it - loads complete in order -
+// is a wait for every load the thread has issued before: the weights.)
+template <typename T>
+__device__ __forceinline__ T pick3(const T (&a)[3], int g) {
+  const T a0 = a[0], a1 = a[1], a2 = a[2];   // (values: a conditional between the elements themselves selects an address)
+  return g == 0 ? a0 : (g == 1 ? a1 : a2);
+}
+
 // the row permutation of the staged activations (gemm_stream32_kernel.h: stream32_row_key)
 __device__ __forceinline__ int proj_row_key(int c16) { return (c16 ^ (c16 >> 2)) & 7; }
 
@@ -1035,11 +1045,12 @@ __global__ __launch_bounds__(kProjThreads) void proj_attention_kernel(ProjAttent
   }
   v4i w[NPROJ][8];
   const int ncol = h * 64 + wn * 32 + li;
+  // (asked for in the order the multiplication takes them: sub-step by sub-step, all projections)
 #pragma unroll
-  for(int g = 0; g < NPROJ; ++g) {
-    const int8_t* wrow = p.Bq[g] + stream32_lane_offset(ncol, lg);
+  for(int pp = 0; pp < 8; ++pp) {
+    const size_t at = stream32_lane_offset(ncol, lg) + (size_t)stream32_clamped_substep(kw * PW + pp, S) * 32u * (size_t)N;
 #pragma unroll
-    for(int pp = 0; pp < 8; ++pp) w[g][pp] = load16(wrow + (size_t)stream32_clamped_substep(kw * PW + pp, S) * 32u * (size_t)N);
+    for(int g = 0; g < NPROJ; ++g) w[g][pp] = load16(p.Bq[g] + at);
   }
   // keys and values of the workgroup's sentences: sixteen threads per position, 32 positions per pass
   constexpr int kStageSegs = STAGED ? SEGS : 1, kStagePasses = STAGED ? PASSES : 1;
@@ -1063,7 +1074,7 @@ __global__ __launch_bounds__(kProjThreads) void proj_attention_kernel(ProjAttent
   for(int it = 0; it < 2; ++it) {
     const int item = min(it * kProjThreads + tid, kItems - 1);
     const int tg = item / (R * 8), pc = item % 8;
-    const float* b = p.bias[tg / 2];
+    const float* b = pick3(p.bias, tg / 2);
     // (no bias: sixteen bytes of the weights instead, not looked at)
     bias4[it] = *reinterpret_cast<const v4f*>(b ? b + h * 64 + (tg % 2) * 32 + pc * 4 : reinterpret_cast<const float*>(p.Bq[0]));
   }
@@ -1152,7 +1163,7 @@ __global__ __launch_bounds__(kProjThreads) void proj_attention_kernel(ProjAttent
       for(int t = 1; t < 4; ++t) sum += *reinterpret_cast<const v4i*>(src + t * (R * 128));
       float uq = unquant[0];
       if constexpr(NPROJ == 3) uq = g == 0 ? unquant[0] : (g == 1 ? unquant[1] : unquant[2]);
-      const bool has_bias = p.bias[g] != nullptr;
+      const bool has_bias = pick3(p.bias, g) != nullptr;
       const float b[4] = {bias4[it].x, bias4[it].y, bias4[it].z, bias4[it].w};
       float y[4];
 #pragma unroll
@@ -1164,7 +1175,8 @@ __global__ __launch_bounds__(kProjThreads) void proj_attention_kernel(ProjAttent
       *reinterpret_cast<v4f*>(proj_lds + (g * R + r) * 64 + col) = yv;
       const int m = row_of(r);
       if(m < M) {
-        if(p.proj_out[g]) *reinterpret_cast<v4f*>(p.proj_out[g] + (size_t)m * (size_t)N + h * 64 + col) = yv;
+        float* const po = pick3(p.proj_out, g);
+        if(po) *reinterpret_cast<v4f*>(po + (size_t)m * (size_t)N + h * 64 + col) = yv;
         if(NPROJ == 3 && g > 0) {
           float* cache = g == 1 ? p.k_cache : p.v_cache;
           const size_t entry = (size_t)m * (size_t)p.heads + (size_t)h;
