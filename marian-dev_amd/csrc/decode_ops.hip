@@ -1012,13 +1012,8 @@ __global__ __launch_bounds__(kProjThreads) void proj_attention_kernel(ProjAttent
   const int wn = wave % 2, kw = wave / 2, li = lane % 32, lg = lane / 32;
   const int h = blockIdx.x;
   // input row r of this workgroup (rows past the end: M or more)
-  const int sent_groups = p.share_shift < 0 ? 1 : p.share_nb >> p.share_shift;
-  const int hyp_base = p.share_shift < 0 ? 0 : ((int)blockIdx.y / sent_groups) * (R >> p.share_shift);
-  const int sent_base = p.share_shift < 0 ? 0 : ((int)blockIdx.y % sent_groups) << p.share_shift;
-  auto row_of = [&](int r) -> int {
-    if(p.share_shift < 0) return (int)blockIdx.y * R + r;
-    return (hyp_base + (r >> p.share_shift)) * p.share_nb + sent_base + (r & ((1 << p.share_shift) - 1));
-  };
+  const int sent_base = p.share_shift < 0 ? 0 : proj_first_sentence(p.share_shift, p.share_nb, (int)blockIdx.y);
+  auto row_of = [&](int r) -> int { return proj_row_of(p.share_shift, p.share_nb, (int)blockIdx.y, r); };
   const int K = p.K, M = p.M, S = K / 32, PW = S / 4, N = p.heads * 64;
   int8_t* a_lds = plds;                                   // 32 rows x K bytes, operand order
   int8_t* part_lds = a_lds + 32 * K;                      // NPROJ x 2 x 4 partial tiles of R rows x 128 bytes
@@ -2232,26 +2227,11 @@ int marian_hip_int8_proj_attention(const float* A, int8_t* Aq, int64_t n_proj, c
       lds_done.fetch_or(1ull << dev, std::memory_order_release);
     }
   }
-  p.share_shift = -1;
-  p.share_nb = 0;
-  p.stage_kv = 0;
-  if(n_proj == 1 && batchKV % heads == 0) {
-    const int64_t nb = batchKV / heads;   // sentences; row m attends to sentence m % nb
-    if(nb < M && M % nb == 0) {
-      const int64_t hyps = M / nb;
-      const int per_wg = hyps % 8 == 0 ? 8 : (hyps % 4 == 0 ? 4 : (hyps % 2 == 0 ? 2 : 1));
-      const int shift = per_wg == 8 ? 0 : (per_wg == 4 ? 1 : 2);
-      if(per_wg > 1 && nb % (1 << shift) == 0) {
-        p.share_shift = shift;
-        p.share_nb = (int)nb;
-        const size_t kv_bytes = (size_t)(2 << shift) * (size_t)len * 256;
-        if(shift <= 1 && len <= kProjStageLen && lds + kv_bytes <= (size_t)kProjMaxLds) {
-          p.stage_kv = 1;
-          lds += kv_bytes;
-        }
-      }
-    }
-  }
+  const ProjRowPlan plan = proj_row_plan(n_proj, M, heads, batchKV, len, kProjStageLen, lds, (size_t)kProjMaxLds);
+  p.share_shift = plan.shift;
+  p.share_nb = plan.sentences;
+  p.stage_kv = plan.stage;
+  if(plan.stage) lds += (size_t)(2 << plan.shift) * (size_t)len * 256;
   const dim3 grid((unsigned)heads, (unsigned)((M + R - 1) / R));
 #define MH_PA(NP, SEGS, PASSES) \
   hipLaunchKernelGGL((proj_attention_kernel<NP, R, SEGS, PASSES>), grid, dim3(kProjThreads), lds, st, p)

@@ -84,4 +84,42 @@ __host__ __device__ __forceinline__ size_t stage_b_offset(int g, int tiles_n, in
 // A last block of 64 columns has no sub-steps 2, 3: such loads go two sub-steps (64 * N bytes) back.
 __host__ __device__ __forceinline__ bool stage_b_goes_back(int g, int tiles_n) { return g / tiles_n >= 2; }
 
+// ---- projections + attention in one launch (proj_attention_kernel): which input rows a workgroup takes ----
+// Caches that are complete and shared - `sentences` entries per head, row m attends to sentence
+// m % sentences, M = hypotheses * sentences - let a workgroup take 8 >> shift hypotheses of
+// 1 << shift neighbouring sentences instead of eight consecutive rows, so that the waves reading
+// the same keys and values sit on one CU.  shift < 0: eight consecutive rows.
+struct ProjRowPlan {
+  int shift;       // log2 of the sentences per workgroup, or -1
+  int sentences;
+  int stage;       // the sentences' keys and values are staged in LDS (shift 0 or 1, len <= stage_len)
+};
+__host__ __device__ __forceinline__ ProjRowPlan proj_row_plan(long long n_proj, long long M, long long heads, long long batchKV,
+                                                              long long len, int stage_len, size_t lds_without,
+                                                              size_t lds_max) {
+  ProjRowPlan plan = {-1, 0, 0};
+  if(n_proj != 1 || heads <= 0 || batchKV % heads != 0) return plan;
+  const long long nb = batchKV / heads;
+  if(nb <= 0 || nb >= M || M % nb != 0) return plan;
+  const long long hyps = M / nb;
+  const int per_wg = hyps % 8 == 0 ? 8 : (hyps % 4 == 0 ? 4 : (hyps % 2 == 0 ? 2 : 1));
+  const int shift = per_wg == 8 ? 0 : (per_wg == 4 ? 1 : 2);
+  if(per_wg == 1 || nb % (1 << shift) != 0 || nb > 2147483647LL) return plan;
+  plan.shift = shift;
+  plan.sentences = (int)nb;
+  const size_t kv_bytes = (size_t)(2 << shift) * (size_t)len * 256;
+  plan.stage = shift <= 1 && len <= stage_len && lds_without + kv_bytes <= lds_max;
+  return plan;
+}
+// input row r (0 .. 7) of workgroup block_y
+__host__ __device__ __forceinline__ int proj_row_of(int shift, int sentences, int block_y, int r) {
+  if(shift < 0) return block_y * 8 + r;
+  const int groups = sentences >> shift;
+  return ((block_y / groups) * (8 >> shift) + (r >> shift)) * sentences + ((block_y % groups) << shift) + (r & ((1 << shift) - 1));
+}
+// first sentence of workgroup block_y (shift >= 0)
+__host__ __device__ __forceinline__ int proj_first_sentence(int shift, int sentences, int block_y) {
+  return (block_y % (sentences >> shift)) << shift;
+}
+
 }  // namespace marian_hip

@@ -153,6 +153,45 @@ static void staged(int BM, int BN, int waves, int M, int K, int N, const std::ve
     }
 }
 
+// The rows the workgroups of the one-launch projections + attention take: every row exactly once,
+// the rows of a workgroup that share a sentence slot attend to that sentence, and every staged
+// key/value load (and LDS slot) lies inside the caches (the staging area).
+static void proj_rows(long long hyps, long long sentences, long long heads, long long len, long long cap) {
+  const long long M = hyps * sentences, batchKV = sentences * heads;
+  const int stage_len = 96;
+  const size_t lds_without = 32 * 1024 + 8 * 8 * 128 + 8 * 64 * 4 + 8 * (size_t)(((len + 3) & ~3LL) + 256) * 4;
+  const size_t lds_max = 160 * 1024 - 256;
+  const ProjRowPlan plan = proj_row_plan(1, M, heads, batchKV, len, stage_len, lds_without, lds_max);
+  char where[160];
+  std::snprintf(where, sizeof(where), "proj rows hyps %lld sentences %lld len %lld shift %d stage %d", hyps, sentences, len,
+                plan.shift, plan.stage);
+  const int blocks = (int)((M + 7) / 8);
+  std::vector<int> seen((size_t)M, 0);
+  for(int by = 0; by < blocks; ++by)
+    for(int r = 0; r < 8; ++r) {
+      const int m = proj_row_of(plan.shift, plan.sentences, by, r);
+      ++g_checked;
+      if(m < 0) { fail("negative row", by, r, where); continue; }
+      if(m >= M) continue;   // rows past the end are skipped by the kernel
+      ++seen[(size_t)m];
+      if(plan.shift >= 0) {
+        const int slot = r & ((1 << plan.shift) - 1);
+        const int sentence = proj_first_sentence(plan.shift, plan.sentences, by) + slot;
+        if(sentence >= sentences || m % sentences != sentence) fail("row outside its sentence", by, r, where);
+        if(plan.stage) {   // the loads of segment 2 * slot (keys) and 2 * slot + 1 (values)
+          const long long entry = (long long)sentence * heads + (heads - 1);
+          const long long last = (entry * cap + (len - 1)) * 64 + 63;
+          if(entry >= batchKV || last >= batchKV * cap * 64) fail("staged load outside the cache", by, r, where);
+          const size_t lds_end = lds_without + (size_t)(2 * slot + 2) * (size_t)len * 256;
+          if(lds_end > lds_max) fail("staging area past the LDS", by, r, where);
+          if(plan.shift > 1 || len > stage_len) fail("staged beyond what the kernels hold", by, r, where);
+        }
+      }
+    }
+  for(long long m = 0; m < M; ++m)
+    if(seen[(size_t)m] != 1) { fail("row coverage", (int)m, seen[(size_t)m], where); break; }
+}
+
 int main() {
   const int Ks[] = {64, 192, 576, 1088, 1024};
   const int Ns[] = {8, 24, 1000, 1032};
@@ -189,6 +228,12 @@ int main() {
             for(auto& sl : shortlists(N, 8)) staged(c[0], c[1], c[2], M, K, N, &sl);
         }
   std::printf("staged: %lld loads checked\n", g_checked - before);
+  before = g_checked;
+  for(long long hyps : {1, 2, 3, 4, 6, 8, 12, 16})
+    for(long long sentences : {1, 2, 3, 5, 8, 10, 32, 33})
+      for(long long len : {1, 31, 32, 33, 60, 96, 97, 300})
+        proj_rows(hyps, sentences, 16, len, len + 3);
+  std::printf("projection rows: %lld rows checked\n", g_checked - before);
   if(g_failures) {
     std::fprintf(stderr, "%d failures\n", g_failures);
     return 1;

@@ -29,7 +29,7 @@ def test_kernels_use_the_checked_helpers():
         "gemm_stream_kernel.h": ["stream16_lane_offset("],
         "gemm_mfma32_kernel.h": ["stage_a_offset(", "stage_b_column(", "stage_b_offset(", "stage_a_tail_adjust(", "stage_b_goes_back("],
         "gemm_pair_kernel.h": ["stage_a_row(", "stage_a_chunk(", "stage_b_offset("],
-        "decode_ops.hip": ["stream32_lane_offset(", "stream32_clamped_substep("],
+        "decode_ops.hip": ["stream32_lane_offset(", "stream32_clamped_substep(", "proj_row_plan(", "proj_row_of(", "proj_first_sentence("],
     }
     for name, calls in uses.items():
         text = open(os.path.join(CSRC, name)).read()
