@@ -211,11 +211,10 @@ int marian_hip_int8_affine_f32_grouped(const float* A, int8_t* Aq, int64_t n_gro
  *     needs M * heads <= 2048; the workspace is only used when absmax_in is NULL).
  * The result has the bits of the separate calls (marian_hip_int8_affine_f32_grouped, then
  * marian_hip_attention_cached).  When to use it (measured with d = 1024, 16 heads, 21 cached / 60
- * source positions, calls back to back): n_proj = 3 is ahead of the two separate calls at 128 rows
- * (12.2 against 13.0 us) and behind from 256 rows on (24.2 against 22.8 us: every eight rows read
- * the head's weights again); n_proj = 1 stays ahead (9.8 against 11.7 us at 128 rows, 35 against
- * 50 us at 512), because the separate attention reads a sentence's keys and values once per
- * hypothesis.
+ * source positions, calls back to back): it is ahead of the two separate calls up to 128 rows
+ * (n_proj = 3: 11.7 against 13.1 us, n_proj = 1: 9.5 against 11.5 us), level at 256 rows (23.2
+ * against 22.7, 17.8 against 17.5 us) and behind beyond (512 rows: 41.8 against 43.4 us, but 34.1
+ * against 28.1 us for n_proj = 1): every eight rows read the head's weights again.
  */
 int marian_hip_int8_proj_attention(const float* A, int8_t* Aq, int64_t n_proj, const int8_t* const* Bq,
                                    const float* const* bias, float* const* proj_out, int64_t M, int64_t K,

@@ -995,6 +995,70 @@ __device__ __forceinline__ float attention_row64(const float* q, const float* kb
   return fabsf(o);
 }
 
+// Attention over caches that several query rows share (the encoder's keys and values: query row
+// r reads cache entry r % batchKV, so rows e, e + batchKV, e + 2 batchKV, .. - the hypotheses of a
+// sentence, for one head - read the same entry).  Workgroup (e, y) takes rows e + (4 y + w) batchKV
+// for its waves w = 0 .. 3, reads entry e's keys and values once (sixteen threads per position,
+// PASSES passes of sixteen positions; positions past the end repeat the last one) into LDS, and each
+// wave then runs attention_row64 on them: the operations of attention_kernel's 64-wide path in the
+// same order, so the same bits, with a quarter (for four hypotheses) of the bytes through the
+// CU's memory path and out of L2.  One position per query row, head size 64, len <= 16 * PASSES.
+constexpr int kSharedAttLen = 96;
+template <int PASSES>
+__global__ __launch_bounds__(256) void attention_shared_kernel(const float* __restrict__ Q, const float* __restrict__ Kt,
+                                                               const float* __restrict__ V, const float* __restrict__ mask,
+                                                               unsigned n_masks, unsigned rows_per_mask,
+                                                               float* __restrict__ out, unsigned rows_total,
+                                                               unsigned batchKV, int len, int kv_cap, float scale,
+                                                               float* __restrict__ absmax_out) {
+  static_assert(PASSES * 16 <= kSharedAttLen, "sixteen positions per pass");
+  extern __shared__ __attribute__((aligned(16))) float satt_lds[];
+  const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
+  const unsigned entry = blockIdx.x;
+  const unsigned wr = entry + (blockIdx.y * 4u + (unsigned)wave) * batchKV;
+  const bool valid = wr < rows_total;
+  if(absmax_out && blockIdx.x == 0 && blockIdx.y == 0)   // slots past the last query row
+    for(int sl = (int)rows_total + tid; sl < kAbsmaxSlots; sl += 256) absmax_out[sl] = 0.0f;
+  // everything is requested before anything is used: keys, values, the mask value of this lane
+  v4f kst[PASSES], vst[PASSES];
+  {
+    const float* ksrc = Kt + (size_t)entry * kv_cap * 64 + (tid % 16) * 4;
+    const float* vsrc = V + (size_t)entry * kv_cap * 64 + (tid % 16) * 4;
+#pragma unroll
+    for(int j = 0; j < PASSES; ++j) kst[j] = *reinterpret_cast<const v4f*>(ksrc + (size_t)min(tid / 16 + 16 * j, len - 1) * 64);
+#pragma unroll
+    for(int j = 0; j < PASSES; ++j) vst[j] = *reinterpret_cast<const v4f*>(vsrc + (size_t)min(tid / 16 + 16 * j, len - 1) * 64);
+  }
+  const float* mk = nullptr;
+  if(mask && valid) {
+    unsigned mask_row = rows_per_mask == 1 ? wr : wr / rows_per_mask;
+    if(mask_row >= n_masks) mask_row %= n_masks;
+    mk = mask + (size_t)mask_row * len;
+  }
+  const float mk0 = *(mk ? mk + min(lane, len - 1) : Q);   // (the latter not looked at)
+  const int len4 = (len + 3) & ~3;
+  float* ks = satt_lds;                       // [len][64]
+  float* vs = ks + (size_t)len * 64;          // [len][64]
+  float* sc = vs + (size_t)len * 64 + wave * (len4 + 256);   // per wave: scores + 256 partial outputs
+#pragma unroll
+  for(int j = 0; j < PASSES; ++j) {
+    const int pos = tid / 16 + 16 * j;
+    if(pos < len) {
+      *reinterpret_cast<v4f*>(ks + (size_t)pos * 64 + (tid % 16) * 4) = kst[j];
+      *reinterpret_cast<v4f*>(vs + (size_t)pos * 64 + (tid % 16) * 4) = vst[j];
+    }
+  }
+  __syncthreads();
+  if(valid) {   // (whole waves)
+    float omax = attention_row64<true>(Q + (size_t)wr * 64, ks, vs, ks + (size_t)(len - 1) * 64, vs + (size_t)(len - 1) * 64, mk,
+                                       mk0, len, scale, sc, sc + len4, out + (size_t)wr * 64, lane);
+    if(absmax_out) {
+      omax = wave_maxf(omax);
+      if(lane == 0) absmax_out[wr] = omax;
+    }
+  }
+}
+
 // NPROJ: 3 (q, k_new, v_new: self-attention, the new key/value row is appended to the caches) or
 // 1 (q only: attention over caches that are complete, e.g. the encoder's).  R: input rows per
 // workgroup, 8 (a wave per row in the attention).
@@ -2135,6 +2199,24 @@ static int attention_impl(const float* q, float* k, float* v, const float* mask,
                                  hipFuncAttributeMaxDynamicSharedMemorySize, 72 * 1024));
       lds_done.fetch_or(1ull << dev, std::memory_order_release);
     }
+  }
+  // Complete caches that several query rows share, head size 64, one position per row, everything
+  // aligned for 16-byte loads: the rows of a cache entry in one workgroup, the entry read once.
+  if(!ancestors && !k_new && dk == 64 && m == 1 && len <= kSharedAttLen && batchKV < rows_total && rows_total % batchKV == 0 &&
+     rows_total / batchKV <= 4 * 65535 && aligned16(q) && aligned16(k) && aligned16(v) && aligned16(out)) {
+    const long long hyps = rows_total / batchKV;
+    const dim3 grid((unsigned)batchKV, (unsigned)((hyps + 3) / 4));
+    const size_t slds = (size_t)2 * (size_t)len * 256 + lds;
+#define MH_SATT(PASSES) \
+    hipLaunchKernelGGL(attention_shared_kernel<PASSES>, grid, dim3(256), slds, st, q, k, v, mask, (unsigned)n_masks, \
+                       (unsigned)rows_per_mask, out, (unsigned)rows_total, (unsigned)batchKV, (int)len, (int)kv_capacity, \
+                       scale, absmax_out)
+    if(len <= 32) MH_SATT(2);
+    else if(len <= 64) MH_SATT(4);
+    else MH_SATT(6);
+#undef MH_SATT
+    MH_HIP(hipGetLastError());
+    return MARIAN_HIP_OK;
   }
   if(ancestors)
     hipLaunchKernelGGL(attention_kernel<true>, dim3((unsigned)((rows_total + 3) / 4)), dim3(256), lds, st, q, k, v,

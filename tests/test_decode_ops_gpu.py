@@ -301,7 +301,11 @@ def test_absmax_outputs_of_layer_norm_and_attention(ops, integer, synth):
 @pytest.mark.parametrize("beam,entries,L,masked,rows_per_mask", [(4, 512, 60, True, 16), (4, 512, 21, False, 1),
                                                                (2, 48, 130, True, 16), (3, 16, 7, True, 1),
                                                                (6, 32, 64, True, 16), (12, 8, 1, False, 1),
-                                                               (8, 5, 1024, True, 1)])
+                                                               (8, 5, 1024, True, 1),
+                                                               # around the lengths up to which the rows of an entry
+                                                               # share its keys and values through LDS (32, 64, 96)
+                                                               (4, 64, 96, True, 16), (5, 16, 97, True, 1),
+                                                               (2, 32, 33, False, 1), (9, 4, 32, True, 1), (4, 32, 65, True, 16)])
 def test_attention_rows_that_share_keys_and_values(ops, synth, beam, entries, L, masked, rows_per_mask):
     """hypotheses of a sentence over the encoder's keys and values: the call that names the shared
     cache once (batchKV = batchQ / beam, query row i reads entry i % batchKV) gives the bits of the
