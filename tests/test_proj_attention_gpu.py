@@ -84,7 +84,9 @@ def test_self_attention_form_equals_the_separate_calls(integer, orc, synth, M, K
                                                               (40, 128, 2, 10, 64, True, False), (20, 128, 2, 5, 30, True, True),
                                                               (128, 1024, 16, 16, 1, True, True),
                                                               # the most LDS the staged form asks for
-                                                              (128, 1024, 16, 32, 96, True, False)])
+                                                              (128, 1024, 16, 32, 96, True, False),
+                                                              # more workgroups than CUs
+                                                              (256, 256, 4, 64, 40, True, True), (512, 128, 2, 64, 20, True, False)])
 def test_context_attention_form_equals_the_separate_calls(integer, orc, synth, M, K, heads, batch, L, masked, chained):
     import torch
     ops = load("ops")
