@@ -123,6 +123,53 @@ def test_context_attention_form_equals_the_separate_calls(integer, orc, synth, M
     assert torch.equal(omax.data, omax_ref.data)
 
 
+def _random_context_cases(n, seed):
+    rng = np.random.RandomState(seed)
+    cases = []
+    for i in range(n):
+        hyps = int(rng.choice([1, 2, 3, 4, 4, 4, 6, 8, 12]))
+        sentences = int(rng.choice([1, 2, 3, 4, 6, 7, 16, 24]))
+        heads = int(rng.choice([1, 2, 4]))
+        K = int(rng.choice([128, 256, 384]))
+        L = int(rng.choice([1, 2, 15, 16, 17, 31, 32, 33, 47, 63, 64, 65, 80, 95, 96, 97, 120]))
+        cases.append((i, hyps, sentences, heads, K, L, L + int(rng.randint(0, 5)), bool(rng.randint(0, 2))))
+    return cases
+
+
+@pytest.mark.parametrize("i,hyps,sentences,heads,K,L,cap,masked", _random_context_cases(28, 77))
+def test_context_attention_form_random_shapes(integer, orc, synth, i, hyps, sentences, heads, K, L, cap, masked):
+    """hypotheses x sentences in every combination the row plan distinguishes (eight, four, two, one
+    hypotheses of a sentence per workgroup; staged in LDS or not; caches with room to grow): the one
+    launch against Wq's affine call followed by the attention, bit for bit"""
+    import torch
+    ops = load("ops")
+    M = hyps * sentences
+    say("proj + context attention, random", i, hyps, sentences, heads, K, L, cap, masked)
+    N = heads * 64
+    X = synth.normal(7100 + i, synth.STREAM_A, (M, K), 1.0)
+    ws = make_weights(integer, orc, synth, torch, 7200 + i, K, N, 1)
+    g = torch.Generator(device="cuda")
+    g.manual_seed(7300 + i)
+    kc = torch.randn(sentences * heads, cap, 64, device="cuda", generator=g)
+    vc = torch.randn(sentences * heads, cap, 64, device="cuda", generator=g)
+    mask = None
+    if masked:
+        lens = torch.randint(1, L + 1, (sentences,), device="cuda", generator=g)
+        mask = (torch.arange(L, device="cuda")[None, :] >= lens[:, None]).float() * -99999999.0
+    x = torch.from_numpy(X).cuda()
+    q, Aq_ref = integer.affine_f32(x, ws[0][1], ws[0][3])
+    o_ref, omax_ref = ops.Attention(q.view(M * heads, 1, 64), kc, vc, mask, rowsPerMask=heads, want_absmax=True, kvLen=L)
+    o, Aq, omax = ops.ProjectedAttention(x, [(ws[0][1], ws[0][3])], kc, vc, heads, kvLen=L, mask=mask, want_absmax=True)
+    torch.cuda.synchronize()
+    assert np.array_equal(Aq.numpy(), Aq_ref.numpy())
+    assert torch.equal(o.view(-1), o_ref.view(-1))
+    assert torch.equal(omax.data, omax_ref.data)
+    # and the attention alone against the same rows on a cache with a copy per query row (the
+    # general kernel: nothing is shared there)
+    o_rep = ops.Attention(q.view(M * heads, 1, 64), kc.repeat(hyps, 1, 1), vc.repeat(hyps, 1, 1), mask, rowsPerMask=heads, kvLen=L)
+    assert torch.equal(o_rep.view(-1), o_ref.view(-1))
+
+
 def test_proj_attention_argument_checks(integer):
     import ctypes
     L = load("_lib")
