@@ -1086,8 +1086,9 @@ __global__ __launch_bounds__(kProjThreads) void proj_attention_kernel(ProjAttent
   const int len4s = (p.len + 3) & ~3;
   float* kv_lds = att_lds + R * (len4s + 256);            // staged keys and values: [sentence][k, v][len][64]
 
-  // ---- everything this workgroup will need is requested now: abs-max slots, weights, the input
-  //      rows, the quantization multipliers of the weights, bias ----
+  // ---- everything this workgroup will need is requested now, in the order of its use (a wave's
+  //      loads complete in the order of their issue): abs-max slots, the input rows, weights, the
+  //      mask value, the quantization multipliers of the weights, bias ----
   float pm[kAbsmaxSlots / kProjThreads];
 #pragma unroll
   for(int i = 0; i < kAbsmaxSlots / kProjThreads; ++i) pm[i] = p.partials[min(tid + i * kProjThreads, p.n_partials - 1)];
