@@ -121,6 +121,8 @@ inline void Attention(Backend& be, Tensor& out, const Tensor& q, Tensor& k, Tens
 // complete, e.g. the encoder's - or {Wq, Wk, Wv} - self-attention, the new key and value go into
 // the caches at position kvLen - 1; biases: one entry per matrix (null entries allowed) or empty.
 // a [M, K] float32; aQuant: the prepareA node's tensor; k, v [entries, capacity, 64]; out [M, heads * 64].
+// Measured ahead of the two separate calls (affineOrDot for the projections, then Attention) up to
+// 128 rows, level with them at 256, behind at 512: a caller with larger batches issues those.
 inline void ProjectedAttention(TensorAllocator& ta, Tensor& out, const Tensor& a, Tensor& aQuant,
                                const std::vector<const Tensor*>& weights, const std::vector<const Tensor*>& biases,
                                Tensor& k, Tensor& v, int64_t heads, int64_t kvLen = 0, const Tensor* mask = nullptr,
