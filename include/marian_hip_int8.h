@@ -196,9 +196,9 @@ int marian_hip_int8_affine_f32_grouped(const float* A, int8_t* Aq, int64_t n_gro
  *   n_proj = 1: Bq / bias / proj_out hold {Wq}; the caches are complete (the encoder's keys and
  *     values), query row r uses cache entry r % batchKV.  With batchKV = sentences * heads and
  *     M = hypotheses * sentences (row m of A belongs to sentence m % sentences, the reference's
- *     [beam, batch] order) and an even number of hypotheses, a workgroup takes hypotheses of the
- *     same sentences and reads their keys and values once (up to 96 positions; other shapes
- *     take the general path, same result).
+ *     [beam, batch] order) and two or more hypotheses a sentence, a workgroup takes hypotheses
+ *     of the same one or two sentences and reads their keys and values once (up to 96 positions;
+ *     other shapes take the general path, same result).
  *   A: fp32 [M x K]; Aq receives what marian_hip_int8_prepare_a would write.  K % 128 == 0,
  *     K <= 1024, len <= 512.  Bq, bias, proj_out: HOST arrays of n_proj device pointers, read
  *     during the call; bias and proj_out (and their entries) may be NULL.  proj_out[g], where

@@ -828,7 +828,9 @@ __global__ __launch_bounds__(256) void attention_kernel(const float* __restrict_
 //      for operation, with q and the newest key/value row read from LDS.
 // Where the caches are complete and shared - the encoder's keys and values, which every hypothesis
 // of a sentence attends to (row m reads sentence m % sentences) - a workgroup takes hypotheses of
-// the same one or two sentences instead of eight consecutive rows, reads these sentences' keys and
+// the same one or two sentences instead of eight consecutive rows (ProjRowPlan in
+// operand_addressing.h: as many hypotheses of a sentence as a workgroup has rows for, the rest in
+// further workgroups; rows without a hypothesis idle), reads these sentences' keys and
 // values once (asked for as soon as the abs-max is known, stored to LDS in step 4) and its waves
 // take them from LDS: a quarter of the bytes through the CU's memory path with four hypotheses a
 // sentence (60 positions: 60 KB instead of 240 KB per workgroup).
@@ -870,11 +872,11 @@ struct ProjAttentionArgs {
   float att_scale;
   float* out;               // [M * heads, 64]
   float* absmax_out;        // slots or null
-  // Which input rows a workgroup takes.  share_shift < 0: eight consecutive ones.  Otherwise the
-  // caches hold `share_nb` sentences that several hypotheses each attend to (row m reads sentence
-  // m % share_nb), and a workgroup takes 8 >> share_shift hypotheses of 1 << share_shift
+  // Which input rows a workgroup takes (ProjRowPlan).  share_shift < 0: eight consecutive ones.
+  // Otherwise the caches hold `share_nb` sentences that share_hyps hypotheses each attend to (row m
+  // reads sentence m % share_nb), and a workgroup takes share_per of them for 1 << share_shift
   // neighbouring sentences, so that the waves that read the same keys and values sit on one CU.
-  int share_shift, share_nb;
+  int share_shift, share_nb, share_hyps, share_per;
   // With it (and sentences two or one to a workgroup, len <= kProjStageLen): the keys and values of
   // the workgroup's sentences are read once, into LDS, and every hypothesis' wave takes them from there.
   int stage_kv;
@@ -1077,7 +1079,7 @@ __global__ __launch_bounds__(kProjThreads) void proj_attention_kernel(ProjAttent
   const int h = blockIdx.x;
   // input row r of this workgroup (rows past the end: M or more)
   const int sent_base = p.share_shift < 0 ? 0 : proj_first_sentence(p.share_shift, p.share_nb, (int)blockIdx.y);
-  auto row_of = [&](int r) -> int { return proj_row_of(p.share_shift, p.share_nb, (int)blockIdx.y, r); };
+  auto row_of = [&](int r) -> int { return proj_row_of(p.share_shift, p.share_nb, p.share_hyps, p.share_per, (int)blockIdx.y, r); };
   const int K = p.K, M = p.M, S = K / 32, PW = S / 4, N = p.heads * 64;
   int8_t* a_lds = plds;                                   // 32 rows x K bytes, operand order
   int8_t* part_lds = a_lds + 32 * K;                      // NPROJ x 2 x 4 partial tiles of R rows x 128 bytes
@@ -2313,9 +2315,12 @@ int marian_hip_int8_proj_attention(const float* A, int8_t* Aq, int64_t n_proj, c
   const ProjRowPlan plan = proj_row_plan(n_proj, M, heads, batchKV, len, kProjStageLen, lds, (size_t)kProjMaxLds);
   p.share_shift = plan.shift;
   p.share_nb = plan.sentences;
+  p.share_hyps = plan.hyps;
+  p.share_per = plan.per_wg;
   p.stage_kv = plan.stage;
+  if(plan.blocks_y > 65535) return MARIAN_HIP_ERR_RANGE;
   if(plan.stage) lds += (size_t)(2 << plan.shift) * (size_t)len * 256;
-  const dim3 grid((unsigned)heads, (unsigned)((M + R - 1) / R));
+  const dim3 grid((unsigned)heads, (unsigned)plan.blocks_y);
 #define MH_PA(NP, SEGS, PASSES) \
   hipLaunchKernelGGL((proj_attention_kernel<NP, R, SEGS, PASSES>), grid, dim3(kProjThreads), lds, st, p)
   if(n_proj == 3) MH_PA(3, 0, 0);

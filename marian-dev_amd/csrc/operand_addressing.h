@@ -86,36 +86,62 @@ __host__ __device__ __forceinline__ bool stage_b_goes_back(int g, int tiles_n) {
 
 // ---- projections + attention in one launch (proj_attention_kernel): which input rows a workgroup takes ----
 // Caches that are complete and shared - `sentences` entries per head, row m attends to sentence
-// m % sentences, M = hypotheses * sentences - let a workgroup take 8 >> shift hypotheses of
-// 1 << shift neighbouring sentences instead of eight consecutive rows, so that the waves reading
-// the same keys and values sit on one CU.  shift < 0: eight consecutive rows.
+// m % sentences, M = hypotheses * sentences - let a workgroup take `per_wg` hypotheses of
+// 1 << shift neighbouring sentences (per_wg << shift <= 8) instead of eight consecutive rows, so
+// that the waves reading the same keys and values sit on one CU; the hypotheses of a sentence are
+// taken in `chunks` of per_wg.  Row r of a workgroup: hypothesis chunk * per_wg + (r >> shift) of
+// sentence first + (r & ((1 << shift) - 1)); rows whose hypothesis does not exist are idle.
+// shift < 0: eight consecutive rows.
 struct ProjRowPlan {
   int shift;       // log2 of the sentences per workgroup, or -1
   int sentences;
+  int hyps;        // hypotheses per sentence
+  int per_wg;      // hypotheses of a sentence a workgroup takes
   int stage;       // the sentences' keys and values are staged in LDS (shift 0 or 1, len <= stage_len)
+  long long blocks_y;   // workgroups per head
 };
 __host__ __device__ __forceinline__ ProjRowPlan proj_row_plan(long long n_proj, long long M, long long heads, long long batchKV,
                                                               long long len, int stage_len, size_t lds_without,
                                                               size_t lds_max) {
-  ProjRowPlan plan = {-1, 0, 0};
+  ProjRowPlan plan = {-1, 0, 0, 0, 0, (M + 7) / 8};
   if(n_proj != 1 || heads <= 0 || batchKV % heads != 0) return plan;
   const long long nb = batchKV / heads;
-  if(nb <= 0 || nb >= M || M % nb != 0) return plan;
+  if(nb <= 0 || nb >= M || M % nb != 0 || nb > 2147483647LL) return plan;
   const long long hyps = M / nb;
-  const int per_wg = hyps % 8 == 0 ? 8 : (hyps % 4 == 0 ? 4 : (hyps % 2 == 0 ? 2 : 1));
-  const int shift = per_wg == 8 ? 0 : (per_wg == 4 ? 1 : 2);
-  if(per_wg == 1 || nb % (1 << shift) != 0 || nb > 2147483647LL) return plan;
-  plan.shift = shift;
+  if(hyps > 2147483647LL) return plan;
+  // the fewest workgroups (each reads the head's weights), then the fewest chunks (each reads the
+  // sentences' keys and values); two hypotheses a sentence keep four sentences per workgroup
+  int best_shift = -1, best_per = 0;
+  long long best_blocks = 0, best_chunks = 0;
+  for(int shift = 2; shift >= 0; --shift) {
+    if(nb % (1 << shift) != 0) continue;
+    const int room = 8 >> shift;                        // hypotheses a workgroup has rows for
+    const long long chunks = (hyps + room - 1) / room;
+    const int per = (int)((hyps + chunks - 1) / chunks);
+    if(per < 2 || (per << shift) < 4) continue;         // (at least half of a workgroup's rows in use)
+    if(shift == 2 && hyps != 2) continue;               // (four sentences are not staged: only where nothing else fits)
+    const long long blocks = chunks * (nb >> shift);
+    if(best_shift < 0 || blocks < best_blocks || (blocks == best_blocks && chunks < best_chunks)) {
+      best_shift = shift; best_per = per; best_blocks = blocks; best_chunks = chunks;
+    }
+  }
+  if(best_shift < 0) return plan;
+  plan.shift = best_shift;
   plan.sentences = (int)nb;
-  const size_t kv_bytes = (size_t)(2 << shift) * (size_t)len * 256;
-  plan.stage = shift <= 1 && len <= stage_len && lds_without + kv_bytes <= lds_max;
+  plan.hyps = (int)hyps;
+  plan.per_wg = best_per;
+  plan.blocks_y = best_blocks;
+  const size_t kv_bytes = (size_t)(2 << best_shift) * (size_t)len * 256;
+  plan.stage = best_shift <= 1 && len <= stage_len && lds_without + kv_bytes <= lds_max;
   return plan;
 }
-// input row r (0 .. 7) of workgroup block_y
-__host__ __device__ __forceinline__ int proj_row_of(int shift, int sentences, int block_y, int r) {
+// input row r (0 .. 7) of workgroup block_y; rows that do not exist: a value of at least M (= hyps * sentences)
+__host__ __device__ __forceinline__ int proj_row_of(int shift, int sentences, int hyps, int per_wg, int block_y, int r) {
   if(shift < 0) return block_y * 8 + r;
   const int groups = sentences >> shift;
-  return ((block_y / groups) * (8 >> shift) + (r >> shift)) * sentences + ((block_y % groups) << shift) + (r & ((1 << shift) - 1));
+  const int j = r >> shift, hyp = (block_y / groups) * per_wg + j;
+  if(j >= per_wg || hyp >= hyps) return 0x7fffffff;
+  return hyp * sentences + ((block_y % groups) << shift) + (r & ((1 << shift) - 1));
 }
 // first sentence of workgroup block_y (shift >= 0)
 __host__ __device__ __forceinline__ int proj_first_sentence(int shift, int sentences, int block_y) {

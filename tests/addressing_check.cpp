@@ -163,13 +163,16 @@ static void proj_rows(long long hyps, long long sentences, long long heads, long
   const size_t lds_max = 160 * 1024 - 256;
   const ProjRowPlan plan = proj_row_plan(1, M, heads, batchKV, len, stage_len, lds_without, lds_max);
   char where[160];
-  std::snprintf(where, sizeof(where), "proj rows hyps %lld sentences %lld len %lld shift %d stage %d", hyps, sentences, len,
-                plan.shift, plan.stage);
-  const int blocks = (int)((M + 7) / 8);
+  std::snprintf(where, sizeof(where), "proj rows hyps %lld sentences %lld len %lld shift %d per %d stage %d", hyps, sentences,
+                len, plan.shift, plan.per_wg, plan.stage);
+  const int blocks = (int)plan.blocks_y;
+  if(plan.shift < 0 && plan.blocks_y != (M + 7) / 8) fail("workgroups of the plain form", plan.blocks_y, (M + 7) / 8, where);
+  if(plan.shift >= 0 && ((plan.per_wg << plan.shift) > 8 || (plan.per_wg << plan.shift) < 4 || plan.hyps != hyps))
+    fail("hypotheses per workgroup", plan.per_wg, plan.shift, where);
   std::vector<int> seen((size_t)M, 0);
   for(int by = 0; by < blocks; ++by)
     for(int r = 0; r < 8; ++r) {
-      const int m = proj_row_of(plan.shift, plan.sentences, by, r);
+      const int m = proj_row_of(plan.shift, plan.sentences, plan.hyps, plan.per_wg, by, r);
       ++g_checked;
       if(m < 0) { fail("negative row", by, r, where); continue; }
       if(m >= M) continue;   // rows past the end are skipped by the kernel
@@ -229,8 +232,8 @@ int main() {
         }
   std::printf("staged: %lld loads checked\n", g_checked - before);
   before = g_checked;
-  for(long long hyps : {1, 2, 3, 4, 6, 8, 12, 16})
-    for(long long sentences : {1, 2, 3, 5, 8, 10, 32, 33})
+  for(long long hyps : {1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 12, 16, 17})
+    for(long long sentences : {1, 2, 3, 4, 5, 8, 10, 32, 33})
       for(long long len : {1, 31, 32, 33, 60, 96, 97, 300})
         proj_rows(hyps, sentences, 16, len, len + 3);
   std::printf("projection rows: %lld rows checked\n", g_checked - before);
