@@ -207,7 +207,7 @@ def test_multiply_half_last_k_block(integer, orc, synth, M, K, N, kernel):
     run_case(integer, orc, synth, 480 + M + N, M, K, N, kernel, bias_on=True, relu=(K % 256 == 64), scale=0.75)
 
 
-@pytest.mark.parametrize("kernel", [0, 369, 371, 372, 373, 374, 375, 376, 377])
+@pytest.mark.parametrize("kernel", [0, 369, 371, 372, 373, 374, 375, 376, 377, 378])
 @pytest.mark.parametrize("M,K,N,bias_on,relu", [(128, 128, 128, True, False), (256, 256, 64, False, True), (640, 384, 1024, True, True),
                                                 (1000, 512, 1032, True, False), (2048, 1024, 1024, False, False),
                                                 (130, 2048, 136, True, True), (4096, 128, 1024, True, False)])
@@ -215,7 +215,8 @@ def test_multiply_split_form(integer, orc, synth, M, K, N, bias_on, relu, kernel
     """The large-M form whose loads are issued by four waves of their own beside the four that
     multiply (three and four LDS stages, 128 x 128 and 128 x 64 tiles, plain and non-temporal
     stores): one K block (nothing to pipeline), fewer blocks than stages, many; tiles that hang over
-    the edge of the output; 369 is the four-wave form the automatic choice took before."""
+    the edge of the output; 369 keeps the four-wave form everywhere, 378 takes the split form
+    wherever K allows (the automatic choice: where CUs stay idle, or K is 6144 or more)."""
     say("multiply split form", M, K, N, "kernel", kernel)
     run_case(integer, orc, synth, 520 + M + N, M, K, N, kernel, bias_on=bias_on, relu=relu, scale=1.25)
 
