@@ -667,16 +667,15 @@ int launch_gemm(const GemmArgs& a, hipStream_t st) {
   // so few 128x128 tiles that half the CUs would idle: 128x64 tiles (measured -20 % to -25 % for
   // M = 512 .. 1024, K = 4096, N = 1024; measurement id 340 keeps the square tiles)
   // Tiles of which a CU gets one: whole K blocks go to the split form - four more waves per workgroup
-  // issue the loads, the multiplying waves spend no issue slots on them (measured -2 % to -9 %;
-  // measurement id 369 keeps the four-wave form, 378 takes the split form wherever K allows).  Not
-  // where every CU has a tile and K is below 6144: a chip full of eight-wave workgroups does not
-  // hold its clock - after two seconds of the same launches 4096 x 2048 x 1024 takes 18.0 us
-  // in the split form against 13.0 us (12.8 against 13.2 us in a short burst), 4096 x 4096 x 1024
-  // 21.7 - 24 against 20.9 - 21.6 us (19.9 against 21.1 us in a short burst); from K = 6144 on, and
-  // wherever CUs stay idle, the split form is ahead in both states.
+  // issue the loads, the multiplying waves spend no issue slots on them (measured -6 % to -10 %;
+  // measurement id 369 keeps the four-wave form, 378 takes the split form wherever K allows).  Only
+  // where CUs stay idle: a chip full of eight-wave workgroups is ahead by 2 - 8 % on a machine that
+  // has been idle (4096 x 4096 x 1024 19.9 against 21.1 us) and far behind on one that has not -
+  // after a minute of other launches 25 - 29 against 23 - 25 us, 4096 x 2048 x 1024 19 - 23 against
+  // 14 us, 4096 x 6144 x 1024 31 - 32 against 29.5 us - while launches of fewer tiles than CUs keep
+  // their gain in both states.
   const int ov_split = kernel_override() % 1000;
-  const bool split = a.K % 128 == 0 && ov_split != 369 &&
-                     (ov_split == 378 || tiles128 < compute_units() || a.K >= 6144);
+  const bool split = a.K % 128 == 0 && ov_split != 369 && (ov_split == 378 || tiles128 < compute_units());
   if(2 * tiles128 <= compute_units() && kernel_override() % 1000 != 340) {
     if(split) return stream_out ? launch_big_split<128, 64, 2, 2, 4, true>(a, st) : launch_big_split<128, 64, 2, 2, 4, false>(a, st);
     if(stream_out) return launch_big<128, 64, 2, 2, 3, true, true>(a, st);

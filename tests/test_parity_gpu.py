@@ -216,7 +216,7 @@ def test_multiply_split_form(integer, orc, synth, M, K, N, bias_on, relu, kernel
     multiply (three and four LDS stages, 128 x 128 and 128 x 64 tiles, plain and non-temporal
     stores): one K block (nothing to pipeline), fewer blocks than stages, many; tiles that hang over
     the edge of the output; 369 keeps the four-wave form everywhere, 378 takes the split form
-    wherever K allows (the automatic choice: where CUs stay idle, or K is 6144 or more)."""
+    wherever K allows (the automatic choice: where CUs stay idle)."""
     say("multiply split form", M, K, N, "kernel", kernel)
     run_case(integer, orc, synth, 520 + M + N, M, K, N, kernel, bias_on=bias_on, relu=relu, scale=1.25)
 
